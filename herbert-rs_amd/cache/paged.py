@@ -1,0 +1,224 @@
+"""The cache on the GPU: paged keys and values per group of layers, and fixed-size state.
+
+Layers (more exactly: the entries of a model's schedule that own a cache) with
+the same need share a group. A group of keys and values owns one pool
+[entries, 2, pages, kv_heads, PAGE_TOKENS, head_dim], a page list of its own
+and a page table [slots, pages per slot]; the page index is shared by the
+group's entries, so one table serves them all. A group with a window gives
+back the pages that no later query can see. A group of fixed-size state owns
+[entries, slots, *shape] and is cleared for a slot when the slot is taken.
+
+Per slot the host keeps the length (positions held = next position), as the
+reference keeps `seq_len` beside its storage
+(crates/backends/backend_common/src/kv_cache.rs:270-273).
+"""
+from dataclasses import dataclass
+
+import numpy as np
+import torch
+
+from ..errors import CacheError
+from .needs import KVNeed, StateNeed
+from .slots import PAGE_TOKENS, FreeList, pages_for
+
+
+@dataclass
+class LayerKV:
+    """What an attention kernel needs of one schedule entry's cache."""
+    k: torch.Tensor            # [pages, kv_heads, PAGE_TOKENS, head_dim]
+    v: torch.Tensor
+    page_table: torch.Tensor   # int32 [slots, pages per slot]
+    page_size: int
+    window: int                # 0 = all keys
+
+
+class KVGroup:
+    def __init__(self, need, entries, n_pages, n_slots, max_positions, dtype, device):
+        self.need = need
+        self.entries = list(entries)
+        self.pages = FreeList(n_pages, "page")
+        self.pages_per_slot = pages_for(max_positions)
+        self.pool = torch.zeros((len(self.entries), 2, n_pages, need.kv_heads, PAGE_TOKENS,
+                                 need.head_dim), dtype=dtype, device=device)
+        self.table_host = np.full((n_slots, self.pages_per_slot), -1, dtype=np.int32)
+        # entries of the device table that are not held point at page 0: a kernel never reads
+        # them for a valid position, and an index that is always in range cannot fault
+        self.table = torch.zeros((n_slots, self.pages_per_slot), dtype=torch.int32, device=device)
+        self.first_page = np.zeros(n_slots, dtype=np.int64)   # first logical page still held
+
+    def view(self, entry):
+        i = self.entries.index(entry)
+        return LayerKV(self.pool[i, 0], self.pool[i, 1], self.table, PAGE_TOKENS,
+                       int(self.need.window or 0))
+
+    def ensure(self, slot, new_length):
+        """Hold a page for every position below new_length that a query may still see."""
+        row = self.table_host[slot]
+        first_new = None
+        last = pages_for(new_length)
+        for p in range(int(self.first_page[slot]), last):
+            if row[p] < 0:
+                row[p] = self.pages.take()
+                if first_new is None:
+                    first_new = p
+        if first_new is not None:
+            self._upload(slot, first_new, last)
+
+    def _upload(self, slot, a, b):
+        self.table[slot, a:b] = torch.from_numpy(np.maximum(self.table_host[slot, a:b], 0)).to(
+            self.table.device)
+
+    def release_unseen(self, slot, length):
+        """With a window: give back pages wholly before the oldest key a later query sees."""
+        if not self.need.window:
+            return
+        # a query at position >= length sees keys >= length + 1 - window
+        oldest = length + 1 - self.need.window
+        row = self.table_host[slot]
+        p = int(self.first_page[slot])
+        while (p + 1) * PAGE_TOKENS <= oldest:
+            if row[p] >= 0:
+                self.pages.give_back(int(row[p]))
+                row[p] = -1
+            p += 1
+        self.first_page[slot] = p
+
+    def truncate(self, slot, length):
+        row = self.table_host[slot]
+        if self.need.window:
+            oldest = max(0, length + 1 - self.need.window)   # oldest key the next query sees
+            if self.first_page[slot] * PAGE_TOKENS > oldest:
+                raise CacheError("cannot roll a windowed cache back past keys it has given up")
+        for p in range(pages_for(length), self.pages_per_slot):
+            if row[p] >= 0:
+                self.pages.give_back(int(row[p]))
+                row[p] = -1
+
+    def free_slot(self, slot):
+        row = self.table_host[slot]
+        for p in np.nonzero(row >= 0)[0]:
+            self.pages.give_back(int(row[p]))
+        row[:] = -1
+        self.first_page[slot] = 0
+
+
+class StateGroup:
+    def __init__(self, need, entries, n_slots, device):
+        self.need = need
+        self.entries = list(entries)
+        self.data = torch.zeros((len(self.entries), n_slots) + tuple(need.shape), dtype=need.dtype,
+                                device=device)
+
+    def view(self, entry):
+        return self.data[self.entries.index(entry)]
+
+    def clear_slot(self, slot):
+        self.data[:, slot].zero_()
+
+
+class Cache:
+    """Slots, their lengths, and the groups of storage behind them.
+
+    `needs` maps a schedule entry (an int) to its need (KVNeed, StateNeed, or a
+    tuple of them); entries that read another entry's cache are not in it.
+    `max_tokens` is the most tokens that live sequences hold at any time, each
+    sequence's count rounded up to a multiple of PAGE_TOKENS.
+    """
+
+    def __init__(self, needs, max_tokens, max_positions, dtype, device, max_slots=None):
+        n_pages = pages_for(max(int(max_tokens), 1))
+        self.n_pages = n_pages
+        self.n_slots = int(max_slots) if max_slots else n_pages
+        self.max_positions = int(max_positions)
+        self.slots = FreeList(self.n_slots, "slot")
+        self.lengths = np.zeros(self.n_slots, dtype=np.int64)
+        self.kv_groups = {}
+        self.state_groups = {}
+        self._kv_of = {}
+        self._state_of = {}
+        by_need = {}
+        for entry, need in needs.items():
+            for one in (need if isinstance(need, (tuple, list)) else (need,)):
+                by_need.setdefault(one, []).append(entry)
+        for need, entries in by_need.items():
+            if isinstance(need, KVNeed):
+                group = KVGroup(need, entries, n_pages, self.n_slots, max_positions, dtype, device)
+                self.kv_groups[need] = group
+                for e in entries:
+                    self._kv_of[e] = group
+            elif isinstance(need, StateNeed):
+                group = StateGroup(need, entries, self.n_slots, device)
+                self.state_groups[need] = group
+                for e in entries:
+                    self._state_of.setdefault(e, []).append(group)
+            else:
+                raise CacheError(f"unknown cache need {need!r}")
+
+    # ---- slots
+    def alloc_slot(self):
+        slot = self.slots.take()
+        self.lengths[slot] = 0
+        for g in self.state_groups.values():
+            g.clear_slot(slot)
+        return slot
+
+    def free_slot(self, slot):
+        self.slots.give_back(slot)
+        for g in self.kv_groups.values():
+            g.free_slot(slot)
+        self.lengths[slot] = 0
+
+    def length(self, slot):
+        if not self.slots.is_held(slot):
+            raise CacheError(f"slot {slot} is not held")
+        return int(self.lengths[slot])
+
+    # ---- one step
+    def reserve(self, slot, new_tokens):
+        """Make room for `new_tokens` more positions of a slot (before the step runs)."""
+        new_length = self.length(slot) + int(new_tokens)
+        if new_length > self.max_positions:
+            raise CacheError(f"slot {slot}: {new_length} positions exceed the model's "
+                             f"{self.max_positions}")
+        for g in self.kv_groups.values():
+            g.ensure(slot, new_length)
+        return new_length
+
+    def commit(self, slot, new_tokens):
+        """The step has run: the slot is longer; windowed groups give up what is out of sight."""
+        self.lengths[slot] += int(new_tokens)
+        for g in self.kv_groups.values():
+            g.release_unseen(slot, int(self.lengths[slot]))
+
+    def truncate(self, slot, length):
+        """Roll a slot back to its first `length` positions (the reference's truncate_kv,
+        crates/backends/backend_common/src/cpu_backend.rs:527-543). Fixed-size state cannot be
+        rolled back and refuses."""
+        if length > self.length(slot) or length < 0:
+            raise CacheError(f"cannot truncate slot {slot} of length {self.length(slot)} to {length}")
+        if self.state_groups and length != self.length(slot):
+            raise CacheError("a cache with per-sequence state cannot be rolled back")
+        for g in self.kv_groups.values():
+            g.truncate(slot, length)
+        self.lengths[slot] = length
+
+    # ---- views for the parts
+    def kv_view(self, entry):
+        return self._kv_of[entry].view(entry)
+
+    def state_views(self, entry):
+        return [g.view(entry) for g in self._state_of.get(entry, [])]
+
+    def check(self):
+        """Bookkeeping invariants: nothing lost, nothing held twice."""
+        self.slots.check()
+        for g in self.kv_groups.values():
+            g.pages.check()
+            held = g.table_host[g.table_host >= 0]
+            if len(set(held.tolist())) != len(held):
+                raise CacheError("a page is in two places of the page table")
+            if len(held) != g.pages.held_count:
+                raise CacheError("held pages and the page table disagree")
+            for slot in range(self.n_slots):
+                if not self.slots.is_held(slot) and (g.table_host[slot] >= 0).any():
+                    raise CacheError(f"free slot {slot} still holds pages")

@@ -1,0 +1,212 @@
+// Row-wise kernels of the decoder: embedding gather, RMSNorm, the fused
+// per-head norm + rotation + cache write, and SwiGLU. All arithmetic is float32;
+// the template parameters are the storage types of inputs and outputs.
+#include "common.h"
+
+HB_MODULE_ERROR_SLOT()
+
+// ---------------------------------------------------------------- embedding
+// x[t, :] = float(table[ids[t], :]); the residual stream is float32.
+template <class TW>
+__global__ void embed_kernel(const int* __restrict__ ids, const TW* __restrict__ table,
+                             float* __restrict__ x, int H) {
+    const int t = blockIdx.x;
+    const TW* row = table + (size_t)ids[t] * H;
+    float* out = x + (size_t)t * H;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) out[i] = hb_to_float(row[i]);
+}
+
+extern "C" int hb_embed(const int* ids, const void* table, int table_dtype, float* x, int T, int H,
+                        hipStream_t stream) {
+    HB_REQUIRE(T > 0 && H > 0, "embed: empty input (T=%d, H=%d)", T, H);
+    if (table_dtype == HB_F32)
+        embed_kernel<float><<<T, 256, 0, stream>>>(ids, (const float*)table, x, H);
+    else if (table_dtype == HB_BF16)
+        embed_kernel<bf16><<<T, 256, 0, stream>>>(ids, (const bf16*)table, x, H);
+    else
+        HB_REQUIRE(false, "embed: unknown table dtype %d", table_dtype);
+    HB_CHECK_LAUNCH("embed");
+    return 0;
+}
+
+// ------------------------------------------------------------------ RMSNorm
+// y[r, :] = x[src(r), :] * rsqrt(mean(x^2) + eps) * w ; src(r) = rows ? rows[r] : r.
+// One block per output row; the sum's order depends on H and the block size only.
+template <class TOut>
+__global__ void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                               TOut* __restrict__ y, const int* __restrict__ rows, int H, float eps) {
+    __shared__ float red[16];
+    const int r = blockIdx.x;
+    const float* in = x + (size_t)(rows ? rows[r] : r) * H;
+    TOut* out = y + (size_t)r * H;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+        const float v = in[i];
+        ss += v * v;
+    }
+    ss = hb_block_sum(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)H + eps);
+    for (int i = threadIdx.x; i < H; i += blockDim.x) out[i] = hb_from_float<TOut>(in[i] * inv * w[i]);
+}
+
+extern "C" int hb_rmsnorm(const float* x, const float* w, void* y, int y_dtype, const int* rows, int R,
+                          int H, float eps, hipStream_t stream) {
+    HB_REQUIRE(R > 0 && H > 0, "rmsnorm: empty input (R=%d, H=%d)", R, H);
+    const int threads = H >= 1024 ? 256 : 64;
+    if (y_dtype == HB_F32)
+        rmsnorm_kernel<float><<<R, threads, 0, stream>>>(x, w, (float*)y, rows, H, eps);
+    else if (y_dtype == HB_BF16)
+        rmsnorm_kernel<bf16><<<R, threads, 0, stream>>>(x, w, (bf16*)y, rows, H, eps);
+    else
+        HB_REQUIRE(false, "rmsnorm: unknown output dtype %d", y_dtype);
+    HB_CHECK_LAUNCH("rmsnorm");
+    return 0;
+}
+
+// ------------------------------------- per-head norm + rotation + cache write
+// One wave per (token, head) of the fused projection row [q heads | k heads | v heads].
+//   q heads: optional RMSNorm over the head, optional rotation, written to q_out.
+//   k heads: the same, written to the key pages of the token's slot.
+//   v heads: copied to the value pages.
+// Rotation pairs dim j with j + R/2 (R = rot_dims), angle table [max_pos, R/2].
+// The page of position p of a slot is page_table[slot * max_pages + p / page_size].
+#define HB_MAX_HEAD_DIM 512
+
+template <class TQ, class TC>
+__global__ void qk_norm_rope_write_kernel(
+    const float* __restrict__ qkv, int ld_qkv, const float* __restrict__ q_norm_w,
+    const float* __restrict__ k_norm_w, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+    int rot_dims, const int* __restrict__ positions, const int* __restrict__ seq_of,
+    const int* __restrict__ slots, const int* __restrict__ page_table, int max_pages, int page_size,
+    TQ* __restrict__ q_out, TC* __restrict__ k_cache, TC* __restrict__ v_cache, int nq, int nkv, int hd,
+    float eps) {
+    __shared__ float vec[HB_MAX_HEAD_DIM];
+    const int t = blockIdx.x;
+    const int h = blockIdx.y;
+    const int lane = threadIdx.x;
+    const float* src = qkv + (size_t)t * ld_qkv + (size_t)h * hd;
+    const bool is_q = h < nq;
+    const bool is_v = h >= nq + nkv;
+    const int pos = positions[t];
+
+    float ss = 0.f;
+    for (int d = lane; d < hd; d += HB_WAVE) {
+        const float v = src[d];
+        vec[d] = v;
+        ss += v * v;
+    }
+    ss = hb_wave_sum(ss);
+    __syncthreads();
+
+    const float* norm_w = is_q ? q_norm_w : k_norm_w;
+    const bool do_norm = !is_v && norm_w != nullptr;
+    const bool do_rope = !is_v && cos_t != nullptr;
+    const float inv = do_norm ? 1.0f / sqrtf(ss / (float)hd + eps) : 1.0f;
+    const int half = rot_dims / 2;
+
+    size_t dst_base = 0;
+    if (!is_q) {
+        const int slot = slots[seq_of[t]];
+        const int page = page_table[(size_t)slot * max_pages + pos / page_size];
+        const int kvh = is_v ? h - nq - nkv : h - nq;
+        dst_base = (((size_t)page * nkv + kvh) * page_size + (pos % page_size)) * hd;
+    }
+
+    for (int d = lane; d < hd; d += HB_WAVE) {
+        float out;
+        if (do_rope && d < rot_dims) {
+            const int j = d < half ? d : d - half;
+            const float c = cos_t[(size_t)pos * half + j];
+            const float s = sin_t[(size_t)pos * half + j];
+            float x0 = vec[j], x1 = vec[j + half];
+            if (do_norm) {
+                x0 = x0 * inv * norm_w[j];
+                x1 = x1 * inv * norm_w[j + half];
+            }
+            out = d < half ? x0 * c - x1 * s : x0 * s + x1 * c;
+        } else {
+            out = vec[d];
+            if (do_norm) out = out * inv * norm_w[d];
+        }
+        if (is_q)
+            q_out[(size_t)t * nq * hd + (size_t)h * hd + d] = hb_from_float<TQ>(out);
+        else if (is_v)
+            v_cache[dst_base + d] = hb_from_float<TC>(out);
+        else
+            k_cache[dst_base + d] = hb_from_float<TC>(out);
+    }
+}
+
+extern "C" int hb_qk_norm_rope_write(const float* qkv, int ld_qkv, const float* q_norm_w,
+                                     const float* k_norm_w, const float* cos_t, const float* sin_t,
+                                     int rot_dims, const int* positions, const int* seq_of,
+                                     const int* slots, const int* page_table, int max_pages,
+                                     int page_size, void* q_out, void* k_cache, void* v_cache, int dtype,
+                                     int T, int nq, int nkv, int hd, float eps, int write_kv,
+                                     hipStream_t stream) {
+    HB_REQUIRE(T > 0 && nq > 0 && nkv > 0, "qk_norm_rope_write: empty input");
+    HB_REQUIRE(hd > 0 && hd <= HB_MAX_HEAD_DIM, "qk_norm_rope_write: head_dim %d not in 1..%d", hd,
+               HB_MAX_HEAD_DIM);
+    HB_REQUIRE(rot_dims % 2 == 0 && rot_dims >= 0 && rot_dims <= hd,
+               "qk_norm_rope_write: rotary dims %d must be even and <= head_dim %d", rot_dims, hd);
+    // write_kv == 0: the row holds query heads only and the cache is left alone
+    const int heads = nq + (write_kv ? 2 * nkv : 0);
+    HB_REQUIRE(ld_qkv >= heads * hd, "qk_norm_rope_write: row stride %d too small", ld_qkv);
+    HB_REQUIRE(heads <= 65535, "qk_norm_rope_write: too many heads for the grid");
+    dim3 grid(T, heads);
+    if (dtype == HB_F32)
+        qk_norm_rope_write_kernel<float, float><<<grid, HB_WAVE, 0, stream>>>(
+            qkv, ld_qkv, q_norm_w, k_norm_w, cos_t, sin_t, rot_dims, positions, seq_of, slots,
+            page_table, max_pages, page_size, (float*)q_out, (float*)k_cache, (float*)v_cache, nq, nkv,
+            hd, eps);
+    else if (dtype == HB_BF16)
+        qk_norm_rope_write_kernel<bf16, bf16><<<grid, HB_WAVE, 0, stream>>>(
+            qkv, ld_qkv, q_norm_w, k_norm_w, cos_t, sin_t, rot_dims, positions, seq_of, slots,
+            page_table, max_pages, page_size, (bf16*)q_out, (bf16*)k_cache, (bf16*)v_cache, nq, nkv, hd,
+            eps);
+    else
+        HB_REQUIRE(false, "qk_norm_rope_write: unknown dtype %d", dtype);
+    HB_CHECK_LAUNCH("qk_norm_rope_write");
+    return 0;
+}
+
+// ------------------------------------------------------------------- SwiGLU
+// act[t, i] = silu(gu[t, i]) * gu[t, I + i], silu(g) = g / (1 + exp(-g)).
+template <class TOut>
+__global__ void swiglu_kernel(const float* __restrict__ gu, TOut* __restrict__ act, int I, size_t total) {
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const size_t t = idx / I;
+    const int i = (int)(idx - t * I);
+    const float g = gu[t * 2 * I + i];
+    const float u = gu[t * 2 * I + I + i];
+    act[idx] = hb_from_float<TOut>(g / (1.0f + expf(-g)) * u);
+}
+
+extern "C" int hb_swiglu(const float* gu, void* act, int act_dtype, int T, int I, hipStream_t stream) {
+    HB_REQUIRE(T > 0 && I > 0, "swiglu: empty input");
+    const size_t total = (size_t)T * I;
+    const unsigned blocks = (unsigned)((total + 255) / 256);
+    if (act_dtype == HB_F32)
+        swiglu_kernel<float><<<blocks, 256, 0, stream>>>(gu, (float*)act, I, total);
+    else if (act_dtype == HB_BF16)
+        swiglu_kernel<bf16><<<blocks, 256, 0, stream>>>(gu, (bf16*)act, I, total);
+    else
+        HB_REQUIRE(false, "swiglu: unknown output dtype %d", act_dtype);
+    HB_CHECK_LAUNCH("swiglu");
+    return 0;
+}
+
+// ------------------------------------------------------------------ fill
+// A small fill kernel: clears memory inside captured graphs, where a memset node may not stand.
+__global__ void fill_u32_kernel(uint32_t* p, uint32_t v, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = v;
+}
+
+extern "C" int hb_fill_u32(void* p, uint32_t value, size_t n, hipStream_t stream) {
+    if (n == 0) return 0;
+    fill_u32_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>((uint32_t*)p, value, n);
+    HB_CHECK_LAUNCH("fill_u32");
+    return 0;
+}

@@ -1,0 +1,480 @@
+// Choosing the next token on the GPU: argmax and temperature / top-k / top-p sampling.
+// The order of candidates is value descending, index ascending among equals; sums that
+// decide a cut or a draw are added one value after the other in that order by one
+// thread, so that a seed gives the same token as the step-by-step host formulation.
+#include "common.h"
+#include <math.h>
+
+HB_MODULE_ERROR_SLOT()
+
+// ------------------------------------------------------------------ argmax
+// First index of the largest value of each row (strict > while scanning upwards).
+__global__ void __launch_bounds__(1024)
+argmax_kernel(const float* __restrict__ logits, int ld, int V, int* __restrict__ out) {
+    __shared__ float best_v[16];
+    __shared__ int best_i[16];
+    const float* row = logits + (size_t)blockIdx.x * ld;
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int i = threadIdx.x; i < V; i += blockDim.x) {
+        const float v = row[i];
+        if (v > bv) {
+            bv = v;
+            bi = i;
+        }
+    }
+#pragma unroll
+    for (int off = HB_WAVE / 2; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(bv, off, HB_WAVE);
+        const int oi = __shfl_xor(bi, off, HB_WAVE);
+        if (ov > bv || (ov == bv && oi < bi)) {
+            bv = ov;
+            bi = oi;
+        }
+    }
+    const int lane = threadIdx.x & (HB_WAVE - 1), wave = threadIdx.x / HB_WAVE;
+    if (lane == 0) {
+        best_v[wave] = bv;
+        best_i[wave] = bi;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const int nw = (blockDim.x + HB_WAVE - 1) / HB_WAVE;
+        for (int w = 1; w < nw; ++w)
+            if (best_v[w] > bv || (best_v[w] == bv && best_i[w] < bi)) {
+                bv = best_v[w];
+                bi = best_i[w];
+            }
+        // a row without any value above -inf (or all NaN) gives index 0, as a scan from 0 would
+        out[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;
+    }
+}
+
+extern "C" int hb_argmax(const float* logits, int ld, int R, int V, int* out, hipStream_t stream) {
+    HB_REQUIRE(R > 0 && V > 0 && ld >= V, "argmax: bad sizes (R=%d, V=%d, ld=%d)", R, V, ld);
+    argmax_kernel<<<R, 1024, 0, stream>>>(logits, ld, V, out);
+    HB_CHECK_LAUNCH("argmax");
+    return 0;
+}
+
+// ---------------------------------------------------------------- sampling
+// xorshift64 (<<13, >>7, <<17); the draw is the upper 24 bits over 2^24.
+__device__ __forceinline__ float xorshift_next_f32(unsigned long long* state) {
+    unsigned long long x = *state;
+    x ^= x << 13;
+    x ^= x >> 7;
+    x ^= x << 17;
+    *state = x;
+    return (float)(x >> 40) / 16777216.0f;
+}
+
+// Order-preserving map float -> uint32 (larger float, larger key).
+__device__ __forceinline__ uint32_t float_key(float v) {
+    const uint32_t u = __float_as_uint(v);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float key_float(uint32_t k) {
+    return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
+}
+
+#define SAMPLE_THREADS 1024
+#define SAMPLE_MAX_K 1024
+
+// (key descending, index ascending) "a before b"
+__device__ __forceinline__ bool cand_before(uint32_t ka, int ia, uint32_t kb, int ib) {
+    return ka > kb || (ka == kb && ia < ib);
+}
+
+__device__ void bitonic_sort_lds(uint32_t* keys, int* idx, int n_pow2) {
+    for (int size = 2; size <= n_pow2; size <<= 1) {
+        for (int stride = size >> 1; stride > 0; stride >>= 1) {
+            __syncthreads();
+            for (int i = threadIdx.x; i < n_pow2 / 2; i += blockDim.x) {
+                const int lo = 2 * i - (i & (stride - 1));
+                const int hi = lo + stride;
+                const bool up = (lo & size) == 0;   // this run is sorted "before first"
+                const bool hi_first = cand_before(keys[hi], idx[hi], keys[lo], idx[lo]);
+                if (hi_first == up) {
+                    const uint32_t tk = keys[lo];
+                    keys[lo] = keys[hi];
+                    keys[hi] = tk;
+                    const int ti = idx[lo];
+                    idx[lo] = idx[hi];
+                    idx[hi] = ti;
+                }
+            }
+        }
+    }
+    __syncthreads();
+}
+
+// One block per row, 0 < top_k <= SAMPLE_MAX_K and top_k < V.
+//  1. scaled = logit / temperature; the top_k largest (ties: lower index first) by a
+//     radix select over the keys, gathered and sorted in LDS;
+//  2. softmax over them; 3. top-p cut and renormalisation; 4. the draw.
+__global__ void __launch_bounds__(SAMPLE_THREADS)
+sample_topk_kernel(const float* __restrict__ logits, int ld, int V, float temperature, int top_k,
+                   float top_p, unsigned long long* __restrict__ rng, const int* __restrict__ rng_index,
+                   int* __restrict__ out) {
+    __shared__ uint32_t keys[SAMPLE_MAX_K];
+    __shared__ int idx[SAMPLE_MAX_K];
+    __shared__ float prob[SAMPLE_MAX_K];
+    __shared__ int hist[256];
+    __shared__ int wave_counts[SAMPLE_THREADS / HB_WAVE];
+    __shared__ uint32_t sel_prefix;
+    __shared__ int sel_remaining;
+    __shared__ int n_gathered;
+    __shared__ int eq_taken;
+
+    const float* row = logits + (size_t)blockIdx.x * ld;
+    const int tid = threadIdx.x;
+
+    // ---- radix select: the key of the top_k-th largest scaled logit
+    if (tid == 0) {
+        sel_prefix = 0;
+        sel_remaining = top_k;
+    }
+    for (int shift = 24; shift >= 0; shift -= 8) {
+        if (tid < 256) hist[tid] = 0;
+        __syncthreads();
+        const uint32_t prefix = sel_prefix;
+        const uint32_t mask = shift == 24 ? 0u : (0xffffffffu << (shift + 8));
+        for (int i = tid; i < V; i += blockDim.x) {
+            const uint32_t k = float_key(row[i] / temperature);
+            if ((k & mask) == prefix) atomicAdd(&hist[(k >> shift) & 0xff], 1);
+        }
+        __syncthreads();
+        if (tid == 0) {
+            int remaining = sel_remaining;
+            int b = 255;
+            for (; b > 0; --b) {
+                if (hist[b] >= remaining) break;
+                remaining -= hist[b];
+            }
+            sel_prefix = prefix | ((uint32_t)b << shift);
+            sel_remaining = remaining;
+        }
+        __syncthreads();
+    }
+    const uint32_t kth = sel_prefix;        // key of the k-th largest
+    const int need_eq = sel_remaining;      // how many of the equal keys belong to the top k
+
+    // ---- gather: all keys above kth in any order, the first need_eq equal ones by index
+    if (tid == 0) {
+        n_gathered = 0;
+        eq_taken = 0;
+    }
+    __syncthreads();
+    const int lane = tid & (HB_WAVE - 1), wave = tid / HB_WAVE;
+    for (int base = 0; base < V; base += blockDim.x) {
+        const int i = base + tid;
+        uint32_t k = 0;
+        bool above = false, equal = false;
+        if (i < V) {
+            k = float_key(row[i] / temperature);
+            above = k > kth;
+            equal = k == kth;
+        }
+        if (above) {
+            const int at = atomicAdd(&n_gathered, 1);
+            keys[at] = k;
+            idx[at] = i;
+        }
+        // ordered rank of the equal ones within this stretch of the row
+        const unsigned long long bal = __ballot(equal);
+        const int before_lane = __popcll(bal & ((1ull << lane) - 1ull));
+        if (lane == 0) wave_counts[wave] = __popcll(bal);
+        __syncthreads();
+        int before = eq_taken;
+        for (int w = 0; w < wave; ++w) before += wave_counts[w];
+        const int rank = before + before_lane;
+        if (equal && rank < need_eq) {
+            const int at = atomicAdd(&n_gathered, 1);
+            keys[at] = k;
+            idx[at] = i;
+        }
+        __syncthreads();
+        if (tid == 0) {
+            int total = 0;
+            for (int w = 0; w < SAMPLE_THREADS / HB_WAVE; ++w) total += wave_counts[w];
+            eq_taken += total;
+        }
+        __syncthreads();
+    }
+    const int n = n_gathered;   // == top_k
+    int n_pow2 = 1;
+    while (n_pow2 < n) n_pow2 <<= 1;
+    for (int i = n + tid; i < n_pow2; i += blockDim.x) {
+        keys[i] = 0u;
+        idx[i] = 0x7fffffff;
+    }
+    bitonic_sort_lds(keys, idx, n_pow2);
+
+    // ---- softmax in candidate order (the first candidate holds the maximum)
+    const float max_val = key_float(keys[0]);
+    for (int i = tid; i < n; i += blockDim.x) prob[i] = expf(key_float(keys[i]) - max_val);
+    __syncthreads();
+    __shared__ float inv_sum_s;
+    if (tid == 0) {
+        float sum = 0.f;
+        for (int i = 0; i < n; ++i) sum += prob[i];
+        inv_sum_s = 1.0f / sum;
+    }
+    __syncthreads();
+    for (int i = tid; i < n; i += blockDim.x) prob[i] *= inv_sum_s;
+    __syncthreads();
+
+    __shared__ int n_kept;
+    if (tid == 0) n_kept = n;
+    if (top_p < 1.0f) {
+        // order by probability descending (index ascending among equals); exp can map two
+        // different keys to one probability, so this is a sort of its own
+        for (int i = tid; i < n_pow2; i += blockDim.x) keys[i] = i < n ? float_key(prob[i]) : 0u;
+        bitonic_sort_lds(keys, idx, n_pow2);
+        for (int i = tid; i < n; i += blockDim.x) prob[i] = key_float(keys[i]);
+        __syncthreads();
+        if (tid == 0) {
+            float cum = 0.f;
+            int cutoff = n;
+            for (int i = 0; i < n; ++i) {
+                cum += prob[i];
+                if (cum >= top_p) {
+                    cutoff = i + 1;
+                    break;
+                }
+            }
+            float sum = 0.f;
+            for (int i = 0; i < cutoff; ++i) sum += prob[i];
+            inv_sum_s = 1.0f / sum;
+            n_kept = cutoff;
+        }
+        __syncthreads();
+        const int kept = n_kept;
+        for (int i = tid; i < kept; i += blockDim.x) prob[i] *= inv_sum_s;
+    }
+    __syncthreads();
+
+    if (tid == 0) {
+        unsigned long long* st = rng + (rng_index ? rng_index[blockIdx.x] : blockIdx.x);
+        const float r = xorshift_next_f32(st);
+        const int kept = n_kept;
+        float cum = 0.f;
+        int chosen = idx[kept - 1];
+        for (int i = 0; i < kept; ++i) {
+            cum += prob[i];
+            if (r < cum) {
+                chosen = idx[i];
+                break;
+            }
+        }
+        out[blockIdx.x] = chosen;
+    }
+}
+
+// ---- the general path: candidates of a row in global scratch as (key, index) pairs.
+// prepare: pairs[r, i] = (key(logit / temperature), i) for i < V, padding up to P2 (a power
+// of two) with (0, INT_MAX), which sorts last.
+__global__ void sample_prepare_kernel(const float* __restrict__ logits, int ld, int V, int P2,
+                                      float temperature, uint32_t* __restrict__ keys,
+                                      int* __restrict__ idx) {
+    const int r = blockIdx.y;
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= P2) return;
+    const size_t o = (size_t)r * P2 + i;
+    if (i < V) {
+        keys[o] = float_key(logits[(size_t)r * ld + i] / temperature);
+        idx[o] = i;
+    } else {
+        keys[o] = 0u;
+        idx[o] = 0x7fffffff;
+    }
+}
+
+// One compare-exchange stage of a bitonic sort over every row.
+__global__ void sample_bitonic_stage_kernel(uint32_t* __restrict__ keys, int* __restrict__ idx, int P2,
+                                            int size, int stride) {
+    const int r = blockIdx.y;
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= P2 / 2) return;
+    uint32_t* k = keys + (size_t)r * P2;
+    int* x = idx + (size_t)r * P2;
+    const int lo = 2 * i - (i & (stride - 1));
+    const int hi = lo + stride;
+    const bool up = (lo & size) == 0;
+    const bool hi_first = cand_before(k[hi], x[hi], k[lo], x[lo]);
+    if (hi_first == up) {
+        const uint32_t tk = k[lo];
+        k[lo] = k[hi];
+        k[hi] = tk;
+        const int ti = x[lo];
+        x[lo] = x[hi];
+        x[hi] = ti;
+    }
+}
+
+// finish: one block per row over its first n candidates (sorted when sorted != 0, else
+// in index order). Values pass through LDS in stretches; thread 0 adds them in order.
+#define FINISH_CHUNK 4096
+__global__ void __launch_bounds__(1024)
+sample_finish_kernel(const uint32_t* __restrict__ keys, const int* __restrict__ idx, int P2, int n,
+                     int sorted, float top_p, unsigned long long* __restrict__ rng,
+                     const int* __restrict__ rng_index, int* __restrict__ out) {
+    __shared__ float buf[FINISH_CHUNK];
+    __shared__ float red[16];
+    __shared__ float s_max, s_inv, s_inv2, s_r;
+    __shared__ int s_kept, s_chosen, s_done;
+    __shared__ float s_cum;
+    const uint32_t* k = keys + (size_t)blockIdx.x * P2;
+    const int* x = idx + (size_t)blockIdx.x * P2;
+    const int tid = threadIdx.x;
+
+    // maximum: the first candidate when sorted, else a reduction (its order does not matter)
+    if (sorted) {
+        if (tid == 0) s_max = key_float(k[0]);
+    } else {
+        float mv = -INFINITY;
+        for (int i = tid; i < n; i += blockDim.x) mv = fmaxf(mv, key_float(k[i]));
+        mv = hb_wave_max(mv);
+        if ((tid & (HB_WAVE - 1)) == 0) red[tid / HB_WAVE] = mv;
+        __syncthreads();
+        if (tid == 0) {
+            for (int w = 1; w < (int)(blockDim.x / HB_WAVE); ++w) mv = fmaxf(mv, red[w]);
+            s_max = mv;
+        }
+    }
+    __syncthreads();
+    const float max_val = s_max;
+
+    // pass 1: the softmax denominator
+    float sum = 0.f;
+    for (int c = 0; c < n; c += FINISH_CHUNK) {
+        const int m = n - c < FINISH_CHUNK ? n - c : FINISH_CHUNK;
+        __syncthreads();
+        for (int i = tid; i < m; i += blockDim.x) buf[i] = expf(key_float(k[c + i]) - max_val);
+        __syncthreads();
+        if (tid == 0)
+            for (int i = 0; i < m; ++i) sum += buf[i];
+    }
+    if (tid == 0) {
+        s_inv = 1.0f / sum;
+        s_kept = n;
+        s_inv2 = 1.0f;
+    }
+    __syncthreads();
+    const float inv = s_inv;
+
+    // pass 2: the top-p cut (candidates are sorted then) and the sum of the kept ones
+    if (top_p < 1.0f) {
+        if (tid == 0) {
+            s_cum = 0.f;
+            s_done = 0;
+        }
+        float cum = 0.f;
+        for (int c = 0; c < n; c += FINISH_CHUNK) {
+            __syncthreads();
+            if (s_done) break;
+            const int m = n - c < FINISH_CHUNK ? n - c : FINISH_CHUNK;
+            for (int i = tid; i < m; i += blockDim.x) buf[i] = expf(key_float(k[c + i]) - max_val) * inv;
+            __syncthreads();
+            if (tid == 0) {
+                for (int i = 0; i < m; ++i) {
+                    cum += buf[i];
+                    if (cum >= top_p) {
+                        s_kept = c + i + 1;
+                        s_done = 1;
+                        break;
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        const int kept = s_kept;
+        float sum2 = 0.f;
+        for (int c = 0; c < kept; c += FINISH_CHUNK) {
+            const int m = kept - c < FINISH_CHUNK ? kept - c : FINISH_CHUNK;
+            __syncthreads();
+            for (int i = tid; i < m; i += blockDim.x) buf[i] = expf(key_float(k[c + i]) - max_val) * inv;
+            __syncthreads();
+            if (tid == 0)
+                for (int i = 0; i < m; ++i) sum2 += buf[i];
+        }
+        if (tid == 0) s_inv2 = 1.0f / sum2;
+        __syncthreads();
+    }
+
+    // pass 3: the draw
+    if (tid == 0) {
+        unsigned long long* st = rng + (rng_index ? rng_index[blockIdx.x] : blockIdx.x);
+        s_r = xorshift_next_f32(st);
+        s_done = 0;
+        s_chosen = x[s_kept - 1];
+    }
+    __syncthreads();
+    const int kept = s_kept;
+    const float inv2 = s_inv2;
+    const float r = s_r;
+    const bool renorm = top_p < 1.0f;
+    float cum = 0.f;
+    for (int c = 0; c < kept; c += FINISH_CHUNK) {
+        __syncthreads();
+        if (s_done) break;
+        const int m = kept - c < FINISH_CHUNK ? kept - c : FINISH_CHUNK;
+        for (int i = tid; i < m; i += blockDim.x) {
+            float p = expf(key_float(k[c + i]) - max_val) * inv;
+            if (renorm) p *= inv2;
+            buf[i] = p;
+        }
+        __syncthreads();
+        if (tid == 0) {
+            for (int i = 0; i < m; ++i) {
+                cum += buf[i];
+                if (r < cum) {
+                    s_chosen = x[c + i];
+                    s_done = 1;
+                    break;
+                }
+            }
+        }
+    }
+    __syncthreads();
+    if (tid == 0) out[blockIdx.x] = s_chosen;
+}
+
+// Sample one token per row. temperature > 0. top_k == 0 means no top-k; top_p >= 1 none.
+// scratch_keys / scratch_idx: [R, P2] each, P2 = the power of two >= V, used by the general
+// path only (top_k == 0, top_k >= V or top_k > 1024).
+extern "C" int hb_sample(const float* logits, int ld, int R, int V, float temperature, int top_k,
+                         float top_p, unsigned long long* rng, const int* rng_index, int* out,
+                         uint32_t* scratch_keys, int* scratch_idx, int P2, hipStream_t stream) {
+    HB_REQUIRE(R > 0 && V > 0 && ld >= V, "sample: bad sizes (R=%d, V=%d, ld=%d)", R, V, ld);
+    HB_REQUIRE(temperature > 0.f, "sample: temperature must be > 0 (0 is argmax)");
+    HB_REQUIRE(top_k >= 0, "sample: top_k must be >= 0");
+    const bool k_active = top_k > 0 && top_k < V;
+    if (k_active && top_k <= SAMPLE_MAX_K) {
+        sample_topk_kernel<<<R, SAMPLE_THREADS, 0, stream>>>(logits, ld, V, temperature, top_k, top_p,
+                                                           rng, rng_index, out);
+        HB_CHECK_LAUNCH("sample_topk");
+        return 0;
+    }
+    HB_REQUIRE(scratch_keys && scratch_idx, "sample: this top_k needs the scratch buffers");
+    HB_REQUIRE(P2 >= V && (P2 & (P2 - 1)) == 0, "sample: scratch width %d is no power of two >= %d", P2,
+               V);
+    dim3 pgrid((P2 + 255) / 256, R);
+    sample_prepare_kernel<<<pgrid, 256, 0, stream>>>(logits, ld, V, P2, temperature, scratch_keys,
+                                                     scratch_idx);
+    HB_CHECK_LAUNCH("sample_prepare");
+    const int sorted = (k_active || top_p < 1.0f) ? 1 : 0;
+    if (sorted) {
+        dim3 sgrid((P2 / 2 + 255) / 256, R);
+        for (int size = 2; size <= P2; size <<= 1)
+            for (int stride = size >> 1; stride > 0; stride >>= 1)
+                sample_bitonic_stage_kernel<<<sgrid, 256, 0, stream>>>(scratch_keys, scratch_idx, P2, size,
+                                                                       stride);
+        HB_CHECK_LAUNCH("sample_sort");
+    }
+    const int n = k_active ? top_k : V;
+    sample_finish_kernel<<<R, 1024, 0, stream>>>(scratch_keys, scratch_idx, P2, n, sorted, top_p, rng,
+                                                 rng_index, out);
+    HB_CHECK_LAUNCH("sample_finish");
+    return 0;
+}

@@ -1,0 +1,76 @@
+"""The tokens of one step, packed over the sequences of the batch, with what kernels need
+to find each token's sequence, position and pages."""
+from dataclasses import dataclass
+from typing import List
+
+import numpy as np
+import torch
+
+
+@dataclass
+class StepEntry:
+    """One sequence's share of a step: its slot, its next tokens and the places among
+    them whose logits are wanted."""
+    slot: int
+    tokens: List[int]
+    want: List[int]
+
+
+@dataclass
+class BatchMeta:
+    token_ids: torch.Tensor    # int32 [T]
+    positions: torch.Tensor    # int32 [T]   absolute position of each token in its sequence
+    seq_of: torch.Tensor       # int32 [T]   index of the token's sequence in this batch
+    slots: torch.Tensor        # int32 [B]   slot of each sequence
+    seq_starts: torch.Tensor   # int32 [B+1] first packed row of each sequence
+    context_lens: torch.Tensor  # int32 [B]  positions held after this step
+    want_rows: torch.Tensor    # int32 [R]   packed rows whose logits are wanted
+    num_tokens: int
+    num_seqs: int
+    max_new: int               # most tokens any sequence brings
+    max_context: int           # largest context length after this step
+    max_position: int          # largest absolute position in the step
+    host_starts: np.ndarray    # host copies, for kernels' grids
+    host_context: np.ndarray
+
+
+def pack(entries, start_lengths, device, staging=None):
+    """Build the BatchMeta of a step. start_lengths[i] is what entry i's slot holds already."""
+    B = len(entries)
+    counts = [len(e.tokens) for e in entries]
+    T = sum(counts)
+    R = sum(len(e.want) for e in entries)
+    starts = np.zeros(B + 1, dtype=np.int32)
+    starts[1:] = np.cumsum(counts)
+    total = 3 * T + B + (B + 1) + B + R
+    host = np.empty(total, dtype=np.int32)
+    tok = host[0:T]
+    pos = host[T:2 * T]
+    seq = host[2 * T:3 * T]
+    o = 3 * T
+    slots = host[o:o + B]
+    o += B
+    host[o:o + B + 1] = starts
+    o += B + 1
+    ctx = host[o:o + B]
+    o += B
+    want = host[o:o + R]
+    w = 0
+    for i, e in enumerate(entries):
+        a, b = starts[i], starts[i + 1]
+        tok[a:b] = e.tokens
+        pos[a:b] = np.arange(start_lengths[i], start_lengths[i] + counts[i], dtype=np.int32)
+        seq[a:b] = i
+        slots[i] = e.slot
+        ctx[i] = start_lengths[i] + counts[i]
+        for j in e.want:
+            want[w] = a + j
+            w += 1
+    dev = torch.from_numpy(host).to(device)
+    o = 3 * T
+    return BatchMeta(
+        token_ids=dev[0:T], positions=dev[T:2 * T], seq_of=dev[2 * T:3 * T],
+        slots=dev[o:o + B], seq_starts=dev[o + B:o + 2 * B + 1],
+        context_lens=dev[o + 2 * B + 1:o + 3 * B + 1], want_rows=dev[o + 3 * B + 1:o + 3 * B + 1 + R],
+        num_tokens=T, num_seqs=B, max_new=max(counts), max_context=int(ctx.max()),
+        max_position=int(pos.max()), host_starts=starts.copy(), host_context=ctx.copy())

@@ -1,0 +1,123 @@
+"""The engine: a model on the GPU, its cache, and the one step function.
+
+`step` takes a batch of sequences with unequal numbers of new tokens (whole
+prompts in a batch's first step, one token each afterwards), runs exactly
+those tokens against the cache as one packed batch and returns the float32
+logits at the wanted places. The reference's counterparts are per sequence:
+prefill_with_token, decode_step and verify_draft_tokens
+(crates/backends/backend_common/src/generic_model.rs:131,524,737); its error
+cases are kept: empty input (:139-152), token id >= vocab (:165-171), position
+beyond max_position_embeddings (:531-537).
+"""
+import torch
+
+from ..cache import Cache
+from ..config import load_config
+from ..errors import BackendError, RequestError
+from ..parts import Runtime
+from ..weights import read_tensors
+from . import batch as batching
+from .batch import StepEntry
+from .model import Model
+
+_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16,
+           torch.float32: torch.float32, torch.bfloat16: torch.bfloat16}
+
+
+def require_gpu():
+    if not torch.cuda.is_available():
+        raise BackendError("no GPU: this library runs on a gfx950 GPU only and has no other path")
+    return torch.device("cuda", torch.cuda.current_device())
+
+
+class Engine:
+    def __init__(self, config, spec, tensors, dtype="bfloat16", max_tokens=4096, max_slots=None,
+                 device=None):
+        """tensors: {name: tensor} for the model's needs (any device)."""
+        if dtype not in _DTYPES:
+            raise BackendError(f"dtype must be float32 or bfloat16, got {dtype!r}")
+        self.device = torch.device(device) if device is not None else require_gpu()
+        self.config = config
+        self.spec = spec
+        self.rt = Runtime(_DTYPES[dtype], self.device)
+        self.model = Model(spec)
+        self.model.load(tensors, self.rt)
+        self.cache = Cache(self.model.cache_needs(), max_tokens, spec.max_positions, self.rt.dtype,
+                           self.device, max_slots)
+        self.steps_run = 0
+
+    # ---- construction
+    @classmethod
+    def from_folder(cls, folder, dtype="bfloat16", max_tokens=4096, max_slots=None, device=None):
+        """The engine of the model in `folder` (config.json + safetensors)."""
+        arch, config = load_config(folder)
+        spec = arch.build_spec(config)
+        needs = Model(spec).tensor_needs()
+        tensors = read_tensors(folder, needs)
+        return cls(config, spec, tensors, dtype, max_tokens, max_slots, device)
+
+    @classmethod
+    def from_config(cls, config, architecture=None, seed=0, dtype="bfloat16", weight_dtype=None,
+                    std=0.02, norm_std=0.0, max_tokens=4096, max_slots=None, device=None):
+        """An engine with seeded random weights drawn on the GPU (no files)."""
+        from ..config.registry import resolve_architecture
+        from ..weights import random_tensors
+        arch = architecture or resolve_architecture(config.to_dict())
+        spec = arch.build_spec(config)
+        dev = torch.device(device) if device is not None else require_gpu()
+        needs = Model(spec).tensor_needs()
+        tensors = random_tensors(needs, seed, weight_dtype or dtype, std, norm_std, device=str(dev))
+        return cls(config, spec, tensors, dtype, max_tokens, max_slots, dev)
+
+    # ---- slots
+    def alloc_slot(self):
+        return self.cache.alloc_slot()
+
+    def free_slot(self, slot):
+        self.cache.free_slot(slot)
+
+    # ---- the step
+    def step(self, entries):
+        """Run the entries' tokens; returns float32 logits [wanted, vocab] on the GPU
+        (rows in the order of the entries and of their `want`), or None if nothing is wanted."""
+        if not entries:
+            raise RequestError("a step needs at least one sequence")
+        vocab = self.spec.vocab_size
+        seen = set()
+        starts = []
+        for e in entries:
+            if e.slot in seen:
+                raise RequestError(f"slot {e.slot} appears twice in one step")
+            seen.add(e.slot)
+            if len(e.tokens) == 0:
+                raise RequestError("a sequence of a step has no tokens")
+            for t in e.tokens:
+                if not 0 <= int(t) < vocab:
+                    raise RequestError(f"token id {t} out of range (vocab_size {vocab})")
+            for j in e.want:
+                if not 0 <= int(j) < len(e.tokens):
+                    raise RequestError(f"wanted place {j} is outside the sequence's "
+                                       f"{len(e.tokens)} tokens")
+            start = self.cache.length(e.slot)
+            if start + len(e.tokens) > self.spec.max_positions:
+                raise RequestError(f"sequence of {start + len(e.tokens)} tokens exceeds "
+                                   f"max_position_embeddings ({self.spec.max_positions})")
+            starts.append(start)
+        for e in entries:
+            self.cache.reserve(e.slot, len(e.tokens))
+        meta = batching.pack(entries, starts, self.device)
+        logits = self.model.forward(self.rt, meta, self.cache)
+        for e in entries:
+            self.cache.commit(e.slot, len(e.tokens))
+        self.steps_run += 1
+        return logits
+
+    def get_tensor(self, name):
+        """A weight as the engine holds it (by the name of the weight files)."""
+        for part in self.model._weight_parts():
+            got = getattr(part, "get_tensor", None)
+            if got is not None:
+                t = got(name)
+                if t is not None:
+                    return t
+        raise KeyError(name)

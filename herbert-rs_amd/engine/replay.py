@@ -1,0 +1,72 @@
+"""Trace replay: feed given token ids through the engine step by step and write logits.
+
+It samples nothing and has no forward pass, cache or loader of its own: every
+step goes through `Engine.step`, the function that generation uses. Input is
+one JSON object per line on standard input:
+
+    {"step": 0, "entries": [{"id": "a", "tokens": [5, 17, 3], "want": [0, 2]}], "end": []}
+
+For a step that wants something, `<out>/<step>.f32` holds the float32 logits
+[wanted, vocab] (little-endian) in the order of the entries and of `want`.
+After each step a line `done <step>` is printed and flushed.
+"""
+import argparse
+import json
+import os
+import sys
+
+import numpy as np
+
+from ..errors import HerbertError, RequestError
+from .batch import StepEntry
+from .engine import Engine
+
+
+class Replayer:
+    def __init__(self, engine, out_dir):
+        self.engine = engine
+        self.out_dir = out_dir
+        self.slots = {}
+        os.makedirs(out_dir, exist_ok=True)
+
+    def run_step(self, record):
+        step = record["step"]
+        entries = []
+        for e in record.get("entries", []):
+            rid = e["id"]
+            if rid not in self.slots:
+                self.slots[rid] = self.engine.alloc_slot()
+            entries.append(StepEntry(self.slots[rid], list(e["tokens"]), list(e.get("want", []))))
+        if entries:
+            logits = self.engine.step(entries)
+            if logits is not None:
+                arr = logits.detach().to("cpu").numpy().astype("<f4", copy=False)
+                arr.tofile(os.path.join(self.out_dir, f"{step}.f32"))
+        for rid in record.get("end", []):
+            if rid not in self.slots:
+                raise RequestError(f"request {rid!r} ends but never started")
+            self.engine.free_slot(self.slots.pop(rid))
+        return step
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser(prog="trace_run", description=__doc__.split("\n\n")[0])
+    ap.add_argument("--model", required=True, help="folder with config.json and model.safetensors")
+    ap.add_argument("--dtype", required=True, choices=["bfloat16", "float32"])
+    ap.add_argument("--out", required=True, help="folder for <step>.f32 files")
+    ap.add_argument("--max-tokens", type=int, required=True,
+                    help="most tokens live requests hold at any time (each rounded up to 64)")
+    args = ap.parse_args(argv)
+    try:
+        engine = Engine.from_folder(args.model, dtype=args.dtype, max_tokens=args.max_tokens)
+        replayer = Replayer(engine, args.out)
+        for line in sys.stdin:
+            line = line.strip()
+            if not line:
+                continue
+            step = replayer.run_step(json.loads(line))
+            print(f"done {step}", flush=True)
+    except HerbertError as e:
+        print(f"trace_run: {e}", file=sys.stderr, flush=True)
+        return 1
+    return 0

@@ -1,0 +1,192 @@
+"""Host side of every kernel: operand checks, then the launch.
+
+Each function checks on the host that shapes, dtypes, devices and layouts are
+what the kernel and its grid assume, and only then launches on the current
+HIP stream. There is no fallback of any kind behind them.
+"""
+import torch
+
+from ..errors import BackendError
+from . import lib
+
+F32 = 0
+BF16 = 1
+_CODES = {torch.float32: F32, torch.bfloat16: BF16}
+
+
+def dtype_code(t):
+    try:
+        return _CODES[t.dtype]
+    except KeyError:
+        raise BackendError(f"dtype {t.dtype} is not supported by the kernels") from None
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _check(t, name, dtype=None, shape=None):
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise BackendError(f"{name} must be a tensor on the GPU")
+    if not t.is_contiguous():
+        raise BackendError(f"{name} must be contiguous")
+    if dtype is not None and t.dtype != dtype:
+        raise BackendError(f"{name} must be {dtype}, got {t.dtype}")
+    if shape is not None:
+        if len(shape) != t.dim() or any(s is not None and s != d for s, d in zip(shape, t.shape)):
+            raise BackendError(f"{name} must have shape {list(shape)}, got {list(t.shape)}")
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def embed(ids, table, out):
+    """out[t, :] = table[ids[t], :] as float32. ids int32 [T], table [V, H], out f32 [T, H]."""
+    T = ids.shape[0]
+    _check(ids, "ids", torch.int32, (T,))
+    _check(table, "table", None, (None, None))
+    H = table.shape[1]
+    _check(out, "out", torch.float32, (T, H))
+    lib.call("elementwise", "hb_embed", ids.data_ptr(), table.data_ptr(), dtype_code(table),
+             out.data_ptr(), T, H, _stream())
+
+
+def rmsnorm(x, weight, out, eps, rows=None):
+    """out[r] = rmsnorm(x[rows[r]] or x[r]) * weight. x f32 [T, H], weight f32 [H]."""
+    _check(x, "x", torch.float32, (None, None))
+    H = x.shape[1]
+    _check(weight, "weight", torch.float32, (H,))
+    if rows is not None:
+        _check(rows, "rows", torch.int32, (None,))
+        R = rows.shape[0]
+    else:
+        R = x.shape[0]
+    _check(out, "out", None, (R, H))
+    lib.call("elementwise", "hb_rmsnorm", x.data_ptr(), weight.data_ptr(), out.data_ptr(),
+             dtype_code(out), _ptr(rows), R, H, float(eps), _stream())
+
+
+def gemm_plain(a, w, c, accumulate=False):
+    """c[M, N] (+)= a[M, K] @ w[N, K]^T in float32 arithmetic, any of f32 / bf16 storage."""
+    _check(a, "a", None, (None, None))
+    _check(w, "w", None, (None, None))
+    M, K = a.shape
+    N = w.shape[0]
+    if w.shape[1] != K:
+        raise BackendError(f"gemm: a is [{M}, {K}] but w is {list(w.shape)}")
+    _check(c, "c", None, (M, N))
+    if accumulate and c.dtype != torch.float32:
+        raise BackendError("gemm: accumulation needs a float32 output")
+    lib.call("gemm_plain", "hb_gemm_plain", a.data_ptr(), dtype_code(a), w.data_ptr(), dtype_code(w),
+             c.data_ptr(), dtype_code(c), M, N, K, K, K, N, 1 if accumulate else 0, _stream())
+
+
+def _check_paged(meta, cache, T):
+    _check(meta.positions, "positions", torch.int32, (T,))
+    _check(meta.seq_of, "seq_of", torch.int32, (T,))
+    _check(meta.slots, "slots", torch.int32, (None,))
+    _check(cache.page_table, "page_table", torch.int32, (None, None))
+    _check(cache.k, "key pages", None, (None, None, cache.page_size, None))
+    _check(cache.v, "value pages", cache.k.dtype, tuple(cache.k.shape))
+
+
+def qk_norm_rope_write(qkv, q_norm_w, k_norm_w, cos, sin, rot_dims, meta, cache, q_out, nq, nkv, hd, eps,
+                       write_kv=True):
+    """Per-head norm (if weights given), rotation (if tables given), q to q_out, k / v to the pages.
+
+    qkv f32 [T, (nq + 2 nkv) hd] (query heads only when write_kv is false); cos / sin f32 [max_pos, rot_dims / 2]; q_out [T, nq hd] in the
+    cache's dtype; cache.k / cache.v [pages, nkv, page_size, hd].
+    """
+    T = qkv.shape[0]
+    _check(qkv, "qkv", torch.float32, (T, (nq + (2 * nkv if write_kv else 0)) * hd))
+    _check_paged(meta, cache, T)
+    _check(q_out, "q_out", cache.k.dtype, (T, nq * hd))
+    if tuple(cache.k.shape[1:]) != (nkv, cache.page_size, hd):
+        raise BackendError(f"cache pages {list(cache.k.shape)} do not fit {nkv} kv heads of {hd}")
+    for w, name in ((q_norm_w, "q_norm"), (k_norm_w, "k_norm")):
+        if w is not None:
+            _check(w, name, torch.float32, (hd,))
+    if cos is not None:
+        _check(cos, "cos", torch.float32, (None, rot_dims // 2))
+        _check(sin, "sin", torch.float32, tuple(cos.shape))
+        if meta.max_position >= cos.shape[0]:
+            raise BackendError(f"position {meta.max_position} beyond the rotation table "
+                               f"({cos.shape[0]} rows)")
+    lib.call("elementwise", "hb_qk_norm_rope_write", qkv.data_ptr(), qkv.shape[1], _ptr(q_norm_w),
+             _ptr(k_norm_w), _ptr(cos), _ptr(sin), rot_dims, meta.positions.data_ptr(),
+             meta.seq_of.data_ptr(), meta.slots.data_ptr(), cache.page_table.data_ptr(),
+             cache.page_table.shape[1], cache.page_size, q_out.data_ptr(), cache.k.data_ptr(),
+             cache.v.data_ptr(), dtype_code(q_out), T, nq, nkv, hd, float(eps), 1 if write_kv else 0,
+             _stream())
+
+
+def attention_plain(q, meta, cache, out, nq, nkv, hd, scale, window):
+    """Causal (and windowed) attention of every token over its slot's pages."""
+    T = q.shape[0]
+    _check(q, "q", cache.k.dtype, (T, nq * hd))
+    _check(out, "out", cache.k.dtype, (T, nq * hd))
+    _check_paged(meta, cache, T)
+    if tuple(cache.k.shape[1:]) != (nkv, cache.page_size, hd):
+        raise BackendError(f"cache pages {list(cache.k.shape)} do not fit {nkv} kv heads of {hd}")
+    lib.call("attention_plain", "hb_attention_plain", q.data_ptr(), cache.k.data_ptr(),
+             cache.v.data_ptr(), out.data_ptr(), dtype_code(q), meta.positions.data_ptr(),
+             meta.seq_of.data_ptr(), meta.slots.data_ptr(), cache.page_table.data_ptr(),
+             cache.page_table.shape[1], cache.page_size, T, nq, nkv, hd, float(scale),
+             int(window or 0), _stream())
+
+
+def swiglu(gu, out):
+    """out[t, i] = silu(gu[t, i]) * gu[t, I + i]; gu f32 [T, 2I]."""
+    _check(gu, "gate_up", torch.float32, (None, None))
+    T, two_i = gu.shape
+    if two_i % 2:
+        raise BackendError("swiglu: the input's width must be even")
+    _check(out, "out", None, (T, two_i // 2))
+    lib.call("elementwise", "hb_swiglu", gu.data_ptr(), out.data_ptr(), dtype_code(out), T, two_i // 2,
+             _stream())
+
+
+def fill_u32(t, value):
+    """Set every 32-bit word of a tensor (through a kernel, safe inside a captured graph)."""
+    _check(t, "tensor")
+    nbytes = t.numel() * t.element_size()
+    if nbytes % 4:
+        raise BackendError("fill: the tensor's size is no multiple of 4 bytes")
+    lib.call("elementwise", "hb_fill_u32", t.data_ptr(), int(value), nbytes // 4, _stream())
+
+
+def argmax(logits, out):
+    """out[r] = first index of the largest value of logits[r]; logits f32 [R, V], out int32 [R]."""
+    _check(logits, "logits", torch.float32, (None, None))
+    R, V = logits.shape
+    _check(out, "out", torch.int32, (R,))
+    lib.call("sampling", "hb_argmax", logits.data_ptr(), V, R, V, out.data_ptr(), _stream())
+
+
+def sample(logits, temperature, top_k, top_p, rng_states, rng_index, out, scratch=None):
+    """One token per row by temperature / top-k / top-p; rng_states int64 [n], advanced in place.
+
+    `scratch` = (keys int32 [R, P2], idx int32 [R, P2]) with P2 the power of two >= V; needed
+    unless 0 < top_k <= 1024 and top_k < V.
+    """
+    _check(logits, "logits", torch.float32, (None, None))
+    R, V = logits.shape
+    _check(out, "out", torch.int32, (R,))
+    _check(rng_states, "rng_states", torch.int64, (None,))
+    if rng_index is not None:
+        _check(rng_index, "rng_index", torch.int32, (R,))
+    elif rng_states.shape[0] < R:
+        raise BackendError("sample: fewer generator states than rows")
+    keys = idx = None
+    p2 = 0
+    if scratch is not None:
+        keys, idx = scratch
+        p2 = keys.shape[1]
+        _check(keys, "scratch keys", torch.int32, (None, p2))
+        _check(idx, "scratch idx", torch.int32, tuple(keys.shape))
+        if keys.shape[0] < R:
+            raise BackendError("sample: scratch has fewer rows than the logits")
+    lib.call("sampling", "hb_sample", logits.data_ptr(), V, R, V, float(temperature), int(top_k),
+             float(top_p), rng_states.data_ptr(), _ptr(rng_index), out.data_ptr(), _ptr(keys),
+             _ptr(idx), p2, _stream())

@@ -1,0 +1,64 @@
+"""Qwen3ForCausalLM as data: which parts each layer has and what its tensors are called.
+
+Tensor names are those of the weight files as the reference classifies them
+(crates/backends/backend_common/src/loader_common.rs:453-566). Fixed for this
+family in the reference and therefore here: per-head q/k RMSNorm on, no biases
+(crates/core/src/config.rs:508-512), plain RMSNorm (:514), SwiGLU
+(loader_common.rs:853), rotation on every layer over the whole head
+(loader_common.rs:978; config.rs:518-525), scale 1/sqrt(head_dim)
+(loader_common.rs:1003-1005).
+"""
+from ..config import Qwen3Config, register_architecture
+from ..parts import LayerSpec, ModelSpec, PartSpec, ScheduleEntry
+
+
+def build_spec(cfg):
+    position = PartSpec("rope", {"theta": cfg.rope_theta, "rotary_dims": cfg.head_dim,
+                                 "max_positions": cfg.max_position_embeddings})
+    layers = []
+    for i in range(cfg.num_hidden_layers):
+        p = f"model.layers.{i}."
+        mixer = PartSpec("attention", {
+            "hidden_size": cfg.hidden_size,
+            "num_heads": cfg.num_attention_heads,
+            "num_kv_heads": cfg.num_key_value_heads,
+            "head_dim": cfg.head_dim,
+            "eps": cfg.rms_norm_eps,
+            "qk_norm": True,
+            "window": cfg.layer_windows[i],
+            "position": position,
+            "names": {"q": p + "self_attn.q_proj.weight", "k": p + "self_attn.k_proj.weight",
+                      "v": p + "self_attn.v_proj.weight", "o": p + "self_attn.o_proj.weight",
+                      "q_norm": p + "self_attn.q_norm.weight", "k_norm": p + "self_attn.k_norm.weight"},
+        })
+        ffn = PartSpec("swiglu", {
+            "hidden_size": cfg.hidden_size,
+            "intermediate_size": cfg.intermediate_size,
+            "names": {"gate": p + "mlp.gate_proj.weight", "up": p + "mlp.up_proj.weight",
+                      "down": p + "mlp.down_proj.weight"},
+        })
+        norms = {
+            "input": PartSpec("rmsnorm", {"size": cfg.hidden_size, "eps": cfg.rms_norm_eps,
+                                          "weight": p + "input_layernorm.weight"}),
+            "post_mixer": PartSpec("rmsnorm", {"size": cfg.hidden_size, "eps": cfg.rms_norm_eps,
+                                               "weight": p + "post_attention_layernorm.weight"}),
+        }
+        layers.append(LayerSpec(PartSpec("prenorm"), mixer, ffn, norms))
+    return ModelSpec(
+        hidden_size=cfg.hidden_size,
+        vocab_size=cfg.vocab_size,
+        max_positions=cfg.max_position_embeddings,
+        embedding=PartSpec("table", {"vocab_size": cfg.vocab_size, "hidden_size": cfg.hidden_size,
+                                     "weight": "model.embed_tokens.weight"}),
+        layers=layers,
+        schedule=[ScheduleEntry(i) for i in range(cfg.num_hidden_layers)],
+        final_norm=PartSpec("rmsnorm", {"size": cfg.hidden_size, "eps": cfg.rms_norm_eps,
+                                        "weight": "model.norm.weight"}),
+        head=PartSpec("linear", {"vocab_size": cfg.vocab_size, "hidden_size": cfg.hidden_size,
+                                 "weight": "lm_head.weight",
+                                 "tied_to_embedding": cfg.tie_word_embeddings}),
+        eos_token_id=cfg.eos_token_id,
+    )
+
+
+ARCHITECTURE = register_architecture("Qwen3ForCausalLM", Qwen3Config, build_spec, model_types=("qwen3",))

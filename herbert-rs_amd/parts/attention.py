@@ -1,0 +1,111 @@
+"""Grouped-query attention over the paged cache.
+
+Formulas as the reference computes them (`bc/` = crates/backends/backend_common/src/):
+q, k, v projections without bias (bc/generic_attention/prefill/mod.rs:73-77),
+optional RMSNorm of every head with one weight [head_dim]
+(bc/generic_attention/mod.rs:62-76), rotation at absolute positions
+(prefill/mod.rs:189-210), keys and values appended to the cache (:232), scores
+scaled by 1/sqrt(head_dim) (bc/generic_attention/decode.rs:126), consecutive
+query heads sharing a kv head (decode.rs:131-140), causal by count
+(prefill/kernel_f32.rs:65-67), output projection added to the residual
+(prefill/mod.rs:293, bc/generic_layer.rs:1234-1236).
+A window (keys of the last `window` positions only) is a parameter that the
+reference does not have.
+"""
+import math
+
+import torch
+
+from ..cache import KVNeed
+from ..kernels import ops
+from ..weights import TensorNeed
+from .base import Part
+from .linear import Linear
+from .registry import register
+
+
+@register("mixer", "attention")
+class Attention(Part):
+    def __init__(self, hidden_size, num_heads, num_kv_heads, head_dim, eps, position, names,
+                 qk_norm=True, window=None, scale=None, shared=None, reads_cache_only=False):
+        """names: dict with q, k, v, o (and q_norm, k_norm when qk_norm) -> tensor names.
+        reads_cache_only: the part has no k / v projections and attends over a cache that
+        another entry of the schedule fills."""
+        if num_heads % num_kv_heads:
+            raise ValueError("num_heads must be divisible by num_kv_heads")
+        self.hidden_size = int(hidden_size)
+        self.nq = int(num_heads)
+        self.nkv = int(num_kv_heads)
+        self.hd = int(head_dim)
+        self.eps = float(eps)
+        self.qk_norm = bool(qk_norm)
+        self.window = int(window) if window else None
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.hd)
+        self.names = dict(names)
+        self.reads_cache_only = bool(reads_cache_only)
+        self.position = shared.position(position)
+        self.qkv = self.o = self.q_norm_w = self.k_norm_w = None
+
+    @property
+    def q_dim(self):
+        return self.nq * self.hd
+
+    @property
+    def kv_dim(self):
+        return self.nkv * self.hd
+
+    def tensor_needs(self):
+        n = self.names
+        needs = {n["q"]: TensorNeed((self.q_dim, self.hidden_size)),
+                 n["o"]: TensorNeed((self.hidden_size, self.q_dim))}
+        if not self.reads_cache_only:
+            needs[n["k"]] = TensorNeed((self.kv_dim, self.hidden_size))
+            needs[n["v"]] = TensorNeed((self.kv_dim, self.hidden_size))
+        if self.qk_norm:
+            needs[n["q_norm"]] = TensorNeed((self.hd,), "scale")
+            if not self.reads_cache_only:
+                needs[n["k_norm"]] = TensorNeed((self.hd,), "scale")
+        return needs
+
+    def cache_need(self):
+        if self.reads_cache_only:
+            return None
+        return KVNeed(self.nkv, self.hd, self.window)
+
+    def load(self, tensors, rt):
+        n = self.names
+        rows = [tensors[n["q"]]]
+        if not self.reads_cache_only:
+            rows += [tensors[n["k"]], tensors[n["v"]]]
+        # one fused projection [q rows | k rows | v rows]: the activations are read once
+        self.qkv = Linear(rt.weight(torch.cat([r.to(rt.device) for r in rows], 0)))
+        self.o = Linear(rt.weight(tensors[n["o"]]))
+        if self.qk_norm:
+            self.q_norm_w = rt.weight(tensors[n["q_norm"]], matrix=False)
+            if not self.reads_cache_only:
+                self.k_norm_w = rt.weight(tensors[n["k_norm"]], matrix=False)
+
+    def forward(self, ctx, y, x):
+        rt = ctx.rt
+        T = y.shape[0]
+        kv = ctx.cache.kv_view(ctx.cache_entry)
+        write_kv = not self.reads_cache_only
+        width = self.q_dim + (2 * self.kv_dim if write_kv else 0)
+        qkv = rt.buffer("qkv", (T, width), torch.float32)
+        self.qkv.forward(y, qkv)
+        q = rt.buffer("q", (T, self.q_dim))
+        rot = self.position.rotation()
+        cos, sin, rot_dims = rot if rot is not None else (None, None, 0)
+        ops.qk_norm_rope_write(qkv, self.q_norm_w, self.k_norm_w, cos, sin, rot_dims, ctx.meta, kv, q,
+                               self.nq, self.nkv, self.hd, self.eps, write_kv=write_kv)
+        attn = rt.buffer("attn", (T, self.q_dim))
+        self.attend(ctx, q, kv, attn)
+        self.o.forward(attn, x, accumulate=True)
+
+    def attend(self, ctx, q, kv, out):
+        if q.dtype == torch.bfloat16:
+            from ..kernels import mfma
+            if mfma.attention_supported(q, kv, self.nq, self.nkv, self.hd):
+                mfma.attention(q, ctx.meta, kv, out, self.nq, self.nkv, self.hd, self.scale, self.window)
+                return
+        ops.attention_plain(q, ctx.meta, kv, out, self.nq, self.nkv, self.hd, self.scale, self.window)

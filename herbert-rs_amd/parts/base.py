@@ -1,0 +1,81 @@
+"""What every part has in common, and the context a step hands to the parts.
+
+Interfaces (x is the float32 residual stream [T, hidden], y a normed copy of it
+in the compute dtype; T counts the tokens of the step, packed over sequences):
+
+  norm          forward(ctx, x, rows=None) -> y            (rows: gather these rows only)
+  mixer         forward(ctx, y, x)                         adds its output to x
+  feed_forward  forward(ctx, y, x)                         adds its output to x
+  position      rotation() -> (cos, sin, rotary_dims) or None, tables on the GPU
+  block         forward(ctx, x)                            runs one layer on x in place
+  embedding     forward(ctx, token_ids) -> x
+  head          forward(ctx, x, rows) -> float32 logits [len(rows), vocab]
+
+Every part also has
+  tensor_needs() -> {tensor name: TensorNeed}   the tensors it reads from the weight files
+  load(tensors, rt)                             take them (converted as its kernels need)
+and a mixer has
+  cache_need() -> None, KVNeed, StateNeed or a tuple of them.
+"""
+from dataclasses import dataclass
+from typing import Any
+
+import torch
+
+
+class Part:
+    kind = "?"
+
+    def tensor_needs(self):
+        return {}
+
+    def load(self, tensors, rt):
+        pass
+
+    def cache_need(self):
+        return None
+
+
+class Runtime:
+    """Compute dtype, device and the scratch buffers that all layers share."""
+
+    def __init__(self, dtype, device):
+        if dtype not in (torch.float32, torch.bfloat16):
+            raise ValueError("compute dtype must be float32 or bfloat16")
+        self.dtype = dtype
+        self.device = torch.device(device)
+        self._buffers = {}
+
+    @property
+    def exact(self):
+        """True in the all-float32 mode."""
+        return self.dtype == torch.float32
+
+    def buffer(self, name, shape, dtype=None):
+        """A scratch tensor of at least this size, reused from call to call under its name."""
+        dtype = dtype or self.dtype
+        n = 1
+        for s in shape:
+            n *= int(s)
+        key = (name, dtype)
+        buf = self._buffers.get(key)
+        if buf is None or buf.numel() < n:
+            buf = torch.empty(max(n, 1), dtype=dtype, device=self.device)
+            self._buffers[key] = buf
+        return buf[:n].view(*shape)
+
+    def weight(self, t, matrix=True):
+        """A stored tensor as the kernels read it: matrices in the compute dtype, scales in float32."""
+        t = t.to(self.device)
+        return t.to(self.dtype if matrix else torch.float32).contiguous()
+
+
+@dataclass
+class StepContext:
+    """What one step hands down to the parts."""
+    rt: Runtime
+    meta: Any            # engine.batch.BatchMeta
+    cache: Any           # cache.Cache
+    entry: int = 0       # the schedule entry that is running
+    cache_entry: int = 0  # the entry whose cache it uses
+    owns_cache: bool = True

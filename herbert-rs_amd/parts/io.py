@@ -1,0 +1,65 @@
+"""The two ends of a model: the embedding table and the output head.
+
+Embedding without multiplier (crates/backends/backend_common/src/generic_model.rs:104-111);
+the head is the final norm of the wanted rows only and a product with
+lm_head, or with the embedding table when the two are tied
+(generic_model.rs:266-283; loader_common.rs:1851-1872).
+"""
+import torch
+
+from ..kernels import ops
+from ..weights import TensorNeed
+from .base import Part
+from .linear import Linear
+from .registry import register
+
+
+@register("embedding", "table")
+class TokenEmbedding(Part):
+    def __init__(self, vocab_size, hidden_size, weight, shared=None):
+        self.vocab_size = int(vocab_size)
+        self.hidden_size = int(hidden_size)
+        self.weight_name = weight
+        self.table = None
+
+    def tensor_needs(self):
+        return {self.weight_name: TensorNeed((self.vocab_size, self.hidden_size), "table")}
+
+    def load(self, tensors, rt):
+        self.table = rt.weight(tensors[self.weight_name])
+
+    def forward(self, ctx, token_ids):
+        x = ctx.rt.buffer("residual", (token_ids.shape[0], self.hidden_size), torch.float32)
+        ops.embed(token_ids, self.table, x)
+        return x
+
+
+@register("head", "linear")
+class OutputHead(Part):
+    def __init__(self, vocab_size, hidden_size, weight, tied_to_embedding, norm, shared=None):
+        """weight: the head's tensor name; tied_to_embedding: use the embedding table instead."""
+        self.vocab_size = int(vocab_size)
+        self.hidden_size = int(hidden_size)
+        self.weight_name = weight
+        self.tied = bool(tied_to_embedding)
+        self.norm = norm                  # a built norm part
+        self.proj = None
+
+    def tensor_needs(self):
+        needs = dict(self.norm.tensor_needs())
+        if not self.tied:
+            needs[self.weight_name] = TensorNeed((self.vocab_size, self.hidden_size))
+        return needs
+
+    def load(self, tensors, rt, embedding=None):
+        self.norm.load(tensors, rt)
+        if self.tied:
+            self.proj = Linear(embedding.table)
+        else:
+            self.proj = Linear(rt.weight(tensors[self.weight_name]))
+
+    def forward(self, ctx, x, rows):
+        y = self.norm.forward(ctx, x, rows, name="head_normed")
+        logits = torch.empty((rows.shape[0], self.vocab_size), dtype=torch.float32, device=x.device)
+        self.proj.forward(y, logits)
+        return logits

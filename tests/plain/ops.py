@@ -1,0 +1,166 @@
+"""Plain, slow, whole-sequence formulas of the dense Qwen3 decoder.
+
+One function for each part, written from the reference's text (paths are
+relative to the reference's root; `bc/` = crates/backends/backend_common/src/).
+No cache, no batching, no code shared with the engine. Everything runs on the
+CPU in the dtype of its inputs (float32 by default, float64 to judge rounding).
+"""
+import math
+
+import torch
+
+
+def embedding(ids, table):
+    """x_t = E[id_t, :], no multiplier; an id >= vocab is an error.
+
+    bc/generic_model.rs:104-111 (lookup), :165-171 (range check).
+    """
+    vocab = table.shape[0]
+    rows = []
+    for t in ids:
+        t = int(t)
+        if t < 0 or t >= vocab:
+            raise ValueError(f"token id {t} out of range (vocab_size {vocab})")
+        rows.append(table[t])
+    return torch.stack(rows, 0)
+
+
+def rms_norm(x, weight, eps):
+    """y_i = x_i * 1/sqrt(sum(x^2)/dim + eps) * w_i over the last axis.
+
+    bc/kernels.rs:54-64: eps is added to the mean inside the square root, the
+    weight multiplies afterwards and is used as it is (not 1 + w).
+    """
+    dim = x.shape[-1]
+    sum_sq = (x * x).sum(-1, keepdim=True)
+    inv_rms = 1.0 / torch.sqrt(sum_sq / dim + eps)
+    return x * inv_rms * weight
+
+
+def linear(x, weight):
+    """C[m, n] = sum_k A[m, k] * W[n, k]; weights are [out, in], no bias.
+
+    crates/backends/backend_bf16/src/kernels.rs:154-164.
+    """
+    out = torch.zeros(x.shape[0], weight.shape[0], dtype=x.dtype)
+    for n in range(weight.shape[0]):
+        out[:, n] = (x * weight[n]).sum(-1)
+    return out
+
+
+def split_heads(x, num_heads, head_dim):
+    """Row layout [head0(hd) | head1(hd) | ...] -> [T, heads, hd].
+
+    bc/generic_attention/mod.rs:63-65 (offset = h * head_dim).
+    """
+    assert x.shape[-1] == num_heads * head_dim
+    return x.reshape(x.shape[0], num_heads, head_dim)
+
+
+def head_rms_norm(x, weight, eps):
+    """RMSNorm of each head vector alone, one weight [hd] for all heads.
+
+    bc/generic_attention/mod.rs:62-76; x is [T, heads, hd].
+    """
+    out = torch.empty_like(x)
+    for h in range(x.shape[1]):
+        out[:, h] = rms_norm(x[:, h], weight, eps)
+    return out
+
+
+def rope_inv_freq(rotary_ndims, theta):
+    """inv_freq_i = 1 / theta^(2i / R) in float32, i in [0, R/2).
+
+    bc/loader_common.rs:185-188.
+    """
+    theta32 = torch.tensor(theta, dtype=torch.float32)
+    i2 = torch.arange(0, rotary_ndims // 2, dtype=torch.float32) * 2.0
+    return 1.0 / torch.pow(theta32, i2 / float(rotary_ndims))
+
+
+def rope_tables(positions, rotary_ndims, theta):
+    """cos/sin of ang = float32(pos) * inv_freq_i, the angle itself in float32.
+
+    bc/loader_common.rs:193-199.
+    """
+    inv = rope_inv_freq(rotary_ndims, theta)
+    pos = torch.as_tensor(positions, dtype=torch.float32)
+    ang = pos[:, None] * inv[None, :]
+    return torch.cos(ang), torch.sin(ang)
+
+
+def apply_rope(x, positions, theta, rotary_ndims=None):
+    """Half-split rotation: pairs (j, j + R/2); dims >= R stay.
+
+    bc/kernels.rs:739-759: u_j = x0*c - x1*s ; u_{j+R/2} = x0*s + x1*c.
+    x is [T, heads, hd]; positions are absolute indices in the sequence.
+    """
+    hd = x.shape[-1]
+    rot = hd if rotary_ndims is None else rotary_ndims
+    half = rot // 2
+    cos, sin = rope_tables(positions, rot, theta)
+    cos = cos.to(x.dtype)[:, None, :]
+    sin = sin.to(x.dtype)[:, None, :]
+    out = x.clone()
+    x0 = x[..., :half]
+    x1 = x[..., half:rot]
+    out[..., :half] = x0 * cos - x1 * sin
+    out[..., half:rot] = x0 * sin + x1 * cos
+    return out
+
+
+def causal_attention(q, k, v, positions, scale=None, window=None):
+    """Scores, causal mask by count, softmax, PV; consecutive query heads share a kv head.
+
+    q [T, nq, hd], k/v [T, nkv, hd] of ONE whole sequence whose token t sits at
+    positions[t] (ascending). Query at position p sees the keys at positions <= p
+    (bc/generic_attention/prefill/kernel_f32.rs:65-67), kv head = h / (nq / nkv)
+    (bc/generic_attention/decode.rs:131-140), scale = 1/sqrt(hd)
+    (bc/generic_attention/decode.rs:126), softmax with the maximum taken off
+    (bc/kernels.rs:716-731), out = sum_j p_j v_j (bc/attention_common.rs:160-177).
+
+    `window` is no part of the reference (it never reads a window); when given,
+    a query at p sees only keys with p - window < position <= p.
+    """
+    T, nq, hd = q.shape
+    nkv = k.shape[1]
+    assert nq % nkv == 0
+    group = nq // nkv
+    if scale is None:
+        scale = 1.0 / math.sqrt(hd)
+    out = torch.zeros_like(q)
+    for h in range(nq):
+        g = h // group
+        for i in range(T):
+            p = int(positions[i])
+            keys = [j for j in range(T) if int(positions[j]) <= p
+                    and (window is None or int(positions[j]) > p - window)]
+            kk = k[keys, g]
+            vv = v[keys, g]
+            s = (kk * q[i, h]).sum(-1) * scale
+            m = s.max()
+            e = torch.exp(s - m)
+            total = e.sum()
+            prob = e / total if total > 0 else e
+            out[i, h] = (prob[:, None] * vv).sum(0)
+    return out
+
+
+def silu(x):
+    """x / (1 + exp(-x)); bc/kernels.rs:676-679."""
+    return x / (1.0 + torch.exp(-x))
+
+
+def swiglu_mlp(x, w_gate, w_up, w_down):
+    """down(silu(gate(x)) * up(x)); bc/generic_mlp.rs:83-96, bc/kernels.rs:681-687."""
+    g = linear(x, w_gate)
+    u = linear(x, w_up)
+    return linear(silu(g) * u, w_down)
+
+
+def softmax(x):
+    """bc/kernels.rs:716-731 (whole vector, guard sum > 0)."""
+    m = x.max()
+    e = torch.exp(x - m)
+    s = e.sum()
+    return e / s if s > 0 else e

@@ -1,0 +1,25 @@
+"""Logits of the plain implementation for a model folder and a token list, computed once."""
+import numpy as np
+import torch
+
+from .plain import model as plain_model
+
+_folders = {}
+_logits = {}
+
+
+def plain_logits(folder, tokens):
+    """float32 array [len(tokens), vocab] from the plain whole-sequence forward pass."""
+    key = (folder, tuple(tokens))
+    if key not in _logits:
+        if folder not in _folders:
+            _folders[folder] = plain_model.read_folder(folder, torch.float32)
+        cfg, w = _folders[folder]
+        _logits[key] = plain_model.forward(cfg, w, list(tokens)).numpy().astype(np.float32)
+    return _logits[key]
+
+
+def plain_folder(folder):
+    if folder not in _folders:
+        _folders[folder] = plain_model.read_folder(folder, torch.float32)
+    return _folders[folder]
