@@ -6,6 +6,9 @@ from .errors import (BackendError, CacheError, ConfigError, HerbertError, ModelL
 from . import config, weights, cache, parts, models
 from .config import Qwen3Config, load_config, register_architecture
 from .engine import Engine, StepEntry
+from .sampling import SamplingParams
+from .api import generate, load, write_random_model
 
 __all__ = ["BackendError", "CacheError", "ConfigError", "Engine", "HerbertError", "ModelLoadError",
-           "Qwen3Config", "RequestError", "StepEntry", "load_config", "register_architecture"]
+           "Qwen3Config", "RequestError", "SamplingParams", "StepEntry", "generate", "load", "load_config",
+           "register_architecture", "write_random_model"]

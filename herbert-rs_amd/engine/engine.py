@@ -112,6 +112,14 @@ class Engine:
         self.steps_run += 1
         return logits
 
+    def generate(self, prompts, params=None, max_batch=64, on_token=None):
+        """Generate from lists of token ids; see engine.generate.Generator."""
+        from .generate import Generator
+        gen = Generator(self, max_batch=max_batch)
+        results = gen.generate(prompts, params, on_token)
+        self.last_generation_stats = gen.stats
+        return results
+
     def get_tensor(self, name):
         """A weight as the engine holds it (by the name of the weight files)."""
         for part in self.model._weight_parts():

@@ -1,0 +1,151 @@
+"""The generation loop above the step function.
+
+Requests are served in batches, one after another: the prompts of a batch in
+one step, then one token for every sequence that still runs. A sequence ends
+on its end-of-sequence token (kept in the output, as the reference keeps it:
+crates/cli/src/main.rs:1272,1357-1359), on a stop token, after max_tokens
+tokens (counting the one the prompt gives, crates/cli/src/chat.rs:231), on
+a repetition loop (crates/core/src/decode_utils.rs:14-33) or at the model's
+last position; it gives its slot back at once and the others go on.
+"""
+import time
+from dataclasses import dataclass, field
+from typing import List
+
+from ..cache import PAGE_TOKENS
+from ..errors import RequestError
+from ..sampling import (EOS, LENGTH, MAX_TOKENS, REPETITION_LOOP, STOP_TOKEN, SamplingParams,
+                        detect_repetition_loop)
+from .batch import StepEntry
+
+
+@dataclass
+class GenerationResult:
+    tokens: List[int]
+    stop_reason: str
+    prompt_tokens: int
+
+
+@dataclass
+class GenerationStats:
+    prompt_tokens: int = 0
+    generated_tokens: int = 0
+    prefill_seconds: float = 0.0
+    decode_seconds: float = 0.0
+    decode_steps: int = 0
+    batches: int = 0
+
+
+def _rounded(n):
+    return (n + PAGE_TOKENS - 1) // PAGE_TOKENS * PAGE_TOKENS
+
+
+def plan_batches(prompt_lengths, max_new, max_batch, capacity_tokens, max_positions):
+    """Lists of request indices, in order, each list one batch that fits the cache."""
+    batches, current, used = [], [], 0
+    for i, n in enumerate(prompt_lengths):
+        if n <= 0:
+            raise RequestError(f"request {i} has an empty prompt")
+        if n > max_positions:
+            raise RequestError(f"request {i}: prompt of {n} tokens exceeds "
+                               f"max_position_embeddings ({max_positions})")
+        need = _rounded(min(n + max_new, max_positions))
+        if need > capacity_tokens:
+            raise RequestError(f"request {i} needs room for {need} tokens but the cache holds "
+                               f"{capacity_tokens}")
+        if current and (len(current) >= max_batch or used + need > capacity_tokens):
+            batches.append(current)
+            current, used = [], 0
+        current.append(i)
+        used += need
+    if current:
+        batches.append(current)
+    return batches
+
+
+def stop_reason(generated, params, eos_id):
+    """Why a sequence ends after its newest token, or None."""
+    tok = generated[-1]
+    if not params.ignore_eos and eos_id is not None and tok == eos_id:
+        return EOS
+    if tok in params.stop_ids:
+        return STOP_TOKEN
+    if len(generated) >= params.max_tokens:
+        return MAX_TOKENS
+    if params.repeat_check and detect_repetition_loop(generated) is not None:
+        return REPETITION_LOOP
+    return None
+
+
+class Generator:
+    """Runs requests through an engine. `make_chooser(params, n, vocab, device)` builds the object
+    whose `choose(logits, sequence_indices)` picks tokens (the GPU sampler by default)."""
+
+    def __init__(self, engine, max_batch=64, make_chooser=None):
+        self.engine = engine
+        self.max_batch = int(max_batch)
+        if make_chooser is None:
+            from ..sampling.sampler import Sampler
+            make_chooser = Sampler
+        self.make_chooser = make_chooser
+        self.stats = GenerationStats()
+
+    def generate(self, prompts, params=None, on_token=None):
+        """One GenerationResult per prompt (a list of token ids), in the prompts' order.
+        on_token(request index, token) is called for every generated token."""
+        params = params or SamplingParams()
+        params.validate()
+        eng = self.engine
+        spec = eng.spec
+        capacity = eng.cache.n_pages * PAGE_TOKENS
+        batches = plan_batches([len(p) for p in prompts], params.max_tokens, self.max_batch,
+                               capacity, spec.max_positions)
+        chooser = self.make_chooser(params, len(prompts), spec.vocab_size, eng.device)
+        results = [None] * len(prompts)
+        self.stats = GenerationStats()
+        for members in batches:
+            self._run_batch(members, prompts, params, chooser, results, on_token)
+            self.stats.batches += 1
+        return results
+
+    def _run_batch(self, members, prompts, params, chooser, results, on_token):
+        eng = self.engine
+        eos = eng.spec.eos_token_id
+        slots = {i: eng.alloc_slot() for i in members}
+        generated = {i: [] for i in members}
+        live = list(members)
+
+        def finish(i, reason):
+            results[i] = GenerationResult(generated[i], reason, len(prompts[i]))
+            eng.free_slot(slots.pop(i))
+            live.remove(i)
+
+        try:
+            t0 = time.perf_counter()
+            entries = [StepEntry(slots[i], list(prompts[i]), [len(prompts[i]) - 1]) for i in live]
+            logits = eng.step(entries)
+            tokens = chooser.choose(logits, list(live))
+            self.stats.prefill_seconds += time.perf_counter() - t0
+            self.stats.prompt_tokens += sum(len(prompts[i]) for i in live)
+            t0 = time.perf_counter()
+            while True:
+                for i, tok in zip(list(live), tokens):
+                    generated[i].append(int(tok))
+                    self.stats.generated_tokens += 1
+                    if on_token is not None:
+                        on_token(i, int(tok))
+                    reason = stop_reason(generated[i], params, eos)
+                    if reason is None and eng.cache.length(slots[i]) >= eng.spec.max_positions:
+                        reason = LENGTH
+                    if reason is not None:
+                        finish(i, reason)
+                if not live:
+                    break
+                entries = [StepEntry(slots[i], [generated[i][-1]], [0]) for i in live]
+                logits = eng.step(entries)
+                tokens = chooser.choose(logits, list(live))
+                self.stats.decode_steps += 1
+            self.stats.decode_seconds += time.perf_counter() - t0
+        finally:
+            for i in list(slots):
+                eng.free_slot(slots.pop(i))

@@ -1,0 +1,54 @@
+"""Choosing tokens on the GPU from float32 logits.
+
+temperature 0: the first index of the largest value (crates/core/src/sampler.rs:244-254).
+Otherwise the reference's algorithm (sampler.rs:72-145): divide by the temperature, keep the
+top_k largest, softmax, keep the shortest prefix by descending probability whose sum reaches
+top_p, renormalise, walk the running sum until it exceeds the draw. Where the reference
+leaves the order of candidates open, it is value descending, index ascending among equals.
+"""
+import torch
+
+from ..kernels import ops
+from . import xorshift
+
+
+def _signed64(v):
+    return v - (1 << 64) if v >= (1 << 63) else v
+
+
+class Sampler:
+    """One generator stream per sequence, kept on the GPU and advanced by the kernel."""
+
+    def __init__(self, params, num_sequences, vocab_size, device):
+        params.validate()
+        self.params = params
+        self.device = device
+        self.vocab_size = vocab_size
+        seed = params.seed if params.seed is not None else xorshift.clock_seed()
+        states = [_signed64(xorshift.sequence_seed(seed, i)) for i in range(num_sequences)]
+        self.states = torch.tensor(states, dtype=torch.int64, device=device)
+        self._scratch = None
+
+    def _scratch_for(self, rows):
+        p = self.params
+        if 0 < p.top_k < self.vocab_size and p.top_k <= 1024:
+            return None
+        p2 = 1
+        while p2 < self.vocab_size:
+            p2 <<= 1
+        if self._scratch is None or self._scratch[0].shape[0] < rows:
+            self._scratch = (torch.empty((rows, p2), dtype=torch.int32, device=self.device),
+                             torch.empty((rows, p2), dtype=torch.int32, device=self.device))
+        return self._scratch
+
+    def choose(self, logits, sequence_indices):
+        """Token for each row of `logits`; row r belongs to sequence sequence_indices[r]."""
+        rows = logits.shape[0]
+        out = torch.empty(rows, dtype=torch.int32, device=self.device)
+        if self.params.greedy:
+            ops.argmax(logits, out)
+        else:
+            index = torch.tensor(list(sequence_indices), dtype=torch.int32, device=self.device)
+            ops.sample(logits, self.params.temperature, self.params.top_k, self.params.top_p,
+                       self.states, index, out, self._scratch_for(rows))
+        return out.tolist()
