@@ -1,0 +1,301 @@
+"""The cache's bookkeeping (no slot or page lost, held twice or freed twice) and the generation
+loop's decisions, on the CPU with a stand-in for the engine's step."""
+import random
+
+import numpy as np
+import pytest
+import torch
+
+from herbert_rs_amd.cache import Cache, FreeList, KVNeed, StateNeed, pages_for
+from herbert_rs_amd.engine.generate import Generator, plan_batches, stop_reason
+from herbert_rs_amd.errors import CacheError, RequestError
+from herbert_rs_amd.sampling import (EOS, LENGTH, MAX_TOKENS, REPETITION_LOOP, STOP_TOKEN,
+                                     SamplingParams, detect_repetition_loop)
+from herbert_rs_amd.sampling import xorshift
+
+
+def test_free_list_is_strict():
+    fl = FreeList(3, "slot")
+    a, b, c = fl.take(), fl.take(), fl.take()
+    assert sorted((a, b, c)) == [0, 1, 2]
+    with pytest.raises(CacheError, match="no free slot"):
+        fl.take()
+    fl.give_back(b)
+    with pytest.raises(CacheError, match="freed twice"):
+        fl.give_back(b)
+    with pytest.raises(CacheError):
+        fl.give_back(7)
+    assert fl.take() == b
+    fl.check()
+
+
+def make_cache(window=None, state=False, max_tokens=64 * 12, max_positions=512):
+    needs = {0: KVNeed(2, 8, None), 1: KVNeed(2, 8, window), 2: KVNeed(2, 8, None)}
+    if state:
+        needs[3] = StateNeed((4,), torch.float32)
+        needs[1] = (KVNeed(2, 8, window), StateNeed((4,), torch.float32))
+    return Cache(needs, max_tokens, max_positions, torch.float32, "cpu")
+
+
+def test_groups_have_storage_of_their_own():
+    c = make_cache(window=100)
+    assert len(c.kv_groups) == 2
+    full = c.kv_groups[KVNeed(2, 8, None)]
+    win = c.kv_groups[KVNeed(2, 8, 100)]
+    assert full.entries == [0, 2] and win.entries == [1]
+    assert full.pool.shape == (2, 2, 12, 2, 64, 8) and win.pool.shape == (1, 2, 12, 2, 64, 8)
+    assert c.kv_view(0).k.data_ptr() != c.kv_view(2).k.data_ptr()
+    assert c.kv_view(1).window == 100 and c.kv_view(0).window == 0
+
+
+def test_pages_follow_lengths_and_come_back():
+    c = make_cache()
+    s = c.alloc_slot()
+    g = c.kv_groups[KVNeed(2, 8, None)]
+    c.reserve(s, 5); c.commit(s, 5)
+    assert g.pages.held_count == 1
+    c.reserve(s, 59); c.commit(s, 59)
+    assert g.pages.held_count == 1 and c.length(s) == 64
+    c.reserve(s, 1); c.commit(s, 1)
+    assert g.pages.held_count == 2
+    assert g.table[s, :2].tolist() == g.table_host[s, :2].tolist()
+    c.check()
+    c.free_slot(s)
+    assert g.pages.held_count == 0
+    c.check()
+    with pytest.raises(CacheError):
+        c.free_slot(s)
+    with pytest.raises(CacheError):
+        c.length(s)
+
+
+def test_window_group_gives_back_unseen_pages():
+    c = make_cache(window=70)
+    s = c.alloc_slot()
+    win = c.kv_groups[KVNeed(2, 8, 70)]
+    full = c.kv_groups[KVNeed(2, 8, None)]
+    c.reserve(s, 200); c.commit(s, 200)
+    # the next query (position 200) sees keys 131..200: pages 0 and 1 (keys 0..127) are out of sight
+    assert win.first_page[s] == 2 and win.pages.held_count == 2 and full.pages.held_count == 4
+    for _ in range(60):
+        c.reserve(s, 1); c.commit(s, 1)
+    assert win.first_page[s] == 2 + (261 - 70 - 128) // 64 and c.length(s) == 260
+    c.check()
+    with pytest.raises(CacheError, match="given up"):
+        c.truncate(s, 100)
+    c.truncate(s, 250)
+    assert c.length(s) == 250
+    c.free_slot(s)
+    assert win.pages.held_count == 0 and full.pages.held_count == 0
+    c.check()
+
+
+def test_exhaustion_and_limits():
+    c = make_cache(max_tokens=64 * 3)
+    a, b = c.alloc_slot(), c.alloc_slot()
+    c.reserve(a, 128); c.commit(a, 128)
+    with pytest.raises(CacheError, match="no free page"):
+        c.reserve(b, 129)
+    c.free_slot(b)
+    c.free_slot(a)
+    c.check()
+    s = c.alloc_slot()
+    with pytest.raises(CacheError, match="exceed"):
+        c.reserve(s, 513)
+    assert Cache({0: KVNeed(1, 8)}, 100, 512, torch.float32, "cpu").n_pages == 2    # rounded up to 64
+
+
+def test_state_is_cleared_when_a_slot_is_taken_again():
+    c = make_cache(state=True)
+    s = c.alloc_slot()
+    views = c.state_views(1)
+    assert len(views) == 1 and views[0].shape == (c.n_slots, 4)
+    views[0][s] = 5.0
+    c.state_views(3)[0][s] = 2.0
+    c.free_slot(s)
+    s2 = c.alloc_slot()
+    assert s2 == s
+    assert float(c.state_views(1)[0][s2].abs().sum()) == 0 and float(c.state_views(3)[0][s2].abs().sum()) == 0
+    c.reserve(s2, 3); c.commit(s2, 3)
+    with pytest.raises(CacheError, match="rolled back"):
+        c.truncate(s2, 1)
+
+
+def test_random_walk_keeps_the_books():
+    rnd = random.Random(3)
+    c = make_cache(window=70, max_tokens=64 * 40)
+    live = {}
+    for _ in range(400):
+        r = rnd.random()
+        if r < 0.3 and len(live) < 10:
+            live[c.alloc_slot()] = 0
+        elif r < 0.5 and live:
+            s = rnd.choice(list(live))
+            c.free_slot(s)
+            del live[s]
+        elif live:
+            s = rnd.choice(list(live))
+            n = rnd.choice([1, 1, 1, 7, 64, 90])
+            if live[s] + n <= 512:
+                try:
+                    c.reserve(s, n)
+                except CacheError:
+                    continue
+                c.commit(s, n)
+                live[s] += n
+        c.check()
+        for s, n in live.items():
+            assert c.length(s) == n
+            full = c.kv_groups[KVNeed(2, 8, None)].table_host[s]
+            assert (full >= 0).sum() == pages_for(n)
+    for s in list(live):
+        c.free_slot(s)
+    c.check()
+    assert all(g.pages.held_count == 0 for g in c.kv_groups.values())
+
+
+# ---- the generation loop with a stand-in engine
+class FakeCache:
+    def __init__(self, n_pages):
+        self.n_pages = n_pages
+        self.slots = FreeList(64, "slot")
+        self.lengths = {}
+
+    def length(self, slot):
+        return self.lengths[slot]
+
+
+class FakeSpec:
+    vocab_size = 50
+    max_positions = 40
+    eos_token_id = 9
+
+
+class FakeEngine:
+    """Logits that make the next token (last token + 1) mod vocab: the loop's decisions show."""
+    device = "cpu"
+
+    def __init__(self, n_pages=64):
+        self.spec = FakeSpec()
+        self.cache = FakeCache(n_pages)
+        self.steps = []
+        self.max_held = 0
+
+    def alloc_slot(self):
+        s = self.cache.slots.take()
+        self.cache.lengths[s] = 0
+        self.max_held = max(self.max_held, self.cache.slots.held_count)
+        return s
+
+    def free_slot(self, s):
+        self.cache.slots.give_back(s)
+        del self.cache.lengths[s]
+
+    def step(self, entries):
+        self.steps.append([(e.slot, len(e.tokens)) for e in entries])
+        rows = []
+        for e in entries:
+            self.cache.lengths[e.slot] += len(e.tokens)
+            for j in e.want:
+                row = np.zeros(self.spec.vocab_size, dtype=np.float32)
+                row[(e.tokens[j] + 1) % self.spec.vocab_size] = 1.0
+                rows.append(row)
+        return np.stack(rows)
+
+
+class ArgmaxChooser:
+    def __init__(self, params, n, vocab, device):
+        self.calls = []
+
+    def choose(self, logits, sequence_indices):
+        self.calls.append(list(sequence_indices))
+        return [int(r.argmax()) for r in logits]
+
+
+def run(prompts, engine=None, **kw):
+    engine = engine or FakeEngine()
+    gen = Generator(engine, max_batch=kw.pop("max_batch", 4), make_chooser=ArgmaxChooser)
+    params = SamplingParams(temperature=0.0, **kw)
+    return engine, gen, gen.generate(prompts, params)
+
+
+def test_stops_eos_max_tokens_stop_token_and_order():
+    eng, gen, res = run([[5], [20, 21], [7, 8]], max_tokens=6, stop_ids=(23,), repeat_check=False)
+    assert res[0].tokens == [6, 7, 8, 9] and res[0].stop_reason == EOS         # eos kept in the output
+    assert res[1].tokens == [22, 23] and res[1].stop_reason == STOP_TOKEN
+    assert res[2].tokens == [9] and res[2].stop_reason == EOS                  # the prompt's own token
+    assert [r.prompt_tokens for r in res] == [1, 2, 2]
+    # one prompt step with all three, then only the unfinished ones, one token each
+    assert eng.steps[0] == [(0, 1), (1, 2), (2, 2)]
+    assert eng.steps[1] == [(0, 1), (1, 1)] and eng.steps[2:] == [[(0, 1)], [(0, 1)]]
+    assert eng.cache.slots.held_count == 0
+    assert gen.stats.generated_tokens == 7 and gen.stats.decode_steps == 3 and gen.stats.prompt_tokens == 5
+
+
+def test_max_tokens_counts_the_first_token_and_ignore_eos():
+    _, _, res = run([[5]], max_tokens=3, repeat_check=False)
+    assert res[0].tokens == [6, 7, 8] and res[0].stop_reason == MAX_TOKENS
+    _, _, res = run([[7]], max_tokens=4, ignore_eos=True, repeat_check=False)
+    assert res[0].tokens == [8, 9, 10, 11] and res[0].stop_reason == MAX_TOKENS
+
+
+def test_batches_follow_one_another_and_slots_are_used_again():
+    prompts = [[i] for i in (10, 11, 12, 13, 14, 15, 30)]
+    eng, gen, res = run(prompts, max_tokens=2, max_batch=3, repeat_check=False)
+    assert [r.tokens for r in res] == [[p[0] + 1, p[0] + 2] for p in prompts]
+    assert gen.stats.batches == 3 and eng.max_held == 3
+    firsts = [s for s in eng.steps if all(n == 1 for _, n in s)][::2]
+    assert [sorted(slot for slot, _ in s) for s in firsts] == [[0, 1, 2], [0, 1, 2], [0]]
+
+
+def test_the_model_s_last_position_ends_a_sequence():
+    eng, _, res = run([list(range(10, 48))], max_tokens=10, repeat_check=False)     # 38 of 40 positions
+    assert res[0].stop_reason == LENGTH and len(res[0].tokens) == 3
+    assert eng.cache.slots.held_count == 0
+
+
+def test_plan_batches_respects_capacity():
+    assert plan_batches([5, 11, 2, 300], 8, 3, 1024, 512) == [[0, 1, 2], [3]]
+    assert plan_batches([100, 100, 100], 28, 8, 256, 512) == [[0, 1], [2]]
+    with pytest.raises(RequestError, match="empty"):
+        plan_batches([3, 0], 8, 4, 1024, 512)
+    with pytest.raises(RequestError, match="exceeds"):
+        plan_batches([600], 8, 4, 4096, 512)
+    with pytest.raises(RequestError, match="holds"):
+        plan_batches([100], 100, 4, 128, 512)
+
+
+def test_stop_reason_rules():
+    p = SamplingParams(temperature=0.0, max_tokens=100, stop_ids=(4,))
+    assert stop_reason([1, 2, 9], p, 9) == EOS
+    assert stop_reason([1, 2, 4], p, 9) == STOP_TOKEN
+    assert stop_reason([1, 2, 3], p, 9) is None
+    loop = [1, 2, 3, 5, 6, 7] * 3
+    assert stop_reason(loop, p, 9) == REPETITION_LOOP
+    assert stop_reason(loop, SamplingParams(temperature=0.0, max_tokens=100, repeat_check=False), 9) is None
+    assert stop_reason([1] * 5, SamplingParams(temperature=0.0, max_tokens=5, repeat_check=False), 9) == MAX_TOKENS
+    assert detect_repetition_loop([1, 2, 3, 4, 5] * 3) is None
+
+
+def test_slots_come_back_when_a_step_fails():
+    class Failing(FakeEngine):
+        def step(self, entries):
+            if len(self.steps) == 1:
+                raise RuntimeError("boom")
+            return super().step(entries)
+    eng = Failing()
+    with pytest.raises(RuntimeError):
+        run([[1], [2]], engine=eng, max_tokens=5, repeat_check=False)
+    assert eng.cache.slots.held_count == 0
+
+
+def test_params_are_checked_and_seeds_give_streams():
+    with pytest.raises(RequestError):
+        SamplingParams(temperature=-1.0).validate()
+    with pytest.raises(RequestError):
+        SamplingParams(max_tokens=0).validate()
+    d = SamplingParams()
+    assert (d.temperature, d.top_k, d.top_p, d.max_tokens) == (0.4, 40, 0.9, 2048)   # the reference's defaults
+    assert xorshift.initial_state(0) == 0xDEADBEEF and xorshift.step(1) == 1082269761
+    assert xorshift.sequence_seed(7, 0) == 7
+    assert len({xorshift.sequence_seed(7, i) for i in range(16)}) == 16

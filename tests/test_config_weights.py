@@ -1,0 +1,183 @@
+"""Configuration (keys, defaults, errors, registry) and weights (reading, errors, random folders)."""
+import json
+import os
+
+import pytest
+import torch
+from safetensors.torch import load_file, save_file
+
+from herbert_rs_amd.config import Qwen3Config, load_config, registered_architectures
+from herbert_rs_amd.config.registry import resolve_architecture
+from herbert_rs_amd.engine.model import Model
+from herbert_rs_amd.errors import ConfigError, ModelLoadError
+from herbert_rs_amd.weights import read_tensors
+from herbert_rs_amd.weights.bf16 import bf16_bits_to_f32, f32_to_bf16_bits
+
+from .tiny import TINY_A, TINY_B, TINY_C, make_folder, spec_of
+
+
+def minimal(**over):
+    raw = dict(vocab_size=100, hidden_size=32, num_hidden_layers=2, num_attention_heads=4,
+               num_key_value_heads=2, intermediate_size=64, max_position_embeddings=64,
+               rope_theta=10000.0)
+    raw.update(over)
+    return {k: v for k, v in raw.items() if v is not ...}
+
+
+def test_defaults_of_the_reference():
+    cfg = Qwen3Config.from_dict(minimal())
+    assert cfg.rms_norm_eps == 1e-5                 # crates/core/src/config.rs:583-585
+    assert cfg.tie_word_embeddings is True          # :199-202
+    assert cfg.head_dim == 8                        # hidden / heads, :496-498
+    assert cfg.eos_token_id == 151643               # :283-287
+    assert cfg.layer_windows == (None, None)
+    assert (cfg.q_dim, cfg.kv_dim, cfg.num_kv_groups) == (32, 16, 2)
+
+
+def test_decoupled_head_dim_and_eos_forms():
+    cfg = Qwen3Config.from_dict(minimal(head_dim=16, eos_token_id=[7, 9]))
+    assert cfg.q_dim == 64 and cfg.eos_token_id == 7
+    assert Qwen3Config.from_dict(minimal(eos_token_id=5)).eos_token_id == 5
+    nested = minimal(rope_theta=..., rope_parameters={"rope_theta": 5e5, "rope_type": "default"})
+    assert Qwen3Config.from_dict(nested).rope_theta == 5e5
+
+
+@pytest.mark.parametrize("over,word", [
+    (dict(rope_theta=...), "rope_theta"),
+    (dict(vocab_size=...), "vocab_size"),
+    (dict(num_key_value_heads=3), "divisible"),
+    (dict(head_dim=7), "even"),
+    (dict(hidden_size=0), "hidden_size"),
+    (dict(num_hidden_layers=0), "num_layers"),
+    (dict(intermediate_size=0), "intermediate_size"),
+    (dict(rms_norm_eps=0.0), "rms_norm_eps"),
+    (dict(rope_theta=-1.0), "rope_theta"),
+    (dict(max_position_embeddings=0), "max_position_embeddings"),
+    (dict(num_experts=8), "expert"),
+    (dict(rope_scaling={"type": "yarn", "factor": 4.0}), "yarn"),
+    (dict(text_config={}), "text_config"),
+    (dict(layer_types=["full_attention"]), "layer_types"),
+    (dict(layer_types=["sliding_attention", "full_attention"]), "sliding_window"),
+    (dict(vocab_size="many"), "integer"),
+])
+def test_config_errors_name_the_key(over, word):
+    with pytest.raises(ConfigError, match=word):
+        Qwen3Config.from_dict(minimal(**over))
+
+
+def test_windows_from_both_forms():
+    cfg = Qwen3Config.from_dict(minimal(sliding_window=16, layer_types=["sliding_attention", "full_attention"]))
+    assert cfg.layer_windows == (16, None)
+    cfg = Qwen3Config.from_dict(minimal(sliding_window=16, use_sliding_window=True, max_window_layers=1))
+    assert cfg.layer_windows == (None, 16)
+    cfg = Qwen3Config.from_dict(minimal(sliding_window=16, use_sliding_window=False))
+    assert cfg.layer_windows == (None, None)
+    assert Qwen3Config.from_dict(cfg.to_dict()) == cfg
+    win = Qwen3Config.from_dict(TINY_C)
+    assert Qwen3Config.from_dict(win.to_dict()) == win
+
+
+def test_registry_by_architecture_and_model_type(tmp_path):
+    assert "Qwen3ForCausalLM" in registered_architectures()
+    assert resolve_architecture({"architectures": ["Qwen3ForCausalLM"]}).name == "Qwen3ForCausalLM"
+    assert resolve_architecture({"model_type": "qwen3"}).name == "Qwen3ForCausalLM"
+    assert resolve_architecture({}).name == "Qwen3ForCausalLM"        # model_type defaults to qwen3
+    with pytest.raises(ConfigError, match="Qwen3ForCausalLM"):
+        resolve_architecture({"architectures": ["LlamaForCausalLM"]})
+    with pytest.raises(ConfigError, match="gpt2"):
+        resolve_architecture({"model_type": "gpt2"})
+    with open(tmp_path / "config.json", "w") as f:
+        json.dump(TINY_B, f)
+    arch, cfg = load_config(str(tmp_path))
+    assert cfg.num_hidden_layers == 3 and cfg.eos_token_id == 383
+    with pytest.raises(ConfigError, match="config.json"):
+        load_config(str(tmp_path / "nothing"))
+
+
+def test_the_tiny_configurations_differ_everywhere():
+    a, b, c = (Qwen3Config.from_dict(t) for t in (TINY_A, TINY_B, TINY_C))
+    for field in ("vocab_size", "hidden_size", "num_attention_heads", "head_dim", "intermediate_size",
+                  "max_position_embeddings", "rope_theta", "rms_norm_eps", "num_kv_groups"):
+        assert len({getattr(a, field), getattr(b, field), getattr(c, field)}) == 3, field
+    assert a.tie_word_embeddings != b.tie_word_embeddings
+    assert a.num_hidden_layers != b.num_hidden_layers
+    assert c.layer_windows != a.layer_windows
+
+
+# ---- weights
+def needs_of(raw):
+    return Model(spec_of(raw)[1]).tensor_needs()
+
+
+def test_random_folder_reads_back(model_root):
+    for dtype, tdt in (("float32", torch.float32), ("bfloat16", torch.bfloat16)):
+        folder = make_folder(model_root, "B", dtype)
+        needs = needs_of(TINY_B)
+        tensors = read_tensors(folder, needs)
+        assert set(tensors) == set(needs)
+        assert "lm_head.weight" in needs and "lm_head.weight" not in needs_of(TINY_A)
+        for name, t in tensors.items():
+            assert tuple(t.shape) == tuple(needs[name].shape) and t.dtype == tdt     # kept as stored
+        q = tensors["model.layers.0.self_attn.q_proj.weight"].float()
+        assert tuple(q.shape) == (192, 96) and 0.04 < float(q.std()) < 0.06
+        n = tensors["model.norm.weight"].float()
+        assert abs(float(n.mean()) - 1.0) < 0.1 and float(n.std()) > 0.01
+    again = make_folder(str(model_root) + "_again", "B", "float32")
+    same = load_file(os.path.join(again, "model.safetensors"))
+    first = load_file(os.path.join(make_folder(model_root, "B", "float32"), "model.safetensors"))
+    assert all(torch.equal(same[k], first[k]) for k in first)          # the seed decides
+
+
+def test_one_error_lists_missing_unexpected_and_wrong(model_root, tmp_path):
+    src = make_folder(model_root, "A", "float32")
+    tensors = load_file(os.path.join(src, "model.safetensors"))
+    del tensors["model.layers.1.self_attn.q_norm.weight"]
+    del tensors["model.norm.weight"]
+    tensors["model.layers.0.mlp.gate_proj.weight"] = torch.zeros(128, 63)
+    tensors["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(8)
+    save_file(tensors, str(tmp_path / "model.safetensors"))
+    with open(tmp_path / "config.json", "w") as f:
+        json.dump(TINY_A, f)
+    with pytest.raises(ModelLoadError) as err:
+        read_tensors(str(tmp_path), needs_of(TINY_A))
+    text = str(err.value)
+    assert "missing (2)" in text and "model.layers.1.self_attn.q_norm.weight" in text
+    assert "model.norm.weight" in text
+    assert "unexpected (1)" in text and "rotary_emb.inv_freq" in text
+    assert "gate_proj.weight: expected [128, 64], got [128, 63]" in text
+
+
+def test_tied_model_refuses_a_stray_head_and_untied_needs_one(model_root, tmp_path):
+    src = make_folder(model_root, "A", "float32")
+    tensors = load_file(os.path.join(src, "model.safetensors"))
+    tensors["lm_head.weight"] = torch.zeros(256, 64)
+    save_file(tensors, str(tmp_path / "model.safetensors"))
+    with pytest.raises(ModelLoadError, match="unexpected"):
+        read_tensors(str(tmp_path), needs_of(TINY_A))
+    with pytest.raises(ModelLoadError, match="lm_head.weight"):
+        read_tensors(src, needs_of(dict(TINY_A, tie_word_embeddings=False)))
+
+
+def test_stored_dtypes_and_shards(tmp_path):
+    from herbert_rs_amd.weights import TensorNeed
+    save_file({"a": torch.ones(2, 2, dtype=torch.float16), "i": torch.arange(3, dtype=torch.int64)},
+              str(tmp_path / "part1.safetensors"))
+    save_file({"b": torch.ones(2, dtype=torch.float32)}, str(tmp_path / "part2.safetensors"))
+    with open(tmp_path / "model.safetensors.index.json", "w") as f:
+        json.dump({"weight_map": {"a": "part1.safetensors", "i": "x/part1.safetensors",
+                                  "b": "part2.safetensors"}}, f)
+    got = read_tensors(str(tmp_path), {"a": TensorNeed((2, 2)), "b": TensorNeed((2,), "scale"),
+                                       "i": TensorNeed((3,), "index")})
+    assert got["a"].dtype == torch.bfloat16 and got["b"].dtype == torch.float32
+    assert got["i"].dtype == torch.int32
+    with pytest.raises(ModelLoadError, match="no model.safetensors"):
+        read_tensors(str(tmp_path / "void"), {})
+
+
+def test_bf16_conversion_bits():
+    x = torch.tensor([1.0, 0.0, -2.5, 3.1415927], dtype=torch.float32)
+    bits = f32_to_bf16_bits(x)
+    assert bits[0] == 0x3F80 and bits[1] == 0
+    assert torch.equal(bf16_bits_to_f32(bits), x.to(torch.bfloat16).float())
+    ties = torch.tensor([0x3F808000, 0x3F818000, 0x3F808001], dtype=torch.int64).to(torch.int32).view(torch.float32)
+    assert f32_to_bf16_bits(ties).tolist() == [0x3F80, 0x3F82, 0x3F81]
