@@ -26,7 +26,7 @@ from .slots import PAGE_TOKENS, FreeList, pages_for
 class LayerKV:
     """What an attention kernel needs of one schedule entry's cache."""
     k: torch.Tensor            # [pages, kv_heads, PAGE_TOKENS, head_dim]
-    v: torch.Tensor
+    v: torch.Tensor            # [pages, kv_heads, head_dim, PAGE_TOKENS]: tokens contiguous
     page_table: torch.Tensor   # int32 [slots, pages per slot]
     page_size: int
     window: int                # 0 = all keys
@@ -48,8 +48,10 @@ class KVGroup:
 
     def view(self, entry):
         i = self.entries.index(entry)
-        return LayerKV(self.pool[i, 0], self.pool[i, 1], self.table, PAGE_TOKENS,
-                       int(self.need.window or 0))
+        n_pages = self.pool.shape[2]
+        k = self.pool[i, 0]
+        v = self.pool[i, 1].view(n_pages, self.need.kv_heads, self.need.head_dim, PAGE_TOKENS)
+        return LayerKV(k, v, self.table, PAGE_TOKENS, int(self.need.window or 0))
 
     def ensure(self, slot, new_length):
         """Hold a page for every position below new_length that a query may still see."""

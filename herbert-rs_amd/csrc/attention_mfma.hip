@@ -1,0 +1,357 @@
+// bfloat16 attention over the paged cache on the gfx950 matrix cores.
+//
+// Cache layout: keys [page, kv head, 64 tokens, hd] (hd contiguous: the contraction of Q K^T),
+// values transposed [page, kv head, hd, 64 tokens] (tokens contiguous: the contraction of P V).
+// Both products are computed transposed with the 32x32x16 MFMA:
+//   S^T[key, query] = K Q^T      first operand K rows, second operand Q rows
+//   O^T[d,   query] = V^T P^T    first operand V^T rows, second operand P^T, which is S^T's
+//                                own accumulator layout, so P never leaves the registers.
+// A lane then owns one query column: the running maximum and sum of the online softmax are
+// per-lane scalars (one exchange with the lane 32 apart). The 32 rows of a key block are
+// assigned to keys in the order perm() below, which makes a lane's 8 values of one PV step
+// 8 consecutive keys: V^T operands are single 16-byte reads.
+//
+// prefill: one workgroup = 32 consecutive tokens of one sequence x up to 4 query heads of one
+//          kv head (one wave each); K and V^T pages are staged in LDS once for all of them.
+// decode:  one wave = one sequence x one kv head x one range of pages, all query heads of the
+//          group as columns; operands stream from global memory (each byte is used once);
+//          partial (max, sum, O) per range are merged by a second kernel.
+#include "common.h"
+#include <math.h>
+
+HB_MODULE_ERROR_SLOT()
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+#define PAGE 64
+#define QTILE 32
+
+// MFMA row rho (0..31) of a key block -> key within the block.
+// rho = 16h + 8b + 4g + r  ->  16h + 8g + 4b + r  (h, b, g in {0,1}, r in 0..3)
+__device__ __forceinline__ int perm(int rho) {
+    return (rho & 16) | ((rho & 4) << 1) | ((rho & 8) >> 1) | (rho & 3);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// accumulator element i of lane group g2 of key block kb -> key within the page
+__device__ __forceinline__ int acc_key(int kb, int g2, int i) { return kb * 32 + 16 * (i >> 3) + 8 * g2 + (i & 7); }
+
+// One page of scores: mask, online-softmax update, P^T as MFMA operands.
+// st[kb]: S^T accumulators (raw dot products). c = scale * log2(e).
+// Keys k with lo <= page0 + k <= hi are visible.
+__device__ __forceinline__ void softmax_page(f32x16 st[2], int g2, int page0, int lo, int hi, float c,
+                                             float& m, float& l, float& corr, bf16x8 pb[2][2]) {
+    float mx = -INFINITY;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int key = page0 + acc_key(kb, g2, i);
+            const float s = (key >= lo && key <= hi) ? st[kb][i] : -INFINITY;
+            st[kb][i] = s;
+            mx = fmaxf(mx, s);
+        }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m, mx);
+    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+    corr = fast_exp2((m - m_use) * c);        // m = -inf: 0
+    float sum = 0.f;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const float p = fast_exp2((st[kb][i] - m_use) * c);
+            sum += p;
+            pb[kb][i >> 3][i & 7] = (__bf16)p;
+        }
+    l = l * corr + sum;      // this lane's keys only; the two halves are added at the end
+    m = m_new;
+}
+
+// ----------------------------------------------------------------- prefill
+template <int HD>
+__global__ void __launch_bounds__(256)
+attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache,
+                    const bf16* __restrict__ v_cache, bf16* __restrict__ out,
+                    const int* __restrict__ tile_seq, const int* __restrict__ tile_row0,
+                    const int* __restrict__ tile_rows, const int* __restrict__ positions,
+                    const int* __restrict__ slots, const int* __restrict__ page_table, int max_pages, int nq,
+                    int nkv, float c, int window) {
+    constexpr int KLD = HD + 8;      // padded rows: 16-byte reads of 32 rows fall on distinct banks
+    constexpr int VLD = PAGE + 8;
+    __shared__ __attribute__((aligned(16))) bf16 Ks[PAGE * KLD];
+    __shared__ __attribute__((aligned(16))) bf16 Vs[HD * VLD];
+
+    const int tile = blockIdx.x;
+    const int G = nq / nkv;
+    const int chunks = (G + 3) / 4;
+    const int kvh = blockIdx.y / chunks;
+    const int chunk = blockIdx.y % chunks;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int c32 = lane & 31, g2 = lane >> 5;
+    const int head_in_group = chunk * 4 + wave;
+    const bool active = head_in_group < G;
+    const int h = kvh * G + (active ? head_in_group : G - 1);
+
+    const int row0 = tile_row0[tile];
+    const int rows = tile_rows[tile];
+    const int slot = slots[tile_seq[tile]];
+    const int* pt = page_table + (size_t)slot * max_pages;
+    const int pos0 = positions[row0];
+    const int my_row = c32 < rows ? c32 : rows - 1;
+    const int pos_q = pos0 + my_row;
+    const int lo_q = (window > 0 && pos_q + 1 > window) ? pos_q + 1 - window : 0;
+    const int hi_tile = pos0 + rows - 1;                                     // last visible key
+    const int lo_tile = (window > 0 && pos0 + 1 > window) ? pos0 + 1 - window : 0;
+
+    bf16x8 qreg[HD / 16];
+    {
+        const bf16* qrow = q + ((size_t)(row0 + my_row) * nq + h) * HD + g2 * 8;
+#pragma unroll
+        for (int s = 0; s < HD / 16; ++s) qreg[s] = *(const bf16x8*)(qrow + s * 16);
+    }
+
+    f32x16 oacc[HD / 32];
+#pragma unroll
+    for (int d = 0; d < HD / 32; ++d)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) oacc[d][i] = 0.f;
+    float m = -INFINITY, l = 0.f;
+
+    const int krow = perm(c32);
+    for (int page_idx = lo_tile / PAGE; page_idx <= hi_tile / PAGE; ++page_idx) {
+        const int page = pt[page_idx];
+        const bf16* kp = k_cache + ((size_t)page * nkv + kvh) * PAGE * HD;
+        const bf16* vp = v_cache + ((size_t)page * nkv + kvh) * HD * PAGE;
+        __syncthreads();      // the previous page has been read by every wave
+#pragma unroll
+        for (int cidx = tid; cidx < PAGE * HD / 8; cidx += 256) {
+            const int kr = cidx / (HD / 8), kc = cidx % (HD / 8);
+            *(bf16x8*)(&Ks[kr * KLD + kc * 8]) = *(const bf16x8*)(kp + (size_t)cidx * 8);
+            const int vr = cidx / (PAGE / 8), vc = cidx % (PAGE / 8);
+            *(bf16x8*)(&Vs[vr * VLD + vc * 8]) = *(const bf16x8*)(vp + (size_t)cidx * 8);
+        }
+        __syncthreads();
+        if (!active) continue;
+
+        f32x16 st[2];
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) st[kb][i] = 0.f;
+            const bf16* krowp = &Ks[(kb * 32 + krow) * KLD + g2 * 8];
+#pragma unroll
+            for (int s = 0; s < HD / 16; ++s) {
+                const bf16x8 ka = *(const bf16x8*)(krowp + s * 16);
+                st[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qreg[s], st[kb], 0, 0, 0);
+            }
+        }
+        float corr;
+        bf16x8 pb[2][2];
+        softmax_page(st, g2, page_idx * PAGE, lo_q, pos_q, c, m, l, corr, pb);
+#pragma unroll
+        for (int d = 0; d < HD / 32; ++d) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) oacc[d][i] *= corr;
+            const bf16* vrowp = &Vs[(d * 32 + c32) * VLD + g2 * 8];
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int h2 = 0; h2 < 2; ++h2) {
+                    const bf16x8 va = *(const bf16x8*)(vrowp + kb * 32 + h2 * 16);
+                    oacc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb[kb][h2], oacc[d], 0, 0, 0);
+                }
+        }
+    }
+    if (!active || c32 >= rows) return;
+    l += __shfl_xor(l, 32, 64);
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    bf16* orow = out + ((size_t)(row0 + c32) * nq + h) * HD;
+#pragma unroll
+    for (int d = 0; d < HD / 32; ++d)
+#pragma unroll
+        for (int qd = 0; qd < 4; ++qd) {
+            bf16x4 v;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) v[r] = (__bf16)(oacc[d][4 * qd + r] * inv);
+            *(bf16x4*)(orow + d * 32 + 8 * qd + 4 * g2) = v;
+        }
+}
+
+// ------------------------------------------------------------------ decode
+// partial_o [B, nq, splits, HD] float, partial_ml [B, nq, splits, 2] float (max, sum).
+template <int HD>
+__global__ void __launch_bounds__(64)
+attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache,
+                   const bf16* __restrict__ v_cache, float* __restrict__ partial_o,
+                   float* __restrict__ partial_ml, const int* __restrict__ context_lens,
+                   const int* __restrict__ slots, const int* __restrict__ page_table, int max_pages, int nq,
+                   int nkv, float c, int window, int pages_per_split) {
+    const int b = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z, splits = gridDim.z;
+    const int G = nq / nkv;
+    const int lane = threadIdx.x, c32 = lane & 31, g2 = lane >> 5;
+    const int ctx = context_lens[b];                 // keys 0 .. ctx-1; the query sits at ctx-1
+    const int hi = ctx - 1;
+    const int lo = (window > 0 && ctx > window) ? ctx - window : 0;
+    const int first_page = lo / PAGE + split * pages_per_split;
+    int last_page = first_page + pages_per_split - 1;
+    if (last_page > hi / PAGE) last_page = hi / PAGE;
+    const int* pt = page_table + (size_t)slots[b] * max_pages;
+    const int head = kvh * G + (c32 < G ? c32 : G - 1);
+
+    // k of the MFMA steps: step s, lane group g2, element j  <->  d = g2 * HD/2 + s * 8 + j,
+    // so a lane reads one contiguous half row of K
+    bf16x8 qreg[HD / 16];
+    {
+        const bf16* qrow = q + ((size_t)b * nq + head) * HD + g2 * (HD / 2);
+#pragma unroll
+        for (int s = 0; s < HD / 16; ++s) qreg[s] = *(const bf16x8*)(qrow + s * 8);
+    }
+    f32x16 oacc[HD / 32];
+#pragma unroll
+    for (int d = 0; d < HD / 32; ++d)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) oacc[d][i] = 0.f;
+    float m = -INFINITY, l = 0.f;
+    const int krow = perm(c32);
+
+    for (int page_idx = first_page; page_idx <= last_page; ++page_idx) {
+        const int page = pt[page_idx];
+        const bf16* kp = k_cache + ((size_t)page * nkv + kvh) * PAGE * HD + g2 * (HD / 2);
+        const bf16* vp = v_cache + ((size_t)page * nkv + kvh) * HD * PAGE + g2 * 8;
+        bf16x8 ka[2][HD / 16];
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int s = 0; s < HD / 16; ++s)
+                ka[kb][s] = *(const bf16x8*)(kp + (size_t)(kb * 32 + krow) * HD + s * 8);
+        bf16x8 va[HD / 32][2][2];
+#pragma unroll
+        for (int d = 0; d < HD / 32; ++d)
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int h2 = 0; h2 < 2; ++h2)
+                    va[d][kb][h2] = *(const bf16x8*)(vp + (size_t)(d * 32 + c32) * PAGE + kb * 32 + h2 * 16);
+        f32x16 st[2];
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) st[kb][i] = 0.f;
+#pragma unroll
+            for (int s = 0; s < HD / 16; ++s)
+                st[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[kb][s], qreg[s], st[kb], 0, 0, 0);
+        }
+        float corr;
+        bf16x8 pb[2][2];
+        softmax_page(st, g2, page_idx * PAGE, lo, hi, c, m, l, corr, pb);
+#pragma unroll
+        for (int d = 0; d < HD / 32; ++d) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) oacc[d][i] *= corr;
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int h2 = 0; h2 < 2; ++h2)
+                    oacc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[d][kb][h2], pb[kb][h2], oacc[d], 0, 0, 0);
+        }
+    }
+    if (c32 >= G) return;
+    l += __shfl_xor(l, 32, 64);
+    const size_t base = ((size_t)b * nq + kvh * G + c32) * splits + split;
+    if (g2 == 0) {
+        partial_ml[base * 2] = m;        // -inf when this range held no visible key
+        partial_ml[base * 2 + 1] = l;
+    }
+    float* po = partial_o + base * HD;
+#pragma unroll
+    for (int d = 0; d < HD / 32; ++d)
+#pragma unroll
+        for (int qd = 0; qd < 4; ++qd) {
+            f32x4 v = {oacc[d][4 * qd], oacc[d][4 * qd + 1], oacc[d][4 * qd + 2], oacc[d][4 * qd + 3]};
+            *(f32x4*)(po + d * 32 + 8 * qd + 4 * g2) = v;
+        }
+}
+
+// Merge the ranges of one (sequence, head): out = sum_s 2^((m_s - M) c) O_s / sum_s 2^((m_s - M) c) l_s.
+__global__ void attn_decode_merge_kernel(const float* __restrict__ partial_o,
+                                         const float* __restrict__ partial_ml, bf16* __restrict__ out,
+                                         int splits, int HD, float c) {
+    const size_t bh = blockIdx.x;
+    const float* ml = partial_ml + bh * splits * 2;
+    float M = -INFINITY;
+    for (int s = 0; s < splits; ++s) M = fmaxf(M, ml[2 * s]);
+    float denom = 0.f;
+    for (int s = 0; s < splits; ++s)
+        if (ml[2 * s] != -INFINITY) denom += fast_exp2((ml[2 * s] - M) * c) * ml[2 * s + 1];
+    const float inv = denom > 0.f ? 1.0f / denom : 0.f;
+    for (int d = threadIdx.x; d < HD; d += blockDim.x) {
+        float acc = 0.f;
+        for (int s = 0; s < splits; ++s)
+            if (ml[2 * s] != -INFINITY)
+                acc += fast_exp2((ml[2 * s] - M) * c) * partial_o[(bh * splits + s) * HD + d];
+        out[bh * HD + d] = hb_from_float<bf16>(acc * inv);
+    }
+}
+
+// ---------------------------------------------------------------- launchers
+#define LOG2E 1.4426950408889634f
+
+extern "C" int hb_attn_prefill_mfma(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                    const int* tile_seq, const int* tile_row0, const int* tile_rows,
+                                    int num_tiles, const int* positions, const int* slots,
+                                    const int* page_table, int max_pages, int page_size, int nq, int nkv,
+                                    int hd, float scale, int window, hipStream_t stream) {
+    HB_REQUIRE(num_tiles > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attn_prefill: bad sizes");
+    HB_REQUIRE(page_size == PAGE, "attn_prefill: pages must hold %d tokens", PAGE);
+    HB_REQUIRE(window >= 0, "attn_prefill: bad window");
+    const int G = nq / nkv;
+    dim3 grid(num_tiles, nkv * ((G + 3) / 4));
+    HB_REQUIRE(grid.y <= 65535, "attn_prefill: too many heads for the grid");
+    const float c = scale * LOG2E;
+#define LAUNCH_PREFILL(HDV)                                                                              \
+    attn_prefill_kernel<HDV><<<grid, 256, 0, stream>>>((const bf16*)q, (const bf16*)k_cache,             \
+                                                      (const bf16*)v_cache, (bf16*)out, tile_seq, tile_row0, \
+                                                      tile_rows, positions, slots, page_table, max_pages, nq, \
+                                                      nkv, c, window)
+    if (hd == 32) LAUNCH_PREFILL(32);
+    else if (hd == 64) LAUNCH_PREFILL(64);
+    else if (hd == 128) LAUNCH_PREFILL(128);
+    else HB_REQUIRE(false, "attn_prefill: head_dim %d is not one of 32, 64, 128", hd);
+#undef LAUNCH_PREFILL
+    HB_CHECK_LAUNCH("attn_prefill");
+    return 0;
+}
+
+extern "C" int hb_attn_decode_mfma(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                   float* partial_o, float* partial_ml, const int* context_lens,
+                                   const int* slots, const int* page_table, int max_pages, int page_size,
+                                   int B, int nq, int nkv, int hd, float scale, int window, int splits,
+                                   int pages_per_split, hipStream_t stream) {
+    HB_REQUIRE(B > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attn_decode: bad sizes");
+    HB_REQUIRE(page_size == PAGE, "attn_decode: pages must hold %d tokens", PAGE);
+    HB_REQUIRE(nq / nkv <= 32, "attn_decode: more than 32 query heads share a kv head");
+    HB_REQUIRE(splits > 0 && splits <= 65535 && pages_per_split > 0 && nkv <= 65535, "attn_decode: bad split");
+    HB_REQUIRE(window >= 0, "attn_decode: bad window");
+    dim3 grid(B, nkv, splits);
+    const float c = scale * LOG2E;
+#define LAUNCH_DECODE(HDV)                                                                               \
+    attn_decode_kernel<HDV><<<grid, 64, 0, stream>>>((const bf16*)q, (const bf16*)k_cache,               \
+                                                    (const bf16*)v_cache, partial_o, partial_ml,         \
+                                                    context_lens, slots, page_table, max_pages, nq, nkv, c, \
+                                                    window, pages_per_split)
+    if (hd == 32) LAUNCH_DECODE(32);
+    else if (hd == 64) LAUNCH_DECODE(64);
+    else if (hd == 128) LAUNCH_DECODE(128);
+    else HB_REQUIRE(false, "attn_decode: head_dim %d is not one of 32, 64, 128", hd);
+#undef LAUNCH_DECODE
+    HB_CHECK_LAUNCH("attn_decode");
+    attn_decode_merge_kernel<<<B * nq, hd < 64 ? 64 : hd, 0, stream>>>(partial_o, partial_ml, (bf16*)out,
+                                                                    splits, hd, c);
+    HB_CHECK_LAUNCH("attn_decode_merge");
+    return 0;
+}

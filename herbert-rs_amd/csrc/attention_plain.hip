@@ -67,12 +67,13 @@ attention_plain_kernel(const TQ* __restrict__ q, const TC* __restrict__ k_cache,
         for (int jj = jj0; jj < jj1; ++jj) {
             const int jv = c + jj;
             const int page = pt[jv / page_size];
-            const TC* vr = v_cache + (((size_t)page * nkv + g) * page_size + (jv % page_size)) * hd;
+            // values are stored transposed: [page, kv head, hd, token]
+            const TC* vr = v_cache + ((size_t)page * nkv + g) * page_size * hd + (jv % page_size);
             const float pj = ps[jj];
 #pragma unroll
             for (int i = 0; i < ACC_REGS; ++i) {
                 const int d = lane + HB_WAVE * i;
-                if (d < hd) acc[i] = fmaf(pj, hb_to_float(vr[d]), acc[i]);
+                if (d < hd) acc[i] = fmaf(pj, hb_to_float(vr[(size_t)d * page_size]), acc[i]);
             }
         }
     }
@@ -86,7 +87,8 @@ attention_plain_kernel(const TQ* __restrict__ q, const TC* __restrict__ k_cache,
     }
 }
 
-// q, out: [T, nq * hd]; caches: [pages, nkv, page_size, hd]; dtype covers q, cache and out.
+// q, out: [T, nq * hd]; keys [pages, nkv, page_size, hd], values [pages, nkv, hd, page_size];
+// dtype covers q, cache and out.
 extern "C" int hb_attention_plain(const void* q, const void* k_cache, const void* v_cache, void* out,
                                   int dtype, const int* positions, const int* seq_of, const int* slots,
                                   const int* page_table, int max_pages, int page_size, int T, int nq,

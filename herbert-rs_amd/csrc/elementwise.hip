@@ -67,7 +67,7 @@ extern "C" int hb_rmsnorm(const float* x, const float* w, void* y, int y_dtype, 
 // One wave per (token, head) of the fused projection row [q heads | k heads | v heads].
 //   q heads: optional RMSNorm over the head, optional rotation, written to q_out.
 //   k heads: the same, written to the key pages of the token's slot.
-//   v heads: copied to the value pages.
+//   v heads: copied to the value pages, which are transposed: [page, kv head, hd, token].
 // Rotation pairs dim j with j + R/2 (R = rot_dims), angle table [max_pos, R/2].
 // The page of position p of a slot is page_table[slot * max_pages + p / page_size].
 #define HB_MAX_HEAD_DIM 512
@@ -104,13 +104,15 @@ __global__ void qk_norm_rope_write_kernel(
     const float inv = do_norm ? 1.0f / sqrtf(ss / (float)hd + eps) : 1.0f;
     const int half = rot_dims / 2;
 
-    size_t dst_base = 0;
+    size_t dst_base = 0;      // keys: start of the token's row; values: start of the (page, head) block
     if (!is_q) {
         const int slot = slots[seq_of[t]];
         const int page = page_table[(size_t)slot * max_pages + pos / page_size];
         const int kvh = is_v ? h - nq - nkv : h - nq;
-        dst_base = (((size_t)page * nkv + kvh) * page_size + (pos % page_size)) * hd;
+        dst_base = ((size_t)page * nkv + kvh) * page_size * hd;
+        if (!is_v) dst_base += (size_t)(pos % page_size) * hd;
     }
+    const int in_page = pos % page_size;
 
     for (int d = lane; d < hd; d += HB_WAVE) {
         float out;
@@ -131,7 +133,7 @@ __global__ void qk_norm_rope_write_kernel(
         if (is_q)
             q_out[(size_t)t * nq * hd + (size_t)h * hd + d] = hb_from_float<TQ>(out);
         else if (is_v)
-            v_cache[dst_base + d] = hb_from_float<TC>(out);
+            v_cache[dst_base + (size_t)d * page_size + in_page] = hb_from_float<TC>(out);
         else
             k_cache[dst_base + d] = hb_from_float<TC>(out);
     }

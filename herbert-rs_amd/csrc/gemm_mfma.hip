@@ -1,0 +1,383 @@
+// bfloat16 matrix products on the gfx950 matrix cores, float32 accumulation:
+//   C[m, n] (+)= sum_k X[m, k] * W[n, k]        X [M, K], W [N, K], both k-contiguous
+// Two kernels share the epilogues:
+//   skinny (M <= 64, decoding): HBM-bound. The weights stream from memory straight into
+//     MFMA operands (each is used once), four waves of a workgroup split K between them
+//     and add their parts through LDS in a fixed order.
+//   tiled (M > 64, prompts): 128 x 128 x 64 tiles staged through LDS, 32x32x16 MFMA,
+//     global loads of the next tile in flight while the current one is multiplied.
+// In both the weight rows are the MFMA's first operand, so a lane ends up with four
+// consecutive n of one m: row-major stores of C are vector stores.
+// Epilogues: 0 store float32, 1 add to float32 (the residual stream), 2 SwiGLU to bfloat16
+// (weight rows interleaved in blocks of 16: gate rows, then the up rows of the same outputs).
+#include "common.h"
+
+HB_MODULE_ERROR_SLOT()
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+#define EPI_STORE 0
+#define EPI_ADD 1
+#define EPI_SWIGLU 2
+
+__device__ __forceinline__ float silu_mul(float g, float u) { return g / (1.0f + __expf(-g)) * u; }
+
+// ------------------------------------------------------------------ skinny
+// Workgroup: WAVES waves, NB blocks of 16 weight rows, MB blocks of 16 activation rows.
+// Wave w takes the k-steps (32 wide) s = w, w + WAVES, ...; it loads U steps ahead of the
+// ones it multiplies, so that enough bytes are in flight to keep HBM busy.
+template <int MB, int NB>
+struct SkinnyOperands {
+    bf16x8 w[NB];
+    bf16x8 x[MB];
+};
+
+template <int MB, int NB, int WAVES, int EPI>
+__global__ void __launch_bounds__(WAVES * 64)
+gemm_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* __restrict__ Cv, int M,
+                   int N, int K, int ldc) {
+    constexpr int U = (NB + MB <= 4) ? 4 : 2;
+    extern __shared__ float red[];   // [WAVES / 2][NB * MB * 4][64]
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int r16 = lane & 15;
+    const int g4 = lane >> 4;
+    const int n0 = blockIdx.x * (NB * 16);
+    const int nsteps = K / 32;
+
+    f32x4 acc[NB][MB];
+#pragma unroll
+    for (int a = 0; a < NB; ++a)
+#pragma unroll
+        for (int b = 0; b < MB; ++b) acc[a][b] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const bf16* wrow[NB];
+#pragma unroll
+    for (int a = 0; a < NB; ++a) {
+        int n = n0 + a * 16 + r16;
+        if (n >= N) n = N - 1;            // rows past the end repeat the last one; never stored
+        wrow[a] = W + (size_t)n * K + g4 * 8;
+    }
+    const bf16* xrow[MB];
+#pragma unroll
+    for (int b = 0; b < MB; ++b) {
+        int m = b * 16 + r16;
+        if (m >= M) m = M - 1;
+        xrow[b] = X + (size_t)m * K + g4 * 8;
+    }
+
+    const int mine = wave < nsteps ? (nsteps - wave + WAVES - 1) / WAVES : 0;   // this wave's steps
+    const int groups = mine / U;
+    SkinnyOperands<MB, NB> cur[U], nxt[U];
+
+#define SKINNY_LOAD(dst, group)                                                  \
+    _Pragma("unroll") for (int u = 0; u < U; ++u) {                              \
+        const int k = (wave + ((group) * U + u) * WAVES) * 32;                   \
+        _Pragma("unroll") for (int a = 0; a < NB; ++a)                           \
+            dst[u].w[a] = *(const bf16x8*)(wrow[a] + k);                         \
+        _Pragma("unroll") for (int b = 0; b < MB; ++b)                           \
+            dst[u].x[b] = *(const bf16x8*)(xrow[b] + k);                         \
+    }
+#define SKINNY_MULTIPLY(src)                                                     \
+    _Pragma("unroll") for (int u = 0; u < U; ++u)                                \
+        _Pragma("unroll") for (int a = 0; a < NB; ++a)                           \
+            _Pragma("unroll") for (int b = 0; b < MB; ++b)                       \
+                acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(src[u].w[a], src[u].x[b], acc[a][b], 0, 0, 0);
+
+    if (groups > 0) { SKINNY_LOAD(cur, 0) }
+    for (int g = 0; g < groups; g += 2) {
+        if (g + 1 < groups) { SKINNY_LOAD(nxt, g + 1) }
+        SKINNY_MULTIPLY(cur)
+        if (g + 1 < groups) {
+            if (g + 2 < groups) { SKINNY_LOAD(cur, g + 2) }
+            SKINNY_MULTIPLY(nxt)
+        }
+    }
+    for (int i = groups * U; i < mine; ++i) {       // what is left over of this wave's steps
+        const int k = (wave + i * WAVES) * 32;
+        bf16x8 wv[NB], xv[MB];
+#pragma unroll
+        for (int a = 0; a < NB; ++a) wv[a] = *(const bf16x8*)(wrow[a] + k);
+#pragma unroll
+        for (int b = 0; b < MB; ++b) xv[b] = *(const bf16x8*)(xrow[b] + k);
+#pragma unroll
+        for (int a = 0; a < NB; ++a)
+#pragma unroll
+            for (int b = 0; b < MB; ++b)
+                acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[a], xv[b], acc[a][b], 0, 0, 0);
+    }
+#undef SKINNY_LOAD
+#undef SKINNY_MULTIPLY
+
+    // a fixed tree over the waves: the upper half adds into the lower half, until wave 0 holds all
+    constexpr int REGS = NB * MB * 4;
+#pragma unroll
+    for (int half = WAVES / 2; half >= 1; half >>= 1) {
+        if (wave >= half && wave < 2 * half) {
+            float* dst = red + (size_t)(wave - half) * REGS * 64;
+#pragma unroll
+            for (int a = 0; a < NB; ++a)
+#pragma unroll
+                for (int b = 0; b < MB; ++b)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) dst[((a * MB + b) * 4 + i) * 64 + lane] = acc[a][b][i];
+        }
+        __syncthreads();
+        if (wave < half) {
+            const float* src = red + (size_t)wave * REGS * 64;
+#pragma unroll
+            for (int a = 0; a < NB; ++a)
+#pragma unroll
+                for (int b = 0; b < MB; ++b)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) acc[a][b][i] += src[((a * MB + b) * 4 + i) * 64 + lane];
+        }
+        __syncthreads();
+    }
+    if (wave != 0) return;
+
+    // lane: m = b * 16 + r16, n = n0 + a * 16 + g4 * 4 + i
+    if (EPI == EPI_SWIGLU) {
+        bf16* C = (bf16*)Cv;
+        const int out_n0 = n0 / 2;
+#pragma unroll
+        for (int a = 0; a + 1 < NB; a += 2)
+#pragma unroll
+            for (int b = 0; b < MB; ++b) {
+                const int m = b * 16 + r16;
+                if (m >= M) continue;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int n = out_n0 + (a / 2) * 16 + g4 * 4 + i;
+                    if (n < N / 2)
+                        C[(size_t)m * ldc + n] = hb_from_float<bf16>(silu_mul(acc[a][b][i], acc[a + 1][b][i]));
+                }
+            }
+    } else {
+        float* C = (float*)Cv;
+#pragma unroll
+        for (int a = 0; a < NB; ++a)
+#pragma unroll
+            for (int b = 0; b < MB; ++b) {
+                const int m = b * 16 + r16;
+                if (m >= M) continue;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int n = n0 + a * 16 + g4 * 4 + i;
+                    if (n < N) {
+                        const size_t idx = (size_t)m * ldc + n;
+                        if (EPI == EPI_ADD)
+                            C[idx] += acc[a][b][i];
+                        else
+                            C[idx] = acc[a][b][i];
+                    }
+                }
+            }
+    }
+}
+
+template <int MB, int NB, int WAVES>
+static void launch_skinny(const void* X, const void* W, void* C, int M, int N, int K, int ldc, int epi,
+                          hipStream_t stream) {
+    const int blocks = (N + NB * 16 - 1) / (NB * 16);
+    const size_t lds = (size_t)(WAVES / 2) * NB * MB * 4 * 64 * sizeof(float);
+    const bf16* x = (const bf16*)X;
+    const bf16* w = (const bf16*)W;
+    if (epi == EPI_STORE)
+        gemm_skinny_kernel<MB, NB, WAVES, EPI_STORE><<<blocks, WAVES * 64, lds, stream>>>(x, w, C, M, N, K, ldc);
+    else if (epi == EPI_ADD)
+        gemm_skinny_kernel<MB, NB, WAVES, EPI_ADD><<<blocks, WAVES * 64, lds, stream>>>(x, w, C, M, N, K, ldc);
+    else
+        gemm_skinny_kernel<MB, NB, WAVES, EPI_SWIGLU><<<blocks, WAVES * 64, lds, stream>>>(x, w, C, M, N, K,
+                                                                                        ldc);
+}
+
+template <int MB>
+static void pick_skinny(const void* X, const void* W, void* C, int M, int N, int K, int ldc, int epi,
+                        hipStream_t stream) {
+    // Few weight rows: one block of 16 rows a workgroup and eight waves splitting K, so that the
+    // 256 CUs all have work. Many rows: more rows a workgroup, so that the activations are
+    // re-read from L2 less often.
+    if (epi == EPI_SWIGLU || N >= 16384) {
+        launch_skinny<MB, 4, 4>(X, W, C, M, N, K, ldc, epi, stream);
+    } else {
+        launch_skinny<MB, 1, 8>(X, W, C, M, N, K, ldc, epi, stream);
+    }
+}
+
+// ------------------------------------------------------------------- tiled
+#define BM 128
+#define BN 128
+#define BK 64
+#define LDT (BK + 8)   // padded row of a tile in LDS, in elements: 144 bytes, conflict-free b128 reads
+
+template <int EPI>
+__global__ void __launch_bounds__(256)
+gemm_tiled_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* __restrict__ Cv, int M, int N,
+                  int K, int ldc, int m_tiles, int n_tiles) {
+    __shared__ __attribute__((aligned(16))) bf16 Ws[2][BN * LDT];
+    __shared__ __attribute__((aligned(16))) bf16 Xs[2][BM * LDT];
+
+    // workgroup ids go round the 8 XCDs; give each XCD a contiguous run of tiles so that the
+    // workgroups that share a weight tile also share an L2
+    const int total = m_tiles * n_tiles;
+    const int chunk = (total + 7) / 8;
+    const int id = (blockIdx.x % 8) * chunk + blockIdx.x / 8;
+    if (id >= total) return;
+    const int n_tile = id / m_tiles;
+    const int m_tile = id % m_tiles;
+    const int m0 = m_tile * BM, n0 = n_tile * BN;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wn = wave >> 1, wm = wave & 1;       // wave's 64 x 64 part of the tile
+    const int c32 = lane & 31, g2 = lane >> 5;
+
+    // global -> registers: 4 chunks of 16 bytes of each operand per thread
+    const int lrow = tid >> 3, lchunk = tid & 7;
+    const bf16* wsrc[4];
+    const bf16* xsrc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        int n = n0 + lrow + 32 * i;
+        if (n >= N) n = N - 1;
+        wsrc[i] = W + (size_t)n * K + lchunk * 8;
+        int m = m0 + lrow + 32 * i;
+        if (m >= M) m = M - 1;
+        xsrc[i] = X + (size_t)m * K + lchunk * 8;
+    }
+    bf16x8 wreg[4], xreg[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        wreg[i] = *(const bf16x8*)(wsrc[i]);
+        xreg[i] = *(const bf16x8*)(xsrc[i]);
+    }
+
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.f;
+
+    const int ktiles = K / BK;
+    for (int kt = 0; kt < ktiles; ++kt) {
+        const int buf = kt & 1;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            *(bf16x8*)(&Ws[buf][(lrow + 32 * i) * LDT + lchunk * 8]) = wreg[i];
+            *(bf16x8*)(&Xs[buf][(lrow + 32 * i) * LDT + lchunk * 8]) = xreg[i];
+        }
+        __syncthreads();
+        if (kt + 1 < ktiles) {
+            const int koff = (kt + 1) * BK;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                wreg[i] = *(const bf16x8*)(wsrc[i] + koff);
+                xreg[i] = *(const bf16x8*)(xsrc[i] + koff);
+            }
+        }
+#pragma unroll
+        for (int ks = 0; ks < BK / 16; ++ks) {
+            bf16x8 wa[2], xb[2];
+#pragma unroll
+            for (int a = 0; a < 2; ++a)
+                wa[a] = *(const bf16x8*)(&Ws[buf][(wn * 64 + a * 32 + c32) * LDT + ks * 16 + g2 * 8]);
+#pragma unroll
+            for (int b = 0; b < 2; ++b)
+                xb[b] = *(const bf16x8*)(&Xs[buf][(wm * 64 + b * 32 + c32) * LDT + ks * 16 + g2 * 8]);
+#pragma unroll
+            for (int a = 0; a < 2; ++a)
+#pragma unroll
+                for (int b = 0; b < 2; ++b)
+                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wa[a], xb[b], acc[a][b], 0, 0, 0);
+        }
+        // the other buffer is written next; everyone has finished reading it a tile ago
+    }
+
+    // lane: m = m0 + wm*64 + b*32 + c32 ; n = n0 + wn*64 + a*32 + 8*(i/4) + 4*g2 + i%4
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+        const int m = m0 + wm * 64 + b * 32 + c32;
+        if (m >= M) continue;
+        if (EPI == EPI_SWIGLU) {
+            // weight rows come in blocks of 16 gate rows then 16 up rows: within a 32-row MFMA block,
+            // rows 0..15 (i/4 in {0,1}) are gate and rows 16..31 (i/4 in {2,3}) the matching up rows
+            bf16* C = (bf16*)Cv;
+#pragma unroll
+            for (int a = 0; a < 2; ++a)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const int fused_n = n0 + wn * 64 + a * 32;            // start of a gate/up pair
+                    const int n = fused_n / 2 + 8 * (i / 4) + 4 * g2 + (i % 4);
+                    if (n < N / 2)
+                        C[(size_t)m * ldc + n] =
+                            hb_from_float<bf16>(silu_mul(acc[a][b][i], acc[a][b][i + 8]));
+                }
+        } else {
+            float* C = (float*)Cv;
+#pragma unroll
+            for (int a = 0; a < 2; ++a)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int n = n0 + wn * 64 + a * 32 + 8 * q + 4 * g2;
+                    float* dst = C + (size_t)m * ldc + n;
+                    if (n + 3 < N && (ldc & 3) == 0) {
+                        f32x4 v = {acc[a][b][4 * q], acc[a][b][4 * q + 1], acc[a][b][4 * q + 2],
+                                   acc[a][b][4 * q + 3]};
+                        if (EPI == EPI_ADD) {
+                            const f32x4 old = *(const f32x4*)dst;
+                            v += old;
+                        }
+                        *(f32x4*)dst = v;
+                    } else {
+#pragma unroll
+                        for (int r = 0; r < 4; ++r)
+                            if (n + r < N) {
+                                if (EPI == EPI_ADD)
+                                    dst[r] += acc[a][b][4 * q + r];
+                                else
+                                    dst[r] = acc[a][b][4 * q + r];
+                            }
+                    }
+                }
+        }
+    }
+}
+
+// C (+)= X @ W^T. X [M, K] bf16, W [N, K] bf16. epi 0: C f32 [M, N] stored; 1: added to;
+// 2: W's rows are gate/up interleaved in blocks of 16 and C is bf16 [M, N / 2] = silu(gate) * up.
+extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N, int K, int ldc, int epi,
+                            hipStream_t stream) {
+    HB_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_mfma: empty problem (M=%d, N=%d, K=%d)", M, N, K);
+    HB_REQUIRE(epi >= 0 && epi <= 2, "gemm_mfma: unknown epilogue %d", epi);
+    HB_REQUIRE(K % 32 == 0, "gemm_mfma: K=%d is no multiple of 32", K);
+    HB_REQUIRE(epi != EPI_SWIGLU || N % 32 == 0, "gemm_mfma: the SwiGLU epilogue needs N %% 32 == 0");
+    HB_REQUIRE(ldc >= (epi == EPI_SWIGLU ? N / 2 : N), "gemm_mfma: output row stride %d too small", ldc);
+    if (M <= 64) {
+        if (M <= 16) pick_skinny<1>(X, W, C, M, N, K, ldc, epi, stream);
+        else if (M <= 32) pick_skinny<2>(X, W, C, M, N, K, ldc, epi, stream);
+        else if (M <= 48) pick_skinny<3>(X, W, C, M, N, K, ldc, epi, stream);
+        else pick_skinny<4>(X, W, C, M, N, K, ldc, epi, stream);
+        HB_CHECK_LAUNCH("gemm_skinny");
+        return 0;
+    }
+    HB_REQUIRE(K % BK == 0, "gemm_mfma: K=%d is no multiple of %d (needed for M > 64)", K, BK);
+    const int m_tiles = (M + BM - 1) / BM, n_tiles = (N + BN - 1) / BN;
+    const long total = (long)m_tiles * n_tiles;
+    HB_REQUIRE(total < (1l << 30), "gemm_mfma: too many tiles");
+    const int blocks = (int)((total + 7) / 8 * 8);
+    const bf16* x = (const bf16*)X;
+    const bf16* w = (const bf16*)W;
+    if (epi == EPI_STORE)
+        gemm_tiled_kernel<EPI_STORE><<<blocks, 256, 0, stream>>>(x, w, C, M, N, K, ldc, m_tiles, n_tiles);
+    else if (epi == EPI_ADD)
+        gemm_tiled_kernel<EPI_ADD><<<blocks, 256, 0, stream>>>(x, w, C, M, N, K, ldc, m_tiles, n_tiles);
+    else
+        gemm_tiled_kernel<EPI_SWIGLU><<<blocks, 256, 0, stream>>>(x, w, C, M, N, K, ldc, m_tiles, n_tiles);
+    HB_CHECK_LAUNCH("gemm_tiled");
+    return 0;
+}

@@ -32,6 +32,7 @@ class BatchMeta:
     max_position: int          # largest absolute position in the step
     host_starts: np.ndarray    # host copies, for kernels' grids
     host_context: np.ndarray
+    derived: dict = None       # what kernels' host sides derive once a step (tile lists and the like)
 
 
 def pack(entries, start_lengths, device, staging=None):
@@ -73,4 +74,4 @@ def pack(entries, start_lengths, device, staging=None):
         slots=dev[o:o + B], seq_starts=dev[o + B:o + 2 * B + 1],
         context_lens=dev[o + 2 * B + 1:o + 3 * B + 1], want_rows=dev[o + 3 * B + 1:o + 3 * B + 1 + R],
         num_tokens=T, num_seqs=B, max_new=max(counts), max_context=int(ctx.max()),
-        max_position=int(pos.max()), host_starts=starts.copy(), host_context=ctx.copy())
+        max_position=int(pos.max()), host_starts=starts.copy(), host_context=ctx.copy(), derived={})

@@ -1,9 +1,158 @@
-"""Host side of the bfloat16 MFMA kernels (matrix products and attention)."""
+"""Host side of the bfloat16 MFMA kernels (matrix products and attention): which shapes they
+take, operand checks, launches. What they refuse goes to the plain kernels."""
+import ctypes
+
+import torch
+
+from ..errors import BackendError
+from . import lib
+from .ops import _check, _stream
+
+_P = ctypes.c_void_p
+_I = ctypes.c_int
+_F = ctypes.c_float
+lib.register_signatures("gemm_mfma", {
+    "hb_gemm_mfma": [_P, _P, _P, _I, _I, _I, _I, _I, _P],
+})
+
+EPI_STORE, EPI_ADD, EPI_SWIGLU = 0, 1, 2
+SKINNY_MAX_M = 64
 
 
-def gemm_supported(a, w, out):
-    return False
+def gemm_supported(a, w, out=None, swiglu=False):
+    """True if hb_gemm_mfma takes this product (bfloat16 operands, K in steps of 32, or of 64 for
+    more than 64 rows; the SwiGLU epilogue pairs blocks of 16 rows)."""
+    if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        return False
+    M, K = a.shape
+    N = w.shape[0]
+    if K % 32 or (M > SKINNY_MAX_M and K % 64):
+        return False
+    if swiglu:
+        return N % 32 == 0
+    return out is None or out.dtype == torch.float32
+
+
+def gemm(a, w, out, accumulate=False):
+    """out f32 [M, N] (+)= a bf16 [M, K] @ w bf16 [N, K]^T."""
+    _check(a, "a", torch.bfloat16, (None, None))
+    M, K = a.shape
+    _check(w, "w", torch.bfloat16, (None, K))
+    N = w.shape[0]
+    _check(out, "out", torch.float32, (M, N))
+    if not gemm_supported(a, w, out):
+        raise BackendError(f"gemm_mfma refuses M={M}, N={N}, K={K}")
+    lib.call("gemm_mfma", "hb_gemm_mfma", a.data_ptr(), w.data_ptr(), out.data_ptr(), M, N, K, N,
+             EPI_ADD if accumulate else EPI_STORE, _stream())
+
+
+def interleave_gate_up(gate, up):
+    """[2I, K] with blocks of 16 gate rows followed by the 16 up rows of the same outputs:
+    the row order the SwiGLU epilogue expects."""
+    I, K = gate.shape
+    if I % 16 or up.shape != gate.shape:
+        raise BackendError("gate and up must have the same shape with rows in steps of 16")
+    return torch.stack([gate.view(I // 16, 16, K), up.view(I // 16, 16, K)], 1).reshape(2 * I, K).contiguous()
+
+
+def gemm_swiglu(a, w_interleaved, out):
+    """out bf16 [M, I] = silu(a @ gate^T) * (a @ up^T), the weights interleaved as above."""
+    _check(a, "a", torch.bfloat16, (None, None))
+    M, K = a.shape
+    _check(w_interleaved, "w", torch.bfloat16, (None, K))
+    N = w_interleaved.shape[0]
+    _check(out, "out", torch.bfloat16, (M, N // 2))
+    if not gemm_supported(a, w_interleaved, swiglu=True):
+        raise BackendError(f"gemm_mfma (SwiGLU) refuses M={M}, N={N}, K={K}")
+    lib.call("gemm_mfma", "hb_gemm_mfma", a.data_ptr(), w_interleaved.data_ptr(), out.data_ptr(), M, N, K,
+             N // 2, EPI_SWIGLU, _stream())
+
+
+lib.register_signatures("attention_mfma", {
+    "hb_attn_prefill_mfma": [_P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P],
+    "hb_attn_decode_mfma": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P],
+})
+
+ATTENTION_HEAD_DIMS = (32, 64, 128)
+QUERY_TILE = 32
+_partials = {}
 
 
 def attention_supported(q, kv, nq, nkv, hd):
-    return False
+    """bfloat16, pages of 64 tokens, a head size the kernels are built for, at most 32 query heads
+    to a kv head."""
+    return (q.dtype == torch.bfloat16 and kv.k.dtype == torch.bfloat16 and kv.page_size == 64
+            and hd in ATTENTION_HEAD_DIMS and nq % nkv == 0 and nq // nkv <= 32)
+
+
+def _prefill_tiles(meta):
+    """Device arrays (sequence, first packed row, rows) of the 32-token query tiles of a step."""
+    tiles = meta.derived.get("prefill_tiles")
+    if tiles is None:
+        seq, row0, rows = [], [], []
+        starts = meta.host_starts
+        for i in range(meta.num_seqs):
+            a, b = int(starts[i]), int(starts[i + 1])
+            for r in range(a, b, QUERY_TILE):
+                seq.append(i)
+                row0.append(r)
+                rows.append(min(QUERY_TILE, b - r))
+        packed = torch.tensor([seq, row0, rows], dtype=torch.int32).to(meta.positions.device)
+        tiles = (packed[0], packed[1], packed[2], len(seq))
+        meta.derived["prefill_tiles"] = tiles
+    return tiles
+
+
+def _decode_split(meta, nkv, window):
+    """(ranges, pages per range): enough waves for the 256 CUs, every range at least one page."""
+    span = (meta.max_context + 63) // 64
+    if window:
+        span = min(span, (window + 63) // 64 + 1)
+    want = max(1, -(-1024 // (meta.num_seqs * nkv)))
+    splits = max(1, min(span, want))
+    per = -(-span // splits)
+    return -(-span // per), per
+
+
+def _partial_buffers(device, n_rows, splits, hd):
+    key = str(device)
+    need_o = n_rows * splits * hd
+    buf = _partials.get(key)
+    if buf is None or buf[0].numel() < need_o or buf[1].numel() < n_rows * splits * 2:
+        buf = (torch.empty(need_o, dtype=torch.float32, device=device),
+               torch.empty(n_rows * splits * 2, dtype=torch.float32, device=device))
+        _partials[key] = buf
+    return buf
+
+
+def attention(q, meta, kv, out, nq, nkv, hd, scale, window):
+    """Causal (and windowed) attention of the step's tokens over their slots' pages.
+    One token a sequence: the split decode kernel; otherwise the tiled prefill kernel."""
+    T = q.shape[0]
+    _check(q, "q", torch.bfloat16, (T, nq * hd))
+    _check(out, "out", torch.bfloat16, (T, nq * hd))
+    pages = kv.k.shape[0]
+    _check(kv.k, "key pages", torch.bfloat16, (pages, nkv, 64, hd))
+    _check(kv.v, "value pages", torch.bfloat16, (pages, nkv, hd, 64))
+    _check(kv.page_table, "page_table", torch.int32, (None, None))
+    _check(meta.slots, "slots", torch.int32, (meta.num_seqs,))
+    if not attention_supported(q, kv, nq, nkv, hd):
+        raise BackendError(f"attention_mfma refuses head_dim {hd} with {nq}/{nkv} heads")
+    window = int(window or 0)
+    if meta.max_new == 1:
+        if T != meta.num_seqs:
+            raise BackendError("decode attention needs one token for each sequence")
+        _check(meta.context_lens, "context_lens", torch.int32, (T,))
+        splits, per = _decode_split(meta, nkv, window)
+        po, pml = _partial_buffers(q.device, T * nq, splits, hd)
+        lib.call("attention_mfma", "hb_attn_decode_mfma", q.data_ptr(), kv.k.data_ptr(), kv.v.data_ptr(),
+                 out.data_ptr(), po.data_ptr(), pml.data_ptr(), meta.context_lens.data_ptr(),
+                 meta.slots.data_ptr(), kv.page_table.data_ptr(), kv.page_table.shape[1], kv.page_size,
+                 T, nq, nkv, hd, float(scale), window, splits, per, _stream())
+        return
+    _check(meta.positions, "positions", torch.int32, (T,))
+    tile_seq, tile_row0, tile_rows, n_tiles = _prefill_tiles(meta)
+    lib.call("attention_mfma", "hb_attn_prefill_mfma", q.data_ptr(), kv.k.data_ptr(), kv.v.data_ptr(),
+             out.data_ptr(), tile_seq.data_ptr(), tile_row0.data_ptr(), tile_rows.data_ptr(), n_tiles,
+             meta.positions.data_ptr(), meta.slots.data_ptr(), kv.page_table.data_ptr(),
+             kv.page_table.shape[1], kv.page_size, nq, nkv, hd, float(scale), window, _stream())

@@ -88,7 +88,8 @@ def _check_paged(meta, cache, T):
     _check(meta.slots, "slots", torch.int32, (None,))
     _check(cache.page_table, "page_table", torch.int32, (None, None))
     _check(cache.k, "key pages", None, (None, None, cache.page_size, None))
-    _check(cache.v, "value pages", cache.k.dtype, tuple(cache.k.shape))
+    pages, nkv, page, hd = cache.k.shape
+    _check(cache.v, "value pages", cache.k.dtype, (pages, nkv, hd, page))
 
 
 def qk_norm_rope_write(qkv, q_norm_w, k_norm_w, cos, sin, rot_dims, meta, cache, q_out, nq, nkv, hd, eps,

@@ -21,6 +21,7 @@ class SwiGLU(Part):
         self.intermediate_size = int(intermediate_size)
         self.names = dict(names)
         self.gate_up = self.down = None
+        self.fused_epilogue = False
 
     def tensor_needs(self):
         n = self.names
@@ -30,15 +31,28 @@ class SwiGLU(Part):
 
     def load(self, tensors, rt):
         n = self.names
-        fused = torch.cat([tensors[n["gate"]].to(rt.device), tensors[n["up"]].to(rt.device)], 0)
-        self.gate_up = Linear(rt.weight(fused))
+        gate, up = rt.weight(tensors[n["gate"]]), rt.weight(tensors[n["up"]])
+        # bfloat16 with sizes the MFMA kernel takes: gate and up rows interleaved so that the
+        # product's epilogue applies silu(gate) * up and the float32 [T, 2I] never exists
+        from ..kernels import mfma
+        self.fused_epilogue = (rt.dtype == torch.bfloat16 and self.intermediate_size % 16 == 0
+                               and self.hidden_size % 64 == 0 and mfma.gemm_supported(
+                                   gate[:1], gate, swiglu=True))
+        if self.fused_epilogue:
+            self.gate_up = Linear(mfma.interleave_gate_up(gate, up))
+        else:
+            self.gate_up = Linear(torch.cat([gate, up], 0))
         self.down = Linear(rt.weight(tensors[n["down"]]))
 
     def forward(self, ctx, y, x):
         rt = ctx.rt
         T = y.shape[0]
-        gu = rt.buffer("gate_up", (T, 2 * self.intermediate_size), torch.float32)
-        self.gate_up.forward(y, gu)
         act = rt.buffer("act", (T, self.intermediate_size))
-        ops.swiglu(gu, act)
+        if self.fused_epilogue:
+            from ..kernels import mfma
+            mfma.gemm_swiglu(y, self.gate_up.weight, act)
+        else:
+            gu = rt.buffer("gate_up", (T, 2 * self.intermediate_size), torch.float32)
+            self.gate_up.forward(y, gu)
+            ops.swiglu(gu, act)
         self.down.forward(act, x, accumulate=True)

@@ -1,0 +1,260 @@
+"""Each kernel alone against a plain float32 formulation in torch, at sizes other than the
+engine's: odd widths, heads and groups, sizes at and across tile edges."""
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def dev():
+    return torch.device("cuda", 0)
+
+
+def rand(*shape, seed=0, scale=1.0, dtype=torch.float32):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(dev())
+
+
+# ---------------------------------------------------------------- plain kernels
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_embed(dtype):
+    from herbert_rs_amd.kernels import ops
+    table = rand(37, 50, dtype=dtype)
+    ids = torch.tensor([0, 36, 5, 5, 17], dtype=torch.int32, device=dev())
+    out = torch.empty(5, 50, device=dev())
+    ops.embed(ids, table, out)
+    assert torch.equal(out, table[ids.long()].float())
+
+
+@pytest.mark.parametrize("H", [64, 96, 1000, 4096, 5120])
+def test_rmsnorm(H):
+    from herbert_rs_amd.kernels import ops
+    x = rand(7, H, seed=1, scale=3.0)
+    w = 1 + 0.1 * rand(H, seed=2)
+    for eps in (1e-6, 1e-5):
+        want = x * torch.rsqrt((x.double() ** 2).mean(-1, keepdim=True) + eps).float() * w
+        out = torch.empty_like(x)
+        ops.rmsnorm(x, w, out, eps)
+        assert torch.allclose(out, want, rtol=2e-6, atol=1e-6)
+    rows = torch.tensor([6, 0, 3], dtype=torch.int32, device=dev())
+    out = torch.empty(3, H, dtype=torch.bfloat16, device=dev())
+    ops.rmsnorm(x, w, out, 1e-6, rows)
+    want = (x[rows.long()] * torch.rsqrt((x[rows.long()] ** 2).mean(-1, keepdim=True) + 1e-6) * w)
+    assert torch.allclose(out.float(), want, rtol=2 ** -8, atol=1e-6)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 7, 5), (3, 65, 33), (64, 64, 16), (70, 130, 100), (129, 31, 257)])
+@pytest.mark.parametrize("dts", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16),
+                                 (torch.float32, torch.bfloat16)])
+def test_gemm_plain(M, N, K, dts):
+    from herbert_rs_amd.kernels import ops
+    a = rand(M, K, seed=3, dtype=dts[0])
+    w = rand(N, K, seed=4, dtype=dts[1])
+    want = (a.double() @ w.double().T).float()
+    c = torch.empty(M, N, device=dev())
+    ops.gemm_plain(a, w, c)
+    assert torch.allclose(c, want, rtol=1e-5, atol=1e-5 * math.sqrt(K))
+    base = rand(M, N, seed=5)
+    c2 = base.clone()
+    ops.gemm_plain(a, w, c2, accumulate=True)
+    assert torch.allclose(c2, base + want, rtol=1e-5, atol=1e-5 * math.sqrt(K))
+    cb = torch.empty(M, N, dtype=torch.bfloat16, device=dev())
+    ops.gemm_plain(a, w, cb)
+    assert torch.allclose(cb.float(), want, rtol=2 ** -8, atol=1e-3)
+
+
+@pytest.mark.parametrize("I", [5, 128, 1000])
+def test_swiglu(I):
+    from herbert_rs_amd.kernels import ops
+    gu = rand(6, 2 * I, seed=6, scale=4.0)
+    gu[0, 0] = -90.0
+    gu[0, 1] = 0.0
+    want = torch.nn.functional.silu(gu[:, :I]) * gu[:, I:]
+    out = torch.empty(6, I, device=dev())
+    ops.swiglu(gu, out)
+    assert torch.allclose(out, want, rtol=1e-5, atol=1e-6) and torch.isfinite(out).all()
+
+
+# ------------------------------------------------------------------ MFMA GEMM
+MFMA_SHAPES = [(1, 48, 32), (8, 4096, 4096), (16, 272, 96), (17, 1000, 224), (33, 96, 64), (48, 100, 128),
+               (64, 24576, 512), (65, 128, 64), (128, 256, 128), (200, 330, 192), (2048, 512, 4096)]
+
+
+@pytest.mark.parametrize("M,N,K", MFMA_SHAPES)
+def test_gemm_mfma_store_and_add(M, N, K):
+    from herbert_rs_amd.kernels import mfma
+    a = rand(M, K, seed=7, dtype=torch.bfloat16)
+    w = rand(N, K, seed=8, dtype=torch.bfloat16)
+    assert mfma.gemm_supported(a, w)
+    want = (a.double() @ w.double().T).float()
+    c = torch.full((M, N), 7.0, device=dev())
+    mfma.gemm(a, w, c)
+    tol = 2e-6 * K ** 0.5 * float(want.abs().max()) + 1e-4      # float32 accumulation of exact products
+    assert float((c - want).abs().max()) <= tol
+    base = rand(M, N, seed=9)
+    c2 = base.clone()
+    mfma.gemm(a, w, c2, accumulate=True)
+    assert float((c2 - (base + want)).abs().max()) <= tol
+
+
+@pytest.mark.parametrize("M,I,K", [(1, 16, 32), (8, 12288, 4096), (40, 48, 96), (64, 1024, 64),
+                                   (100, 176, 128), (300, 256, 64)])
+def test_gemm_mfma_swiglu(M, I, K):
+    from herbert_rs_amd.kernels import mfma
+    a = rand(M, K, seed=10, dtype=torch.bfloat16, scale=0.5)
+    gate = rand(I, K, seed=11, dtype=torch.bfloat16, scale=0.3)
+    up = rand(I, K, seed=12, dtype=torch.bfloat16, scale=0.3)
+    w = mfma.interleave_gate_up(gate, up)
+    g = a.double() @ gate.double().T
+    u = a.double() @ up.double().T
+    want = (g / (1 + torch.exp(-g)) * u).float()
+    out = torch.empty(M, I, dtype=torch.bfloat16, device=dev())
+    mfma.gemm_swiglu(a, w, out)
+    err = (out.float() - want).abs()
+    assert float((err - 2 ** -8 * want.abs()).max()) <= 1e-3 * float(want.abs().max()) + 1e-5
+
+
+def test_gemm_mfma_refuses_what_it_cannot_do():
+    from herbert_rs_amd.kernels import mfma
+    a = rand(4, 40, dtype=torch.bfloat16)
+    w = rand(8, 40, dtype=torch.bfloat16)
+    assert not mfma.gemm_supported(a, w)
+    assert not mfma.gemm_supported(rand(100, 96, dtype=torch.bfloat16), rand(8, 96, dtype=torch.bfloat16))
+    assert not mfma.gemm_supported(a.float(), w)
+
+
+# ------------------------------------------------------------------ attention
+class FakeMeta:
+    pass
+
+
+def paged_case(lengths, new_counts, nkv, hd, dtype, seed=0, n_pages=64, shuffle=True):
+    """A cache filled with random keys and values for sequences of the given lengths, the last
+    new_counts[i] positions of each being the step's tokens. Returns (meta, kv, K, V) with K, V
+    the dense per-sequence tensors [len, nkv, hd]."""
+    from herbert_rs_amd.cache.paged import LayerKV
+    g = torch.Generator().manual_seed(seed)
+    pages_per_slot = 16
+    B = len(lengths)
+    table = torch.zeros(B + 2, pages_per_slot, dtype=torch.int32)
+    order = torch.randperm(n_pages, generator=g).tolist() if shuffle else list(range(n_pages))
+    k_pool = torch.zeros(n_pages, nkv, 64, hd)
+    v_pool = torch.zeros(n_pages, nkv, hd, 64)
+    dense = []
+    slots = [b + 1 for b in range(B)]          # slot ids differ from batch indices
+    for b, n in enumerate(lengths):
+        K = torch.randn(n, nkv, hd, generator=g).to(dtype).float()
+        V = torch.randn(n, nkv, hd, generator=g).to(dtype).float()
+        dense.append((K, V))
+        for p in range((n + 63) // 64):
+            page = order.pop()
+            table[slots[b], p] = page
+            chunk = slice(p * 64, min(n, (p + 1) * 64))
+            cnt = chunk.stop - chunk.start
+            k_pool[page, :, :cnt] = K[chunk].transpose(0, 1)
+            v_pool[page, :, :, :cnt] = V[chunk].permute(1, 2, 0)
+    kv = LayerKV(k_pool.to(dtype).to(dev()), v_pool.to(dtype).to(dev()), table.to(dev()), 64, 0)
+    meta = FakeMeta()
+    pos, seq = [], []
+    starts = [0]
+    for b, (n, c) in enumerate(zip(lengths, new_counts)):
+        pos += list(range(n - c, n))
+        seq += [b] * c
+        starts.append(starts[-1] + c)
+    meta.positions = torch.tensor(pos, dtype=torch.int32, device=dev())
+    meta.seq_of = torch.tensor(seq, dtype=torch.int32, device=dev())
+    meta.slots = torch.tensor(slots, dtype=torch.int32, device=dev())
+    meta.context_lens = torch.tensor(lengths, dtype=torch.int32, device=dev())
+    meta.num_seqs, meta.num_tokens = B, len(pos)
+    meta.max_new, meta.max_context, meta.max_position = max(new_counts), max(lengths), max(lengths) - 1
+    import numpy as np
+    meta.host_starts = np.array(starts, dtype=np.int32)
+    meta.derived = {}
+    return meta, kv, dense
+
+
+def attention_reference(q, meta, dense, nq, nkv, hd, scale, window):
+    out = torch.zeros(q.shape[0], nq, hd)
+    qf = q.float().cpu().view(-1, nq, hd)
+    pos = meta.positions.cpu().tolist()
+    seq = meta.seq_of.cpu().tolist()
+    for t in range(q.shape[0]):
+        K, V = dense[seq[t]]
+        lo = max(0, pos[t] + 1 - window) if window else 0
+        for h in range(nq):
+            g = h // (nq // nkv)
+            s = (K[lo:pos[t] + 1, g] @ qf[t, h]) * scale
+            p = torch.softmax(s.double(), 0).float()
+            out[t, h] = (p[:, None] * V[lo:pos[t] + 1, g]).sum(0)
+    return out.view(q.shape[0], nq * hd)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nq,nkv,hd,window", [(4, 2, 16, 0), (6, 2, 32, 0), (5, 1, 48, 70), (3, 3, 80, 0),
+                                              (2, 1, 256, 130)])
+def test_attention_plain(nq, nkv, hd, window, dtype):
+    from herbert_rs_amd.kernels import ops
+    lengths, new = [5, 200, 64, 129], [5, 70, 1, 129]
+    meta, kv, dense = paged_case(lengths, new, nkv, hd, dtype, seed=nq)
+    q = rand(sum(new), nq * hd, seed=20, dtype=dtype)
+    out = torch.empty_like(q)
+    scale = hd ** -0.5
+    ops.attention_plain(q, meta, kv, out, nq, nkv, hd, scale, window)
+    want = attention_reference(q, meta, dense, nq, nkv, hd, scale, window)
+    tol = 2e-5 if dtype == torch.float32 else 2 ** -7
+    assert float((out.float().cpu() - want).abs().max()) <= tol * float(want.abs().max())
+
+
+@pytest.mark.parametrize("nq,nkv,hd,window", [(4, 1, 128, 0), (8, 2, 64, 0), (6, 2, 32, 0), (5, 1, 64, 70),
+                                              (3, 3, 128, 100), (16, 2, 128, 0), (2, 2, 32, 0)])
+def test_attention_mfma_prefill(nq, nkv, hd, window):
+    from herbert_rs_amd.kernels import mfma
+    lengths, new = [5, 200, 64, 129, 33, 300], [5, 70, 2, 129, 32, 300]
+    meta, kv, dense = paged_case(lengths, new, nkv, hd, torch.bfloat16, seed=nq + hd)
+    q = rand(sum(new), nq * hd, seed=21, dtype=torch.bfloat16)
+    out = torch.full_like(q, 9.0)
+    scale = hd ** -0.5
+    assert mfma.attention_supported(q, kv, nq, nkv, hd)
+    mfma.attention(q, meta, kv, out, nq, nkv, hd, scale, window)
+    want = attention_reference(q, meta, dense, nq, nkv, hd, scale, window)
+    # probabilities and the output are rounded to bfloat16 (2^-9 each)
+    assert float((out.float().cpu() - want).abs().max()) <= 2 ** -7 * float(want.abs().max())
+
+
+@pytest.mark.parametrize("nq,nkv,hd,window", [(4, 1, 128, 0), (32, 8, 128, 0), (6, 2, 32, 0), (5, 1, 64, 70),
+                                              (3, 3, 128, 100), (64, 2, 64, 0)])
+@pytest.mark.parametrize("lengths", [[1, 64, 65, 700], [1000], [130, 3, 512, 999, 77, 640, 64, 128, 256]])
+def test_attention_mfma_decode(nq, nkv, hd, window, lengths):
+    from herbert_rs_amd.kernels import mfma
+    meta, kv, dense = paged_case(lengths, [1] * len(lengths), nkv, hd, torch.bfloat16, seed=nq + hd,
+                                 n_pages=80)
+    q = rand(len(lengths), nq * hd, seed=22, dtype=torch.bfloat16)
+    out = torch.full_like(q, 9.0)
+    scale = hd ** -0.5
+    mfma.attention(q, meta, kv, out, nq, nkv, hd, scale, window)
+    want = attention_reference(q, meta, dense, nq, nkv, hd, scale, window)
+    assert float((out.float().cpu() - want).abs().max()) <= 2 ** -7 * float(want.abs().max())
+
+
+def test_attention_finds_one_far_key_among_hundreds():
+    """One key far back scores far above the rest: the output must be its value, whichever page
+    and split it lies in. Random keys would hide a page or a split that is skipped."""
+    from herbert_rs_amd.kernels import mfma, ops
+    nq, nkv, hd = 4, 1, 64
+    for n, target in ((900, 3), (900, 64 * 7 + 63), (900, 899), (257, 192)):
+        for mode in ("decode", "prefill"):
+            new = 1 if mode == "decode" else 40
+            meta, kv, dense = paged_case([n], [new], nkv, hd, torch.bfloat16, seed=target)
+            K, V = dense[0]
+            q = torch.zeros(new, nq * hd)
+            q[:, :] = (K[target, 0] * 8).repeat(nq)          # aligned with that key, scaled up
+            q = q.to(torch.bfloat16).to(dev())
+            if target >= n - new:
+                continue
+            for fn in (mfma.attention, ops.attention_plain):
+                out = torch.empty_like(q)
+                fn(q, meta, kv, out, nq, nkv, hd, 1.0, 0)
+                got = out.float().cpu().view(new, nq, hd)
+                assert float((got - V[target, 0]).abs().max()) < 0.02, (n, target, mode, fn.__name__)
