@@ -1,0 +1,269 @@
+"""The engine through its Python entry points: long decoding, greedy generation, slots used
+again, the window's edge, errors of the step function, sampling on the GPU."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import herbert_rs_amd as hb
+from herbert_rs_amd.engine import StepEntry
+from herbert_rs_amd.errors import CacheError, RequestError
+
+from .plain import model as plain
+from .plain import sampler as plain_sampler
+from .plain_cache import plain_folder, plain_logits
+from .tiny import CONFIGS, make_folder, random_tokens
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def close(got, ref, dtype):
+    err = float(np.abs(got - ref).max())
+    if dtype == "float32":
+        return err <= 1e-4, err
+    rms = float(np.sqrt((ref.astype(np.float64) ** 2).mean()))
+    return err <= 0.05 * rms, err
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["B", "C"])
+def test_long_decoding_one_token_at_a_time(name, dtype, model_root):
+    """A short prompt, then hundreds of single tokens: across page edges, beyond the window, up
+    to the model's last position."""
+    folder = make_folder(model_root, name, dtype)
+    raw = CONFIGS[name][0]
+    n = raw["max_position_embeddings"] if name == "B" else 330
+    tokens = random_tokens(raw["vocab_size"], n, 5)
+    engine = hb.load(folder, dtype=dtype, cache_tokens=n + 64)
+    slot = engine.alloc_slot()
+    ref = plain_logits(folder, tokens)
+    got = [engine.step([StepEntry(slot, tokens[:3], [0, 1, 2])]).cpu().numpy()]
+    for p in range(3, n):
+        got.append(engine.step([StepEntry(slot, [tokens[p]], [0])]).cpu().numpy())
+    got = np.concatenate(got)
+    for p in range(n):
+        ok, err = close(got[p], ref[p], dtype)
+        assert ok, f"position {p}: err {err}"
+    if name == "B":
+        with pytest.raises(RequestError, match="max_position_embeddings"):
+            engine.step([StepEntry(slot, [1], [0])])
+    engine.free_slot(slot)
+    engine.cache.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_chunks_of_a_prompt_and_slots_used_again(dtype, model_root):
+    """A prompt fed in uneven pieces gives the logits of the whole; a slot that held another
+    sequence gives the same logits as a fresh one."""
+    folder = make_folder(model_root, "C", dtype)
+    vocab = CONFIGS["C"][0]["vocab_size"]
+    a, b = random_tokens(vocab, 150, 8), random_tokens(vocab, 90, 9)
+    engine = hb.load(folder, dtype=dtype, cache_tokens=64 * 6)
+    s = engine.alloc_slot()
+    whole = engine.step([StepEntry(s, a, list(range(len(a))))]).cpu().numpy()
+    engine.free_slot(s)
+    s2 = engine.alloc_slot()
+    assert s2 == s
+    engine.step([StepEntry(s2, b, [])])                       # leaves other keys in the pages
+    engine.free_slot(s2)
+    s3 = engine.alloc_slot()
+    pieces, at = [], 0
+    for n in (1, 63, 1, 20, 65):
+        pieces.append(engine.step([StepEntry(s3, a[at:at + n], list(range(n)))]).cpu().numpy())
+        at += n
+    pieces = np.concatenate(pieces)
+    ref = plain_logits(folder, a)
+    for p in range(len(a)):
+        assert close(whole[p], ref[p], dtype)[0] and close(pieces[p], ref[p], dtype)[0], p
+    if dtype == "float32":
+        assert float(np.abs(pieces - whole).max()) <= 2e-5
+    engine.free_slot(s3)
+    engine.cache.check()
+
+
+def test_window_edge_shows_in_the_logits(model_root):
+    """Config C's first layer sees 70 keys. Changing the token just outside every later query's
+    window must change nothing there; changing the one just inside must."""
+    folder = make_folder(model_root, "C", "float32")
+    raw = CONFIGS["C"][0]
+    base = random_tokens(raw["vocab_size"], 120, 12)
+    engine = hb.load(folder, dtype="float32", cache_tokens=256)
+
+    def last_logits(tokens):
+        s = engine.alloc_slot()
+        out = engine.step([StepEntry(s, tokens, [len(tokens) - 1])]).cpu().numpy()[0]
+        engine.free_slot(s)
+        return out
+    ref = last_logits(base)
+    assert float(np.abs(ref - plain_logits(folder, base)[-1]).max()) <= 1e-4
+    # the second layer sees everything, so any earlier token reaches the last logits; the check
+    # is therefore made against the plain implementation on both sides of the edge
+    for changed in (119 - 70, 119 - 69):
+        other = list(base)
+        other[changed] = (other[changed] + 1) % raw["vocab_size"]
+        got = last_logits(other)
+        assert float(np.abs(got - plain_logits(folder, other)[-1]).max()) <= 1e-4
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_greedy_generation_through_the_entry_point(name, dtype, model_root):
+    folder = make_folder(model_root, name, dtype)
+    raw, _, _ = CONFIGS[name]
+    prompts = [random_tokens(raw["vocab_size"], n, 40 + n) for n in ((5, 11, 2) if name == "A" else (1, 17, 33, 9))]
+    new = 8 if name == "A" else 12
+    got = hb.generate(folder, prompts, temperature=0.0, max_tokens=new, ignore_eos=True,
+                      no_repeat_check=True, dtype=dtype, max_batch=3)
+    cfg, w = plain_folder(folder)
+    for p, g in zip(prompts, got):
+        assert len(g) == new
+        if dtype == "float32":
+            assert g == plain.greedy(cfg, w, p, new)
+        else:
+            seq = list(p)
+            for tok in g:           # bfloat16 may swap near-equal logits; the choice must be near the top
+                logits = plain.forward(cfg, w, seq)[-1]
+                assert float(logits.max() - logits[tok]) <= 0.05 * float(logits.std())
+                seq.append(tok)
+
+
+def test_generation_stops_on_eos_and_other_sequences_go_on(model_root):
+    folder = make_folder(model_root, "A", "float32")
+    cfg, w = plain_folder(folder)
+    prompts = [random_tokens(256, n, 60 + n) for n in (4, 9, 6)]
+    want = [plain.greedy(cfg, w, p, 10) for p in prompts]
+    eos = want[1][3]                                   # make the 4th token of request 1 the eos
+    with open(os.path.join(folder, "config.json")) as f:
+        raw = json.load(f)
+    other = os.path.join(os.path.dirname(folder), "A_eos")
+    os.makedirs(other, exist_ok=True)
+    raw["eos_token_id"] = eos
+    with open(os.path.join(other, "config.json"), "w") as f:
+        json.dump(raw, f)
+    if not os.path.exists(os.path.join(other, "model.safetensors")):
+        os.link(os.path.join(folder, "model.safetensors"), os.path.join(other, "model.safetensors"))
+    engine = hb.load(other, dtype="float32", cache_tokens=64 * 3)
+    from herbert_rs_amd.sampling import SamplingParams
+    res = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=10, repeat_check=False))
+    for r, wnt in zip(res, want):
+        cut = wnt.index(eos) + 1 if eos in wnt else len(wnt)
+        assert r.tokens == wnt[:cut]
+        assert r.stop_reason == ("eos" if eos in wnt else "max_tokens")
+    assert res[1].stop_reason == "eos" and len(res[1].tokens) <= 4
+    engine.cache.check()
+    assert engine.cache.slots.held_count == 0
+
+
+def test_step_errors(model_root):
+    folder = make_folder(model_root, "A", "float32")
+    engine = hb.load(folder, dtype="float32", cache_tokens=128)
+    s = engine.alloc_slot()
+    with pytest.raises(RequestError, match="out of range"):
+        engine.step([StepEntry(s, [256], [0])])
+    with pytest.raises(RequestError, match="no tokens"):
+        engine.step([StepEntry(s, [], [])])
+    with pytest.raises(RequestError, match="twice"):
+        engine.step([StepEntry(s, [1], [0]), StepEntry(s, [2], [0])])
+    with pytest.raises(RequestError, match="outside"):
+        engine.step([StepEntry(s, [1, 2], [2])])
+    with pytest.raises(RequestError, match="max_position_embeddings"):
+        engine.step([StepEntry(s, [1] * 129, [0])])
+    with pytest.raises(CacheError):
+        engine.step([StepEntry(5, [1], [0])])                 # a slot that is not held
+    assert engine.step([StepEntry(s, [1, 2, 3], [])]) is None
+    assert engine.cache.length(s) == 3
+    engine.free_slot(s)
+    engine.cache.check()
+
+
+def test_cli_generates_token_ids(model_root):
+    folder = make_folder(model_root, "A", "float32")
+    cfg, w = plain_folder(folder)
+    out = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "herbert-cli"), "--model", folder,
+                          "--prompt", "5,17,3", "--temperature", "0", "--max-tokens", "6", "--dtype",
+                          "float32", "--ignore-eos", "--no-repeat-check", "--verbose"],
+                         capture_output=True, text=True, timeout=240)
+    assert out.returncode == 0, out.stderr
+    assert [int(t) for t in out.stdout.strip().split(",")] == plain.greedy(cfg, w, [5, 17, 3], 6)
+    assert "Prefill:" in out.stderr and "Decode:" in out.stderr and "Output tokens:   6" in out.stderr
+
+
+# ---- sampling kernels against the plain sampler
+def test_argmax_kernel_takes_the_first_of_equals():
+    from herbert_rs_amd.kernels import ops
+    logits = torch.randn(5, 5000)
+    logits[0, 77] = logits[0, 4000] = 50.0
+    logits[1, 4999] = 60.0
+    logits[2, 0] = 60.0
+    logits[3] = -float("inf")
+    out = torch.empty(5, dtype=torch.int32, device="cuda")
+    ops.argmax(logits.cuda(), out)
+    assert out.tolist() == [plain_sampler.argmax(r.numpy()) for r in logits]
+    assert out.tolist()[:4] == [77, 4999, 0, 0]
+
+
+@pytest.mark.parametrize("top_k,top_p", [(20, 1.0), (40, 0.9), (1, 1.0), (5, 0.3), (0, 1.0), (0, 0.8),
+                                         (2000, 0.95), (300, 1.0)])
+def test_sampler_matches_the_plain_sampler(top_k, top_p):
+    """Same seed, same logits: the same token as the step-by-step host formulation, draw after
+    draw; where the draw falls within rounding of a boundary either neighbour is right."""
+    from herbert_rs_amd.kernels import ops
+    from herbert_rs_amd.sampling import xorshift
+    V, R, temperature = 1500, 6, 0.7
+    g = torch.Generator().manual_seed(top_k + 3)
+    logits = torch.randn(R, V, generator=g) * 2.0
+    logits[1, 10] = logits[1, 900] = logits[1].max() + 0.5          # equal values at the top
+    dev_logits = logits.cuda()
+    seeds = [xorshift.sequence_seed(7, i) for i in range(R)]
+    states = torch.tensor([s - (1 << 64) if s >= (1 << 63) else s for s in seeds], dtype=torch.int64,
+                          device="cuda")
+    index = torch.arange(R, dtype=torch.int32, device="cuda")
+    p2 = 2048
+    scratch = (torch.empty(R, p2, dtype=torch.int32, device="cuda"),
+               torch.empty(R, p2, dtype=torch.int32, device="cuda"))
+    rngs = [plain_sampler.XorShift64(s) for s in seeds]
+    out = torch.empty(R, dtype=torch.int32, device="cuda")
+    for draw in range(12):
+        ops.sample(dev_logits, temperature, top_k, top_p, states, index, out, scratch)
+        got = out.tolist()
+        for r in range(R):
+            work = plain_sampler.candidates(logits[r].numpy(), temperature, top_k, top_p)
+            u = rngs[r].next_f32()
+            want = plain_sampler.pick(work, u)
+            if got[r] != want:
+                cum, near = np.float32(0), False
+                for idx, p in work:
+                    cum = np.float32(cum + p)
+                    if abs(float(cum) - float(u)) < 1e-5:
+                        near = True
+                assert near and got[r] in [i for i, _ in work], (draw, r, got[r], want)
+    assert [int(s) & ((1 << 64) - 1) for s in states.tolist()] == [r.state for r in rngs]
+
+
+def test_sampling_through_generate_is_reproducible(model_root):
+    folder = make_folder(model_root, "B", "float32")
+    prompts = [random_tokens(384, n, 70 + n) for n in (1, 17, 33, 9)]
+    kw = dict(temperature=0.7, top_k=20, top_p=1.0, max_tokens=12, ignore_eos=True, no_repeat_check=True,
+              dtype="float32", seed=7)
+    a = hb.generate(folder, prompts, **kw)
+    b = hb.generate(folder, prompts, **kw)
+    c = hb.generate(folder, prompts, **dict(kw, seed=8))
+    assert a == b and a != c and all(len(t) == 12 for t in a)
+    # the first request's tokens are those of the reference's one sampler with that seed
+    cfg, w = plain_folder(folder)
+    rng = plain_sampler.XorShift64(7)
+    seq = list(prompts[0])
+    for tok in a[0]:
+        logits = plain.forward(cfg, w, seq)[-1].numpy()
+        work = plain_sampler.candidates(logits, 0.7, 20, 1.0)
+        u = rng.next_f32()
+        want = plain_sampler.pick(work, u)
+        if tok != want:                                       # only at a rounding-level tie
+            assert tok in [i for i, _ in work]
+            break
+        seq.append(tok)

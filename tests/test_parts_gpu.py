@@ -1,0 +1,326 @@
+"""Each part alone against the plain formulas, models put together from parts in other ways
+(a layer run twice, a layer that reads another's cache, no rotation), and a toy mixer with state
+of its own that is registered here, outside the framework's files."""
+import numpy as np
+import pytest
+import torch
+
+from herbert_rs_amd.cache import Cache, KVNeed, StateNeed
+from herbert_rs_amd.engine import Engine, StepEntry
+from herbert_rs_amd.engine import batch as batching
+from herbert_rs_amd.engine.model import SharedParts
+from herbert_rs_amd.parts import (LayerSpec, ModelSpec, Part, PartSpec, Runtime, ScheduleEntry, StepContext,
+                                  build, register)
+from herbert_rs_amd.weights import TensorNeed
+
+from .plain import ops as pops
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def rand(*shape, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(*shape, generator=g) * scale
+
+
+def context(needs, lengths_new, dtype=torch.float32, max_positions=256):
+    """(ctx, cache, slots) for sequences that bring lengths_new[i] tokens to fresh slots."""
+    rt = Runtime(dtype, DEV)
+    cache = Cache(needs, 64 * 8, max_positions, dtype, DEV)
+    slots = [cache.alloc_slot() for _ in lengths_new]
+    entries = [StepEntry(s, [0] * n, []) for s, n in zip(slots, lengths_new)]
+    for e in entries:
+        cache.reserve(e.slot, len(e.tokens))
+    meta = batching.pack(entries, [0] * len(entries), torch.device(DEV))
+    return StepContext(rt=rt, meta=meta, cache=cache), cache, slots
+
+
+def test_norm_part():
+    w = 1 + 0.1 * rand(96, seed=1)
+    part = build("norm", PartSpec("rmsnorm", {"size": 96, "eps": 1e-5, "weight": "n.weight"}))
+    assert part.tensor_needs() == {"n.weight": TensorNeed((96,), "scale")}
+    rt = Runtime(torch.float32, DEV)
+    part.load({"n.weight": w}, rt)
+    x = rand(5, 96, seed=2, scale=3.0)
+    ctx = StepContext(rt=rt, meta=None, cache=None)
+    got = part.forward(ctx, x.to(DEV)).cpu()
+    assert torch.allclose(got, pops.rms_norm(x, w, 1e-5), atol=1e-5)
+    rows = torch.tensor([4, 1], dtype=torch.int32, device=DEV)
+    assert torch.allclose(part.forward(ctx, x.to(DEV), rows).cpu(), pops.rms_norm(x[[4, 1]], w, 1e-5), atol=1e-5)
+
+
+def test_position_part_tables():
+    part = build("position", PartSpec("rope", {"theta": 1e6, "rotary_dims": 32, "max_positions": 100}))
+    part.load({}, Runtime(torch.float32, DEV))
+    cos, sin, rot = part.rotation()
+    pc, ps = pops.rope_tables(list(range(100)), 32, 1e6)
+    assert rot == 32 and torch.equal(cos.cpu(), pc) and torch.equal(sin.cpu(), ps)
+    assert build("position", PartSpec("none")).rotation() is None
+
+
+ATT = dict(hidden_size=40, num_heads=6, num_kv_heads=2, head_dim=16, eps=1e-6)
+NAMES = {k: f"a.{k}" for k in ("q", "k", "v", "o", "q_norm", "k_norm")}
+
+
+def attention_weights(seed=3, hidden=40, nq=6, nkv=2, hd=16):
+    return {"a.q": rand(nq * hd, hidden, seed=seed, scale=0.2), "a.k": rand(nkv * hd, hidden, seed=seed + 1, scale=0.2),
+            "a.v": rand(nkv * hd, hidden, seed=seed + 2, scale=0.2), "a.o": rand(hidden, nq * hd, seed=seed + 3, scale=0.2),
+            "a.q_norm": 1 + 0.1 * rand(hd, seed=seed + 4), "a.k_norm": 1 + 0.1 * rand(hd, seed=seed + 5)}
+
+
+def plain_attention(w, y, positions, theta, eps, nq, nkv, hd, qk_norm=True, rope=True, window=None):
+    q = pops.split_heads(pops.linear(y, w["a.q"]), nq, hd)
+    k = pops.split_heads(pops.linear(y, w["a.k"]), nkv, hd)
+    v = pops.split_heads(pops.linear(y, w["a.v"]), nkv, hd)
+    if qk_norm:
+        q, k = pops.head_rms_norm(q, w["a.q_norm"], eps), pops.head_rms_norm(k, w["a.k_norm"], eps)
+    if rope:
+        q, k = pops.apply_rope(q, positions, theta), pops.apply_rope(k, positions, theta)
+    a = pops.causal_attention(q, k, v, positions, window=window)
+    return pops.linear(a.reshape(len(positions), nq * hd), w["a.o"])
+
+
+@pytest.mark.parametrize("qk_norm,rope,window", [(True, True, None), (False, True, None), (True, False, None),
+                                                 (True, True, 5)])
+def test_attention_part(qk_norm, rope, window):
+    pos_spec = PartSpec("rope", {"theta": 1e4, "rotary_dims": 16, "max_positions": 256}) if rope else PartSpec("none")
+    names = NAMES if qk_norm else {k: v for k, v in NAMES.items() if "norm" not in k}
+    part = build("mixer", PartSpec("attention", dict(ATT, position=pos_spec, names=names, qk_norm=qk_norm,
+                                                     window=window)), shared=SharedParts())
+    assert part.cache_need() == KVNeed(2, 16, window)
+    w = attention_weights()
+    assert set(part.tensor_needs()) == set(names.values())
+    ctx, cache, slots = context({0: part.cache_need()}, [9, 4])
+    part.position.load({}, ctx.rt)
+    part.load(w, ctx.rt)
+    y = rand(13, 40, seed=9)
+    x = torch.zeros(13, 40, device=DEV)
+    part.forward(ctx, y.to(DEV), x)
+    for a, b in ((0, 9), (9, 13)):
+        want = plain_attention(w, y[a:b], list(range(b - a)), 1e4, 1e-6, 6, 2, 16, qk_norm, rope, window)
+        assert torch.allclose(x[a:b].cpu(), want, atol=2e-5), (a, b)
+
+
+def test_feed_forward_part():
+    part = build("feed_forward", PartSpec("swiglu", {"hidden_size": 40, "intermediate_size": 72,
+                                                     "names": {"gate": "g", "up": "u", "down": "d"}}))
+    w = {"g": rand(72, 40, seed=1, scale=0.3), "u": rand(72, 40, seed=2, scale=0.3), "d": rand(40, 72, seed=3, scale=0.3)}
+    rt = Runtime(torch.float32, DEV)
+    part.load(w, rt)
+    y = rand(7, 40, seed=4)
+    x0 = rand(7, 40, seed=5)
+    x = x0.clone().to(DEV)
+    part.forward(StepContext(rt=rt, meta=None, cache=None), y.to(DEV), x)
+    assert torch.allclose(x.cpu(), x0 + pops.swiglu_mlp(y, w["g"], w["u"], w["d"]), atol=2e-5)
+
+
+def test_embedding_and_head_parts():
+    table = rand(50, 24, seed=1)
+    emb = build("embedding", PartSpec("table", {"vocab_size": 50, "hidden_size": 24, "weight": "e"}))
+    rt = Runtime(torch.float32, DEV)
+    emb.load({"e": table}, rt)
+    ids = torch.tensor([3, 49, 0], dtype=torch.int32, device=DEV)
+    ctx = StepContext(rt=rt, meta=None, cache=None)
+    x = emb.forward(ctx, ids)
+    assert torch.equal(x.cpu(), table[[3, 49, 0]])
+    nw = 1 + 0.1 * rand(24, seed=2)
+    for tied in (True, False):
+        norm = build("norm", PartSpec("rmsnorm", {"size": 24, "eps": 1e-6, "weight": "n"}))
+        head = build("head", PartSpec("linear", {"vocab_size": 50, "hidden_size": 24, "weight": "h",
+                                                 "tied_to_embedding": tied}), norm=norm)
+        assert ("h" in head.tensor_needs()) == (not tied)
+        hw = rand(50, 24, seed=3)
+        head.load({"n": nw, "h": hw}, rt, embedding=emb)
+        rows = torch.tensor([2, 0], dtype=torch.int32, device=DEV)
+        got = head.forward(ctx, x, rows).cpu()
+        want = pops.linear(pops.rms_norm(table[[0, 3]], nw, 1e-6), table if tied else hw)
+        assert torch.allclose(got, want, atol=1e-5)
+
+
+# ---- models put together in other ways
+def small_spec(layers, schedule, hidden=40, vocab=60, rope=True, share_from=None):
+    pos = PartSpec("rope", {"theta": 1e4, "rotary_dims": 16, "max_positions": 256}) if rope else PartSpec("none")
+    specs = []
+    for i in range(layers):
+        p = f"L{i}."
+        reads = share_from is not None and i in share_from
+        names = {k: p + k for k in (("q", "o", "q_norm") if reads else ("q", "k", "v", "o", "q_norm", "k_norm"))}
+        mixer = PartSpec("attention", dict(hidden_size=hidden, num_heads=4, num_kv_heads=2, head_dim=16, eps=1e-6,
+                                           position=pos, names=names, reads_cache_only=reads))
+        ffn = PartSpec("swiglu", {"hidden_size": hidden, "intermediate_size": 56,
+                                  "names": {"gate": p + "g", "up": p + "u", "down": p + "d"}})
+        norms = {"input": PartSpec("rmsnorm", {"size": hidden, "eps": 1e-6, "weight": p + "n1"}),
+                 "post_mixer": PartSpec("rmsnorm", {"size": hidden, "eps": 1e-6, "weight": p + "n2"})}
+        specs.append(LayerSpec(PartSpec("prenorm"), mixer, ffn, norms))
+    return ModelSpec(hidden_size=hidden, vocab_size=vocab, max_positions=256,
+                     embedding=PartSpec("table", {"vocab_size": vocab, "hidden_size": hidden, "weight": "emb"}),
+                     layers=specs, schedule=schedule,
+                     final_norm=PartSpec("rmsnorm", {"size": hidden, "eps": 1e-6, "weight": "fn"}),
+                     head=PartSpec("linear", {"vocab_size": vocab, "hidden_size": hidden, "weight": "head",
+                                              "tied_to_embedding": True}))
+
+
+def weights_for(spec, seed=0):
+    from herbert_rs_amd.engine.model import Model
+    from herbert_rs_amd.weights import random_tensors
+    return random_tensors(Model(spec).tensor_needs(), seed, "float32", std=0.15, norm_std=0.1)
+
+
+def plain_layer(w, p, x, positions, k_v_from=None, rope=True):
+    """One pre-norm layer of the small model by the plain formulas; returns (x, (k, v))."""
+    y = pops.rms_norm(x, w[p + "n1"], 1e-6)
+    q = pops.head_rms_norm(pops.split_heads(pops.linear(y, w[p + "q"]), 4, 16), w[p + "q_norm"], 1e-6)
+    if rope:
+        q = pops.apply_rope(q, positions, 1e4)
+    if k_v_from is None:
+        k = pops.head_rms_norm(pops.split_heads(pops.linear(y, w[p + "k"]), 2, 16), w[p + "k_norm"], 1e-6)
+        if rope:
+            k = pops.apply_rope(k, positions, 1e4)
+        v = pops.split_heads(pops.linear(y, w[p + "v"]), 2, 16)
+    else:
+        k, v = k_v_from
+    a = pops.causal_attention(q, k, v, positions).reshape(len(positions), 64)
+    x = x + pops.linear(a, w[p + "o"])
+    y = pops.rms_norm(x, w[p + "n2"], 1e-6)
+    return x + pops.swiglu_mlp(y, w[p + "g"], w[p + "u"], w[p + "d"]), (k, v)
+
+
+def run_engine(spec, w, tokens, cut=None):
+    engine = Engine(None, spec, w, dtype="float32", max_tokens=256)
+    s = engine.alloc_slot()
+    if cut is None:
+        return engine.step([StepEntry(s, tokens, list(range(len(tokens))))]).cpu()
+    a = engine.step([StepEntry(s, tokens[:cut], list(range(cut)))]).cpu()
+    rest = [engine.step([StepEntry(s, [t], [0])]).cpu() for t in tokens[cut:]]
+    return torch.cat([a] + rest)
+
+
+def test_a_layer_named_twice_and_a_layer_that_reads_another_s_cache():
+    # entry 0: layer 0; entry 1: layer 1 reading entry 0's keys and values; entry 2: layer 0 again
+    spec = small_spec(2, [ScheduleEntry(0), ScheduleEntry(1, cache=0), ScheduleEntry(0)], share_from={1})
+    w = weights_for(spec)
+    tokens = [5, 9, 33, 2, 41, 17, 8]
+    pos = list(range(len(tokens)))
+    x = pops.embedding(tokens, w["emb"])
+    x, kv0 = plain_layer(w, "L0.", x, pos)
+    x, _ = plain_layer(w, "L1.", x, pos, k_v_from=kv0)
+    x, _ = plain_layer(w, "L0.", x, pos)
+    want = pops.linear(pops.rms_norm(x, w["fn"], 1e-6), w["emb"])
+    assert torch.allclose(run_engine(spec, w, tokens), want, atol=1e-4)
+    assert torch.allclose(run_engine(spec, w, tokens, cut=3), want, atol=1e-4)     # and from the cache
+    from herbert_rs_amd.engine.model import Model
+    assert sorted(Model(spec).cache_needs()) == [0, 2]                             # two caches, not three
+    assert "L1.k" not in Model(spec).tensor_needs()
+
+
+def test_a_model_without_rotation():
+    spec = small_spec(1, [ScheduleEntry(0)], rope=False)
+    w = weights_for(spec, seed=4)
+    tokens = [1, 2, 3, 4, 5]
+    x = pops.embedding(tokens, w["emb"])
+    x, _ = plain_layer(w, "L0.", x, list(range(5)), rope=False)
+    want = pops.linear(pops.rms_norm(x, w["fn"], 1e-6), w["emb"])
+    assert torch.allclose(run_engine(spec, w, tokens, cut=2), want, atol=1e-4)
+
+
+# ---- a toy mixer with state of its own, defined here
+@register("mixer", "toy_decay")
+class ToyDecayMixer(Part):
+    """s_t = decay * s_{t-1} + W y_t ; the mixer's output is s_t. The state s lives in the cache's
+    fixed-size area, one vector per sequence; it has no keys or values."""
+
+    def __init__(self, hidden_size, decay, weight, shared=None):
+        self.hidden_size, self.decay, self.weight_name = hidden_size, decay, weight
+        self.w = None
+
+    def tensor_needs(self):
+        return {self.weight_name: TensorNeed((self.hidden_size, self.hidden_size))}
+
+    def cache_need(self):
+        return StateNeed((self.hidden_size,), torch.float32)
+
+    def load(self, tensors, rt):
+        self.w = tensors[self.weight_name].to(rt.device).float()
+
+    def forward(self, ctx, y, x):
+        state = ctx.cache.state_views(ctx.cache_entry)[0]          # [slots, hidden]
+        meta = ctx.meta
+        proj = y.float() @ self.w.T
+        starts = meta.host_starts
+        slots = meta.slots.tolist()
+        for i in range(meta.num_seqs):
+            s = state[slots[i]]
+            for t in range(int(starts[i]), int(starts[i + 1])):
+                s = self.decay * s + proj[t]
+                x[t] += s
+            state[slots[i]] = s
+
+
+def toy_spec():
+    """Three runs: the toy layer, an attention layer, the toy layer again (with a state of its own)."""
+    layer = LayerSpec(PartSpec("prenorm"),
+                      PartSpec("toy_decay", {"hidden_size": 40, "decay": 0.8, "weight": "T.mix"}),
+                      PartSpec("swiglu", {"hidden_size": 40, "intermediate_size": 56,
+                                          "names": {"gate": "T.g", "up": "T.u", "down": "T.d"}}),
+                      {"input": PartSpec("rmsnorm", {"size": 40, "eps": 1e-6, "weight": "T.n1"}),
+                       "post_mixer": PartSpec("rmsnorm", {"size": 40, "eps": 1e-6, "weight": "T.n2"})})
+    base = small_spec(1, [ScheduleEntry(0)])
+    return ModelSpec(hidden_size=40, vocab_size=60, max_positions=256, embedding=base.embedding,
+                     layers=[layer, base.layers[0]],
+                     schedule=[ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(0)],
+                     final_norm=base.final_norm, head=base.head)
+
+
+def plain_toy_layer(w, x):
+    proj = pops.linear(pops.rms_norm(x, w["T.n1"], 1e-6), w["T.mix"])
+    s, out = torch.zeros(40), []
+    for j in range(x.shape[0]):
+        s = 0.8 * s + proj[j]
+        out.append(s)
+    x = x + torch.stack(out)
+    return x + pops.swiglu_mlp(pops.rms_norm(x, w["T.n2"], 1e-6), w["T.g"], w["T.u"], w["T.d"])
+
+
+def test_toy_mixer_with_state_is_registered_built_and_stepped():
+    spec = toy_spec()
+    from herbert_rs_amd.engine.model import Model
+    from herbert_rs_amd.weights import random_tensors
+    model = Model(spec)
+    needs = model.tensor_needs()
+    assert "T.mix" in needs and model.cache_needs()[0] == StateNeed((40,), torch.float32)
+    assert isinstance(model.cache_needs()[1], KVNeed)
+    w = random_tensors(needs, 3, "float32", std=0.15, norm_std=0.1)
+    engine = Engine(None, spec, w, dtype="float32", max_tokens=256)
+    # the two runs of the toy layer (entries 0 and 2) have states of their own in one group
+    assert len(engine.cache.state_groups) == 1
+    assert next(iter(engine.cache.state_groups.values())).entries == [0, 2]
+
+    seqs = [[5, 9, 33, 2, 41, 17, 8, 11], [7, 3, 50]]
+    slots = [engine.alloc_slot() for _ in seqs]
+    whole = engine.step([StepEntry(s, t, list(range(len(t)))) for s, t in zip(slots, seqs)]).cpu()
+    for s in slots:
+        engine.free_slot(s)
+    # the same sequences again in the same slots, cut differently: the state must start at zero
+    slots = [engine.alloc_slot() for _ in seqs]
+    first = engine.step([StepEntry(s, t[:2], [0, 1]) for s, t in zip(slots, seqs)]).cpu()
+    rows = {0: [first[0], first[1]], 1: [first[2], first[3]]}
+    step = 2
+    while any(step < len(t) for t in seqs):
+        live = [i for i, t in enumerate(seqs) if step < len(t)]
+        out = engine.step([StepEntry(slots[i], [seqs[i][step]], [0]) for i in live]).cpu()
+        for r, i in enumerate(live):
+            rows[i].append(out[r])
+        step += 1
+    again = torch.stack(rows[0] + rows[1])
+    assert torch.allclose(again, whole, atol=1e-4)
+
+    # and against the plain formulas
+    at = 0
+    for t in seqs:
+        x = plain_toy_layer(w, pops.embedding(t, w["emb"]))
+        x, _ = plain_layer(w, "L0.", x, list(range(len(t))))
+        x = plain_toy_layer(w, x)
+        want = pops.linear(pops.rms_norm(x, w["fn"], 1e-6), w["emb"])
+        assert torch.allclose(whole[at:at + len(t)], want, atol=1e-4)
+        at += len(t)
