@@ -7,22 +7,35 @@ HB_MODULE_ERROR_SLOT()
 
 // ---------------------------------------------------------------- embedding
 // x[t, :] = float(table[ids[t], :]); the residual stream is float32.
-template <class TW>
+// PACKED: the table is stored in the MFMA kernels' order [V / 16][H / 32][64 lanes][8], element
+// (n, k) at ((n / 16 * (H / 32) + k / 32) * 64 + (k / 8 % 4) * 16 + n % 16) * 8 + k % 8.
+template <class TW, bool PACKED>
 __global__ void embed_kernel(const int* __restrict__ ids, const TW* __restrict__ table,
                              float* __restrict__ x, int H) {
     const int t = blockIdx.x;
-    const TW* row = table + (size_t)ids[t] * H;
+    const int n = ids[t];
     float* out = x + (size_t)t * H;
-    for (int i = threadIdx.x; i < H; i += blockDim.x) out[i] = hb_to_float(row[i]);
+    if (PACKED) {
+        const TW* blk = table + (size_t)(n / 16) * (H / 32) * 512 + (n % 16) * 8;
+        for (int k = threadIdx.x; k < H; k += blockDim.x)
+            out[k] = hb_to_float(blk[(size_t)(k / 32) * 512 + ((k / 8) % 4) * 128 + (k % 8)]);
+    } else {
+        const TW* row = table + (size_t)n * H;
+        for (int i = threadIdx.x; i < H; i += blockDim.x) out[i] = hb_to_float(row[i]);
+    }
 }
 
 extern "C" int hb_embed(const int* ids, const void* table, int table_dtype, float* x, int T, int H,
-                        hipStream_t stream) {
+                        int packed, hipStream_t stream) {
     HB_REQUIRE(T > 0 && H > 0, "embed: empty input (T=%d, H=%d)", T, H);
+    HB_REQUIRE(!packed || (table_dtype == HB_BF16 && H % 32 == 0), "embed: a packed table is bfloat16 with "
+               "a width in steps of 32");
     if (table_dtype == HB_F32)
-        embed_kernel<float><<<T, 256, 0, stream>>>(ids, (const float*)table, x, H);
+        embed_kernel<float, false><<<T, 256, 0, stream>>>(ids, (const float*)table, x, H);
+    else if (table_dtype == HB_BF16 && packed)
+        embed_kernel<bf16, true><<<T, 256, 0, stream>>>(ids, (const bf16*)table, x, H);
     else if (table_dtype == HB_BF16)
-        embed_kernel<bf16><<<T, 256, 0, stream>>>(ids, (const bf16*)table, x, H);
+        embed_kernel<bf16, false><<<T, 256, 0, stream>>>(ids, (const bf16*)table, x, H);
     else
         HB_REQUIRE(false, "embed: unknown table dtype %d", table_dtype);
     HB_CHECK_LAUNCH("embed");
@@ -49,16 +62,61 @@ __global__ void rmsnorm_kernel(const float* __restrict__ x, const float* __restr
     for (int i = threadIdx.x; i < H; i += blockDim.x) out[i] = hb_from_float<TOut>(in[i] * inv * w[i]);
 }
 
+// The same for rows that fit the registers of one block (H in steps of 4, at most 8192): every
+// element is loaded once, 16 bytes a lane, all loads in flight together.
+typedef float hb_f4 __attribute__((ext_vector_type(4)));
+template <class TOut>
+__global__ void __launch_bounds__(256)
+rmsnorm_row_kernel(const float* __restrict__ x, const float* __restrict__ w, TOut* __restrict__ y,
+                   const int* __restrict__ rows, int H, float eps) {
+    __shared__ float red[16];
+    const int r = blockIdx.x;
+    const hb_f4* in = (const hb_f4*)(x + (size_t)(rows ? rows[r] : r) * H);
+    const hb_f4* w4 = (const hb_f4*)w;
+    const int nv = H / 4;
+    hb_f4 v[8], g[8];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+        const int i = threadIdx.x + 256 * c;
+        if (i < nv) {
+            v[c] = in[i];
+            g[c] = w4[i];
+        } else {
+            v[c] = hb_f4{0.f, 0.f, 0.f, 0.f};
+        }
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) ss += v[c][0] * v[c][0] + v[c][1] * v[c][1] + v[c][2] * v[c][2] + v[c][3] * v[c][3];
+    ss = hb_block_sum(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)H + eps);
+    TOut* out = y + (size_t)r * H;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+        const int i = threadIdx.x + 256 * c;
+        if (i < nv) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) out[4 * i + e] = hb_from_float<TOut>(v[c][e] * inv * g[c][e]);
+        }
+    }
+}
+
 extern "C" int hb_rmsnorm(const float* x, const float* w, void* y, int y_dtype, const int* rows, int R,
                           int H, float eps, hipStream_t stream) {
     HB_REQUIRE(R > 0 && H > 0, "rmsnorm: empty input (R=%d, H=%d)", R, H);
-    const int threads = H >= 1024 ? 256 : 64;
-    if (y_dtype == HB_F32)
-        rmsnorm_kernel<float><<<R, threads, 0, stream>>>(x, w, (float*)y, rows, H, eps);
-    else if (y_dtype == HB_BF16)
-        rmsnorm_kernel<bf16><<<R, threads, 0, stream>>>(x, w, (bf16*)y, rows, H, eps);
-    else
-        HB_REQUIRE(false, "rmsnorm: unknown output dtype %d", y_dtype);
+    HB_REQUIRE(y_dtype == HB_F32 || y_dtype == HB_BF16, "rmsnorm: unknown output dtype %d", y_dtype);
+    if (H % 4 == 0 && H >= 1024 && H <= 8192) {
+        if (y_dtype == HB_F32)
+            rmsnorm_row_kernel<float><<<R, 256, 0, stream>>>(x, w, (float*)y, rows, H, eps);
+        else
+            rmsnorm_row_kernel<bf16><<<R, 256, 0, stream>>>(x, w, (bf16*)y, rows, H, eps);
+    } else {
+        const int threads = H >= 1024 ? 256 : 64;
+        if (y_dtype == HB_F32)
+            rmsnorm_kernel<float><<<R, threads, 0, stream>>>(x, w, (float*)y, rows, H, eps);
+        else
+            rmsnorm_kernel<bf16><<<R, threads, 0, stream>>>(x, w, (bf16*)y, rows, H, eps);
+    }
     HB_CHECK_LAUNCH("rmsnorm");
     return 0;
 }

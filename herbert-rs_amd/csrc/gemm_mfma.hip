@@ -34,7 +34,7 @@ struct SkinnyOperands {
     bf16x8 x[MB];
 };
 
-template <int MB, int NB, int WAVES, int EPI>
+template <int MB, int NB, int WAVES, int EPI, bool PACKED>
 __global__ void __launch_bounds__(WAVES * 64)
 gemm_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* __restrict__ Cv, int M,
                    int N, int K, int ldc) {
@@ -53,12 +53,21 @@ gemm_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void*
 #pragma unroll
         for (int b = 0; b < MB; ++b) acc[a][b] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+    // row-major weights: lane (r16, g4) reads 16 bytes of row n at k = 32 s + 8 g4.
+    // packed weights: the 1 KB operand of (block of 16 rows, k-step) is contiguous, lane-major.
     const bf16* wrow[NB];
+    constexpr int WSTEP = PACKED ? 64 * 8 : 32;      // elements between this lane's chunks of two k-steps
 #pragma unroll
     for (int a = 0; a < NB; ++a) {
-        int n = n0 + a * 16 + r16;
-        if (n >= N) n = N - 1;            // rows past the end repeat the last one; never stored
-        wrow[a] = W + (size_t)n * K + g4 * 8;
+        if (PACKED) {
+            int nb = n0 / 16 + a;
+            if (nb * 16 >= N) nb = (N - 1) / 16;
+            wrow[a] = W + ((size_t)nb * nsteps * 64 + lane) * 8;
+        } else {
+            int n = n0 + a * 16 + r16;
+            if (n >= N) n = N - 1;            // rows past the end repeat the last one; never stored
+            wrow[a] = W + (size_t)n * K + g4 * 8;
+        }
     }
     const bf16* xrow[MB];
 #pragma unroll
@@ -74,9 +83,10 @@ gemm_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void*
 
 #define SKINNY_LOAD(dst, group)                                                  \
     _Pragma("unroll") for (int u = 0; u < U; ++u) {                              \
-        const int k = (wave + ((group) * U + u) * WAVES) * 32;                   \
+        const int st = wave + ((group) * U + u) * WAVES;                         \
+        const int k = st * 32;                                                   \
         _Pragma("unroll") for (int a = 0; a < NB; ++a)                           \
-            dst[u].w[a] = *(const bf16x8*)(wrow[a] + k);                         \
+            dst[u].w[a] = *(const bf16x8*)(wrow[a] + (size_t)st * WSTEP);        \
         _Pragma("unroll") for (int b = 0; b < MB; ++b)                           \
             dst[u].x[b] = *(const bf16x8*)(xrow[b] + k);                         \
     }
@@ -96,10 +106,11 @@ gemm_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void*
         }
     }
     for (int i = groups * U; i < mine; ++i) {       // what is left over of this wave's steps
-        const int k = (wave + i * WAVES) * 32;
+        const int st = wave + i * WAVES;
+        const int k = st * 32;
         bf16x8 wv[NB], xv[MB];
 #pragma unroll
-        for (int a = 0; a < NB; ++a) wv[a] = *(const bf16x8*)(wrow[a] + k);
+        for (int a = 0; a < NB; ++a) wv[a] = *(const bf16x8*)(wrow[a] + (size_t)st * WSTEP);
 #pragma unroll
         for (int b = 0; b < MB; ++b) xv[b] = *(const bf16x8*)(xrow[b] + k);
 #pragma unroll
@@ -180,30 +191,35 @@ gemm_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void*
 
 template <int MB, int NB, int WAVES>
 static void launch_skinny(const void* X, const void* W, void* C, int M, int N, int K, int ldc, int epi,
-                          hipStream_t stream) {
+                          int packed, hipStream_t stream) {
     const int blocks = (N + NB * 16 - 1) / (NB * 16);
     const size_t lds = (size_t)(WAVES / 2) * NB * MB * 4 * 64 * sizeof(float);
     const bf16* x = (const bf16*)X;
     const bf16* w = (const bf16*)W;
-    if (epi == EPI_STORE)
-        gemm_skinny_kernel<MB, NB, WAVES, EPI_STORE><<<blocks, WAVES * 64, lds, stream>>>(x, w, C, M, N, K, ldc);
-    else if (epi == EPI_ADD)
-        gemm_skinny_kernel<MB, NB, WAVES, EPI_ADD><<<blocks, WAVES * 64, lds, stream>>>(x, w, C, M, N, K, ldc);
-    else
-        gemm_skinny_kernel<MB, NB, WAVES, EPI_SWIGLU><<<blocks, WAVES * 64, lds, stream>>>(x, w, C, M, N, K,
-                                                                                        ldc);
+#define SKINNY_GO(EPIV, PK) \
+    gemm_skinny_kernel<MB, NB, WAVES, EPIV, PK><<<blocks, WAVES * 64, lds, stream>>>(x, w, C, M, N, K, ldc)
+    if (packed) {
+        if (epi == EPI_STORE) SKINNY_GO(EPI_STORE, true);
+        else if (epi == EPI_ADD) SKINNY_GO(EPI_ADD, true);
+        else SKINNY_GO(EPI_SWIGLU, true);
+    } else {
+        if (epi == EPI_STORE) SKINNY_GO(EPI_STORE, false);
+        else if (epi == EPI_ADD) SKINNY_GO(EPI_ADD, false);
+        else SKINNY_GO(EPI_SWIGLU, false);
+    }
+#undef SKINNY_GO
 }
 
 template <int MB>
 static void pick_skinny(const void* X, const void* W, void* C, int M, int N, int K, int ldc, int epi,
-                        hipStream_t stream) {
+                        int packed, hipStream_t stream) {
     // Few weight rows: one block of 16 rows a workgroup and eight waves splitting K, so that the
     // 256 CUs all have work. Many rows: more rows a workgroup, so that the activations are
     // re-read from L2 less often.
     if (epi == EPI_SWIGLU || N >= 16384) {
-        launch_skinny<MB, 4, 4>(X, W, C, M, N, K, ldc, epi, stream);
+        launch_skinny<MB, 4, 4>(X, W, C, M, N, K, ldc, epi, packed, stream);
     } else {
-        launch_skinny<MB, 1, 8>(X, W, C, M, N, K, ldc, epi, stream);
+        launch_skinny<MB, 1, 8>(X, W, C, M, N, K, ldc, epi, packed, stream);
     }
 }
 
@@ -213,7 +229,7 @@ static void pick_skinny(const void* X, const void* W, void* C, int M, int N, int
 #define BK 64
 #define LDT (BK + 8)   // padded row of a tile in LDS, in elements: 144 bytes, conflict-free b128 reads
 
-template <int EPI>
+template <int EPI, bool PACKED>
 __global__ void __launch_bounds__(256)
 gemm_tiled_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* __restrict__ Cv, int M, int N,
                   int K, int ldc, int m_tiles, int n_tiles) {
@@ -235,19 +251,35 @@ gemm_tiled_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* 
     const int wn = wave >> 1, wm = wave & 1;       // wave's 64 x 64 part of the tile
     const int c32 = lane & 31, g2 = lane >> 5;
 
-    // global -> registers: 4 chunks of 16 bytes of each operand per thread
+    // global -> registers: 4 chunks of 16 bytes of each operand per thread.
+    // Row-major: thread (lrow, lchunk) takes k-chunk lchunk of rows lrow + 32 i.
+    // Packed weights: chunk c = tid + 256 i is lane c % 64 of operand c / 64 (8 row blocks x 2 k-steps
+    // of the tile), 1 KB contiguous per 64 threads.
     const int lrow = tid >> 3, lchunk = tid & 7;
     const bf16* wsrc[4];
     const bf16* xsrc[4];
+    int wdst[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        int n = n0 + lrow + 32 * i;
-        if (n >= N) n = N - 1;
-        wsrc[i] = W + (size_t)n * K + lchunk * 8;
+        if (PACKED) {
+            const int c = tid + 256 * i;
+            const int pl = c & 63, op = c >> 6;
+            const int nb_local = op >> 1, ks_local = op & 1;
+            int nb = n0 / 16 + nb_local;
+            if (nb * 16 >= N) nb = (N - 1) / 16;
+            wsrc[i] = W + (((size_t)nb * (K / 32) + ks_local) * 64 + pl) * 8;
+            wdst[i] = (nb_local * 16 + (pl & 15)) * LDT + ks_local * 32 + (pl >> 4) * 8;
+        } else {
+            int n = n0 + lrow + 32 * i;
+            if (n >= N) n = N - 1;
+            wsrc[i] = W + (size_t)n * K + lchunk * 8;
+            wdst[i] = (lrow + 32 * i) * LDT + lchunk * 8;
+        }
         int m = m0 + lrow + 32 * i;
         if (m >= M) m = M - 1;
         xsrc[i] = X + (size_t)m * K + lchunk * 8;
     }
+    constexpr int WTILE_STEP = PACKED ? 2 * 64 * 8 : BK;     // elements from one k-tile to the next
     bf16x8 wreg[4], xreg[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -268,7 +300,7 @@ gemm_tiled_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* 
         const int buf = kt & 1;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            *(bf16x8*)(&Ws[buf][(lrow + 32 * i) * LDT + lchunk * 8]) = wreg[i];
+            *(bf16x8*)(&Ws[buf][wdst[i]]) = wreg[i];
             *(bf16x8*)(&Xs[buf][(lrow + 32 * i) * LDT + lchunk * 8]) = xreg[i];
         }
         __syncthreads();
@@ -276,7 +308,7 @@ gemm_tiled_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* 
             const int koff = (kt + 1) * BK;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                wreg[i] = *(const bf16x8*)(wsrc[i] + koff);
+                wreg[i] = *(const bf16x8*)(wsrc[i] + (size_t)(kt + 1) * WTILE_STEP);
                 xreg[i] = *(const bf16x8*)(xsrc[i] + koff);
             }
         }
@@ -350,18 +382,20 @@ gemm_tiled_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* 
 
 // C (+)= X @ W^T. X [M, K] bf16, W [N, K] bf16. epi 0: C f32 [M, N] stored; 1: added to;
 // 2: W's rows are gate/up interleaved in blocks of 16 and C is bf16 [M, N / 2] = silu(gate) * up.
+// packed != 0: W is stored as [N / 16][K / 32][64 lanes][8]: lane = 16 * (k / 8 % 4) + n % 16.
 extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N, int K, int ldc, int epi,
-                            hipStream_t stream) {
+                            int packed, hipStream_t stream) {
+    HB_REQUIRE(!packed || N % 16 == 0, "gemm_mfma: packed weights need N %% 16 == 0");
     HB_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_mfma: empty problem (M=%d, N=%d, K=%d)", M, N, K);
     HB_REQUIRE(epi >= 0 && epi <= 2, "gemm_mfma: unknown epilogue %d", epi);
     HB_REQUIRE(K % 32 == 0, "gemm_mfma: K=%d is no multiple of 32", K);
     HB_REQUIRE(epi != EPI_SWIGLU || N % 32 == 0, "gemm_mfma: the SwiGLU epilogue needs N %% 32 == 0");
     HB_REQUIRE(ldc >= (epi == EPI_SWIGLU ? N / 2 : N), "gemm_mfma: output row stride %d too small", ldc);
     if (M <= 64) {
-        if (M <= 16) pick_skinny<1>(X, W, C, M, N, K, ldc, epi, stream);
-        else if (M <= 32) pick_skinny<2>(X, W, C, M, N, K, ldc, epi, stream);
-        else if (M <= 48) pick_skinny<3>(X, W, C, M, N, K, ldc, epi, stream);
-        else pick_skinny<4>(X, W, C, M, N, K, ldc, epi, stream);
+        if (M <= 16) pick_skinny<1>(X, W, C, M, N, K, ldc, epi, packed, stream);
+        else if (M <= 32) pick_skinny<2>(X, W, C, M, N, K, ldc, epi, packed, stream);
+        else if (M <= 48) pick_skinny<3>(X, W, C, M, N, K, ldc, epi, packed, stream);
+        else pick_skinny<4>(X, W, C, M, N, K, ldc, epi, packed, stream);
         HB_CHECK_LAUNCH("gemm_skinny");
         return 0;
     }
@@ -372,12 +406,18 @@ extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N,
     const int blocks = (int)((total + 7) / 8 * 8);
     const bf16* x = (const bf16*)X;
     const bf16* w = (const bf16*)W;
-    if (epi == EPI_STORE)
-        gemm_tiled_kernel<EPI_STORE><<<blocks, 256, 0, stream>>>(x, w, C, M, N, K, ldc, m_tiles, n_tiles);
-    else if (epi == EPI_ADD)
-        gemm_tiled_kernel<EPI_ADD><<<blocks, 256, 0, stream>>>(x, w, C, M, N, K, ldc, m_tiles, n_tiles);
-    else
-        gemm_tiled_kernel<EPI_SWIGLU><<<blocks, 256, 0, stream>>>(x, w, C, M, N, K, ldc, m_tiles, n_tiles);
+#define TILED_GO(EPIV, PK) \
+    gemm_tiled_kernel<EPIV, PK><<<blocks, 256, 0, stream>>>(x, w, C, M, N, K, ldc, m_tiles, n_tiles)
+    if (packed) {
+        if (epi == EPI_STORE) TILED_GO(EPI_STORE, true);
+        else if (epi == EPI_ADD) TILED_GO(EPI_ADD, true);
+        else TILED_GO(EPI_SWIGLU, true);
+    } else {
+        if (epi == EPI_STORE) TILED_GO(EPI_STORE, false);
+        else if (epi == EPI_ADD) TILED_GO(EPI_ADD, false);
+        else TILED_GO(EPI_SWIGLU, false);
+    }
+#undef TILED_GO
     HB_CHECK_LAUNCH("gemm_tiled");
     return 0;
 }

@@ -119,13 +119,3 @@ class Engine:
         results = gen.generate(prompts, params, on_token)
         self.last_generation_stats = gen.stats
         return results
-
-    def get_tensor(self, name):
-        """A weight as the engine holds it (by the name of the weight files)."""
-        for part in self.model._weight_parts():
-            got = getattr(part, "get_tensor", None)
-            if got is not None:
-                t = got(name)
-                if t is not None:
-                    return t
-        raise KeyError(name)

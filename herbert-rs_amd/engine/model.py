@@ -67,7 +67,7 @@ class Model:
         return parts
 
     def load(self, tensors, rt):
-        self.embedding.load(tensors, rt)
+        self.embedding.load(tensors, rt, shared_with_head=getattr(self.head, "tied", False))
         for p in self.shared.all():
             p.load(tensors, rt)
         for b in self.blocks:

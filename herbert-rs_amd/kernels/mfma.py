@@ -12,7 +12,7 @@ _P = ctypes.c_void_p
 _I = ctypes.c_int
 _F = ctypes.c_float
 lib.register_signatures("gemm_mfma", {
-    "hb_gemm_mfma": [_P, _P, _P, _I, _I, _I, _I, _I, _P],
+    "hb_gemm_mfma": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
 })
 
 EPI_STORE, EPI_ADD, EPI_SWIGLU = 0, 1, 2
@@ -33,8 +33,17 @@ def gemm_supported(a, w, out=None, swiglu=False):
     return out is None or out.dtype == torch.float32
 
 
-def gemm(a, w, out, accumulate=False):
-    """out f32 [M, N] (+)= a bf16 [M, K] @ w bf16 [N, K]^T."""
+def pack_weight(w):
+    """[N, K] -> the same values as [N / 16, K / 32, 64, 8]: the 1 KB MFMA operand of 16 rows and
+    32 k is contiguous, lane-major (lane = 16 * (k / 8 % 4) + n % 16)."""
+    N, K = w.shape
+    if N % 16 or K % 32:
+        raise BackendError("packed weights need N in steps of 16 and K in steps of 32")
+    return w.view(N // 16, 16, K // 32, 4, 8).permute(0, 2, 3, 1, 4).contiguous().view(N, K)
+
+
+def gemm(a, w, out, accumulate=False, packed=False):
+    """out f32 [M, N] (+)= a bf16 [M, K] @ w bf16 [N, K]^T (w as stored, or as pack_weight gives it)."""
     _check(a, "a", torch.bfloat16, (None, None))
     M, K = a.shape
     _check(w, "w", torch.bfloat16, (None, K))
@@ -43,7 +52,7 @@ def gemm(a, w, out, accumulate=False):
     if not gemm_supported(a, w, out):
         raise BackendError(f"gemm_mfma refuses M={M}, N={N}, K={K}")
     lib.call("gemm_mfma", "hb_gemm_mfma", a.data_ptr(), w.data_ptr(), out.data_ptr(), M, N, K, N,
-             EPI_ADD if accumulate else EPI_STORE, _stream())
+             EPI_ADD if accumulate else EPI_STORE, 1 if packed else 0, _stream())
 
 
 def interleave_gate_up(gate, up):
@@ -55,7 +64,7 @@ def interleave_gate_up(gate, up):
     return torch.stack([gate.view(I // 16, 16, K), up.view(I // 16, 16, K)], 1).reshape(2 * I, K).contiguous()
 
 
-def gemm_swiglu(a, w_interleaved, out):
+def gemm_swiglu(a, w_interleaved, out, packed=False):
     """out bf16 [M, I] = silu(a @ gate^T) * (a @ up^T), the weights interleaved as above."""
     _check(a, "a", torch.bfloat16, (None, None))
     M, K = a.shape
@@ -65,7 +74,7 @@ def gemm_swiglu(a, w_interleaved, out):
     if not gemm_supported(a, w_interleaved, swiglu=True):
         raise BackendError(f"gemm_mfma (SwiGLU) refuses M={M}, N={N}, K={K}")
     lib.call("gemm_mfma", "hb_gemm_mfma", a.data_ptr(), w_interleaved.data_ptr(), out.data_ptr(), M, N, K,
-             N // 2, EPI_SWIGLU, _stream())
+             N // 2, EPI_SWIGLU, 1 if packed else 0, _stream())
 
 
 lib.register_signatures("attention_mfma", {

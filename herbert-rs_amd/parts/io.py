@@ -25,12 +25,15 @@ class TokenEmbedding(Part):
     def tensor_needs(self):
         return {self.weight_name: TensorNeed((self.vocab_size, self.hidden_size), "table")}
 
-    def load(self, tensors, rt):
-        self.table = rt.weight(tensors[self.weight_name])
+    def load(self, tensors, rt, shared_with_head=False):
+        """shared_with_head: the table is also the head's matrix; it is then kept in the order the
+        head's kernels want, and rows are gathered from that order."""
+        self.linear = Linear(rt.weight(tensors[self.weight_name]), pack=shared_with_head)
+        self.table = self.linear.weight
 
     def forward(self, ctx, token_ids):
         x = ctx.rt.buffer("residual", (token_ids.shape[0], self.hidden_size), torch.float32)
-        ops.embed(token_ids, self.table, x)
+        ops.embed(token_ids, self.table, x, packed=self.linear.packed)
         return x
 
 
@@ -54,7 +57,7 @@ class OutputHead(Part):
     def load(self, tensors, rt, embedding=None):
         self.norm.load(tensors, rt)
         if self.tied:
-            self.proj = Linear(embedding.table)
+            self.proj = embedding.linear
         else:
             self.proj = Linear(rt.weight(tensors[self.weight_name]))
 

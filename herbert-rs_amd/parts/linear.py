@@ -1,8 +1,9 @@
 """A weight matrix [out, in] and its product with activations.
 
-In the float32 mode the plain kernel does all products. In the bfloat16 mode
-the MFMA kernels do them where they take the shape and the plain kernel (same
-storage types, float32 arithmetic) does the rest.
+In the float32 mode the plain kernel does all products. In the bfloat16 mode the MFMA kernels
+do them where they take the shape, and then the matrix is kept in their packed order (the 1 KB
+operand of 16 rows and 32 k contiguous), which streams from HBM in whole contiguous blocks;
+the plain kernel (same storage types, float32 arithmetic) does the rest from row-major weights.
 """
 import torch
 
@@ -10,15 +11,27 @@ from ..kernels import ops
 
 
 class Linear:
-    def __init__(self, weight):
-        self.weight = weight           # [N, K], compute dtype, on the GPU
+    def __init__(self, weight, pack=True):
+        """weight: [N, K] in the compute dtype on the GPU."""
         self.out_features, self.in_features = weight.shape
+        self.packed = False
+        if pack and weight.dtype == torch.bfloat16 and weight.is_cuda \
+                and self.out_features % 16 == 0 and self.in_features % 64 == 0:
+            from ..kernels import mfma
+            weight = mfma.pack_weight(weight)
+            self.packed = True
+        self.weight = weight
 
     def forward(self, a, out, accumulate=False):
         """out[M, N] (+)= a[M, K] @ W^T."""
         if self.weight.dtype == torch.bfloat16 and a.dtype == torch.bfloat16:
             from ..kernels import mfma
-            if mfma.gemm_supported(a, self.weight, out):
-                mfma.gemm(a, self.weight, out, accumulate)
+            if self.packed or mfma.gemm_supported(a, self.weight, out):
+                mfma.gemm(a, self.weight, out, accumulate, packed=self.packed)
                 return
         ops.gemm_plain(a, self.weight, out, accumulate)
+
+    def forward_swiglu(self, a, out):
+        """out bf16 [M, N / 2] = silu(gate) * up for a weight whose rows are gate/up interleaved."""
+        from ..kernels import mfma
+        mfma.gemm_swiglu(a, self.weight, out, packed=self.packed)

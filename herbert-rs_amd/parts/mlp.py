@@ -49,8 +49,7 @@ class SwiGLU(Part):
         T = y.shape[0]
         act = rt.buffer("act", (T, self.intermediate_size))
         if self.fused_epilogue:
-            from ..kernels import mfma
-            mfma.gemm_swiglu(y, self.gate_up.weight, act)
+            self.gate_up.forward_swiglu(y, act)
         else:
             gu = rt.buffer("gate_up", (T, 2 * self.intermediate_size), torch.float32)
             self.gate_up.forward(y, gu)

@@ -258,3 +258,16 @@ def test_attention_finds_one_far_key_among_hundreds():
                 fn(q, meta, kv, out, nq, nkv, hd, 1.0, 0)
                 got = out.float().cpu().view(new, nq, hd)
                 assert float((got - V[target, 0]).abs().max()) < 0.02, (n, target, mode, fn.__name__)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 48, 32), (8, 4096, 4096), (17, 1008, 224), (64, 24576, 512),
+                                   (65, 128, 64), (200, 336, 192), (2048, 512, 4096)])
+def test_gemm_mfma_packed_weights(M, N, K):
+    from herbert_rs_amd.kernels import mfma
+    a = rand(M, K, seed=7, dtype=torch.bfloat16)
+    w = rand(N, K, seed=8, dtype=torch.bfloat16)
+    plain = torch.empty(M, N, device=dev())
+    mfma.gemm(a, w, plain)
+    packed = torch.empty(M, N, device=dev())
+    mfma.gemm(a, mfma.pack_weight(w), packed, packed=True)
+    assert torch.equal(plain, packed)
