@@ -15,7 +15,8 @@
 //          kv head (one wave each); K and V^T pages are staged in LDS once for all of them.
 // decode:  one wave = one sequence x one kv head x one range of pages, all query heads of the
 //          group as columns; operands stream from global memory (each byte is used once);
-//          partial (max, sum, O) per range are merged by a second kernel.
+//          partial (max, sum, O) per range are merged by a second kernel in the fixed order
+//          of the ranges.
 #include "common.h"
 #include <math.h>
 
@@ -260,41 +261,74 @@ attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache,
                     oacc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[d][kb][h2], pb[kb][h2], oacc[d], 0, 0, 0);
         }
     }
-    if (c32 >= G) return;
     l += __shfl_xor(l, 32, 64);
-    const size_t base = ((size_t)b * nq + kvh * G + c32) * splits + split;
-    if (g2 == 0) {
-        partial_ml[base * 2] = m;        // -inf when this range held no visible key
-        partial_ml[base * 2 + 1] = l;
-    }
-    float* po = partial_o + base * HD;
-#pragma unroll
-    for (int d = 0; d < HD / 32; ++d)
-#pragma unroll
-        for (int qd = 0; qd < 4; ++qd) {
-            f32x4 v = {oacc[d][4 * qd], oacc[d][4 * qd + 1], oacc[d][4 * qd + 2], oacc[d][4 * qd + 3]};
-            *(f32x4*)(po + d * 32 + 8 * qd + 4 * g2) = v;
+    if (c32 < G) {
+        const size_t base = ((size_t)b * nq + kvh * G + c32) * splits + split;
+        if (g2 == 0) {
+            partial_ml[base * 2] = m;        // -inf when this range held no visible key
+            partial_ml[base * 2 + 1] = l;
         }
+        float* po = partial_o + base * HD;
+#pragma unroll
+        for (int d = 0; d < HD / 32; ++d)
+#pragma unroll
+            for (int qd = 0; qd < 4; ++qd) {
+                f32x4 v = {oacc[d][4 * qd], oacc[d][4 * qd + 1], oacc[d][4 * qd + 2], oacc[d][4 * qd + 3]};
+                *(f32x4*)(po + d * 32 + 8 * qd + 4 * g2) = v;
+            }
+    }
 }
 
-// Merge the ranges of one (sequence, head): out = sum_s 2^((m_s - M) c) O_s / sum_s 2^((m_s - M) c) l_s.
-__global__ void attn_decode_merge_kernel(const float* __restrict__ partial_o,
-                                         const float* __restrict__ partial_ml, bf16* __restrict__ out,
-                                         int splits, int HD, float c) {
+// Merge the ranges of one (sequence, head), in the order of the ranges:
+//   out = sum_s 2^((m_s - M) c) O_s / sum_s 2^((m_s - M) c) l_s.
+// One wave per (sequence, head). A kernel of its own: the partial results of waves on other
+// XCDs are visible at a kernel boundary without any fence that would write back an L2.
+template <int HD>
+__global__ void __launch_bounds__(64)
+attn_decode_merge_kernel(const float* __restrict__ partial_o, const float* __restrict__ partial_ml,
+                         bf16* __restrict__ out, int splits, float c) {
+    const int lane = threadIdx.x;
     const size_t bh = blockIdx.x;
-    const float* ml = partial_ml + bh * splits * 2;
-    float M = -INFINITY;
-    for (int s = 0; s < splits; ++s) M = fmaxf(M, ml[2 * s]);
-    float denom = 0.f;
-    for (int s = 0; s < splits; ++s)
-        if (ml[2 * s] != -INFINITY) denom += fast_exp2((ml[2 * s] - M) * c) * ml[2 * s + 1];
-    const float inv = denom > 0.f ? 1.0f / denom : 0.f;
-    for (int d = threadIdx.x; d < HD; d += blockDim.x) {
-        float acc = 0.f;
-        for (int s = 0; s < splits; ++s)
-            if (ml[2 * s] != -INFINITY)
-                acc += fast_exp2((ml[2 * s] - M) * c) * partial_o[(bh * splits + s) * HD + d];
-        out[bh * HD + d] = hb_from_float<bf16>(acc * inv);
+    {   // lanes over the ranges for the weights, then lanes over d for the sums
+        const float* ml = partial_ml + bh * splits * 2;
+        float M = -INFINITY;
+        for (int s = lane; s < splits; s += 64) M = fmaxf(M, ml[2 * s]);
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) M = fmaxf(M, __shfl_xor(M, off, 64));
+        float denom = 0.f;
+        for (int s0 = 0; s0 < splits; s0 += 64) {       // ranges in order, 64 at a time
+            const int s = s0 + lane;
+            float term = 0.f;
+            if (s < splits && ml[2 * s] != -INFINITY) term = fast_exp2((ml[2 * s] - M) * c) * ml[2 * s + 1];
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) term += __shfl_xor(term, off, 64);
+            denom += term;
+        }
+        const float inv = denom > 0.f ? 1.0f / denom : 0.f;
+        float acc[HD / 64 > 0 ? HD / 64 : 1];
+#pragma unroll
+        for (int j = 0; j < (HD + 63) / 64; ++j) acc[j] = 0.f;
+        for (int s0 = 0; s0 < splits; s0 += 64) {
+            const int sl = s0 + lane;
+            float wl = 0.f;
+            if (sl < splits && ml[2 * sl] != -INFINITY) wl = fast_exp2((ml[2 * sl] - M) * c);
+            const int n = splits - s0 < 64 ? splits - s0 : 64;
+#pragma unroll 8
+            for (int j = 0; j < n; ++j) {
+                const float wgt = __shfl(wl, j, 64);
+                const float* po = partial_o + (bh * splits + s0 + j) * HD;
+#pragma unroll
+                for (int e = 0; e < (HD + 63) / 64; ++e) {
+                    const int d = lane + 64 * e;
+                    if (d < HD) acc[e] = fmaf(wgt, po[d], acc[e]);
+                }
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < (HD + 63) / 64; ++e) {
+            const int d = lane + 64 * e;
+            if (d < HD) out[bh * HD + d] = hb_from_float<bf16>(acc[e] * inv);
+        }
     }
 }
 
@@ -339,19 +373,18 @@ extern "C" int hb_attn_decode_mfma(const void* q, const void* k_cache, const voi
     HB_REQUIRE(window >= 0, "attn_decode: bad window");
     dim3 grid(B, nkv, splits);
     const float c = scale * LOG2E;
-#define LAUNCH_DECODE(HDV)                                                                               \
+#define LAUNCH_DECODE(HDV) do {                                                                          \
     attn_decode_kernel<HDV><<<grid, 64, 0, stream>>>((const bf16*)q, (const bf16*)k_cache,               \
                                                     (const bf16*)v_cache, partial_o, partial_ml,         \
                                                     context_lens, slots, page_table, max_pages, nq, nkv, c, \
-                                                    window, pages_per_split)
+                                                    window, pages_per_split);                          \
+    attn_decode_merge_kernel<HDV><<<B * nq, 64, 0, stream>>>(partial_o, partial_ml, (bf16*)out, splits, c); \
+    } while (0)
     if (hd == 32) LAUNCH_DECODE(32);
     else if (hd == 64) LAUNCH_DECODE(64);
     else if (hd == 128) LAUNCH_DECODE(128);
     else HB_REQUIRE(false, "attn_decode: head_dim %d is not one of 32, 64, 128", hd);
 #undef LAUNCH_DECODE
     HB_CHECK_LAUNCH("attn_decode");
-    attn_decode_merge_kernel<<<B * nq, hd < 64 ? 64 : hd, 0, stream>>>(partial_o, partial_ml, (bf16*)out,
-                                                                    splits, hd, c);
-    HB_CHECK_LAUNCH("attn_decode_merge");
     return 0;
 }

@@ -28,17 +28,39 @@ __device__ __forceinline__ float silu_mul(float g, float u) { return g / (1.0f +
 // Workgroup: WAVES waves, NB blocks of 16 weight rows, MB blocks of 16 activation rows.
 // Wave w takes the k-steps (32 wide) s = w, w + WAVES, ...; it loads U steps ahead of the
 // ones it multiplies, so that enough bytes are in flight to keep HBM busy.
-template <int MB, int NB>
+// x * g of 8 consecutive k as an MFMA operand; the squares of x are added to ss.
+__device__ __forceinline__ bf16x8 normed_operand(const f32x4 xf[2], const f32x4 g[2], float& ss) {
+    bf16x8 r;
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float v = xf[h][e];
+            ss = fmaf(v, v, ss);
+            r[h * 4 + e] = (__bf16)(v * g[h][e]);
+        }
+    return r;
+}
+
+// NORM: the activations are the float32 residual stream and the product is RMSNorm(x) W^T:
+//   y = (x * inv * g) W^T = inv * ((x * g) W^T),  inv = 1 / sqrt(mean(x^2) + eps) per row,
+// so x * g goes through the matrix cores (rounded to bfloat16) and inv scales the sums at the
+// end; the sum of squares comes from the values the lanes load anyway.
+template <int MB, int NB, bool NORM>
 struct SkinnyOperands {
     bf16x8 w[NB];
-    bf16x8 x[MB];
+    bf16x8 x[NORM ? 1 : MB];
+    f32x4 xf[NORM ? MB : 1][2];
+    f32x4 g[2];
 };
 
-template <int MB, int NB, int WAVES, int EPI, bool PACKED>
+template <int MB, int NB, int WAVES, int EPI, bool PACKED, bool NORM>
 __global__ void __launch_bounds__(WAVES * 64)
-gemm_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* __restrict__ Cv, int M,
-                   int N, int K, int ldc) {
-    constexpr int U = (NB + MB <= 4) ? 4 : 2;
+gemm_skinny_kernel(const void* __restrict__ Xv, const bf16* __restrict__ W, void* __restrict__ Cv, int M,
+                   int N, int K, int ldc, const float* __restrict__ norm_w, float eps) {
+    constexpr int U = NORM ? 2 : ((NB + MB <= 4) ? 4 : 2);
+    const bf16* X = (const bf16*)Xv;
+    const float* XF = (const float*)Xv;
     extern __shared__ float red[];   // [WAVES / 2][NB * MB * 4][64]
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -70,16 +92,21 @@ gemm_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void*
         }
     }
     const bf16* xrow[MB];
+    const float* xfrow[MB];
 #pragma unroll
     for (int b = 0; b < MB; ++b) {
         int m = b * 16 + r16;
         if (m >= M) m = M - 1;
         xrow[b] = X + (size_t)m * K + g4 * 8;
+        xfrow[b] = XF + (size_t)m * K + g4 * 8;
     }
+    float sumsq[MB];
+#pragma unroll
+    for (int b = 0; b < MB; ++b) sumsq[b] = 0.f;
 
     const int mine = wave < nsteps ? (nsteps - wave + WAVES - 1) / WAVES : 0;   // this wave's steps
     const int groups = mine / U;
-    SkinnyOperands<MB, NB> cur[U], nxt[U];
+    SkinnyOperands<MB, NB, NORM> cur[U], nxt[U];
 
 #define SKINNY_LOAD(dst, group)                                                  \
     _Pragma("unroll") for (int u = 0; u < U; ++u) {                              \
@@ -87,14 +114,30 @@ gemm_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void*
         const int k = st * 32;                                                   \
         _Pragma("unroll") for (int a = 0; a < NB; ++a)                           \
             dst[u].w[a] = *(const bf16x8*)(wrow[a] + (size_t)st * WSTEP);        \
-        _Pragma("unroll") for (int b = 0; b < MB; ++b)                           \
-            dst[u].x[b] = *(const bf16x8*)(xrow[b] + k);                         \
+        if (NORM) {                                                              \
+            dst[u].g[0] = *(const f32x4*)(norm_w + k + g4 * 8);                  \
+            dst[u].g[1] = *(const f32x4*)(norm_w + k + g4 * 8 + 4);              \
+            _Pragma("unroll") for (int b = 0; b < MB; ++b) {                     \
+                dst[u].xf[b][0] = *(const f32x4*)(xfrow[b] + k);                 \
+                dst[u].xf[b][1] = *(const f32x4*)(xfrow[b] + k + 4);             \
+            }                                                                    \
+        } else {                                                                 \
+            _Pragma("unroll") for (int b = 0; b < MB; ++b)                       \
+                dst[u].x[b] = *(const bf16x8*)(xrow[b] + k);                     \
+        }                                                                        \
     }
 #define SKINNY_MULTIPLY(src)                                                     \
     _Pragma("unroll") for (int u = 0; u < U; ++u)                                \
-        _Pragma("unroll") for (int a = 0; a < NB; ++a)                           \
-            _Pragma("unroll") for (int b = 0; b < MB; ++b)                       \
-                acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(src[u].w[a], src[u].x[b], acc[a][b], 0, 0, 0);
+        _Pragma("unroll") for (int b = 0; b < MB; ++b) {                         \
+            bf16x8 xop;                                                          \
+            if (NORM) {                                                          \
+                xop = normed_operand(src[u].xf[b], src[u].g, sumsq[b]);          \
+            } else {                                                             \
+                xop = src[u].x[b];                                               \
+            }                                                                    \
+            _Pragma("unroll") for (int a = 0; a < NB; ++a)                       \
+                acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(src[u].w[a], xop, acc[a][b], 0, 0, 0); \
+        }
 
     if (groups > 0) { SKINNY_LOAD(cur, 0) }
     for (int g = 0; g < groups; g += 2) {
@@ -112,7 +155,15 @@ gemm_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void*
 #pragma unroll
         for (int a = 0; a < NB; ++a) wv[a] = *(const bf16x8*)(wrow[a] + (size_t)st * WSTEP);
 #pragma unroll
-        for (int b = 0; b < MB; ++b) xv[b] = *(const bf16x8*)(xrow[b] + k);
+        for (int b = 0; b < MB; ++b) {
+            if (NORM) {
+                f32x4 xf[2] = {*(const f32x4*)(xfrow[b] + k), *(const f32x4*)(xfrow[b] + k + 4)};
+                f32x4 gg[2] = {*(const f32x4*)(norm_w + k + g4 * 8), *(const f32x4*)(norm_w + k + g4 * 8 + 4)};
+                xv[b] = normed_operand(xf, gg, sumsq[b]);
+            } else {
+                xv[b] = *(const bf16x8*)(xrow[b] + k);
+            }
+        }
 #pragma unroll
         for (int a = 0; a < NB; ++a)
 #pragma unroll
@@ -124,6 +175,24 @@ gemm_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void*
 
     // a fixed tree over the waves: the upper half adds into the lower half, until wave 0 holds all
     constexpr int REGS = NB * MB * 4;
+    float inv_rms[MB];
+    if (NORM) {
+        // a row's squares: over the four lane groups of this wave, then over the waves in order
+#pragma unroll
+        for (int b = 0; b < MB; ++b) {
+            sumsq[b] += __shfl_xor(sumsq[b], 16, 64);
+            sumsq[b] += __shfl_xor(sumsq[b], 32, 64);
+            if (lane < 16) red[(wave * MB + b) * 16 + lane] = sumsq[b];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int b = 0; b < MB; ++b) {
+            float total = 0.f;
+            for (int w = 0; w < WAVES; ++w) total += red[(w * MB + b) * 16 + r16];
+            inv_rms[b] = 1.0f / sqrtf(total / (float)K + eps);
+        }
+        __syncthreads();
+    }
 #pragma unroll
     for (int half = WAVES / 2; half >= 1; half >>= 1) {
         if (wave >= half && wave < 2 * half) {
@@ -148,6 +217,14 @@ gemm_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void*
         __syncthreads();
     }
     if (wave != 0) return;
+    if (NORM) {
+#pragma unroll
+        for (int a = 0; a < NB; ++a)
+#pragma unroll
+            for (int b = 0; b < MB; ++b)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[a][b][i] *= inv_rms[b];
+    }
 
     // lane: m = b * 16 + r16, n = n0 + a * 16 + g4 * 4 + i
     if (EPI == EPI_SWIGLU) {
@@ -191,35 +268,44 @@ gemm_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void*
 
 template <int MB, int NB, int WAVES>
 static void launch_skinny(const void* X, const void* W, void* C, int M, int N, int K, int ldc, int epi,
-                          int packed, hipStream_t stream) {
+                          int packed, const float* norm_w, float eps, hipStream_t stream) {
     const int blocks = (N + NB * 16 - 1) / (NB * 16);
-    const size_t lds = (size_t)(WAVES / 2) * NB * MB * 4 * 64 * sizeof(float);
-    const bf16* x = (const bf16*)X;
+    size_t lds = (size_t)(WAVES / 2) * NB * MB * 4 * 64 * sizeof(float);
+    if (lds < (size_t)WAVES * MB * 16 * sizeof(float)) lds = (size_t)WAVES * MB * 16 * sizeof(float);
     const bf16* w = (const bf16*)W;
-#define SKINNY_GO(EPIV, PK) \
-    gemm_skinny_kernel<MB, NB, WAVES, EPIV, PK><<<blocks, WAVES * 64, lds, stream>>>(x, w, C, M, N, K, ldc)
-    if (packed) {
-        if (epi == EPI_STORE) SKINNY_GO(EPI_STORE, true);
-        else if (epi == EPI_ADD) SKINNY_GO(EPI_ADD, true);
-        else SKINNY_GO(EPI_SWIGLU, true);
+#define SKINNY_GO(EPIV, PK, NM)                                                                        \
+    gemm_skinny_kernel<MB, NB, WAVES, EPIV, PK, NM><<<blocks, WAVES * 64, lds, stream>>>(X, w, C, M, N, K, \
+                                                                                          ldc, norm_w, eps)
+    if (norm_w) {       // the normed input never meets the add epilogue
+        if (packed) {
+            if (epi == EPI_STORE) SKINNY_GO(EPI_STORE, true, true);
+            else SKINNY_GO(EPI_SWIGLU, true, true);
+        } else {
+            if (epi == EPI_STORE) SKINNY_GO(EPI_STORE, false, true);
+            else SKINNY_GO(EPI_SWIGLU, false, true);
+        }
+    } else if (packed) {
+        if (epi == EPI_STORE) SKINNY_GO(EPI_STORE, true, false);
+        else if (epi == EPI_ADD) SKINNY_GO(EPI_ADD, true, false);
+        else SKINNY_GO(EPI_SWIGLU, true, false);
     } else {
-        if (epi == EPI_STORE) SKINNY_GO(EPI_STORE, false);
-        else if (epi == EPI_ADD) SKINNY_GO(EPI_ADD, false);
-        else SKINNY_GO(EPI_SWIGLU, false);
+        if (epi == EPI_STORE) SKINNY_GO(EPI_STORE, false, false);
+        else if (epi == EPI_ADD) SKINNY_GO(EPI_ADD, false, false);
+        else SKINNY_GO(EPI_SWIGLU, false, false);
     }
 #undef SKINNY_GO
 }
 
 template <int MB>
 static void pick_skinny(const void* X, const void* W, void* C, int M, int N, int K, int ldc, int epi,
-                        int packed, hipStream_t stream) {
+                        int packed, const float* norm_w, float eps, hipStream_t stream) {
     // Few weight rows: one block of 16 rows a workgroup and eight waves splitting K, so that the
     // 256 CUs all have work. Many rows: more rows a workgroup, so that the activations are
     // re-read from L2 less often.
     if (epi == EPI_SWIGLU || N >= 16384) {
-        launch_skinny<MB, 4, 4>(X, W, C, M, N, K, ldc, epi, packed, stream);
+        launch_skinny<MB, 4, 4>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream);
     } else {
-        launch_skinny<MB, 1, 8>(X, W, C, M, N, K, ldc, epi, packed, stream);
+        launch_skinny<MB, 1, 8>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream);
     }
 }
 
@@ -383,8 +469,11 @@ gemm_tiled_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* 
 // C (+)= X @ W^T. X [M, K] bf16, W [N, K] bf16. epi 0: C f32 [M, N] stored; 1: added to;
 // 2: W's rows are gate/up interleaved in blocks of 16 and C is bf16 [M, N / 2] = silu(gate) * up.
 // packed != 0: W is stored as [N / 16][K / 32][64 lanes][8]: lane = 16 * (k / 8 % 4) + n % 16.
+// norm_w != null: X is the float32 residual stream [M, K] and the product is RMSNorm(X; norm_w, eps) W^T
+// (M <= 64 only, never with the add epilogue).
 extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N, int K, int ldc, int epi,
-                            int packed, hipStream_t stream) {
+                            int packed, const float* norm_w, float eps, hipStream_t stream) {
+    HB_REQUIRE(!norm_w || (M <= 64 && epi != EPI_ADD), "gemm_mfma: the fused norm takes M <= 64 and no add");
     HB_REQUIRE(!packed || N % 16 == 0, "gemm_mfma: packed weights need N %% 16 == 0");
     HB_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_mfma: empty problem (M=%d, N=%d, K=%d)", M, N, K);
     HB_REQUIRE(epi >= 0 && epi <= 2, "gemm_mfma: unknown epilogue %d", epi);
@@ -392,10 +481,10 @@ extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N,
     HB_REQUIRE(epi != EPI_SWIGLU || N % 32 == 0, "gemm_mfma: the SwiGLU epilogue needs N %% 32 == 0");
     HB_REQUIRE(ldc >= (epi == EPI_SWIGLU ? N / 2 : N), "gemm_mfma: output row stride %d too small", ldc);
     if (M <= 64) {
-        if (M <= 16) pick_skinny<1>(X, W, C, M, N, K, ldc, epi, packed, stream);
-        else if (M <= 32) pick_skinny<2>(X, W, C, M, N, K, ldc, epi, packed, stream);
-        else if (M <= 48) pick_skinny<3>(X, W, C, M, N, K, ldc, epi, packed, stream);
-        else pick_skinny<4>(X, W, C, M, N, K, ldc, epi, packed, stream);
+        if (M <= 16) pick_skinny<1>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream);
+        else if (M <= 32) pick_skinny<2>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream);
+        else if (M <= 48) pick_skinny<3>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream);
+        else pick_skinny<4>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream);
         HB_CHECK_LAUNCH("gemm_skinny");
         return 0;
     }

@@ -33,6 +33,14 @@ class BatchMeta:
     host_starts: np.ndarray    # host copies, for kernels' grids
     host_context: np.ndarray
     derived: dict = None       # what kernels' host sides derive once a step (tile lists and the like)
+    context_bucket: int = 0    # max_context rounded up to CONTEXT_BUCKET: sizes the decode kernels' grids
+
+
+CONTEXT_BUCKET = 256
+
+
+def bucket(context):
+    return (int(context) + CONTEXT_BUCKET - 1) // CONTEXT_BUCKET * CONTEXT_BUCKET
 
 
 def pack(entries, start_lengths, device, staging=None):
@@ -74,4 +82,48 @@ def pack(entries, start_lengths, device, staging=None):
         slots=dev[o:o + B], seq_starts=dev[o + B:o + 2 * B + 1],
         context_lens=dev[o + 2 * B + 1:o + 3 * B + 1], want_rows=dev[o + 3 * B + 1:o + 3 * B + 1 + R],
         num_tokens=T, num_seqs=B, max_new=max(counts), max_context=int(ctx.max()),
-        max_position=int(pos.max()), host_starts=starts.copy(), host_context=ctx.copy(), derived={})
+        max_position=int(pos.max()), host_starts=starts.copy(), host_context=ctx.copy(), derived={},
+        context_bucket=bucket(int(ctx.max())))
+
+
+class StaticDecodeMeta:
+    """The metadata of a step of B sequences with one token each, every logit wanted, in buffers
+    that stay where they are: a captured graph reads them, `update` refills them."""
+
+    def __init__(self, batch_size, device):
+        B = self.batch_size = batch_size
+        self.host = torch.empty(7 * B + 1, dtype=torch.int32, pin_memory=True)
+        self.copied = None       # event after the last copy out of `host`
+        self.dev = torch.zeros(7 * B + 1, dtype=torch.int32, device=device)
+        h = self.host.numpy()
+        h[2 * B:3 * B] = np.arange(B)            # seq_of
+        h[4 * B:5 * B + 1] = np.arange(B + 1)    # seq_starts
+        h[6 * B + 1:7 * B + 1] = np.arange(B)    # want_rows
+        d = self.dev
+        self.meta = BatchMeta(
+            token_ids=d[0:B], positions=d[B:2 * B], seq_of=d[2 * B:3 * B], slots=d[3 * B:4 * B],
+            seq_starts=d[4 * B:5 * B + 1], context_lens=d[5 * B + 1:6 * B + 1],
+            want_rows=d[6 * B + 1:7 * B + 1], num_tokens=B, num_seqs=B, max_new=1, max_context=0,
+            max_position=0, host_starts=np.arange(B + 1, dtype=np.int32),
+            host_context=np.zeros(B, dtype=np.int32), derived={}, context_bucket=0)
+
+    def update(self, entries, start_lengths):
+        B = self.batch_size
+        if self.copied is not None:
+            self.copied.synchronize()        # the pinned buffer is free to be written again
+        h = self.host.numpy()
+        for i, e in enumerate(entries):
+            h[i] = e.tokens[0]
+            h[B + i] = start_lengths[i]
+            h[3 * B + i] = e.slot
+            h[5 * B + 1 + i] = start_lengths[i] + 1
+        self.dev.copy_(self.host, non_blocking=True)
+        if self.dev.is_cuda:
+            self.copied = torch.cuda.Event()
+            self.copied.record()
+        m = self.meta
+        m.host_context = h[5 * B + 1:6 * B + 1].copy()
+        m.max_context = int(m.host_context.max())
+        m.max_position = m.max_context - 1
+        m.context_bucket = bucket(m.max_context)
+        return m

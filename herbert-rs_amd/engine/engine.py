@@ -17,11 +17,19 @@ from ..errors import BackendError, RequestError
 from ..parts import Runtime
 from ..weights import read_tensors
 from . import batch as batching
-from .batch import StepEntry
+from .batch import StaticDecodeMeta, StepEntry
 from .model import Model
 
 _DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16,
            torch.float32: torch.float32, torch.bfloat16: torch.bfloat16}
+
+
+class _DecodeState:
+    def __init__(self, static):
+        self.static = static
+        self.seen = {}
+        self.graphs = {}
+        self.logits = {}
 
 
 def require_gpu():
@@ -32,7 +40,7 @@ def require_gpu():
 
 class Engine:
     def __init__(self, config, spec, tensors, dtype="bfloat16", max_tokens=4096, max_slots=None,
-                 device=None):
+                 device=None, use_graphs=True):
         """tensors: {name: tensor} for the model's needs (any device)."""
         if dtype not in _DTYPES:
             raise BackendError(f"dtype must be float32 or bfloat16, got {dtype!r}")
@@ -45,20 +53,23 @@ class Engine:
         self.cache = Cache(self.model.cache_needs(), max_tokens, spec.max_positions, self.rt.dtype,
                            self.device, max_slots)
         self.steps_run = 0
+        self.use_graphs = bool(use_graphs) and self.model.graph_safe
+        self._decode = {}       # batch size -> _DecodeState
 
     # ---- construction
     @classmethod
-    def from_folder(cls, folder, dtype="bfloat16", max_tokens=4096, max_slots=None, device=None):
+    def from_folder(cls, folder, dtype="bfloat16", max_tokens=4096, max_slots=None, device=None,
+                    use_graphs=True):
         """The engine of the model in `folder` (config.json + safetensors)."""
         arch, config = load_config(folder)
         spec = arch.build_spec(config)
         needs = Model(spec).tensor_needs()
         tensors = read_tensors(folder, needs)
-        return cls(config, spec, tensors, dtype, max_tokens, max_slots, device)
+        return cls(config, spec, tensors, dtype, max_tokens, max_slots, device, use_graphs)
 
     @classmethod
     def from_config(cls, config, architecture=None, seed=0, dtype="bfloat16", weight_dtype=None,
-                    std=0.02, norm_std=0.0, max_tokens=4096, max_slots=None, device=None):
+                    std=0.02, norm_std=0.0, max_tokens=4096, max_slots=None, device=None, use_graphs=True):
         """An engine with seeded random weights drawn on the GPU (no files)."""
         from ..config.registry import resolve_architecture
         from ..weights import random_tensors
@@ -67,7 +78,7 @@ class Engine:
         dev = torch.device(device) if device is not None else require_gpu()
         needs = Model(spec).tensor_needs()
         tensors = random_tensors(needs, seed, weight_dtype or dtype, std, norm_std, device=str(dev))
-        return cls(config, spec, tensors, dtype, max_tokens, max_slots, dev)
+        return cls(config, spec, tensors, dtype, max_tokens, max_slots, dev, use_graphs)
 
     # ---- slots
     def alloc_slot(self):
@@ -105,11 +116,43 @@ class Engine:
             starts.append(start)
         for e in entries:
             self.cache.reserve(e.slot, len(e.tokens))
-        meta = batching.pack(entries, starts, self.device)
-        logits = self.model.forward(self.rt, meta, self.cache)
+        if self.use_graphs and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
+            logits = self._decode_step(entries, starts)
+        else:
+            meta = batching.pack(entries, starts, self.device)
+            logits = self.model.forward(self.rt, meta, self.cache)
         for e in entries:
             self.cache.commit(e.slot, len(e.tokens))
         self.steps_run += 1
+        return logits
+
+    def _decode_step(self, entries, starts):
+        """One token for each sequence, every logit wanted: the launch-bound case. The step's
+        metadata lives in fixed buffers; from the second step of a shape on, the forward pass is a
+        captured HIP graph that is replayed, so that the host launches one graph and not hundreds
+        of kernels. A graph is tied to the batch size and to the bucket of the longest context
+        (which sizes the attention grid); the logits it returns are overwritten by its next replay."""
+        B = len(entries)
+        state = self._decode.get(B)
+        if state is None:
+            state = self._decode[B] = _DecodeState(StaticDecodeMeta(B, self.device))
+        meta = state.static.update(entries, starts)
+        key = meta.context_bucket
+        graph = state.graphs.get(key)
+        if graph is not None:
+            graph.replay()
+            return state.logits[key]
+        seen = state.seen.get(key, 0)
+        state.seen[key] = seen + 1
+        if seen == 0:
+            return self.model.forward(self.rt, meta, self.cache)      # also sizes every scratch buffer
+        torch.cuda.synchronize(self.device)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            logits = self.model.forward(self.rt, meta, self.cache)
+        state.graphs[key] = graph
+        state.logits[key] = logits
+        graph.replay()
         return logits
 
     def generate(self, prompts, params=None, max_batch=64, on_token=None):

@@ -76,6 +76,12 @@ class Model:
         self.head.load(tensors, rt, embedding=self.embedding)
         self.loaded = True
 
+    @property
+    def graph_safe(self):
+        """True if every part only enqueues GPU work, so that a step can be captured and replayed."""
+        parts = self._weight_parts() + self.blocks + self.shared.all()
+        return all(getattr(p, "graph_safe", False) for p in parts)
+
     # ---- cache
     def cache_needs(self):
         """{schedule entry: need} for the entries that own a cache."""

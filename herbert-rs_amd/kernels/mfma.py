@@ -12,7 +12,7 @@ _P = ctypes.c_void_p
 _I = ctypes.c_int
 _F = ctypes.c_float
 lib.register_signatures("gemm_mfma", {
-    "hb_gemm_mfma": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
+    "hb_gemm_mfma": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _F, _P],
 })
 
 EPI_STORE, EPI_ADD, EPI_SWIGLU = 0, 1, 2
@@ -42,17 +42,37 @@ def pack_weight(w):
     return w.view(N // 16, 16, K // 32, 4, 8).permute(0, 2, 3, 1, 4).contiguous().view(N, K)
 
 
-def gemm(a, w, out, accumulate=False, packed=False):
-    """out f32 [M, N] (+)= a bf16 [M, K] @ w bf16 [N, K]^T (w as stored, or as pack_weight gives it)."""
-    _check(a, "a", torch.bfloat16, (None, None))
+def _norm_args(a, norm, K):
+    """(pointer, eps) of a fused RMSNorm, after checks; (None, 0) without one."""
+    if norm is None:
+        _check(a, "a", torch.bfloat16, (None, None))
+        return None, 0.0
+    weight, eps = norm
+    _check(a, "a", torch.float32, (None, None))
+    _check(weight, "norm weight", torch.float32, (K,))
+    if a.shape[0] > SKINNY_MAX_M:
+        raise BackendError(f"the fused norm takes at most {SKINNY_MAX_M} rows")
+    return weight.data_ptr(), float(eps)
+
+
+def norm_fusable(a, w):
+    """True if RMSNorm(a) @ w^T can run as one kernel: few rows of the float32 residual stream."""
+    return (a.dtype == torch.float32 and w.dtype == torch.bfloat16 and a.shape[0] <= SKINNY_MAX_M
+            and a.shape[1] % 32 == 0)
+
+
+def gemm(a, w, out, accumulate=False, packed=False, norm=None):
+    """out f32 [M, N] (+)= a bf16 [M, K] @ w bf16 [N, K]^T (w as stored, or as pack_weight gives it).
+    norm = (weight f32 [K], eps): a is the float32 residual stream and is RMS-normed on the way."""
     M, K = a.shape
+    norm_ptr, eps = _norm_args(a, norm, K)
     _check(w, "w", torch.bfloat16, (None, K))
     N = w.shape[0]
     _check(out, "out", torch.float32, (M, N))
-    if not gemm_supported(a, w, out):
+    if K % 32 or (M > SKINNY_MAX_M and K % 64) or (norm is not None and accumulate):
         raise BackendError(f"gemm_mfma refuses M={M}, N={N}, K={K}")
     lib.call("gemm_mfma", "hb_gemm_mfma", a.data_ptr(), w.data_ptr(), out.data_ptr(), M, N, K, N,
-             EPI_ADD if accumulate else EPI_STORE, 1 if packed else 0, _stream())
+             EPI_ADD if accumulate else EPI_STORE, 1 if packed else 0, norm_ptr, eps, _stream())
 
 
 def interleave_gate_up(gate, up):
@@ -64,17 +84,17 @@ def interleave_gate_up(gate, up):
     return torch.stack([gate.view(I // 16, 16, K), up.view(I // 16, 16, K)], 1).reshape(2 * I, K).contiguous()
 
 
-def gemm_swiglu(a, w_interleaved, out, packed=False):
+def gemm_swiglu(a, w_interleaved, out, packed=False, norm=None):
     """out bf16 [M, I] = silu(a @ gate^T) * (a @ up^T), the weights interleaved as above."""
-    _check(a, "a", torch.bfloat16, (None, None))
     M, K = a.shape
+    norm_ptr, eps = _norm_args(a, norm, K)
     _check(w_interleaved, "w", torch.bfloat16, (None, K))
     N = w_interleaved.shape[0]
     _check(out, "out", torch.bfloat16, (M, N // 2))
-    if not gemm_supported(a, w_interleaved, swiglu=True):
+    if K % 32 or (M > SKINNY_MAX_M and K % 64) or N % 32:
         raise BackendError(f"gemm_mfma (SwiGLU) refuses M={M}, N={N}, K={K}")
     lib.call("gemm_mfma", "hb_gemm_mfma", a.data_ptr(), w_interleaved.data_ptr(), out.data_ptr(), M, N, K,
-             N // 2, EPI_SWIGLU, 1 if packed else 0, _stream())
+             N // 2, EPI_SWIGLU, 1 if packed else 0, norm_ptr, eps, _stream())
 
 
 lib.register_signatures("attention_mfma", {
@@ -114,16 +134,17 @@ def _prefill_tiles(meta):
 
 def _decode_split(meta, nkv, window):
     """(ranges, pages per range): enough waves for the 256 CUs, every range at least one page."""
-    span = (meta.max_context + 63) // 64
+    span = (meta.context_bucket + 63) // 64     # by bucket, so that a captured graph's grid stays right
     if window:
         span = min(span, (window + 63) // 64 + 1)
     want = max(1, -(-1024 // (meta.num_seqs * nkv)))
-    splits = max(1, min(span, want))
+    splits = max(1, min(span, want, 32))      # the merge's cost grows with the ranges
     per = -(-span // splits)
     return -(-span // per), per
 
 
 def _partial_buffers(device, n_rows, splits, hd):
+    """(partial outputs, partial max / sum) of the decode kernel's ranges."""
     key = str(device)
     need_o = n_rows * splits * hd
     buf = _partials.get(key)

@@ -26,6 +26,8 @@ from .registry import register
 
 @register("mixer", "attention")
 class Attention(Part):
+    graph_safe = True
+
     def __init__(self, hidden_size, num_heads, num_kv_heads, head_dim, eps, position, names,
                  qk_norm=True, window=None, scale=None, shared=None, reads_cache_only=False):
         """names: dict with q, k, v, o (and q_norm, k_norm when qk_norm) -> tensor names.
@@ -85,14 +87,24 @@ class Attention(Part):
             if not self.reads_cache_only:
                 self.k_norm_w = rt.weight(tensors[n["k_norm"]], matrix=False)
 
-    def forward(self, ctx, y, x):
+    def forward_from_residual(self, ctx, x, norm):
+        """With few rows and bfloat16 weights the input norm runs inside the projection kernel."""
+        if not (hasattr(norm, "w") and hasattr(norm, "eps") and self.qkv.fuses_norm(x)):
+            return False
+        self.forward(ctx, None, x, fused_norm=norm)
+        return True
+
+    def forward(self, ctx, y, x, fused_norm=None):
         rt = ctx.rt
-        T = y.shape[0]
+        T = x.shape[0]
         kv = ctx.cache.kv_view(ctx.cache_entry)
         write_kv = not self.reads_cache_only
         width = self.q_dim + (2 * self.kv_dim if write_kv else 0)
         qkv = rt.buffer("qkv", (T, width), torch.float32)
-        self.qkv.forward(y, qkv)
+        if fused_norm is not None:
+            self.qkv.forward_normed(x, fused_norm.w, fused_norm.eps, qkv)
+        else:
+            self.qkv.forward(y, qkv)
         q = rt.buffer("q", (T, self.q_dim))
         rot = self.position.rotation()
         cos, sin, rot_dims = rot if rot is not None else (None, None, 0)

@@ -16,6 +16,7 @@ Every part also has
   load(tensors, rt)                             take them (converted as its kernels need)
 and a mixer has
   cache_need() -> None, KVNeed, StateNeed or a tuple of them.
+A part whose forward() only enqueues GPU work sets `graph_safe = True`.
 """
 from dataclasses import dataclass
 from typing import Any
@@ -25,6 +26,9 @@ import torch
 
 class Part:
     kind = "?"
+    # True if forward() only enqueues GPU work (no host synchronisation, no host-side copies):
+    # a step made of such parts may be captured into a HIP graph and replayed.
+    graph_safe = False
 
     def tensor_needs(self):
         return {}

@@ -11,6 +11,8 @@ from .registry import register
 
 @register("block", "prenorm")
 class PreNormBlock(Part):
+    graph_safe = True
+
     norm_roles = ("input", "post_mixer")
 
     def __init__(self, mixer, feed_forward, norms):
@@ -25,7 +27,14 @@ class PreNormBlock(Part):
         return [self.norms["input"], self.mixer, self.norms["post_mixer"], self.feed_forward]
 
     def forward(self, ctx, x):
-        y = self.norms["input"].forward(ctx, x)
-        self.mixer.forward(ctx, y, x)
-        y = self.norms["post_mixer"].forward(ctx, x)
-        self.feed_forward.forward(ctx, y, x)
+        self._run(ctx, x, self.norms["input"], self.mixer)
+        self._run(ctx, x, self.norms["post_mixer"], self.feed_forward)
+
+    @staticmethod
+    def _run(ctx, x, norm, part):
+        """part(norm(x)) added to x. A part may offer forward_from_residual(ctx, x, norm), which
+        returns True if it has done the norm itself inside its first kernel."""
+        fused = getattr(part, "forward_from_residual", None)
+        if fused is not None and fused(ctx, x, norm):
+            return
+        part.forward(ctx, norm.forward(ctx, x), x)

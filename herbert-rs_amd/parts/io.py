@@ -16,6 +16,8 @@ from .registry import register
 
 @register("embedding", "table")
 class TokenEmbedding(Part):
+    graph_safe = True
+
     def __init__(self, vocab_size, hidden_size, weight, shared=None):
         self.vocab_size = int(vocab_size)
         self.hidden_size = int(hidden_size)
@@ -39,6 +41,8 @@ class TokenEmbedding(Part):
 
 @register("head", "linear")
 class OutputHead(Part):
+    graph_safe = True
+
     def __init__(self, vocab_size, hidden_size, weight, tied_to_embedding, norm, shared=None):
         """weight: the head's tensor name; tied_to_embedding: use the embedding table instead."""
         self.vocab_size = int(vocab_size)

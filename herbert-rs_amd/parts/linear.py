@@ -31,7 +31,19 @@ class Linear:
                 return
         ops.gemm_plain(a, self.weight, out, accumulate)
 
-    def forward_swiglu(self, a, out):
+    def forward_swiglu(self, a, out, norm=None):
         """out bf16 [M, N / 2] = silu(gate) * up for a weight whose rows are gate/up interleaved."""
         from ..kernels import mfma
-        mfma.gemm_swiglu(a, self.weight, out, packed=self.packed)
+        mfma.gemm_swiglu(a, self.weight, out, packed=self.packed, norm=norm)
+
+    def fuses_norm(self, x):
+        """True if RMSNorm(x) @ W^T runs as one kernel for this input (few rows, bfloat16 weights)."""
+        if self.weight.dtype != torch.bfloat16:
+            return False
+        from ..kernels import mfma
+        return mfma.norm_fusable(x, self.weight)
+
+    def forward_normed(self, x, norm_weight, eps, out):
+        """out[M, N] = RMSNorm(x; norm_weight, eps) @ W^T in one kernel (see fuses_norm)."""
+        from ..kernels import mfma
+        mfma.gemm(x, self.weight, out, packed=self.packed, norm=(norm_weight, eps))

@@ -15,6 +15,8 @@ from .registry import register
 
 @register("feed_forward", "swiglu")
 class SwiGLU(Part):
+    graph_safe = True
+
     def __init__(self, hidden_size, intermediate_size, names, shared=None):
         """names: dict with gate, up, down -> tensor names."""
         self.hidden_size = int(hidden_size)
@@ -44,11 +46,21 @@ class SwiGLU(Part):
             self.gate_up = Linear(torch.cat([gate, up], 0))
         self.down = Linear(rt.weight(tensors[n["down"]]))
 
-    def forward(self, ctx, y, x):
+    def forward_from_residual(self, ctx, x, norm):
+        """With few rows and the fused epilogue the input norm runs inside the gate/up kernel."""
+        if not (self.fused_epilogue and hasattr(norm, "w") and hasattr(norm, "eps")
+                and self.gate_up.fuses_norm(x)):
+            return False
+        self.forward(ctx, None, x, fused_norm=norm)
+        return True
+
+    def forward(self, ctx, y, x, fused_norm=None):
         rt = ctx.rt
-        T = y.shape[0]
+        T = x.shape[0]
         act = rt.buffer("act", (T, self.intermediate_size))
-        if self.fused_epilogue:
+        if fused_norm is not None:
+            self.gate_up.forward_swiglu(x, act, norm=(fused_norm.w, fused_norm.eps))
+        elif self.fused_epilogue:
             self.gate_up.forward_swiglu(y, act)
         else:
             gu = rt.buffer("gate_up", (T, 2 * self.intermediate_size), torch.float32)

@@ -8,6 +8,8 @@ from .registry import register
 
 @register("norm", "rmsnorm")
 class RMSNorm(Part):
+    graph_safe = True
+
     def __init__(self, size, eps, weight):
         self.size = int(size)
         self.eps = float(eps)

@@ -13,6 +13,8 @@ from .registry import register
 
 @register("position", "none")
 class NoPosition(Part):
+    graph_safe = True
+
     def __init__(self, **_):
         pass
 
@@ -22,6 +24,8 @@ class NoPosition(Part):
 
 @register("position", "rope")
 class RotaryHalfSplit(Part):
+    graph_safe = True
+
     def __init__(self, theta, rotary_dims, max_positions):
         if rotary_dims % 2:
             raise ValueError("rotary_dims must be even")

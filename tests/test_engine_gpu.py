@@ -267,3 +267,35 @@ def test_sampling_through_generate_is_reproducible(model_root):
             assert tok in [i for i, _ in work]
             break
         seq.append(tok)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_graph_replays_equal_eager_steps(dtype, model_root):
+    """Decoding through captured graphs gives, replay after replay, what eager steps give; eager
+    work of other sequences (prompts, frees, a batch of another size) runs between the replays."""
+    folder = make_folder(model_root, "B", dtype)
+    vocab = 384
+    seqs = [random_tokens(vocab, 150, 90 + i) for i in range(3)]
+    other = random_tokens(vocab, 40, 99)
+    outs = {}
+    for graphs in (False, True):
+        engine = hb.Engine.from_folder(folder, dtype=dtype, max_tokens=64 * 16, use_graphs=graphs)
+        assert engine.use_graphs == graphs
+        slots = [engine.alloc_slot() for _ in seqs]
+        engine.step([StepEntry(s, t[:20], []) for s, t in zip(slots, seqs)])
+        got = []
+        for p in range(20, 150):
+            if p % 37 == 0:                       # eager work in between, with a synchronisation
+                extra = engine.alloc_slot()
+                engine.step([StepEntry(extra, other, [39])]).cpu()
+                engine.step([StepEntry(extra, [5], [0])]).cpu()
+                engine.free_slot(extra)
+            got.append(engine.step([StepEntry(s, [t[p]], [0]) for s, t in zip(slots, seqs)]).cpu().numpy())
+        outs[graphs] = np.stack(got)
+        if graphs:
+            assert any(st.graphs for st in engine._decode.values())
+        engine.cache.check()
+    assert np.array_equal(outs[True], outs[False])
+    ref = plain_logits(folder, seqs[1])
+    for i, p in enumerate(range(20, 150)):
+        assert close(outs[True][i][1], ref[p], dtype)[0], p

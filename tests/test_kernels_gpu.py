@@ -172,6 +172,8 @@ def paged_case(lengths, new_counts, nkv, hd, dtype, seed=0, n_pages=64, shuffle=
     import numpy as np
     meta.host_starts = np.array(starts, dtype=np.int32)
     meta.derived = {}
+    from herbert_rs_amd.engine.batch import bucket
+    meta.context_bucket = bucket(max(lengths))
     return meta, kv, dense
 
 
@@ -271,3 +273,30 @@ def test_gemm_mfma_packed_weights(M, N, K):
     packed = torch.empty(M, N, device=dev())
     mfma.gemm(a, mfma.pack_weight(w), packed, packed=True)
     assert torch.equal(plain, packed)
+
+
+@pytest.mark.parametrize("M,N,K,packed", [(1, 48, 32, False), (8, 6144, 4096, True), (16, 272, 96, False),
+                                          (33, 96, 64, True), (64, 1024, 512, True)])
+def test_gemm_mfma_with_fused_norm(M, N, K, packed):
+    from herbert_rs_amd.kernels import mfma
+    x = rand(M, K, seed=30, scale=2.0)
+    g = 1 + 0.1 * rand(K, seed=31)
+    w = rand(N, K, seed=32, dtype=torch.bfloat16, scale=0.1)
+    eps = 1e-6
+    inv = torch.rsqrt((x.double() ** 2).mean(-1, keepdim=True) + eps)
+    # the kernel rounds x * g to bfloat16 and applies inv to the float32 sums
+    xg = (x * g).to(torch.bfloat16).double()
+    want = ((xg @ w.double().T) * inv).float()
+    out = torch.empty(M, N, device=dev())
+    mfma.gemm(x, mfma.pack_weight(w) if packed else w, out, packed=packed, norm=(g, eps))
+    assert float((out - want).abs().max()) <= 1e-5 * float(want.abs().max()) + 1e-5
+    exact = ((x.double() * inv * g) @ w.double().T).float()          # and near the unrounded norm
+    assert float((out - exact).abs().max()) <= 2 ** -7 * float(exact.abs().max())
+    if N % 32 == 0:
+        gate, up = w[:N // 2].contiguous(), w[N // 2:].contiguous()
+        wi = mfma.interleave_gate_up(gate, up)
+        act = torch.empty(M, N // 2, dtype=torch.bfloat16, device=dev())
+        mfma.gemm_swiglu(x, mfma.pack_weight(wi) if packed else wi, act, packed=packed, norm=(g, eps))
+        gg, uu = (xg @ gate.double().T) * inv, (xg @ up.double().T) * inv
+        wanted = (gg / (1 + torch.exp(-gg)) * uu).float()
+        assert float((act.float() - wanted).abs().max()) <= 2 ** -7 * float(wanted.abs().max()) + 1e-5

@@ -228,7 +228,8 @@ def test_a_model_without_rotation():
 @register("mixer", "toy_decay")
 class ToyDecayMixer(Part):
     """s_t = decay * s_{t-1} + W y_t ; the mixer's output is s_t. The state s lives in the cache's
-    fixed-size area, one vector per sequence; it has no keys or values."""
+    fixed-size area, one vector per sequence; it has no keys or values. It loops on the host,
+    so it is not graph_safe (the default) and the engine runs its steps eagerly."""
 
     def __init__(self, hidden_size, decay, weight, shared=None):
         self.hidden_size, self.decay, self.weight_name = hidden_size, decay, weight
