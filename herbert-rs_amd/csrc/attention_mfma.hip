@@ -220,24 +220,30 @@ attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache,
     float m = -INFINITY, l = 0.f;
     const int krow = perm(c32);
 
+    // The loads of the next page go out as soon as the registers of the current one are free:
+    // keys right after Q K^T, values right after P V, so that memory works while the wave computes.
+    bf16x8 ka[2][HD / 16];
+    bf16x8 va[HD / 32][2][2];
+#define LOAD_K(PAGE_IDX)                                                                     \
+    {                                                                                        \
+        const bf16* kp = k_cache + ((size_t)pt[PAGE_IDX] * nkv + kvh) * PAGE * HD + g2 * (HD / 2); \
+        _Pragma("unroll") for (int kb = 0; kb < 2; ++kb)                                     \
+            _Pragma("unroll") for (int s = 0; s < HD / 16; ++s)                              \
+                ka[kb][s] = *(const bf16x8*)(kp + (size_t)(kb * 32 + krow) * HD + s * 8);    \
+    }
+#define LOAD_V(PAGE_IDX)                                                                     \
+    {                                                                                        \
+        const bf16* vp = v_cache + ((size_t)pt[PAGE_IDX] * nkv + kvh) * HD * PAGE + g2 * 8;  \
+        _Pragma("unroll") for (int d = 0; d < HD / 32; ++d)                                  \
+            _Pragma("unroll") for (int kb = 0; kb < 2; ++kb)                                 \
+                _Pragma("unroll") for (int h2 = 0; h2 < 2; ++h2)                             \
+                    va[d][kb][h2] = *(const bf16x8*)(vp + (size_t)(d * 32 + c32) * PAGE + kb * 32 + h2 * 16); \
+    }
+    if (first_page <= last_page) {
+        LOAD_K(first_page)
+        LOAD_V(first_page)
+    }
     for (int page_idx = first_page; page_idx <= last_page; ++page_idx) {
-        const int page = pt[page_idx];
-        const bf16* kp = k_cache + ((size_t)page * nkv + kvh) * PAGE * HD + g2 * (HD / 2);
-        const bf16* vp = v_cache + ((size_t)page * nkv + kvh) * HD * PAGE + g2 * 8;
-        bf16x8 ka[2][HD / 16];
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-            for (int s = 0; s < HD / 16; ++s)
-                ka[kb][s] = *(const bf16x8*)(kp + (size_t)(kb * 32 + krow) * HD + s * 8);
-        bf16x8 va[HD / 32][2][2];
-#pragma unroll
-        for (int d = 0; d < HD / 32; ++d)
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                for (int h2 = 0; h2 < 2; ++h2)
-                    va[d][kb][h2] = *(const bf16x8*)(vp + (size_t)(d * 32 + c32) * PAGE + kb * 32 + h2 * 16);
         f32x16 st[2];
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
@@ -247,6 +253,7 @@ attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache,
             for (int s = 0; s < HD / 16; ++s)
                 st[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[kb][s], qreg[s], st[kb], 0, 0, 0);
         }
+        if (page_idx < last_page) LOAD_K(page_idx + 1)
         float corr;
         bf16x8 pb[2][2];
         softmax_page(st, g2, page_idx * PAGE, lo, hi, c, m, l, corr, pb);
@@ -260,7 +267,10 @@ attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache,
                 for (int h2 = 0; h2 < 2; ++h2)
                     oacc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[d][kb][h2], pb[kb][h2], oacc[d], 0, 0, 0);
         }
+        if (page_idx < last_page) LOAD_V(page_idx + 1)
     }
+#undef LOAD_K
+#undef LOAD_V
     l += __shfl_xor(l, 32, 64);
     if (c32 < G) {
         const size_t base = ((size_t)b * nq + kvh * G + c32) * splits + split;
@@ -284,51 +294,58 @@ attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache,
 // One wave per (sequence, head). A kernel of its own: the partial results of waves on other
 // XCDs are visible at a kernel boundary without any fence that would write back an L2.
 template <int HD>
-__global__ void __launch_bounds__(64)
+__global__ void __launch_bounds__(256)
 attn_decode_merge_kernel(const float* __restrict__ partial_o, const float* __restrict__ partial_ml,
                          bf16* __restrict__ out, int splits, float c) {
-    const int lane = threadIdx.x;
+    // thread = (group of ranges, 4 consecutive d): its partial sums over ranges g, g + GROUPS, ...
+    // are loaded while the weights are worked out; the groups are then added in order through LDS.
+    constexpr int CHUNKS = HD / 4;             // float4 chunks of a row
+    constexpr int GROUPS = 256 / CHUNKS;       // 8 for HD = 128
+    __shared__ float wgt[1024];
+    __shared__ float sums[GROUPS][HD];
+    __shared__ float s_inv;
+    const int tid = threadIdx.x;
     const size_t bh = blockIdx.x;
-    {   // lanes over the ranges for the weights, then lanes over d for the sums
-        const float* ml = partial_ml + bh * splits * 2;
+    const float* ml = partial_ml + bh * splits * 2;
+    const int chunk = tid % CHUNKS, grp = tid / CHUNKS;
+
+    if (tid < 64) {
         float M = -INFINITY;
-        for (int s = lane; s < splits; s += 64) M = fmaxf(M, ml[2 * s]);
+        for (int s = tid; s < splits; s += 64) M = fmaxf(M, ml[2 * s]);
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) M = fmaxf(M, __shfl_xor(M, off, 64));
         float denom = 0.f;
-        for (int s0 = 0; s0 < splits; s0 += 64) {       // ranges in order, 64 at a time
-            const int s = s0 + lane;
-            float term = 0.f;
-            if (s < splits && ml[2 * s] != -INFINITY) term = fast_exp2((ml[2 * s] - M) * c) * ml[2 * s + 1];
+        for (int s0 = 0; s0 < splits; s0 += 64) {
+            const int s = s0 + tid;
+            float w = 0.f, term = 0.f;
+            if (s < splits && ml[2 * s] != -INFINITY) {
+                w = fast_exp2((ml[2 * s] - M) * c);
+                term = w * ml[2 * s + 1];
+            }
+            if (s < splits) wgt[s] = w;
 #pragma unroll
             for (int off = 32; off > 0; off >>= 1) term += __shfl_xor(term, off, 64);
             denom += term;
         }
-        const float inv = denom > 0.f ? 1.0f / denom : 0.f;
-        float acc[HD / 64 > 0 ? HD / 64 : 1];
-#pragma unroll
-        for (int j = 0; j < (HD + 63) / 64; ++j) acc[j] = 0.f;
-        for (int s0 = 0; s0 < splits; s0 += 64) {
-            const int sl = s0 + lane;
-            float wl = 0.f;
-            if (sl < splits && ml[2 * sl] != -INFINITY) wl = fast_exp2((ml[2 * sl] - M) * c);
-            const int n = splits - s0 < 64 ? splits - s0 : 64;
-#pragma unroll 8
-            for (int j = 0; j < n; ++j) {
-                const float wgt = __shfl(wl, j, 64);
-                const float* po = partial_o + (bh * splits + s0 + j) * HD;
-#pragma unroll
-                for (int e = 0; e < (HD + 63) / 64; ++e) {
-                    const int d = lane + 64 * e;
-                    if (d < HD) acc[e] = fmaf(wgt, po[d], acc[e]);
-                }
-            }
+        if (tid == 0) s_inv = denom > 0.f ? 1.0f / denom : 0.f;
+    }
+    __syncthreads();
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    if (grp < GROUPS)
+        for (int s = grp; s < splits; s += GROUPS) {
+            const f32x4 v = *(const f32x4*)(partial_o + (bh * splits + s) * HD + chunk * 4);
+            acc += v * wgt[s];
         }
+    if (grp < GROUPS) {
 #pragma unroll
-        for (int e = 0; e < (HD + 63) / 64; ++e) {
-            const int d = lane + 64 * e;
-            if (d < HD) out[bh * HD + d] = hb_from_float<bf16>(acc[e] * inv);
-        }
+        for (int e = 0; e < 4; ++e) sums[grp][chunk * 4 + e] = acc[e];
+    }
+    __syncthreads();
+    if (tid < HD) {
+        float total = 0.f;
+#pragma unroll
+        for (int g = 0; g < GROUPS; ++g) total += sums[g][tid];
+        out[bh * HD + tid] = hb_from_float<bf16>(total * s_inv);
     }
 }
 
@@ -369,7 +386,7 @@ extern "C" int hb_attn_decode_mfma(const void* q, const void* k_cache, const voi
     HB_REQUIRE(B > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attn_decode: bad sizes");
     HB_REQUIRE(page_size == PAGE, "attn_decode: pages must hold %d tokens", PAGE);
     HB_REQUIRE(nq / nkv <= 32, "attn_decode: more than 32 query heads share a kv head");
-    HB_REQUIRE(splits > 0 && splits <= 65535 && pages_per_split > 0 && nkv <= 65535, "attn_decode: bad split");
+    HB_REQUIRE(splits > 0 && splits <= 1024 && pages_per_split > 0 && nkv <= 65535, "attn_decode: bad split");
     HB_REQUIRE(window >= 0, "attn_decode: bad window");
     dim3 grid(B, nkv, splits);
     const float c = scale * LOG2E;
@@ -378,7 +395,7 @@ extern "C" int hb_attn_decode_mfma(const void* q, const void* k_cache, const voi
                                                     (const bf16*)v_cache, partial_o, partial_ml,         \
                                                     context_lens, slots, page_table, max_pages, nq, nkv, c, \
                                                     window, pages_per_split);                          \
-    attn_decode_merge_kernel<HDV><<<B * nq, 64, 0, stream>>>(partial_o, partial_ml, (bf16*)out, splits, c); \
+    attn_decode_merge_kernel<HDV><<<B * nq, 256, 0, stream>>>(partial_o, partial_ml, (bf16*)out, splits, c); \
     } while (0)
     if (hd == 32) LAUNCH_DECODE(32);
     else if (hd == 64) LAUNCH_DECODE(64);

@@ -9,25 +9,49 @@ HB_MODULE_ERROR_SLOT()
 
 // ------------------------------------------------------------------ argmax
 // First index of the largest value of each row (strict > while scanning upwards).
+// A row is cut into gridDim.y stretches; each block reduces one stretch to (value, index);
+// with more than one stretch a second launch reduces those.
+__device__ __forceinline__ bool better(float v, int i, float bv, int bi) {
+    return v > bv || (v == bv && i < bi);
+}
+
 __global__ void __launch_bounds__(1024)
-argmax_kernel(const float* __restrict__ logits, int ld, int V, int* __restrict__ out) {
+argmax_kernel(const float* __restrict__ logits, int ld, int V, int* __restrict__ out,
+              float* __restrict__ part_v, int* __restrict__ part_i, const float* __restrict__ in_v,
+              const int* __restrict__ in_i) {
     __shared__ float best_v[16];
     __shared__ int best_i[16];
-    const float* row = logits + (size_t)blockIdx.x * ld;
+    const int r = blockIdx.x;
+    const int chunks = gridDim.y;
+    const int per = (V + chunks - 1) / chunks;
+    const int begin = blockIdx.y * per;
+    const int end = begin + per < V ? begin + per : V;
     float bv = -INFINITY;
     int bi = 0x7fffffff;
-    for (int i = threadIdx.x; i < V; i += blockDim.x) {
-        const float v = row[i];
-        if (v > bv) {
-            bv = v;
-            bi = i;
+    if (in_v) {                       // second stage: V candidates (value, index) of this row
+        for (int i = threadIdx.x; i < V; i += blockDim.x) {
+            const float v = in_v[(size_t)r * V + i];
+            const int idx = in_i[(size_t)r * V + i];
+            if (better(v, idx, bv, bi)) {
+                bv = v;
+                bi = idx;
+            }
+        }
+    } else {
+        const float* row = logits + (size_t)r * ld;
+        for (int i = begin + threadIdx.x; i < end; i += blockDim.x) {
+            const float v = row[i];
+            if (v > bv) {
+                bv = v;
+                bi = i;
+            }
         }
     }
 #pragma unroll
     for (int off = HB_WAVE / 2; off > 0; off >>= 1) {
         const float ov = __shfl_xor(bv, off, HB_WAVE);
         const int oi = __shfl_xor(bi, off, HB_WAVE);
-        if (ov > bv || (ov == bv && oi < bi)) {
+        if (better(ov, oi, bv, bi)) {
             bv = ov;
             bi = oi;
         }
@@ -41,18 +65,33 @@ argmax_kernel(const float* __restrict__ logits, int ld, int V, int* __restrict__
     if (threadIdx.x == 0) {
         const int nw = (blockDim.x + HB_WAVE - 1) / HB_WAVE;
         for (int w = 1; w < nw; ++w)
-            if (best_v[w] > bv || (best_v[w] == bv && best_i[w] < bi)) {
+            if (better(best_v[w], best_i[w], bv, bi)) {
                 bv = best_v[w];
                 bi = best_i[w];
             }
-        // a row without any value above -inf (or all NaN) gives index 0, as a scan from 0 would
-        out[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;
+        if (part_v) {
+            part_v[(size_t)r * chunks + blockIdx.y] = bv;
+            part_i[(size_t)r * chunks + blockIdx.y] = bi;
+        } else {
+            // a row without any value above -inf (or all NaN) gives index 0, as a scan from 0 would
+            out[r] = bi == 0x7fffffff ? 0 : bi;
+        }
     }
 }
 
-extern "C" int hb_argmax(const float* logits, int ld, int R, int V, int* out, hipStream_t stream) {
+// scratch_v / scratch_i: [R, chunks] each when chunks > 1 (long rows are cut to fill the GPU).
+extern "C" int hb_argmax(const float* logits, int ld, int R, int V, int* out, float* scratch_v,
+                         int* scratch_i, int chunks, hipStream_t stream) {
     HB_REQUIRE(R > 0 && V > 0 && ld >= V, "argmax: bad sizes (R=%d, V=%d, ld=%d)", R, V, ld);
-    argmax_kernel<<<R, 1024, 0, stream>>>(logits, ld, V, out);
+    if (chunks <= 1 || !scratch_v || !scratch_i) {
+        argmax_kernel<<<dim3(R, 1), 1024, 0, stream>>>(logits, ld, V, out, nullptr, nullptr, nullptr, nullptr);
+    } else {
+        HB_REQUIRE(chunks <= 1024, "argmax: too many stretches");
+        argmax_kernel<<<dim3(R, chunks), 1024, 0, stream>>>(logits, ld, V, out, scratch_v, scratch_i, nullptr,
+                                                            nullptr);
+        argmax_kernel<<<dim3(R, 1), 64, 0, stream>>>(nullptr, 0, chunks, out, nullptr, nullptr, scratch_v,
+                                                     scratch_i);
+    }
     HB_CHECK_LAUNCH("argmax");
     return 0;
 }

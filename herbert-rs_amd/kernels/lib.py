@@ -34,7 +34,7 @@ SIGNATURES = {
         "hb_attention_plain": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P],
     },
     "sampling": {
-        "hb_argmax": [_P, _I, _I, _I, _P, _P],
+        "hb_argmax": [_P, _I, _I, _I, _P, _P, _P, _I, _P],
         "hb_sample": [_P, _I, _I, _I, _F, _I, _F, _P, _P, _P, _P, _P, _I, _P],
     },
 }

@@ -163,7 +163,13 @@ def argmax(logits, out):
     _check(logits, "logits", torch.float32, (None, None))
     R, V = logits.shape
     _check(out, "out", torch.int32, (R,))
-    lib.call("sampling", "hb_argmax", logits.data_ptr(), V, R, V, out.data_ptr(), _stream())
+    chunks = max(1, min(64, V // 8192, 1024 // R if R <= 1024 else 1))
+    sv = si = None
+    if chunks > 1:
+        sv = torch.empty((R, chunks), dtype=torch.float32, device=logits.device)
+        si = torch.empty((R, chunks), dtype=torch.int32, device=logits.device)
+    lib.call("sampling", "hb_argmax", logits.data_ptr(), V, R, V, out.data_ptr(), _ptr(sv), _ptr(si),
+             chunks, _stream())
 
 
 def sample(logits, temperature, top_k, top_p, rng_states, rng_index, out, scratch=None):

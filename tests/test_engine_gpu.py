@@ -194,17 +194,18 @@ def test_cli_generates_token_ids(model_root):
 
 
 # ---- sampling kernels against the plain sampler
-def test_argmax_kernel_takes_the_first_of_equals():
+@pytest.mark.parametrize("V", [5000, 70001])
+def test_argmax_kernel_takes_the_first_of_equals(V):
     from herbert_rs_amd.kernels import ops
-    logits = torch.randn(5, 5000)
+    logits = torch.randn(5, V)
     logits[0, 77] = logits[0, 4000] = 50.0
-    logits[1, 4999] = 60.0
+    logits[1, V - 1] = 60.0
     logits[2, 0] = 60.0
     logits[3] = -float("inf")
     out = torch.empty(5, dtype=torch.int32, device="cuda")
     ops.argmax(logits.cuda(), out)
     assert out.tolist() == [plain_sampler.argmax(r.numpy()) for r in logits]
-    assert out.tolist()[:4] == [77, 4999, 0, 0]
+    assert out.tolist()[:4] == [77, V - 1, 0, 0]
 
 
 @pytest.mark.parametrize("top_k,top_p", [(20, 1.0), (40, 0.9), (1, 1.0), (5, 0.3), (0, 1.0), (0, 0.8),
