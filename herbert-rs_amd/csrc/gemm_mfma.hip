@@ -15,6 +15,7 @@
 HB_MODULE_ERROR_SLOT()
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
@@ -310,17 +311,21 @@ static void pick_skinny(const void* X, const void* W, void* C, int M, int N, int
 }
 
 // ------------------------------------------------------------------- tiled
-#define BM 128
-#define BN 128
+// Workgroup tile BN x BM x 64 with BN = 64 TN, BM = 64 TM; 4 waves as 2 x 2, each wave
+// (32 TN) x (32 TM) outputs = TN x TM MFMA tiles of 32 x 32. The larger a wave's tile, the
+// fewer LDS reads per MFMA: (TN + TM) operand reads feed TN * TM instructions.
 #define BK 64
 #define LDT (BK + 8)   // padded row of a tile in LDS, in elements: 144 bytes, conflict-free b128 reads
 
-template <int EPI, bool PACKED>
+template <int EPI, bool PACKED, int TN, int TM>
 __global__ void __launch_bounds__(256)
 gemm_tiled_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* __restrict__ Cv, int M, int N,
                   int K, int ldc, int m_tiles, int n_tiles) {
-    __shared__ __attribute__((aligned(16))) bf16 Ws[2][BN * LDT];
-    __shared__ __attribute__((aligned(16))) bf16 Xs[2][BM * LDT];
+    constexpr int BN = 64 * TN, BM = 64 * TM;
+    constexpr int WCH = BN / 32, XCH = BM / 32;        // 16-byte chunks per thread of each operand tile
+    extern __shared__ __attribute__((aligned(16))) bf16 lds[];
+    bf16* Ws = lds;                                     // [2][BN * LDT]
+    bf16* Xs = lds + 2 * BN * LDT;                      // [2][BM * LDT]
 
     // workgroup ids go round the 8 XCDs; give each XCD a contiguous run of tiles so that the
     // workgroups that share a weight tile also share an L2
@@ -334,19 +339,18 @@ gemm_tiled_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* 
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
-    const int wn = wave >> 1, wm = wave & 1;       // wave's 64 x 64 part of the tile
+    const int wn = wave >> 1, wm = wave & 1;
     const int c32 = lane & 31, g2 = lane >> 5;
 
-    // global -> registers: 4 chunks of 16 bytes of each operand per thread.
-    // Row-major: thread (lrow, lchunk) takes k-chunk lchunk of rows lrow + 32 i.
-    // Packed weights: chunk c = tid + 256 i is lane c % 64 of operand c / 64 (8 row blocks x 2 k-steps
+    // global -> registers. Row-major: thread (lrow, lchunk) takes k-chunk lchunk of rows lrow + 32 i.
+    // Packed weights: chunk c = tid + 256 i is lane c % 64 of operand c / 64 (row blocks x 2 k-steps
     // of the tile), 1 KB contiguous per 64 threads.
     const int lrow = tid >> 3, lchunk = tid & 7;
-    const bf16* wsrc[4];
-    const bf16* xsrc[4];
-    int wdst[4];
+    const bf16* wsrc[WCH];
+    const bf16* xsrc[XCH];
+    int wdst[WCH];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < WCH; ++i) {
         if (PACKED) {
             const int c = tid + 256 * i;
             const int pl = c & 63, op = c >> 6;
@@ -361,87 +365,98 @@ gemm_tiled_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* 
             wsrc[i] = W + (size_t)n * K + lchunk * 8;
             wdst[i] = (lrow + 32 * i) * LDT + lchunk * 8;
         }
+    }
+#pragma unroll
+    for (int i = 0; i < XCH; ++i) {
         int m = m0 + lrow + 32 * i;
         if (m >= M) m = M - 1;
         xsrc[i] = X + (size_t)m * K + lchunk * 8;
     }
     constexpr int WTILE_STEP = PACKED ? 2 * 64 * 8 : BK;     // elements from one k-tile to the next
-    bf16x8 wreg[4], xreg[4];
+    bf16x8 wreg[WCH], xreg[XCH];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        wreg[i] = *(const bf16x8*)(wsrc[i]);
-        xreg[i] = *(const bf16x8*)(xsrc[i]);
-    }
+    for (int i = 0; i < WCH; ++i) wreg[i] = *(const bf16x8*)(wsrc[i]);
+#pragma unroll
+    for (int i = 0; i < XCH; ++i) xreg[i] = *(const bf16x8*)(xsrc[i]);
 
-    f32x16 acc[2][2];
+    f32x16 acc[TN][TM];
 #pragma unroll
-    for (int a = 0; a < 2; ++a)
+    for (int a = 0; a < TN; ++a)
 #pragma unroll
-        for (int b = 0; b < 2; ++b)
+        for (int b = 0; b < TM; ++b)
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.f;
 
     const int ktiles = K / BK;
     for (int kt = 0; kt < ktiles; ++kt) {
-        const int buf = kt & 1;
+        bf16* wbuf = Ws + (kt & 1) * BN * LDT;
+        bf16* xbuf = Xs + (kt & 1) * BM * LDT;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            *(bf16x8*)(&Ws[buf][wdst[i]]) = wreg[i];
-            *(bf16x8*)(&Xs[buf][(lrow + 32 * i) * LDT + lchunk * 8]) = xreg[i];
-        }
+        for (int i = 0; i < WCH; ++i) *(bf16x8*)(&wbuf[wdst[i]]) = wreg[i];
+#pragma unroll
+        for (int i = 0; i < XCH; ++i) *(bf16x8*)(&xbuf[(lrow + 32 * i) * LDT + lchunk * 8]) = xreg[i];
         __syncthreads();
         if (kt + 1 < ktiles) {
-            const int koff = (kt + 1) * BK;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                wreg[i] = *(const bf16x8*)(wsrc[i] + (size_t)(kt + 1) * WTILE_STEP);
-                xreg[i] = *(const bf16x8*)(xsrc[i] + koff);
-            }
+            for (int i = 0; i < WCH; ++i) wreg[i] = *(const bf16x8*)(wsrc[i] + (size_t)(kt + 1) * WTILE_STEP);
+#pragma unroll
+            for (int i = 0; i < XCH; ++i) xreg[i] = *(const bf16x8*)(xsrc[i] + (kt + 1) * BK);
         }
 #pragma unroll
         for (int ks = 0; ks < BK / 16; ++ks) {
-            bf16x8 wa[2], xb[2];
+            bf16x8 wa[TN], xb[TM];
 #pragma unroll
-            for (int a = 0; a < 2; ++a)
-                wa[a] = *(const bf16x8*)(&Ws[buf][(wn * 64 + a * 32 + c32) * LDT + ks * 16 + g2 * 8]);
+            for (int a = 0; a < TN; ++a)
+                wa[a] = *(const bf16x8*)(&wbuf[(wn * 32 * TN + a * 32 + c32) * LDT + ks * 16 + g2 * 8]);
 #pragma unroll
-            for (int b = 0; b < 2; ++b)
-                xb[b] = *(const bf16x8*)(&Xs[buf][(wm * 64 + b * 32 + c32) * LDT + ks * 16 + g2 * 8]);
+            for (int b = 0; b < TM; ++b)
+                xb[b] = *(const bf16x8*)(&xbuf[(wm * 32 * TM + b * 32 + c32) * LDT + ks * 16 + g2 * 8]);
 #pragma unroll
-            for (int a = 0; a < 2; ++a)
+            for (int a = 0; a < TN; ++a)
 #pragma unroll
-                for (int b = 0; b < 2; ++b)
+                for (int b = 0; b < TM; ++b)
                     acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wa[a], xb[b], acc[a][b], 0, 0, 0);
         }
         // the other buffer is written next; everyone has finished reading it a tile ago
     }
 
-    // lane: m = m0 + wm*64 + b*32 + c32 ; n = n0 + wn*64 + a*32 + 8*(i/4) + 4*g2 + i%4
+    // lane: m = m0 + wm*32*TM + b*32 + c32 ; n = n0 + wn*32*TN + a*32 + 8*(i/4) + 4*g2 + i%4
 #pragma unroll
-    for (int b = 0; b < 2; ++b) {
-        const int m = m0 + wm * 64 + b * 32 + c32;
+    for (int b = 0; b < TM; ++b) {
+        const int m = m0 + wm * 32 * TM + b * 32 + c32;
         if (m >= M) continue;
         if (EPI == EPI_SWIGLU) {
             // weight rows come in blocks of 16 gate rows then 16 up rows: within a 32-row MFMA block,
             // rows 0..15 (i/4 in {0,1}) are gate and rows 16..31 (i/4 in {2,3}) the matching up rows
             bf16* C = (bf16*)Cv;
 #pragma unroll
-            for (int a = 0; a < 2; ++a)
+            for (int a = 0; a < TN; ++a) {
+                const int fused_n = n0 + wn * 32 * TN + a * 32;            // start of a gate/up pair
 #pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    const int fused_n = n0 + wn * 64 + a * 32;            // start of a gate/up pair
-                    const int n = fused_n / 2 + 8 * (i / 4) + 4 * g2 + (i % 4);
-                    if (n < N / 2)
-                        C[(size_t)m * ldc + n] =
-                            hb_from_float<bf16>(silu_mul(acc[a][b][i], acc[a][b][i + 8]));
+                for (int q = 0; q < 2; ++q) {
+                    const int n = fused_n / 2 + 8 * q + 4 * g2;
+                    if (n + 3 < N / 2 && (ldc & 3) == 0) {
+                        bf16x4 v;
+#pragma unroll
+                        for (int r = 0; r < 4; ++r)
+                            v[r] = (__bf16)silu_mul(acc[a][b][4 * q + r], acc[a][b][4 * q + r + 8]);
+                        *(bf16x4*)((__bf16*)C + (size_t)m * ldc + n) = v;
+                    } else {
+#pragma unroll
+                        for (int r = 0; r < 4; ++r)
+                            if (n + r < N / 2)
+                                C[(size_t)m * ldc + n + r] = hb_from_float<bf16>(
+                                    silu_mul(acc[a][b][4 * q + r], acc[a][b][4 * q + r + 8]));
+                    }
                 }
+            }
         } else {
             float* C = (float*)Cv;
 #pragma unroll
-            for (int a = 0; a < 2; ++a)
+            for (int a = 0; a < TN; ++a)
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
-                    const int n = n0 + wn * 64 + a * 32 + 8 * q + 4 * g2;
+                    const int n = n0 + wn * 32 * TN + a * 32 + 8 * q + 4 * g2;
                     float* dst = C + (size_t)m * ldc + n;
                     if (n + 3 < N && (ldc & 3) == 0) {
                         f32x4 v = {acc[a][b][4 * q], acc[a][b][4 * q + 1], acc[a][b][4 * q + 2],
@@ -466,13 +481,53 @@ gemm_tiled_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* 
     }
 }
 
+template <int TN, int TM>
+static int launch_tiled(const void* X, const void* W, void* C, int M, int N, int K, int ldc, int epi,
+                        int packed, hipStream_t stream) {
+    constexpr int BN = 64 * TN, BM = 64 * TM;
+    const int m_tiles = (M + BM - 1) / BM, n_tiles = (N + BN - 1) / BN;
+    const long total = (long)m_tiles * n_tiles;
+    HB_REQUIRE(total < (1l << 30), "gemm_mfma: too many tiles");
+    const int blocks = (int)((total + 7) / 8 * 8);
+    const size_t lds = (size_t)2 * (BN + BM) * LDT * sizeof(bf16);
+    const bf16* x = (const bf16*)X;
+    const bf16* w = (const bf16*)W;
+#define TILED_GO(EPIV, PK)                                                                          \
+    do {                                                                                            \
+        auto kern = gemm_tiled_kernel<EPIV, PK, TN, TM>;                                            \
+        if (lds > 64 * 1024) {                                                                      \
+            static bool raised = false;                                                             \
+            if (!raised) {                                                                          \
+                hipError_t e = hipFuncSetAttribute((const void*)kern,                               \
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
+                HB_REQUIRE(e == hipSuccess, "gemm_mfma: cannot have %zu bytes of LDS: %s", lds,     \
+                           hipGetErrorString(e));                                                   \
+                raised = true;                                                                      \
+            }                                                                                       \
+        }                                                                                           \
+        kern<<<blocks, 256, lds, stream>>>(x, w, C, M, N, K, ldc, m_tiles, n_tiles);                \
+    } while (0)
+    if (packed) {
+        if (epi == EPI_STORE) TILED_GO(EPI_STORE, true);
+        else if (epi == EPI_ADD) TILED_GO(EPI_ADD, true);
+        else TILED_GO(EPI_SWIGLU, true);
+    } else {
+        if (epi == EPI_STORE) TILED_GO(EPI_STORE, false);
+        else if (epi == EPI_ADD) TILED_GO(EPI_ADD, false);
+        else TILED_GO(EPI_SWIGLU, false);
+    }
+#undef TILED_GO
+    HB_CHECK_LAUNCH("gemm_tiled");
+    return 0;
+}
+
 // C (+)= X @ W^T. X [M, K] bf16, W [N, K] bf16. epi 0: C f32 [M, N] stored; 1: added to;
 // 2: W's rows are gate/up interleaved in blocks of 16 and C is bf16 [M, N / 2] = silu(gate) * up.
 // packed != 0: W is stored as [N / 16][K / 32][64 lanes][8]: lane = 16 * (k / 8 % 4) + n % 16.
 // norm_w != null: X is the float32 residual stream [M, K] and the product is RMSNorm(X; norm_w, eps) W^T
 // (M <= 64 only, never with the add epilogue).
 extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N, int K, int ldc, int epi,
-                            int packed, const float* norm_w, float eps, hipStream_t stream) {
+                            int packed, const float* norm_w, float eps, int tile_hint, hipStream_t stream) {
     HB_REQUIRE(!norm_w || (M <= 64 && epi != EPI_ADD), "gemm_mfma: the fused norm takes M <= 64 and no add");
     HB_REQUIRE(!packed || N % 16 == 0, "gemm_mfma: packed weights need N %% 16 == 0");
     HB_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_mfma: empty problem (M=%d, N=%d, K=%d)", M, N, K);
@@ -489,24 +544,17 @@ extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N,
         return 0;
     }
     HB_REQUIRE(K % BK == 0, "gemm_mfma: K=%d is no multiple of %d (needed for M > 64)", K, BK);
-    const int m_tiles = (M + BM - 1) / BM, n_tiles = (N + BN - 1) / BN;
-    const long total = (long)m_tiles * n_tiles;
-    HB_REQUIRE(total < (1l << 30), "gemm_mfma: too many tiles");
-    const int blocks = (int)((total + 7) / 8 * 8);
-    const bf16* x = (const bf16*)X;
-    const bf16* w = (const bf16*)W;
-#define TILED_GO(EPIV, PK) \
-    gemm_tiled_kernel<EPIV, PK><<<blocks, 256, 0, stream>>>(x, w, C, M, N, K, ldc, m_tiles, n_tiles)
-    if (packed) {
-        if (epi == EPI_STORE) TILED_GO(EPI_STORE, true);
-        else if (epi == EPI_ADD) TILED_GO(EPI_ADD, true);
-        else TILED_GO(EPI_SWIGLU, true);
-    } else {
-        if (epi == EPI_STORE) TILED_GO(EPI_STORE, false);
-        else if (epi == EPI_ADD) TILED_GO(EPI_ADD, false);
-        else TILED_GO(EPI_SWIGLU, false);
+    // tile_hint: 0 = choose; otherwise 10 * TN + TM (for measurements)
+    int tile = tile_hint;
+    // 256 x 256 tiles read LDS and L1 half as often per MFMA, but only pay with enough of them
+    // to keep every CU busy (one fits a CU at a time)
+    if (tile == 0) tile = ((long)((M + 255) / 256) * ((N + 255) / 256) >= 512) ? 44 : 22;
+    switch (tile) {
+        case 22: return launch_tiled<2, 2>(X, W, C, M, N, K, ldc, epi, packed, stream);
+        case 24: return launch_tiled<2, 4>(X, W, C, M, N, K, ldc, epi, packed, stream);
+        case 42: return launch_tiled<4, 2>(X, W, C, M, N, K, ldc, epi, packed, stream);
+        case 44: return launch_tiled<4, 4>(X, W, C, M, N, K, ldc, epi, packed, stream);
+        default: HB_REQUIRE(false, "gemm_mfma: unknown tile %d", tile);
     }
-#undef TILED_GO
-    HB_CHECK_LAUNCH("gemm_tiled");
     return 0;
 }

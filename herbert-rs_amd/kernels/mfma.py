@@ -12,7 +12,7 @@ _P = ctypes.c_void_p
 _I = ctypes.c_int
 _F = ctypes.c_float
 lib.register_signatures("gemm_mfma", {
-    "hb_gemm_mfma": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _F, _P],
+    "hb_gemm_mfma": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _F, _I, _P],
 })
 
 EPI_STORE, EPI_ADD, EPI_SWIGLU = 0, 1, 2
@@ -55,13 +55,17 @@ def _norm_args(a, norm, K):
     return weight.data_ptr(), float(eps)
 
 
+NORM_FUSE_MAX_M = 16
+
+
 def norm_fusable(a, w):
-    """True if RMSNorm(a) @ w^T can run as one kernel: few rows of the float32 residual stream."""
-    return (a.dtype == torch.float32 and w.dtype == torch.bfloat16 and a.shape[0] <= SKINNY_MAX_M
+    """True if RMSNorm(a) @ w^T should run as one kernel: at most 16 rows of the float32 residual
+    stream (every workgroup reads all of them; with more rows that costs more than a norm kernel)."""
+    return (a.dtype == torch.float32 and w.dtype == torch.bfloat16 and a.shape[0] <= NORM_FUSE_MAX_M
             and a.shape[1] % 32 == 0)
 
 
-def gemm(a, w, out, accumulate=False, packed=False, norm=None):
+def gemm(a, w, out, accumulate=False, packed=False, norm=None, tile=0):
     """out f32 [M, N] (+)= a bf16 [M, K] @ w bf16 [N, K]^T (w as stored, or as pack_weight gives it).
     norm = (weight f32 [K], eps): a is the float32 residual stream and is RMS-normed on the way."""
     M, K = a.shape
@@ -72,7 +76,7 @@ def gemm(a, w, out, accumulate=False, packed=False, norm=None):
     if K % 32 or (M > SKINNY_MAX_M and K % 64) or (norm is not None and accumulate):
         raise BackendError(f"gemm_mfma refuses M={M}, N={N}, K={K}")
     lib.call("gemm_mfma", "hb_gemm_mfma", a.data_ptr(), w.data_ptr(), out.data_ptr(), M, N, K, N,
-             EPI_ADD if accumulate else EPI_STORE, 1 if packed else 0, norm_ptr, eps, _stream())
+             EPI_ADD if accumulate else EPI_STORE, 1 if packed else 0, norm_ptr, eps, int(tile), _stream())
 
 
 def interleave_gate_up(gate, up):
@@ -84,7 +88,7 @@ def interleave_gate_up(gate, up):
     return torch.stack([gate.view(I // 16, 16, K), up.view(I // 16, 16, K)], 1).reshape(2 * I, K).contiguous()
 
 
-def gemm_swiglu(a, w_interleaved, out, packed=False, norm=None):
+def gemm_swiglu(a, w_interleaved, out, packed=False, norm=None, tile=0):
     """out bf16 [M, I] = silu(a @ gate^T) * (a @ up^T), the weights interleaved as above."""
     M, K = a.shape
     norm_ptr, eps = _norm_args(a, norm, K)
@@ -94,7 +98,7 @@ def gemm_swiglu(a, w_interleaved, out, packed=False, norm=None):
     if K % 32 or (M > SKINNY_MAX_M and K % 64) or N % 32:
         raise BackendError(f"gemm_mfma (SwiGLU) refuses M={M}, N={N}, K={K}")
     lib.call("gemm_mfma", "hb_gemm_mfma", a.data_ptr(), w_interleaved.data_ptr(), out.data_ptr(), M, N, K,
-             N // 2, EPI_SWIGLU, 1 if packed else 0, norm_ptr, eps, _stream())
+             N // 2, EPI_SWIGLU, 1 if packed else 0, norm_ptr, eps, int(tile), _stream())
 
 
 lib.register_signatures("attention_mfma", {
