@@ -46,6 +46,8 @@ def main():
     ap.add_argument("--context", type=int, default=None)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
+    ap.add_argument("--prefill-only", action="store_true",
+                    help="run the 2,048-token prefill alone (for profiles); prints no JSON line")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU only: --gpus {args.gpus} is not supported (this library "
@@ -126,6 +128,10 @@ def main():
         torch.cuda.synchronize()
         return (time.perf_counter() - t) / reps
 
+    if args.prefill_only:
+        sec = prefill_run(2048, max(1, args.steps))
+        print(f"[bench] prefill 2048: {2048 / sec:.0f} tok/s, {sec * 1e3:.2f} ms", file=sys.stderr, flush=True)
+        return 0
     value, ms = decode_run(args.batch, args.steps, args.warmup)
     print(f"[bench] decode b{args.batch}: {value:.1f} tok/s, {ms:.3f} ms/step", file=sys.stderr, flush=True)
     avg_ctx = context - args.steps / 2.0
