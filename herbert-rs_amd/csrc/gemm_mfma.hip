@@ -4,8 +4,8 @@
 //   skinny (M <= 64, decoding): HBM-bound. The weights stream from memory straight into
 //     MFMA operands (each is used once), four waves of a workgroup split K between them
 //     and add their parts through LDS in a fixed order.
-//   tiled (M > 64, prompts): 128 x 128 x 64 tiles staged through LDS, 32x32x16 MFMA,
-//     global loads of the next tile in flight while the current one is multiplied.
+//   tiled (M > 64, prompts): 256 x 256 or 128 x 128 tiles loaded from global memory straight
+//     into a ring of LDS stages, one or two k-steps ahead of the MFMAs that consume them.
 // In both the weight rows are the MFMA's first operand, so a lane ends up with four
 // consecutive n of one m: row-major stores of C are vector stores.
 // Epilogues: 0 store float32, 1 add to float32 (the residual stream), 2 SwiGLU to bfloat16
@@ -311,190 +311,186 @@ static void pick_skinny(const void* X, const void* W, void* C, int M, int N, int
 }
 
 // ------------------------------------------------------------------- tiled
-// Workgroup tile BN x BM x 64 with BN = 64 TN, BM = 64 TM; 4 waves as 2 x 2, each wave
-// (32 TN) x (32 TM) outputs = TN x TM MFMA tiles of 32 x 32. The larger a wave's tile, the
-// fewer LDS reads per MFMA: (TN + TM) operand reads feed TN * TM instructions.
-#define BK 64
-#define LDT (BK + 8)   // padded row of a tile in LDS, in elements: 144 bytes, conflict-free b128 reads
+// The product for many rows (prompts), with the tiles going from global memory straight into LDS
+// (global_load_lds_dwordx4: a lane's 16 bytes land at base + 16 * lane, no registers, no
+// ds_write) and a ring of STAGES k-steps of 32 in LDS, loaded STAGES - 1 steps ahead.
+// LDS holds MFMA operands as they are used: a block of 16 rows x 32 k is 1 KB in lane order
+// (lane = 16 * (k / 8 % 4) + row % 16), which is the packed weight order, so a packed weight
+// block is one contiguous 1 KB load and an operand read is lane * 16 bytes, free of conflicts.
+// 16x16x32 MFMA, weight rows first: a lane ends with four consecutive n of one m.
+// Workgroup: WNW x WMW waves, each TNB x TMB blocks of 16: BN = 16 TNB WNW, BM = 16 TMB WMW.
+template <int N_OUTSTANDING>
+__device__ __forceinline__ void wait_vmcnt() {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N_OUTSTANDING) : "memory");
+}
 
-template <int EPI, bool PACKED, int TN, int TM>
-__global__ void __launch_bounds__(256)
-gemm_tiled_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* __restrict__ Cv, int M, int N,
-                  int K, int ldc, int m_tiles, int n_tiles) {
-    constexpr int BN = 64 * TN, BM = 64 * TM;
-    constexpr int WCH = BN / 32, XCH = BM / 32;        // 16-byte chunks per thread of each operand tile
-    extern __shared__ __attribute__((aligned(16))) bf16 lds[];
-    bf16* Ws = lds;                                     // [2][BN * LDT]
-    bf16* Xs = lds + 2 * BN * LDT;                      // [2][BM * LDT]
+template <int EPI, bool PACKED, int TNB, int TMB, int WNW, int WMW, int STAGES, int KS>
+__global__ void __launch_bounds__(64 * WNW * WMW)
+gemm_dma_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* __restrict__ Cv, int M, int N,
+                int K, int ldc, int m_tiles, int n_tiles) {
+    constexpr int NW = WNW * WMW;
+    constexpr int BN = 16 * TNB * WNW, BM = 16 * TMB * WMW;
+    constexpr int WBLK = BN / 16, XBLK = BM / 16, BLKS = WBLK + XBLK;   // 1 KB blocks of a stage
+    constexpr int WL = WBLK / NW, XL = XBLK / NW;                      // loads of a wave per stage
+    static_assert(WBLK % NW == 0 && XBLK % NW == 0, "blocks must divide over the waves");
+    extern __shared__ __attribute__((aligned(1024))) bf16 lds[];        // [STAGES][KS][BLKS][512]
 
-    // workgroup ids go round the 8 XCDs; give each XCD a contiguous run of tiles so that the
-    // workgroups that share a weight tile also share an L2
     const int total = m_tiles * n_tiles;
     const int chunk = (total + 7) / 8;
-    const int id = (blockIdx.x % 8) * chunk + blockIdx.x / 8;
+    const int id = (blockIdx.x % 8) * chunk + blockIdx.x / 8;          // a run of tiles per XCD
     if (id >= total) return;
-    const int n_tile = id / m_tiles;
-    const int m_tile = id % m_tiles;
+    const int n_tile = id / m_tiles, m_tile = id % m_tiles;
     const int m0 = m_tile * BM, n0 = n_tile * BN;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
-    const int wn = wave >> 1, wm = wave & 1;
-    const int c32 = lane & 31, g2 = lane >> 5;
+    const int r16 = lane & 15, g4 = lane >> 4;
+    const int wn = wave / WMW, wm = wave % WMW;
+    const int k32 = K / 32;              // k-steps of 32 in all
+    const int nsteps = k32 / KS;         // stages' worth of them (K is a multiple of 32 KS)
 
-    // global -> registers. Row-major: thread (lrow, lchunk) takes k-chunk lchunk of rows lrow + 32 i.
-    // Packed weights: chunk c = tid + 256 i is lane c % 64 of operand c / 64 (row blocks x 2 k-steps
-    // of the tile), 1 KB contiguous per 64 threads.
-    const int lrow = tid >> 3, lchunk = tid & 7;
-    const bf16* wsrc[WCH];
-    const bf16* xsrc[XCH];
-    int wdst[WCH];
+    // this wave's loads: W blocks wave * WL + i, X blocks wave * XL + i
+    const bf16* wsrc[WL];
+    const bf16* xsrc[XL];
 #pragma unroll
-    for (int i = 0; i < WCH; ++i) {
+    for (int i = 0; i < WL; ++i) {
+        const int blk = wave * WL + i;
         if (PACKED) {
-            const int c = tid + 256 * i;
-            const int pl = c & 63, op = c >> 6;
-            const int nb_local = op >> 1, ks_local = op & 1;
-            int nb = n0 / 16 + nb_local;
+            int nb = n0 / 16 + blk;
             if (nb * 16 >= N) nb = (N - 1) / 16;
-            wsrc[i] = W + (((size_t)nb * (K / 32) + ks_local) * 64 + pl) * 8;
-            wdst[i] = (nb_local * 16 + (pl & 15)) * LDT + ks_local * 32 + (pl >> 4) * 8;
+            wsrc[i] = W + ((size_t)nb * k32 * 64 + lane) * 8;
         } else {
-            int n = n0 + lrow + 32 * i;
+            int n = n0 + blk * 16 + r16;
             if (n >= N) n = N - 1;
-            wsrc[i] = W + (size_t)n * K + lchunk * 8;
-            wdst[i] = (lrow + 32 * i) * LDT + lchunk * 8;
+            wsrc[i] = W + (size_t)n * K + g4 * 8;
         }
     }
 #pragma unroll
-    for (int i = 0; i < XCH; ++i) {
-        int m = m0 + lrow + 32 * i;
+    for (int i = 0; i < XL; ++i) {
+        int m = m0 + (wave * XL + i) * 16 + r16;
         if (m >= M) m = M - 1;
-        xsrc[i] = X + (size_t)m * K + lchunk * 8;
+        xsrc[i] = X + (size_t)m * K + g4 * 8;
     }
-    constexpr int WTILE_STEP = PACKED ? 2 * 64 * 8 : BK;     // elements from one k-tile to the next
-    bf16x8 wreg[WCH], xreg[XCH];
-#pragma unroll
-    for (int i = 0; i < WCH; ++i) wreg[i] = *(const bf16x8*)(wsrc[i]);
-#pragma unroll
-    for (int i = 0; i < XCH; ++i) xreg[i] = *(const bf16x8*)(xsrc[i]);
+    constexpr int WSTEP = PACKED ? 512 : 32;
 
-    f32x16 acc[TN][TM];
+    auto issue = [&](int step, int stage) {
 #pragma unroll
-    for (int a = 0; a < TN; ++a)
+        for (int ks = 0; ks < KS; ++ks) {
+            bf16* base = lds + (size_t)(stage * KS + ks) * BLKS * 512;
+            const size_t k = (size_t)step * KS + ks;
 #pragma unroll
-        for (int b = 0; b < TM; ++b)
+            for (int i = 0; i < WL; ++i)
+                __builtin_amdgcn_global_load_lds(
+                    (const __attribute__((address_space(1))) void*)(wsrc[i] + k * WSTEP),
+                    (__attribute__((address_space(3))) void*)(base + (wave * WL + i) * 512), 16, 0, 0);
 #pragma unroll
-            for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.f;
+            for (int i = 0; i < XL; ++i)
+                __builtin_amdgcn_global_load_lds(
+                    (const __attribute__((address_space(1))) void*)(xsrc[i] + k * 32),
+                    (__attribute__((address_space(3))) void*)(base + (WBLK + wave * XL + i) * 512), 16, 0, 0);
+        }
+    };
 
-    const int ktiles = K / BK;
-    for (int kt = 0; kt < ktiles; ++kt) {
-        bf16* wbuf = Ws + (kt & 1) * BN * LDT;
-        bf16* xbuf = Xs + (kt & 1) * BM * LDT;
+    f32x4 acc[TNB][TMB];
 #pragma unroll
-        for (int i = 0; i < WCH; ++i) *(bf16x8*)(&wbuf[wdst[i]]) = wreg[i];
+    for (int a = 0; a < TNB; ++a)
 #pragma unroll
-        for (int i = 0; i < XCH; ++i) *(bf16x8*)(&xbuf[(lrow + 32 * i) * LDT + lchunk * 8]) = xreg[i];
+        for (int b = 0; b < TMB; ++b) acc[a][b] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+#pragma unroll
+    for (int st = 0; st < STAGES - 1; ++st) issue(st < nsteps ? st : nsteps - 1, st);
+
+    for (int t = 0; t < nsteps; ++t) {
+        // this wave's loads of step t have landed (those of the STAGES - 2 later steps may be in flight);
+        // after the barrier everyone's have, and everyone has finished reading step t - 1
+        wait_vmcnt<(STAGES - 2) * (WL + XL) * KS>();
         __syncthreads();
-        if (kt + 1 < ktiles) {
-#pragma unroll
-            for (int i = 0; i < WCH; ++i) wreg[i] = *(const bf16x8*)(wsrc[i] + (size_t)(kt + 1) * WTILE_STEP);
-#pragma unroll
-            for (int i = 0; i < XCH; ++i) xreg[i] = *(const bf16x8*)(xsrc[i] + (kt + 1) * BK);
+        {
+            const int nt = t + STAGES - 1;
+            issue(nt < nsteps ? nt : nsteps - 1, nt % STAGES);
         }
 #pragma unroll
-        for (int ks = 0; ks < BK / 16; ++ks) {
-            bf16x8 wa[TN], xb[TM];
+        for (int ks = 0; ks < KS; ++ks) {
+            const bf16* base = lds + (size_t)((t % STAGES) * KS + ks) * BLKS * 512 + lane * 8;
+            bf16x8 wv[TNB], xv[TMB];
 #pragma unroll
-            for (int a = 0; a < TN; ++a)
-                wa[a] = *(const bf16x8*)(&wbuf[(wn * 32 * TN + a * 32 + c32) * LDT + ks * 16 + g2 * 8]);
+            for (int a = 0; a < TNB; ++a) wv[a] = *(const bf16x8*)(base + (wn * TNB + a) * 512);
 #pragma unroll
-            for (int b = 0; b < TM; ++b)
-                xb[b] = *(const bf16x8*)(&xbuf[(wm * 32 * TM + b * 32 + c32) * LDT + ks * 16 + g2 * 8]);
+            for (int b = 0; b < TMB; ++b) xv[b] = *(const bf16x8*)(base + (WBLK + wm * TMB + b) * 512);
+            // all operand reads go out before the first MFMA: the other wave of the SIMD computes meanwhile
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int a = 0; a < TN; ++a)
+            for (int a = 0; a < TNB; ++a)
 #pragma unroll
-                for (int b = 0; b < TM; ++b)
-                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wa[a], xb[b], acc[a][b], 0, 0, 0);
+                for (int b = 0; b < TMB; ++b)
+                    acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[a], xv[b], acc[a][b], 0, 0, 0);
         }
-        // the other buffer is written next; everyone has finished reading it a tile ago
     }
+    wait_vmcnt<0>();      // the loads past the end (repeats of the last step) have landed too
 
-    // lane: m = m0 + wm*32*TM + b*32 + c32 ; n = n0 + wn*32*TN + a*32 + 8*(i/4) + 4*g2 + i%4
+    // lane: m = m0 + (wm * TMB + b) * 16 + r16 ; n = n0 + (wn * TNB + a) * 16 + g4 * 4 + i
 #pragma unroll
-    for (int b = 0; b < TM; ++b) {
-        const int m = m0 + wm * 32 * TM + b * 32 + c32;
+    for (int b = 0; b < TMB; ++b) {
+        const int m = m0 + (wm * TMB + b) * 16 + r16;
         if (m >= M) continue;
         if (EPI == EPI_SWIGLU) {
-            // weight rows come in blocks of 16 gate rows then 16 up rows: within a 32-row MFMA block,
-            // rows 0..15 (i/4 in {0,1}) are gate and rows 16..31 (i/4 in {2,3}) the matching up rows
             bf16* C = (bf16*)Cv;
 #pragma unroll
-            for (int a = 0; a < TN; ++a) {
-                const int fused_n = n0 + wn * 32 * TN + a * 32;            // start of a gate/up pair
+            for (int a = 0; a + 1 < TNB; a += 2) {
+                const int n = (n0 + (wn * TNB + a) * 16) / 2 + g4 * 4;     // blocks a, a + 1 = gate, up
+                if (n + 3 < N / 2 && (ldc & 3) == 0) {
+                    bf16x4 v;
 #pragma unroll
-                for (int q = 0; q < 2; ++q) {
-                    const int n = fused_n / 2 + 8 * q + 4 * g2;
-                    if (n + 3 < N / 2 && (ldc & 3) == 0) {
-                        bf16x4 v;
+                    for (int i = 0; i < 4; ++i) v[i] = (__bf16)silu_mul(acc[a][b][i], acc[a + 1][b][i]);
+                    *(bf16x4*)((__bf16*)C + (size_t)m * ldc + n) = v;
+                } else {
 #pragma unroll
-                        for (int r = 0; r < 4; ++r)
-                            v[r] = (__bf16)silu_mul(acc[a][b][4 * q + r], acc[a][b][4 * q + r + 8]);
-                        *(bf16x4*)((__bf16*)C + (size_t)m * ldc + n) = v;
-                    } else {
-#pragma unroll
-                        for (int r = 0; r < 4; ++r)
-                            if (n + r < N / 2)
-                                C[(size_t)m * ldc + n + r] = hb_from_float<bf16>(
-                                    silu_mul(acc[a][b][4 * q + r], acc[a][b][4 * q + r + 8]));
-                    }
+                    for (int i = 0; i < 4; ++i)
+                        if (n + i < N / 2)
+                            C[(size_t)m * ldc + n + i] =
+                                hb_from_float<bf16>(silu_mul(acc[a][b][i], acc[a + 1][b][i]));
                 }
             }
         } else {
             float* C = (float*)Cv;
 #pragma unroll
-            for (int a = 0; a < TN; ++a)
+            for (int a = 0; a < TNB; ++a) {
+                const int n = n0 + (wn * TNB + a) * 16 + g4 * 4;
+                float* dst = C + (size_t)m * ldc + n;
+                if (n + 3 < N && (ldc & 3) == 0) {
+                    f32x4 v = acc[a][b];
+                    if (EPI == EPI_ADD) v += *(const f32x4*)dst;
+                    *(f32x4*)dst = v;
+                } else {
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const int n = n0 + wn * 32 * TN + a * 32 + 8 * q + 4 * g2;
-                    float* dst = C + (size_t)m * ldc + n;
-                    if (n + 3 < N && (ldc & 3) == 0) {
-                        f32x4 v = {acc[a][b][4 * q], acc[a][b][4 * q + 1], acc[a][b][4 * q + 2],
-                                   acc[a][b][4 * q + 3]};
-                        if (EPI == EPI_ADD) {
-                            const f32x4 old = *(const f32x4*)dst;
-                            v += old;
+                    for (int i = 0; i < 4; ++i)
+                        if (n + i < N) {
+                            if (EPI == EPI_ADD)
+                                dst[i] += acc[a][b][i];
+                            else
+                                dst[i] = acc[a][b][i];
                         }
-                        *(f32x4*)dst = v;
-                    } else {
-#pragma unroll
-                        for (int r = 0; r < 4; ++r)
-                            if (n + r < N) {
-                                if (EPI == EPI_ADD)
-                                    dst[r] += acc[a][b][4 * q + r];
-                                else
-                                    dst[r] = acc[a][b][4 * q + r];
-                            }
-                    }
                 }
+            }
         }
     }
 }
 
-template <int TN, int TM>
-static int launch_tiled(const void* X, const void* W, void* C, int M, int N, int K, int ldc, int epi,
-                        int packed, hipStream_t stream) {
-    constexpr int BN = 64 * TN, BM = 64 * TM;
+template <int TNB, int TMB, int WNW, int WMW, int STAGES, int KS>
+static int launch_dma(const void* X, const void* W, void* C, int M, int N, int K, int ldc, int epi, int packed,
+                      hipStream_t stream) {
+    constexpr int BN = 16 * TNB * WNW, BM = 16 * TMB * WMW;
     const int m_tiles = (M + BM - 1) / BM, n_tiles = (N + BN - 1) / BN;
     const long total = (long)m_tiles * n_tiles;
     HB_REQUIRE(total < (1l << 30), "gemm_mfma: too many tiles");
     const int blocks = (int)((total + 7) / 8 * 8);
-    const size_t lds = (size_t)2 * (BN + BM) * LDT * sizeof(bf16);
+    HB_REQUIRE(K % (32 * KS) == 0, "gemm_mfma: K=%d is no multiple of %d", K, 32 * KS);
+    const size_t lds = (size_t)STAGES * KS * (BN + BM) / 16 * 1024;
     const bf16* x = (const bf16*)X;
     const bf16* w = (const bf16*)W;
-#define TILED_GO(EPIV, PK)                                                                          \
+#define DMA_GO(EPIV, PK)                                                                            \
     do {                                                                                            \
-        auto kern = gemm_tiled_kernel<EPIV, PK, TN, TM>;                                            \
+        auto kern = gemm_dma_kernel<EPIV, PK, TNB, TMB, WNW, WMW, STAGES, KS>;                          \
         if (lds > 64 * 1024) {                                                                      \
             static bool raised = false;                                                             \
             if (!raised) {                                                                          \
@@ -505,19 +501,19 @@ static int launch_tiled(const void* X, const void* W, void* C, int M, int N, int
                 raised = true;                                                                      \
             }                                                                                       \
         }                                                                                           \
-        kern<<<blocks, 256, lds, stream>>>(x, w, C, M, N, K, ldc, m_tiles, n_tiles);                \
+        kern<<<blocks, 64 * WNW * WMW, lds, stream>>>(x, w, C, M, N, K, ldc, m_tiles, n_tiles);     \
     } while (0)
     if (packed) {
-        if (epi == EPI_STORE) TILED_GO(EPI_STORE, true);
-        else if (epi == EPI_ADD) TILED_GO(EPI_ADD, true);
-        else TILED_GO(EPI_SWIGLU, true);
+        if (epi == EPI_STORE) DMA_GO(EPI_STORE, true);
+        else if (epi == EPI_ADD) DMA_GO(EPI_ADD, true);
+        else DMA_GO(EPI_SWIGLU, true);
     } else {
-        if (epi == EPI_STORE) TILED_GO(EPI_STORE, false);
-        else if (epi == EPI_ADD) TILED_GO(EPI_ADD, false);
-        else TILED_GO(EPI_SWIGLU, false);
+        if (epi == EPI_STORE) DMA_GO(EPI_STORE, false);
+        else if (epi == EPI_ADD) DMA_GO(EPI_ADD, false);
+        else DMA_GO(EPI_SWIGLU, false);
     }
-#undef TILED_GO
-    HB_CHECK_LAUNCH("gemm_tiled");
+#undef DMA_GO
+    HB_CHECK_LAUNCH("gemm_dma");
     return 0;
 }
 
@@ -543,17 +539,20 @@ extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N,
         HB_CHECK_LAUNCH("gemm_skinny");
         return 0;
     }
-    HB_REQUIRE(K % BK == 0, "gemm_mfma: K=%d is no multiple of %d (needed for M > 64)", K, BK);
-    // tile_hint: 0 = choose; otherwise 10 * TN + TM (for measurements)
+    // tile_hint: 0 = choose (otherwise a variant by number, for measurements and tests).
+    // 256 x 256 tiles do the most arithmetic per byte moved, but one fits a CU at a time: they pay
+    // when there are enough of them for most of the 256 CUs; otherwise 128 x 128, two to a CU.
     int tile = tile_hint;
-    // 256 x 256 tiles read LDS and L1 half as often per MFMA, but only pay with enough of them
-    // to keep every CU busy (one fits a CU at a time)
-    if (tile == 0) tile = ((long)((M + 255) / 256) * ((N + 255) / 256) >= 512) ? 44 : 22;
+    if (tile == 0) {
+        const long big = (long)((M + 255) / 256) * ((N + 255) / 256);
+        tile = K % 64 ? 123 : (big >= 192 ? 185 : 122);
+    }
     switch (tile) {
-        case 22: return launch_tiled<2, 2>(X, W, C, M, N, K, ldc, epi, packed, stream);
-        case 24: return launch_tiled<2, 4>(X, W, C, M, N, K, ldc, epi, packed, stream);
-        case 42: return launch_tiled<4, 2>(X, W, C, M, N, K, ldc, epi, packed, stream);
-        case 44: return launch_tiled<4, 4>(X, W, C, M, N, K, ldc, epi, packed, stream);
+        case 184: return launch_dma<8, 4, 2, 4, 4, 1>(X, W, C, M, N, K, ldc, epi, packed, stream);   // 256 x 256, 4 stages of 32 k
+        case 185: return launch_dma<8, 4, 2, 4, 2, 2>(X, W, C, M, N, K, ldc, epi, packed, stream);   // 256 x 256, 2 stages of 64 k
+        case 182: return launch_dma<4, 4, 2, 4, 3, 2>(X, W, C, M, N, K, ldc, epi, packed, stream);   // 128 x 256, 3 stages of 64 k
+        case 122: return launch_dma<4, 4, 2, 2, 2, 2>(X, W, C, M, N, K, ldc, epi, packed, stream);   // 128 x 128, 2 stages of 64 k
+        case 123: return launch_dma<4, 4, 2, 2, 4, 1>(X, W, C, M, N, K, ldc, epi, packed, stream);   // 128 x 128, 4 stages of 32 k
         default: HB_REQUIRE(false, "gemm_mfma: unknown tile %d", tile);
     }
     return 0;

@@ -20,13 +20,13 @@ SKINNY_MAX_M = 64
 
 
 def gemm_supported(a, w, out=None, swiglu=False):
-    """True if hb_gemm_mfma takes this product (bfloat16 operands, K in steps of 32, or of 64 for
-    more than 64 rows; the SwiGLU epilogue pairs blocks of 16 rows)."""
+    """True if hb_gemm_mfma takes this product (bfloat16 operands, K in steps of 32; the SwiGLU
+    epilogue pairs blocks of 16 rows)."""
     if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         return False
     M, K = a.shape
     N = w.shape[0]
-    if K % 32 or (M > SKINNY_MAX_M and K % 64):
+    if K % 32:
         return False
     if swiglu:
         return N % 32 == 0
@@ -73,7 +73,7 @@ def gemm(a, w, out, accumulate=False, packed=False, norm=None, tile=0):
     _check(w, "w", torch.bfloat16, (None, K))
     N = w.shape[0]
     _check(out, "out", torch.float32, (M, N))
-    if K % 32 or (M > SKINNY_MAX_M and K % 64) or (norm is not None and accumulate):
+    if K % 32 or (norm is not None and accumulate):
         raise BackendError(f"gemm_mfma refuses M={M}, N={N}, K={K}")
     lib.call("gemm_mfma", "hb_gemm_mfma", a.data_ptr(), w.data_ptr(), out.data_ptr(), M, N, K, N,
              EPI_ADD if accumulate else EPI_STORE, 1 if packed else 0, norm_ptr, eps, int(tile), _stream())
@@ -95,7 +95,7 @@ def gemm_swiglu(a, w_interleaved, out, packed=False, norm=None, tile=0):
     _check(w_interleaved, "w", torch.bfloat16, (None, K))
     N = w_interleaved.shape[0]
     _check(out, "out", torch.bfloat16, (M, N // 2))
-    if K % 32 or (M > SKINNY_MAX_M and K % 64) or N % 32:
+    if K % 32 or N % 32:
         raise BackendError(f"gemm_mfma (SwiGLU) refuses M={M}, N={N}, K={K}")
     lib.call("gemm_mfma", "hb_gemm_mfma", a.data_ptr(), w_interleaved.data_ptr(), out.data_ptr(), M, N, K,
              N // 2, EPI_SWIGLU, 1 if packed else 0, norm_ptr, eps, int(tile), _stream())

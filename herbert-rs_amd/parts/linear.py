@@ -16,7 +16,7 @@ class Linear:
         self.out_features, self.in_features = weight.shape
         self.packed = False
         if pack and weight.dtype == torch.bfloat16 and weight.is_cuda \
-                and self.out_features % 16 == 0 and self.in_features % 64 == 0:
+                and self.out_features % 16 == 0 and self.in_features % 32 == 0:
             from ..kernels import mfma
             weight = mfma.pack_weight(weight)
             self.packed = True

@@ -38,7 +38,7 @@ class SwiGLU(Part):
         # product's epilogue applies silu(gate) * up and the float32 [T, 2I] never exists
         from ..kernels import mfma
         self.fused_epilogue = (rt.dtype == torch.bfloat16 and self.intermediate_size % 16 == 0
-                               and self.hidden_size % 64 == 0 and mfma.gemm_supported(
+                               and self.hidden_size % 32 == 0 and mfma.gemm_supported(
                                    gate[:1], gate, swiglu=True))
         if self.fused_epilogue:
             self.gate_up = Linear(mfma.interleave_gate_up(gate, up))

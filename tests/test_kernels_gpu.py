@@ -121,7 +121,6 @@ def test_gemm_mfma_refuses_what_it_cannot_do():
     a = rand(4, 40, dtype=torch.bfloat16)
     w = rand(8, 40, dtype=torch.bfloat16)
     assert not mfma.gemm_supported(a, w)
-    assert not mfma.gemm_supported(rand(100, 96, dtype=torch.bfloat16), rand(8, 96, dtype=torch.bfloat16))
     assert not mfma.gemm_supported(a.float(), w)
 
 
@@ -300,3 +299,32 @@ def test_gemm_mfma_with_fused_norm(M, N, K, packed):
         gg, uu = (xg @ gate.double().T) * inv, (xg @ up.double().T) * inv
         wanted = (gg / (1 + torch.exp(-gg)) * uu).float()
         assert float((act.float() - wanted).abs().max()) <= 2 ** -7 * float(wanted.abs().max()) + 1e-5
+
+
+@pytest.mark.parametrize("tile", [0, 184, 185, 182, 122, 123])
+@pytest.mark.parametrize("M,N,K,packed", [(65, 128, 64, True), (200, 336, 192, True), (300, 530, 96, False),
+                                          (513, 1040, 256, True)])
+def test_gemm_mfma_tile_variants(tile, M, N, K, packed):
+    from herbert_rs_amd.kernels import mfma
+    if K % 64 and tile not in (0, 184, 123):
+        pytest.skip("this tile takes K in steps of 64")
+    a = rand(M, K, seed=7, dtype=torch.bfloat16)
+    w = rand(N, K, seed=8, dtype=torch.bfloat16)
+    want = (a.double() @ w.double().T).float()
+    wp = mfma.pack_weight(w) if packed else w
+    c = torch.full((M, N), 7.0, device=dev())
+    mfma.gemm(a, wp, c, packed=packed, tile=tile)
+    tol = 2e-6 * K ** 0.5 * float(want.abs().max()) + 1e-4
+    assert float((c - want).abs().max()) <= tol
+    base = rand(M, N, seed=9)
+    c2 = base.clone()
+    mfma.gemm(a, wp, c2, accumulate=True, packed=packed, tile=tile)
+    assert float((c2 - (base + want)).abs().max()) <= tol
+    if N % 32 == 0:
+        gate, up = w[:N // 2].contiguous(), w[N // 2:].contiguous()
+        wi = mfma.interleave_gate_up(gate, up)
+        out = torch.empty(M, N // 2, dtype=torch.bfloat16, device=dev())
+        mfma.gemm_swiglu(a, mfma.pack_weight(wi) if packed else wi, out, packed=packed, tile=tile)
+        g, u = a.double() @ gate.double().T, a.double() @ up.double().T
+        wanted = (g / (1 + torch.exp(-g)) * u).float()
+        assert float((out.float() - wanted).abs().max()) <= 2 ** -7 * float(wanted.abs().max()) + 1e-4
