@@ -56,13 +56,15 @@ def _norm_args(a, norm, K):
 
 
 NORM_FUSE_MAX_M = 16
+NORM_FUSE_MIN_N = 16384     # measured: for narrower products a norm kernel of its own is as fast or faster
 
 
 def norm_fusable(a, w):
     """True if RMSNorm(a) @ w^T should run as one kernel: at most 16 rows of the float32 residual
-    stream (every workgroup reads all of them; with more rows that costs more than a norm kernel)."""
+    stream (every workgroup reads all of them; with more rows that costs more than a norm kernel)
+    and many weight rows (each workgroup then has enough of them to pay for reading the rows)."""
     return (a.dtype == torch.float32 and w.dtype == torch.bfloat16 and a.shape[0] <= NORM_FUSE_MAX_M
-            and a.shape[1] % 32 == 0)
+            and a.shape[1] % 32 == 0 and w.shape[0] >= NORM_FUSE_MIN_N)
 
 
 def gemm(a, w, out, accumulate=False, packed=False, norm=None, tile=0):
