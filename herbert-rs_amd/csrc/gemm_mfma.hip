@@ -58,7 +58,8 @@ struct SkinnyOperands {
 template <int MB, int NB, int WAVES, int EPI, bool PACKED, bool NORM>
 __global__ void __launch_bounds__(WAVES * 64)
 gemm_skinny_kernel(const void* __restrict__ Xv, const bf16* __restrict__ W, void* __restrict__ Cv, int M,
-                   int N, int K, int ldc, const float* __restrict__ norm_w, float eps) {
+                   int N, int K, int ldc, const float* __restrict__ norm_w, float eps,
+                   float* __restrict__ partial) {
     constexpr int U = NORM ? 2 : ((NB + MB <= 4) ? 4 : 2);
     const bf16* X = (const bf16*)Xv;
     const float* XF = (const float*)Xv;
@@ -68,7 +69,12 @@ gemm_skinny_kernel(const void* __restrict__ Xv, const bf16* __restrict__ W, void
     const int r16 = lane & 15;
     const int g4 = lane >> 4;
     const int n0 = blockIdx.x * (NB * 16);
-    const int nsteps = K / 32;
+    const int k32 = K / 32;                       // k-steps of the whole product
+    // gridDim.y > 1: this workgroup sums one slice of K only and leaves its sums in `partial`
+    // [slice][M][N]; a second kernel adds the slices in order (see gemm_slices_kernel)
+    const int per_slice = (k32 + gridDim.y - 1) / gridDim.y;
+    const int step0 = blockIdx.y * per_slice;
+    const int nsteps = k32 - step0 < per_slice ? (k32 - step0 > 0 ? k32 - step0 : 0) : per_slice;
 
     f32x4 acc[NB][MB];
 #pragma unroll
@@ -85,7 +91,7 @@ gemm_skinny_kernel(const void* __restrict__ Xv, const bf16* __restrict__ W, void
         if (PACKED) {
             int nb = n0 / 16 + a;
             if (nb * 16 >= N) nb = (N - 1) / 16;
-            wrow[a] = W + ((size_t)nb * nsteps * 64 + lane) * 8;
+            wrow[a] = W + ((size_t)nb * k32 * 64 + lane) * 8;
         } else {
             int n = n0 + a * 16 + r16;
             if (n >= N) n = N - 1;            // rows past the end repeat the last one; never stored
@@ -111,7 +117,7 @@ gemm_skinny_kernel(const void* __restrict__ Xv, const bf16* __restrict__ W, void
 
 #define SKINNY_LOAD(dst, group)                                                  \
     _Pragma("unroll") for (int u = 0; u < U; ++u) {                              \
-        const int st = wave + ((group) * U + u) * WAVES;                         \
+        const int st = step0 + wave + ((group) * U + u) * WAVES;                 \
         const int k = st * 32;                                                   \
         _Pragma("unroll") for (int a = 0; a < NB; ++a)                           \
             dst[u].w[a] = *(const bf16x8*)(wrow[a] + (size_t)st * WSTEP);        \
@@ -150,7 +156,7 @@ gemm_skinny_kernel(const void* __restrict__ Xv, const bf16* __restrict__ W, void
         }
     }
     for (int i = groups * U; i < mine; ++i) {       // what is left over of this wave's steps
-        const int st = wave + i * WAVES;
+        const int st = step0 + wave + i * WAVES;
         const int k = st * 32;
         bf16x8 wv[NB], xv[MB];
 #pragma unroll
@@ -228,6 +234,22 @@ gemm_skinny_kernel(const void* __restrict__ Xv, const bf16* __restrict__ W, void
     }
 
     // lane: m = b * 16 + r16, n = n0 + a * 16 + g4 * 4 + i
+    if (gridDim.y > 1) {
+        float* P = partial + (size_t)blockIdx.y * M * N;
+#pragma unroll
+        for (int a = 0; a < NB; ++a)
+#pragma unroll
+            for (int b = 0; b < MB; ++b) {
+                const int m = b * 16 + r16;
+                if (m >= M) continue;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int n = n0 + a * 16 + g4 * 4 + i;
+                    if (n < N) P[(size_t)m * N + n] = acc[a][b][i];
+                }
+            }
+        return;
+    }
     if (EPI == EPI_SWIGLU) {
         bf16* C = (bf16*)Cv;
         const int out_n0 = n0 / 2;
@@ -267,16 +289,28 @@ gemm_skinny_kernel(const void* __restrict__ Xv, const bf16* __restrict__ W, void
     }
 }
 
+// C[m, n] (+)= sum over the slices, in their order, of partial[slice][m][n].
+__global__ void gemm_slices_kernel(const float* __restrict__ partial, float* __restrict__ C, int M, int N,
+                                   int ldc, int slices, int add) {
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (size_t)M * N) return;
+    const int m = (int)(idx / N), n = (int)(idx % N);
+    float sum = add ? C[(size_t)m * ldc + n] : 0.f;
+    for (int s = 0; s < slices; ++s) sum += partial[(size_t)s * M * N + idx];
+    C[(size_t)m * ldc + n] = sum;
+}
+
 template <int MB, int NB, int WAVES>
 static void launch_skinny(const void* X, const void* W, void* C, int M, int N, int K, int ldc, int epi,
-                          int packed, const float* norm_w, float eps, hipStream_t stream) {
-    const int blocks = (N + NB * 16 - 1) / (NB * 16);
+                          int packed, const float* norm_w, float eps, hipStream_t stream,
+                          float* partial = nullptr, int slices = 1) {
+    const dim3 blocks((N + NB * 16 - 1) / (NB * 16), slices);
     size_t lds = (size_t)(WAVES / 2) * NB * MB * 4 * 64 * sizeof(float);
     if (lds < (size_t)WAVES * MB * 16 * sizeof(float)) lds = (size_t)WAVES * MB * 16 * sizeof(float);
     const bf16* w = (const bf16*)W;
 #define SKINNY_GO(EPIV, PK, NM)                                                                        \
     gemm_skinny_kernel<MB, NB, WAVES, EPIV, PK, NM><<<blocks, WAVES * 64, lds, stream>>>(X, w, C, M, N, K, \
-                                                                                          ldc, norm_w, eps)
+                                                                                          ldc, norm_w, eps, partial)
     if (norm_w) {       // the normed input never meets the add epilogue
         if (packed) {
             if (epi == EPI_STORE) SKINNY_GO(EPI_STORE, true, true);
@@ -295,11 +329,38 @@ static void launch_skinny(const void* X, const void* W, void* C, int M, int N, i
         else SKINNY_GO(EPI_SWIGLU, false, false);
     }
 #undef SKINNY_GO
+    if (slices > 1) {
+        const size_t total = (size_t)M * N;
+        gemm_slices_kernel<<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(partial, (float*)C, M, N, ldc, slices,
+                                                                              epi == EPI_ADD);
+    }
 }
 
 template <int MB>
 static void pick_skinny(const void* X, const void* W, void* C, int M, int N, int K, int ldc, int epi,
-                        int packed, const float* norm_w, float eps, hipStream_t stream) {
+                        int packed, const float* norm_w, float eps, hipStream_t stream, float* workspace,
+                        size_t workspace_floats) {
+    if (MB >= 2 && !norm_w) {
+        // More than 16 rows: every workgroup re-reads its slice of the activations from L2, so a
+        // workgroup takes 64 weight rows (the activations are then read as often as the weights),
+        // and K is cut into slices over further workgroups until the 256 CUs have work; the slices'
+        // sums are added in order by a second kernel, so the result does not depend on timing.
+        const int groups = (N + 63) / 64;
+        int slices = 1;
+        if (epi != EPI_SWIGLU) {
+            slices = 256 / groups;
+            const int most = K / 32 / 8;                 // at least one k-step a wave
+            if (slices > most) slices = most;
+            if (slices > 8) slices = 8;
+            if (slices < 1) slices = 1;
+            if ((size_t)slices * M * N > workspace_floats) slices = 1;
+        }
+        if (slices == 1 && N >= 16384)      // wide enough without slices: four waves a workgroup, more of them a CU
+            launch_skinny<MB, 4, 4>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream);
+        else
+            launch_skinny<MB, 4, 8>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream, workspace, slices);
+        return;
+    }
     // Few weight rows: one block of 16 rows a workgroup and eight waves splitting K, so that the
     // 256 CUs all have work. Many rows: more rows a workgroup, so that the activations are
     // re-read from L2 less often.
@@ -520,10 +581,12 @@ static int launch_dma(const void* X, const void* W, void* C, int M, int N, int K
 // C (+)= X @ W^T. X [M, K] bf16, W [N, K] bf16. epi 0: C f32 [M, N] stored; 1: added to;
 // 2: W's rows are gate/up interleaved in blocks of 16 and C is bf16 [M, N / 2] = silu(gate) * up.
 // packed != 0: W is stored as [N / 16][K / 32][64 lanes][8]: lane = 16 * (k / 8 % 4) + n % 16.
+// workspace: float scratch for K cut into slices (17 to 64 rows); without it K is not cut.
 // norm_w != null: X is the float32 residual stream [M, K] and the product is RMSNorm(X; norm_w, eps) W^T
 // (M <= 64 only, never with the add epilogue).
 extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N, int K, int ldc, int epi,
-                            int packed, const float* norm_w, float eps, int tile_hint, hipStream_t stream) {
+                            int packed, const float* norm_w, float eps, int tile_hint, float* workspace,
+                            size_t workspace_floats, hipStream_t stream) {
     HB_REQUIRE(!norm_w || (M <= 64 && epi != EPI_ADD), "gemm_mfma: the fused norm takes M <= 64 and no add");
     HB_REQUIRE(!packed || N % 16 == 0, "gemm_mfma: packed weights need N %% 16 == 0");
     HB_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_mfma: empty problem (M=%d, N=%d, K=%d)", M, N, K);
@@ -532,10 +595,10 @@ extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N,
     HB_REQUIRE(epi != EPI_SWIGLU || N % 32 == 0, "gemm_mfma: the SwiGLU epilogue needs N %% 32 == 0");
     HB_REQUIRE(ldc >= (epi == EPI_SWIGLU ? N / 2 : N), "gemm_mfma: output row stride %d too small", ldc);
     if (M <= 64) {
-        if (M <= 16) pick_skinny<1>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream);
-        else if (M <= 32) pick_skinny<2>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream);
-        else if (M <= 48) pick_skinny<3>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream);
-        else pick_skinny<4>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream);
+        if (M <= 16) pick_skinny<1>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream, workspace, workspace_floats);
+        else if (M <= 32) pick_skinny<2>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream, workspace, workspace_floats);
+        else if (M <= 48) pick_skinny<3>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream, workspace, workspace_floats);
+        else pick_skinny<4>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream, workspace, workspace_floats);
         HB_CHECK_LAUNCH("gemm_skinny");
         return 0;
     }

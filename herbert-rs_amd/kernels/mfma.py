@@ -12,11 +12,27 @@ _P = ctypes.c_void_p
 _I = ctypes.c_int
 _F = ctypes.c_float
 lib.register_signatures("gemm_mfma", {
-    "hb_gemm_mfma": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _F, _I, _P],
+    "hb_gemm_mfma": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _F, _I, _P, ctypes.c_size_t, _P],
 })
 
 EPI_STORE, EPI_ADD, EPI_SWIGLU = 0, 1, 2
 SKINNY_MAX_M = 64
+_workspaces = {}
+
+
+def _slice_workspace(device, M, N, K):
+    """(pointer, floats) of the scratch for products whose K is cut into slices (17 to 64 rows).
+    A buffer that was handed out is kept for good: a captured graph may hold its address."""
+    if M <= 16 or M > SKINNY_MAX_M:
+        return None, 0
+    slices = min(8, 256 // max(1, (N + 63) // 64), K // 256)
+    if slices < 2:
+        return None, 0
+    need = slices * M * N
+    kept = _workspaces.setdefault(str(device), [])
+    if not kept or kept[-1].numel() < need:
+        kept.append(torch.empty(need, dtype=torch.float32, device=device))
+    return kept[-1].data_ptr(), kept[-1].numel()
 
 
 def gemm_supported(a, w, out=None, swiglu=False):
@@ -77,8 +93,10 @@ def gemm(a, w, out, accumulate=False, packed=False, norm=None, tile=0):
     _check(out, "out", torch.float32, (M, N))
     if K % 32 or (norm is not None and accumulate):
         raise BackendError(f"gemm_mfma refuses M={M}, N={N}, K={K}")
+    ws_ptr, ws_floats = _slice_workspace(a.device, M, N, K)
     lib.call("gemm_mfma", "hb_gemm_mfma", a.data_ptr(), w.data_ptr(), out.data_ptr(), M, N, K, N,
-             EPI_ADD if accumulate else EPI_STORE, 1 if packed else 0, norm_ptr, eps, int(tile), _stream())
+             EPI_ADD if accumulate else EPI_STORE, 1 if packed else 0, norm_ptr, eps, int(tile), ws_ptr,
+             ws_floats, _stream())
 
 
 def interleave_gate_up(gate, up):
@@ -100,7 +118,7 @@ def gemm_swiglu(a, w_interleaved, out, packed=False, norm=None, tile=0):
     if K % 32 or N % 32:
         raise BackendError(f"gemm_mfma (SwiGLU) refuses M={M}, N={N}, K={K}")
     lib.call("gemm_mfma", "hb_gemm_mfma", a.data_ptr(), w_interleaved.data_ptr(), out.data_ptr(), M, N, K,
-             N // 2, EPI_SWIGLU, 1 if packed else 0, norm_ptr, eps, int(tile), _stream())
+             N // 2, EPI_SWIGLU, 1 if packed else 0, norm_ptr, eps, int(tile), None, 0, _stream())
 
 
 lib.register_signatures("attention_mfma", {

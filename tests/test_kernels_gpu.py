@@ -328,3 +328,26 @@ def test_gemm_mfma_tile_variants(tile, M, N, K, packed):
         g, u = a.double() @ gate.double().T, a.double() @ up.double().T
         wanted = (g / (1 + torch.exp(-g)) * u).float()
         assert float((out.float() - wanted).abs().max()) <= 2 ** -7 * float(wanted.abs().max()) + 1e-4
+
+
+@pytest.mark.parametrize("M,N,K", [(17, 4096, 4096), (40, 1024, 512), (64, 4096, 12288), (64, 6144, 4096),
+                                   (33, 272, 96)])
+def test_gemm_mfma_with_k_slices(M, N, K):
+    """17 to 64 rows: K is cut into slices over several workgroups whose sums a second kernel adds."""
+    from herbert_rs_amd.kernels import mfma
+    a = rand(M, K, seed=40, dtype=torch.bfloat16)
+    w = rand(N, K, seed=41, dtype=torch.bfloat16, scale=0.05)
+    want = (a.double() @ w.double().T).float()
+    tol = 2e-6 * K ** 0.5 * float(want.abs().max()) + 1e-4
+    for packed in (False, True):
+        wp = mfma.pack_weight(w) if packed else w
+        c = torch.full((M, N), 3.0, device=dev())
+        mfma.gemm(a, wp, c, packed=packed)
+        assert float((c - want).abs().max()) <= tol
+        base = rand(M, N, seed=42)
+        c2 = base.clone()
+        mfma.gemm(a, wp, c2, accumulate=True, packed=packed)
+        assert float((c2 - (base + want)).abs().max()) <= tol
+        c3 = base.clone()
+        mfma.gemm(a, wp, c3, accumulate=True, packed=packed)
+        assert torch.equal(c2, c3)                      # the same bits on every run
