@@ -20,11 +20,11 @@ HBM_GBS = 8000.0
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
 
 
-def load_shape():
-    """Layer sizes of the benchmark configuration, parsed from BASELINE.json's configs[2]."""
+def load_shape(index=2):
+    """Layer sizes of a benchmark configuration, parsed from BASELINE.json's configs[index]."""
     import re
     with open(os.path.join(ROOT, "BASELINE.json")) as f:
-        text = json.load(f)["configs"][2]
+        text = json.load(f)["configs"][index]
 
     def num(pattern):
         return int(re.search(pattern, text).group(1))
@@ -32,8 +32,63 @@ def load_shape():
         num_hidden_layers=num(r"(\d+) layers"), hidden_size=num(r"hidden (\d+)"),
         num_attention_heads=num(r"(\d+) query heads"), num_key_value_heads=num(r"(\d+) KV heads"),
         head_dim=num(r"head_dim (\d+)"), intermediate_size=num(r"intermediate (\d+)"),
-        vocab_size=num(r"vocab (\d+)"), context=num(r"Context length (\d+)"),
-        rope_theta=1e6, rms_norm_eps=1e-6, tie_word_embeddings=False)
+        vocab_size=num(r"vocab (\d+)"),
+        context=num(r"Context length (\d+)") if "Context length" in text else 0,
+        rope_theta=1e6, rms_norm_eps=1e-6, tie_word_embeddings="tied embeddings" in text)
+
+
+def run_workload(args, index):
+    """The other two workloads of the benchmark description, through the generation loop:
+    configs[3] (1.7B shape: 16 prompts of 64..1024 tokens, 256 new tokens each) and configs[4]
+    (32B shape: 8 prompts of 2048 tokens, 512 new tokens each)."""
+    import torch
+    import herbert_rs_amd as hb
+    from herbert_rs_amd.sampling import SamplingParams
+    shape = load_shape(index)
+    shape.pop("context")
+    if args.layers:
+        shape["num_hidden_layers"] = args.layers
+    gen = torch.Generator().manual_seed(index)
+    if index == 3:
+        lengths = torch.randint(64, 1025, (16,), generator=gen).tolist()
+        new, name = 256, "Qwen3-1.7B shape"
+    else:
+        lengths, new, name = [2048] * 8, 512, "Qwen3-32B shape"
+    if args.steps != 32:
+        new = args.steps
+    raw = dict(shape, architectures=["Qwen3ForCausalLM"], model_type="qwen3",
+               max_position_embeddings=4096, eos_token_id=151645)
+    cfg = hb.Qwen3Config.from_dict(raw)
+    torch.cuda.set_device(0)
+    t0 = time.time()
+    room = sum((n + new + 127) // 64 * 64 for n in lengths)
+    engine = hb.Engine.from_config(cfg, seed=index, dtype=args.dtype, max_tokens=room, max_slots=len(lengths))
+    print(f"[bench] {name} built in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
+    prompts = [torch.randint(0, cfg.vocab_size, (n,), generator=gen).tolist() for n in lengths]
+    params = SamplingParams(temperature=0.0, max_tokens=new, ignore_eos=True, repeat_check=False)
+    engine.generate(prompts[:2], SamplingParams(temperature=0.0, max_tokens=3, ignore_eos=True,
+                                                repeat_check=False))              # compiles, warms
+    results = engine.generate(prompts, params, max_batch=len(prompts))
+    st = engine.last_generation_stats
+    assert all(len(r.tokens) == new for r in results)
+    decoded = st.generated_tokens - len(prompts)
+    print(json.dumps({
+        "metric": f"decode tok/s, {name}, batch {len(prompts)}, {new} new tokens each",
+        "value": round(decoded / st.decode_seconds, 2), "unit": "tokens/s", "n_gpus": 1,
+        "steps": st.decode_steps, "warmup": 0, "ms_per_step": round(st.decode_seconds / st.decode_steps * 1e3, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic: random weights N(0, 0.02), random token ids",
+        "config": {"model": name, "layers": cfg.num_hidden_layers, "hidden_size": cfg.hidden_size,
+                   "num_attention_heads": cfg.num_attention_heads,
+                   "num_key_value_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
+                   "intermediate_size": cfg.intermediate_size, "vocab_size": cfg.vocab_size,
+                   "tie_word_embeddings": cfg.tie_word_embeddings, "global_batch": len(prompts),
+                   "prompt_tokens": st.prompt_tokens, "new_tokens": new, "parallelism": "single GPU"},
+        "prefill": {"value": round(st.prompt_tokens / st.prefill_seconds, 1), "tokens": st.prompt_tokens,
+                    "ms": round(st.prefill_seconds * 1e3, 3)},
+    }))
+    return 0
 
 
 def main():
@@ -46,6 +101,8 @@ def main():
     ap.add_argument("--context", type=int, default=None)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
+    ap.add_argument("--workload", default="headline", choices=["headline", "qwen3-1.7b", "qwen3-32b"],
+                    help="headline: BASELINE.json configs[2]; the others: configs[3] and configs[4]")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run the 2,048-token prefill alone (for profiles); prints no JSON line")
     args = ap.parse_args()
@@ -53,6 +110,9 @@ def main():
         print(f"bench.py measures one GPU only: --gpus {args.gpus} is not supported (this library "
               "does no work on several GPUs)")
         return 2
+
+    if args.workload != "headline":
+        return run_workload(args, 3 if args.workload == "qwen3-1.7b" else 4)
 
     import torch
     import herbert_rs_amd as hb

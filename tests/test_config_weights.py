@@ -181,3 +181,38 @@ def test_bf16_conversion_bits():
     assert torch.equal(bf16_bits_to_f32(bits), x.to(torch.bfloat16).float())
     ties = torch.tensor([0x3F808000, 0x3F818000, 0x3F808001], dtype=torch.int64).to(torch.int32).view(torch.float32)
     assert f32_to_bf16_bits(ties).tolist() == [0x3F80, 0x3F82, 0x3F81]
+
+
+def test_names_are_normalised_and_fused_tensors_cut(model_root, tmp_path):
+    """The spellings the reference's loader accepts (bc/loader_common.rs:423-451, 475-566) and its
+    fused q/k/v and gate/up tensors (:1469-1528) give the same weights as the plain names."""
+    from herbert_rs_amd.weights.store import canonical_name
+    assert canonical_name("language_model.model.layers.0.mlp.up_proj.weight") == "model.layers.0.mlp.up_proj.weight"
+    assert canonical_name("language_model.lm_head.weight") == "lm_head.weight"
+    assert canonical_name("model.language_model.norm.weight") == "model.norm.weight"
+    assert canonical_name("layers.3.self_attn.out_proj.weight") == "model.layers.3.self_attn.o_proj.weight"
+    assert canonical_name("model.layers.1.self_attn.q_proj.base_layer.weight") == "model.layers.1.self_attn.q_proj.weight"
+    assert canonical_name("model.layers.1.feed_forward.w3.weight") == "model.layers.1.mlp.up_proj.weight"
+    assert canonical_name("model.layers.1.ffn_norm.weight") == "model.layers.1.post_attention_layernorm.weight"
+
+    src = make_folder(model_root, "B", "float32")
+    plain = load_file(os.path.join(src, "model.safetensors"))
+    other = {}
+    for name, t in plain.items():
+        if any(part in name for part in (".self_attn.q_proj.", ".self_attn.k_proj.", ".self_attn.v_proj.",
+                                         ".mlp.gate_proj.", ".mlp.up_proj.")):
+            continue
+        other[name.replace("model.", "model.language_model.", 1).replace("o_proj", "out_proj")] = t
+    for l in range(3):
+        p = f"model.layers.{l}."
+        other[f"model.language_model.layers.{l}.self_attn.qkv_proj.weight"] = torch.cat(
+            [plain[p + f"self_attn.{x}_proj.weight"] for x in "qkv"], 0)
+        other[f"model.language_model.layers.{l}.mlp.gate_up_proj.weight"] = torch.cat(
+            [plain[p + "mlp.gate_proj.weight"], plain[p + "mlp.up_proj.weight"]], 0)
+    save_file(other, str(tmp_path / "model.safetensors"))
+    got = read_tensors(str(tmp_path), needs_of(TINY_B))
+    assert set(got) == set(plain) and all(torch.equal(got[k], plain[k]) for k in plain)
+    other["model.language_model.layers.0.self_attn.qkv_proj.weight"] = torch.zeros(10, 96)
+    save_file(other, str(tmp_path / "model.safetensors"))
+    with pytest.raises(ModelLoadError, match=r"qkv_proj.weight: expected \[320, 96\], got \[10, 96\]"):
+        read_tensors(str(tmp_path), needs_of(TINY_B))
