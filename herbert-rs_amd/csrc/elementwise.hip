@@ -7,35 +7,36 @@ HB_MODULE_ERROR_SLOT()
 
 // ---------------------------------------------------------------- embedding
 // x[t, :] = float(table[ids[t], :]); the residual stream is float32.
-// PACKED: the table is stored in the MFMA kernels' order [V / 16][H / 32][64 lanes][8], element
-// (n, k) at ((n / 16 * (H / 32) + k / 32) * 64 + (k / 8 % 4) * 16 + n % 16) * 8 + k % 8.
+// PACKED: the table is stored in the MFMA kernels' order [H / 32][V / 16][64 lanes][8], element
+// (n, k) at ((k / 32 * (V / 16) + n / 16) * 64 + (k / 8 % 4) * 16 + n % 16) * 8 + k % 8.
 template <class TW, bool PACKED>
 __global__ void embed_kernel(const int* __restrict__ ids, const TW* __restrict__ table,
-                             float* __restrict__ x, int H) {
+                             float* __restrict__ x, int H, int V) {
     const int t = blockIdx.x;
     const int n = ids[t];
     float* out = x + (size_t)t * H;
     if (PACKED) {
-        const TW* blk = table + (size_t)(n / 16) * (H / 32) * 512 + (n % 16) * 8;
+        const TW* blk = table + (size_t)(n / 16) * 512 + (n % 16) * 8;
+        const size_t plane = (size_t)(V / 16) * 512;
         for (int k = threadIdx.x; k < H; k += blockDim.x)
-            out[k] = hb_to_float(blk[(size_t)(k / 32) * 512 + ((k / 8) % 4) * 128 + (k % 8)]);
+            out[k] = hb_to_float(blk[(size_t)(k / 32) * plane + ((k / 8) % 4) * 128 + (k % 8)]);
     } else {
         const TW* row = table + (size_t)n * H;
         for (int i = threadIdx.x; i < H; i += blockDim.x) out[i] = hb_to_float(row[i]);
     }
 }
 
-extern "C" int hb_embed(const int* ids, const void* table, int table_dtype, float* x, int T, int H,
+extern "C" int hb_embed(const int* ids, const void* table, int table_dtype, float* x, int T, int H, int V,
                         int packed, hipStream_t stream) {
     HB_REQUIRE(T > 0 && H > 0, "embed: empty input (T=%d, H=%d)", T, H);
-    HB_REQUIRE(!packed || (table_dtype == HB_BF16 && H % 32 == 0), "embed: a packed table is bfloat16 with "
-               "a width in steps of 32");
+    HB_REQUIRE(!packed || (table_dtype == HB_BF16 && H % 32 == 0 && V % 16 == 0),
+               "embed: a packed table is bfloat16 with a width in steps of 32 and rows in steps of 16");
     if (table_dtype == HB_F32)
-        embed_kernel<float, false><<<T, 256, 0, stream>>>(ids, (const float*)table, x, H);
+        embed_kernel<float, false><<<T, 256, 0, stream>>>(ids, (const float*)table, x, H, V);
     else if (table_dtype == HB_BF16 && packed)
-        embed_kernel<bf16, true><<<T, 256, 0, stream>>>(ids, (const bf16*)table, x, H);
+        embed_kernel<bf16, true><<<T, 256, 0, stream>>>(ids, (const bf16*)table, x, H, V);
     else if (table_dtype == HB_BF16)
-        embed_kernel<bf16, false><<<T, 256, 0, stream>>>(ids, (const bf16*)table, x, H);
+        embed_kernel<bf16, false><<<T, 256, 0, stream>>>(ids, (const bf16*)table, x, H, V);
     else
         HB_REQUIRE(false, "embed: unknown table dtype %d", table_dtype);
     HB_CHECK_LAUNCH("embed");

@@ -85,13 +85,14 @@ gemm_skinny_kernel(const void* __restrict__ Xv, const bf16* __restrict__ W, void
     // row-major weights: lane (r16, g4) reads 16 bytes of row n at k = 32 s + 8 g4.
     // packed weights: the 1 KB operand of (block of 16 rows, k-step) is contiguous, lane-major.
     const bf16* wrow[NB];
-    constexpr int WSTEP = PACKED ? 64 * 8 : 32;      // elements between this lane's chunks of two k-steps
+    // elements between this lane's chunks of two k-steps: packed weights are [K / 32][N / 16][64][8]
+    const size_t WSTEP = PACKED ? (size_t)(N / 16) * 512 : 32;
 #pragma unroll
     for (int a = 0; a < NB; ++a) {
         if (PACKED) {
             int nb = n0 / 16 + a;
             if (nb * 16 >= N) nb = (N - 1) / 16;
-            wrow[a] = W + ((size_t)nb * k32 * 64 + lane) * 8;
+            wrow[a] = W + ((size_t)nb * 64 + lane) * 8;
         } else {
             int n = n0 + a * 16 + r16;
             if (n >= N) n = N - 1;            // rows past the end repeat the last one; never stored
@@ -419,7 +420,7 @@ gemm_dma_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* __
         if (PACKED) {
             int nb = n0 / 16 + blk;
             if (nb * 16 >= N) nb = (N - 1) / 16;
-            wsrc[i] = W + ((size_t)nb * k32 * 64 + lane) * 8;
+            wsrc[i] = W + ((size_t)nb * 64 + lane) * 8;
         } else {
             int n = n0 + blk * 16 + r16;
             if (n >= N) n = N - 1;
@@ -432,7 +433,7 @@ gemm_dma_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* __
         if (m >= M) m = M - 1;
         xsrc[i] = X + (size_t)m * K + g4 * 8;
     }
-    constexpr int WSTEP = PACKED ? 512 : 32;
+    const size_t WSTEP = PACKED ? (size_t)(N / 16) * 512 : 32;
 
     auto issue = [&](int step, int stage) {
 #pragma unroll
@@ -580,7 +581,9 @@ static int launch_dma(const void* X, const void* W, void* C, int M, int N, int K
 
 // C (+)= X @ W^T. X [M, K] bf16, W [N, K] bf16. epi 0: C f32 [M, N] stored; 1: added to;
 // 2: W's rows are gate/up interleaved in blocks of 16 and C is bf16 [M, N / 2] = silu(gate) * up.
-// packed != 0: W is stored as [N / 16][K / 32][64 lanes][8]: lane = 16 * (k / 8 % 4) + n % 16.
+// packed != 0: W is stored as [K / 32][N / 16][64 lanes][8]: lane = 16 * (k / 8 % 4) + n % 16.
+// All blocks of one k-step lie together: workgroups that advance through K side by side read one
+// contiguous stretch of memory at a time, as a streaming copy would.
 // workspace: float scratch for K cut into slices (17 to 64 rows); without it K is not cut.
 // norm_w != null: X is the float32 residual stream [M, K] and the product is RMSNorm(X; norm_w, eps) W^T
 // (M <= 64 only, never with the add epilogue).

@@ -20,7 +20,7 @@ _SZ = ctypes.c_size_t
 # module -> function -> argument types (every function returns int, 0 = ok)
 SIGNATURES = {
     "elementwise": {
-        "hb_embed": [_P, _P, _I, _P, _I, _I, _I, _P],
+        "hb_embed": [_P, _P, _I, _P, _I, _I, _I, _I, _P],
         "hb_rmsnorm": [_P, _P, _P, _I, _P, _I, _I, _F, _P],
         "hb_qk_norm_rope_write": [_P, _I, _P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _P, _P, _P, _I,
                                   _I, _I, _I, _I, _F, _I, _P],

@@ -50,12 +50,14 @@ def gemm_supported(a, w, out=None, swiglu=False):
 
 
 def pack_weight(w):
-    """[N, K] -> the same values as [N / 16, K / 32, 64, 8]: the 1 KB MFMA operand of 16 rows and
-    32 k is contiguous, lane-major (lane = 16 * (k / 8 % 4) + n % 16)."""
+    """[N, K] -> the same values as [K / 32, N / 16, 64, 8]: the 1 KB MFMA operand of 16 rows and
+    32 k is contiguous, lane-major (lane = 16 * (k / 8 % 4) + n % 16), and the operands of one
+    k-step lie together, so that workgroups advancing through K side by side read memory as a
+    streaming copy does."""
     N, K = w.shape
     if N % 16 or K % 32:
         raise BackendError("packed weights need N in steps of 16 and K in steps of 32")
-    return w.view(N // 16, 16, K // 32, 4, 8).permute(0, 2, 3, 1, 4).contiguous().view(N, K)
+    return w.view(N // 16, 16, K // 32, 4, 8).permute(2, 0, 3, 1, 4).contiguous().view(N, K)
 
 
 def _norm_args(a, norm, K):

@@ -43,14 +43,14 @@ def _ptr(t):
 
 def embed(ids, table, out, packed=False):
     """out[t, :] = table[ids[t], :] as float32. ids int32 [T], table [V, H], out f32 [T, H].
-    packed: the table is stored in the MFMA kernels' order ([V / 16, H / 32, 64, 8])."""
+    packed: the table is stored in the MFMA kernels' order ([H / 32, V / 16, 64, 8])."""
     T = ids.shape[0]
     _check(ids, "ids", torch.int32, (T,))
     _check(table, "table", None, (None, None))
     H = table.shape[1]
     _check(out, "out", torch.float32, (T, H))
     lib.call("elementwise", "hb_embed", ids.data_ptr(), table.data_ptr(), dtype_code(table),
-             out.data_ptr(), T, H, 1 if packed else 0, _stream())
+             out.data_ptr(), T, H, table.shape[0], 1 if packed else 0, _stream())
 
 
 def rmsnorm(x, weight, out, eps, rows=None):

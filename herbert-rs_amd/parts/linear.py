@@ -2,7 +2,8 @@
 
 In the float32 mode the plain kernel does all products. In the bfloat16 mode the MFMA kernels
 do them where they take the shape, and then the matrix is kept in their packed order (the 1 KB
-operand of 16 rows and 32 k contiguous), which streams from HBM in whole contiguous blocks;
+operand of 16 rows and 32 k contiguous, all operands of a k-step together), which streams from
+HBM as a copy does;
 the plain kernel (same storage types, float32 arithmetic) does the rest from row-major weights.
 """
 import torch
