@@ -312,13 +312,15 @@ static void launch_skinny(const void* X, const void* W, void* C, int M, int N, i
 #define SKINNY_GO(EPIV, PK, NM)                                                                        \
     gemm_skinny_kernel<MB, NB, WAVES, EPIV, PK, NM><<<blocks, WAVES * 64, lds, stream>>>(X, w, C, M, N, K, \
                                                                                           ldc, norm_w, eps, partial)
-    if (norm_w) {       // the normed input never meets the add epilogue
-        if (packed) {
-            if (epi == EPI_STORE) SKINNY_GO(EPI_STORE, true, true);
-            else SKINNY_GO(EPI_SWIGLU, true, true);
-        } else {
-            if (epi == EPI_STORE) SKINNY_GO(EPI_STORE, false, true);
-            else SKINNY_GO(EPI_SWIGLU, false, true);
+    if (norm_w) {       // the normed input never meets the add epilogue; built for one block of rows
+        if constexpr (MB == 1 && WAVES == 4) {
+            if (packed) {
+                if (epi == EPI_STORE) SKINNY_GO(EPI_STORE, true, true);
+                else SKINNY_GO(EPI_SWIGLU, true, true);
+            } else {
+                if (epi == EPI_STORE) SKINNY_GO(EPI_STORE, false, true);
+                else SKINNY_GO(EPI_SWIGLU, false, true);
+            }
         }
     } else if (packed) {
         if (epi == EPI_STORE) SKINNY_GO(EPI_STORE, true, false);
@@ -590,7 +592,8 @@ static int launch_dma(const void* X, const void* W, void* C, int M, int N, int K
 extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N, int K, int ldc, int epi,
                             int packed, const float* norm_w, float eps, int tile_hint, float* workspace,
                             size_t workspace_floats, hipStream_t stream) {
-    HB_REQUIRE(!norm_w || (M <= 64 && epi != EPI_ADD), "gemm_mfma: the fused norm takes M <= 64 and no add");
+    HB_REQUIRE(!norm_w || (M <= 16 && epi != EPI_ADD && (epi == EPI_SWIGLU || N >= 16384)),
+               "gemm_mfma: the fused norm takes M <= 16, N >= 16384 and no add");
     HB_REQUIRE(!packed || N % 16 == 0, "gemm_mfma: packed weights need N %% 16 == 0");
     HB_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_mfma: empty problem (M=%d, N=%d, K=%d)", M, N, K);
     HB_REQUIRE(epi >= 0 && epi <= 2, "gemm_mfma: unknown epilogue %d", epi);
@@ -614,9 +617,7 @@ extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N,
         tile = K % 64 ? 123 : (big >= 192 ? 185 : 122);
     }
     switch (tile) {
-        case 184: return launch_dma<8, 4, 2, 4, 4, 1>(X, W, C, M, N, K, ldc, epi, packed, stream);   // 256 x 256, 4 stages of 32 k
         case 185: return launch_dma<8, 4, 2, 4, 2, 2>(X, W, C, M, N, K, ldc, epi, packed, stream);   // 256 x 256, 2 stages of 64 k
-        case 182: return launch_dma<4, 4, 2, 4, 3, 2>(X, W, C, M, N, K, ldc, epi, packed, stream);   // 128 x 256, 3 stages of 64 k
         case 122: return launch_dma<4, 4, 2, 2, 2, 2>(X, W, C, M, N, K, ldc, epi, packed, stream);   // 128 x 128, 2 stages of 64 k
         case 123: return launch_dma<4, 4, 2, 2, 4, 1>(X, W, C, M, N, K, ldc, epi, packed, stream);   // 128 x 128, 4 stages of 32 k
         default: HB_REQUIRE(false, "gemm_mfma: unknown tile %d", tile);

@@ -68,8 +68,8 @@ def _norm_args(a, norm, K):
     weight, eps = norm
     _check(a, "a", torch.float32, (None, None))
     _check(weight, "norm weight", torch.float32, (K,))
-    if a.shape[0] > SKINNY_MAX_M:
-        raise BackendError(f"the fused norm takes at most {SKINNY_MAX_M} rows")
+    if a.shape[0] > NORM_FUSE_MAX_M:
+        raise BackendError(f"the fused norm takes at most {NORM_FUSE_MAX_M} rows")
     return weight.data_ptr(), float(eps)
 
 

@@ -274,8 +274,8 @@ def test_gemm_mfma_packed_weights(M, N, K):
     assert torch.equal(plain, packed)
 
 
-@pytest.mark.parametrize("M,N,K,packed", [(1, 48, 32, False), (8, 6144, 4096, True), (16, 272, 96, False),
-                                          (33, 96, 64, True), (64, 1024, 512, True)])
+@pytest.mark.parametrize("M,N,K,packed", [(1, 16384, 32, False), (8, 24576, 4096, True), (16, 16400, 96, False),
+                                          (3, 17024, 64, True)])
 def test_gemm_mfma_with_fused_norm(M, N, K, packed):
     from herbert_rs_amd.kernels import mfma
     x = rand(M, K, seed=30, scale=2.0)
@@ -301,12 +301,12 @@ def test_gemm_mfma_with_fused_norm(M, N, K, packed):
         assert float((act.float() - wanted).abs().max()) <= 2 ** -7 * float(wanted.abs().max()) + 1e-5
 
 
-@pytest.mark.parametrize("tile", [0, 184, 185, 182, 122, 123])
+@pytest.mark.parametrize("tile", [0, 185, 122, 123])
 @pytest.mark.parametrize("M,N,K,packed", [(65, 128, 64, True), (200, 336, 192, True), (300, 530, 96, False),
                                           (513, 1040, 256, True)])
 def test_gemm_mfma_tile_variants(tile, M, N, K, packed):
     from herbert_rs_amd.kernels import mfma
-    if K % 64 and tile not in (0, 184, 123):
+    if K % 64 and tile not in (0, 123):
         pytest.skip("this tile takes K in steps of 64")
     a = rand(M, K, seed=7, dtype=torch.bfloat16)
     w = rand(N, K, seed=8, dtype=torch.bfloat16)
