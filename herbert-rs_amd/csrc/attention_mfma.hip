@@ -185,13 +185,28 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache
 
 // ------------------------------------------------------------------ decode
 // partial_o [B, nq, splits, HD] float, partial_ml [B, nq, splits, 2] float (max, sum).
-template <int HD>
+// FUSED: q is not given; the kernel takes the float32 projection rows qkv [B, (nq + 2 nkv) HD]
+// instead and does the per-head RMSNorm (if weights are given) and the rotation (if tables are
+// given, over the whole head) itself: every wave for its query heads, and the one wave whose
+// range holds the new position also for the new key and value, which it writes to the pages
+// before it reads them (write_kv == 0: the keys and values are another layer's).
+struct DecodeFusion {
+    const float* qkv;
+    const float* q_norm_w;
+    const float* k_norm_w;
+    const float* cos_t;
+    const float* sin_t;
+    float eps;
+    int write_kv;
+};
+
+template <int HD, bool FUSED>
 __global__ void __launch_bounds__(64)
-attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache,
-                   const bf16* __restrict__ v_cache, float* __restrict__ partial_o,
-                   float* __restrict__ partial_ml, const int* __restrict__ context_lens,
-                   const int* __restrict__ slots, const int* __restrict__ page_table, int max_pages, int nq,
-                   int nkv, float c, int window, int pages_per_split) {
+attn_decode_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_cache, bf16* __restrict__ v_cache,
+                   float* __restrict__ partial_o, float* __restrict__ partial_ml,
+                   const int* __restrict__ context_lens, const int* __restrict__ slots,
+                   const int* __restrict__ page_table, int max_pages, int nq, int nkv, float c, int window,
+                   int pages_per_split, DecodeFusion fu) {
     const int b = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z, splits = gridDim.z;
     const int G = nq / nkv;
     const int lane = threadIdx.x, c32 = lane & 31, g2 = lane >> 5;
@@ -204,13 +219,58 @@ attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache,
     const int* pt = page_table + (size_t)slots[b] * max_pages;
     const int head = kvh * G + (c32 < G ? c32 : G - 1);
 
+    constexpr int HALF = HD / 2;
     // k of the MFMA steps: step s, lane group g2, element j  <->  d = g2 * HD/2 + s * 8 + j,
     // so a lane reads one contiguous half row of K
     bf16x8 qreg[HD / 16];
-    {
-        const bf16* qrow = q + ((size_t)b * nq + head) * HD + g2 * (HD / 2);
+    if (!FUSED) {
+        const bf16* qrow = q + ((size_t)b * nq + head) * HD + g2 * HALF;
 #pragma unroll
         for (int s = 0; s < HD / 16; ++s) qreg[s] = *(const bf16x8*)(qrow + s * 8);
+    }
+
+    // FUSED: lane -> the pair of elements (j, j + HD/2) of head `sub` of each round of 64 / (HD/2)
+    // heads. What the norm and the rotation need is loaded before the first page's operands, so
+    // that it arrives first.
+    constexpr int PER = 64 / HALF;                 // heads a round of the wave covers
+    constexpr int PRE = 4;                         // rounds whose inputs are loaded ahead
+    const int j = lane % HALF, sub = lane / HALF;
+    const int hp = hi / PAGE;
+    const bool writer = FUSED && fu.write_kv && hp >= first_page && hp < first_page + pages_per_split;
+    float cs = 1.f, sn = 0.f, qw0 = 1.f, qw1 = 1.f, kw0 = 1.f, kw1 = 1.f;
+    float xq0[PRE], xq1[PRE], k0 = 0.f, k1 = 0.f, v0 = 0.f, v1 = 0.f;
+    int new_page = 0;
+    const float* qin = nullptr;
+    if (FUSED) {
+        const float* row = fu.qkv + (size_t)b * (nq + 2 * nkv) * HD;
+        qin = row + (size_t)kvh * G * HD;
+        if (fu.cos_t) {
+            cs = fu.cos_t[(size_t)hi * HALF + j];
+            sn = fu.sin_t[(size_t)hi * HALF + j];
+        }
+        if (fu.q_norm_w) {
+            qw0 = fu.q_norm_w[j];
+            qw1 = fu.q_norm_w[j + HALF];
+        }
+#pragma unroll
+        for (int it = 0; it < PRE; ++it) {
+            const int hl = it * PER + sub < G ? it * PER + sub : G - 1;
+            xq0[it] = qin[hl * HD + j];
+            xq1[it] = qin[hl * HD + j + HALF];
+        }
+        if (writer) {
+            const float* kin = row + (size_t)(nq + kvh) * HD;
+            const float* vin = row + (size_t)(nq + nkv + kvh) * HD;
+            k0 = kin[j];
+            k1 = kin[j + HALF];
+            v0 = vin[j];
+            v1 = vin[j + HALF];
+            if (fu.k_norm_w) {
+                kw0 = fu.k_norm_w[j];
+                kw1 = fu.k_norm_w[j + HALF];
+            }
+            new_page = pt[hp];
+        }
     }
     f32x16 oacc[HD / 32];
 #pragma unroll
@@ -239,9 +299,78 @@ attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache,
                 _Pragma("unroll") for (int h2 = 0; h2 < 2; ++h2)                             \
                     va[d][kb][h2] = *(const bf16x8*)(vp + (size_t)(d * 32 + c32) * PAGE + kb * 32 + h2 * 16); \
     }
-    if (first_page <= last_page) {
+    __shared__ __attribute__((aligned(16))) bf16 qs[FUSED ? 32 * HD : 8];
+    // norm and rotation of the new key and of the query heads; the key and the value go to the pages,
+    // the queries to LDS, from where each lane takes its operand
+    auto prologue = [&]() {
+        if (writer) {
+            float ss = k0 * k0 + k1 * k1;
+#pragma unroll
+            for (int off = HALF / 2; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+            if (fu.k_norm_w) {
+                const float inv = 1.0f / sqrtf(ss / (float)HD + fu.eps);
+                k0 = k0 * inv * kw0;
+                k1 = k1 * inv * kw1;
+            }
+            const float r0 = k0 * cs - k1 * sn, r1 = k0 * sn + k1 * cs;
+            if (sub == 0) {
+                const int in_page = hi % PAGE;
+                bf16* kdst = k_cache + (((size_t)new_page * nkv + kvh) * PAGE + in_page) * HD;
+                kdst[j] = hb_from_float<bf16>(r0);
+                kdst[j + HALF] = hb_from_float<bf16>(r1);
+                bf16* vdst = v_cache + ((size_t)new_page * nkv + kvh) * HD * PAGE + in_page;
+                vdst[(size_t)j * PAGE] = hb_from_float<bf16>(v0);
+                vdst[(size_t)(j + HALF) * PAGE] = hb_from_float<bf16>(v1);
+            }
+            __threadfence_block();      // this wave's later loads of that page see what it has just written
+        }
+        auto finish_head = [&](int hl, float x0, float x1) {
+            if (fu.q_norm_w) {
+                float ss = x0 * x0 + x1 * x1;
+#pragma unroll
+                for (int off = HALF / 2; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+                const float inv = 1.0f / sqrtf(ss / (float)HD + fu.eps);
+                x0 = x0 * inv * qw0;
+                x1 = x1 * inv * qw1;
+            }
+            if (hl < G) {
+                qs[hl * HD + j] = hb_from_float<bf16>(x0 * cs - x1 * sn);
+                qs[hl * HD + j + HALF] = hb_from_float<bf16>(x0 * sn + x1 * cs);
+            }
+        };
+#pragma unroll
+        for (int it = 0; it < PRE; ++it)
+            if (it * PER < G) finish_head(it * PER + sub, xq0[it], xq1[it]);
+        for (int it = PRE; it * PER < G; ++it) {
+            const int hl = it * PER + sub;
+            const int hs = hl < G ? hl : G - 1;
+            finish_head(hl, qin[hs * HD + j], qin[hs * HD + j + HALF]);
+        }
+    };
+    // The first page's operands go out before that work, so that it hides their way from memory,
+    // unless this wave has yet to write the new key into that very page. (Two copies of the code:
+    // each then knows how many loads are in flight behind the small ones it waits for.)
+    if (!FUSED) {
+        if (first_page <= last_page) {
+            LOAD_K(first_page)
+            LOAD_V(first_page)
+        }
+    } else if (first_page <= last_page && !(writer && first_page == hp)) {
         LOAD_K(first_page)
         LOAD_V(first_page)
+        prologue();
+    } else {
+        prologue();
+        if (first_page <= last_page) {
+            LOAD_K(first_page)
+            LOAD_V(first_page)
+        }
+    }
+    if (FUSED) {
+        __syncthreads();
+        const bf16* qrow = qs + (c32 < G ? c32 : G - 1) * HD + g2 * HALF;
+#pragma unroll
+        for (int s2 = 0; s2 < HD / 16; ++s2) qreg[s2] = *(const bf16x8*)(qrow + s2 * 8);
     }
     for (int page_idx = first_page; page_idx <= last_page; ++page_idx) {
         f32x16 st[2];
@@ -378,11 +507,14 @@ extern "C" int hb_attn_prefill_mfma(const void* q, const void* k_cache, const vo
     return 0;
 }
 
-extern "C" int hb_attn_decode_mfma(const void* q, const void* k_cache, const void* v_cache, void* out,
+// qkv != null: the fused form (see DecodeFusion); q is then not read.
+extern "C" int hb_attn_decode_mfma(const void* q, void* k_cache, void* v_cache, void* out,
                                    float* partial_o, float* partial_ml, const int* context_lens,
                                    const int* slots, const int* page_table, int max_pages, int page_size,
                                    int B, int nq, int nkv, int hd, float scale, int window, int splits,
-                                   int pages_per_split, hipStream_t stream) {
+                                   int pages_per_split, const float* qkv, const float* q_norm_w,
+                                   const float* k_norm_w, const float* cos_t, const float* sin_t, float eps,
+                                   int write_kv, hipStream_t stream) {
     HB_REQUIRE(B > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attn_decode: bad sizes");
     HB_REQUIRE(page_size == PAGE, "attn_decode: pages must hold %d tokens", PAGE);
     HB_REQUIRE(nq / nkv <= 32, "attn_decode: more than 32 query heads share a kv head");
@@ -390,11 +522,18 @@ extern "C" int hb_attn_decode_mfma(const void* q, const void* k_cache, const voi
     HB_REQUIRE(window >= 0, "attn_decode: bad window");
     dim3 grid(B, nkv, splits);
     const float c = scale * LOG2E;
+    const DecodeFusion fu = {qkv, q_norm_w, k_norm_w, cos_t, sin_t, eps, write_kv};
+    HB_REQUIRE(qkv || q, "attn_decode: neither q nor the projection rows are given");
+    HB_REQUIRE((cos_t == nullptr) == (sin_t == nullptr), "attn_decode: cos and sin tables come together");
 #define LAUNCH_DECODE(HDV) do {                                                                          \
-    attn_decode_kernel<HDV><<<grid, 64, 0, stream>>>((const bf16*)q, (const bf16*)k_cache,               \
-                                                    (const bf16*)v_cache, partial_o, partial_ml,         \
-                                                    context_lens, slots, page_table, max_pages, nq, nkv, c, \
-                                                    window, pages_per_split);                          \
+    if (qkv)                                                                                             \
+        attn_decode_kernel<HDV, true><<<grid, 64, 0, stream>>>(nullptr, (bf16*)k_cache, (bf16*)v_cache,  \
+            partial_o, partial_ml, context_lens, slots, page_table, max_pages, nq, nkv, c, window,       \
+            pages_per_split, fu);                                                                        \
+    else                                                                                                 \
+        attn_decode_kernel<HDV, false><<<grid, 64, 0, stream>>>((const bf16*)q, (bf16*)k_cache,          \
+            (bf16*)v_cache, partial_o, partial_ml, context_lens, slots, page_table, max_pages, nq, nkv,  \
+            c, window, pages_per_split, fu);                                                             \
     attn_decode_merge_kernel<HDV><<<B * nq, 256, 0, stream>>>(partial_o, partial_ml, (bf16*)out, splits, c); \
     } while (0)
     if (hd == 32) LAUNCH_DECODE(32);

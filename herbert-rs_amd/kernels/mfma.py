@@ -125,7 +125,8 @@ def gemm_swiglu(a, w_interleaved, out, packed=False, norm=None, tile=0):
 
 lib.register_signatures("attention_mfma", {
     "hb_attn_prefill_mfma": [_P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P],
-    "hb_attn_decode_mfma": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P],
+    "hb_attn_decode_mfma": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I,
+                            _P, _P, _P, _P, _P, _F, _I, _P],
 })
 
 ATTENTION_HEAD_DIMS = (32, 64, 128)
@@ -181,6 +182,50 @@ def _partial_buffers(device, n_rows, splits, hd):
     return buf
 
 
+def decode_fusable(meta, kv, nq, nkv, hd, rot_dims, dtype):
+    """True if the decode kernel can do the per-head norm, the rotation and the cache write itself:
+    one token a sequence, bfloat16, a head size it is built for, rotation over the whole head or none."""
+    return (meta.max_new == 1 and meta.num_tokens == meta.num_seqs and dtype == torch.bfloat16
+            and kv.k.dtype == torch.bfloat16 and kv.page_size == 64 and hd in ATTENTION_HEAD_DIMS
+            and nq % nkv == 0 and nq // nkv <= 32 and rot_dims in (0, hd))
+
+
+def attention_decode_fused(qkv, q_norm_w, k_norm_w, cos, sin, meta, kv, out, nq, nkv, hd, eps, scale, window):
+    """One token a sequence: per-head norm (if weights are given), rotation (if tables are given),
+    the new key and value written to the pages, and attention over them, in one kernel (+ merge).
+    qkv f32 [B, (nq + 2 nkv) hd]; cos / sin f32 [max_pos, hd / 2]; out bf16 [B, nq hd]."""
+    B = meta.num_seqs
+    _check(qkv, "qkv", torch.float32, (B, (nq + 2 * nkv) * hd))
+    _check(out, "out", torch.bfloat16, (B, nq * hd))
+    pages = kv.k.shape[0]
+    _check(kv.k, "key pages", torch.bfloat16, (pages, nkv, 64, hd))
+    _check(kv.v, "value pages", torch.bfloat16, (pages, nkv, hd, 64))
+    _check(kv.page_table, "page_table", torch.int32, (None, None))
+    _check(meta.slots, "slots", torch.int32, (B,))
+    _check(meta.context_lens, "context_lens", torch.int32, (B,))
+    if not decode_fusable(meta, kv, nq, nkv, hd, hd if cos is not None else 0, torch.bfloat16):
+        raise BackendError(f"fused decode attention refuses head_dim {hd} with {nq}/{nkv} heads in this step")
+    for w, name in ((q_norm_w, "q_norm"), (k_norm_w, "k_norm")):
+        if w is not None:
+            _check(w, name, torch.float32, (hd,))
+    if (cos is None) != (sin is None):
+        raise BackendError("cos and sin tables come together")
+    if cos is not None:
+        _check(cos, "cos", torch.float32, (None, hd // 2))
+        _check(sin, "sin", torch.float32, tuple(cos.shape))
+        if meta.max_position >= cos.shape[0]:
+            raise BackendError(f"position {meta.max_position} beyond the rotation table ({cos.shape[0]} rows)")
+    window = int(window or 0)
+    splits, per = _decode_split(meta, nkv, window)
+    po, pml = _partial_buffers(qkv.device, B * nq, splits, hd)
+    lib.call("attention_mfma", "hb_attn_decode_mfma", None, kv.k.data_ptr(), kv.v.data_ptr(), out.data_ptr(),
+             po.data_ptr(), pml.data_ptr(), meta.context_lens.data_ptr(), meta.slots.data_ptr(),
+             kv.page_table.data_ptr(), kv.page_table.shape[1], kv.page_size, B, nq, nkv, hd, float(scale),
+             window, splits, per, qkv.data_ptr(), None if q_norm_w is None else q_norm_w.data_ptr(),
+             None if k_norm_w is None else k_norm_w.data_ptr(), None if cos is None else cos.data_ptr(),
+             None if sin is None else sin.data_ptr(), float(eps), 1, _stream())
+
+
 def attention(q, meta, kv, out, nq, nkv, hd, scale, window):
     """Causal (and windowed) attention of the step's tokens over their slots' pages.
     One token a sequence: the split decode kernel; otherwise the tiled prefill kernel."""
@@ -204,7 +249,8 @@ def attention(q, meta, kv, out, nq, nkv, hd, scale, window):
         lib.call("attention_mfma", "hb_attn_decode_mfma", q.data_ptr(), kv.k.data_ptr(), kv.v.data_ptr(),
                  out.data_ptr(), po.data_ptr(), pml.data_ptr(), meta.context_lens.data_ptr(),
                  meta.slots.data_ptr(), kv.page_table.data_ptr(), kv.page_table.shape[1], kv.page_size,
-                 T, nq, nkv, hd, float(scale), window, splits, per, _stream())
+                 T, nq, nkv, hd, float(scale), window, splits, per, None, None, None, None, None, 0.0, 0,
+                 _stream())
         return
     _check(meta.positions, "positions", torch.int32, (T,))
     tile_seq, tile_row0, tile_rows, n_tiles = _prefill_tiles(meta)

@@ -105,12 +105,20 @@ class Attention(Part):
             self.qkv.forward_normed(x, fused_norm.w, fused_norm.eps, qkv)
         else:
             self.qkv.forward(y, qkv)
-        q = rt.buffer("q", (T, self.q_dim))
         rot = self.position.rotation()
         cos, sin, rot_dims = rot if rot is not None else (None, None, 0)
+        attn = rt.buffer("attn", (T, self.q_dim))
+        if write_kv and rt.dtype == torch.bfloat16:
+            from ..kernels import mfma
+            if mfma.decode_fusable(ctx.meta, kv, self.nq, self.nkv, self.hd, rot_dims, rt.dtype):
+                # one token a sequence: norm, rotation, cache write and attention in one kernel
+                mfma.attention_decode_fused(qkv, self.q_norm_w, self.k_norm_w, cos, sin, ctx.meta, kv, attn,
+                                            self.nq, self.nkv, self.hd, self.eps, self.scale, self.window)
+                self.o.forward(attn, x, accumulate=True)
+                return
+        q = rt.buffer("q", (T, self.q_dim))
         ops.qk_norm_rope_write(qkv, self.q_norm_w, self.k_norm_w, cos, sin, rot_dims, ctx.meta, kv, q,
                                self.nq, self.nkv, self.hd, self.eps, write_kv=write_kv)
-        attn = rt.buffer("attn", (T, self.q_dim))
         self.attend(ctx, q, kv, attn)
         self.o.forward(attn, x, accumulate=True)
 

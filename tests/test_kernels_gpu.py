@@ -239,6 +239,42 @@ def test_attention_mfma_decode(nq, nkv, hd, window, lengths):
     assert float((out.float().cpu() - want).abs().max()) <= 2 ** -7 * float(want.abs().max())
 
 
+@pytest.mark.parametrize("nq,nkv,hd,window,norm,rope", [(4, 1, 128, 0, True, True), (32, 8, 128, 0, True, True),
+                                                        (6, 2, 32, 0, True, False), (5, 1, 64, 70, False, True),
+                                                        (3, 3, 128, 100, True, True), (64, 2, 64, 0, False, False)])
+@pytest.mark.parametrize("lengths", [[1, 64, 65, 700], [1000], [130, 3, 512, 999, 77, 640, 64, 128, 256]])
+def test_attention_mfma_decode_fused_with_norm_rotation_and_cache_write(nq, nkv, hd, window, norm, rope, lengths):
+    """The decode kernel that norms, rotates and writes the new key and value itself against the
+    separate kernels: same pages afterwards, same output."""
+    from herbert_rs_amd.cache.paged import LayerKV
+    from herbert_rs_amd.kernels import mfma, ops
+    B = len(lengths)
+    meta, kv, _ = paged_case(lengths, [1] * B, nkv, hd, torch.bfloat16, seed=nq + hd, n_pages=80)
+    kv2 = LayerKV(kv.k.clone(), kv.v.clone(), kv.page_table, 64, 0)
+    qkv = rand(B, (nq + 2 * nkv) * hd, seed=23, scale=1.5)
+    qw = (1 + rand(hd, seed=24, scale=0.3)) if norm else None
+    kw = (1 + rand(hd, seed=25, scale=0.3)) if norm else None
+    cos = sin = None
+    if rope:
+        ang = torch.arange(1024, dtype=torch.float32)[:, None] * (10000.0 ** (-torch.arange(hd // 2) / (hd // 2)))[None]
+        cos, sin = ang.cos().to(dev()).contiguous(), ang.sin().to(dev()).contiguous()
+    scale, eps = hd ** -0.5, 1e-5
+    assert mfma.decode_fusable(meta, kv, nq, nkv, hd, hd if rope else 0, torch.bfloat16)
+    q = torch.empty(B, nq * hd, dtype=torch.bfloat16, device=dev())
+    want = torch.full_like(q, 9.0)
+    ops.qk_norm_rope_write(qkv, qw, kw, cos, sin, hd if rope else 0, meta, kv, q, nq, nkv, hd, eps)
+    mfma.attention(q, meta, kv, want, nq, nkv, hd, scale, window)
+    got = torch.full_like(q, 7.0)
+    mfma.attention_decode_fused(qkv, qw, kw, cos, sin, meta, kv2, got, nq, nkv, hd, eps, scale, window)
+    assert torch.equal(kv.v, kv2.v)
+    # the two kernels sum the squares in another order: a key element may round the other way
+    dk = (kv.k.float() - kv2.k.float()).abs()
+    assert float(dk.max()) <= 2 ** -7 * float(kv.k.float().abs().max())
+    assert float((dk > 0).float().mean()) < 1e-3
+    w = want.float()
+    assert float((got.float() - w).abs().max()) <= 2 ** -6 * float(w.abs().max())
+
+
 def test_attention_finds_one_far_key_among_hundreds():
     """One key far back scores far above the rest: the output must be its value, whichever page
     and split it lies in. Random keys would hide a page or a split that is skipped."""
