@@ -388,6 +388,13 @@ __device__ __forceinline__ void wait_vmcnt() {
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N_OUTSTANDING) : "memory");
 }
 
+// The barrier alone: __syncthreads() would first wait for every load in flight, the later stages'
+// too, and so undo the ring. What has to have landed is waited for by wait_vmcnt before it; the
+// operand reads of the step before are in registers already (the matrix cores have used them).
+__device__ __forceinline__ void workgroup_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 template <int EPI, bool PACKED, int TNB, int TMB, int WNW, int WMW, int STAGES, int KS>
 __global__ void __launch_bounds__(64 * WNW * WMW)
 gemm_dma_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* __restrict__ Cv, int M, int N,
@@ -399,15 +406,21 @@ gemm_dma_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* __
     static_assert(WBLK % NW == 0 && XBLK % NW == 0, "blocks must divide over the waves");
     extern __shared__ __attribute__((aligned(1024))) bf16 lds[];        // [STAGES][KS][BLKS][512]
 
+    // Workgroups go round the 8 XCDs, each with an L2 of its own: an XCD takes a run of tiles, and
+    // within it bands of 8 tiles in m are walked n first, so that the workgroups that are resident
+    // together share both their weight and their activation panels in that L2.
     const int total = m_tiles * n_tiles;
     const int chunk = (total + 7) / 8;
-    const int id = (blockIdx.x % 8) * chunk + blockIdx.x / 8;          // a run of tiles per XCD
+    const int id = (blockIdx.x % 8) * chunk + blockIdx.x / 8;
     if (id >= total) return;
-    const int n_tile = id / m_tiles, m_tile = id % m_tiles;
+    constexpr int BAND = 8;
+    const int band = id / (BAND * n_tiles), in_band = id % (BAND * n_tiles);
+    const int band_rows = m_tiles - band * BAND < BAND ? m_tiles - band * BAND : BAND;
+    const int n_tile = in_band / band_rows, m_tile = band * BAND + in_band % band_rows;
     const int m0 = m_tile * BM, n0 = n_tile * BN;
 
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // uniform: LDS addresses stay scalar
     const int r16 = lane & 15, g4 = lane >> 4;
     const int wn = wave / WMW, wm = wave % WMW;
     const int k32 = K / 32;              // k-steps of 32 in all
@@ -435,107 +448,269 @@ gemm_dma_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* __
         if (m >= M) m = M - 1;
         xsrc[i] = X + (size_t)m * K + g4 * 8;
     }
+    // Stages of 64 k: the activations lie in LDS as rows of 128 bytes, so that a load fetches
+    // whole 128-byte lines (8 rows an instruction, 8 lanes a row) instead of half lines twice.
+    // The 16-byte chunk c of row r sits at chunk c ^ ((r >> 1) & 7) of its row: the operand reads
+    // of 16 rows at one k then fall into 16 different bank groups.
+    constexpr bool XROWS = KS == 2;
+    constexpr int XR = XROWS ? BM / 8 / NW : 1;                       // row loads of a wave per stage
+    static_assert(!XROWS || BM % (8 * NW) == 0, "rows must divide over the waves");
+    const bf16* xrsrc[XR];
+#pragma unroll
+    for (int i = 0; i < XR; ++i) {
+        const int r = (wave * XR + i) * 8 + (lane >> 3);
+        int m = m0 + r;
+        if (m >= M) m = M - 1;
+        xrsrc[i] = X + (size_t)m * K + (((lane & 7) ^ ((r >> 1) & 7)) * 8);
+    }
     const size_t WSTEP = PACKED ? (size_t)(N / 16) * 512 : 32;
 
     auto issue = [&](int step, int stage) {
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            bf16* base = lds + (size_t)(stage * KS + ks) * BLKS * 512;
+            bf16* base = lds + (XROWS ? (size_t)stage * KS * BLKS * 512 + ks * WBLK * 512
+                                      : (size_t)(stage * KS + ks) * BLKS * 512);
             const size_t k = (size_t)step * KS + ks;
 #pragma unroll
             for (int i = 0; i < WL; ++i)
                 __builtin_amdgcn_global_load_lds(
                     (const __attribute__((address_space(1))) void*)(wsrc[i] + k * WSTEP),
                     (__attribute__((address_space(3))) void*)(base + (wave * WL + i) * 512), 16, 0, 0);
+            if (!XROWS) {
 #pragma unroll
-            for (int i = 0; i < XL; ++i)
+                for (int i = 0; i < XL; ++i)
+                    __builtin_amdgcn_global_load_lds(
+                        (const __attribute__((address_space(1))) void*)(xsrc[i] + k * 32),
+                        (__attribute__((address_space(3))) void*)(base + (WBLK + wave * XL + i) * 512), 16, 0, 0);
+            }
+        }
+        if (XROWS) {
+            // the stage's activations follow the weight blocks of its two k-steps: [BM][64]
+            bf16* xbase = lds + (size_t)stage * KS * BLKS * 512 + KS * WBLK * 512;
+#pragma unroll
+            for (int i = 0; i < XR; ++i)
                 __builtin_amdgcn_global_load_lds(
-                    (const __attribute__((address_space(1))) void*)(xsrc[i] + k * 32),
-                    (__attribute__((address_space(3))) void*)(base + (WBLK + wave * XL + i) * 512), 16, 0, 0);
+                    (const __attribute__((address_space(1))) void*)(xrsrc[i] + (size_t)step * 64),
+                    (__attribute__((address_space(3))) void*)(xbase + (wave * XR + i) * 512), 16, 0, 0);
         }
     };
 
-    f32x4 acc[TNB][TMB];
+    // 32x32x16 MFMA (it has the higher rate of the two bf16 shapes): an operand is 32 rows x 16 k,
+    // lane l = row l % 32, k 8 (l / 32) .. + 8. In the 1 KB blocks of 16 rows x 32 k that is, for the
+    // k-half h: block (l % 32) / 16 of a pair of blocks, chunk 16 (2 h + l / 32) + l % 16.
+    static_assert(TNB % 2 == 0 && TMB % 2 == 0, "a wave's tile is made of 32 x 32 pieces");
+    constexpr int TN32 = TNB / 2, TM32 = TMB / 2;
+    const int c32 = lane & 31, g2 = lane >> 5;
+    const int lane_off = (c32 >> 4) * 512 + (16 * g2 + (lane & 15)) * 8;   // + 32 * 8 for the second k-half
+    f32x16 acc[TN32][TM32];
 #pragma unroll
-    for (int a = 0; a < TNB; ++a)
+    for (int a = 0; a < TN32; ++a)
 #pragma unroll
-        for (int b = 0; b < TMB; ++b) acc[a][b] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int b = 0; b < TM32; ++b)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.f;
+
+    // Operands in two sets of registers: while the matrix cores work on one k-step of 32, the
+    // reads of the next one are on their way, so a wave never waits for LDS with nothing to do.
+    bf16x8 wv[2][2][TN32], xv[2][2][TM32];       // [set][k-half][piece]
+    const int x_swizzle = (c32 >> 1) & 7;           // of this lane's rows: they are c32 + a multiple of 16
+    auto read_operands = [&](int set, int stage, int ks) {
+        const bf16* base = lds + (XROWS ? (size_t)stage * KS * BLKS * 512 + ks * WBLK * 512
+                                        : (size_t)(stage * KS + ks) * BLKS * 512) + lane_off;
+        const bf16* xrows = lds + (size_t)stage * KS * BLKS * 512 + KS * WBLK * 512 +
+                            ((wm * TMB) * 16 + c32) * 64;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+#pragma unroll
+            for (int a = 0; a < TN32; ++a)
+                wv[set][h][a] = *(const bf16x8*)(base + (wn * TNB + 2 * a) * 512 + h * 256);
+#pragma unroll
+            for (int b = 0; b < TM32; ++b) {
+                if (XROWS)
+                    xv[set][h][b] = *(const bf16x8*)(xrows + b * 32 * 64 + (((4 * ks + 2 * h + g2) ^ x_swizzle) * 8));
+                else
+                    xv[set][h][b] = *(const bf16x8*)(base + (WBLK + wm * TMB + 2 * b) * 512 + h * 256);
+            }
+        }
+    };
+    auto multiply = [&](int set) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int a = 0; a < TN32; ++a)
+#pragma unroll
+                for (int b = 0; b < TM32; ++b)
+                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wv[set][h][a], xv[set][h][b], acc[a][b],
+                                                                        0, 0, 0);
+    };
+    // Before step t + 1 is read: this wave's loads of it have landed (those of the STAGES - 2 later
+    // steps may be in flight) and its reads of step t are in registers; after the barrier that
+    // holds for every wave, so the stage of step t can take the loads of step t + STAGES.
+    auto advance = [&](int t) {
+        wait_vmcnt<(STAGES - 2) * (XROWS ? WL * KS + XR : (WL + XL) * KS)>();
+        workgroup_barrier();
+        const int nt = t + STAGES;
+        issue(nt < nsteps ? nt : nsteps - 1, nt % STAGES);
+    };
+    // one step; `first` is the register set that holds its first k-step (a constant once unrolled)
+    auto run_step = [&](int first, int t) {
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            const int set = (first + ks) & 1;
+            if (ks + 1 < KS) {
+                read_operands(set ^ 1, t % STAGES, ks + 1);
+            } else if (t + 1 < nsteps) {
+                advance(t);
+                read_operands(set ^ 1, (t + 1) % STAGES, 0);
+            }
+            multiply(set);
+        }
+    };
 
 #pragma unroll
     for (int st = 0; st < STAGES - 1; ++st) issue(st < nsteps ? st : nsteps - 1, st);
-
-    for (int t = 0; t < nsteps; ++t) {
-        // this wave's loads of step t have landed (those of the STAGES - 2 later steps may be in flight);
-        // after the barrier everyone's have, and everyone has finished reading step t - 1
-        wait_vmcnt<(STAGES - 2) * (WL + XL) * KS>();
-        __syncthreads();
-        {
-            const int nt = t + STAGES - 1;
-            issue(nt < nsteps ? nt : nsteps - 1, nt % STAGES);
+    advance(-1);
+    read_operands(0, 0, 0);
+    if constexpr (KS == 2) {
+        // Stages of two k-steps: no branch in the loop (the last step is peeled off), and the work
+        // other than MFMAs is dealt out between them by hand: a wave then has an MFMA in the pipe
+        // while it issues its reads and loads, also right after the barrier, where the other wave
+        // of its SIMD stands at the same place and cannot fill in.
+        constexpr int NM = 2 * TN32 * TM32;              // MFMAs of a k-step
+        constexpr int NR = 2 * (TN32 + TM32);            // operand reads of a k-step
+        constexpr int ND = WL * KS + XR;                 // loads of a stage
+        constexpr int SLOTS = NM > 6 ? NM - 4 : NM;      // the last MFMAs cover the latency of the last reads
+        auto mfma_one = [&](int set, int j) {
+            const int h = j / (TN32 * TM32), a = j / TM32 % TN32, b = j % TM32;
+            acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wv[set][h][a], xv[set][h][b], acc[a][b], 0, 0, 0);
+        };
+        auto read_one = [&](int set, int stage, int ks, int idx) {
+            const int h = idx / (TN32 + TM32), r = idx % (TN32 + TM32);
+            const bf16* sbase = lds + (size_t)stage * KS * BLKS * 512;
+            if (r < TN32) {
+                wv[set][h][r] = *(const bf16x8*)(sbase + ks * WBLK * 512 + lane_off + (wn * TNB + 2 * r) * 512 + h * 256);
+            } else {
+                const int b = r - TN32;
+                xv[set][h][b] = *(const bf16x8*)(sbase + KS * WBLK * 512 + ((wm * TMB) * 16 + c32 + b * 32) * 64 +
+                                                 (((4 * ks + 2 * h + g2) ^ x_swizzle) * 8));
+            }
+        };
+        auto load_one = [&](int step, int stage, int idx) {
+            bf16* sbase = lds + (size_t)stage * KS * BLKS * 512;
+            if (idx < WL * KS) {
+                const int ks = idx / WL, i = idx % WL;
+                __builtin_amdgcn_global_load_lds(
+                    (const __attribute__((address_space(1))) void*)(wsrc[i] + ((size_t)step * KS + ks) * WSTEP),
+                    (__attribute__((address_space(3))) void*)(sbase + ks * WBLK * 512 + (wave * WL + i) * 512), 16, 0, 0);
+            } else {
+                const int i = idx - WL * KS;
+                __builtin_amdgcn_global_load_lds(
+                    (const __attribute__((address_space(1))) void*)(xrsrc[i] + (size_t)step * 64),
+                    (__attribute__((address_space(3))) void*)(sbase + KS * WBLK * 512 + (wave * XR + i) * 512), 16, 0, 0);
+            }
+        };
+        for (int t = 0; t + 1 < nsteps; ++t) {
+            const int stage = t % STAGES, next_stage = (t + 1) % STAGES;
+            // first k-step: its MFMAs, with the reads of the second k-step between them
+#pragma unroll
+            for (int j = 0; j < NM; ++j) {
+                mfma_one(0, j);
+#pragma unroll
+                for (int o = (j < SLOTS ? j : SLOTS) * NR / SLOTS; o < (j + 1 < SLOTS ? j + 1 : SLOTS) * NR / SLOTS; ++o)
+                    read_one(1, stage, 1, o);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            // second k-step: step t + 1 has landed for everyone and nobody reads this stage any more;
+            // between the MFMAs go the loads of step t + STAGES into it, then the reads of step t + 1
+            wait_vmcnt<(STAGES - 2) * ND>();
+            workgroup_barrier();
+            const int nt = t + STAGES < nsteps ? t + STAGES : nsteps - 1;
+#pragma unroll
+            for (int j = 0; j < NM; ++j) {
+                mfma_one(1, j);
+#pragma unroll
+                for (int o = (j < SLOTS ? j : SLOTS) * (ND + NR) / SLOTS;
+                     o < (j + 1 < SLOTS ? j + 1 : SLOTS) * (ND + NR) / SLOTS; ++o) {
+                    if (o < ND) load_one(nt, stage, o);
+                    else read_one(0, next_stage, 0, o - ND);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
+        {
+            const int stage = (nsteps - 1) % STAGES;
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            const bf16* base = lds + (size_t)((t % STAGES) * KS + ks) * BLKS * 512 + lane * 8;
-            bf16x8 wv[TNB], xv[TMB];
+            for (int j = 0; j < NM; ++j) {
+                mfma_one(0, j);
 #pragma unroll
-            for (int a = 0; a < TNB; ++a) wv[a] = *(const bf16x8*)(base + (wn * TNB + a) * 512);
-#pragma unroll
-            for (int b = 0; b < TMB; ++b) xv[b] = *(const bf16x8*)(base + (WBLK + wm * TMB + b) * 512);
-            // all operand reads go out before the first MFMA: the other wave of the SIMD computes meanwhile
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int a = 0; a < TNB; ++a)
-#pragma unroll
-                for (int b = 0; b < TMB; ++b)
-                    acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[a], xv[b], acc[a][b], 0, 0, 0);
+                for (int o = (j < SLOTS ? j : SLOTS) * NR / SLOTS; o < (j + 1 < SLOTS ? j + 1 : SLOTS) * NR / SLOTS; ++o)
+                    read_one(1, stage, 1, o);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            multiply(1);
+        }
+    } else if (KS % 2 == 0) {
+        for (int t = 0; t < nsteps; ++t) run_step(0, t);
+    } else {
+        for (int t = 0; t < nsteps; t += 2) {
+            run_step(0, t);
+            if (t + 1 < nsteps) run_step(1, t + 1);
         }
     }
     wait_vmcnt<0>();      // the loads past the end (repeats of the last step) have landed too
 
-    // lane: m = m0 + (wm * TMB + b) * 16 + r16 ; n = n0 + (wn * TNB + a) * 16 + g4 * 4 + i
+    // lane: m = m0 + (wm * TMB + 2 b) * 16 + c32 ; register 4 q + j of a piece:
+    // n = n0 + (wn * TNB + 2 a) * 16 + 8 q + 4 g2 + j, four consecutive n for each q
 #pragma unroll
-    for (int b = 0; b < TMB; ++b) {
-        const int m = m0 + (wm * TMB + b) * 16 + r16;
+    for (int b = 0; b < TM32; ++b) {
+        const int m = m0 + (wm * TMB + 2 * b) * 16 + c32;
         if (m >= M) continue;
         if (EPI == EPI_SWIGLU) {
             bf16* C = (bf16*)Cv;
 #pragma unroll
-            for (int a = 0; a + 1 < TNB; a += 2) {
-                const int n = (n0 + (wn * TNB + a) * 16) / 2 + g4 * 4;     // blocks a, a + 1 = gate, up
-                if (n + 3 < N / 2 && (ldc & 3) == 0) {
-                    bf16x4 v;
+            for (int a = 0; a < TN32; ++a)
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) v[i] = (__bf16)silu_mul(acc[a][b][i], acc[a + 1][b][i]);
-                    *(bf16x4*)((__bf16*)C + (size_t)m * ldc + n) = v;
-                } else {
+                for (int q = 0; q < 2; ++q) {
+                    // rows 0..15 of the piece are gate rows, 16..31 the up rows of the same outputs
+                    const int n = (n0 + (wn * TNB + 2 * a) * 16) / 2 + 8 * q + 4 * g2;
+                    if (n + 3 < N / 2 && (ldc & 3) == 0) {
+                        bf16x4 v;
 #pragma unroll
-                    for (int i = 0; i < 4; ++i)
-                        if (n + i < N / 2)
-                            C[(size_t)m * ldc + n + i] =
-                                hb_from_float<bf16>(silu_mul(acc[a][b][i], acc[a + 1][b][i]));
+                        for (int j = 0; j < 4; ++j)
+                            v[j] = (__bf16)silu_mul(acc[a][b][4 * q + j], acc[a][b][4 * q + 8 + j]);
+                        *(bf16x4*)((__bf16*)C + (size_t)m * ldc + n) = v;
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+                            if (n + j < N / 2)
+                                C[(size_t)m * ldc + n + j] = hb_from_float<bf16>(
+                                    silu_mul(acc[a][b][4 * q + j], acc[a][b][4 * q + 8 + j]));
+                    }
                 }
-            }
         } else {
             float* C = (float*)Cv;
 #pragma unroll
-            for (int a = 0; a < TNB; ++a) {
-                const int n = n0 + (wn * TNB + a) * 16 + g4 * 4;
-                float* dst = C + (size_t)m * ldc + n;
-                if (n + 3 < N && (ldc & 3) == 0) {
-                    f32x4 v = acc[a][b];
-                    if (EPI == EPI_ADD) v += *(const f32x4*)dst;
-                    *(f32x4*)dst = v;
-                } else {
+            for (int a = 0; a < TN32; ++a)
 #pragma unroll
-                    for (int i = 0; i < 4; ++i)
-                        if (n + i < N) {
-                            if (EPI == EPI_ADD)
-                                dst[i] += acc[a][b][i];
-                            else
-                                dst[i] = acc[a][b][i];
-                        }
+                for (int q = 0; q < 4; ++q) {
+                    const int n = n0 + (wn * TNB + 2 * a) * 16 + 8 * q + 4 * g2;
+                    float* dst = C + (size_t)m * ldc + n;
+                    if (n + 3 < N && (ldc & 3) == 0) {
+                        f32x4 v = {acc[a][b][4 * q], acc[a][b][4 * q + 1], acc[a][b][4 * q + 2],
+                                   acc[a][b][4 * q + 3]};
+                        if (EPI == EPI_ADD) v += *(const f32x4*)dst;
+                        *(f32x4*)dst = v;
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+                            if (n + j < N) {
+                                if (EPI == EPI_ADD)
+                                    dst[j] += acc[a][b][4 * q + j];
+                                else
+                                    dst[j] = acc[a][b][4 * q + j];
+                            }
+                    }
                 }
-            }
         }
     }
 }
@@ -620,6 +795,7 @@ extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N,
         case 185: return launch_dma<8, 4, 2, 4, 2, 2>(X, W, C, M, N, K, ldc, epi, packed, stream);   // 256 x 256, 2 stages of 64 k
         case 122: return launch_dma<4, 4, 2, 2, 2, 2>(X, W, C, M, N, K, ldc, epi, packed, stream);   // 128 x 128, 2 stages of 64 k
         case 123: return launch_dma<4, 4, 2, 2, 4, 1>(X, W, C, M, N, K, ldc, epi, packed, stream);   // 128 x 128, 4 stages of 32 k
+        case 188: return launch_dma<8, 8, 2, 2, 2, 2>(X, W, C, M, N, K, ldc, epi, packed, stream);   // 256 x 256, 4 waves
         default: HB_REQUIRE(false, "gemm_mfma: unknown tile %d", tile);
     }
     return 0;
