@@ -375,13 +375,16 @@ static void pick_skinny(const void* X, const void* W, void* C, int M, int N, int
 }
 
 // ------------------------------------------------------------------- tiled
-// The product for many rows (prompts), with the tiles going from global memory straight into LDS
-// (global_load_lds_dwordx4: a lane's 16 bytes land at base + 16 * lane, no registers, no
-// ds_write) and a ring of STAGES k-steps of 32 in LDS, loaded STAGES - 1 steps ahead.
-// LDS holds MFMA operands as they are used: a block of 16 rows x 32 k is 1 KB in lane order
-// (lane = 16 * (k / 8 % 4) + row % 16), which is the packed weight order, so a packed weight
-// block is one contiguous 1 KB load and an operand read is lane * 16 bytes, free of conflicts.
-// 16x16x32 MFMA, weight rows first: a lane ends with four consecutive n of one m.
+// The product for many rows (prompts). Tiles go from global memory straight into LDS
+// (global_load_lds_dwordx4: a lane's 16 bytes land at base + 16 * lane; no registers, no
+// ds_write) through rings of stages that are loaded ahead of the MFMAs.
+// 32x32x16 MFMA (of the two bf16 shapes the one with the higher rate), weight rows first: an
+// operand is 32 rows x 16 k, lane l = row l % 32, k 8 (l / 32) .. + 8; a lane ends with 16 sums
+// of one m: n = 8 q + 4 (l / 32) + j for register 4 q + j.
+// Weights lie in LDS as in memory when packed: 1 KB blocks of 16 rows x 32 k, chunk
+// 16 (k / 8 % 4) + row % 16. For the k-half h of a k-step of 32 an operand is then: block
+// (l % 32) / 16 of a pair of blocks, chunk 16 (2 h + l / 32) + l % 16: 16 lanes read 256
+// contiguous bytes, free of bank conflicts.
 // Workgroup: WNW x WMW waves, each TNB x TMB blocks of 16: BN = 16 TNB WNW, BM = 16 TMB WMW.
 template <int N_OUTSTANDING>
 __device__ __forceinline__ void wait_vmcnt() {
@@ -389,281 +392,35 @@ __device__ __forceinline__ void wait_vmcnt() {
 }
 
 // The barrier alone: __syncthreads() would first wait for every load in flight, the later stages'
-// too, and so undo the ring. What has to have landed is waited for by wait_vmcnt before it; the
-// operand reads of the step before are in registers already (the matrix cores have used them).
+// too, and so undo the rings. What has to have landed is waited for by wait_vmcnt before it; the
+// reads of LDS issued so far are waited for here, so that their stage may be overwritten.
 __device__ __forceinline__ void workgroup_barrier() {
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
-template <int EPI, bool PACKED, int TNB, int TMB, int WNW, int WMW, int STAGES, int KS>
-__global__ void __launch_bounds__(64 * WNW * WMW)
-gemm_dma_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* __restrict__ Cv, int M, int N,
-                int K, int ldc, int m_tiles, int n_tiles) {
-    constexpr int NW = WNW * WMW;
-    constexpr int BN = 16 * TNB * WNW, BM = 16 * TMB * WMW;
-    constexpr int WBLK = BN / 16, XBLK = BM / 16, BLKS = WBLK + XBLK;   // 1 KB blocks of a stage
-    constexpr int WL = WBLK / NW, XL = XBLK / NW;                      // loads of a wave per stage
-    static_assert(WBLK % NW == 0 && XBLK % NW == 0, "blocks must divide over the waves");
-    extern __shared__ __attribute__((aligned(1024))) bf16 lds[];        // [STAGES][KS][BLKS][512]
-
-    // Workgroups go round the 8 XCDs, each with an L2 of its own: an XCD takes a run of tiles, and
-    // within it bands of 8 tiles in m are walked n first, so that the workgroups that are resident
-    // together share both their weight and their activation panels in that L2.
+// Workgroups go round the 8 XCDs, each with an L2 of its own: an XCD takes a run of tiles, and
+// within it bands of 8 tiles in m are walked n first, so that the workgroups that are resident
+// together share both their weight and their activation panels in that L2.
+__device__ __forceinline__ bool tile_of_workgroup(int m_tiles, int n_tiles, int& m_tile, int& n_tile) {
     const int total = m_tiles * n_tiles;
     const int chunk = (total + 7) / 8;
     const int id = (blockIdx.x % 8) * chunk + blockIdx.x / 8;
-    if (id >= total) return;
+    if (id >= total) return false;
     constexpr int BAND = 8;
     const int band = id / (BAND * n_tiles), in_band = id % (BAND * n_tiles);
     const int band_rows = m_tiles - band * BAND < BAND ? m_tiles - band * BAND : BAND;
-    const int n_tile = in_band / band_rows, m_tile = band * BAND + in_band % band_rows;
-    const int m0 = m_tile * BM, n0 = n_tile * BN;
+    n_tile = in_band / band_rows;
+    m_tile = band * BAND + in_band % band_rows;
+    return true;
+}
 
-    const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // uniform: LDS addresses stay scalar
-    const int r16 = lane & 15, g4 = lane >> 4;
-    const int wn = wave / WMW, wm = wave % WMW;
-    const int k32 = K / 32;              // k-steps of 32 in all
-    const int nsteps = k32 / KS;         // stages' worth of them (K is a multiple of 32 KS)
-
-    // this wave's loads: W blocks wave * WL + i, X blocks wave * XL + i
-    const bf16* wsrc[WL];
-    const bf16* xsrc[XL];
-#pragma unroll
-    for (int i = 0; i < WL; ++i) {
-        const int blk = wave * WL + i;
-        if (PACKED) {
-            int nb = n0 / 16 + blk;
-            if (nb * 16 >= N) nb = (N - 1) / 16;
-            wsrc[i] = W + ((size_t)nb * 64 + lane) * 8;
-        } else {
-            int n = n0 + blk * 16 + r16;
-            if (n >= N) n = N - 1;
-            wsrc[i] = W + (size_t)n * K + g4 * 8;
-        }
-    }
-#pragma unroll
-    for (int i = 0; i < XL; ++i) {
-        int m = m0 + (wave * XL + i) * 16 + r16;
-        if (m >= M) m = M - 1;
-        xsrc[i] = X + (size_t)m * K + g4 * 8;
-    }
-    // Stages of 64 k: the activations lie in LDS as rows of 128 bytes, so that a load fetches
-    // whole 128-byte lines (8 rows an instruction, 8 lanes a row) instead of half lines twice.
-    // The 16-byte chunk c of row r sits at chunk c ^ ((r >> 1) & 7) of its row: the operand reads
-    // of 16 rows at one k then fall into 16 different bank groups.
-    constexpr bool XROWS = KS == 2;
-    constexpr int XR = XROWS ? BM / 8 / NW : 1;                       // row loads of a wave per stage
-    static_assert(!XROWS || BM % (8 * NW) == 0, "rows must divide over the waves");
-    const bf16* xrsrc[XR];
-#pragma unroll
-    for (int i = 0; i < XR; ++i) {
-        const int r = (wave * XR + i) * 8 + (lane >> 3);
-        int m = m0 + r;
-        if (m >= M) m = M - 1;
-        xrsrc[i] = X + (size_t)m * K + (((lane & 7) ^ ((r >> 1) & 7)) * 8);
-    }
-    const size_t WSTEP = PACKED ? (size_t)(N / 16) * 512 : 32;
-
-    auto issue = [&](int step, int stage) {
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            bf16* base = lds + (XROWS ? (size_t)stage * KS * BLKS * 512 + ks * WBLK * 512
-                                      : (size_t)(stage * KS + ks) * BLKS * 512);
-            const size_t k = (size_t)step * KS + ks;
-#pragma unroll
-            for (int i = 0; i < WL; ++i)
-                __builtin_amdgcn_global_load_lds(
-                    (const __attribute__((address_space(1))) void*)(wsrc[i] + k * WSTEP),
-                    (__attribute__((address_space(3))) void*)(base + (wave * WL + i) * 512), 16, 0, 0);
-            if (!XROWS) {
-#pragma unroll
-                for (int i = 0; i < XL; ++i)
-                    __builtin_amdgcn_global_load_lds(
-                        (const __attribute__((address_space(1))) void*)(xsrc[i] + k * 32),
-                        (__attribute__((address_space(3))) void*)(base + (WBLK + wave * XL + i) * 512), 16, 0, 0);
-            }
-        }
-        if (XROWS) {
-            // the stage's activations follow the weight blocks of its two k-steps: [BM][64]
-            bf16* xbase = lds + (size_t)stage * KS * BLKS * 512 + KS * WBLK * 512;
-#pragma unroll
-            for (int i = 0; i < XR; ++i)
-                __builtin_amdgcn_global_load_lds(
-                    (const __attribute__((address_space(1))) void*)(xrsrc[i] + (size_t)step * 64),
-                    (__attribute__((address_space(3))) void*)(xbase + (wave * XR + i) * 512), 16, 0, 0);
-        }
-    };
-
-    // 32x32x16 MFMA (it has the higher rate of the two bf16 shapes): an operand is 32 rows x 16 k,
-    // lane l = row l % 32, k 8 (l / 32) .. + 8. In the 1 KB blocks of 16 rows x 32 k that is, for the
-    // k-half h: block (l % 32) / 16 of a pair of blocks, chunk 16 (2 h + l / 32) + l % 16.
-    static_assert(TNB % 2 == 0 && TMB % 2 == 0, "a wave's tile is made of 32 x 32 pieces");
-    constexpr int TN32 = TNB / 2, TM32 = TMB / 2;
-    const int c32 = lane & 31, g2 = lane >> 5;
-    const int lane_off = (c32 >> 4) * 512 + (16 * g2 + (lane & 15)) * 8;   // + 32 * 8 for the second k-half
-    f32x16 acc[TN32][TM32];
-#pragma unroll
-    for (int a = 0; a < TN32; ++a)
-#pragma unroll
-        for (int b = 0; b < TM32; ++b)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.f;
-
-    // Operands in two sets of registers: while the matrix cores work on one k-step of 32, the
-    // reads of the next one are on their way, so a wave never waits for LDS with nothing to do.
-    bf16x8 wv[2][2][TN32], xv[2][2][TM32];       // [set][k-half][piece]
-    const int x_swizzle = (c32 >> 1) & 7;           // of this lane's rows: they are c32 + a multiple of 16
-    auto read_operands = [&](int set, int stage, int ks) {
-        const bf16* base = lds + (XROWS ? (size_t)stage * KS * BLKS * 512 + ks * WBLK * 512
-                                        : (size_t)(stage * KS + ks) * BLKS * 512) + lane_off;
-        const bf16* xrows = lds + (size_t)stage * KS * BLKS * 512 + KS * WBLK * 512 +
-                            ((wm * TMB) * 16 + c32) * 64;
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-#pragma unroll
-            for (int a = 0; a < TN32; ++a)
-                wv[set][h][a] = *(const bf16x8*)(base + (wn * TNB + 2 * a) * 512 + h * 256);
-#pragma unroll
-            for (int b = 0; b < TM32; ++b) {
-                if (XROWS)
-                    xv[set][h][b] = *(const bf16x8*)(xrows + b * 32 * 64 + (((4 * ks + 2 * h + g2) ^ x_swizzle) * 8));
-                else
-                    xv[set][h][b] = *(const bf16x8*)(base + (WBLK + wm * TMB + 2 * b) * 512 + h * 256);
-            }
-        }
-    };
-    auto multiply = [&](int set) {
-#pragma unroll
-        for (int h = 0; h < 2; ++h)
-#pragma unroll
-            for (int a = 0; a < TN32; ++a)
-#pragma unroll
-                for (int b = 0; b < TM32; ++b)
-                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wv[set][h][a], xv[set][h][b], acc[a][b],
-                                                                        0, 0, 0);
-    };
-    // Before step t + 1 is read: this wave's loads of it have landed (those of the STAGES - 2 later
-    // steps may be in flight) and its reads of step t are in registers; after the barrier that
-    // holds for every wave, so the stage of step t can take the loads of step t + STAGES.
-    auto advance = [&](int t) {
-        wait_vmcnt<(STAGES - 2) * (XROWS ? WL * KS + XR : (WL + XL) * KS)>();
-        workgroup_barrier();
-        const int nt = t + STAGES;
-        issue(nt < nsteps ? nt : nsteps - 1, nt % STAGES);
-    };
-    // one step; `first` is the register set that holds its first k-step (a constant once unrolled)
-    auto run_step = [&](int first, int t) {
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            const int set = (first + ks) & 1;
-            if (ks + 1 < KS) {
-                read_operands(set ^ 1, t % STAGES, ks + 1);
-            } else if (t + 1 < nsteps) {
-                advance(t);
-                read_operands(set ^ 1, (t + 1) % STAGES, 0);
-            }
-            multiply(set);
-        }
-    };
-
-#pragma unroll
-    for (int st = 0; st < STAGES - 1; ++st) issue(st < nsteps ? st : nsteps - 1, st);
-    advance(-1);
-    read_operands(0, 0, 0);
-    if constexpr (KS == 2) {
-        // Stages of two k-steps: no branch in the loop (the last step is peeled off), and the work
-        // other than MFMAs is dealt out between them by hand: a wave then has an MFMA in the pipe
-        // while it issues its reads and loads, also right after the barrier, where the other wave
-        // of its SIMD stands at the same place and cannot fill in.
-        constexpr int NM = 2 * TN32 * TM32;              // MFMAs of a k-step
-        constexpr int NR = 2 * (TN32 + TM32);            // operand reads of a k-step
-        constexpr int ND = WL * KS + XR;                 // loads of a stage
-        constexpr int SLOTS = NM > 6 ? NM - 4 : NM;      // the last MFMAs cover the latency of the last reads
-        auto mfma_one = [&](int set, int j) {
-            const int h = j / (TN32 * TM32), a = j / TM32 % TN32, b = j % TM32;
-            acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wv[set][h][a], xv[set][h][b], acc[a][b], 0, 0, 0);
-        };
-        auto read_one = [&](int set, int stage, int ks, int idx) {
-            const int h = idx / (TN32 + TM32), r = idx % (TN32 + TM32);
-            const bf16* sbase = lds + (size_t)stage * KS * BLKS * 512;
-            if (r < TN32) {
-                wv[set][h][r] = *(const bf16x8*)(sbase + ks * WBLK * 512 + lane_off + (wn * TNB + 2 * r) * 512 + h * 256);
-            } else {
-                const int b = r - TN32;
-                xv[set][h][b] = *(const bf16x8*)(sbase + KS * WBLK * 512 + ((wm * TMB) * 16 + c32 + b * 32) * 64 +
-                                                 (((4 * ks + 2 * h + g2) ^ x_swizzle) * 8));
-            }
-        };
-        auto load_one = [&](int step, int stage, int idx) {
-            bf16* sbase = lds + (size_t)stage * KS * BLKS * 512;
-            if (idx < WL * KS) {
-                const int ks = idx / WL, i = idx % WL;
-                __builtin_amdgcn_global_load_lds(
-                    (const __attribute__((address_space(1))) void*)(wsrc[i] + ((size_t)step * KS + ks) * WSTEP),
-                    (__attribute__((address_space(3))) void*)(sbase + ks * WBLK * 512 + (wave * WL + i) * 512), 16, 0, 0);
-            } else {
-                const int i = idx - WL * KS;
-                __builtin_amdgcn_global_load_lds(
-                    (const __attribute__((address_space(1))) void*)(xrsrc[i] + (size_t)step * 64),
-                    (__attribute__((address_space(3))) void*)(sbase + KS * WBLK * 512 + (wave * XR + i) * 512), 16, 0, 0);
-            }
-        };
-        for (int t = 0; t + 1 < nsteps; ++t) {
-            const int stage = t % STAGES, next_stage = (t + 1) % STAGES;
-            // first k-step: its MFMAs, with the reads of the second k-step between them
-#pragma unroll
-            for (int j = 0; j < NM; ++j) {
-                mfma_one(0, j);
-#pragma unroll
-                for (int o = (j < SLOTS ? j : SLOTS) * NR / SLOTS; o < (j + 1 < SLOTS ? j + 1 : SLOTS) * NR / SLOTS; ++o)
-                    read_one(1, stage, 1, o);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            // second k-step: step t + 1 has landed for everyone and nobody reads this stage any more;
-            // between the MFMAs go the loads of step t + STAGES into it, then the reads of step t + 1
-            wait_vmcnt<(STAGES - 2) * ND>();
-            workgroup_barrier();
-            const int nt = t + STAGES < nsteps ? t + STAGES : nsteps - 1;
-#pragma unroll
-            for (int j = 0; j < NM; ++j) {
-                mfma_one(1, j);
-#pragma unroll
-                for (int o = (j < SLOTS ? j : SLOTS) * (ND + NR) / SLOTS;
-                     o < (j + 1 < SLOTS ? j + 1 : SLOTS) * (ND + NR) / SLOTS; ++o) {
-                    if (o < ND) load_one(nt, stage, o);
-                    else read_one(0, next_stage, 0, o - ND);
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        }
-        {
-            const int stage = (nsteps - 1) % STAGES;
-#pragma unroll
-            for (int j = 0; j < NM; ++j) {
-                mfma_one(0, j);
-#pragma unroll
-                for (int o = (j < SLOTS ? j : SLOTS) * NR / SLOTS; o < (j + 1 < SLOTS ? j + 1 : SLOTS) * NR / SLOTS; ++o)
-                    read_one(1, stage, 1, o);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            multiply(1);
-        }
-    } else if (KS % 2 == 0) {
-        for (int t = 0; t < nsteps; ++t) run_step(0, t);
-    } else {
-        for (int t = 0; t < nsteps; t += 2) {
-            run_step(0, t);
-            if (t + 1 < nsteps) run_step(1, t + 1);
-        }
-    }
-    wait_vmcnt<0>();      // the loads past the end (repeats of the last step) have landed too
-
-    // lane: m = m0 + (wm * TMB + 2 b) * 16 + c32 ; register 4 q + j of a piece:
-    // n = n0 + (wn * TNB + 2 a) * 16 + 8 q + 4 g2 + j, four consecutive n for each q
+// A wave's sums to memory. m_base, n_base: first row and column of the wave's tile.
+template <int EPI, int TN32, int TM32>
+__device__ __forceinline__ void store_wave_tile(const f32x16 (&acc)[TN32][TM32], void* Cv, int M, int N, int ldc,
+                                                int m_base, int n_base, int c32, int g2) {
 #pragma unroll
     for (int b = 0; b < TM32; ++b) {
-        const int m = m0 + (wm * TMB + 2 * b) * 16 + c32;
+        const int m = m_base + 32 * b + c32;
         if (m >= M) continue;
         if (EPI == EPI_SWIGLU) {
             bf16* C = (bf16*)Cv;
@@ -671,8 +428,8 @@ gemm_dma_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* __
             for (int a = 0; a < TN32; ++a)
 #pragma unroll
                 for (int q = 0; q < 2; ++q) {
-                    // rows 0..15 of the piece are gate rows, 16..31 the up rows of the same outputs
-                    const int n = (n0 + (wn * TNB + 2 * a) * 16) / 2 + 8 * q + 4 * g2;
+                    // rows 0..15 of a piece are gate rows, 16..31 the up rows of the same outputs
+                    const int n = (n_base + 32 * a) / 2 + 8 * q + 4 * g2;
                     if (n + 3 < N / 2 && (ldc & 3) == 0) {
                         bf16x4 v;
 #pragma unroll
@@ -693,7 +450,7 @@ gemm_dma_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* __
             for (int a = 0; a < TN32; ++a)
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
-                    const int n = n0 + (wn * TNB + 2 * a) * 16 + 8 * q + 4 * g2;
+                    const int n = n_base + 32 * a + 8 * q + 4 * g2;
                     float* dst = C + (size_t)m * ldc + n;
                     if (n + 3 < N && (ldc & 3) == 0) {
                         f32x4 v = {acc[a][b][4 * q], acc[a][b][4 * q + 1], acc[a][b][4 * q + 2],
@@ -715,46 +472,373 @@ gemm_dma_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* __
     }
 }
 
-template <int TNB, int TMB, int WNW, int WMW, int STAGES, int KS>
-static int launch_dma(const void* X, const void* W, void* C, int M, int N, int K, int ldc, int epi, int packed,
-                      hipStream_t stream) {
+// K in steps of 64. A step's weights are two k-steps of 32 (blocks as above); its activations lie
+// in LDS as rows of 128 bytes, so that a load fetches whole 128-byte lines (8 rows an
+// instruction, 8 lanes a row) and not half lines twice; the 16-byte chunk c of row r sits at
+// chunk c ^ ((r >> 1) & 7) of its row, so that the operand reads of 16 rows at one k fall into
+// 16 different bank groups. The weights, which come from HBM, have a ring of WST stages; the
+// activations, which the L2 holds, one of 2.
+// There is no branch in the main loop (the last step is peeled off), and what is no MFMA is
+// dealt out between the MFMAs by hand: a wave has an MFMA in the pipe while it issues its reads
+// and loads, also right after the barrier, where no other wave could fill in. Operands are in
+// two sets of registers: the reads of a k-step go out during the MFMAs of the one before.
+template <int EPI, bool PACKED, int TNB, int TMB, int WNW, int WMW, int WST>
+__global__ void __launch_bounds__(64 * WNW * WMW)
+gemm_tile_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* __restrict__ Cv, int M, int N,
+                 int K, int ldc, int m_tiles, int n_tiles) {
+    constexpr int NW = WNW * WMW;
+    constexpr int BN = 16 * TNB * WNW, BM = 16 * TMB * WMW;
+    constexpr int WBLK = BN / 16;                       // weight blocks of a k-step of 32
+    constexpr int WL = WBLK / NW;                       // of which a wave loads
+    constexpr int XR = BM / 8 / NW;                     // loads of 8 activation rows of a wave per step
+    constexpr int W_STAGE = 2 * WBLK * 512, X_STAGE = BM * 64;      // elements
+    constexpr int NLW = 2 * WL, NLX = XR;               // a wave's loads per step
+    static_assert(WBLK % NW == 0 && BM % (8 * NW) == 0, "the loads must divide over the waves");
+    static_assert(TNB % 2 == 0 && TMB % 2 == 0, "a wave's tile is made of 32 x 32 pieces");
+    static_assert(WST == 2 || WST == 3, "the wait before the barrier counts on the loads of at most one later step");
+    constexpr int TN32 = TNB / 2, TM32 = TMB / 2;
+    extern __shared__ __attribute__((aligned(1024))) bf16 lds[];    // [WST][W_STAGE], then [2][X_STAGE]
+    bf16* const xlds = lds + WST * W_STAGE;
+
+    int m_tile, n_tile;
+    if (!tile_of_workgroup(m_tiles, n_tiles, m_tile, n_tile)) return;
+    const int m0 = m_tile * BM, n0 = n_tile * BN;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // uniform: LDS addresses stay scalar
+    const int r16 = lane & 15, g4 = lane >> 4, c32 = lane & 31, g2 = lane >> 5;
+    const int wn = wave / WMW, wm = wave % WMW;
+    const int nsteps = K / 64;
+
+    const bf16* wsrc[WL];
+#pragma unroll
+    for (int i = 0; i < WL; ++i) {
+        const int blk = wave * WL + i;
+        if (PACKED) {
+            int nb = n0 / 16 + blk;
+            if (nb * 16 >= N) nb = (N - 1) / 16;
+            wsrc[i] = W + ((size_t)nb * 64 + lane) * 8;
+        } else {
+            int n = n0 + blk * 16 + r16;
+            if (n >= N) n = N - 1;                      // rows past the end repeat the last one; never stored
+            wsrc[i] = W + (size_t)n * K + g4 * 8;
+        }
+    }
+    const size_t WSTEP = PACKED ? (size_t)(N / 16) * 512 : 32;      // elements between two k-steps of 32
+    const bf16* xsrc[XR];
+#pragma unroll
+    for (int i = 0; i < XR; ++i) {
+        const int r = (wave * XR + i) * 8 + (lane >> 3);
+        int m = m0 + r;
+        if (m >= M) m = M - 1;
+        xsrc[i] = X + (size_t)m * K + (((lane & 7) ^ ((r >> 1) & 7)) * 8);
+    }
+    // loads of a step, the activations first: those are waited for one step earlier than the weights
+    auto load_one = [&](int xstep, int wstep, int idx) {
+        if (idx < NLX) {
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void*)(xsrc[idx] + (size_t)xstep * 64),
+                (__attribute__((address_space(3))) void*)(xlds + (xstep & 1) * X_STAGE + (wave * XR + idx) * 512),
+                16, 0, 0);
+        } else {
+            const int ks = (idx - NLX) / WL, i = (idx - NLX) % WL;
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void*)(wsrc[i] + ((size_t)wstep * 2 + ks) * WSTEP),
+                (__attribute__((address_space(3))) void*)(lds + (wstep % WST) * W_STAGE + ks * WBLK * 512 +
+                                                          (wave * WL + i) * 512),
+                16, 0, 0);
+        }
+    };
+
+    f32x16 acc[TN32][TM32];
+#pragma unroll
+    for (int a = 0; a < TN32; ++a)
+#pragma unroll
+        for (int b = 0; b < TM32; ++b)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.f;
+
+    constexpr int NM = 2 * TN32 * TM32;              // MFMAs of a k-step of 32
+    constexpr int NR = 2 * (TN32 + TM32);            // operand reads of a k-step
+    constexpr int SLOTS = NM > 6 ? NM - 4 : NM;      // the last MFMAs cover the latency of the last reads
+    const int w_lane = (c32 >> 4) * 512 + (16 * g2 + (lane & 15)) * 8 + wn * TNB * 512;
+    const int x_lane = (wm * TMB * 16 + c32) * 64;
+    const int x_swizzle = (c32 >> 1) & 7;            // of this lane's rows: they are c32 + a multiple of 16
+    bf16x8 wv[2][2][TN32], xv[2][2][TM32];           // [set][k-half][piece]
+    auto mfma_one = [&](int set, int j) {
+        const int h = j / (TN32 * TM32), a = j / TM32 % TN32, b = j % TM32;
+        acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wv[set][h][a], xv[set][h][b], acc[a][b], 0, 0, 0);
+    };
+    auto read_one = [&](int set, int step, int ks, int idx) {
+        const int h = idx / (TN32 + TM32), r = idx % (TN32 + TM32);
+        if (r < TN32)
+            wv[set][h][r] = *(const bf16x8*)(lds + (step % WST) * W_STAGE + ks * WBLK * 512 + w_lane + r * 1024 + h * 256);
+        else
+            xv[set][h][r - TN32] = *(const bf16x8*)(xlds + (step & 1) * X_STAGE + x_lane + (r - TN32) * 32 * 64 +
+                                                    (((4 * ks + 2 * h + g2) ^ x_swizzle) * 8));
+    };
+    // between the MFMAs j and j + 1 of a k-step: nl loads and NR reads, dealt out evenly over the
+    // first SLOTS MFMAs, the loads spread among the reads (a burst of loads from all waves at
+    // once backs up the memory pipeline and holds the waves at their issue)
+    auto between = [&](int j, int nl, auto&& load, auto&& read) {
+        const int no = nl + NR;
+        const int from = (j < SLOTS ? j : SLOTS) * no / SLOTS, to = (j + 1 < SLOTS ? j + 1 : SLOTS) * no / SLOTS;
+#pragma unroll
+        for (int o = from; o < to; ++o) {
+            const int loads_before = o * nl / no, loads_after = (o + 1) * nl / no;
+            if (loads_after > loads_before) load(loads_before);
+            else read(o - loads_before);
+        }
+    };
+    auto clamp = [&](int step) { return step < nsteps ? step : nsteps - 1; };   // past the end: the last step again
+
+    // in flight before the loop: activations of steps 0 and 1, weights of steps 0 .. WST - 1
+#pragma unroll
+    for (int i = 0; i < NLX + NLW; ++i) load_one(0, 0, i);
+#pragma unroll
+    for (int i = 0; i < NLX + NLW; ++i) load_one(clamp(1), clamp(1), i);
+#pragma unroll
+    for (int st = 2; st < WST; ++st)
+#pragma unroll
+        for (int i = NLX; i < NLX + NLW; ++i) load_one(0, clamp(st), i);
+    wait_vmcnt<NLX + (WST - 1) * NLW>();
+    workgroup_barrier();
+#pragma unroll
+    for (int i = 0; i < NR; ++i) read_one(0, 0, 0, i);
+
+    for (int t = 0; t + 1 < nsteps; ++t) {
+        // first k-step of step t; between its MFMAs the reads of the second one
+#pragma unroll
+        for (int j = 0; j < NM; ++j) {
+            mfma_one(0, j);
+            between(j, 0, [&](int) {}, [&](int i) { read_one(1, t, 1, i); });
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // Step t + 1 has landed (of what this wave has in flight only the weights of the later
+        // steps may be missing), after the barrier for every wave, and nobody reads step t any
+        // more: between the MFMAs of its second k-step go the loads into its stages, the
+        // activations of step t + 2 and the weights of step t + WST, and the reads of step t + 1.
+        wait_vmcnt<(WST - 2) * NLW>();
+        workgroup_barrier();
+        const int xstep = clamp(t + 2), wstep = clamp(t + WST);
+#pragma unroll
+        for (int j = 0; j < NM; ++j) {
+            mfma_one(1, j);
+            between(j, NLX + NLW,
+                    [&](int i) {
+                        // a clamped step goes where step t + 2 (t + WST) would: into the stage just freed
+                        if (i < NLX) {
+                            __builtin_amdgcn_global_load_lds(
+                                (const __attribute__((address_space(1))) void*)(xsrc[i] + (size_t)xstep * 64),
+                                (__attribute__((address_space(3))) void*)(xlds + (t & 1) * X_STAGE + (wave * XR + i) * 512),
+                                16, 0, 0);
+                        } else {
+                            const int ks = (i - NLX) / WL, w = (i - NLX) % WL;
+                            __builtin_amdgcn_global_load_lds(
+                                (const __attribute__((address_space(1))) void*)(wsrc[w] + ((size_t)wstep * 2 + ks) * WSTEP),
+                                (__attribute__((address_space(3))) void*)(lds + (t % WST) * W_STAGE + ks * WBLK * 512 +
+                                                                          (wave * WL + w) * 512),
+                                16, 0, 0);
+                        }
+                    },
+                    [&](int i) { read_one(0, t + 1, 0, i); });
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    {
+        const int t = nsteps - 1;
+#pragma unroll
+        for (int j = 0; j < NM; ++j) {
+            mfma_one(0, j);
+            between(j, 0, [&](int) {}, [&](int i) { read_one(1, t, 1, i); });
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int j = 0; j < NM; ++j) mfma_one(1, j);
+    }
+    wait_vmcnt<0>();      // the loads past the end (repeats of the last step) have landed too
+    store_wave_tile<EPI, TN32, TM32>(acc, Cv, M, N, ldc, m0 + wm * TMB * 16, n0 + wn * TNB * 16, c32, g2);
+}
+
+// K in steps of 32 only: one k-step a stage, everything in 1 KB blocks (the activations too: a
+// block of 16 rows x 32 k is loaded as 16 half lines), a ring of STAGES stages loaded STAGES - 1
+// steps ahead, the plain order read / multiply with the operands in two sets of registers.
+template <int EPI, bool PACKED, int TNB, int TMB, int WNW, int WMW, int STAGES>
+__global__ void __launch_bounds__(64 * WNW * WMW)
+gemm_tile32_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* __restrict__ Cv, int M, int N,
+                   int K, int ldc, int m_tiles, int n_tiles) {
+    constexpr int NW = WNW * WMW;
+    constexpr int BN = 16 * TNB * WNW, BM = 16 * TMB * WMW;
+    constexpr int WBLK = BN / 16, XBLK = BM / 16, BLKS = WBLK + XBLK;   // 1 KB blocks of a stage
+    constexpr int WL = WBLK / NW, XL = XBLK / NW;                      // loads of a wave per stage
+    static_assert(WBLK % NW == 0 && XBLK % NW == 0, "blocks must divide over the waves");
+    static_assert(TNB % 2 == 0 && TMB % 2 == 0, "a wave's tile is made of 32 x 32 pieces");
+    constexpr int TN32 = TNB / 2, TM32 = TMB / 2;
+    extern __shared__ __attribute__((aligned(1024))) bf16 lds[];        // [STAGES][BLKS][512]
+
+    int m_tile, n_tile;
+    if (!tile_of_workgroup(m_tiles, n_tiles, m_tile, n_tile)) return;
+    const int m0 = m_tile * BM, n0 = n_tile * BN;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r16 = lane & 15, g4 = lane >> 4, c32 = lane & 31, g2 = lane >> 5;
+    const int wn = wave / WMW, wm = wave % WMW;
+    const int nsteps = K / 32;
+
+    const bf16* wsrc[WL];
+    const bf16* xsrc[XL];
+#pragma unroll
+    for (int i = 0; i < WL; ++i) {
+        const int blk = wave * WL + i;
+        if (PACKED) {
+            int nb = n0 / 16 + blk;
+            if (nb * 16 >= N) nb = (N - 1) / 16;
+            wsrc[i] = W + ((size_t)nb * 64 + lane) * 8;
+        } else {
+            int n = n0 + blk * 16 + r16;
+            if (n >= N) n = N - 1;
+            wsrc[i] = W + (size_t)n * K + g4 * 8;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < XL; ++i) {
+        int m = m0 + (wave * XL + i) * 16 + r16;
+        if (m >= M) m = M - 1;
+        xsrc[i] = X + (size_t)m * K + g4 * 8;
+    }
+    const size_t WSTEP = PACKED ? (size_t)(N / 16) * 512 : 32;
+    auto issue = [&](int step, int stage) {
+        bf16* base = lds + (size_t)stage * BLKS * 512;
+#pragma unroll
+        for (int i = 0; i < WL; ++i)
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void*)(wsrc[i] + (size_t)step * WSTEP),
+                (__attribute__((address_space(3))) void*)(base + (wave * WL + i) * 512), 16, 0, 0);
+#pragma unroll
+        for (int i = 0; i < XL; ++i)
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void*)(xsrc[i] + (size_t)step * 32),
+                (__attribute__((address_space(3))) void*)(base + (WBLK + wave * XL + i) * 512), 16, 0, 0);
+    };
+
+    f32x16 acc[TN32][TM32];
+#pragma unroll
+    for (int a = 0; a < TN32; ++a)
+#pragma unroll
+        for (int b = 0; b < TM32; ++b)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.f;
+
+    const int lane_off = (c32 >> 4) * 512 + (16 * g2 + (lane & 15)) * 8;   // + 32 * 8 for the second k-half
+    bf16x8 wv[2][2][TN32], xv[2][2][TM32];       // [set][k-half][piece]
+    auto read_operands = [&](int set, int stage) {
+        const bf16* base = lds + (size_t)stage * BLKS * 512 + lane_off;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+#pragma unroll
+            for (int a = 0; a < TN32; ++a)
+                wv[set][h][a] = *(const bf16x8*)(base + (wn * TNB + 2 * a) * 512 + h * 256);
+#pragma unroll
+            for (int b = 0; b < TM32; ++b)
+                xv[set][h][b] = *(const bf16x8*)(base + (WBLK + wm * TMB + 2 * b) * 512 + h * 256);
+        }
+    };
+    auto multiply = [&](int set) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int a = 0; a < TN32; ++a)
+#pragma unroll
+                for (int b = 0; b < TM32; ++b)
+                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wv[set][h][a], xv[set][h][b], acc[a][b],
+                                                                        0, 0, 0);
+    };
+    // Before step t + 1 is read: this wave's loads of it have landed (those of the STAGES - 2 later
+    // steps may be in flight) and its reads of step t are in registers; after the barrier that
+    // holds for every wave, so the stage of step t can take the loads of step t + STAGES.
+    auto advance = [&](int t) {
+        wait_vmcnt<(STAGES - 2) * (WL + XL)>();
+        workgroup_barrier();
+        const int nt = t + STAGES;
+        issue(nt < nsteps ? nt : nsteps - 1, nt % STAGES);
+    };
+    auto run_step = [&](int set, int t) {
+        if (t + 1 < nsteps) {
+            advance(t);
+            read_operands(set ^ 1, (t + 1) % STAGES);
+        }
+        multiply(set);
+    };
+#pragma unroll
+    for (int st = 0; st < STAGES - 1; ++st) issue(st < nsteps ? st : nsteps - 1, st);
+    advance(-1);
+    read_operands(0, 0);
+    for (int t = 0; t < nsteps; t += 2) {
+        run_step(0, t);
+        if (t + 1 < nsteps) run_step(1, t + 1);
+    }
+    wait_vmcnt<0>();      // the loads past the end (repeats of the last step) have landed too
+    store_wave_tile<EPI, TN32, TM32>(acc, Cv, M, N, ldc, m0 + wm * TMB * 16, n0 + wn * TNB * 16, c32, g2);
+}
+
+template <class Kernel>
+static int launch_tiles(Kernel kern, size_t lds, int threads, long total, const bf16* x, const bf16* w, void* C,
+                        int M, int N, int K, int ldc, int m_tiles, int n_tiles, hipStream_t stream) {
+    HB_REQUIRE(total < (1l << 30), "gemm_mfma: too many tiles");
+    HB_REQUIRE(lds <= 160 * 1024, "gemm_mfma: %zu bytes of LDS asked for", lds);
+    if (lds > 64 * 1024) {
+        // once per kernel (this function is instantiated per kernel type)
+        static bool raised = false;
+        if (!raised) {
+            hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            HB_REQUIRE(e == hipSuccess, "gemm_mfma: cannot have %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+            raised = true;
+        }
+    }
+    const int blocks = (int)((total + 7) / 8 * 8);
+    kern<<<blocks, threads, lds, stream>>>(x, w, C, M, N, K, ldc, m_tiles, n_tiles);
+    HB_CHECK_LAUNCH("gemm_tile");
+    return 0;
+}
+
+#define TILE_DISPATCH(KERNEL, ...)                                                                   \
+    do {                                                                                             \
+        if (packed) {                                                                                \
+            if (epi == EPI_STORE) return launch_tiles(KERNEL<EPI_STORE, true, __VA_ARGS__>, lds, threads, total, x, w, C, M, N, K, ldc, m_tiles, n_tiles, stream); \
+            if (epi == EPI_ADD) return launch_tiles(KERNEL<EPI_ADD, true, __VA_ARGS__>, lds, threads, total, x, w, C, M, N, K, ldc, m_tiles, n_tiles, stream); \
+            return launch_tiles(KERNEL<EPI_SWIGLU, true, __VA_ARGS__>, lds, threads, total, x, w, C, M, N, K, ldc, m_tiles, n_tiles, stream); \
+        }                                                                                            \
+        if (epi == EPI_STORE) return launch_tiles(KERNEL<EPI_STORE, false, __VA_ARGS__>, lds, threads, total, x, w, C, M, N, K, ldc, m_tiles, n_tiles, stream); \
+        if (epi == EPI_ADD) return launch_tiles(KERNEL<EPI_ADD, false, __VA_ARGS__>, lds, threads, total, x, w, C, M, N, K, ldc, m_tiles, n_tiles, stream); \
+        return launch_tiles(KERNEL<EPI_SWIGLU, false, __VA_ARGS__>, lds, threads, total, x, w, C, M, N, K, ldc, m_tiles, n_tiles, stream); \
+    } while (0)
+
+template <int TNB, int TMB, int WNW, int WMW, int WST>
+static int launch_tile64(const void* X, const void* W, void* C, int M, int N, int K, int ldc, int epi, int packed,
+                         hipStream_t stream) {
+    constexpr int BN = 16 * TNB * WNW, BM = 16 * TMB * WMW;
+    HB_REQUIRE(K % 64 == 0, "gemm_mfma: K=%d is no multiple of 64", K);
+    const int m_tiles = (M + BM - 1) / BM, n_tiles = (N + BN - 1) / BN;
+    const long total = (long)m_tiles * n_tiles;
+    const size_t lds = (size_t)(WST * BN + 2 * BM) * 64 * sizeof(bf16);
+    const int threads = 64 * WNW * WMW;
+    const bf16* x = (const bf16*)X;
+    const bf16* w = (const bf16*)W;
+    TILE_DISPATCH(gemm_tile_kernel, TNB, TMB, WNW, WMW, WST);
+}
+
+template <int TNB, int TMB, int WNW, int WMW, int STAGES>
+static int launch_tile32(const void* X, const void* W, void* C, int M, int N, int K, int ldc, int epi, int packed,
+                         hipStream_t stream) {
     constexpr int BN = 16 * TNB * WNW, BM = 16 * TMB * WMW;
     const int m_tiles = (M + BM - 1) / BM, n_tiles = (N + BN - 1) / BN;
     const long total = (long)m_tiles * n_tiles;
-    HB_REQUIRE(total < (1l << 30), "gemm_mfma: too many tiles");
-    const int blocks = (int)((total + 7) / 8 * 8);
-    HB_REQUIRE(K % (32 * KS) == 0, "gemm_mfma: K=%d is no multiple of %d", K, 32 * KS);
-    const size_t lds = (size_t)STAGES * KS * (BN + BM) / 16 * 1024;
+    const size_t lds = (size_t)STAGES * (BN + BM) * 32 * sizeof(bf16);
+    const int threads = 64 * WNW * WMW;
     const bf16* x = (const bf16*)X;
     const bf16* w = (const bf16*)W;
-#define DMA_GO(EPIV, PK)                                                                            \
-    do {                                                                                            \
-        auto kern = gemm_dma_kernel<EPIV, PK, TNB, TMB, WNW, WMW, STAGES, KS>;                          \
-        if (lds > 64 * 1024) {                                                                      \
-            static bool raised = false;                                                             \
-            if (!raised) {                                                                          \
-                hipError_t e = hipFuncSetAttribute((const void*)kern,                               \
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
-                HB_REQUIRE(e == hipSuccess, "gemm_mfma: cannot have %zu bytes of LDS: %s", lds,     \
-                           hipGetErrorString(e));                                                   \
-                raised = true;                                                                      \
-            }                                                                                       \
-        }                                                                                           \
-        kern<<<blocks, 64 * WNW * WMW, lds, stream>>>(x, w, C, M, N, K, ldc, m_tiles, n_tiles);     \
-    } while (0)
-    if (packed) {
-        if (epi == EPI_STORE) DMA_GO(EPI_STORE, true);
-        else if (epi == EPI_ADD) DMA_GO(EPI_ADD, true);
-        else DMA_GO(EPI_SWIGLU, true);
-    } else {
-        if (epi == EPI_STORE) DMA_GO(EPI_STORE, false);
-        else if (epi == EPI_ADD) DMA_GO(EPI_ADD, false);
-        else DMA_GO(EPI_SWIGLU, false);
-    }
-#undef DMA_GO
-    HB_CHECK_LAUNCH("gemm_dma");
-    return 0;
+    TILE_DISPATCH(gemm_tile32_kernel, TNB, TMB, WNW, WMW, STAGES);
 }
+#undef TILE_DISPATCH
 
 // C (+)= X @ W^T. X [M, K] bf16, W [N, K] bf16. epi 0: C f32 [M, N] stored; 1: added to;
 // 2: W's rows are gate/up interleaved in blocks of 16 and C is bf16 [M, N / 2] = silu(gate) * up.
@@ -784,18 +868,35 @@ extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N,
         return 0;
     }
     // tile_hint: 0 = choose (otherwise a variant by number, for measurements and tests).
-    // 256 x 256 tiles do the most arithmetic per byte moved, but one fits a CU at a time: they pay
-    // when there are enough of them for most of the 256 CUs; otherwise 128 x 128, two to a CU.
+    // The bigger the tile, the more arithmetic per byte moved and the higher its rate, but the
+    // fewer tiles there are for the 256 CUs: take the variant with the least estimated time,
+    // rounds of tiles over the CUs x the time of a tile at the rate measured for the variant.
     int tile = tile_hint;
     if (tile == 0) {
-        const long big = (long)((M + 255) / 256) * ((N + 255) / 256);
-        tile = K % 64 ? 123 : (big >= 192 ? 185 : 122);
+        if (K % 64) {
+            tile = 123;
+        } else {
+            struct Variant { int id, bn, bm, per_cu; double rate; };
+            static const Variant variants[] = {{188, 256, 256, 1, 1.27}, {142, 256, 128, 1, 1.10}, {122, 128, 128, 2, 1.00}};
+            double best = 0;
+            for (const Variant& v : variants) {
+                const long tiles = (long)((M + v.bm - 1) / v.bm) * ((N + v.bn - 1) / v.bn);
+                const long rounds = (tiles + 256 * v.per_cu - 1) / (256 * v.per_cu);
+                const double cost = (double)rounds * v.per_cu * v.bn * v.bm / v.rate;
+                if (tile == 0 || cost < best) {
+                    tile = v.id;
+                    best = cost;
+                }
+            }
+        }
     }
     switch (tile) {
-        case 185: return launch_dma<8, 4, 2, 4, 2, 2>(X, W, C, M, N, K, ldc, epi, packed, stream);   // 256 x 256, 2 stages of 64 k
-        case 122: return launch_dma<4, 4, 2, 2, 2, 2>(X, W, C, M, N, K, ldc, epi, packed, stream);   // 128 x 128, 2 stages of 64 k
-        case 123: return launch_dma<4, 4, 2, 2, 4, 1>(X, W, C, M, N, K, ldc, epi, packed, stream);   // 128 x 128, 4 stages of 32 k
-        case 188: return launch_dma<8, 8, 2, 2, 2, 2>(X, W, C, M, N, K, ldc, epi, packed, stream);   // 256 x 256, 4 waves
+        // (a third weight stage, measured with weights that come from HBM: a gain of a tenth for
+        // 256 x 128, none for the other two)
+        case 188: return launch_tile64<8, 8, 2, 2, 2>(X, W, C, M, N, K, ldc, epi, packed, stream);   // 256 x 256
+        case 142: return launch_tile64<8, 4, 2, 2, 3>(X, W, C, M, N, K, ldc, epi, packed, stream);   // 256 (n) x 128 (m)
+        case 122: return launch_tile64<4, 4, 2, 2, 2>(X, W, C, M, N, K, ldc, epi, packed, stream);   // 128 x 128, two to a CU
+        case 123: return launch_tile32<4, 4, 2, 2, 4>(X, W, C, M, N, K, ldc, epi, packed, stream);   // 128 x 128, K in steps of 32
         default: HB_REQUIRE(false, "gemm_mfma: unknown tile %d", tile);
     }
     return 0;
