@@ -43,7 +43,13 @@ __device__ __forceinline__ int acc_key(int kb, int g2, int i) { return kb * 32 +
 
 // One page of scores: mask, online-softmax update, P^T as MFMA operands.
 // st[kb]: S^T accumulators (raw dot products). c = scale * log2(e).
-// Keys k with lo <= page0 + k <= hi are visible.
+// Keys k with lo <= page0 + k <= hi are visible; MASKED = false: the caller knows that all are.
+// m is the reference of the exponents, not always the maximum: it is moved up (and the sums so
+// far scaled by corr < 1) only when a score exceeds it by more than 8 / c, that is when a
+// probability would exceed 2^8 times the largest so far; till then corr is 1 and the caller
+// need not touch its sums. Any reference gives the same quotient in the end.
+#define RESCALE_LOG2 8.0f
+template <bool MASKED>
 __device__ __forceinline__ void softmax_page(f32x16 st[2], int g2, int page0, int lo, int hi, float c,
                                              float& m, float& l, float& corr, bf16x8 pb[2][2]) {
     float mx = -INFINITY;
@@ -51,48 +57,77 @@ __device__ __forceinline__ void softmax_page(f32x16 st[2], int g2, int page0, in
     for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            const int key = page0 + acc_key(kb, g2, i);
-            const float s = (key >= lo && key <= hi) ? st[kb][i] : -INFINITY;
-            st[kb][i] = s;
-            mx = fmaxf(mx, s);
+            if (MASKED) {
+                const int key = page0 + acc_key(kb, g2, i);
+                st[kb][i] = (key >= lo && key <= hi) ? st[kb][i] : -INFINITY;
+            }
+            mx = fmaxf(mx, st[kb][i]);
         }
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float m_new = fmaxf(m, mx);
-    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-    corr = fast_exp2((m - m_use) * c);        // m = -inf: 0
+    corr = 1.0f;
+    if ((mx - m) * c > RESCALE_LOG2 || m == -INFINITY) {       // (-inf) - (-inf) is NaN: compares false
+        const float m_new = (mx == -INFINITY) ? m : mx;
+        corr = (m == -INFINITY) ? 0.f : fast_exp2((m - m_new) * c);
+        m = m_new;
+    }
+    const float mc = (m == -INFINITY) ? 0.f : m * c;
     float sum = 0.f;
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            const float p = fast_exp2((st[kb][i] - m_use) * c);
+            const float p = fast_exp2(fmaf(st[kb][i], c, -mc));
             sum += p;
             pb[kb][i >> 3][i & 7] = (__bf16)p;
         }
     l = l * corr + sum;      // this lane's keys only; the two halves are added at the end
-    m = m_new;
+}
+
+// oacc *= corr, unless corr is 1 in every lane
+template <int NACC>
+__device__ __forceinline__ void rescale(f32x16 (&oacc)[NACC], float corr) {
+    if (__builtin_amdgcn_ballot_w64(corr != 1.0f) == 0) return;
+#pragma unroll
+    for (int d = 0; d < NACC; ++d)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) oacc[d][i] *= corr;
 }
 
 // ----------------------------------------------------------------- prefill
+// A workgroup: 32 queries x up to 4 query heads of one kv head (a wave a head). The pages go
+// from global memory straight into a ring of two LDS stages, the next page's loads in flight
+// while this page is worked on. Rows lie unpadded; the 16-byte chunk c of row r sits at chunk
+// c ^ (r / rows in 256 bytes), so that the operand reads of 16 rows at one chunk fall into 16
+// different bank groups.
+// Workgroups are numbered by falling work (the host sorts the tiles) and every other round of
+// 256 backwards: with one round per CU the heaviest tiles then share a CU with the lightest.
 template <int HD>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256, 2)
 attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache,
                     const bf16* __restrict__ v_cache, bf16* __restrict__ out,
                     const int* __restrict__ tile_seq, const int* __restrict__ tile_row0,
                     const int* __restrict__ tile_rows, const int* __restrict__ positions,
                     const int* __restrict__ slots, const int* __restrict__ page_table, int max_pages, int nq,
-                    int nkv, float c, int window) {
-    constexpr int KLD = HD + 8;      // padded rows: 16-byte reads of 32 rows fall on distinct banks
-    constexpr int VLD = PAGE + 8;
-    __shared__ __attribute__((aligned(16))) bf16 Ks[PAGE * KLD];
-    __shared__ __attribute__((aligned(16))) bf16 Vs[HD * VLD];
+                    int nkv, float c, int window, int per_tile, int total) {
+    constexpr int KCH = HD / 8;                   // 16-byte chunks of a key row
+    constexpr int KRPB = 128 / HD > 0 ? 128 / HD : 1;   // key rows in 256 bytes
+    constexpr int KROWS = 512 / HD;               // key rows a load instruction brings (1 KB)
+    constexpr int LOADS = HD / 32;                // a wave's load instructions for the keys of a page; as many for the values
+    __shared__ __attribute__((aligned(1024))) bf16 Ks[2][PAGE * HD];
+    __shared__ __attribute__((aligned(1024))) bf16 Vs[2][HD * PAGE];
 
-    const int tile = blockIdx.x;
+    int w = blockIdx.x;
+    {
+        const int round = w / 256, base = round * 256;
+        const int count = total - base < 256 ? total - base : 256;
+        if (round & 1) w = base + count - 1 - (w - base);
+    }
+    const int tile = w / per_tile, y = w % per_tile;
     const int G = nq / nkv;
     const int chunks = (G + 3) / 4;
-    const int kvh = blockIdx.y / chunks;
-    const int chunk = blockIdx.y % chunks;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int kvh = y / chunks;
+    const int chunk = y % chunks;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int c32 = lane & 31, g2 = lane >> 5;
     const int head_in_group = chunk * 4 + wave;
     const bool active = head_in_group < G;
@@ -108,6 +143,33 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache
     const int lo_q = (window > 0 && pos_q + 1 > window) ? pos_q + 1 - window : 0;
     const int hi_tile = pos0 + rows - 1;                                     // last visible key
     const int lo_tile = (window > 0 && pos0 + 1 > window) ? pos0 + 1 - window : 0;
+    const int first_page = lo_tile / PAGE, last_page = hi_tile / PAGE;
+
+    // this lane's part of the loads of a page: element offsets within the page's keys and values
+    int k_off[LOADS], v_off[LOADS];
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) {
+        const int instr = wave * LOADS + i;
+        const int kr = instr * KROWS + lane / KCH;
+        k_off[i] = kr * HD + (((lane % KCH) ^ ((kr / KRPB) % KCH)) * 8);
+        const int vr = instr * 8 + lane / 8;
+        v_off[i] = vr * PAGE + (((lane & 7) ^ ((vr >> 1) & 7)) * 8);
+    }
+    auto issue_keys = [&](int page_idx, int stage) {
+        const bf16* kp = k_cache + ((size_t)pt[page_idx] * nkv + kvh) * PAGE * HD;
+#pragma unroll
+        for (int i = 0; i < LOADS; ++i) hb_load_to_lds(kp + k_off[i], &Ks[stage][(wave * LOADS + i) * 512]);
+    };
+    auto issue_values = [&](int page_idx, int stage) {
+        const bf16* vp = v_cache + ((size_t)pt[page_idx] * nkv + kvh) * HD * PAGE;
+#pragma unroll
+        for (int i = 0; i < LOADS; ++i) hb_load_to_lds(vp + v_off[i], &Vs[stage][(wave * LOADS + i) * 512]);
+    };
+    // The keys run one page ahead of the values: the scores of page p + 1 are on the matrix cores
+    // while the softmax of page p runs on the vector units.
+    issue_keys(first_page, 0);
+    issue_values(first_page, 0);
+    if (first_page < last_page) issue_keys(first_page + 1, 1);
 
     bf16x8 qreg[HD / 16];
     {
@@ -124,48 +186,64 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache
     float m = -INFINITY, l = 0.f;
 
     const int krow = perm(c32);
-    for (int page_idx = lo_tile / PAGE; page_idx <= hi_tile / PAGE; ++page_idx) {
-        const int page = pt[page_idx];
-        const bf16* kp = k_cache + ((size_t)page * nkv + kvh) * PAGE * HD;
-        const bf16* vp = v_cache + ((size_t)page * nkv + kvh) * HD * PAGE;
-        __syncthreads();      // the previous page has been read by every wave
+    int k_read[2];
 #pragma unroll
-        for (int cidx = tid; cidx < PAGE * HD / 8; cidx += 256) {
-            const int kr = cidx / (HD / 8), kc = cidx % (HD / 8);
-            *(bf16x8*)(&Ks[kr * KLD + kc * 8]) = *(const bf16x8*)(kp + (size_t)cidx * 8);
-            const int vr = cidx / (PAGE / 8), vc = cidx % (PAGE / 8);
-            *(bf16x8*)(&Vs[vr * VLD + vc * 8]) = *(const bf16x8*)(vp + (size_t)cidx * 8);
-        }
-        __syncthreads();
-        if (!active) continue;
-
-        f32x16 st[2];
+    for (int kb = 0; kb < 2; ++kb) k_read[kb] = ((kb * 32 + krow) / KRPB) % KCH;
+    const int v_swz = (c32 >> 1) & 7;            // of rows d * 32 + c32
+    // raw scores of the page in a key stage; the two key blocks alternate, so that no MFMA waits
+    // for the one before it
+    auto scores = [&](int stage, f32x16 (&st)[2]) {
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
+        for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
             for (int i = 0; i < 16; ++i) st[kb][i] = 0.f;
-            const bf16* krowp = &Ks[(kb * 32 + krow) * KLD + g2 * 8];
 #pragma unroll
-            for (int s = 0; s < HD / 16; ++s) {
-                const bf16x8 ka = *(const bf16x8*)(krowp + s * 16);
+        for (int s = 0; s < HD / 16; ++s)
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+                const bf16x8 ka = *(const bf16x8*)(&Ks[stage][(kb * 32 + krow) * HD + (((2 * s + g2) ^ k_read[kb]) * 8)]);
                 st[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qreg[s], st[kb], 0, 0, 0);
             }
-        }
+    };
+    hb_wait_vmcnt<0>();
+    hb_workgroup_barrier();
+    f32x16 st[2];
+    if (active) scores(0, st);
+    for (int page_idx = first_page; page_idx <= last_page; ++page_idx) {
+        const int it = page_idx - first_page;
+        // landed, for every wave after the barrier: the values of this page and the keys of the
+        // next; and nobody reads any more the key stage of this page (its scores are done, those of
+        // the first page too) nor the value stage of the page before, which the next loads fill
+        hb_wait_vmcnt<0>();
+        hb_workgroup_barrier();
+        if (page_idx + 2 <= last_page) issue_keys(page_idx + 2, it & 1);
+        if (page_idx + 1 <= last_page) issue_values(page_idx + 1, (it + 1) & 1);
+        if (!active) continue;
+
+        f32x16 st_next[2];
+        if (page_idx < last_page) scores((it + 1) & 1, st_next);
         float corr;
         bf16x8 pb[2][2];
-        softmax_page(st, g2, page_idx * PAGE, lo_q, pos_q, c, m, l, corr, pb);
+        // a page that every query of the tile sees whole needs no mask
+        const int page0 = page_idx * PAGE;
+        if (page0 + PAGE - 1 <= pos0 && (window == 0 || page0 >= hi_tile + 1 - window))
+            softmax_page<false>(st, g2, page0, lo_q, pos_q, c, m, l, corr, pb);
+        else
+            softmax_page<true>(st, g2, page0, lo_q, pos_q, c, m, l, corr, pb);
+        rescale(oacc, corr);
 #pragma unroll
-        for (int d = 0; d < HD / 32; ++d) {
+        for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) oacc[d][i] *= corr;
-            const bf16* vrowp = &Vs[(d * 32 + c32) * VLD + g2 * 8];
+            for (int h2 = 0; h2 < 2; ++h2)
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                for (int h2 = 0; h2 < 2; ++h2) {
-                    const bf16x8 va = *(const bf16x8*)(vrowp + kb * 32 + h2 * 16);
+                for (int d = 0; d < HD / 32; ++d) {
+                    const bf16x8 va = *(const bf16x8*)(&Vs[it & 1][(d * 32 + c32) * PAGE +
+                                                                 (((kb * 4 + h2 * 2 + g2) ^ v_swz) * 8)]);
                     oacc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb[kb][h2], oacc[d], 0, 0, 0);
                 }
+        if (page_idx < last_page) {
+            st[0] = st_next[0];
+            st[1] = st_next[1];
         }
     }
     if (!active || c32 >= rows) return;
@@ -385,11 +463,13 @@ attn_decode_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_cache, bf16*
         if (page_idx < last_page) LOAD_K(page_idx + 1)
         float corr;
         bf16x8 pb[2][2];
-        softmax_page(st, g2, page_idx * PAGE, lo, hi, c, m, l, corr, pb);
+        if (page_idx * PAGE >= lo && page_idx * PAGE + PAGE - 1 <= hi)
+            softmax_page<false>(st, g2, page_idx * PAGE, lo, hi, c, m, l, corr, pb);
+        else
+            softmax_page<true>(st, g2, page_idx * PAGE, lo, hi, c, m, l, corr, pb);
+        rescale(oacc, corr);
 #pragma unroll
         for (int d = 0; d < HD / 32; ++d) {
-#pragma unroll
-            for (int i = 0; i < 16; ++i) oacc[d][i] *= corr;
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
@@ -489,15 +569,17 @@ extern "C" int hb_attn_prefill_mfma(const void* q, const void* k_cache, const vo
     HB_REQUIRE(num_tiles > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attn_prefill: bad sizes");
     HB_REQUIRE(page_size == PAGE, "attn_prefill: pages must hold %d tokens", PAGE);
     HB_REQUIRE(window >= 0, "attn_prefill: bad window");
+    HB_REQUIRE(scale > 0.f, "attn_prefill: the score scale must be positive");
     const int G = nq / nkv;
-    dim3 grid(num_tiles, nkv * ((G + 3) / 4));
-    HB_REQUIRE(grid.y <= 65535, "attn_prefill: too many heads for the grid");
+    const int per_tile = nkv * ((G + 3) / 4);
+    HB_REQUIRE((long)num_tiles * per_tile < (1l << 30), "attn_prefill: too many tiles");
+    const int total = num_tiles * per_tile;
     const float c = scale * LOG2E;
 #define LAUNCH_PREFILL(HDV)                                                                              \
-    attn_prefill_kernel<HDV><<<grid, 256, 0, stream>>>((const bf16*)q, (const bf16*)k_cache,             \
-                                                      (const bf16*)v_cache, (bf16*)out, tile_seq, tile_row0, \
-                                                      tile_rows, positions, slots, page_table, max_pages, nq, \
-                                                      nkv, c, window)
+    attn_prefill_kernel<HDV><<<total, 256, 0, stream>>>((const bf16*)q, (const bf16*)k_cache,            \
+                                                       (const bf16*)v_cache, (bf16*)out, tile_seq, tile_row0, \
+                                                       tile_rows, positions, slots, page_table, max_pages, nq, \
+                                                       nkv, c, window, per_tile, total)
     if (hd == 32) LAUNCH_PREFILL(32);
     else if (hd == 64) LAUNCH_PREFILL(64);
     else if (hd == 128) LAUNCH_PREFILL(128);
@@ -520,6 +602,7 @@ extern "C" int hb_attn_decode_mfma(const void* q, void* k_cache, void* v_cache, 
     HB_REQUIRE(nq / nkv <= 32, "attn_decode: more than 32 query heads share a kv head");
     HB_REQUIRE(splits > 0 && splits <= 1024 && pages_per_split > 0 && nkv <= 65535, "attn_decode: bad split");
     HB_REQUIRE(window >= 0, "attn_decode: bad window");
+    HB_REQUIRE(scale > 0.f, "attn_decode: the score scale must be positive");
     dim3 grid(B, nkv, splits);
     const float c = scale * LOG2E;
     const DecodeFusion fu = {qkv, q_norm_w, k_norm_w, cos_t, sin_t, eps, write_kv};

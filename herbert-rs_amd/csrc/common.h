@@ -49,6 +49,26 @@ __device__ __forceinline__ float hb_wave_max(float v) {
     return v;
 }
 
+// ---- loads from global memory straight into LDS, and what orders them ----
+// global_load_lds_dwordx4: a lane's 16 bytes land at lds_base + 16 * lane (lds_base is uniform);
+// no registers, no ds_write. The loads count in vmcnt like any other.
+__device__ __forceinline__ void hb_load_to_lds(const void* global_src, void* lds_base) {
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)global_src,
+                                     (__attribute__((address_space(3))) void*)lds_base, 16, 0, 0);
+}
+
+template <int N_OUTSTANDING>
+__device__ __forceinline__ void hb_wait_vmcnt() {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N_OUTSTANDING) : "memory");
+}
+
+// The barrier alone: __syncthreads() would first wait for every load in flight, those of later
+// stages too. What has to have landed is waited for by hb_wait_vmcnt before it; the reads of
+// LDS issued so far are waited for here, so that what they read may be overwritten afterwards.
+__device__ __forceinline__ void hb_workgroup_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 // Sum over a block of up to 1024 threads; `red` holds one float per wave.
 // Every thread gets the result; the order of additions is fixed.
 __device__ __forceinline__ float hb_block_sum(float v, float* red) {

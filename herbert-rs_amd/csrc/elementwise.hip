@@ -198,6 +198,95 @@ __global__ void qk_norm_rope_write_kernel(
     }
 }
 
+// The same for many tokens (prompts), bfloat16 output, rotation over the whole head or none,
+// head size up to 128: a workgroup takes 64 consecutive tokens of one head. Query and key heads:
+// a wave per token, lane = the pair (j, j + hd/2), rows read and written whole. Value heads go
+// through LDS, so that the transposed pages are written along the tokens: lane = token, 64
+// consecutive tokens of a page are one 128-byte line.
+#define HB_TILED_HEAD_DIM 128
+template <class TQ, class TC>
+__global__ void __launch_bounds__(256) qk_norm_rope_write_tiled_kernel(
+    const float* __restrict__ qkv, int ld_qkv, const float* __restrict__ q_norm_w,
+    const float* __restrict__ k_norm_w, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+    const int* __restrict__ positions, const int* __restrict__ seq_of, const int* __restrict__ slots,
+    const int* __restrict__ page_table, int max_pages, int page_size, TQ* __restrict__ q_out,
+    TC* __restrict__ k_cache, TC* __restrict__ v_cache, int T, int nq, int nkv, int hd, float eps) {
+    __shared__ float vt[64][HB_TILED_HEAD_DIM + 1];
+    const int t0 = blockIdx.x * 64, h = blockIdx.y;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const bool is_q = h < nq, is_v = h >= nq + nkv;
+    const int half = hd / 2;
+    if (is_v) {
+        const int kvh = h - nq - nkv;
+        for (int idx = tid; idx < 64 * hd; idx += 256) {
+            const int r = idx / hd, c = idx - r * hd;
+            const int t = t0 + r;
+            vt[r][c] = t < T ? qkv[(size_t)t * ld_qkv + (size_t)h * hd + c] : 0.f;
+        }
+        __syncthreads();
+        const int t = t0 + lane;
+        if (t >= T) return;
+        const int pos = positions[t];
+        const int page = page_table[(size_t)slots[seq_of[t]] * max_pages + pos / page_size];
+        TC* dst = v_cache + ((size_t)page * nkv + kvh) * page_size * hd + pos % page_size;
+        for (int d = wave; d < hd; d += 4) dst[(size_t)d * page_size] = hb_from_float<TC>(vt[lane][d]);
+        return;
+    }
+    const float* norm_w = is_q ? q_norm_w : k_norm_w;
+    const bool mine = lane < half;
+    const int j = mine ? lane : 0;
+    const float w0 = norm_w ? norm_w[j] : 1.f, w1 = norm_w ? norm_w[j + half] : 1.f;
+    // a wave's 16 tokens in two rounds of 8: all loads of a round go out before anything waits for them
+#pragma unroll
+    for (int round = 0; round < 2; ++round) {
+        float x0[8], x1[8], c[8], sn[8];
+        int pos[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int t = t0 + wave + 4 * (round * 8 + u);
+            const int tc = t < T ? t : T - 1;
+            const float* src = qkv + (size_t)tc * ld_qkv + (size_t)h * hd;
+            pos[u] = positions[tc];
+            x0[u] = mine ? src[j] : 0.f;
+            x1[u] = mine ? src[j + half] : 0.f;
+        }
+        if (cos_t) {
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                c[u] = cos_t[(size_t)pos[u] * half + j];
+                sn[u] = sin_t[(size_t)pos[u] * half + j];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int t = t0 + wave + 4 * (round * 8 + u);
+            float a0 = x0[u], a1 = x1[u];
+            if (norm_w) {
+                const float ss = hb_wave_sum(a0 * a0 + a1 * a1);
+                const float inv = 1.0f / sqrtf(ss / (float)hd + eps);
+                a0 = a0 * inv * w0;
+                a1 = a1 * inv * w1;
+            }
+            if (cos_t) {
+                const float r0 = a0 * c[u] - a1 * sn[u], r1 = a0 * sn[u] + a1 * c[u];
+                a0 = r0;
+                a1 = r1;
+            }
+            if (!mine || t >= T) continue;
+            if (is_q) {
+                TQ* dst = q_out + ((size_t)t * nq + h) * hd;
+                dst[j] = hb_from_float<TQ>(a0);
+                dst[j + half] = hb_from_float<TQ>(a1);
+            } else {
+                const int page = page_table[(size_t)slots[seq_of[t]] * max_pages + pos[u] / page_size];
+                TC* dst = k_cache + (((size_t)page * nkv + (h - nq)) * page_size + pos[u] % page_size) * hd;
+                dst[j] = hb_from_float<TC>(a0);
+                dst[j + half] = hb_from_float<TC>(a1);
+            }
+        }
+    }
+}
+
 extern "C" int hb_qk_norm_rope_write(const float* qkv, int ld_qkv, const float* q_norm_w,
                                      const float* k_norm_w, const float* cos_t, const float* sin_t,
                                      int rot_dims, const int* positions, const int* seq_of,
@@ -214,6 +303,15 @@ extern "C" int hb_qk_norm_rope_write(const float* qkv, int ld_qkv, const float* 
     const int heads = nq + (write_kv ? 2 * nkv : 0);
     HB_REQUIRE(ld_qkv >= heads * hd, "qk_norm_rope_write: row stride %d too small", ld_qkv);
     HB_REQUIRE(heads <= 65535, "qk_norm_rope_write: too many heads for the grid");
+    if (dtype == HB_BF16 && write_kv && T >= 64 && hd <= HB_TILED_HEAD_DIM && hd % 2 == 0 &&
+        (cos_t == nullptr || rot_dims == hd) && (T + 63) / 64 <= 0x7fffffff) {
+        dim3 tiles((T + 63) / 64, heads);
+        qk_norm_rope_write_tiled_kernel<bf16, bf16><<<tiles, 256, 0, stream>>>(
+            qkv, ld_qkv, q_norm_w, k_norm_w, cos_t, sin_t, positions, seq_of, slots, page_table, max_pages,
+            page_size, (bf16*)q_out, (bf16*)k_cache, (bf16*)v_cache, T, nq, nkv, hd, eps);
+        HB_CHECK_LAUNCH("qk_norm_rope_write_tiled");
+        return 0;
+    }
     dim3 grid(T, heads);
     if (dtype == HB_F32)
         qk_norm_rope_write_kernel<float, float><<<grid, HB_WAVE, 0, stream>>>(

@@ -376,8 +376,8 @@ static void pick_skinny(const void* X, const void* W, void* C, int M, int N, int
 
 // ------------------------------------------------------------------- tiled
 // The product for many rows (prompts). Tiles go from global memory straight into LDS
-// (global_load_lds_dwordx4: a lane's 16 bytes land at base + 16 * lane; no registers, no
-// ds_write) through rings of stages that are loaded ahead of the MFMAs.
+// (hb_load_to_lds) through rings of stages that are loaded ahead of the MFMAs; what has landed
+// is waited for by count (hb_wait_vmcnt) before a bare barrier (hb_workgroup_barrier).
 // 32x32x16 MFMA (of the two bf16 shapes the one with the higher rate), weight rows first: an
 // operand is 32 rows x 16 k, lane l = row l % 32, k 8 (l / 32) .. + 8; a lane ends with 16 sums
 // of one m: n = 8 q + 4 (l / 32) + j for register 4 q + j.
@@ -386,18 +386,6 @@ static void pick_skinny(const void* X, const void* W, void* C, int M, int N, int
 // (l % 32) / 16 of a pair of blocks, chunk 16 (2 h + l / 32) + l % 16: 16 lanes read 256
 // contiguous bytes, free of bank conflicts.
 // Workgroup: WNW x WMW waves, each TNB x TMB blocks of 16: BN = 16 TNB WNW, BM = 16 TMB WMW.
-template <int N_OUTSTANDING>
-__device__ __forceinline__ void wait_vmcnt() {
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N_OUTSTANDING) : "memory");
-}
-
-// The barrier alone: __syncthreads() would first wait for every load in flight, the later stages'
-// too, and so undo the rings. What has to have landed is waited for by wait_vmcnt before it; the
-// reads of LDS issued so far are waited for here, so that their stage may be overwritten.
-__device__ __forceinline__ void workgroup_barrier() {
-    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-}
-
 // Workgroups go round the 8 XCDs, each with an L2 of its own: an XCD takes a run of tiles, and
 // within it bands of 8 tiles in m are walked n first, so that the workgroups that are resident
 // together share both their weight and their activation panels in that L2.
@@ -535,17 +523,10 @@ gemm_tile_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* _
     // loads of a step, the activations first: those are waited for one step earlier than the weights
     auto load_one = [&](int xstep, int wstep, int idx) {
         if (idx < NLX) {
-            __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void*)(xsrc[idx] + (size_t)xstep * 64),
-                (__attribute__((address_space(3))) void*)(xlds + (xstep & 1) * X_STAGE + (wave * XR + idx) * 512),
-                16, 0, 0);
+            hb_load_to_lds(xsrc[idx] + (size_t)xstep * 64, xlds + (xstep & 1) * X_STAGE + (wave * XR + idx) * 512);
         } else {
             const int ks = (idx - NLX) / WL, i = (idx - NLX) % WL;
-            __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void*)(wsrc[i] + ((size_t)wstep * 2 + ks) * WSTEP),
-                (__attribute__((address_space(3))) void*)(lds + (wstep % WST) * W_STAGE + ks * WBLK * 512 +
-                                                          (wave * WL + i) * 512),
-                16, 0, 0);
+            hb_load_to_lds(wsrc[i] + ((size_t)wstep * 2 + ks) * WSTEP, lds + (wstep % WST) * W_STAGE + ks * WBLK * 512 + (wave * WL + i) * 512);
         }
     };
 
@@ -600,8 +581,8 @@ gemm_tile_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* _
     for (int st = 2; st < WST; ++st)
 #pragma unroll
         for (int i = NLX; i < NLX + NLW; ++i) load_one(0, clamp(st), i);
-    wait_vmcnt<NLX + (WST - 1) * NLW>();
-    workgroup_barrier();
+    hb_wait_vmcnt<NLX + (WST - 1) * NLW>();
+    hb_workgroup_barrier();
 #pragma unroll
     for (int i = 0; i < NR; ++i) read_one(0, 0, 0, i);
 
@@ -617,8 +598,8 @@ gemm_tile_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* _
         // steps may be missing), after the barrier for every wave, and nobody reads step t any
         // more: between the MFMAs of its second k-step go the loads into its stages, the
         // activations of step t + 2 and the weights of step t + WST, and the reads of step t + 1.
-        wait_vmcnt<(WST - 2) * NLW>();
-        workgroup_barrier();
+        hb_wait_vmcnt<(WST - 2) * NLW>();
+        hb_workgroup_barrier();
         const int xstep = clamp(t + 2), wstep = clamp(t + WST);
 #pragma unroll
         for (int j = 0; j < NM; ++j) {
@@ -627,17 +608,10 @@ gemm_tile_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* _
                     [&](int i) {
                         // a clamped step goes where step t + 2 (t + WST) would: into the stage just freed
                         if (i < NLX) {
-                            __builtin_amdgcn_global_load_lds(
-                                (const __attribute__((address_space(1))) void*)(xsrc[i] + (size_t)xstep * 64),
-                                (__attribute__((address_space(3))) void*)(xlds + (t & 1) * X_STAGE + (wave * XR + i) * 512),
-                                16, 0, 0);
+                            hb_load_to_lds(xsrc[i] + (size_t)xstep * 64, xlds + (t & 1) * X_STAGE + (wave * XR + i) * 512);
                         } else {
                             const int ks = (i - NLX) / WL, w = (i - NLX) % WL;
-                            __builtin_amdgcn_global_load_lds(
-                                (const __attribute__((address_space(1))) void*)(wsrc[w] + ((size_t)wstep * 2 + ks) * WSTEP),
-                                (__attribute__((address_space(3))) void*)(lds + (t % WST) * W_STAGE + ks * WBLK * 512 +
-                                                                          (wave * WL + w) * 512),
-                                16, 0, 0);
+                            hb_load_to_lds(wsrc[w] + ((size_t)wstep * 2 + ks) * WSTEP, lds + (t % WST) * W_STAGE + ks * WBLK * 512 + (wave * WL + w) * 512);
                         }
                     },
                     [&](int i) { read_one(0, t + 1, 0, i); });
@@ -655,7 +629,7 @@ gemm_tile_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* _
 #pragma unroll
         for (int j = 0; j < NM; ++j) mfma_one(1, j);
     }
-    wait_vmcnt<0>();      // the loads past the end (repeats of the last step) have landed too
+    hb_wait_vmcnt<0>();      // the loads past the end (repeats of the last step) have landed too
     store_wave_tile<EPI, TN32, TM32>(acc, Cv, M, N, ldc, m0 + wm * TMB * 16, n0 + wn * TNB * 16, c32, g2);
 }
 
@@ -710,14 +684,10 @@ gemm_tile32_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void*
         bf16* base = lds + (size_t)stage * BLKS * 512;
 #pragma unroll
         for (int i = 0; i < WL; ++i)
-            __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void*)(wsrc[i] + (size_t)step * WSTEP),
-                (__attribute__((address_space(3))) void*)(base + (wave * WL + i) * 512), 16, 0, 0);
+            hb_load_to_lds(wsrc[i] + (size_t)step * WSTEP, base + (wave * WL + i) * 512);
 #pragma unroll
         for (int i = 0; i < XL; ++i)
-            __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void*)(xsrc[i] + (size_t)step * 32),
-                (__attribute__((address_space(3))) void*)(base + (WBLK + wave * XL + i) * 512), 16, 0, 0);
+            hb_load_to_lds(xsrc[i] + (size_t)step * 32, base + (WBLK + wave * XL + i) * 512);
     };
 
     f32x16 acc[TN32][TM32];
@@ -756,8 +726,8 @@ gemm_tile32_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void*
     // steps may be in flight) and its reads of step t are in registers; after the barrier that
     // holds for every wave, so the stage of step t can take the loads of step t + STAGES.
     auto advance = [&](int t) {
-        wait_vmcnt<(STAGES - 2) * (WL + XL)>();
-        workgroup_barrier();
+        hb_wait_vmcnt<(STAGES - 2) * (WL + XL)>();
+        hb_workgroup_barrier();
         const int nt = t + STAGES;
         issue(nt < nsteps ? nt : nsteps - 1, nt % STAGES);
     };
@@ -776,7 +746,7 @@ gemm_tile32_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void*
         run_step(0, t);
         if (t + 1 < nsteps) run_step(1, t + 1);
     }
-    wait_vmcnt<0>();      // the loads past the end (repeats of the last step) have landed too
+    hb_wait_vmcnt<0>();      // the loads past the end (repeats of the last step) have landed too
     store_wave_tile<EPI, TN32, TM32>(acc, Cv, M, N, ldc, m0 + wm * TMB * 16, n0 + wn * TNB * 16, c32, g2);
 }
 

@@ -142,17 +142,20 @@ def attention_supported(q, kv, nq, nkv, hd):
 
 
 def _prefill_tiles(meta):
-    """Device arrays (sequence, first packed row, rows) of the 32-token query tiles of a step."""
+    """Device arrays (sequence, first packed row, rows) of the 32-token query tiles of a step,
+    those that see the most keys first: the kernel deals them out heaviest first."""
     tiles = meta.derived.get("prefill_tiles")
     if tiles is None:
-        seq, row0, rows = [], [], []
-        starts = meta.host_starts
+        items = []
+        starts, context = meta.host_starts, meta.host_context
         for i in range(meta.num_seqs):
             a, b = int(starts[i]), int(starts[i + 1])
             for r in range(a, b, QUERY_TILE):
-                seq.append(i)
-                row0.append(r)
-                rows.append(min(QUERY_TILE, b - r))
+                n = min(QUERY_TILE, b - r)
+                last_position = int(context[i]) - (b - (r + n)) - 1
+                items.append((-last_position, i, r, n))
+        items.sort()
+        seq, row0, rows = [it[1] for it in items], [it[2] for it in items], [it[3] for it in items]
         packed = torch.tensor([seq, row0, rows], dtype=torch.int32).to(meta.positions.device)
         tiles = (packed[0], packed[1], packed[2], len(seq))
         meta.derived["prefill_tiles"] = tiles

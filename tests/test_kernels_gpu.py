@@ -170,6 +170,7 @@ def paged_case(lengths, new_counts, nkv, hd, dtype, seed=0, n_pages=64, shuffle=
     meta.max_new, meta.max_context, meta.max_position = max(new_counts), max(lengths), max(lengths) - 1
     import numpy as np
     meta.host_starts = np.array(starts, dtype=np.int32)
+    meta.host_context = np.array(lengths, dtype=np.int32)
     meta.derived = {}
     from herbert_rs_amd.engine.batch import bucket
     meta.context_bucket = bucket(max(lengths))
@@ -237,6 +238,57 @@ def test_attention_mfma_decode(nq, nkv, hd, window, lengths):
     mfma.attention(q, meta, kv, out, nq, nkv, hd, scale, window)
     want = attention_reference(q, meta, dense, nq, nkv, hd, scale, window)
     assert float((out.float().cpu() - want).abs().max()) <= 2 ** -7 * float(want.abs().max())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nq,nkv,hd,rot,norm", [(4, 2, 128, 128, True), (3, 1, 64, 64, False), (2, 2, 96, 0, True),
+                                                (5, 1, 32, 32, True), (2, 1, 80, 40, True), (1, 1, 256, 256, True)])
+def test_qk_norm_rope_write(nq, nkv, hd, rot, norm, dtype):
+    """Per-head norm, rotation and the write into the pages, for prompts that cross pages and a
+    step that is no multiple of 64 tokens (the tiled kernel), and for a few tokens (the plain one)."""
+    from herbert_rs_amd.kernels import ops
+    for lengths, new in (([130, 70, 300, 64], [130, 7, 190, 64]), ([5, 90], [2, 1])):
+        meta, kv, _ = paged_case(lengths, new, nkv, hd, dtype, seed=hd)
+        before_k, before_v = kv.k.clone(), kv.v.clone()
+        T = sum(new)
+        qkv = rand(T, (nq + 2 * nkv) * hd, seed=50, scale=1.3)
+        qw = (1 + rand(hd, seed=51, scale=0.3)) if norm else None
+        kw = (1 + rand(hd, seed=52, scale=0.3)) if norm else None
+        cos = sin = None
+        if rot:
+            ang = torch.arange(512, dtype=torch.float32)[:, None] * (10000.0 ** (-torch.arange(rot // 2) / (rot // 2)))[None]
+            cos, sin = ang.cos().to(dev()).contiguous(), ang.sin().to(dev()).contiguous()
+        eps = 1e-5
+        q = torch.full((T, nq * hd), 9.0, dtype=dtype, device=dev())
+        ops.qk_norm_rope_write(qkv, qw, kw, cos, sin, rot, meta, kv, q, nq, nkv, hd, eps)
+
+        x = qkv.double().cpu().view(T, nq + 2 * nkv, hd)
+        pos = meta.positions.cpu().long()
+
+        def head_op(v, w):
+            if w is not None:
+                v = v / torch.sqrt((v ** 2).mean(-1, keepdim=True) + eps) * w.double().cpu()
+            if rot:
+                c, s_ = cos.double().cpu()[pos][:, None, :], sin.double().cpu()[pos][:, None, :]
+                a, b = v[..., :rot // 2], v[..., rot // 2:rot]
+                v = torch.cat([a * c - b * s_, a * s_ + b * c, v[..., rot:]], -1)
+            return v
+        want_q = head_op(x[:, :nq], qw).reshape(T, nq * hd)
+        want_k = head_op(x[:, nq:nq + nkv], kw)
+        want_v = x[:, nq + nkv:]
+        tol = 1e-5 if dtype == torch.float32 else 2 ** -8
+        assert float((q.double().cpu() - want_q).abs().max()) <= tol * float(want_q.abs().max())
+        table = kv.page_table.cpu()
+        slots, seq = meta.slots.cpu().tolist(), meta.seq_of.cpu().tolist()
+        exp_k, exp_v = before_k.double().cpu(), before_v.double().cpu()
+        for t in range(T):
+            p = int(pos[t])
+            page = int(table[slots[seq[t]], p // 64])
+            exp_k[page, :, p % 64] = want_k[t]
+            exp_v[page, :, :, p % 64] = want_v[t]
+        # every other place of the pages is as it was
+        assert float((kv.k.double().cpu() - exp_k).abs().max()) <= tol * float(exp_k.abs().max())
+        assert float((kv.v.double().cpu() - exp_v).abs().max()) <= tol * float(exp_v.abs().max())
 
 
 @pytest.mark.parametrize("nq,nkv,hd,window,norm,rope", [(4, 1, 128, 0, True, True), (32, 8, 128, 0, True, True),
