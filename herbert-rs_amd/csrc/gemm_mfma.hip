@@ -473,7 +473,7 @@ __device__ __forceinline__ void store_wave_tile(const f32x16 (&acc)[TN32][TM32],
 template <int EPI, bool PACKED, int TNB, int TMB, int WNW, int WMW, int WST>
 __global__ void __launch_bounds__(64 * WNW * WMW)
 gemm_tile_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* __restrict__ Cv, int M, int N,
-                 int K, int ldc, int m_tiles, int n_tiles) {
+                 int K, int ldc, int m_tiles, int n_tiles, float* __restrict__ partial) {
     constexpr int NW = WNW * WMW;
     constexpr int BN = 16 * TNB * WNW, BM = 16 * TMB * WMW;
     constexpr int WBLK = BN / 16;                       // weight blocks of a k-step of 32
@@ -495,8 +495,14 @@ gemm_tile_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* _
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // uniform: LDS addresses stay scalar
     const int r16 = lane & 15, g4 = lane >> 4, c32 = lane & 31, g2 = lane >> 5;
     const int wn = wave / WMW, wm = wave % WMW;
-    const int nsteps = K / 64;
+    // gridDim.y > 1: K is cut into slices over workgroups (few tiles, long K); a workgroup leaves the
+    // sums of its slice in `partial` [slice][M][N] and gemm_slices_kernel adds the slices in order
+    const int all_steps = K / 64;
+    const int per_slice = (all_steps + gridDim.y - 1) / gridDim.y;
+    const int step0 = blockIdx.y * per_slice;
+    const int nsteps = all_steps - step0 < per_slice ? all_steps - step0 : per_slice;    // >= 1: the host sees to it
 
+    const size_t WSTEP = PACKED ? (size_t)(N / 16) * 512 : 32;      // elements between two k-steps of 32
     const bf16* wsrc[WL];
 #pragma unroll
     for (int i = 0; i < WL; ++i) {
@@ -504,21 +510,20 @@ gemm_tile_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* _
         if (PACKED) {
             int nb = n0 / 16 + blk;
             if (nb * 16 >= N) nb = (N - 1) / 16;
-            wsrc[i] = W + ((size_t)nb * 64 + lane) * 8;
+            wsrc[i] = W + ((size_t)nb * 64 + lane) * 8 + (size_t)step0 * 2 * WSTEP;
         } else {
             int n = n0 + blk * 16 + r16;
             if (n >= N) n = N - 1;                      // rows past the end repeat the last one; never stored
-            wsrc[i] = W + (size_t)n * K + g4 * 8;
+            wsrc[i] = W + (size_t)n * K + g4 * 8 + (size_t)step0 * 2 * WSTEP;
         }
     }
-    const size_t WSTEP = PACKED ? (size_t)(N / 16) * 512 : 32;      // elements between two k-steps of 32
     const bf16* xsrc[XR];
 #pragma unroll
     for (int i = 0; i < XR; ++i) {
         const int r = (wave * XR + i) * 8 + (lane >> 3);
         int m = m0 + r;
         if (m >= M) m = M - 1;
-        xsrc[i] = X + (size_t)m * K + (((lane & 7) ^ ((r >> 1) & 7)) * 8);
+        xsrc[i] = X + (size_t)m * K + (((lane & 7) ^ ((r >> 1) & 7)) * 8) + (size_t)step0 * 64;
     }
     // loads of a step, the activations first: those are waited for one step earlier than the weights
     auto load_one = [&](int xstep, int wstep, int idx) {
@@ -630,7 +635,11 @@ gemm_tile_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* _
         for (int j = 0; j < NM; ++j) mfma_one(1, j);
     }
     hb_wait_vmcnt<0>();      // the loads past the end (repeats of the last step) have landed too
-    store_wave_tile<EPI, TN32, TM32>(acc, Cv, M, N, ldc, m0 + wm * TMB * 16, n0 + wn * TNB * 16, c32, g2);
+    if (gridDim.y > 1)
+        store_wave_tile<EPI_STORE, TN32, TM32>(acc, partial + (size_t)blockIdx.y * M * N, M, N, N,
+                                               m0 + wm * TMB * 16, n0 + wn * TNB * 16, c32, g2);
+    else
+        store_wave_tile<EPI, TN32, TM32>(acc, Cv, M, N, ldc, m0 + wm * TMB * 16, n0 + wn * TNB * 16, c32, g2);
 }
 
 // K in steps of 32 only: one k-step a stage, everything in 1 KB blocks (the activations too: a
@@ -750,9 +759,10 @@ gemm_tile32_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void*
     store_wave_tile<EPI, TN32, TM32>(acc, Cv, M, N, ldc, m0 + wm * TMB * 16, n0 + wn * TNB * 16, c32, g2);
 }
 
-template <class Kernel>
-static int launch_tiles(Kernel kern, size_t lds, int threads, long total, const bf16* x, const bf16* w, void* C,
-                        int M, int N, int K, int ldc, int m_tiles, int n_tiles, hipStream_t stream) {
+template <class Kernel, class... Extra>
+static int launch_tiles(Kernel kern, size_t lds, int threads, long total, int slices, const bf16* x, const bf16* w,
+                        void* C, int M, int N, int K, int ldc, int m_tiles, int n_tiles, hipStream_t stream,
+                        Extra... extra) {
     HB_REQUIRE(total < (1l << 30), "gemm_mfma: too many tiles");
     HB_REQUIRE(lds <= 160 * 1024, "gemm_mfma: %zu bytes of LDS asked for", lds);
     if (lds > 64 * 1024) {
@@ -764,8 +774,8 @@ static int launch_tiles(Kernel kern, size_t lds, int threads, long total, const 
             raised = true;
         }
     }
-    const int blocks = (int)((total + 7) / 8 * 8);
-    kern<<<blocks, threads, lds, stream>>>(x, w, C, M, N, K, ldc, m_tiles, n_tiles);
+    const dim3 blocks((unsigned)((total + 7) / 8 * 8), slices);
+    kern<<<blocks, threads, lds, stream>>>(x, w, C, M, N, K, ldc, m_tiles, n_tiles, extra...);
     HB_CHECK_LAUNCH("gemm_tile");
     return 0;
 }
@@ -773,18 +783,19 @@ static int launch_tiles(Kernel kern, size_t lds, int threads, long total, const 
 #define TILE_DISPATCH(KERNEL, ...)                                                                   \
     do {                                                                                             \
         if (packed) {                                                                                \
-            if (epi == EPI_STORE) return launch_tiles(KERNEL<EPI_STORE, true, __VA_ARGS__>, lds, threads, total, x, w, C, M, N, K, ldc, m_tiles, n_tiles, stream); \
-            if (epi == EPI_ADD) return launch_tiles(KERNEL<EPI_ADD, true, __VA_ARGS__>, lds, threads, total, x, w, C, M, N, K, ldc, m_tiles, n_tiles, stream); \
-            return launch_tiles(KERNEL<EPI_SWIGLU, true, __VA_ARGS__>, lds, threads, total, x, w, C, M, N, K, ldc, m_tiles, n_tiles, stream); \
+            if (epi == EPI_STORE) return launch_tiles(KERNEL<EPI_STORE, true, __VA_ARGS__>, lds, threads, total, slices, x, w, C, M, N, K, ldc, m_tiles, n_tiles, stream EXTRA); \
+            if (epi == EPI_ADD) return launch_tiles(KERNEL<EPI_ADD, true, __VA_ARGS__>, lds, threads, total, slices, x, w, C, M, N, K, ldc, m_tiles, n_tiles, stream EXTRA); \
+            return launch_tiles(KERNEL<EPI_SWIGLU, true, __VA_ARGS__>, lds, threads, total, slices, x, w, C, M, N, K, ldc, m_tiles, n_tiles, stream EXTRA); \
         }                                                                                            \
-        if (epi == EPI_STORE) return launch_tiles(KERNEL<EPI_STORE, false, __VA_ARGS__>, lds, threads, total, x, w, C, M, N, K, ldc, m_tiles, n_tiles, stream); \
-        if (epi == EPI_ADD) return launch_tiles(KERNEL<EPI_ADD, false, __VA_ARGS__>, lds, threads, total, x, w, C, M, N, K, ldc, m_tiles, n_tiles, stream); \
-        return launch_tiles(KERNEL<EPI_SWIGLU, false, __VA_ARGS__>, lds, threads, total, x, w, C, M, N, K, ldc, m_tiles, n_tiles, stream); \
+        if (epi == EPI_STORE) return launch_tiles(KERNEL<EPI_STORE, false, __VA_ARGS__>, lds, threads, total, slices, x, w, C, M, N, K, ldc, m_tiles, n_tiles, stream EXTRA); \
+        if (epi == EPI_ADD) return launch_tiles(KERNEL<EPI_ADD, false, __VA_ARGS__>, lds, threads, total, slices, x, w, C, M, N, K, ldc, m_tiles, n_tiles, stream EXTRA); \
+        return launch_tiles(KERNEL<EPI_SWIGLU, false, __VA_ARGS__>, lds, threads, total, slices, x, w, C, M, N, K, ldc, m_tiles, n_tiles, stream EXTRA); \
     } while (0)
 
+// slices > 1: the sums of the slices go to `partial`; the caller adds them up afterwards
 template <int TNB, int TMB, int WNW, int WMW, int WST>
 static int launch_tile64(const void* X, const void* W, void* C, int M, int N, int K, int ldc, int epi, int packed,
-                         hipStream_t stream) {
+                         hipStream_t stream, int slices = 1, float* partial = nullptr) {
     constexpr int BN = 16 * TNB * WNW, BM = 16 * TMB * WMW;
     HB_REQUIRE(K % 64 == 0, "gemm_mfma: K=%d is no multiple of 64", K);
     const int m_tiles = (M + BM - 1) / BM, n_tiles = (N + BN - 1) / BN;
@@ -793,7 +804,11 @@ static int launch_tile64(const void* X, const void* W, void* C, int M, int N, in
     const int threads = 64 * WNW * WMW;
     const bf16* x = (const bf16*)X;
     const bf16* w = (const bf16*)W;
+    HB_REQUIRE(slices >= 1 && (slices == 1 || (partial && epi != EPI_SWIGLU)), "gemm_mfma: bad slices");
+    HB_REQUIRE((K / 64 + slices - 1) / slices * (slices - 1) < K / 64, "gemm_mfma: a slice of K would be empty");
+#define EXTRA , partial
     TILE_DISPATCH(gemm_tile_kernel, TNB, TMB, WNW, WMW, WST);
+#undef EXTRA
 }
 
 template <int TNB, int TMB, int WNW, int WMW, int STAGES>
@@ -806,7 +821,10 @@ static int launch_tile32(const void* X, const void* W, void* C, int M, int N, in
     const int threads = 64 * WNW * WMW;
     const bf16* x = (const bf16*)X;
     const bf16* w = (const bf16*)W;
+    const int slices = 1;
+#define EXTRA
     TILE_DISPATCH(gemm_tile32_kernel, TNB, TMB, WNW, WMW, STAGES);
+#undef EXTRA
 }
 #undef TILE_DISPATCH
 
@@ -837,37 +855,54 @@ extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N,
         HB_CHECK_LAUNCH("gemm_skinny");
         return 0;
     }
-    // tile_hint: 0 = choose (otherwise a variant by number, for measurements and tests).
-    // The bigger the tile, the more arithmetic per byte moved and the higher its rate, but the
-    // fewer tiles there are for the 256 CUs: take the variant with the least estimated time,
-    // rounds of tiles over the CUs x the time of a tile at the rate measured for the variant.
-    int tile = tile_hint;
+    // tile_hint: 0 = choose (otherwise a variant by number, for measurements and tests; + 1000 x the
+    // number of K slices). The bigger the tile, the more arithmetic per byte moved and the higher
+    // its rate, but the fewer tiles there are for the 256 CUs; with few tiles and a long K, K is
+    // cut into slices over further workgroups, whose sums a second kernel adds in their order.
+    // Taken: the variant and the slices with the least estimated time (us): rounds of workgroups
+    // over the CUs x steps x the time of a step as measured, + what the second pass moves.
+    struct Variant { int id, bn, bm, per_cu; double step_us; };
+    static const Variant variants[] = {{188, 256, 256, 1, 1.69}, {142, 256, 128, 1, 0.98}, {122, 128, 128, 2, 0.55}};
+    int tile = tile_hint % 1000, slices = tile_hint >= 1000 ? tile_hint / 1000 : 1;
+    if (tile == 0 && K % 64) tile = 123;
     if (tile == 0) {
-        if (K % 64) {
-            tile = 123;
-        } else {
-            struct Variant { int id, bn, bm, per_cu; double rate; };
-            static const Variant variants[] = {{188, 256, 256, 1, 1.27}, {142, 256, 128, 1, 1.10}, {122, 128, 128, 2, 1.00}};
-            double best = 0;
-            for (const Variant& v : variants) {
-                const long tiles = (long)((M + v.bm - 1) / v.bm) * ((N + v.bn - 1) / v.bn);
-                const long rounds = (tiles + 256 * v.per_cu - 1) / (256 * v.per_cu);
-                const double cost = (double)rounds * v.per_cu * v.bn * v.bm / v.rate;
+        const int steps = K / 64;
+        double best = 0;
+        for (const Variant& v : variants) {
+            const long tiles = (long)((M + v.bm - 1) / v.bm) * ((N + v.bn - 1) / v.bn);
+            for (int sl = 1; sl <= 16; sl *= 2) {
+                if (sl > 1 && (epi == EPI_SWIGLU || steps / sl < 4 || (size_t)sl * M * N > workspace_floats)) break;
+                const long wgs = tiles * sl;
+                const long rounds = (wgs + 256 * v.per_cu - 1) / (256 * v.per_cu);
+                const int share = wgs > 256 ? v.per_cu : 1;
+                double cost = (double)rounds * share * ((steps + sl - 1) / sl) * v.step_us + 5.0;
+                if (sl > 1) cost += 4.0 + (double)(sl + 2) * M * N * 4 / 2.5e6;
                 if (tile == 0 || cost < best) {
                     tile = v.id;
+                    slices = sl;
                     best = cost;
                 }
             }
         }
     }
+    HB_REQUIRE(slices == 1 || (size_t)slices * M * N <= workspace_floats, "gemm_mfma: no room for %d slices", slices);
+    int rc;
     switch (tile) {
         // (a third weight stage, measured with weights that come from HBM: a gain of a tenth for
         // 256 x 128, none for the other two)
-        case 188: return launch_tile64<8, 8, 2, 2, 2>(X, W, C, M, N, K, ldc, epi, packed, stream);   // 256 x 256
-        case 142: return launch_tile64<8, 4, 2, 2, 3>(X, W, C, M, N, K, ldc, epi, packed, stream);   // 256 (n) x 128 (m)
-        case 122: return launch_tile64<4, 4, 2, 2, 2>(X, W, C, M, N, K, ldc, epi, packed, stream);   // 128 x 128, two to a CU
-        case 123: return launch_tile32<4, 4, 2, 2, 4>(X, W, C, M, N, K, ldc, epi, packed, stream);   // 128 x 128, K in steps of 32
+        case 188: rc = launch_tile64<8, 8, 2, 2, 2>(X, W, C, M, N, K, ldc, epi, packed, stream, slices, workspace); break;   // 256 x 256
+        case 142: rc = launch_tile64<8, 4, 2, 2, 3>(X, W, C, M, N, K, ldc, epi, packed, stream, slices, workspace); break;   // 256 (n) x 128 (m)
+        case 122: rc = launch_tile64<4, 4, 2, 2, 2>(X, W, C, M, N, K, ldc, epi, packed, stream, slices, workspace); break;   // 128 x 128, two to a CU
+        case 123:                                                                                                           // 128 x 128, K in steps of 32
+            HB_REQUIRE(slices == 1, "gemm_mfma: this tile does not cut K");
+            return launch_tile32<4, 4, 2, 2, 4>(X, W, C, M, N, K, ldc, epi, packed, stream);
         default: HB_REQUIRE(false, "gemm_mfma: unknown tile %d", tile);
     }
-    return 0;
+    if (rc == 0 && slices > 1) {
+        const size_t total = (size_t)M * N;
+        gemm_slices_kernel<<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(workspace, (float*)C, M, N, ldc, slices,
+                                                                              epi == EPI_ADD);
+        HB_CHECK_LAUNCH("gemm_slices");
+    }
+    return rc;
 }

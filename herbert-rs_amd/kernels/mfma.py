@@ -20,15 +20,24 @@ SKINNY_MAX_M = 64
 _workspaces = {}
 
 
+SLICE_WORKSPACE_FLOATS = 16 << 20     # most that the tiled product may use for its K slices (64 MB)
+
+
 def _slice_workspace(device, M, N, K):
-    """(pointer, floats) of the scratch for products whose K is cut into slices (17 to 64 rows).
-    A buffer that was handed out is kept for good: a captured graph may hold its address."""
-    if M <= 16 or M > SKINNY_MAX_M:
+    """(pointer, floats) of the scratch for products whose K is cut into slices: 17 to 64 rows, and
+    the tiled product when it has few tiles. A buffer that was handed out is kept for good: a
+    captured graph may hold its address."""
+    if M <= 16:
         return None, 0
-    slices = min(8, 256 // max(1, (N + 63) // 64), K // 256)
-    if slices < 2:
+    if M <= SKINNY_MAX_M:
+        slices = min(8, 256 // max(1, (N + 63) // 64), K // 256)
+        need = slices * M * N
+    else:
+        tiles = ((M + 127) // 128) * ((N + 127) // 128)
+        slices = min(16, K // 256) if tiles < 256 else 1
+        need = min(slices * M * N, SLICE_WORKSPACE_FLOATS)
+    if slices < 2 or need < 2 * M * N:
         return None, 0
-    need = slices * M * N
     kept = _workspaces.setdefault(str(device), [])
     if not kept or kept[-1].numel() < need:
         kept.append(torch.empty(need, dtype=torch.float32, device=device))

@@ -418,6 +418,33 @@ def test_gemm_mfma_tile_variants(tile, M, N, K, packed):
         assert float((out.float() - wanted).abs().max()) <= 2 ** -7 * float(wanted.abs().max()) + 1e-4
 
 
+@pytest.mark.parametrize("tile", [0, 2122, 4188, 3142, 8122])
+@pytest.mark.parametrize("M,N,K,packed", [(200, 336, 512, True), (513, 1040, 768, True), (128, 1024, 4096, True),
+                                          (300, 530, 1024, False)])
+def test_gemm_mfma_tiled_with_k_slices(tile, M, N, K, packed):
+    """More than 64 rows and few tiles: K is cut into slices over workgroups (thousands of the tile
+    number = slices), the sums added in order by a second kernel; tile 0 chooses by itself."""
+    from herbert_rs_amd.kernels import mfma
+    slices, steps = tile // 1000, K // 64
+    if slices > 1 and (slices > min(16, K // 256) or -(-steps // slices) * (slices - 1) >= steps):
+        pytest.skip("more slices than the workspace is sized for, or than K has steps for")
+    a = rand(M, K, seed=60, dtype=torch.bfloat16)
+    w = rand(N, K, seed=61, dtype=torch.bfloat16, scale=0.05)
+    want = (a.double() @ w.double().T).float()
+    wp = mfma.pack_weight(w) if packed else w
+    tol = 2e-6 * K ** 0.5 * float(want.abs().max()) + 1e-4
+    c = torch.full((M, N), 7.0, device=dev())
+    mfma.gemm(a, wp, c, packed=packed, tile=tile)
+    assert float((c - want).abs().max()) <= tol
+    base = rand(M, N, seed=62)
+    c2 = base.clone()
+    mfma.gemm(a, wp, c2, accumulate=True, packed=packed, tile=tile)
+    assert float((c2 - (base + want)).abs().max()) <= tol
+    c3 = base.clone()
+    mfma.gemm(a, wp, c3, accumulate=True, packed=packed, tile=tile)
+    assert torch.equal(c2, c3)          # the slices are added in a fixed order
+
+
 @pytest.mark.parametrize("M,N,K", [(17, 4096, 4096), (40, 1024, 512), (64, 4096, 12288), (64, 6144, 4096),
                                    (33, 272, 96)])
 def test_gemm_mfma_with_k_slices(M, N, K):
