@@ -103,6 +103,7 @@ def main():
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
     ap.add_argument("--workload", default="headline", choices=["headline", "qwen3-1.7b", "qwen3-32b"],
                     help="headline: BASELINE.json configs[2]; the others: configs[3] and configs[4]")
+    ap.add_argument("--prefill-tokens", type=int, default=2048, help="length of the prompt of the prefill figure")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run the 2,048-token prefill alone (for profiles); prints no JSON line")
     args = ap.parse_args()
@@ -189,8 +190,9 @@ def main():
         return (time.perf_counter() - t) / reps
 
     if args.prefill_only:
-        sec = prefill_run(2048, max(1, args.steps))
-        print(f"[bench] prefill 2048: {2048 / sec:.0f} tok/s, {sec * 1e3:.2f} ms", file=sys.stderr, flush=True)
+        sec = prefill_run(args.prefill_tokens, max(1, args.steps))
+        print(f"[bench] prefill {args.prefill_tokens}: {args.prefill_tokens / sec:.0f} tok/s, {sec * 1e3:.2f} ms",
+              file=sys.stderr, flush=True)
         return 0
     value, ms = decode_run(args.batch, args.steps, args.warmup)
     print(f"[bench] decode b{args.batch}: {value:.1f} tok/s, {ms:.3f} ms/step", file=sys.stderr, flush=True)
@@ -212,15 +214,15 @@ def main():
             "num_key_value_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
             "intermediate_size": I, "vocab_size": V, "rope_theta": cfg.rope_theta,
             "rms_norm_eps": cfg.rms_norm_eps, "tie_word_embeddings": cfg.tie_word_embeddings,
-            "global_batch": args.batch, "seq_len": context, "prefill_tokens": 2048,
+            "global_batch": args.batch, "seq_len": context, "prefill_tokens": args.prefill_tokens,
             "parallelism": "single GPU",
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_GBS, 4)},
     }
     if not args.no_points:
-        T = 2048
-        sec = prefill_run(T, 3)
+        T = args.prefill_tokens
+        sec = prefill_run(T, 5)
         flops = 2.0 * T * (layers * per_layer) + 2.0 * V * H \
             + layers * 4.0 * cfg.q_dim * T * (T + 1) / 2.0
         peak = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
