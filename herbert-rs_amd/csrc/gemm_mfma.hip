@@ -464,13 +464,12 @@ __device__ __forceinline__ void store_wave_tile(const f32x16 (&acc)[TN32][TM32],
 // in LDS as rows of 128 bytes, so that a load fetches whole 128-byte lines (8 rows an
 // instruction, 8 lanes a row) and not half lines twice; the 16-byte chunk c of row r sits at
 // chunk c ^ ((r >> 1) & 7) of its row, so that the operand reads of 16 rows at one k fall into
-// 16 different bank groups. The weights, which come from HBM, have a ring of WST stages; the
-// activations, which the L2 holds, one of 2.
+// 16 different bank groups. The weights have a ring of WST stages, the activations one of XST.
 // There is no branch in the main loop (the last step is peeled off), and what is no MFMA is
 // dealt out between the MFMAs by hand: a wave has an MFMA in the pipe while it issues its reads
 // and loads, also right after the barrier, where no other wave could fill in. Operands are in
 // two sets of registers: the reads of a k-step go out during the MFMAs of the one before.
-template <int EPI, bool PACKED, int TNB, int TMB, int WNW, int WMW, int WST>
+template <int EPI, bool PACKED, int TNB, int TMB, int WNW, int WMW, int WST, int XST>
 __global__ void __launch_bounds__(64 * WNW * WMW)
 gemm_tile_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* __restrict__ Cv, int M, int N,
                  int K, int ldc, int m_tiles, int n_tiles, float* __restrict__ partial) {
@@ -483,9 +482,12 @@ gemm_tile_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* _
     constexpr int NLW = 2 * WL, NLX = XR;               // a wave's loads per step
     static_assert(WBLK % NW == 0 && BM % (8 * NW) == 0, "the loads must divide over the waves");
     static_assert(TNB % 2 == 0 && TMB % 2 == 0, "a wave's tile is made of 32 x 32 pieces");
-    static_assert(WST == 2 || WST == 3, "the wait before the barrier counts on the loads of at most one later step");
+    static_assert((WST == 2 || WST == 3) && (XST == 2 || XST == 3),
+                  "the wait before the barrier counts on the loads of at most one later step");
+    constexpr bool X_FIRST = XST <= WST;                // in a step's loads: the operand with the shorter ring first
+    constexpr int LATER = (WST == 3 ? NLW : 0) + (XST == 3 ? NLX : 0);   // loads that may be in flight at the barrier
     constexpr int TN32 = TNB / 2, TM32 = TMB / 2;
-    extern __shared__ __attribute__((aligned(1024))) bf16 lds[];    // [WST][W_STAGE], then [2][X_STAGE]
+    extern __shared__ __attribute__((aligned(1024))) bf16 lds[];    // [WST][W_STAGE], then [XST][X_STAGE]
     bf16* const xlds = lds + WST * W_STAGE;
 
     int m_tile, n_tile;
@@ -525,15 +527,21 @@ gemm_tile_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* _
         if (m >= M) m = M - 1;
         xsrc[i] = X + (size_t)m * K + (((lane & 7) ^ ((r >> 1) & 7)) * 8) + (size_t)step0 * 64;
     }
-    // loads of a step, the activations first: those are waited for one step earlier than the weights
-    auto load_one = [&](int xstep, int wstep, int idx) {
-        if (idx < NLX) {
-            hb_load_to_lds(xsrc[idx] + (size_t)xstep * 64, xlds + (xstep & 1) * X_STAGE + (wave * XR + idx) * 512);
+    // The idx-th load of a step: activations of step xstep into stage xstage, weights of step
+    // wstep into stage wstage. The operand with the shorter ring comes first: it is the one
+    // that is needed a step earlier.
+    auto load_one = [&](int xstep, int xstage, int wstep, int wstage, int idx) {
+        const bool is_x = X_FIRST ? idx < NLX : idx >= NLW;
+        const int i = X_FIRST ? (is_x ? idx : idx - NLX) : (is_x ? idx - NLW : idx);
+        if (is_x) {
+            hb_load_to_lds(xsrc[i] + (size_t)xstep * 64, xlds + xstage * X_STAGE + (wave * XR + i) * 512);
         } else {
-            const int ks = (idx - NLX) / WL, i = (idx - NLX) % WL;
-            hb_load_to_lds(wsrc[i] + ((size_t)wstep * 2 + ks) * WSTEP, lds + (wstep % WST) * W_STAGE + ks * WBLK * 512 + (wave * WL + i) * 512);
+            const int ks = i / WL, w = i % WL;
+            hb_load_to_lds(wsrc[w] + ((size_t)wstep * 2 + ks) * WSTEP,
+                           lds + wstage * W_STAGE + ks * WBLK * 512 + (wave * WL + w) * 512);
         }
     };
+    auto load_is_x = [&](int idx) { return X_FIRST ? idx < NLX : idx >= NLW; };
 
     f32x16 acc[TN32][TM32];
 #pragma unroll
@@ -559,7 +567,7 @@ gemm_tile_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* _
         if (r < TN32)
             wv[set][h][r] = *(const bf16x8*)(lds + (step % WST) * W_STAGE + ks * WBLK * 512 + w_lane + r * 1024 + h * 256);
         else
-            xv[set][h][r - TN32] = *(const bf16x8*)(xlds + (step & 1) * X_STAGE + x_lane + (r - TN32) * 32 * 64 +
+            xv[set][h][r - TN32] = *(const bf16x8*)(xlds + (step % XST) * X_STAGE + x_lane + (r - TN32) * 32 * 64 +
                                                     (((4 * ks + 2 * h + g2) ^ x_swizzle) * 8));
     };
     // between the MFMAs j and j + 1 of a k-step: nl loads and NR reads, dealt out evenly over the
@@ -577,16 +585,15 @@ gemm_tile_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* _
     };
     auto clamp = [&](int step) { return step < nsteps ? step : nsteps - 1; };   // past the end: the last step again
 
-    // in flight before the loop: activations of steps 0 and 1, weights of steps 0 .. WST - 1
+    // in flight before the loop: steps 0 and 1, and step 2 of what has a ring of three stages
 #pragma unroll
-    for (int i = 0; i < NLX + NLW; ++i) load_one(0, 0, i);
+    for (int i = 0; i < NLX + NLW; ++i) load_one(0, 0, 0, 0, i);
 #pragma unroll
-    for (int i = 0; i < NLX + NLW; ++i) load_one(clamp(1), clamp(1), i);
+    for (int i = 0; i < NLX + NLW; ++i) load_one(clamp(1), 1, clamp(1), 1, i);
 #pragma unroll
-    for (int st = 2; st < WST; ++st)
-#pragma unroll
-        for (int i = NLX; i < NLX + NLW; ++i) load_one(0, clamp(st), i);
-    hb_wait_vmcnt<NLX + (WST - 1) * NLW>();
+    for (int i = 0; i < NLX + NLW; ++i)
+        if (load_is_x(i) ? XST == 3 : WST == 3) load_one(clamp(2), 2, clamp(2), 2, i);
+    hb_wait_vmcnt<NLX + NLW + LATER>();
     hb_workgroup_barrier();
 #pragma unroll
     for (int i = 0; i < NR; ++i) read_one(0, 0, 0, i);
@@ -602,23 +609,15 @@ gemm_tile_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* _
         // Step t + 1 has landed (of what this wave has in flight only the weights of the later
         // steps may be missing), after the barrier for every wave, and nobody reads step t any
         // more: between the MFMAs of its second k-step go the loads into its stages, the
-        // activations of step t + 2 and the weights of step t + WST, and the reads of step t + 1.
-        hb_wait_vmcnt<(WST - 2) * NLW>();
+        // activations of step t + XST and the weights of step t + WST, and the reads of step t + 1.
+        hb_wait_vmcnt<LATER>();
         hb_workgroup_barrier();
-        const int xstep = clamp(t + 2), wstep = clamp(t + WST);
+        const int xstep = clamp(t + XST), wstep = clamp(t + WST);
 #pragma unroll
         for (int j = 0; j < NM; ++j) {
             mfma_one(1, j);
-            between(j, NLX + NLW,
-                    [&](int i) {
-                        // a clamped step goes where step t + 2 (t + WST) would: into the stage just freed
-                        if (i < NLX) {
-                            hb_load_to_lds(xsrc[i] + (size_t)xstep * 64, xlds + (t & 1) * X_STAGE + (wave * XR + i) * 512);
-                        } else {
-                            const int ks = (i - NLX) / WL, w = (i - NLX) % WL;
-                            hb_load_to_lds(wsrc[w] + ((size_t)wstep * 2 + ks) * WSTEP, lds + (t % WST) * W_STAGE + ks * WBLK * 512 + (wave * WL + w) * 512);
-                        }
-                    },
+            // (a clamped step goes where step t + XST or t + WST would: into the stage just freed)
+            between(j, NLX + NLW, [&](int i) { load_one(xstep, t % XST, wstep, t % WST, i); },
                     [&](int i) { read_one(0, t + 1, 0, i); });
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -793,21 +792,21 @@ static int launch_tiles(Kernel kern, size_t lds, int threads, long total, int sl
     } while (0)
 
 // slices > 1: the sums of the slices go to `partial`; the caller adds them up afterwards
-template <int TNB, int TMB, int WNW, int WMW, int WST>
+template <int TNB, int TMB, int WNW, int WMW, int WST, int XST>
 static int launch_tile64(const void* X, const void* W, void* C, int M, int N, int K, int ldc, int epi, int packed,
                          hipStream_t stream, int slices = 1, float* partial = nullptr) {
     constexpr int BN = 16 * TNB * WNW, BM = 16 * TMB * WMW;
     HB_REQUIRE(K % 64 == 0, "gemm_mfma: K=%d is no multiple of 64", K);
     const int m_tiles = (M + BM - 1) / BM, n_tiles = (N + BN - 1) / BN;
     const long total = (long)m_tiles * n_tiles;
-    const size_t lds = (size_t)(WST * BN + 2 * BM) * 64 * sizeof(bf16);
+    const size_t lds = (size_t)(WST * BN + XST * BM) * 64 * sizeof(bf16);
     const int threads = 64 * WNW * WMW;
     const bf16* x = (const bf16*)X;
     const bf16* w = (const bf16*)W;
     HB_REQUIRE(slices >= 1 && (slices == 1 || (partial && epi != EPI_SWIGLU)), "gemm_mfma: bad slices");
     HB_REQUIRE((K / 64 + slices - 1) / slices * (slices - 1) < K / 64, "gemm_mfma: a slice of K would be empty");
 #define EXTRA , partial
-    TILE_DISPATCH(gemm_tile_kernel, TNB, TMB, WNW, WMW, WST);
+    TILE_DISPATCH(gemm_tile_kernel, TNB, TMB, WNW, WMW, WST, XST);
 #undef EXTRA
 }
 
@@ -888,11 +887,11 @@ extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N,
     HB_REQUIRE(slices == 1 || (size_t)slices * M * N <= workspace_floats, "gemm_mfma: no room for %d slices", slices);
     int rc;
     switch (tile) {
-        // (a third weight stage, measured with weights that come from HBM: a gain of a tenth for
-        // 256 x 128, none for the other two)
-        case 188: rc = launch_tile64<8, 8, 2, 2, 2>(X, W, C, M, N, K, ldc, epi, packed, stream, slices, workspace); break;   // 256 x 256
-        case 142: rc = launch_tile64<8, 4, 2, 2, 3>(X, W, C, M, N, K, ldc, epi, packed, stream, slices, workspace); break;   // 256 (n) x 128 (m)
-        case 122: rc = launch_tile64<4, 4, 2, 2, 2>(X, W, C, M, N, K, ldc, epi, packed, stream, slices, workspace); break;   // 128 x 128, two to a CU
+        // (ring depths, measured with weights that come from HBM: a third weight stage gains a
+        // tenth for 256 x 128 and nothing for the other two; a third activation stage nothing)
+        case 188: rc = launch_tile64<8, 8, 2, 2, 2, 2>(X, W, C, M, N, K, ldc, epi, packed, stream, slices, workspace); break;   // 256 x 256
+        case 142: rc = launch_tile64<8, 4, 2, 2, 3, 2>(X, W, C, M, N, K, ldc, epi, packed, stream, slices, workspace); break;   // 256 (n) x 128 (m)
+        case 122: rc = launch_tile64<4, 4, 2, 2, 2, 2>(X, W, C, M, N, K, ldc, epi, packed, stream, slices, workspace); break;   // 128 x 128, two to a CU
         case 123:                                                                                                           // 128 x 128, K in steps of 32
             HB_REQUIRE(slices == 1, "gemm_mfma: this tile does not cut K");
             return launch_tile32<4, 4, 2, 2, 4>(X, W, C, M, N, K, ldc, epi, packed, stream);
