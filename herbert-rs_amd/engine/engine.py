@@ -13,9 +13,9 @@ import torch
 
 from ..cache import Cache
 from ..config import load_config
-from ..errors import BackendError, RequestError
+from ..errors import BackendError, ModelLoadError, RequestError
 from ..parts import Runtime
-from ..weights import read_tensors
+from ..weights import random_tensor, read_tensor, read_tensors
 from . import batch as batching
 from .batch import StaticDecodeMeta, StepEntry
 from .model import Model
@@ -55,6 +55,7 @@ class Engine:
         self.steps_run = 0
         self.use_graphs = bool(use_graphs) and self.model.graph_safe
         self._decode = {}       # batch size -> _DecodeState
+        self._tensor_source = None      # how get_tensor finds a tensor again: set by the constructors below
 
     # ---- construction
     @classmethod
@@ -65,7 +66,9 @@ class Engine:
         spec = arch.build_spec(config)
         needs = Model(spec).tensor_needs()
         tensors = read_tensors(folder, needs)
-        return cls(config, spec, tensors, dtype, max_tokens, max_slots, device, use_graphs)
+        engine = cls(config, spec, tensors, dtype, max_tokens, max_slots, device, use_graphs)
+        engine._tensor_source = lambda name: read_tensor(folder, name, needs)
+        return engine
 
     @classmethod
     def from_config(cls, config, architecture=None, seed=0, dtype="bfloat16", weight_dtype=None,
@@ -78,7 +81,22 @@ class Engine:
         dev = torch.device(device) if device is not None else require_gpu()
         needs = Model(spec).tensor_needs()
         tensors = random_tensors(needs, seed, weight_dtype or dtype, std, norm_std, device=str(dev))
-        return cls(config, spec, tensors, dtype, max_tokens, max_slots, dev, use_graphs)
+        engine = cls(config, spec, tensors, dtype, max_tokens, max_slots, dev, use_graphs)
+
+        def again(name):
+            if name not in needs:
+                raise ModelLoadError(f"the model has no tensor {name!r}; it has: " + ", ".join(sorted(needs)))
+            return random_tensor(name, needs[name], seed, weight_dtype or dtype, std, norm_std, device=str(dev)).cpu()
+        engine._tensor_source = again
+        return engine
+
+    def get_tensor(self, name):
+        """The weight tensor `name` (the checkpoint's own name) as it is stored, on the CPU. The
+        parts keep their weights in the order their kernels want; this reads the tensor again from
+        where the engine's weights came from."""
+        if self._tensor_source is None:
+            raise ModelLoadError("this engine was built from tensors in memory; it cannot read them again")
+        return self._tensor_source(name)
 
     # ---- slots
     def alloc_slot(self):

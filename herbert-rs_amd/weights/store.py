@@ -166,3 +166,23 @@ def read_tensors(folder, needs, device="cpu"):
             parts.append(f"  stored twice ({len(duplicate)}): " + ", ".join(sorted(duplicate)))
         raise ModelLoadError("\n".join(parts))
     return found
+
+
+def read_tensor(folder, name, needs):
+    """The one tensor `name` of `needs` as `folder` stores it (cut out of a fused tensor if that is
+    how it is stored), on the CPU."""
+    if name not in needs:
+        raise ModelLoadError(f"the model has no tensor {name!r}; it has: " + ", ".join(sorted(needs)))
+    for path in shard_files(folder):
+        with safe_open(path, framework="pt", device="cpu") as f:
+            for stored in f.keys():
+                cname = canonical_name(stored)
+                if cname == name:
+                    t = f.get_tensor(stored)
+                    return t.to(stored_dtype(t))
+                targets = _fused_targets(cname, needs)
+                if targets and name in targets:
+                    t = f.get_tensor(stored)
+                    row = sum(needs[n].shape[0] for n in targets[:targets.index(name)])
+                    return t[row:row + needs[name].shape[0]].contiguous().to(stored_dtype(t))
+    raise ModelLoadError(f"{folder} holds no tensor {name!r}")

@@ -212,6 +212,12 @@ def test_names_are_normalised_and_fused_tensors_cut(model_root, tmp_path):
     save_file(other, str(tmp_path / "model.safetensors"))
     got = read_tensors(str(tmp_path), needs_of(TINY_B))
     assert set(got) == set(plain) and all(torch.equal(got[k], plain[k]) for k in plain)
+    # one tensor by its own name, also out of a fused one
+    from herbert_rs_amd.weights import read_tensor
+    for name in ("model.layers.2.self_attn.k_proj.weight", "model.layers.1.mlp.up_proj.weight", "model.norm.weight"):
+        assert torch.equal(read_tensor(str(tmp_path), name, needs_of(TINY_B)), plain[name])
+    with pytest.raises(ModelLoadError, match="no tensor"):
+        read_tensor(str(tmp_path), "model.layers.9.mlp.up_proj.weight", needs_of(TINY_B))
     other["model.language_model.layers.0.self_attn.qkv_proj.weight"] = torch.zeros(10, 96)
     save_file(other, str(tmp_path / "model.safetensors"))
     with pytest.raises(ModelLoadError, match=r"qkv_proj.weight: expected \[320, 96\], got \[10, 96\]"):

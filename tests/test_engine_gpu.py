@@ -159,6 +159,25 @@ def test_generation_stops_on_eos_and_other_sequences_go_on(model_root):
     assert engine.cache.slots.held_count == 0
 
 
+def test_get_tensor_gives_the_weights_as_stored(model_root):
+    from safetensors.torch import load_file
+    from herbert_rs_amd.errors import ModelLoadError
+    folder = make_folder(model_root, "B", "bfloat16")
+    stored = load_file(os.path.join(folder, "model.safetensors"))
+    engine = hb.load(folder, dtype="bfloat16", cache_tokens=128)
+    for name in ("model.layers.1.self_attn.q_proj.weight", "model.layers.2.mlp.gate_proj.weight", "lm_head.weight"):
+        assert torch.equal(engine.get_tensor(name), stored[name])
+    with pytest.raises(ModelLoadError, match="no tensor"):
+        engine.get_tensor("model.layers.7.mlp.gate_proj.weight")
+    from herbert_rs_amd.engine import Engine
+    from herbert_rs_amd.config import load_config
+    _, config = load_config(folder)
+    seeded = Engine.from_config(config, seed=5, dtype="bfloat16", max_tokens=128)
+    again = Engine.from_config(config, seed=5, dtype="bfloat16", max_tokens=128)
+    t = seeded.get_tensor("model.layers.0.mlp.down_proj.weight")
+    assert t.shape == (96, 224) and torch.equal(t, again.get_tensor("model.layers.0.mlp.down_proj.weight"))
+
+
 def test_step_errors(model_root):
     folder = make_folder(model_root, "A", "float32")
     engine = hb.load(folder, dtype="float32", cache_tokens=128)
