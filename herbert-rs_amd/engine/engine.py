@@ -15,7 +15,7 @@ from ..cache import Cache
 from ..config import load_config
 from ..errors import BackendError, ModelLoadError, RequestError
 from ..parts import Runtime
-from ..weights import random_tensor, read_tensor, read_tensors
+from ..weights import read_tensor, read_tensors
 from . import batch as batching
 from .batch import StaticDecodeMeta, StepEntry
 from .model import Model
@@ -86,7 +86,8 @@ class Engine:
         def again(name):
             if name not in needs:
                 raise ModelLoadError(f"the model has no tensor {name!r}; it has: " + ", ".join(sorted(needs)))
-            return random_tensor(name, needs[name], seed, weight_dtype or dtype, std, norm_std, device=str(dev)).cpu()
+            return random_tensors({name: needs[name]}, seed, weight_dtype or dtype, std, norm_std,
+                                  device=str(dev))[name].cpu()
         engine._tensor_source = again
         return engine
 
