@@ -22,6 +22,7 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 #define EPI_STORE 0
 #define EPI_ADD 1
 #define EPI_SWIGLU 2
+#define EPI_QKV 3
 
 __device__ __forceinline__ float silu_mul(float g, float u) { return g / (1.0f + __expf(-g)) * u; }
 
@@ -460,6 +461,115 @@ __device__ __forceinline__ void store_wave_tile(const f32x16 (&acc)[TN32][TM32],
     }
 }
 
+// The q/k/v projection of prompts with what follows it, for heads of 128 (a wave's tile is 128
+// columns wide: one head): per-head RMSNorm (if weights are given), rotation over the whole head
+// (if tables are given), queries to q_out [M, nq 128] and keys and values into the pages (values
+// transposed), all bfloat16. The float32 sums never go to memory.
+struct QkvEpilogue {
+    bf16* q_out;
+    bf16* k_cache;               // [pages, nkv, 64, 128]
+    bf16* v_cache;               // [pages, nkv, 128, 64]
+    const int* positions;        // of every row
+    const int* seq_of;           // row -> sequence of the step
+    const int* slots;            // sequence -> slot
+    const int* page_table;       // [slots, max_pages]
+    int max_pages;
+    const float* q_norm_w;
+    const float* k_norm_w;
+    const float* cos_t;          // [positions, 64]
+    const float* sin_t;
+    float eps;
+    int nq, nkv;
+};
+
+// lane: row m = m_base + 32 b + c32; register 4 q + j of piece a: element 32 a + 8 q + 4 g2 + j of the head
+template <int TN32, int TM32>
+__device__ __forceinline__ void store_wave_tile_qkv(f32x16 (&acc)[TN32][TM32], const QkvEpilogue& e, int M, int N,
+                                                    int m_base, int n_base, int c32, int g2) {
+    static_assert(TN32 == 4, "a wave's tile must be one head of 128 wide");
+    if (n_base >= N) return;
+    const int head = n_base / 128;
+    const bool is_q = head < e.nq, is_v = head >= e.nq + e.nkv;
+    const float* norm_w = is_q ? e.q_norm_w : e.k_norm_w;
+#pragma unroll
+    for (int b = 0; b < TM32; ++b) {
+        const int m = m_base + 32 * b + c32;
+        const int mc = m < M ? m : M - 1;
+        const int pos = e.positions[mc];
+        if (!is_v) {
+            if (norm_w) {
+                float ss = 0.f;
+#pragma unroll
+                for (int a = 0; a < 4; ++a)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) ss = fmaf(acc[a][b][i], acc[a][b][i], ss);
+                ss += __shfl_xor(ss, 32, 64);
+                const float inv = 1.0f / sqrtf(ss / 128.0f + e.eps);
+#pragma unroll
+                for (int a = 0; a < 4; ++a)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const f32x4 w = *(const f32x4*)(norm_w + 32 * a + 8 * q + 4 * g2);
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) acc[a][b][4 * q + j] = acc[a][b][4 * q + j] * inv * w[j];
+                    }
+            }
+            if (e.cos_t) {
+                // element d < 64 pairs with d + 64: pieces a and a + 2, the same register
+#pragma unroll
+                for (int a = 0; a < 2; ++a)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const size_t at = (size_t)pos * 64 + 32 * a + 8 * q + 4 * g2;
+                        const f32x4 c = *(const f32x4*)(e.cos_t + at), s = *(const f32x4*)(e.sin_t + at);
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            const float x0 = acc[a][b][4 * q + j], x1 = acc[a + 2][b][4 * q + j];
+                            acc[a][b][4 * q + j] = x0 * c[j] - x1 * s[j];
+                            acc[a + 2][b][4 * q + j] = x0 * s[j] + x1 * c[j];
+                        }
+                    }
+            }
+        }
+        if (m >= M) continue;
+        if (is_q) {
+            bf16* dst = e.q_out + ((size_t)m * e.nq + head) * 128;
+#pragma unroll
+            for (int a = 0; a < 4; ++a)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    bf16x4 v;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) v[j] = (__bf16)acc[a][b][4 * q + j];
+                    *(bf16x4*)((__bf16*)dst + 32 * a + 8 * q + 4 * g2) = v;
+                }
+            continue;
+        }
+        const int page = e.page_table[(size_t)e.slots[e.seq_of[m]] * e.max_pages + pos / 64];
+        const int in_page = pos % 64;
+        if (!is_v) {
+            bf16* dst = e.k_cache + (((size_t)page * e.nkv + (head - e.nq)) * 64 + in_page) * 128;
+#pragma unroll
+            for (int a = 0; a < 4; ++a)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    bf16x4 v;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) v[j] = (__bf16)acc[a][b][4 * q + j];
+                    *(bf16x4*)((__bf16*)dst + 32 * a + 8 * q + 4 * g2) = v;
+                }
+        } else {
+            // transposed pages: for one element the 32 lanes of a half wave write 32 neighbouring tokens
+            bf16* dst = e.v_cache + ((size_t)page * e.nkv + (head - e.nq - e.nkv)) * 128 * 64 + in_page;
+#pragma unroll
+            for (int a = 0; a < 4; ++a)
+#pragma unroll
+                for (int i = 0; i < 16; ++i)
+                    dst[(size_t)(32 * a + 8 * (i >> 2) + 4 * g2 + (i & 3)) * 64] = hb_from_float<bf16>(acc[a][b][i]);
+        }
+    }
+}
+
 // K in steps of 64. A step's weights are two k-steps of 32 (blocks as above); its activations lie
 // in LDS as rows of 128 bytes, so that a load fetches whole 128-byte lines (8 rows an
 // instruction, 8 lanes a row) and not half lines twice; the 16-byte chunk c of row r sits at
@@ -472,7 +582,7 @@ __device__ __forceinline__ void store_wave_tile(const f32x16 (&acc)[TN32][TM32],
 template <int EPI, bool PACKED, int TNB, int TMB, int WNW, int WMW, int WST, int XST>
 __global__ void __launch_bounds__(64 * WNW * WMW)
 gemm_tile_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* __restrict__ Cv, int M, int N,
-                 int K, int ldc, int m_tiles, int n_tiles, float* __restrict__ partial) {
+                 int K, int ldc, int m_tiles, int n_tiles, float* __restrict__ partial, QkvEpilogue qkv) {
     constexpr int NW = WNW * WMW;
     constexpr int BN = 16 * TNB * WNW, BM = 16 * TMB * WMW;
     constexpr int WBLK = BN / 16;                       // weight blocks of a k-step of 32
@@ -634,7 +744,9 @@ gemm_tile_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* _
         for (int j = 0; j < NM; ++j) mfma_one(1, j);
     }
     hb_wait_vmcnt<0>();      // the loads past the end (repeats of the last step) have landed too
-    if (gridDim.y > 1)
+    if constexpr (EPI == EPI_QKV)
+        store_wave_tile_qkv<TN32, TM32>(acc, qkv, M, N, m0 + wm * TMB * 16, n0 + wn * TNB * 16, c32, g2);
+    else if (gridDim.y > 1)
         store_wave_tile<EPI_STORE, TN32, TM32>(acc, partial + (size_t)blockIdx.y * M * N, M, N, N,
                                                m0 + wm * TMB * 16, n0 + wn * TNB * 16, c32, g2);
     else
@@ -805,7 +917,7 @@ static int launch_tile64(const void* X, const void* W, void* C, int M, int N, in
     const bf16* w = (const bf16*)W;
     HB_REQUIRE(slices >= 1 && (slices == 1 || (partial && epi != EPI_SWIGLU)), "gemm_mfma: bad slices");
     HB_REQUIRE((K / 64 + slices - 1) / slices * (slices - 1) < K / 64, "gemm_mfma: a slice of K would be empty");
-#define EXTRA , partial
+#define EXTRA , partial, QkvEpilogue{}
     TILE_DISPATCH(gemm_tile_kernel, TNB, TMB, WNW, WMW, WST, XST);
 #undef EXTRA
 }
@@ -826,6 +938,31 @@ static int launch_tile32(const void* X, const void* W, void* C, int M, int N, in
 #undef EXTRA
 }
 #undef TILE_DISPATCH
+
+// The q/k/v projection of a step with many rows, fused with norm, rotation and cache write
+// (see QkvEpilogue). X [M, K] bf16; W [(nq + 2 nkv) 128, K] bf16, rows q | k | v; 256 x 256 tiles.
+extern "C" int hb_gemm_qkv_mfma(const void* X, const void* W, int M, int K, int packed, void* q_out, void* k_cache,
+                                void* v_cache, const int* positions, const int* seq_of, const int* slots,
+                                const int* page_table, int max_pages, int page_size, const float* q_norm_w,
+                                const float* k_norm_w, const float* cos_t, const float* sin_t, float eps, int nq,
+                                int nkv, int hd, hipStream_t stream) {
+    HB_REQUIRE(hd == 128 && page_size == 64, "gemm_qkv: heads of 128 and pages of 64 tokens only");
+    HB_REQUIRE(M > 0 && nq > 0 && nkv > 0 && K > 0 && K % 64 == 0, "gemm_qkv: bad sizes (M=%d, K=%d)", M, K);
+    HB_REQUIRE((cos_t == nullptr) == (sin_t == nullptr), "gemm_qkv: cos and sin tables come together");
+    const int N = (nq + 2 * nkv) * 128;
+    const QkvEpilogue e = {(bf16*)q_out, (bf16*)k_cache, (bf16*)v_cache, positions, seq_of, slots, page_table,
+                           max_pages, q_norm_w, k_norm_w, cos_t, sin_t, eps, nq, nkv};
+    const int m_tiles = (M + 255) / 256, n_tiles = (N + 255) / 256;
+    const long total = (long)m_tiles * n_tiles;
+    const size_t lds = (size_t)(2 * 256 + 2 * 256) * 64 * sizeof(bf16);
+    const bf16* x = (const bf16*)X;
+    const bf16* w = (const bf16*)W;
+    if (packed)
+        return launch_tiles(gemm_tile_kernel<EPI_QKV, true, 8, 8, 2, 2, 2, 2>, lds, 256, total, 1, x, w, nullptr, M, N, K,
+                            N, m_tiles, n_tiles, stream, (float*)nullptr, e);
+    return launch_tiles(gemm_tile_kernel<EPI_QKV, false, 8, 8, 2, 2, 2, 2>, lds, 256, total, 1, x, w, nullptr, M, N, K, N,
+                        m_tiles, n_tiles, stream, (float*)nullptr, e);
+}
 
 // C (+)= X @ W^T. X [M, K] bf16, W [N, K] bf16. epi 0: C f32 [M, N] stored; 1: added to;
 // 2: W's rows are gate/up interleaved in blocks of 16 and C is bf16 [M, N / 2] = silu(gate) * up.

@@ -13,6 +13,7 @@ _I = ctypes.c_int
 _F = ctypes.c_float
 lib.register_signatures("gemm_mfma", {
     "hb_gemm_mfma": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _F, _I, _P, ctypes.c_size_t, _P],
+    "hb_gemm_qkv_mfma": [_P, _P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _F, _I, _I, _I, _P],
 })
 
 EPI_STORE, EPI_ADD, EPI_SWIGLU = 0, 1, 2
@@ -108,6 +109,51 @@ def gemm(a, w, out, accumulate=False, packed=False, norm=None, tile=0):
     lib.call("gemm_mfma", "hb_gemm_mfma", a.data_ptr(), w.data_ptr(), out.data_ptr(), M, N, K, N,
              EPI_ADD if accumulate else EPI_STORE, 1 if packed else 0, norm_ptr, eps, int(tile), ws_ptr,
              ws_floats, _stream())
+
+
+QKV_FUSE_MIN_M = 1024      # below that the plain product picks smaller tiles or cuts K, and wins
+
+
+def gemm_qkv_fusable(a, w, meta, kv, nq, nkv, hd, rot_dims):
+    """True if the q/k/v projection of this step should norm, rotate and write the cache itself:
+    a long bfloat16 prompt step, heads of 128 rotated whole or not at all, pages of 64 tokens."""
+    return (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and kv.k.dtype == torch.bfloat16
+            and a.shape[0] >= QKV_FUSE_MIN_M and a.shape[1] % 64 == 0 and hd == 128 and kv.page_size == 64
+            and rot_dims in (0, hd) and w.shape[0] == (nq + 2 * nkv) * hd and meta.num_tokens == a.shape[0])
+
+
+def gemm_qkv(a, w, packed, q_norm_w, k_norm_w, cos, sin, meta, kv, q_out, nq, nkv, hd, eps):
+    """q_out bf16 [M, nq hd] and the pages of kv from a bf16 [M, K] @ w[(nq + 2 nkv) hd, K]^T: the
+    product, the per-head norm (if weights are given), the rotation (if tables are given) and the
+    cache write in one kernel."""
+    M, K = a.shape
+    _check(a, "a", torch.bfloat16, (M, K))
+    _check(w, "w", torch.bfloat16, ((nq + 2 * nkv) * hd, K))
+    _check(q_out, "q_out", torch.bfloat16, (M, nq * hd))
+    pages = kv.k.shape[0]
+    _check(kv.k, "key pages", torch.bfloat16, (pages, nkv, 64, hd))
+    _check(kv.v, "value pages", torch.bfloat16, (pages, nkv, hd, 64))
+    _check(kv.page_table, "page_table", torch.int32, (None, None))
+    _check(meta.positions, "positions", torch.int32, (M,))
+    _check(meta.seq_of, "seq_of", torch.int32, (M,))
+    _check(meta.slots, "slots", torch.int32, (meta.num_seqs,))
+    if hd != 128 or K % 64:
+        raise BackendError(f"the fused q/k/v product refuses head_dim {hd}, K={K}")
+    for t, name in ((q_norm_w, "q_norm"), (k_norm_w, "k_norm")):
+        if t is not None:
+            _check(t, name, torch.float32, (hd,))
+    if (cos is None) != (sin is None):
+        raise BackendError("cos and sin tables come together")
+    if cos is not None:
+        _check(cos, "cos", torch.float32, (None, hd // 2))
+        _check(sin, "sin", torch.float32, tuple(cos.shape))
+        if meta.max_position >= cos.shape[0]:
+            raise BackendError(f"position {meta.max_position} beyond the rotation table ({cos.shape[0]} rows)")
+    ptr = lambda t: None if t is None else t.data_ptr()
+    lib.call("gemm_mfma", "hb_gemm_qkv_mfma", a.data_ptr(), w.data_ptr(), M, K, 1 if packed else 0, q_out.data_ptr(),
+             kv.k.data_ptr(), kv.v.data_ptr(), meta.positions.data_ptr(), meta.seq_of.data_ptr(),
+             meta.slots.data_ptr(), kv.page_table.data_ptr(), kv.page_table.shape[1], kv.page_size, ptr(q_norm_w),
+             ptr(k_norm_w), ptr(cos), ptr(sin), float(eps), nq, nkv, hd, _stream())
 
 
 def interleave_gate_up(gate, up):

@@ -100,13 +100,24 @@ class Attention(Part):
         kv = ctx.cache.kv_view(ctx.cache_entry)
         write_kv = not self.reads_cache_only
         width = self.q_dim + (2 * self.kv_dim if write_kv else 0)
+        rot = self.position.rotation()
+        cos, sin, rot_dims = rot if rot is not None else (None, None, 0)
+        if write_kv and fused_norm is None and rt.dtype == torch.bfloat16:
+            from ..kernels import mfma
+            if mfma.gemm_qkv_fusable(y, self.qkv.weight, ctx.meta, kv, self.nq, self.nkv, self.hd, rot_dims):
+                # a long prompt: the projection norms, rotates and writes the cache in its epilogue
+                q = rt.buffer("q", (T, self.q_dim))
+                mfma.gemm_qkv(y, self.qkv.weight, self.qkv.packed, self.q_norm_w, self.k_norm_w, cos, sin, ctx.meta,
+                              kv, q, self.nq, self.nkv, self.hd, self.eps)
+                attn = rt.buffer("attn", (T, self.q_dim))
+                self.attend(ctx, q, kv, attn)
+                self.o.forward(attn, x, accumulate=True)
+                return
         qkv = rt.buffer("qkv", (T, width), torch.float32)
         if fused_norm is not None:
             self.qkv.forward_normed(x, fused_norm.w, fused_norm.eps, qkv)
         else:
             self.qkv.forward(y, qkv)
-        rot = self.position.rotation()
-        cos, sin, rot_dims = rot if rot is not None else (None, None, 0)
         attn = rt.buffer("attn", (T, self.q_dim))
         if write_kv and rt.dtype == torch.bfloat16:
             from ..kernels import mfma

@@ -291,6 +291,48 @@ def test_qk_norm_rope_write(nq, nkv, hd, rot, norm, dtype):
         assert float((kv.v.double().cpu() - exp_v).abs().max()) <= tol * float(exp_v.abs().max())
 
 
+@pytest.mark.parametrize("packed", [True, False])
+@pytest.mark.parametrize("nq,nkv,norm,rope", [(4, 2, True, True), (3, 1, False, True), (2, 2, True, False), (1, 1, True, True)])
+def test_gemm_qkv_with_norm_rotation_and_cache_write(nq, nkv, norm, rope, packed):
+    """The q/k/v projection that norms, rotates and writes the pages in its epilogue against the
+    product followed by the kernel of its own: prompts that cross pages, rows that are no
+    multiple of the tile, an odd number of heads (half a tile of columns is empty)."""
+    from herbert_rs_amd.cache.paged import LayerKV
+    from herbert_rs_amd.kernels import mfma, ops
+    hd, K = 128, 192
+    lengths, new = [330, 70, 300, 64], [330, 7, 190, 64]
+    meta, kv, _ = paged_case(lengths, new, nkv, hd, torch.bfloat16, seed=nq)
+    kv2 = LayerKV(kv.k.clone(), kv.v.clone(), kv.page_table, 64, 0)
+    T = sum(new)
+    a = rand(T, K, seed=70, dtype=torch.bfloat16)
+    w = rand((nq + 2 * nkv) * hd, K, seed=71, dtype=torch.bfloat16, scale=0.1)
+    qw = (1 + rand(hd, seed=72, scale=0.3)) if norm else None
+    kw = (1 + rand(hd, seed=73, scale=0.3)) if norm else None
+    cos = sin = None
+    if rope:
+        ang = torch.arange(512, dtype=torch.float32)[:, None] * (10000.0 ** (-torch.arange(hd // 2) / (hd // 2)))[None]
+        cos, sin = ang.cos().to(dev()).contiguous(), ang.sin().to(dev()).contiguous()
+    eps = 1e-5
+    wp = mfma.pack_weight(w) if packed else w
+    qkv = torch.empty(T, (nq + 2 * nkv) * hd, device=dev())
+    mfma.gemm(a, wp, qkv, packed=packed)
+    want_q = torch.full((T, nq * hd), 9.0, dtype=torch.bfloat16, device=dev())
+    ops.qk_norm_rope_write(qkv, qw, kw, cos, sin, hd if rope else 0, meta, kv, want_q, nq, nkv, hd, eps)
+    got_q = torch.full((T, nq * hd), 7.0, dtype=torch.bfloat16, device=dev())
+    old = mfma.QKV_FUSE_MIN_M
+    mfma.QKV_FUSE_MIN_M = 64
+    try:
+        assert mfma.gemm_qkv_fusable(a, wp, meta, kv2, nq, nkv, hd, hd if rope else 0)
+    finally:
+        mfma.QKV_FUSE_MIN_M = old
+    mfma.gemm_qkv(a, wp, packed, qw, kw, cos, sin, meta, kv2, got_q, nq, nkv, hd, eps)
+    # the two paths add the squares and the products in other orders: an element may round the other way
+    for got, want in ((got_q, want_q), (kv2.k, kv.k), (kv2.v, kv.v)):
+        d = (got.float() - want.float()).abs()
+        assert float(d.max()) <= 2 ** -7 * float(want.float().abs().max())
+        assert float((d > 0).float().mean()) < 2e-2
+
+
 @pytest.mark.parametrize("nq,nkv,hd,window,norm,rope", [(4, 1, 128, 0, True, True), (32, 8, 128, 0, True, True),
                                                         (6, 2, 32, 0, True, False), (5, 1, 64, 70, False, True),
                                                         (3, 3, 128, 100, True, True), (64, 2, 64, 0, False, False)])
