@@ -12,11 +12,13 @@
 // 8 consecutive keys: V^T operands are single 16-byte reads.
 //
 // prefill: one workgroup = 32 consecutive tokens of one sequence x up to 4 query heads of one
-//          kv head (one wave each); K and V^T pages are staged in LDS once for all of them.
+//          kv head (one wave each); K and V^T pages go through a ring of two LDS stages once
+//          for all of them, the keys a page ahead of the values.
 // decode:  one wave = one sequence x one kv head x one range of pages, all query heads of the
 //          group as columns; operands stream from global memory (each byte is used once);
-//          partial (max, sum, O) per range are merged by a second kernel in the fixed order
-//          of the ranges.
+//          partial (reference, sum, O) per range are merged by a second kernel in the fixed
+//          order of the ranges. The kernel can also norm and rotate q and k and write the new
+//          token's key and value itself.
 #include "common.h"
 #include <math.h>
 

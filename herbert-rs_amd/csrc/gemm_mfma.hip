@@ -1,15 +1,17 @@
 // bfloat16 matrix products on the gfx950 matrix cores, float32 accumulation:
 //   C[m, n] (+)= sum_k X[m, k] * W[n, k]        X [M, K], W [N, K], both k-contiguous
-// Two kernels share the epilogues:
 //   skinny (M <= 64, decoding): HBM-bound. The weights stream from memory straight into
-//     MFMA operands (each is used once), four waves of a workgroup split K between them
-//     and add their parts through LDS in a fixed order.
-//   tiled (M > 64, prompts): 256 x 256 or 128 x 128 tiles loaded from global memory straight
-//     into a ring of LDS stages, one or two k-steps ahead of the MFMAs that consume them.
-// In both the weight rows are the MFMA's first operand, so a lane ends up with four
+//     16x16x32 MFMA operands (each is used once), the waves of a workgroup split K between
+//     them and add their parts through LDS in a fixed order.
+//   tiled (M > 64, prompts): 32x32x16 MFMA; tiles of 256 x 256, 256 x 128 or 128 x 128 loaded
+//     from global memory straight into rings of LDS stages, a step of 64 k ahead of the MFMAs
+//     that consume them; with few tiles K is cut into slices over further workgroups.
+// In both the weight rows are the MFMA's first operand, so a lane ends up with runs of four
 // consecutive n of one m: row-major stores of C are vector stores.
 // Epilogues: 0 store float32, 1 add to float32 (the residual stream), 2 SwiGLU to bfloat16
-// (weight rows interleaved in blocks of 16: gate rows, then the up rows of the same outputs).
+// (weight rows interleaved in blocks of 16: gate rows, then the up rows of the same outputs),
+// 3 (tiled, an entry point of its own) the q/k/v projection with per-head norm, rotation and
+// cache write.
 #include "common.h"
 
 HB_MODULE_ERROR_SLOT()
