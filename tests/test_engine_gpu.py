@@ -86,6 +86,39 @@ def test_chunks_of_a_prompt_and_slots_used_again(dtype, model_root):
     engine.cache.check()
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_prompts_with_heads_of_128(dtype, model_root):
+    """Heads of 128 and prompts of more than a thousand tokens: in bfloat16 the q/k/v projection
+    then norms, rotates and writes the cache itself, and decoding does so inside its attention
+    kernel. Whole, in a batch with a short prompt, in pieces, and decoded on: the plain logits."""
+    folder = make_folder(model_root, "D", dtype)
+    vocab = CONFIGS["D"][0]["vocab_size"]
+    a, b = random_tokens(vocab, 1100, 30), random_tokens(vocab, 45, 31)
+    ref_a, ref_b = plain_logits(folder, a), plain_logits(folder, b)
+    at = [0, 1, 63, 64, 500, 1023, 1024, 1087, 1088, 1099]          # rows of the first and of the last tiles
+    engine = hb.load(folder, dtype=dtype, cache_tokens=64 * 40)
+    s = engine.alloc_slot()
+    whole = engine.step([StepEntry(s, a[:1090], at[:-1])]).cpu().numpy()
+    for row, p in enumerate(at[:-1]):
+        assert close(whole[row], ref_a[p], dtype)[0], p
+    for p in range(1090, 1100):                                       # decoded on, one token a step
+        got = engine.step([StepEntry(s, [a[p]], [0])]).cpu().numpy()[0]
+        assert close(got, ref_a[p], dtype)[0], p
+    engine.free_slot(s)
+    s1, s2 = engine.alloc_slot(), engine.alloc_slot()                 # two prompts of unequal length in one step
+    both = engine.step([StepEntry(s1, b, [0, 44]), StepEntry(s2, a, [0, 1099])]).cpu().numpy()
+    for row, (ref, p) in enumerate(((ref_b, 0), (ref_b, 44), (ref_a, 0), (ref_a, 1099))):
+        assert close(both[row], ref[p], dtype)[0], (row, p)
+    engine.free_slot(s1)
+    engine.free_slot(s2)
+    s3 = engine.alloc_slot()                                          # pieces: short ones take the other kernels
+    engine.step([StepEntry(s3, a[:70], [])])
+    piece = engine.step([StepEntry(s3, a[70:], [1099 - 70])]).cpu().numpy()[0]
+    assert close(piece, ref_a[1099], dtype)[0]
+    engine.free_slot(s3)
+    engine.cache.check()
+
+
 def test_window_edge_shows_in_the_logits(model_root):
     """Config C's first layer sees 70 keys. Changing the token just outside every later query's
     window must change nothing there; changing the one just inside must."""
