@@ -1,6 +1,7 @@
 """Each part alone against the plain formulas, models put together from parts in other ways
 (a layer run twice, a layer that reads another's cache, no rotation), and a toy mixer with state
-of its own that is registered here, outside the framework's files."""
+of its own, a toy feed-forward with routing and a toy position encoding that are registered here,
+outside the framework's files."""
 import numpy as np
 import pytest
 import torch
@@ -325,3 +326,96 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped():
         want = pops.linear(pops.rms_norm(x, w["fn"], 1e-6), w["emb"])
         assert torch.allclose(whole[at:at + len(t)], want, atol=1e-4)
         at += len(t)
+
+
+# ---- a toy feed-forward with routing and a toy position encoding, defined here
+@register("feed_forward", "toy_routed")
+class ToyRoutedFeedForward(Part):
+    """Two experts; the router's larger logit (float32) picks one for each token:
+    out = W2[e] relu(W1[e] y). The routing stays inside the part."""
+
+    def __init__(self, hidden_size, intermediate_size, names, shared=None):
+        self.h, self.i, self.names = hidden_size, intermediate_size, dict(names)
+
+    def tensor_needs(self):
+        n = self.names
+        return {n["router"]: TensorNeed((2, self.h)), n["w1"]: TensorNeed((2 * self.i, self.h)),
+                n["w2"]: TensorNeed((2 * self.h, self.i))}
+
+    def load(self, tensors, rt):
+        n = self.names
+        self.router = tensors[n["router"]].to(rt.device).float()
+        self.w1 = tensors[n["w1"]].to(rt.device).float().view(2, self.i, self.h)
+        self.w2 = tensors[n["w2"]].to(rt.device).float().view(2, self.h, self.i)
+
+    def forward(self, ctx, y, x):
+        y = y.float()
+        expert = (y @ self.router.T).argmax(-1)
+        for e in range(2):
+            rows = (expert == e).nonzero().flatten()
+            if len(rows):
+                x[rows] += torch.relu(y[rows] @ self.w1[e].T) @ self.w2[e].T
+
+
+@register("position", "toy_slow_rope")
+class ToySlowRope(Part):
+    """Half-split rotation of the first `rotary_dims` of a head by angles of position / 4: another
+    table behind the hook the attention part asks (`rotation()`)."""
+    graph_safe = True
+
+    def __init__(self, rotary_dims, max_positions):
+        self.rotary_dims, self.max_positions = rotary_dims, max_positions
+
+    def angles(self):
+        inv_freq = 1.0 / (100.0 ** (2.0 * torch.arange(self.rotary_dims // 2, dtype=torch.float32) / self.rotary_dims))
+        return (torch.arange(self.max_positions, dtype=torch.float32) / 4.0)[:, None] * inv_freq[None]
+
+    def load(self, tensors, rt):
+        a = self.angles()
+        self.cos, self.sin = torch.cos(a).contiguous().to(rt.device), torch.sin(a).contiguous().to(rt.device)
+
+    def rotation(self):
+        return self.cos, self.sin, self.rotary_dims
+
+
+def test_toy_routed_feed_forward_and_toy_position_encoding():
+    hidden, inter = 40, 24
+    pos = PartSpec("toy_slow_rope", {"rotary_dims": 8, "max_positions": 256})
+    names = {k: "L." + k for k in ("q", "k", "v", "o", "q_norm", "k_norm")}
+    layer = LayerSpec(PartSpec("prenorm"),
+                      PartSpec("attention", dict(hidden_size=hidden, num_heads=4, num_kv_heads=2, head_dim=16, eps=1e-6,
+                                                 position=pos, names=names)),
+                      PartSpec("toy_routed", {"hidden_size": hidden, "intermediate_size": inter,
+                                              "names": {"router": "L.r", "w1": "L.w1", "w2": "L.w2"}}),
+                      {"input": PartSpec("rmsnorm", {"size": hidden, "eps": 1e-6, "weight": "L.n1"}),
+                       "post_mixer": PartSpec("rmsnorm", {"size": hidden, "eps": 1e-6, "weight": "L.n2"})})
+    base = small_spec(1, [ScheduleEntry(0)])
+    spec = ModelSpec(hidden_size=hidden, vocab_size=60, max_positions=256, embedding=base.embedding, layers=[layer],
+                     schedule=[ScheduleEntry(0), ScheduleEntry(0)], final_norm=base.final_norm, head=base.head)
+    w = weights_for(spec, seed=6)
+    tokens = [5, 9, 33, 2, 41, 17, 8, 11, 3, 50, 27]
+    positions = list(range(len(tokens)))
+    table = ToySlowRope(8, 256).angles()
+
+    def rotate(u):          # [T, heads, 16]: the first 8 of a head, pairs (j, j + 4)
+        c, s = torch.cos(table[positions])[:, None, :], torch.sin(table[positions])[:, None, :]
+        a, b = u[..., :4], u[..., 4:8]
+        return torch.cat([a * c - b * s, a * s + b * c, u[..., 8:]], -1)
+
+    x = pops.embedding(tokens, w["emb"])
+    picked = []
+    for _ in range(2):
+        y = pops.rms_norm(x, w["L.n1"], 1e-6)
+        q = rotate(pops.head_rms_norm(pops.split_heads(pops.linear(y, w["L.q"]), 4, 16), w["L.q_norm"], 1e-6))
+        k = rotate(pops.head_rms_norm(pops.split_heads(pops.linear(y, w["L.k"]), 2, 16), w["L.k_norm"], 1e-6))
+        v = pops.split_heads(pops.linear(y, w["L.v"]), 2, 16)
+        x = x + pops.linear(pops.causal_attention(q, k, v, positions).reshape(len(tokens), 64), w["L.o"])
+        y = pops.rms_norm(x, w["L.n2"], 1e-6)
+        expert = (y @ w["L.r"].T).argmax(-1)
+        picked += expert.tolist()
+        w1, w2 = w["L.w1"].view(2, inter, hidden), w["L.w2"].view(2, hidden, inter)
+        x = x + torch.stack([torch.relu(y[t] @ w1[e].T) @ w2[e].T for t, e in enumerate(expert.tolist())])
+    assert 0 < sum(picked) < len(picked)                    # both experts are in use
+    want = pops.linear(pops.rms_norm(x, w["fn"], 1e-6), w["emb"])
+    assert torch.allclose(run_engine(spec, w, tokens), want, atol=1e-4)
+    assert torch.allclose(run_engine(spec, w, tokens, cut=4), want, atol=1e-4)
