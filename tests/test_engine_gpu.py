@@ -119,6 +119,29 @@ def test_long_prompts_with_heads_of_128(dtype, model_root):
     engine.cache.check()
 
 
+def test_a_batch_of_more_than_64_decodes_like_each_sequence_alone(model_root):
+    """With more than 64 sequences a decode step is no longer a skinny product: the tiled kernels
+    (and, in bfloat16, HIP graphs of them) take over. Every sequence must still get the logits
+    it gets alone."""
+    folder = make_folder(model_root, "D", "bfloat16")
+    vocab = CONFIGS["D"][0]["vocab_size"]
+    B = 80
+    prompts = [random_tokens(vocab, 3 + (7 * i) % 40, 100 + i) for i in range(B)]
+    nexts = [random_tokens(vocab, 4, 500 + i) for i in range(B)]
+    engine = hb.load(folder, dtype="bfloat16", cache_tokens=64 * 2 * B)
+    slots = [engine.alloc_slot() for _ in range(B)]
+    engine.step([StepEntry(s, p, []) for s, p in zip(slots, prompts)])
+    steps = [engine.step([StepEntry(s, [n[j]], [0]) for s, n in zip(slots, nexts)]).cpu().numpy() for j in range(4)]
+    for s in slots:
+        engine.free_slot(s)
+    for i in (0, 1, 17, 40, 63, 64, 79):
+        ref = plain_logits(folder, prompts[i] + nexts[i])
+        for j in range(4):
+            ok, err = close(steps[j][i], ref[len(prompts[i]) + j], "bfloat16")
+            assert ok, (i, j, err)
+    engine.cache.check()
+
+
 def test_window_edge_shows_in_the_logits(model_root):
     """Config C's first layer sees 70 keys. Changing the token just outside every later query's
     window must change nothing there; changing the one just inside must."""
