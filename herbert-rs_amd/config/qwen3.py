@@ -34,9 +34,17 @@ class Qwen3Config:
     rms_norm_eps: float
     tie_word_embeddings: bool
     eos_token_id: int
+    # the fraction of a head that is rotated
+    partial_rotary_factor: float = 1.0
     # one entry per layer: the number of keys a query sees, None = all of them
     layer_windows: Tuple[Optional[int], ...] = field(default=())
     model_type: str = "qwen3"
+
+    @property
+    def rotary_dims(self):
+        """float32(head_dim) * float32(factor), cut to an integer (config.rs:525)."""
+        import numpy as np
+        return int(np.float32(self.head_dim) * np.float32(self.partial_rotary_factor))
 
     # derived sizes (crates/core/src/config.rs:303-319)
     @property
@@ -72,9 +80,12 @@ class Qwen3Config:
                 kind = holder.get("rope_type", holder.get("type", "default"))
                 if kind not in (None, "default"):
                     raise ConfigError(f"config.json: rope scaling of type {kind!r} is not supported")
-        if r.number("partial_rotary_factor", 1.0) != 1.0:
-            raise ConfigError("config.json: partial_rotary_factor other than 1.0 is not supported "
-                              "for this architecture")
+        # crates/core/src/config.rs:516-525: top level first, then rope_parameters; 1.0 if absent
+        partial = r.number("partial_rotary_factor")
+        if partial is None and isinstance(rope_params, dict):
+            partial = Reader(rope_params).number("partial_rotary_factor")
+        if partial is None:
+            partial = 1.0
         hidden = r.integer("hidden_size", required=True)
         heads = r.integer("num_attention_heads", required=True)
         layers = r.integer("num_hidden_layers", required=True)
@@ -101,6 +112,7 @@ class Qwen3Config:
             rms_norm_eps=r.number("rms_norm_eps", 1e-5),
             tie_word_embeddings=r.boolean("tie_word_embeddings", True),
             eos_token_id=eos,
+            partial_rotary_factor=float(partial),
             layer_windows=_layer_windows(r, layers),
             model_type=raw.get("model_type", "qwen3"),
         )
@@ -131,6 +143,9 @@ class Qwen3Config:
             raise ConfigError("rms_norm_eps must be > 0")
         if not self.rope_theta > 0.0:
             raise ConfigError("rope_theta must be > 0")
+        if not 0.0 < self.partial_rotary_factor <= 1.0 or self.rotary_dims < 2 or self.rotary_dims % 2:
+            raise ConfigError(f"partial_rotary_factor ({self.partial_rotary_factor}) must rotate an even number "
+                              f"of at least 2 of the head's {self.head_dim} dimensions")
         if self.max_position_embeddings <= 0:
             raise ConfigError("max_position_embeddings must be > 0")
         if len(self.layer_windows) != self.num_hidden_layers:
@@ -153,6 +168,7 @@ class Qwen3Config:
             "intermediate_size": self.intermediate_size,
             "max_position_embeddings": self.max_position_embeddings,
             "rope_theta": self.rope_theta,
+            "partial_rotary_factor": self.partial_rotary_factor,
             "rms_norm_eps": self.rms_norm_eps,
             "tie_word_embeddings": self.tie_word_embeddings,
             "eos_token_id": self.eos_token_id,

@@ -13,7 +13,7 @@ from ..parts import LayerSpec, ModelSpec, PartSpec, ScheduleEntry
 
 
 def build_spec(cfg):
-    position = PartSpec("rope", {"theta": cfg.rope_theta, "rotary_dims": cfg.head_dim,
+    position = PartSpec("rope", {"theta": cfg.rope_theta, "rotary_dims": cfg.rotary_dims,
                                  "max_positions": cfg.max_position_embeddings})
     layers = []
     for i in range(cfg.num_hidden_layers):

@@ -8,6 +8,7 @@ crates/backends/backend_common/src/.
 import json
 import os
 
+import numpy as np
 import torch
 from safetensors import safe_open
 
@@ -56,6 +57,8 @@ def decoder_layer(x, positions, cfg, w, layer):
     hd = cfg.get("head_dim") or cfg["hidden_size"] // nq
     eps = cfg.get("rms_norm_eps", 1e-5)
     theta = cfg["rope_theta"]
+    # crates/core/src/config.rs:518-525: rotary_ndims = (head_dim as f32 * partial_rotary_factor) as usize
+    rot = int(np.float32(hd) * np.float32(cfg.get("partial_rotary_factor", 1.0)))
 
     y = ops.rms_norm(x, w[p + "input_layernorm.weight"], eps)
     q = ops.split_heads(ops.linear(y, w[p + "self_attn.q_proj.weight"]), nq, hd)
@@ -63,8 +66,8 @@ def decoder_layer(x, positions, cfg, w, layer):
     v = ops.split_heads(ops.linear(y, w[p + "self_attn.v_proj.weight"]), nkv, hd)
     q = ops.head_rms_norm(q, w[p + "self_attn.q_norm.weight"], eps)
     k = ops.head_rms_norm(k, w[p + "self_attn.k_norm.weight"], eps)
-    q = ops.apply_rope(q, positions, theta)
-    k = ops.apply_rope(k, positions, theta)
+    q = ops.apply_rope(q, positions, theta, rot)
+    k = ops.apply_rope(k, positions, theta, rot)
     a = ops.causal_attention(q, k, v, positions, window=layer_window(cfg, layer))
     a = a.reshape(a.shape[0], nq * hd)
     x = x + ops.linear(a, w[p + "self_attn.o_proj.weight"])

@@ -59,10 +59,24 @@ def test_decoupled_head_dim_and_eos_forms():
     (dict(layer_types=["full_attention"]), "layer_types"),
     (dict(layer_types=["sliding_attention", "full_attention"]), "sliding_window"),
     (dict(vocab_size="many"), "integer"),
+    (dict(partial_rotary_factor=1.5), "partial_rotary_factor"),
+    (dict(partial_rotary_factor=0.1), "partial_rotary_factor"),          # 1.6 of 16 dimensions: cut to 1
 ])
 def test_config_errors_name_the_key(over, word):
     with pytest.raises(ConfigError, match=word):
         Qwen3Config.from_dict(minimal(**over))
+
+
+def test_partial_rotation_as_the_reference_derives_it():
+    """crates/core/src/config.rs:516-525: top level, else rope_parameters; float32 product cut to an integer."""
+    assert Qwen3Config.from_dict(TINY_A).rotary_dims == 16
+    assert Qwen3Config.from_dict(dict(TINY_A, partial_rotary_factor=0.5)).rotary_dims == 8
+    nested = dict(TINY_B, rope_parameters={"partial_rotary_factor": 0.25, "rope_theta": 5.0})
+    cfg = Qwen3Config.from_dict(nested)
+    assert cfg.rotary_dims == 8 and cfg.rope_theta == 1000000.0          # the top-level theta wins
+    assert Qwen3Config.from_dict(cfg.to_dict()) == cfg
+    from herbert_rs_amd.models.qwen3 import build_spec
+    assert build_spec(cfg).layers[0].mixer.params["position"].params["rotary_dims"] == 8
 
 
 def test_windows_from_both_forms():

@@ -142,6 +142,25 @@ def test_a_batch_of_more_than_64_decodes_like_each_sequence_alone(model_root):
     engine.cache.check()
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_heads_rotated_in_part(dtype, model_root):
+    """partial_rotary_factor 0.5: the first half of a head is rotated, the rest is left as it is."""
+    folder = make_folder(model_root, "B", dtype, overrides={"partial_rotary_factor": 0.5})
+    vocab = CONFIGS["B"][0]["vocab_size"]
+    tokens = random_tokens(vocab, 90, 44)
+    ref = plain_logits(folder, tokens)
+    full = plain_logits(make_folder(model_root, "B", dtype), tokens)
+    assert float(np.abs(ref - full).max()) > 1e-2                     # the factor does matter
+    engine = hb.load(folder, dtype=dtype, cache_tokens=128)
+    s = engine.alloc_slot()
+    got = engine.step([StepEntry(s, tokens[:70], list(range(70)))]).cpu().numpy()
+    for p in range(70):
+        assert close(got[p], ref[p], dtype)[0], p
+    for p in range(70, 90):
+        assert close(engine.step([StepEntry(s, [tokens[p]], [0])]).cpu().numpy()[0], ref[p], dtype)[0], p
+    engine.free_slot(s)
+
+
 def test_window_edge_shows_in_the_logits(model_root):
     """Config C's first layer sees 70 keys. Changing the token just outside every later query's
     window must change nothing there; changing the one just inside must."""
