@@ -36,6 +36,8 @@ class Qwen3Config:
     eos_token_id: int
     # the fraction of a head that is rotated
     partial_rotary_factor: float = 1.0
+    # (type, factor, original_max_position_embeddings, beta_fast, beta_slow); type default, linear or yarn
+    rope_scaling: Tuple = ("default", 1.0, None, 32.0, 1.0)
     # one entry per layer: the number of keys a query sees, None = all of them
     layer_windows: Tuple[Optional[int], ...] = field(default=())
     model_type: str = "qwen3"
@@ -75,11 +77,23 @@ class Qwen3Config:
             rope_theta = Reader(rope_params).number("rope_theta")
         if rope_theta is None:
             raise ConfigError("config.json: missing rope_theta")
-        for holder in (raw.get("rope_scaling"), rope_params):
-            if isinstance(holder, dict):
-                kind = holder.get("rope_type", holder.get("type", "default"))
-                if kind not in (None, "default"):
-                    raise ConfigError(f"config.json: rope scaling of type {kind!r} is not supported")
+        # crates/core/src/config.rs:547-580: the type from rope_parameters, else rope_scaling
+        holder = rope_params if isinstance(rope_params, dict) else raw.get("rope_scaling")
+        scaling = ("default", 1.0, None, 32.0, 1.0)
+        if isinstance(holder, dict):
+            kind = holder.get("rope_type", holder.get("type"))
+            h = Reader(holder)
+            factor = h.number("factor", 1.0)
+            if kind == "linear":
+                if factor > 1.0:                    # a factor of at most 1 is the plain rotation (:553-560)
+                    scaling = ("linear", float(factor), None, 32.0, 1.0)
+            elif kind == "yarn":
+                scaling = ("yarn", float(factor), h.integer("original_max_position_embeddings"),
+                           float(h.number("beta_fast", 32.0)), float(h.number("beta_slow", 1.0)))
+            elif kind not in (None, "default"):
+                # the reference falls back to the plain rotation here (:580); a model asking for
+                # another scaling would then run with wrong angles, so this is an error instead
+                raise ConfigError(f"config.json: rope scaling of type {kind!r} is not supported")
         # crates/core/src/config.rs:516-525: top level first, then rope_parameters; 1.0 if absent
         partial = r.number("partial_rotary_factor")
         if partial is None and isinstance(rope_params, dict):
@@ -113,6 +127,7 @@ class Qwen3Config:
             tie_word_embeddings=r.boolean("tie_word_embeddings", True),
             eos_token_id=eos,
             partial_rotary_factor=float(partial),
+            rope_scaling=scaling,
             layer_windows=_layer_windows(r, layers),
             model_type=raw.get("model_type", "qwen3"),
         )
@@ -143,6 +158,11 @@ class Qwen3Config:
             raise ConfigError("rms_norm_eps must be > 0")
         if not self.rope_theta > 0.0:
             raise ConfigError("rope_theta must be > 0")
+        kind, factor, original, beta_fast, beta_slow = self.rope_scaling
+        if kind not in ("default", "linear", "yarn") or not factor > 0.0:
+            raise ConfigError(f"rope scaling {self.rope_scaling!r}: unknown type or a factor that is not > 0")
+        if kind == "yarn" and (beta_fast == beta_slow or (original is not None and original <= 0)):
+            raise ConfigError("yarn rope scaling needs beta_fast != beta_slow and original_max_position_embeddings > 0")
         if not 0.0 < self.partial_rotary_factor <= 1.0 or self.rotary_dims < 2 or self.rotary_dims % 2:
             raise ConfigError(f"partial_rotary_factor ({self.partial_rotary_factor}) must rotate an even number "
                               f"of at least 2 of the head's {self.head_dim} dimensions")
@@ -173,6 +193,13 @@ class Qwen3Config:
             "tie_word_embeddings": self.tie_word_embeddings,
             "eos_token_id": self.eos_token_id,
         }
+        kind, factor, original, beta_fast, beta_slow = self.rope_scaling
+        if kind == "linear":
+            d["rope_scaling"] = {"rope_type": "linear", "factor": factor}
+        elif kind == "yarn":
+            d["rope_scaling"] = {"rope_type": "yarn", "factor": factor, "beta_fast": beta_fast, "beta_slow": beta_slow}
+            if original is not None:
+                d["rope_scaling"]["original_max_position_embeddings"] = original
         windows = [w for w in self.layer_windows if w is not None]
         if windows:
             if len(set(windows)) != 1:

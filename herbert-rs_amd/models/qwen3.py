@@ -14,7 +14,7 @@ from ..parts import LayerSpec, ModelSpec, PartSpec, ScheduleEntry
 
 def build_spec(cfg):
     position = PartSpec("rope", {"theta": cfg.rope_theta, "rotary_dims": cfg.rotary_dims,
-                                 "max_positions": cfg.max_position_embeddings})
+                                 "max_positions": cfg.max_position_embeddings, "scaling": cfg.rope_scaling})
     layers = []
     for i in range(cfg.num_hidden_layers):
         p = f"model.layers.{i}."

@@ -43,6 +43,25 @@ def layer_window(cfg, layer):
     return None
 
 
+def rope_scaling(cfg):
+    """crates/core/src/config.rs:547-580: rope_parameters, else rope_scaling; `rope_type`, else `type`;
+    linear only with a factor above 1; yarn's defaults: factor 1, original = max_position_embeddings,
+    beta_fast 32, beta_slow 1; anything else is the plain rotation."""
+    holder = cfg.get("rope_parameters") or cfg.get("rope_scaling")
+    if not isinstance(holder, dict):
+        return None
+    kind = holder.get("rope_type", holder.get("type"))
+    factor = float(holder.get("factor", 1.0))
+    if kind == "linear" and factor > 1.0:
+        return {"type": "linear", "factor": factor}
+    if kind == "yarn":
+        return {"type": "yarn", "factor": factor,
+                "original_max_position_embeddings": holder.get("original_max_position_embeddings",
+                                                               cfg["max_position_embeddings"]),
+                "beta_fast": float(holder.get("beta_fast", 32.0)), "beta_slow": float(holder.get("beta_slow", 1.0))}
+    return None
+
+
 def decoder_layer(x, positions, cfg, w, layer):
     """Pre-norm block: x + attn(norm1(x)), then x + mlp(norm2(x)).
 
@@ -66,8 +85,8 @@ def decoder_layer(x, positions, cfg, w, layer):
     v = ops.split_heads(ops.linear(y, w[p + "self_attn.v_proj.weight"]), nkv, hd)
     q = ops.head_rms_norm(q, w[p + "self_attn.q_norm.weight"], eps)
     k = ops.head_rms_norm(k, w[p + "self_attn.k_norm.weight"], eps)
-    q = ops.apply_rope(q, positions, theta, rot)
-    k = ops.apply_rope(k, positions, theta, rot)
+    q = ops.apply_rope(q, positions, theta, rot, rope_scaling(cfg))
+    k = ops.apply_rope(k, positions, theta, rot, rope_scaling(cfg))
     a = ops.causal_attention(q, k, v, positions, window=layer_window(cfg, layer))
     a = a.reshape(a.shape[0], nq * hd)
     x = x + ops.linear(a, w[p + "self_attn.o_proj.weight"])

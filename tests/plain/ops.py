@@ -7,6 +7,7 @@ CPU in the dtype of its inputs (float32 by default, float64 to judge rounding).
 """
 import math
 
+import numpy as np
 import torch
 
 
@@ -68,28 +69,54 @@ def head_rms_norm(x, weight, eps):
     return out
 
 
-def rope_inv_freq(rotary_ndims, theta):
-    """inv_freq_i = 1 / theta^(2i / R) in float32, i in [0, R/2).
+def rope_inv_freq(rotary_ndims, theta, scaling=None):
+    """inv_freq_i = 1 / theta^(2i / R) in float32, i in [0, R/2), one frequency at a time.
 
-    bc/loader_common.rs:185-188.
+    bc/loader_common.rs:185-188. scaling (a dict as config.json holds it, already reduced to
+    type / factor / original_max_position_embeddings / beta_fast / beta_slow):
+    linear, bc/loader_common.rs:212-215: 1 / (theta^(2i / R) * factor);
+    yarn, bc/loader_common.rs:252-276: wavelen = 2 pi / freq; below original / beta_fast the
+    frequency stays, above original / beta_slow it is divided by the factor, in between
+    smooth = (original / wavelen - beta_slow) / (beta_fast - beta_slow) and
+    (1 - smooth) * freq / factor + smooth * freq. All in float32.
     """
+    f = np.float32
     theta32 = torch.tensor(theta, dtype=torch.float32)
     i2 = torch.arange(0, rotary_ndims // 2, dtype=torch.float32) * 2.0
-    return 1.0 / torch.pow(theta32, i2 / float(rotary_ndims))
+    powers = torch.pow(theta32, i2 / float(rotary_ndims)).numpy()
+    out = []
+    for i in range(rotary_ndims // 2):
+        power = f(powers[i])
+        freq = f(1.0) / power
+        if scaling and scaling["type"] == "linear":
+            freq = f(1.0) / f(power * f(scaling["factor"]))
+        elif scaling and scaling["type"] == "yarn":
+            original = f(scaling["original_max_position_embeddings"])
+            low, high = original / f(scaling["beta_fast"]), original / f(scaling["beta_slow"])
+            wavelen = f(f(2.0) * f(np.pi)) / freq
+            if wavelen < low:
+                pass
+            elif wavelen > high:
+                freq = freq / f(scaling["factor"])
+            else:
+                smooth = f(original / wavelen - f(scaling["beta_slow"])) / f(f(scaling["beta_fast"]) - f(scaling["beta_slow"]))
+                freq = f(f(f(1.0) - smooth) * f(freq / f(scaling["factor"]))) + f(smooth * freq)
+        out.append(freq)
+    return torch.tensor(np.array(out, dtype=np.float32))
 
 
-def rope_tables(positions, rotary_ndims, theta):
+def rope_tables(positions, rotary_ndims, theta, scaling=None):
     """cos/sin of ang = float32(pos) * inv_freq_i, the angle itself in float32.
 
     bc/loader_common.rs:193-199.
     """
-    inv = rope_inv_freq(rotary_ndims, theta)
+    inv = rope_inv_freq(rotary_ndims, theta, scaling)
     pos = torch.as_tensor(positions, dtype=torch.float32)
     ang = pos[:, None] * inv[None, :]
     return torch.cos(ang), torch.sin(ang)
 
 
-def apply_rope(x, positions, theta, rotary_ndims=None):
+def apply_rope(x, positions, theta, rotary_ndims=None, scaling=None):
     """Half-split rotation: pairs (j, j + R/2); dims >= R stay.
 
     bc/kernels.rs:739-759: u_j = x0*c - x1*s ; u_{j+R/2} = x0*s + x1*c.
@@ -98,7 +125,7 @@ def apply_rope(x, positions, theta, rotary_ndims=None):
     hd = x.shape[-1]
     rot = hd if rotary_ndims is None else rotary_ndims
     half = rot // 2
-    cos, sin = rope_tables(positions, rot, theta)
+    cos, sin = rope_tables(positions, rot, theta, scaling)
     cos = cos.to(x.dtype)[:, None, :]
     sin = sin.to(x.dtype)[:, None, :]
     out = x.clone()

@@ -54,7 +54,8 @@ def test_decoupled_head_dim_and_eos_forms():
     (dict(rope_theta=-1.0), "rope_theta"),
     (dict(max_position_embeddings=0), "max_position_embeddings"),
     (dict(num_experts=8), "expert"),
-    (dict(rope_scaling={"type": "yarn", "factor": 4.0}), "yarn"),
+    (dict(rope_scaling={"type": "llama3", "factor": 4.0}), "llama3"),
+    (dict(rope_scaling={"type": "yarn", "factor": 4.0, "beta_fast": 2.0, "beta_slow": 2.0}), "beta_fast"),
     (dict(text_config={}), "text_config"),
     (dict(layer_types=["full_attention"]), "layer_types"),
     (dict(layer_types=["sliding_attention", "full_attention"]), "sliding_window"),
@@ -77,6 +78,23 @@ def test_partial_rotation_as_the_reference_derives_it():
     assert Qwen3Config.from_dict(cfg.to_dict()) == cfg
     from herbert_rs_amd.models.qwen3 import build_spec
     assert build_spec(cfg).layers[0].mixer.params["position"].params["rotary_dims"] == 8
+
+
+def test_rope_scaling_as_the_reference_reads_it():
+    """crates/core/src/config.rs:547-580."""
+    plain = Qwen3Config.from_dict(TINY_A)
+    assert plain.rope_scaling[0] == "default"
+    assert Qwen3Config.from_dict(dict(TINY_A, rope_scaling={"type": "linear", "factor": 1.0})).rope_scaling[0] == "default"
+    lin = Qwen3Config.from_dict(dict(TINY_A, rope_scaling={"type": "linear", "factor": 2.5}))
+    assert lin.rope_scaling[:2] == ("linear", 2.5)
+    yarn = Qwen3Config.from_dict(dict(TINY_A, rope_scaling={"rope_type": "yarn", "factor": 4.0,
+                                                             "original_max_position_embeddings": 32}))
+    assert yarn.rope_scaling == ("yarn", 4.0, 32, 32.0, 1.0)
+    nested = Qwen3Config.from_dict(dict(TINY_A, rope_parameters={"rope_type": "yarn", "factor": 2.0, "beta_slow": 2.0},
+                                        rope_scaling={"type": "linear", "factor": 8.0}))
+    assert nested.rope_scaling == ("yarn", 2.0, None, 32.0, 2.0)          # rope_parameters wins
+    for cfg in (lin, yarn, nested):
+        assert Qwen3Config.from_dict(cfg.to_dict()) == cfg
 
 
 def test_windows_from_both_forms():

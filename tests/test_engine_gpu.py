@@ -161,6 +161,26 @@ def test_heads_rotated_in_part(dtype, model_root):
     engine.free_slot(s)
 
 
+def test_yarn_scaled_rotation_through_the_engine(model_root):
+    over = {"rope_scaling": {"rope_type": "yarn", "factor": 4.0, "original_max_position_embeddings": 64}}
+    raw, seed, std = CONFIGS["B"]
+    folder = os.path.join(str(model_root), "B_yarn")
+    if not os.path.exists(os.path.join(folder, "model.safetensors")):
+        from herbert_rs_amd.weights import write_model_folder
+        from herbert_rs_amd.engine.model import Model
+        from .tiny import spec_of
+        cfg, spec = spec_of(dict(raw, **over))
+        write_model_folder(folder, dict(raw, **over), Model(spec).tensor_needs(), seed, dtype="float32", std=std, norm_std=0.1)
+    tokens = random_tokens(raw["vocab_size"], 120, 45)
+    ref = plain_logits(folder, tokens)
+    assert float(np.abs(ref - plain_logits(make_folder(model_root, "B", "float32"), tokens)).max()) > 1e-2
+    engine = hb.load(folder, dtype="float32", cache_tokens=128)
+    s = engine.alloc_slot()
+    got = engine.step([StepEntry(s, tokens, list(range(120)))]).cpu().numpy()
+    assert float(np.abs(got - ref).max()) <= 1e-4
+    engine.free_slot(s)
+
+
 def test_window_edge_shows_in_the_logits(model_root):
     """Config C's first layer sees 70 keys. Changing the token just outside every later query's
     window must change nothing there; changing the one just inside must."""

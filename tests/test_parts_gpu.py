@@ -58,6 +58,16 @@ def test_position_part_tables():
     pc, ps = pops.rope_tables(list(range(100)), 32, 1e6)
     assert rot == 32 and torch.equal(cos.cpu(), pc) and torch.equal(sin.cpu(), ps)
     assert build("position", PartSpec("none")).rotation() is None
+    for scaling, plain_scaling in ((("linear", 4.0, None, 32.0, 1.0), {"type": "linear", "factor": 4.0}),
+                                   (("yarn", 8.0, 40, 16.0, 2.0), {"type": "yarn", "factor": 8.0, "beta_fast": 16.0,
+                                                                   "original_max_position_embeddings": 40, "beta_slow": 2.0}),
+                                   (("yarn", 2.0, None, 32.0, 1.0), {"type": "yarn", "factor": 2.0, "beta_fast": 32.0,
+                                                                     "original_max_position_embeddings": 100, "beta_slow": 1.0})):
+        part = build("position", PartSpec("rope", {"theta": 1e4, "rotary_dims": 32, "max_positions": 100, "scaling": scaling}))
+        part.load({}, Runtime(torch.float32, DEV))
+        cos, sin, _ = part.rotation()
+        pc, ps = pops.rope_tables(list(range(100)), 32, 1e4, plain_scaling)
+        assert torch.allclose(cos.cpu(), pc, atol=2e-6) and torch.allclose(sin.cpu(), ps, atol=2e-6), scaling
 
 
 ATT = dict(hidden_size=40, num_heads=6, num_kv_heads=2, head_dim=16, eps=1e-6)

@@ -320,3 +320,29 @@ def test_bf16_vectors_of_the_reference():
     half_up_odd = np.uint32(0x3F818000).view(np.float32)  # between 0x3F81 and 0x3F82
     assert ps.f32_to_bf16_bits(half_up_odd) == 0x3F82
     assert ps.f32_to_bf16_bits(np.uint32(0x3F808001).view(np.float32)) == 0x3F81
+
+
+def test_scaled_rotation_frequencies():
+    """Linear and yarn scaling pinned by what they reduce to: a factor of 1 is the plain rotation;
+    linear scaling by f gives at position f p the angles of the plain rotation at p; yarn keeps the
+    fast frequencies, divides the slow ones by the factor, and lies between in between."""
+    R, theta = 32, 10000.0
+    base = ops.rope_inv_freq(R, theta)
+    assert torch.equal(ops.rope_inv_freq(R, theta, {"type": "linear", "factor": 1.0}), base)
+    lin = ops.rope_inv_freq(R, theta, {"type": "linear", "factor": 4.0})
+    assert torch.allclose(lin * 4.0, base, rtol=1e-6)
+    c1, s1 = ops.rope_tables([12], R, theta, {"type": "linear", "factor": 4.0})
+    c0, s0 = ops.rope_tables([3], R, theta)
+    assert torch.allclose(c1, c0, atol=1e-6) and torch.allclose(s1, s0, atol=1e-6)
+    y = {"type": "yarn", "factor": 1.0, "original_max_position_embeddings": 512, "beta_fast": 32.0, "beta_slow": 1.0}
+    assert torch.allclose(ops.rope_inv_freq(R, theta, y), base, rtol=1e-6)
+    y["factor"] = 8.0
+    got = ops.rope_inv_freq(R, theta, y)
+    wavelen = 2 * math.pi / base.double()
+    fast, slow = wavelen < 512 / 32.0, wavelen > 512 / 1.0
+    assert fast.any() and slow.any() and (~fast & ~slow).any()
+    assert torch.equal(got[fast], base[fast]) and torch.allclose(got[slow] * 8.0, base[slow], rtol=1e-6)
+    mid = ~fast & ~slow
+    assert ((got[mid] < base[mid]) & (got[mid] > base[mid] / 8.0)).all()
+    smooth = (512 / wavelen[mid] - 1.0) / 31.0
+    assert torch.allclose(got[mid].double(), (1 - smooth) * base[mid].double() / 8.0 + smooth * base[mid].double(), rtol=1e-5)
