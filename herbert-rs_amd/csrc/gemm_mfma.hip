@@ -13,6 +13,8 @@
 // 3 (tiled, an entry point of its own) the q/k/v projection with per-head norm, rotation and
 // cache write.
 #include "common.h"
+#include <mutex>
+#include <unordered_set>
 
 HB_MODULE_ERROR_SLOT()
 
@@ -872,21 +874,25 @@ gemm_tile32_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void*
     store_wave_tile<EPI, TN32, TM32>(acc, Cv, M, N, ldc, m0 + wm * TMB * 16, n0 + wn * TNB * 16, c32, g2);
 }
 
+// More than 64 KB of dynamic LDS has to be allowed per kernel, once.
+static int allow_lds(const void* kernel, size_t lds) {
+    static std::mutex lock;
+    static std::unordered_set<const void*> allowed;
+    std::lock_guard<std::mutex> guard(lock);
+    if (allowed.count(kernel)) return 0;
+    hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    HB_REQUIRE(e == hipSuccess, "gemm_mfma: cannot have %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+    allowed.insert(kernel);
+    return 0;
+}
+
 template <class Kernel, class... Extra>
 static int launch_tiles(Kernel kern, size_t lds, int threads, long total, int slices, const bf16* x, const bf16* w,
                         void* C, int M, int N, int K, int ldc, int m_tiles, int n_tiles, hipStream_t stream,
                         Extra... extra) {
     HB_REQUIRE(total < (1l << 30), "gemm_mfma: too many tiles");
     HB_REQUIRE(lds <= 160 * 1024, "gemm_mfma: %zu bytes of LDS asked for", lds);
-    if (lds > 64 * 1024) {
-        // once per kernel (this function is instantiated per kernel type)
-        static bool raised = false;
-        if (!raised) {
-            hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-            HB_REQUIRE(e == hipSuccess, "gemm_mfma: cannot have %zu bytes of LDS: %s", lds, hipGetErrorString(e));
-            raised = true;
-        }
-    }
+    if (lds > 64 * 1024 && allow_lds((const void*)kern, lds) != 0) return 1;
     const dim3 blocks((unsigned)((total + 7) / 8 * 8), slices);
     kern<<<blocks, threads, lds, stream>>>(x, w, C, M, N, K, ldc, m_tiles, n_tiles, extra...);
     HB_CHECK_LAUNCH("gemm_tile");
