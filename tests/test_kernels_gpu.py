@@ -135,7 +135,7 @@ def paged_case(lengths, new_counts, nkv, hd, dtype, seed=0, n_pages=64, shuffle=
     the dense per-sequence tensors [len, nkv, hd]."""
     from herbert_rs_amd.cache.paged import LayerKV
     g = torch.Generator().manual_seed(seed)
-    pages_per_slot = 16
+    pages_per_slot = max(16, (max(lengths) + 63) // 64)
     B = len(lengths)
     table = torch.zeros(B + 2, pages_per_slot, dtype=torch.int32)
     order = torch.randperm(n_pages, generator=g).tolist() if shuffle else list(range(n_pages))
@@ -374,10 +374,10 @@ def test_attention_finds_one_far_key_among_hundreds():
     and split it lies in. Random keys would hide a page or a split that is skipped."""
     from herbert_rs_amd.kernels import mfma, ops
     nq, nkv, hd = 4, 1, 64
-    for n, target in ((900, 3), (900, 64 * 7 + 63), (900, 899), (257, 192)):
+    for n, target in ((900, 3), (900, 64 * 7 + 63), (900, 899), (257, 192), (20000, 11), (20000, 64 * 200 + 5)):
         for mode in ("decode", "prefill"):
             new = 1 if mode == "decode" else 40
-            meta, kv, dense = paged_case([n], [new], nkv, hd, torch.bfloat16, seed=target)
+            meta, kv, dense = paged_case([n], [new], nkv, hd, torch.bfloat16, seed=target, n_pages=max(64, n // 64 + 2))
             K, V = dense[0]
             q = torch.zeros(new, nq * hd)
             q[:, :] = (K[target, 0] * 8).repeat(nq)          # aligned with that key, scaled up
