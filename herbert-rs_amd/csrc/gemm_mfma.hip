@@ -60,11 +60,26 @@ struct SkinnyOperands {
     f32x4 g[2];
 };
 
+// An RMSNorm handed from the product before it to the product after it, for at most 16 rows:
+//   RMSNorm(x; g) W^T = inv * (bf16(x * g) W^T),  inv = 1 / sqrt(sum(x^2) / width + eps) per row.
+// The product that adds to the residual stream x (epilogue 1) also leaves xg = bf16(x * g) and,
+// for every block of 16 columns, the sum of x^2 over the block (emit_*); the product that follows
+// reads xg as its input and scales its sums by inv, which it gets by adding up those partial
+// sums in a fixed order (scale_*). No norm kernel runs in between.
+struct NormHandoff {
+    const float* emit_g;         // weight of the norm that follows, [N]; null: nothing is left behind
+    bf16* emit_xg;               // [M, N]
+    float* emit_partial;         // [ceil(N / 16), MP], MP = M rounded up to a power of two; rows from M on hold zeros
+    const float* scale_partial;  // [scale_parts, MP] of the product before; null: no scaling
+    int scale_parts;
+    float scale_eps;             // the width of the normed rows is this product's K
+};
+
 template <int MB, int NB, int WAVES, int EPI, bool PACKED, bool NORM>
 __global__ void __launch_bounds__(WAVES * 64)
 gemm_skinny_kernel(const void* __restrict__ Xv, const bf16* __restrict__ W, void* __restrict__ Cv, int M,
                    int N, int K, int ldc, const float* __restrict__ norm_w, float eps,
-                   float* __restrict__ partial) {
+                   float* __restrict__ partial, NormHandoff hand) {
     constexpr int U = NORM ? 2 : ((NB + MB <= 4) ? 4 : 2);
     const bf16* X = (const bf16*)Xv;
     const float* XF = (const float*)Xv;
@@ -116,7 +131,6 @@ gemm_skinny_kernel(const void* __restrict__ Xv, const bf16* __restrict__ W, void
     float sumsq[MB];
 #pragma unroll
     for (int b = 0; b < MB; ++b) sumsq[b] = 0.f;
-
     const int mine = wave < nsteps ? (nsteps - wave + WAVES - 1) / WAVES : 0;   // this wave's steps
     const int groups = mine / U;
     SkinnyOperands<MB, NB, NORM> cur[U], nxt[U];
@@ -153,6 +167,21 @@ gemm_skinny_kernel(const void* __restrict__ Xv, const bf16* __restrict__ W, void
         }
 
     if (groups > 0) { SKINNY_LOAD(cur, 0) }
+    // The row's sums of squares from the product before, [parts][MP], MP = the rows rounded up to a
+    // power of two: thread t takes row t % MP of the parts t / MP, t / MP + threads / MP, ...; the
+    // first HP of them are asked for here, behind the first weights, and land while the weights
+    // stream; the sum is formed in the epilogue.
+    constexpr int HP = 8;
+    float hp[HP];
+    const int MP = M <= 1 ? 1 : (M <= 2 ? 2 : (M <= 4 ? 4 : (M <= 8 ? 8 : 16)));
+    const int hp_first = (int)threadIdx.x / MP, hp_step = WAVES * 64 / MP;
+    if (MB == 1 && hand.scale_partial) {
+#pragma unroll
+        for (int j = 0; j < HP; ++j) {
+            const int p = hp_first + j * hp_step;
+            hp[j] = hand.scale_partial[(size_t)(p < hand.scale_parts ? p : hand.scale_parts - 1) * MP + (lane & (MP - 1))];
+        }
+    }
     for (int g = 0; g < groups; g += 2) {
         if (g + 1 < groups) { SKINNY_LOAD(nxt, g + 1) }
         SKINNY_MULTIPLY(cur)
@@ -206,6 +235,17 @@ gemm_skinny_kernel(const void* __restrict__ Xv, const bf16* __restrict__ W, void
         }
         __syncthreads();
     }
+    float* handed_of_wave = red + (size_t)(WAVES / 2) * REGS * 64;   // [WAVES][16], behind the tree's space
+    if (MB == 1 && hand.scale_partial) {
+        float handed = 0.f;
+#pragma unroll
+        for (int j = 0; j < HP; ++j)     // past the end the last part was read once more: left out here
+            handed += hp_first + j * hp_step < hand.scale_parts ? hp[j] : 0.f;
+        for (int p = hp_first + HP * hp_step; p < hand.scale_parts; p += hp_step)
+            handed += hand.scale_partial[(size_t)p * MP + (lane & (MP - 1))];
+        for (int d = 32; d >= MP; d >>= 1) handed += __shfl_xor(handed, d, 64);   // lanes of the same row
+        if (lane < MP) handed_of_wave[wave * 16 + lane] = handed;    // read by wave 0 after the tree's barriers
+    }
 #pragma unroll
     for (int half = WAVES / 2; half >= 1; half >>= 1) {
         if (wave >= half && wave < 2 * half) {
@@ -237,6 +277,15 @@ gemm_skinny_kernel(const void* __restrict__ Xv, const bf16* __restrict__ W, void
             for (int b = 0; b < MB; ++b)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) acc[a][b][i] *= inv_rms[b];
+    }
+    if (MB == 1 && hand.scale_partial) {
+        float handed = 0.f;
+        for (int w = 0; w < WAVES; ++w) handed += handed_of_wave[w * 16 + (r16 & (MP - 1))];
+        const float inv = 1.0f / sqrtf(handed / (float)K + hand.scale_eps);
+#pragma unroll
+        for (int a = 0; a < NB; ++a)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[a][0][i] *= inv;
     }
 
     // lane: m = b * 16 + r16, n = n0 + a * 16 + g4 * 4 + i
@@ -274,8 +323,10 @@ gemm_skinny_kernel(const void* __restrict__ Xv, const bf16* __restrict__ W, void
             }
     } else {
         float* C = (float*)Cv;
+        const bool emit = EPI == EPI_ADD && MB == 1 && hand.emit_g;
 #pragma unroll
-        for (int a = 0; a < NB; ++a)
+        for (int a = 0; a < NB; ++a) {
+            float squares = 0.f;      // of the new x over this lane's 4 of the block's 16 columns
 #pragma unroll
             for (int b = 0; b < MB; ++b) {
                 const int m = b * 16 + r16;
@@ -285,13 +336,23 @@ gemm_skinny_kernel(const void* __restrict__ Xv, const bf16* __restrict__ W, void
                     const int n = n0 + a * 16 + g4 * 4 + i;
                     if (n < N) {
                         const size_t idx = (size_t)m * ldc + n;
-                        if (EPI == EPI_ADD)
-                            C[idx] += acc[a][b][i];
-                        else
-                            C[idx] = acc[a][b][i];
+                        float x = acc[a][b][i];
+                        if (EPI == EPI_ADD) x += C[idx];
+                        C[idx] = x;
+                        if (emit) {
+                            squares = fmaf(x, x, squares);
+                            hand.emit_xg[(size_t)m * N + n] = hb_from_float<bf16>(x * hand.emit_g[n]);
+                        }
                     }
                 }
             }
+            if (emit) {               // the same for the whole wave
+                squares += __shfl_xor(squares, 16, 64);
+                squares += __shfl_xor(squares, 32, 64);
+                const int block = n0 / 16 + a;
+                if (g4 == 0 && r16 < MP && block * 16 < N) hand.emit_partial[(size_t)block * MP + r16] = squares;
+            }
+        }
     }
 }
 
@@ -308,15 +369,16 @@ __global__ void gemm_slices_kernel(const float* __restrict__ partial, float* __r
 
 template <int MB, int NB, int WAVES>
 static void launch_skinny(const void* X, const void* W, void* C, int M, int N, int K, int ldc, int epi,
-                          int packed, const float* norm_w, float eps, hipStream_t stream,
+                          int packed, const float* norm_w, float eps, hipStream_t stream, const NormHandoff& hand,
                           float* partial = nullptr, int slices = 1) {
     const dim3 blocks((N + NB * 16 - 1) / (NB * 16), slices);
     size_t lds = (size_t)(WAVES / 2) * NB * MB * 4 * 64 * sizeof(float);
     if (lds < (size_t)WAVES * MB * 16 * sizeof(float)) lds = (size_t)WAVES * MB * 16 * sizeof(float);
+    lds += (size_t)WAVES * 16 * sizeof(float);      // a handed-on norm's sums, one row of 16 a wave
     const bf16* w = (const bf16*)W;
 #define SKINNY_GO(EPIV, PK, NM)                                                                        \
     gemm_skinny_kernel<MB, NB, WAVES, EPIV, PK, NM><<<blocks, WAVES * 64, lds, stream>>>(X, w, C, M, N, K, \
-                                                                                          ldc, norm_w, eps, partial)
+                                                                                          ldc, norm_w, eps, partial, hand)
     if (norm_w) {       // the normed input never meets the add epilogue; built for one block of rows
         if constexpr (MB == 1 && WAVES == 4) {
             if (packed) {
@@ -347,7 +409,7 @@ static void launch_skinny(const void* X, const void* W, void* C, int M, int N, i
 template <int MB>
 static void pick_skinny(const void* X, const void* W, void* C, int M, int N, int K, int ldc, int epi,
                         int packed, const float* norm_w, float eps, hipStream_t stream, float* workspace,
-                        size_t workspace_floats) {
+                        size_t workspace_floats, const NormHandoff& hand) {
     if (MB >= 2 && !norm_w) {
         // More than 16 rows: every workgroup re-reads its slice of the activations from L2, so a
         // workgroup takes 64 weight rows (the activations are then read as often as the weights),
@@ -364,18 +426,18 @@ static void pick_skinny(const void* X, const void* W, void* C, int M, int N, int
             if ((size_t)slices * M * N > workspace_floats) slices = 1;
         }
         if (slices == 1 && N >= 16384)      // wide enough without slices: four waves a workgroup, more of them a CU
-            launch_skinny<MB, 4, 4>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream);
+            launch_skinny<MB, 4, 4>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream, hand);
         else
-            launch_skinny<MB, 4, 8>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream, workspace, slices);
+            launch_skinny<MB, 4, 8>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream, hand, workspace, slices);
         return;
     }
     // Few weight rows: one block of 16 rows a workgroup and eight waves splitting K, so that the
     // 256 CUs all have work. Many rows: more rows a workgroup, so that the activations are
     // re-read from L2 less often.
     if (epi == EPI_SWIGLU || N >= 16384) {
-        launch_skinny<MB, 4, 4>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream);
+        launch_skinny<MB, 4, 4>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream, hand);
     } else {
-        launch_skinny<MB, 1, 8>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream);
+        launch_skinny<MB, 1, 8>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream, hand);
     }
 }
 
@@ -980,9 +1042,15 @@ extern "C" int hb_gemm_qkv_mfma(const void* X, const void* W, int M, int K, int 
 // workspace: float scratch for K cut into slices (17 to 64 rows); without it K is not cut.
 // norm_w != null: X is the float32 residual stream [M, K] and the product is RMSNorm(X; norm_w, eps) W^T
 // (M <= 64 only, never with the add epilogue).
+// hand_*: see NormHandoff (all null / 0 for a product that neither leaves nor takes a norm).
 extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N, int K, int ldc, int epi,
                             int packed, const float* norm_w, float eps, int tile_hint, float* workspace,
-                            size_t workspace_floats, hipStream_t stream) {
+                            size_t workspace_floats, const float* emit_g, void* emit_xg, float* emit_partial,
+                            const float* scale_partial, int scale_parts, float scale_eps, hipStream_t stream) {
+    const NormHandoff hand = {emit_g, (bf16*)emit_xg, emit_partial, scale_partial, scale_parts, scale_eps};
+    HB_REQUIRE(!(emit_g || scale_partial) || (M <= 16 && !norm_w), "gemm_mfma: a norm is handed on for at most 16 rows");
+    HB_REQUIRE(!emit_g || (epi == EPI_ADD && emit_xg && emit_partial), "gemm_mfma: only the adding product leaves a norm behind");
+    HB_REQUIRE(!scale_partial || (scale_parts > 0 && epi != EPI_ADD), "gemm_mfma: bad partial sums of a handed-on norm");
     HB_REQUIRE(!norm_w || (M <= 16 && epi != EPI_ADD && (epi == EPI_SWIGLU || N >= 16384)),
                "gemm_mfma: the fused norm takes M <= 16, N >= 16384 and no add");
     HB_REQUIRE(!packed || N % 16 == 0, "gemm_mfma: packed weights need N %% 16 == 0");
@@ -992,10 +1060,10 @@ extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N,
     HB_REQUIRE(epi != EPI_SWIGLU || N % 32 == 0, "gemm_mfma: the SwiGLU epilogue needs N %% 32 == 0");
     HB_REQUIRE(ldc >= (epi == EPI_SWIGLU ? N / 2 : N), "gemm_mfma: output row stride %d too small", ldc);
     if (M <= 64) {
-        if (M <= 16) pick_skinny<1>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream, workspace, workspace_floats);
-        else if (M <= 32) pick_skinny<2>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream, workspace, workspace_floats);
-        else if (M <= 48) pick_skinny<3>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream, workspace, workspace_floats);
-        else pick_skinny<4>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream, workspace, workspace_floats);
+        if (M <= 16) pick_skinny<1>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream, workspace, workspace_floats, hand);
+        else if (M <= 32) pick_skinny<2>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream, workspace, workspace_floats, hand);
+        else if (M <= 48) pick_skinny<3>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream, workspace, workspace_floats, hand);
+        else pick_skinny<4>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream, workspace, workspace_floats, hand);
         HB_CHECK_LAUNCH("gemm_skinny");
         return 0;
     }

@@ -102,6 +102,12 @@ class Model:
             ctx.entry = i
             ctx.cache_entry = i if e.cache is None else e.cache
             ctx.owns_cache = e.cache is None
+            # the norm that the residual stream meets after this block, for parts that can prepare it
+            ctx.norm_after_block = None
+            if i + 1 < len(self.schedule):
+                first_norm = getattr(self.blocks[self.schedule[i + 1].layer], "first_norm", None)
+                if first_norm is not None:
+                    ctx.norm_after_block = (first_norm(), i + 1)
             self.blocks[e.layer].forward(ctx, x)
         if meta.want_rows.shape[0] == 0:
             return None

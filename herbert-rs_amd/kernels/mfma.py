@@ -12,7 +12,8 @@ _P = ctypes.c_void_p
 _I = ctypes.c_int
 _F = ctypes.c_float
 lib.register_signatures("gemm_mfma", {
-    "hb_gemm_mfma": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _F, _I, _P, ctypes.c_size_t, _P],
+    "hb_gemm_mfma": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _F, _I, _P, ctypes.c_size_t, _P, _P, _P, _P, _I, _F,
+                     _P],
     "hb_gemm_qkv_mfma": [_P, _P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _F, _I, _I, _I, _P],
 })
 
@@ -95,9 +96,46 @@ def norm_fusable(a, w):
             and a.shape[1] % 32 == 0 and w.shape[0] >= NORM_FUSE_MIN_N)
 
 
-def gemm(a, w, out, accumulate=False, packed=False, norm=None, tile=0):
+NORM_HANDOFF_MAX_M = 16
+
+
+def padded_rows(M):
+    """The rows of a handed-on norm's sums of squares: M rounded up to a power of two."""
+    return 1 << max(0, int(M) - 1).bit_length()
+
+
+def _handoff_args(M, N, K, leave, row_scale, accumulate, norm):
+    """The six arguments of a norm that is handed from one product to the next, after checks.
+    leave = (norm weight f32 [N], xg bf16 [M, N], squares f32 [ceil(N / 16), padded_rows(M)]): the
+    product adds to the residual stream and leaves bf16(x * weight) and the sums of x^2 over blocks
+    of 16 columns. row_scale = (squares f32 [ceil(K / 16), padded_rows(M)], eps): the input is such an xg, and every row of the
+    product is scaled by 1 / sqrt(sum of its squares / K + eps)."""
+    args = [None, None, None, None, 0, 0.0]
+    if leave is None and row_scale is None:
+        return args
+    if M > NORM_HANDOFF_MAX_M or norm is not None:
+        raise BackendError(f"a norm is handed on for at most {NORM_HANDOFF_MAX_M} rows and never beside a fused one")
+    if leave is not None:
+        weight, xg, squares = leave
+        if not accumulate:
+            raise BackendError("only a product that adds to the residual stream leaves a norm behind")
+        _check(weight, "norm weight", torch.float32, (N,))
+        _check(xg, "xg", torch.bfloat16, (M, N))
+        _check(squares, "squares", torch.float32, ((N + 15) // 16, padded_rows(M)))
+        args[:3] = [weight.data_ptr(), xg.data_ptr(), squares.data_ptr()]
+    if row_scale is not None:
+        squares, eps = row_scale
+        if accumulate:
+            raise BackendError("a product that adds takes no handed-on norm")
+        _check(squares, "squares", torch.float32, ((K + 15) // 16, padded_rows(M)))
+        args[3:] = [squares.data_ptr(), squares.shape[0], float(eps)]
+    return args
+
+
+def gemm(a, w, out, accumulate=False, packed=False, norm=None, tile=0, leave=None, row_scale=None):
     """out f32 [M, N] (+)= a bf16 [M, K] @ w bf16 [N, K]^T (w as stored, or as pack_weight gives it).
-    norm = (weight f32 [K], eps): a is the float32 residual stream and is RMS-normed on the way."""
+    norm = (weight f32 [K], eps): a is the float32 residual stream and is RMS-normed on the way.
+    leave, row_scale: see _handoff_args."""
     M, K = a.shape
     norm_ptr, eps = _norm_args(a, norm, K)
     _check(w, "w", torch.bfloat16, (None, K))
@@ -105,10 +143,11 @@ def gemm(a, w, out, accumulate=False, packed=False, norm=None, tile=0):
     _check(out, "out", torch.float32, (M, N))
     if K % 32 or (norm is not None and accumulate):
         raise BackendError(f"gemm_mfma refuses M={M}, N={N}, K={K}")
+    hand = _handoff_args(M, N, K, leave, row_scale, accumulate, norm)
     ws_ptr, ws_floats = _slice_workspace(a.device, M, N, K)
     lib.call("gemm_mfma", "hb_gemm_mfma", a.data_ptr(), w.data_ptr(), out.data_ptr(), M, N, K, N,
              EPI_ADD if accumulate else EPI_STORE, 1 if packed else 0, norm_ptr, eps, int(tile), ws_ptr,
-             ws_floats, _stream())
+             ws_floats, *hand, _stream())
 
 
 QKV_FUSE_MIN_M = 1024      # below that the plain product picks smaller tiles or cuts K, and wins
@@ -165,8 +204,9 @@ def interleave_gate_up(gate, up):
     return torch.stack([gate.view(I // 16, 16, K), up.view(I // 16, 16, K)], 1).reshape(2 * I, K).contiguous()
 
 
-def gemm_swiglu(a, w_interleaved, out, packed=False, norm=None, tile=0):
-    """out bf16 [M, I] = silu(a @ gate^T) * (a @ up^T), the weights interleaved as above."""
+def gemm_swiglu(a, w_interleaved, out, packed=False, norm=None, tile=0, row_scale=None):
+    """out bf16 [M, I] = silu(a @ gate^T) * (a @ up^T), the weights interleaved as above.
+    row_scale: see _handoff_args (gate and up are scaled before the activation)."""
     M, K = a.shape
     norm_ptr, eps = _norm_args(a, norm, K)
     _check(w_interleaved, "w", torch.bfloat16, (None, K))
@@ -174,8 +214,9 @@ def gemm_swiglu(a, w_interleaved, out, packed=False, norm=None, tile=0):
     _check(out, "out", torch.bfloat16, (M, N // 2))
     if K % 32 or N % 32:
         raise BackendError(f"gemm_mfma (SwiGLU) refuses M={M}, N={N}, K={K}")
+    hand = _handoff_args(M, N, K, None, row_scale, False, norm)
     lib.call("gemm_mfma", "hb_gemm_mfma", a.data_ptr(), w_interleaved.data_ptr(), out.data_ptr(), M, N, K,
-             N // 2, EPI_SWIGLU, 1 if packed else 0, norm_ptr, eps, int(tile), None, 0, _stream())
+             N // 2, EPI_SWIGLU, 1 if packed else 0, norm_ptr, eps, int(tile), None, 0, *hand, _stream())
 
 
 lib.register_signatures("attention_mfma", {

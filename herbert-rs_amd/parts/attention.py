@@ -88,13 +88,23 @@ class Attention(Part):
                 self.k_norm_w = rt.weight(tensors[n["k_norm"]], matrix=False)
 
     def forward_from_residual(self, ctx, x, norm):
-        """With few rows and bfloat16 weights the input norm runs inside the projection kernel."""
+        """With few rows and bfloat16 weights no norm kernel runs: the projection takes what the
+        product before left of the norm, or else does the norm itself on the way."""
+        handed = ctx.take_handed(self.qkv, x)
+        if handed is not None:
+            self.forward(ctx, handed.xg, x, row_scale=handed.row_scale())
+            return True
         if not (hasattr(norm, "w") and hasattr(norm, "eps") and self.qkv.fuses_norm(x)):
             return False
         self.forward(ctx, None, x, fused_norm=norm)
         return True
 
-    def forward(self, ctx, y, x, fused_norm=None):
+    def project_out(self, ctx, attn, x):
+        """x += attn @ Wo^T, the part's last product into the residual stream."""
+        left = ctx.leave_norm(self.o, x)
+        self.o.forward(attn, x, accumulate=True, leave=None if left is None else left.leave())
+
+    def forward(self, ctx, y, x, fused_norm=None, row_scale=None):
         rt = ctx.rt
         T = x.shape[0]
         kv = ctx.cache.kv_view(ctx.cache_entry)
@@ -102,7 +112,7 @@ class Attention(Part):
         width = self.q_dim + (2 * self.kv_dim if write_kv else 0)
         rot = self.position.rotation()
         cos, sin, rot_dims = rot if rot is not None else (None, None, 0)
-        if write_kv and fused_norm is None and rt.dtype == torch.bfloat16:
+        if write_kv and fused_norm is None and row_scale is None and rt.dtype == torch.bfloat16:
             from ..kernels import mfma
             if mfma.gemm_qkv_fusable(y, self.qkv.weight, ctx.meta, kv, self.nq, self.nkv, self.hd, rot_dims):
                 # a long prompt: the projection norms, rotates and writes the cache in its epilogue
@@ -111,13 +121,13 @@ class Attention(Part):
                               kv, q, self.nq, self.nkv, self.hd, self.eps)
                 attn = rt.buffer("attn", (T, self.q_dim))
                 self.attend(ctx, q, kv, attn)
-                self.o.forward(attn, x, accumulate=True)
+                self.project_out(ctx, attn, x)
                 return
         qkv = rt.buffer("qkv", (T, width), torch.float32)
         if fused_norm is not None:
             self.qkv.forward_normed(x, fused_norm.w, fused_norm.eps, qkv)
         else:
-            self.qkv.forward(y, qkv)
+            self.qkv.forward(y, qkv, row_scale=row_scale)
         attn = rt.buffer("attn", (T, self.q_dim))
         if write_kv and rt.dtype == torch.bfloat16:
             from ..kernels import mfma
@@ -125,13 +135,13 @@ class Attention(Part):
                 # one token a sequence: norm, rotation, cache write and attention in one kernel
                 mfma.attention_decode_fused(qkv, self.q_norm_w, self.k_norm_w, cos, sin, ctx.meta, kv, attn,
                                             self.nq, self.nkv, self.hd, self.eps, self.scale, self.window)
-                self.o.forward(attn, x, accumulate=True)
+                self.project_out(ctx, attn, x)
                 return
         q = rt.buffer("q", (T, self.q_dim))
         ops.qk_norm_rope_write(qkv, self.q_norm_w, self.k_norm_w, cos, sin, rot_dims, ctx.meta, kv, q,
                                self.nq, self.nkv, self.hd, self.eps, write_kv=write_kv)
         self.attend(ctx, q, kv, attn)
-        self.o.forward(attn, x, accumulate=True)
+        self.project_out(ctx, attn, x)
 
     def attend(self, ctx, q, kv, out):
         if q.dtype == torch.bfloat16:

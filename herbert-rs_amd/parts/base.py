@@ -75,6 +75,25 @@ class Runtime:
 
 
 @dataclass
+class NormedRows:
+    """An RMSNorm of the residual stream x that the product which last added to x has half done:
+    xg = bfloat16(x * norm.w), and squares[b, m] = the sum of x[m]^2 over the b-th block of 16
+    columns (its rows padded to a power of two). A product that reads xg and scales its rows by 1 / sqrt(sum of squares / width + eps)
+    gives what it would give for norm(x); no norm kernel runs."""
+    norm: Any
+    entry: int           # the schedule entry whose part may use it
+    x: Any
+    xg: Any
+    squares: Any
+
+    def row_scale(self):
+        return self.squares, self.norm.eps
+
+    def leave(self):
+        return self.norm.w, self.xg, self.squares
+
+
+@dataclass
 class StepContext:
     """What one step hands down to the parts."""
     rt: Runtime
@@ -83,3 +102,33 @@ class StepContext:
     entry: int = 0       # the schedule entry that is running
     cache_entry: int = 0  # the entry whose cache it uses
     owns_cache: bool = True
+    # A norm handed from part to part (NormedRows). The block sets `handed` to what the part that
+    # runs may use in place of norm(x), and `norm_ahead` to (norm, entry): the norm that x meets
+    # after this part. A part whose last product into x can do so calls leave_norm and passes the
+    # result to that product; parts that know nothing of this are served by the norm's own kernel.
+    handed: Any = None
+    norm_ahead: Any = None
+    left: Any = None
+    norm_after_block: Any = None     # set by the model: (first norm of the next entry's block, entry)
+
+    def leave_norm(self, linear, x):
+        """For a part, just before `linear` adds its last product into x: a NormedRows that product
+        is to fill (Linear.forward(..., leave=rows.leave())), or None."""
+        if self.norm_ahead is None:
+            return None
+        norm, entry = self.norm_ahead
+        if norm is None or not getattr(norm, "hands_on", False) or not linear.hands_norm(x.shape[0]):
+            return None
+        rows, width = x.shape
+        import torch
+        xg = self.rt.buffer("handed_rows", (rows, width), torch.bfloat16)
+        squares = self.rt.buffer("handed_squares", ((width + 15) // 16, linear.handed_rows(rows)), torch.float32)
+        self.left = NormedRows(norm, entry, x, xg, squares)
+        return self.left
+
+    def take_handed(self, linear, x):
+        """For a part that starts with `linear` on norm(x): the NormedRows to use instead, or None."""
+        h = self.handed
+        if h is None or not linear.hands_norm(x.shape[0]):
+            return None
+        return h

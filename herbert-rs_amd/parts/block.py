@@ -26,15 +26,27 @@ class PreNormBlock(Part):
     def parts(self):
         return [self.norms["input"], self.mixer, self.norms["post_mixer"], self.feed_forward]
 
+    def first_norm(self):
+        """The norm that the residual stream meets first in this block."""
+        return self.norms["input"]
+
     def forward(self, ctx, x):
-        self._run(ctx, x, self.norms["input"], self.mixer)
-        self._run(ctx, x, self.norms["post_mixer"], self.feed_forward)
+        after = ctx.norm_after_block
+        self._run(ctx, x, self.norms["input"], self.mixer, (self.norms["post_mixer"], ctx.entry))
+        self._run(ctx, x, self.norms["post_mixer"], self.feed_forward, after)
 
     @staticmethod
-    def _run(ctx, x, norm, part):
+    def _run(ctx, x, norm, part, ahead):
         """part(norm(x)) added to x. A part may offer forward_from_residual(ctx, x, norm), which
-        returns True if it has done the norm itself inside its first kernel."""
+        returns True if it has done the norm itself inside its first kernel, or has used what the
+        part before left of it (ctx.handed). `ahead` is (the norm that x meets next, its entry)."""
+        left, ctx.left = ctx.left, None
+        valid = (left is not None and left.norm is norm and left.entry == ctx.entry
+                 and left.x.data_ptr() == x.data_ptr() and left.x.shape == x.shape)
+        ctx.handed = left if valid else None
+        ctx.norm_ahead = ahead
         fused = getattr(part, "forward_from_residual", None)
         if fused is not None and fused(ctx, x, norm):
             return
+        ctx.handed = None
         part.forward(ctx, norm.forward(ctx, x), x)

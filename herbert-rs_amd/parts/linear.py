@@ -23,19 +23,36 @@ class Linear:
             self.packed = True
         self.weight = weight
 
-    def forward(self, a, out, accumulate=False):
-        """out[M, N] (+)= a[M, K] @ W^T."""
+    def forward(self, a, out, accumulate=False, leave=None, row_scale=None):
+        """out[M, N] (+)= a[M, K] @ W^T. leave and row_scale hand an RMSNorm from one product to the
+        next (see hands_norm); they go to the MFMA kernel as kernels.mfma.gemm describes them."""
         if self.weight.dtype == torch.bfloat16 and a.dtype == torch.bfloat16:
             from ..kernels import mfma
             if self.packed or mfma.gemm_supported(a, self.weight, out):
-                mfma.gemm(a, self.weight, out, accumulate, packed=self.packed)
+                mfma.gemm(a, self.weight, out, accumulate, packed=self.packed, leave=leave, row_scale=row_scale)
                 return
+        if leave is not None or row_scale is not None:
+            raise ValueError("this product cannot hand a norm on (ask hands_norm first)")
         ops.gemm_plain(a, self.weight, out, accumulate)
 
-    def forward_swiglu(self, a, out, norm=None):
+    def hands_norm(self, rows):
+        """True if this product, for that many rows, can leave a half-done RMSNorm of its output behind
+        or take one for its input: the few-row MFMA kernel does both in its epilogue."""
+        if self.weight.dtype != torch.bfloat16 or self.in_features % 32:
+            return False
+        from ..kernels import mfma
+        return rows <= mfma.NORM_HANDOFF_MAX_M
+
+    @staticmethod
+    def handed_rows(rows):
+        """Rows of the sums of squares that go with a handed-on norm of that many rows."""
+        from ..kernels import mfma
+        return mfma.padded_rows(rows)
+
+    def forward_swiglu(self, a, out, norm=None, row_scale=None):
         """out bf16 [M, N / 2] = silu(gate) * up for a weight whose rows are gate/up interleaved."""
         from ..kernels import mfma
-        mfma.gemm_swiglu(a, self.weight, out, packed=self.packed, norm=norm)
+        mfma.gemm_swiglu(a, self.weight, out, packed=self.packed, norm=norm, row_scale=row_scale)
 
     def fuses_norm(self, x):
         """True if RMSNorm(x) @ W^T runs as one kernel for this input (few rows, bfloat16 weights)."""

@@ -47,23 +47,30 @@ class SwiGLU(Part):
         self.down = Linear(rt.weight(tensors[n["down"]]))
 
     def forward_from_residual(self, ctx, x, norm):
-        """With few rows and the fused epilogue the input norm runs inside the gate/up kernel."""
-        if not (self.fused_epilogue and hasattr(norm, "w") and hasattr(norm, "eps")
-                and self.gate_up.fuses_norm(x)):
+        """With few rows and the fused epilogue no norm kernel runs: the gate/up kernel takes what the
+        product before left of the norm, or else does the norm itself on the way."""
+        if not self.fused_epilogue:
+            return False
+        handed = ctx.take_handed(self.gate_up, x)
+        if handed is not None:
+            self.forward(ctx, handed.xg, x, row_scale=handed.row_scale())
+            return True
+        if not (hasattr(norm, "w") and hasattr(norm, "eps") and self.gate_up.fuses_norm(x)):
             return False
         self.forward(ctx, None, x, fused_norm=norm)
         return True
 
-    def forward(self, ctx, y, x, fused_norm=None):
+    def forward(self, ctx, y, x, fused_norm=None, row_scale=None):
         rt = ctx.rt
         T = x.shape[0]
         act = rt.buffer("act", (T, self.intermediate_size))
         if fused_norm is not None:
             self.gate_up.forward_swiglu(x, act, norm=(fused_norm.w, fused_norm.eps))
         elif self.fused_epilogue:
-            self.gate_up.forward_swiglu(y, act)
+            self.gate_up.forward_swiglu(y, act, row_scale=row_scale)
         else:
             gu = rt.buffer("gate_up", (T, 2 * self.intermediate_size), torch.float32)
             self.gate_up.forward(y, gu)
             ops.swiglu(gu, act)
-        self.down.forward(act, x, accumulate=True)
+        left = ctx.leave_norm(self.down, x)
+        self.down.forward(act, x, accumulate=True, leave=None if left is None else left.leave())

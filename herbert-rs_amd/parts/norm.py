@@ -9,6 +9,7 @@ from .registry import register
 @register("norm", "rmsnorm")
 class RMSNorm(Part):
     graph_safe = True
+    hands_on = True      # y = x * w / rms(x): a product may apply the 1 / rms to its sums instead (NormedRows)
 
     def __init__(self, size, eps, weight):
         self.size = int(size)

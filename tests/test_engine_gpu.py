@@ -414,3 +414,40 @@ def test_graph_replays_equal_eager_steps(dtype, model_root):
     ref = plain_logits(folder, seqs[1])
     for i, p in enumerate(range(20, 150)):
         assert close(outs[True][i][1], ref[p], dtype)[0], p
+
+
+@pytest.mark.parametrize("name,batch", [("D", 1), ("D", 5), ("B", 16), ("B", 17)])
+def test_norms_handed_from_product_to_product(name, batch, model_root, monkeypatch):
+    """With at most 16 rows in bfloat16 the product that adds to the residual stream prepares the norm
+    that follows and the next product finishes it: between a step's first norm and its last no
+    norm kernel runs. With 17 rows every norm has its kernel again. Both ways give the plain
+    implementation's logits, and nearly each other's (they differ in the order in which a row's
+    squares are added up)."""
+    from herbert_rs_amd.kernels import ops
+    from herbert_rs_amd.parts.norm import RMSNorm
+    folder = make_folder(model_root, name, "bfloat16")
+    raw = CONFIGS[name][0]
+    layers = raw["num_hidden_layers"]
+    seqs = [random_tokens(raw["vocab_size"], 9 + i % 5, 300 + i) for i in range(batch)]
+    calls = []
+    real = ops.rmsnorm
+    monkeypatch.setattr(ops, "rmsnorm", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
+    got = {}
+    for hands_on in (True, False):
+        monkeypatch.setattr(RMSNorm, "hands_on", hands_on)
+        engine = hb.Engine.from_folder(folder, dtype="bfloat16", max_tokens=64 * batch, use_graphs=False)
+        slots = [engine.alloc_slot() for _ in seqs]
+        engine.step([StepEntry(s, t[:-1], []) for s, t in zip(slots, seqs)])
+        del calls[:]
+        got[hands_on] = engine.step([StepEntry(s, [t[-1]], [0]) for s, t in zip(slots, seqs)]).cpu().numpy()
+        if hands_on and batch <= 16:
+            assert len(calls) == 2, len(calls)              # the first layer's input norm and the final norm
+        else:
+            assert layers + 1 <= len(calls) <= 2 * layers + 1, len(calls)
+    for i, t in enumerate(seqs):
+        ref = plain_logits(folder, t)[-1]
+        for hands_on in (True, False):
+            ok, err = close(got[hands_on][i], ref, "bfloat16")
+            assert ok, (i, hands_on, err)
+    if batch <= 16:
+        assert float(np.abs(got[True] - got[False]).max()) <= 2 ** -7 * float(np.abs(got[False]).max())

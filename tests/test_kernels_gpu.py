@@ -431,6 +431,78 @@ def test_gemm_mfma_with_fused_norm(M, N, K, packed):
         assert float((act.float() - wanted).abs().max()) <= 2 ** -7 * float(wanted.abs().max()) + 1e-5
 
 
+@pytest.mark.parametrize("M,H,K1,N2,packed", [(1, 64, 32, 48, False), (8, 4096, 1024, 6144, True), (16, 1056, 96, 16448, False),
+                                              (5, 2336, 160, 2304, True), (13, 17024, 64, 64, True),
+                                              (7, 1048, 64, 0, False)])
+def test_gemm_mfma_hands_a_norm_to_the_next_product(M, H, K1, N2, packed):
+    """x += a W1^T leaves bf16(x g) and the squares of x by blocks of 16 columns; the next product
+    reads those and scales its rows: together RMSNorm(x) W2^T, with no norm kernel between. The
+    parts are checked one by one, then the whole against the unrounded norm. Widths: no multiple of
+    64 (one and four blocks a workgroup both meet an edge), more parts than a thread keeps in
+    registers (17024 / 16 > 8 * 32), and the SwiGLU epilogue."""
+    from herbert_rs_amd.kernels import mfma
+    a = rand(M, K1, seed=40, dtype=torch.bfloat16)
+    w1 = rand(H, K1, seed=41, dtype=torch.bfloat16, scale=0.2)
+    x0 = rand(M, H, seed=42, scale=2.0)
+    g = 1 + 0.1 * rand(H, seed=43)
+    w2 = rand(max(N2, 16), H, seed=44, dtype=torch.bfloat16, scale=0.1)
+    eps = 1e-5
+    pack = (lambda w: mfma.pack_weight(w)) if packed else (lambda w: w)
+    x = x0.clone()
+    mfma.gemm(a, pack(w1), x, accumulate=True, packed=packed)          # what x becomes without the hand-off
+    got_x = x0.clone()
+    xg = torch.full((M, H), 7.0, dtype=torch.bfloat16, device=dev())
+    blocks = (H + 15) // 16
+    MP = mfma.padded_rows(M)
+    assert MP >= M and MP < 2 * max(M, 1) and MP & (MP - 1) == 0
+    squares = torch.full((blocks, MP), 7.0, device=dev())
+    mfma.gemm(a, pack(w1), got_x, accumulate=True, packed=packed, leave=(g, xg, squares))
+    assert torch.equal(got_x, x)
+    assert torch.equal(xg, (x * g).to(torch.bfloat16))
+    padded = torch.zeros(M, blocks * 16, dtype=torch.float64, device=dev())
+    padded[:, :H] = x.double() ** 2
+    want_squares = padded.view(M, blocks, 16).sum(-1).T
+    assert torch.allclose(squares[:, :M].double(), want_squares, rtol=1e-6, atol=0)
+    assert M == MP or float(squares[:, M:].abs().max()) == 0
+    if H % 32:
+        return          # a width the next product does not take: what was left goes unused
+
+    inv = torch.rsqrt((x.double() ** 2).mean(-1, keepdim=True) + eps)
+    want = ((xg.double() @ w2.double().T) * inv).float()
+    out = torch.empty(M, N2, device=dev())
+    mfma.gemm(xg, pack(w2), out, packed=packed, row_scale=(squares, eps))
+    assert float((out - want).abs().max()) <= 1e-5 * float(want.abs().max()) + 1e-5
+    exact = ((x.double() * inv * g) @ w2.double().T).float()
+    assert float((out - exact).abs().max()) <= 2 ** -7 * float(exact.abs().max())
+    if N2 % 32 == 0:
+        gate, up = w2[:N2 // 2].contiguous(), w2[N2 // 2:].contiguous()
+        wi = mfma.interleave_gate_up(gate, up)
+        act = torch.empty(M, N2 // 2, dtype=torch.bfloat16, device=dev())
+        mfma.gemm_swiglu(xg, pack(wi), act, packed=packed, row_scale=(squares, eps))
+        gg, uu = (xg.double() @ gate.double().T) * inv, (xg.double() @ up.double().T) * inv
+        wanted = (gg / (1 + torch.exp(-gg)) * uu).float()
+        assert float((act.float() - wanted).abs().max()) <= 2 ** -7 * float(wanted.abs().max()) + 1e-5
+
+
+def test_gemm_mfma_refuses_a_handed_norm_it_cannot_do():
+    from herbert_rs_amd.errors import BackendError
+    from herbert_rs_amd.kernels import mfma
+    M, H = 17, 64
+    a = rand(M, 32, seed=1, dtype=torch.bfloat16)
+    w = rand(H, 32, seed=2, dtype=torch.bfloat16)
+    x = torch.zeros(M, H, device=dev())
+    g = torch.ones(H, device=dev())
+    xg = torch.empty(M, H, dtype=torch.bfloat16, device=dev())
+    squares = torch.empty(4, 4, device=dev())
+    with pytest.raises(BackendError):
+        mfma.gemm(a, w, x, accumulate=True, leave=(g, xg, squares))                 # more than 16 rows
+    with pytest.raises(BackendError):
+        mfma.gemm(a[:4], w, x[:4], accumulate=False, leave=(g, xg[:4], squares))    # nothing is added
+    with pytest.raises(BackendError):
+        mfma.gemm(xg[:4], rand(32, H, seed=3, dtype=torch.bfloat16), torch.zeros(4, 32, device=dev()),
+                  accumulate=True, row_scale=(squares, 1e-6))
+
+
 @pytest.mark.parametrize("tile", [0, 188, 142, 122, 123])
 @pytest.mark.parametrize("M,N,K,packed", [(65, 128, 64, True), (200, 336, 192, True), (300, 530, 96, False),
                                           (513, 1040, 256, True), (2300, 528, 128, True)])
