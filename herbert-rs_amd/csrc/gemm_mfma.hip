@@ -78,8 +78,7 @@ struct NormHandoff {
 template <int MB, int NB, int WAVES, int EPI, bool PACKED, bool NORM>
 __global__ void __launch_bounds__(WAVES * 64)
 gemm_skinny_kernel(const void* __restrict__ Xv, const bf16* __restrict__ W, void* __restrict__ Cv, int M,
-                   int N, int K, int ldc, const float* __restrict__ norm_w, float eps,
-                   float* __restrict__ partial, NormHandoff hand) {
+                   int N, int K, int ldc, const float* __restrict__ norm_w, float eps, NormHandoff hand) {
     constexpr int U = NORM ? 2 : ((NB + MB <= 4) ? 4 : 2);
     const bf16* X = (const bf16*)Xv;
     const float* XF = (const float*)Xv;
@@ -89,12 +88,7 @@ gemm_skinny_kernel(const void* __restrict__ Xv, const bf16* __restrict__ W, void
     const int r16 = lane & 15;
     const int g4 = lane >> 4;
     const int n0 = blockIdx.x * (NB * 16);
-    const int k32 = K / 32;                       // k-steps of the whole product
-    // gridDim.y > 1: this workgroup sums one slice of K only and leaves its sums in `partial`
-    // [slice][M][N]; a second kernel adds the slices in order (see gemm_slices_kernel)
-    const int per_slice = (k32 + gridDim.y - 1) / gridDim.y;
-    const int step0 = blockIdx.y * per_slice;
-    const int nsteps = k32 - step0 < per_slice ? (k32 - step0 > 0 ? k32 - step0 : 0) : per_slice;
+    const int nsteps = K / 32;                    // k-steps of the product
 
     f32x4 acc[NB][MB];
 #pragma unroll
@@ -137,7 +131,7 @@ gemm_skinny_kernel(const void* __restrict__ Xv, const bf16* __restrict__ W, void
 
 #define SKINNY_LOAD(dst, group)                                                  \
     _Pragma("unroll") for (int u = 0; u < U; ++u) {                              \
-        const int st = step0 + wave + ((group) * U + u) * WAVES;                 \
+        const int st = wave + ((group) * U + u) * WAVES;                         \
         const int k = st * 32;                                                   \
         _Pragma("unroll") for (int a = 0; a < NB; ++a)                           \
             dst[u].w[a] = *(const bf16x8*)(wrow[a] + (size_t)st * WSTEP);        \
@@ -191,7 +185,7 @@ gemm_skinny_kernel(const void* __restrict__ Xv, const bf16* __restrict__ W, void
         }
     }
     for (int i = groups * U; i < mine; ++i) {       // what is left over of this wave's steps
-        const int st = step0 + wave + i * WAVES;
+        const int st = wave + i * WAVES;
         const int k = st * 32;
         bf16x8 wv[NB], xv[MB];
 #pragma unroll
@@ -289,22 +283,6 @@ gemm_skinny_kernel(const void* __restrict__ Xv, const bf16* __restrict__ W, void
     }
 
     // lane: m = b * 16 + r16, n = n0 + a * 16 + g4 * 4 + i
-    if (gridDim.y > 1) {
-        float* P = partial + (size_t)blockIdx.y * M * N;
-#pragma unroll
-        for (int a = 0; a < NB; ++a)
-#pragma unroll
-            for (int b = 0; b < MB; ++b) {
-                const int m = b * 16 + r16;
-                if (m >= M) continue;
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int n = n0 + a * 16 + g4 * 4 + i;
-                    if (n < N) P[(size_t)m * N + n] = acc[a][b][i];
-                }
-            }
-        return;
-    }
     if (EPI == EPI_SWIGLU) {
         bf16* C = (bf16*)Cv;
         const int out_n0 = n0 / 2;
@@ -367,18 +345,34 @@ __global__ void gemm_slices_kernel(const float* __restrict__ partial, float* __r
     C[(size_t)m * ldc + n] = sum;
 }
 
+// The same for the SwiGLU epilogue: column j of the output pairs the sums of the gate row
+// 32 (j / 16) + j % 16 and of the up row 16 further on; C bf16 [M, N / 2].
+__global__ void gemm_slices_swiglu_kernel(const float* __restrict__ partial, bf16* __restrict__ C, int M, int N,
+                                          int ldc, int slices) {
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int half = N / 2;
+    if (idx >= (size_t)M * half) return;
+    const int m = (int)(idx / half), j = (int)(idx % half);
+    const size_t at = (size_t)m * N + 32 * (j / 16) + j % 16;
+    float gate = 0.f, up = 0.f;
+    for (int s = 0; s < slices; ++s) {
+        gate += partial[(size_t)s * M * N + at];
+        up += partial[(size_t)s * M * N + at + 16];
+    }
+    C[(size_t)m * ldc + j] = hb_from_float<bf16>(silu_mul(gate, up));
+}
+
 template <int MB, int NB, int WAVES>
 static void launch_skinny(const void* X, const void* W, void* C, int M, int N, int K, int ldc, int epi,
-                          int packed, const float* norm_w, float eps, hipStream_t stream, const NormHandoff& hand,
-                          float* partial = nullptr, int slices = 1) {
-    const dim3 blocks((N + NB * 16 - 1) / (NB * 16), slices);
+                          int packed, const float* norm_w, float eps, hipStream_t stream, const NormHandoff& hand) {
+    const dim3 blocks((N + NB * 16 - 1) / (NB * 16));
     size_t lds = (size_t)(WAVES / 2) * NB * MB * 4 * 64 * sizeof(float);
     if (lds < (size_t)WAVES * MB * 16 * sizeof(float)) lds = (size_t)WAVES * MB * 16 * sizeof(float);
     lds += (size_t)WAVES * 16 * sizeof(float);      // a handed-on norm's sums, one row of 16 a wave
     const bf16* w = (const bf16*)W;
 #define SKINNY_GO(EPIV, PK, NM)                                                                        \
     gemm_skinny_kernel<MB, NB, WAVES, EPIV, PK, NM><<<blocks, WAVES * 64, lds, stream>>>(X, w, C, M, N, K, \
-                                                                                          ldc, norm_w, eps, partial, hand)
+                                                                                          ldc, norm_w, eps, hand)
     if (norm_w) {       // the normed input never meets the add epilogue; built for one block of rows
         if constexpr (MB == 1 && WAVES == 4) {
             if (packed) {
@@ -399,45 +393,16 @@ static void launch_skinny(const void* X, const void* W, void* C, int M, int N, i
         else SKINNY_GO(EPI_SWIGLU, false, false);
     }
 #undef SKINNY_GO
-    if (slices > 1) {
-        const size_t total = (size_t)M * N;
-        gemm_slices_kernel<<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(partial, (float*)C, M, N, ldc, slices,
-                                                                              epi == EPI_ADD);
-    }
 }
 
-template <int MB>
+// At most 16 rows. Few weight rows: one block of 16 rows a workgroup and eight waves splitting K,
+// so that the 256 CUs all have work. Many rows: four blocks a workgroup.
 static void pick_skinny(const void* X, const void* W, void* C, int M, int N, int K, int ldc, int epi,
-                        int packed, const float* norm_w, float eps, hipStream_t stream, float* workspace,
-                        size_t workspace_floats, const NormHandoff& hand) {
-    if (MB >= 2 && !norm_w) {
-        // More than 16 rows: every workgroup re-reads its slice of the activations from L2, so a
-        // workgroup takes 64 weight rows (the activations are then read as often as the weights),
-        // and K is cut into slices over further workgroups until the 256 CUs have work; the slices'
-        // sums are added in order by a second kernel, so the result does not depend on timing.
-        const int groups = (N + 63) / 64;
-        int slices = 1;
-        if (epi != EPI_SWIGLU) {
-            slices = 256 / groups;
-            const int most = K / 32 / 8;                 // at least one k-step a wave
-            if (slices > most) slices = most;
-            if (slices > 8) slices = 8;
-            if (slices < 1) slices = 1;
-            if ((size_t)slices * M * N > workspace_floats) slices = 1;
-        }
-        if (slices == 1 && N >= 16384)      // wide enough without slices: four waves a workgroup, more of them a CU
-            launch_skinny<MB, 4, 4>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream, hand);
-        else
-            launch_skinny<MB, 4, 8>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream, hand, workspace, slices);
-        return;
-    }
-    // Few weight rows: one block of 16 rows a workgroup and eight waves splitting K, so that the
-    // 256 CUs all have work. Many rows: more rows a workgroup, so that the activations are
-    // re-read from L2 less often.
+                        int packed, const float* norm_w, float eps, hipStream_t stream, const NormHandoff& hand) {
     if (epi == EPI_SWIGLU || N >= 16384) {
-        launch_skinny<MB, 4, 4>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream, hand);
+        launch_skinny<1, 4, 4>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream, hand);
     } else {
-        launch_skinny<MB, 1, 8>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream, hand);
+        launch_skinny<1, 1, 8>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream, hand);
     }
 }
 
@@ -636,6 +601,13 @@ __device__ __forceinline__ void store_wave_tile_qkv(f32x16 (&acc)[TN32][TM32], c
     }
 }
 
+// The second half of a handed-on norm (see NormHandoff) for the tiled product: at most 16 rows.
+struct RowScale {
+    const float* partial;        // [parts, MP]; null: no scaling
+    int parts;
+    float eps;
+};
+
 // K in steps of 64. A step's weights are two k-steps of 32 (blocks as above); its activations lie
 // in LDS as rows of 128 bytes, so that a load fetches whole 128-byte lines (8 rows an
 // instruction, 8 lanes a row) and not half lines twice; the 16-byte chunk c of row r sits at
@@ -648,7 +620,8 @@ __device__ __forceinline__ void store_wave_tile_qkv(f32x16 (&acc)[TN32][TM32], c
 template <int EPI, bool PACKED, int TNB, int TMB, int WNW, int WMW, int WST, int XST>
 __global__ void __launch_bounds__(64 * WNW * WMW)
 gemm_tile_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* __restrict__ Cv, int M, int N,
-                 int K, int ldc, int m_tiles, int n_tiles, float* __restrict__ partial, QkvEpilogue qkv) {
+                 int K, int ldc, int m_tiles, int n_tiles, float* __restrict__ partial, QkvEpilogue qkv,
+                 RowScale scale) {
     constexpr int NW = WNW * WMW;
     constexpr int BN = 16 * TNB * WNW, BM = 16 * TMB * WMW;
     constexpr int WBLK = BN / 16;                       // weight blocks of a k-step of 32
@@ -769,8 +742,36 @@ gemm_tile_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* _
 #pragma unroll
     for (int i = 0; i < NLX + NLW; ++i)
         if (load_is_x(i) ? XST == 3 : WST == 3) load_one(clamp(2), 2, clamp(2), 2, i);
+    // A handed-on norm: every row's sum of squares is added up here, behind the first loads, by
+    // all threads (thread t: row t % MP, parts t / MP, t / MP + threads / MP, ...), then over the
+    // lanes of a row and, after the barrier, over the waves in their order.
+    float* const row_sums = (float*)(xlds + XST * X_STAGE);       // [NW][16]
+    const int MP = M <= 1 ? 1 : (M <= 2 ? 2 : (M <= 4 ? 4 : (M <= 8 ? 8 : 16)));
+    if (scale.partial) {
+        constexpr int HP = 8;
+        float hp[HP];
+        const int first = tid / MP, stride = 64 * NW / MP;
+#pragma unroll
+        for (int j = 0; j < HP; ++j) {
+            const int p = first + j * stride;
+            hp[j] = scale.partial[(size_t)(p < scale.parts ? p : scale.parts - 1) * MP + (lane & (MP - 1))];
+        }
+        float sum = 0.f;
+#pragma unroll
+        for (int j = 0; j < HP; ++j) sum += first + j * stride < scale.parts ? hp[j] : 0.f;
+        for (int p = first + HP * stride; p < scale.parts; p += stride)
+            sum += scale.partial[(size_t)p * MP + (lane & (MP - 1))];
+        for (int d = 32; d >= MP; d >>= 1) sum += __shfl_xor(sum, d, 64);
+        if (lane < MP) row_sums[wave * 16 + lane] = sum;
+    }
     hb_wait_vmcnt<NLX + NLW + LATER>();
     hb_workgroup_barrier();
+    float inv_rms = 1.f;          // of row c32 (the scaled product has at most 16 rows, all in the first piece)
+    if (scale.partial) {
+        float sum = 0.f;
+        for (int w = 0; w < NW; ++w) sum += row_sums[w * 16 + (c32 & (MP - 1))];
+        inv_rms = 1.0f / sqrtf(sum / (float)K + scale.eps);
+    }
 #pragma unroll
     for (int i = 0; i < NR; ++i) read_one(0, 0, 0, i);
 
@@ -810,6 +811,12 @@ gemm_tile_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* _
         for (int j = 0; j < NM; ++j) mfma_one(1, j);
     }
     hb_wait_vmcnt<0>();      // the loads past the end (repeats of the last step) have landed too
+    if (scale.partial) {
+#pragma unroll
+        for (int a = 0; a < TN32; ++a)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[a][0][i] *= inv_rms;
+    }
     if constexpr (EPI == EPI_QKV)
         store_wave_tile_qkv<TN32, TM32>(acc, qkv, M, N, m0 + wm * TMB * 16, n0 + wn * TNB * 16, c32, g2);
     else if (gridDim.y > 1)
@@ -976,18 +983,19 @@ static int launch_tiles(Kernel kern, size_t lds, int threads, long total, int sl
 // slices > 1: the sums of the slices go to `partial`; the caller adds them up afterwards
 template <int TNB, int TMB, int WNW, int WMW, int WST, int XST>
 static int launch_tile64(const void* X, const void* W, void* C, int M, int N, int K, int ldc, int epi, int packed,
-                         hipStream_t stream, int slices = 1, float* partial = nullptr) {
+                         hipStream_t stream, int slices = 1, float* partial = nullptr, RowScale scale = RowScale{}) {
     constexpr int BN = 16 * TNB * WNW, BM = 16 * TMB * WMW;
     HB_REQUIRE(K % 64 == 0, "gemm_mfma: K=%d is no multiple of 64", K);
     const int m_tiles = (M + BM - 1) / BM, n_tiles = (N + BN - 1) / BN;
     const long total = (long)m_tiles * n_tiles;
-    const size_t lds = (size_t)(WST * BN + XST * BM) * 64 * sizeof(bf16);
+    const size_t lds = (size_t)(WST * BN + XST * BM) * 64 * sizeof(bf16) + WNW * WMW * 16 * sizeof(float);
     const int threads = 64 * WNW * WMW;
     const bf16* x = (const bf16*)X;
     const bf16* w = (const bf16*)W;
-    HB_REQUIRE(slices >= 1 && (slices == 1 || (partial && epi != EPI_SWIGLU)), "gemm_mfma: bad slices");
+    HB_REQUIRE(slices >= 1 && (slices == 1 || partial), "gemm_mfma: bad slices");
+    HB_REQUIRE(!scale.partial || (M <= 16 && slices == 1 && epi != EPI_ADD), "gemm_mfma: this product takes no handed-on norm");
     HB_REQUIRE((K / 64 + slices - 1) / slices * (slices - 1) < K / 64, "gemm_mfma: a slice of K would be empty");
-#define EXTRA , partial, QkvEpilogue{}
+#define EXTRA , partial, QkvEpilogue{}, scale
     TILE_DISPATCH(gemm_tile_kernel, TNB, TMB, WNW, WMW, WST, XST);
 #undef EXTRA
 }
@@ -1029,9 +1037,9 @@ extern "C" int hb_gemm_qkv_mfma(const void* X, const void* W, int M, int K, int 
     const bf16* w = (const bf16*)W;
     if (packed)
         return launch_tiles(gemm_tile_kernel<EPI_QKV, true, 8, 8, 2, 2, 2, 2>, lds, 256, total, 1, x, w, nullptr, M, N, K,
-                            N, m_tiles, n_tiles, stream, (float*)nullptr, e);
+                            N, m_tiles, n_tiles, stream, (float*)nullptr, e, RowScale{});
     return launch_tiles(gemm_tile_kernel<EPI_QKV, false, 8, 8, 2, 2, 2, 2>, lds, 256, total, 1, x, w, nullptr, M, N, K, N,
-                        m_tiles, n_tiles, stream, (float*)nullptr, e);
+                        m_tiles, n_tiles, stream, (float*)nullptr, e, RowScale{});
 }
 
 // C (+)= X @ W^T. X [M, K] bf16, W [N, K] bf16. epi 0: C f32 [M, N] stored; 1: added to;
@@ -1039,9 +1047,9 @@ extern "C" int hb_gemm_qkv_mfma(const void* X, const void* W, int M, int K, int 
 // packed != 0: W is stored as [K / 32][N / 16][64 lanes][8]: lane = 16 * (k / 8 % 4) + n % 16.
 // All blocks of one k-step lie together: workgroups that advance through K side by side read one
 // contiguous stretch of memory at a time, as a streaming copy would.
-// workspace: float scratch for K cut into slices (17 to 64 rows); without it K is not cut.
+// workspace: float scratch for K cut into slices (more than 16 rows); without it K is not cut.
 // norm_w != null: X is the float32 residual stream [M, K] and the product is RMSNorm(X; norm_w, eps) W^T
-// (M <= 64 only, never with the add epilogue).
+// (M <= 16 only, never with the add epilogue).
 // hand_*: see NormHandoff (all null / 0 for a product that neither leaves nor takes a norm).
 extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N, int K, int ldc, int epi,
                             int packed, const float* norm_w, float eps, int tile_hint, float* workspace,
@@ -1059,13 +1067,35 @@ extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N,
     HB_REQUIRE(K % 32 == 0, "gemm_mfma: K=%d is no multiple of 32", K);
     HB_REQUIRE(epi != EPI_SWIGLU || N % 32 == 0, "gemm_mfma: the SwiGLU epilogue needs N %% 32 == 0");
     HB_REQUIRE(ldc >= (epi == EPI_SWIGLU ? N / 2 : N), "gemm_mfma: output row stride %d too small", ldc);
-    if (M <= 64) {
-        if (M <= 16) pick_skinny<1>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream, workspace, workspace_floats, hand);
-        else if (M <= 32) pick_skinny<2>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream, workspace, workspace_floats, hand);
-        else if (M <= 48) pick_skinny<3>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream, workspace, workspace_floats, hand);
-        else pick_skinny<4>(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream, workspace, workspace_floats, hand);
-        HB_CHECK_LAUNCH("gemm_skinny");
-        return 0;
+    const RowScale row_scale = {scale_partial, scale_parts, scale_eps};
+    int tile = tile_hint % 1000, slices = tile_hint >= 1000 ? tile_hint / 1000 : 1;
+    // no slice of K may be empty, and each has at least four steps to run through its ring
+    auto slices_fit = [&](int steps, int sl) {
+        const int per = (steps + sl - 1) / sl;
+        return steps / sl >= 4 && per * (sl - 1) < steps && (size_t)sl * M * N <= workspace_floats;
+    };
+    if (tile == 0 && M <= 16) {
+        // At most 16 rows. The waves of the few-row kernel take the weights from HBM straight into
+        // their MFMA operands. Wide products that fill the CUs with 128 x 32 tiles (gate/up) are a
+        // sixth faster through the LDS rings of the tiled kernel (36 against 42 us for 24576 x 4096).
+        const long tiles = (N + 127) / 128;
+        if (!norm_w && !emit_g && K % 64 == 0 && N >= 16384 && tiles <= 512) {
+            tile = 112;
+        } else {
+            pick_skinny(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream, hand);
+            HB_CHECK_LAUNCH("gemm_skinny");
+            return 0;
+        }
+    }
+    HB_REQUIRE(!norm_w && !emit_g, "gemm_mfma: the tiled product neither norms its input nor leaves a norm behind");
+    if (tile == 0 && K % 64) tile = 123;
+    if (tile == 0 && M <= 64) {
+        // 17 to 64 rows: the product is bound by the weights it reads. Tiles one block of rows high,
+        // 128 wide (256 for wide products of more than 32 rows: fewer activations are read again), and
+        // K cut until about 192 workgroups stream: measured best for 4096- to 24576-wide products.
+        tile = M <= 32 ? 112 : (N >= 8192 ? 184 : 124);
+        const long tiles = (N + (tile == 184 ? 255 : 127)) / (tile == 184 ? 256 : 128);
+        while (tiles * slices < 192 && slices < 16 && slices_fit(K / 64, 2 * slices)) slices *= 2;
     }
     // tile_hint: 0 = choose (otherwise a variant by number, for measurements and tests; + 1000 x the
     // number of K slices). The bigger the tile, the more arithmetic per byte moved and the higher
@@ -1075,15 +1105,13 @@ extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N,
     // over the CUs x steps x the time of a step as measured, + what the second pass moves.
     struct Variant { int id, bn, bm, per_cu; double step_us; };
     static const Variant variants[] = {{188, 256, 256, 1, 1.69}, {142, 256, 128, 1, 0.98}, {122, 128, 128, 2, 0.55}};
-    int tile = tile_hint % 1000, slices = tile_hint >= 1000 ? tile_hint / 1000 : 1;
-    if (tile == 0 && K % 64) tile = 123;
     if (tile == 0) {
         const int steps = K / 64;
         double best = 0;
         for (const Variant& v : variants) {
             const long tiles = (long)((M + v.bm - 1) / v.bm) * ((N + v.bn - 1) / v.bn);
             for (int sl = 1; sl <= 16; sl *= 2) {
-                if (sl > 1 && (epi == EPI_SWIGLU || steps / sl < 4 || (size_t)sl * M * N > workspace_floats)) break;
+                if (sl > 1 && !slices_fit(steps, sl)) break;
                 const long wgs = tiles * sl;
                 const long rounds = (wgs + 256 * v.per_cu - 1) / (256 * v.per_cu);
                 const int share = wgs > 256 ? v.per_cu : 1;
@@ -1098,6 +1126,7 @@ extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N,
         }
     }
     HB_REQUIRE(slices == 1 || (size_t)slices * M * N <= workspace_floats, "gemm_mfma: no room for %d slices", slices);
+    HB_REQUIRE(!scale_partial || tile == 112, "gemm_mfma: only the few-row kernels take a handed-on norm");
     int rc;
     switch (tile) {
         // (ring depths, measured with weights that come from HBM: a third weight stage gains a
@@ -1105,6 +1134,9 @@ extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N,
         case 188: rc = launch_tile64<8, 8, 2, 2, 2, 2>(X, W, C, M, N, K, ldc, epi, packed, stream, slices, workspace); break;   // 256 x 256
         case 142: rc = launch_tile64<8, 4, 2, 2, 3, 2>(X, W, C, M, N, K, ldc, epi, packed, stream, slices, workspace); break;   // 256 (n) x 128 (m)
         case 122: rc = launch_tile64<4, 4, 2, 2, 2, 2>(X, W, C, M, N, K, ldc, epi, packed, stream, slices, workspace); break;   // 128 x 128, two to a CU
+        case 124: rc = launch_tile64<2, 4, 4, 1, 3, 2>(X, W, C, M, N, K, ldc, epi, packed, stream, slices, workspace); break;   // 128 (n) x 64 (m)
+        case 112: rc = launch_tile64<2, 2, 4, 1, 3, 2>(X, W, C, M, N, K, ldc, epi, packed, stream, slices, workspace, row_scale); break;   // 128 (n) x 32 (m)
+        case 184: rc = launch_tile64<4, 4, 4, 1, 3, 2>(X, W, C, M, N, K, ldc, epi, packed, stream, slices, workspace); break;   // 256 (n) x 64 (m)
         case 123:                                                                                                           // 128 x 128, K in steps of 32
             HB_REQUIRE(slices == 1, "gemm_mfma: this tile does not cut K");
             return launch_tile32<4, 4, 2, 2, 4>(X, W, C, M, N, K, ldc, epi, packed, stream);
@@ -1112,8 +1144,12 @@ extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N,
     }
     if (rc == 0 && slices > 1) {
         const size_t total = (size_t)M * N;
-        gemm_slices_kernel<<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(workspace, (float*)C, M, N, ldc, slices,
-                                                                              epi == EPI_ADD);
+        if (epi == EPI_SWIGLU)
+            gemm_slices_swiglu_kernel<<<(unsigned)((total / 2 + 255) / 256), 256, 0, stream>>>(workspace, (bf16*)C, M, N,
+                                                                                             ldc, slices);
+        else
+            gemm_slices_kernel<<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(workspace, (float*)C, M, N, ldc,
+                                                                                  slices, epi == EPI_ADD);
         HB_CHECK_LAUNCH("gemm_slices");
     }
     return rc;

@@ -18,26 +18,21 @@ lib.register_signatures("gemm_mfma", {
 })
 
 EPI_STORE, EPI_ADD, EPI_SWIGLU = 0, 1, 2
-SKINNY_MAX_M = 64
 _workspaces = {}
 
 
 SLICE_WORKSPACE_FLOATS = 16 << 20     # most that the tiled product may use for its K slices (64 MB)
 
 
-def _slice_workspace(device, M, N, K):
-    """(pointer, floats) of the scratch for products whose K is cut into slices: 17 to 64 rows, and
-    the tiled product when it has few tiles. A buffer that was handed out is kept for good: a
-    captured graph may hold its address."""
-    if M <= 16:
+def _slice_workspace(device, M, N, K, tile=0):
+    """(pointer, floats) of the scratch for products whose K is cut into slices: more than 16 rows
+    and too few tiles of 128 x 128 to give every CU one. The kernel takes as many slices as fit in
+    it. A buffer that was handed out is kept for good: a captured graph may hold its address."""
+    if M <= 16 and not tile:
         return None, 0
-    if M <= SKINNY_MAX_M:
-        slices = min(8, 256 // max(1, (N + 63) // 64), K // 256)
-        need = slices * M * N
-    else:
-        tiles = ((M + 127) // 128) * ((N + 127) // 128)
-        slices = min(16, K // 256) if tiles < 256 else 1
-        need = min(slices * M * N, SLICE_WORKSPACE_FLOATS)
+    tiles = ((M + 127) // 128) * ((N + 127) // 128)
+    slices = min(16, K // 256) if tiles < 256 or tile else 1
+    need = min(slices * M * N, SLICE_WORKSPACE_FLOATS)
     if slices < 2 or need < 2 * M * N:
         return None, 0
     kept = _workspaces.setdefault(str(device), [])
@@ -144,7 +139,7 @@ def gemm(a, w, out, accumulate=False, packed=False, norm=None, tile=0, leave=Non
     if K % 32 or (norm is not None and accumulate):
         raise BackendError(f"gemm_mfma refuses M={M}, N={N}, K={K}")
     hand = _handoff_args(M, N, K, leave, row_scale, accumulate, norm)
-    ws_ptr, ws_floats = _slice_workspace(a.device, M, N, K)
+    ws_ptr, ws_floats = _slice_workspace(a.device, M, N, K, tile)
     lib.call("gemm_mfma", "hb_gemm_mfma", a.data_ptr(), w.data_ptr(), out.data_ptr(), M, N, K, N,
              EPI_ADD if accumulate else EPI_STORE, 1 if packed else 0, norm_ptr, eps, int(tile), ws_ptr,
              ws_floats, *hand, _stream())
@@ -215,8 +210,9 @@ def gemm_swiglu(a, w_interleaved, out, packed=False, norm=None, tile=0, row_scal
     if K % 32 or N % 32:
         raise BackendError(f"gemm_mfma (SwiGLU) refuses M={M}, N={N}, K={K}")
     hand = _handoff_args(M, N, K, None, row_scale, False, norm)
+    ws_ptr, ws_floats = _slice_workspace(a.device, M, N, K, tile)
     lib.call("gemm_mfma", "hb_gemm_mfma", a.data_ptr(), w_interleaved.data_ptr(), out.data_ptr(), M, N, K,
-             N // 2, EPI_SWIGLU, 1 if packed else 0, norm_ptr, eps, int(tile), None, 0, *hand, _stream())
+             N // 2, EPI_SWIGLU, 1 if packed else 0, norm_ptr, eps, int(tile), ws_ptr, ws_floats, *hand, _stream())
 
 
 lib.register_signatures("attention_mfma", {

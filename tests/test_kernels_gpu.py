@@ -433,13 +433,15 @@ def test_gemm_mfma_with_fused_norm(M, N, K, packed):
 
 @pytest.mark.parametrize("M,H,K1,N2,packed", [(1, 64, 32, 48, False), (8, 4096, 1024, 6144, True), (16, 1056, 96, 16448, False),
                                               (5, 2336, 160, 2304, True), (13, 17024, 64, 64, True),
-                                              (7, 1048, 64, 0, False)])
+                                              (7, 1048, 64, 0, False), (8, 4096, 64, 24576, True),
+                                              (11, 1088, 96, 16512, False), (1, 576, 32, 16384, True)])
 def test_gemm_mfma_hands_a_norm_to_the_next_product(M, H, K1, N2, packed):
     """x += a W1^T leaves bf16(x g) and the squares of x by blocks of 16 columns; the next product
     reads those and scales its rows: together RMSNorm(x) W2^T, with no norm kernel between. The
     parts are checked one by one, then the whole against the unrounded norm. Widths: no multiple of
     64 (one and four blocks a workgroup both meet an edge), more parts than a thread keeps in
-    registers (17024 / 16 > 8 * 32), and the SwiGLU epilogue."""
+    registers (17024 / 16 > 8 * 32), and the SwiGLU epilogue. Wide second products with K in steps
+    of 64 go through the tiled kernel, which finishes the norm in the same way."""
     from herbert_rs_amd.kernels import mfma
     a = rand(M, K1, seed=40, dtype=torch.bfloat16)
     w1 = rand(H, K1, seed=41, dtype=torch.bfloat16, scale=0.2)
@@ -448,8 +450,7 @@ def test_gemm_mfma_hands_a_norm_to_the_next_product(M, H, K1, N2, packed):
     w2 = rand(max(N2, 16), H, seed=44, dtype=torch.bfloat16, scale=0.1)
     eps = 1e-5
     pack = (lambda w: mfma.pack_weight(w)) if packed else (lambda w: w)
-    x = x0.clone()
-    mfma.gemm(a, pack(w1), x, accumulate=True, packed=packed)          # what x becomes without the hand-off
+    want_x = (x0.double() + a.double() @ w1.double().T).float()
     got_x = x0.clone()
     xg = torch.full((M, H), 7.0, dtype=torch.bfloat16, device=dev())
     blocks = (H + 15) // 16
@@ -457,7 +458,8 @@ def test_gemm_mfma_hands_a_norm_to_the_next_product(M, H, K1, N2, packed):
     assert MP >= M and MP < 2 * max(M, 1) and MP & (MP - 1) == 0
     squares = torch.full((blocks, MP), 7.0, device=dev())
     mfma.gemm(a, pack(w1), got_x, accumulate=True, packed=packed, leave=(g, xg, squares))
-    assert torch.equal(got_x, x)
+    assert float((got_x - want_x).abs().max()) <= 2e-6 * K1 ** 0.5 * float(want_x.abs().max()) + 1e-4
+    x = got_x                                   # what is left behind is made from the sums as stored
     assert torch.equal(xg, (x * g).to(torch.bfloat16))
     padded = torch.zeros(M, blocks * 16, dtype=torch.float64, device=dev())
     padded[:, :H] = x.double() ** 2
@@ -503,9 +505,10 @@ def test_gemm_mfma_refuses_a_handed_norm_it_cannot_do():
                   accumulate=True, row_scale=(squares, 1e-6))
 
 
-@pytest.mark.parametrize("tile", [0, 188, 142, 122, 123])
+@pytest.mark.parametrize("tile", [0, 188, 142, 122, 123, 112, 124, 184])
 @pytest.mark.parametrize("M,N,K,packed", [(65, 128, 64, True), (200, 336, 192, True), (300, 530, 96, False),
-                                          (513, 1040, 256, True), (2300, 528, 128, True)])
+                                          (513, 1040, 256, True), (2300, 528, 128, True), (17, 272, 64, True),
+                                          (40, 530, 320, False), (64, 1040, 128, True)])
 def test_gemm_mfma_tile_variants(tile, M, N, K, packed):
     from herbert_rs_amd.kernels import mfma
     if K % 64 and tile not in (0, 123):
@@ -532,12 +535,14 @@ def test_gemm_mfma_tile_variants(tile, M, N, K, packed):
         assert float((out.float() - wanted).abs().max()) <= 2 ** -7 * float(wanted.abs().max()) + 1e-4
 
 
-@pytest.mark.parametrize("tile", [0, 2122, 4188, 3142, 8122])
+@pytest.mark.parametrize("tile", [0, 2122, 4188, 3142, 8122, 4112, 16124, 2184])
 @pytest.mark.parametrize("M,N,K,packed", [(200, 336, 512, True), (513, 1040, 768, True), (128, 1024, 4096, True),
-                                          (300, 530, 1024, False)])
+                                          (300, 530, 1024, False), (24, 1056, 2112, True), (64, 8192, 1024, True),
+                                          (33, 336, 4096, False)])
 def test_gemm_mfma_tiled_with_k_slices(tile, M, N, K, packed):
-    """More than 64 rows and few tiles: K is cut into slices over workgroups (thousands of the tile
-    number = slices), the sums added in order by a second kernel; tile 0 chooses by itself."""
+    """Few tiles: K is cut into slices over workgroups (thousands of the tile number = slices), the
+    sums added in order by a second kernel, also under the SwiGLU epilogue; tile 0 chooses by
+    itself (K = 2112 = 33 steps: eight slices of five steps would leave the last one empty)."""
     from herbert_rs_amd.kernels import mfma
     slices, steps = tile // 1000, K // 64
     if slices > 1 and (slices > min(16, K // 256) or -(-steps // slices) * (slices - 1) >= steps):
@@ -557,6 +562,14 @@ def test_gemm_mfma_tiled_with_k_slices(tile, M, N, K, packed):
     c3 = base.clone()
     mfma.gemm(a, wp, c3, accumulate=True, packed=packed, tile=tile)
     assert torch.equal(c2, c3)          # the slices are added in a fixed order
+    if N % 32 == 0:
+        gate, up = w[:N // 2].contiguous(), w[N // 2:].contiguous()
+        wi = mfma.interleave_gate_up(gate, up)
+        out = torch.full((M, N // 2), 7.0, dtype=torch.bfloat16, device=dev())
+        mfma.gemm_swiglu(a, mfma.pack_weight(wi) if packed else wi, out, packed=packed, tile=tile)
+        g, u = a.double() @ gate.double().T, a.double() @ up.double().T
+        wanted = (g / (1 + torch.exp(-g)) * u).float()
+        assert float((out.float() - wanted).abs().max()) <= 2 ** -7 * float(wanted.abs().max()) + 1e-4
 
 
 @pytest.mark.parametrize("M,N,K", [(17, 4096, 4096), (40, 1024, 512), (64, 4096, 12288), (64, 6144, 4096),
