@@ -66,6 +66,8 @@ struct SkinnyOperands {
 // for every block of 16 columns, the sum of x^2 over the block (emit_*); the product that follows
 // reads xg as its input and scales its sums by inv, which it gets by adding up those partial
 // sums in a fixed order (scale_*). No norm kernel runs in between.
+// With 17 to 64 rows K is cut into slices and a second kernel adds them up: it sees whole rows and
+// does the whole norm (emit_partial null, emit_eps its eps; emit_xg is then the normed rows).
 struct NormHandoff {
     const float* emit_g;         // weight of the norm that follows, [N]; null: nothing is left behind
     bf16* emit_xg;               // [M, N]
@@ -73,6 +75,7 @@ struct NormHandoff {
     const float* scale_partial;  // [scale_parts, MP] of the product before; null: no scaling
     int scale_parts;
     float scale_eps;             // the width of the normed rows is this product's K
+    float emit_eps;
 };
 
 template <int MB, int NB, int WAVES, int EPI, bool PACKED, bool NORM>
@@ -343,6 +346,69 @@ __global__ void gemm_slices_kernel(const float* __restrict__ partial, float* __r
     float sum = add ? C[(size_t)m * ldc + n] : 0.f;
     for (int s = 0; s < slices; ++s) sum += partial[(size_t)s * M * N + idx];
     C[(size_t)m * ldc + n] = sum;
+}
+
+// The same for a product that adds to the residual stream and is followed by an RMSNorm: a block a
+// row adds the slices to x, stores x and writes y = bf16(x / rms(x) * g) as well. A thread has at
+// most two chunks of four columns (N in steps of 4, at most 8192, 1024 threads) and asks for its
+// part of up to eight slices at once: with at most 64 rows there are few blocks, and what counts is
+// that each has all its loads in flight together.
+__global__ void __launch_bounds__(1024)
+gemm_slices_norm_kernel(const float* __restrict__ partial, float* __restrict__ C, int M, int N, int ldc, int slices,
+                        const float* __restrict__ g, float eps, bf16* __restrict__ y) {
+    __shared__ float red[16];
+    const int m = blockIdx.x;
+    f32x4* row = (f32x4*)(C + (size_t)m * ldc);
+    const f32x4* g4 = (const f32x4*)g;
+    const int nv = N / 4;
+    f32x4 v[2], gv[2];
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+        const int i = threadIdx.x + 1024 * c;
+        const int at = i < nv ? i : nv - 1;              // past the end: the last chunk again, never stored
+        v[c] = row[at];
+        gv[c] = g4[at];
+    }
+    for (int s0 = 0; s0 < slices; s0 += 8) {
+        f32x4 p[2][8];
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            const int i = threadIdx.x + 1024 * c;
+            const int at = i < nv ? i : nv - 1;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int sl = s0 + j < slices ? s0 + j : slices - 1;
+                p[c][j] = ((const f32x4*)(partial + ((size_t)sl * M + m) * N))[at];
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < 2; ++c)
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                if (s0 + j < slices) v[c] += p[c][j];     // in the order of the slices
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+        const int i = threadIdx.x + 1024 * c;
+        if (i < nv) {
+            row[i] = v[c];
+            ss += v[c][0] * v[c][0] + v[c][1] * v[c][1] + v[c][2] * v[c][2] + v[c][3] * v[c][3];
+        }
+    }
+    ss = hb_block_sum(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)N + eps);
+    bf16* out = y + (size_t)m * N;
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+        const int i = threadIdx.x + 1024 * c;
+        if (i < nv) {
+            bf16x4 o;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[e] = (__bf16)(v[c][e] * inv * gv[c][e]);
+            *(bf16x4*)((__bf16*)out + 4 * i) = o;
+        }
+    }
 }
 
 // The same for the SwiGLU epilogue: column j of the output pairs the sums of the gate row
@@ -1054,10 +1120,15 @@ extern "C" int hb_gemm_qkv_mfma(const void* X, const void* W, int M, int K, int 
 extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N, int K, int ldc, int epi,
                             int packed, const float* norm_w, float eps, int tile_hint, float* workspace,
                             size_t workspace_floats, const float* emit_g, void* emit_xg, float* emit_partial,
-                            const float* scale_partial, int scale_parts, float scale_eps, hipStream_t stream) {
-    const NormHandoff hand = {emit_g, (bf16*)emit_xg, emit_partial, scale_partial, scale_parts, scale_eps};
-    HB_REQUIRE(!(emit_g || scale_partial) || (M <= 16 && !norm_w), "gemm_mfma: a norm is handed on for at most 16 rows");
-    HB_REQUIRE(!emit_g || (epi == EPI_ADD && emit_xg && emit_partial), "gemm_mfma: only the adding product leaves a norm behind");
+                            const float* scale_partial, int scale_parts, float scale_eps, float emit_eps,
+                            hipStream_t stream) {
+    const NormHandoff hand = {emit_g, (bf16*)emit_xg, emit_partial, scale_partial, scale_parts, scale_eps, emit_eps};
+    const bool emit_whole = emit_g && !emit_partial;      // the second kernel of a product cut into slices norms
+    HB_REQUIRE(!scale_partial || (M <= 16 && !norm_w), "gemm_mfma: a norm is handed on for at most 16 rows");
+    HB_REQUIRE(!emit_g || (epi == EPI_ADD && emit_xg && !norm_w), "gemm_mfma: only the adding product leaves a norm behind");
+    HB_REQUIRE(!emit_g || (emit_whole ? M > 16 && M <= 64 && N % 4 == 0 && N <= 8192 && ldc % 4 == 0 && K % 64 == 0 && tile_hint == 0
+                                      : M <= 16),
+               "gemm_mfma: a norm is left half done for at most 16 rows, whole for 17 to 64 rows of at most 8192");
     HB_REQUIRE(!scale_partial || (scale_parts > 0 && epi != EPI_ADD), "gemm_mfma: bad partial sums of a handed-on norm");
     HB_REQUIRE(!norm_w || (M <= 16 && epi != EPI_ADD && (epi == EPI_SWIGLU || N >= 16384)),
                "gemm_mfma: the fused norm takes M <= 16, N >= 16384 and no add");
@@ -1087,7 +1158,7 @@ extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N,
             return 0;
         }
     }
-    HB_REQUIRE(!norm_w && !emit_g, "gemm_mfma: the tiled product neither norms its input nor leaves a norm behind");
+    HB_REQUIRE(!norm_w && (!emit_g || emit_whole), "gemm_mfma: the tiled product neither norms its input nor leaves half a norm");
     if (tile == 0 && K % 64) tile = 123;
     if (tile == 0 && M <= 64) {
         // 17 to 64 rows: the product is bound by the weights it reads. Tiles one block of rows high,
@@ -1096,6 +1167,10 @@ extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N,
         tile = M <= 32 ? 112 : (N >= 8192 ? 184 : 124);
         const long tiles = (N + (tile == 184 ? 255 : 127)) / (tile == 184 ? 256 : 128);
         while (tiles * slices < 192 && slices < 16 && slices_fit(K / 64, 2 * slices)) slices *= 2;
+        if (emit_whole && slices == 1) {
+            HB_REQUIRE(slices_fit(K / 64, 2), "gemm_mfma: K=%d or the workspace is too small to leave a norm behind", K);
+            slices = 2;
+        }
     }
     // tile_hint: 0 = choose (otherwise a variant by number, for measurements and tests; + 1000 x the
     // number of K slices). The bigger the tile, the more arithmetic per byte moved and the higher
@@ -1144,7 +1219,10 @@ extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N,
     }
     if (rc == 0 && slices > 1) {
         const size_t total = (size_t)M * N;
-        if (epi == EPI_SWIGLU)
+        if (emit_whole)
+            gemm_slices_norm_kernel<<<M, 1024, 0, stream>>>(workspace, (float*)C, M, N, ldc, slices, emit_g, emit_eps,
+                                                           (bf16*)emit_xg);
+        else if (epi == EPI_SWIGLU)
             gemm_slices_swiglu_kernel<<<(unsigned)((total / 2 + 255) / 256), 256, 0, stream>>>(workspace, (bf16*)C, M, N,
                                                                                              ldc, slices);
         else

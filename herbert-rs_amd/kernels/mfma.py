@@ -13,7 +13,7 @@ _I = ctypes.c_int
 _F = ctypes.c_float
 lib.register_signatures("gemm_mfma", {
     "hb_gemm_mfma": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _F, _I, _P, ctypes.c_size_t, _P, _P, _P, _P, _I, _F,
-                     _P],
+                     _F, _P],
     "hb_gemm_qkv_mfma": [_P, _P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _F, _I, _I, _I, _P],
 })
 
@@ -99,31 +99,53 @@ def padded_rows(M):
     return 1 << max(0, int(M) - 1).bit_length()
 
 
+NORM_WHOLE_MAX_M = 64         # rows of a product whose second kernel (the sum of its K slices) can norm as well
+NORM_WHOLE_MAX_N = 8192
+
+
+def norm_handoff(M, N, K):
+    """How a product of these sizes that adds to the residual stream can prepare the RMSNorm that
+    follows: "half" (at most 16 rows: bf16(x * g) and sums of squares, finished by the next product),
+    "whole" (17 to 64 rows: the kernel that adds up the K slices norms the rows too) or None."""
+    if K % 32:
+        return None
+    if M <= NORM_HANDOFF_MAX_M:
+        return "half"
+    if M <= NORM_WHOLE_MAX_M and K % 64 == 0 and K >= 512 and N % 4 == 0 and N <= NORM_WHOLE_MAX_N:
+        return "whole"
+    return None
+
+
 def _handoff_args(M, N, K, leave, row_scale, accumulate, norm):
-    """The six arguments of a norm that is handed from one product to the next, after checks.
-    leave = (norm weight f32 [N], xg bf16 [M, N], squares f32 [ceil(N / 16), padded_rows(M)]): the
+    """The seven arguments of a norm that is handed from one product to the next, after checks.
+    leave = (norm weight f32 [N], xg bf16 [M, N], squares f32 [ceil(N / 16), padded_rows(M)], eps): the
     product adds to the residual stream and leaves bf16(x * weight) and the sums of x^2 over blocks
-    of 16 columns. row_scale = (squares f32 [ceil(K / 16), padded_rows(M)], eps): the input is such an xg, and every row of the
-    product is scaled by 1 / sqrt(sum of its squares / K + eps)."""
-    args = [None, None, None, None, 0, 0.0]
+    of 16 columns; with squares = None (17 to 64 rows) it leaves the whole norm in xg.
+    row_scale = (squares f32 [ceil(K / 16), padded_rows(M)], eps): the input is such an xg, and every
+    row of the product is scaled by 1 / sqrt(sum of its squares / K + eps)."""
+    args = [None, None, None, None, 0, 0.0, 0.0]
     if leave is None and row_scale is None:
         return args
-    if M > NORM_HANDOFF_MAX_M or norm is not None:
-        raise BackendError(f"a norm is handed on for at most {NORM_HANDOFF_MAX_M} rows and never beside a fused one")
+    if norm is not None:
+        raise BackendError("a norm is never handed on beside a fused one")
     if leave is not None:
-        weight, xg, squares = leave
-        if not accumulate:
-            raise BackendError("only a product that adds to the residual stream leaves a norm behind")
+        weight, xg, squares, eps = leave
+        how = norm_handoff(M, N, K)
+        if not accumulate or how != ("half" if squares is not None else "whole"):
+            raise BackendError(f"a product of M={M}, N={N}, K={K} cannot leave this norm behind")
         _check(weight, "norm weight", torch.float32, (N,))
         _check(xg, "xg", torch.bfloat16, (M, N))
-        _check(squares, "squares", torch.float32, ((N + 15) // 16, padded_rows(M)))
-        args[:3] = [weight.data_ptr(), xg.data_ptr(), squares.data_ptr()]
+        args[:2] = [weight.data_ptr(), xg.data_ptr()]
+        args[6] = float(eps)
+        if squares is not None:
+            _check(squares, "squares", torch.float32, ((N + 15) // 16, padded_rows(M)))
+            args[2] = squares.data_ptr()
     if row_scale is not None:
         squares, eps = row_scale
-        if accumulate:
-            raise BackendError("a product that adds takes no handed-on norm")
+        if accumulate or M > NORM_HANDOFF_MAX_M:
+            raise BackendError("a handed-on norm is finished by a product of at most 16 rows that does not add")
         _check(squares, "squares", torch.float32, ((K + 15) // 16, padded_rows(M)))
-        args[3:] = [squares.data_ptr(), squares.shape[0], float(eps)]
+        args[3:6] = [squares.data_ptr(), squares.shape[0], float(eps)]
     return args
 
 
@@ -139,6 +161,8 @@ def gemm(a, w, out, accumulate=False, packed=False, norm=None, tile=0, leave=Non
     if K % 32 or (norm is not None and accumulate):
         raise BackendError(f"gemm_mfma refuses M={M}, N={N}, K={K}")
     hand = _handoff_args(M, N, K, leave, row_scale, accumulate, norm)
+    if tile and leave is not None and leave[2] is None:
+        raise BackendError("the whole norm is left behind by the product's own choice of tile")
     ws_ptr, ws_floats = _slice_workspace(a.device, M, N, K, tile)
     lib.call("gemm_mfma", "hb_gemm_mfma", a.data_ptr(), w.data_ptr(), out.data_ptr(), M, N, K, N,
              EPI_ADD if accumulate else EPI_STORE, 1 if packed else 0, norm_ptr, eps, int(tile), ws_ptr,

@@ -76,10 +76,11 @@ class Runtime:
 
 @dataclass
 class NormedRows:
-    """An RMSNorm of the residual stream x that the product which last added to x has half done:
-    xg = bfloat16(x * norm.w), and squares[b, m] = the sum of x[m]^2 over the b-th block of 16
-    columns (its rows padded to a power of two). A product that reads xg and scales its rows by 1 / sqrt(sum of squares / width + eps)
-    gives what it would give for norm(x); no norm kernel runs."""
+    """An RMSNorm of the residual stream x that the product which last added to x has prepared.
+    Half done (squares given): xg = bfloat16(x * norm.w), and squares[b, m] = the sum of x[m]^2 over
+    the b-th block of 16 columns (its rows padded to a power of two); a product that reads xg and
+    scales its rows by 1 / sqrt(sum of squares / width + eps) gives what it would give for norm(x).
+    Whole (squares None): xg is norm(x). No norm kernel runs in either case."""
     norm: Any
     entry: int           # the schedule entry whose part may use it
     x: Any
@@ -90,7 +91,7 @@ class NormedRows:
         return self.squares, self.norm.eps
 
     def leave(self):
-        return self.norm.w, self.xg, self.squares
+        return self.norm.w, self.xg, self.squares, self.norm.eps
 
 
 @dataclass
@@ -117,18 +118,23 @@ class StepContext:
         if self.norm_ahead is None:
             return None
         norm, entry = self.norm_ahead
-        if norm is None or not getattr(norm, "hands_on", False) or not linear.hands_norm(x.shape[0]):
+        if norm is None or not getattr(norm, "hands_on", False):
+            return None
+        how = linear.norm_handoff(x.shape[0])
+        if how is None:
             return None
         rows, width = x.shape
         import torch
+        squares = None
         xg = self.rt.buffer("handed_rows", (rows, width), torch.bfloat16)
-        squares = self.rt.buffer("handed_squares", ((width + 15) // 16, linear.handed_rows(rows)), torch.float32)
+        if how == "half":
+            squares = self.rt.buffer("handed_squares", ((width + 15) // 16, linear.handed_rows(rows)), torch.float32)
         self.left = NormedRows(norm, entry, x, xg, squares)
         return self.left
 
     def take_handed(self, linear, x):
         """For a part that starts with `linear` on norm(x): the NormedRows to use instead, or None."""
         h = self.handed
-        if h is None or not linear.hands_norm(x.shape[0]):
+        if h is None or not linear.finishes_norm(x.shape[0]):
             return None
         return h

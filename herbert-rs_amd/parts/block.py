@@ -43,8 +43,12 @@ class PreNormBlock(Part):
         left, ctx.left = ctx.left, None
         valid = (left is not None and left.norm is norm and left.entry == ctx.entry
                  and left.x.data_ptr() == x.data_ptr() and left.x.shape == x.shape)
-        ctx.handed = left if valid else None
         ctx.norm_ahead = ahead
+        if valid and left.squares is None:          # the product before has normed the rows as well
+            ctx.handed = None
+            part.forward(ctx, left.xg, x)
+            return
+        ctx.handed = left if valid else None
         fused = getattr(part, "forward_from_residual", None)
         if fused is not None and fused(ctx, x, norm):
             return

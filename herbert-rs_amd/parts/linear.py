@@ -25,19 +25,26 @@ class Linear:
 
     def forward(self, a, out, accumulate=False, leave=None, row_scale=None):
         """out[M, N] (+)= a[M, K] @ W^T. leave and row_scale hand an RMSNorm from one product to the
-        next (see hands_norm); they go to the MFMA kernel as kernels.mfma.gemm describes them."""
+        next (see norm_handoff); they go to the MFMA kernel as kernels.mfma.gemm describes them."""
         if self.weight.dtype == torch.bfloat16 and a.dtype == torch.bfloat16:
             from ..kernels import mfma
             if self.packed or mfma.gemm_supported(a, self.weight, out):
                 mfma.gemm(a, self.weight, out, accumulate, packed=self.packed, leave=leave, row_scale=row_scale)
                 return
         if leave is not None or row_scale is not None:
-            raise ValueError("this product cannot hand a norm on (ask hands_norm first)")
+            raise ValueError("this product cannot hand a norm on (ask norm_handoff first)")
         ops.gemm_plain(a, self.weight, out, accumulate)
 
-    def hands_norm(self, rows):
-        """True if this product, for that many rows, can leave a half-done RMSNorm of its output behind
-        or take one for its input: the few-row MFMA kernel does both in its epilogue."""
+    def norm_handoff(self, rows):
+        """How this product, for that many rows, can prepare the RMSNorm of the rows it adds to: "half"
+        (the next product finishes it), "whole" or None; see kernels.mfma.norm_handoff."""
+        if self.weight.dtype != torch.bfloat16:
+            return None
+        from ..kernels import mfma
+        return mfma.norm_handoff(rows, self.out_features, self.in_features)
+
+    def finishes_norm(self, rows):
+        """True if this product can take rows that are half normed (bf16(x * g) and sums of squares)."""
         if self.weight.dtype != torch.bfloat16 or self.in_features % 32:
             return False
         from ..kernels import mfma

@@ -457,7 +457,7 @@ def test_gemm_mfma_hands_a_norm_to_the_next_product(M, H, K1, N2, packed):
     MP = mfma.padded_rows(M)
     assert MP >= M and MP < 2 * max(M, 1) and MP & (MP - 1) == 0
     squares = torch.full((blocks, MP), 7.0, device=dev())
-    mfma.gemm(a, pack(w1), got_x, accumulate=True, packed=packed, leave=(g, xg, squares))
+    mfma.gemm(a, pack(w1), got_x, accumulate=True, packed=packed, leave=(g, xg, squares, eps))
     assert float((got_x - want_x).abs().max()) <= 2e-6 * K1 ** 0.5 * float(want_x.abs().max()) + 1e-4
     x = got_x                                   # what is left behind is made from the sums as stored
     assert torch.equal(xg, (x * g).to(torch.bfloat16))
@@ -486,9 +486,37 @@ def test_gemm_mfma_hands_a_norm_to_the_next_product(M, H, K1, N2, packed):
         assert float((act.float() - wanted).abs().max()) <= 2 ** -7 * float(wanted.abs().max()) + 1e-5
 
 
+@pytest.mark.parametrize("M,H,K,packed", [(17, 64, 512, True), (64, 4096, 4096, True), (40, 1028, 576, False),
+                                          (33, 8192, 1024, True)])
+def test_gemm_mfma_leaves_the_whole_norm_for_17_to_64_rows(M, H, K, packed):
+    """K is cut into slices and the kernel that adds them to x norms the rows too: x as the plain
+    product gives it, and y the bfloat16 nearest to the norm of that x (or its neighbour)."""
+    from herbert_rs_amd.kernels import mfma
+    assert mfma.norm_handoff(M, H, K) == "whole"
+    a = rand(M, K, seed=45, dtype=torch.bfloat16)
+    w = rand(H, K, seed=46, dtype=torch.bfloat16, scale=0.1)
+    x0 = rand(M, H, seed=47, scale=2.0)
+    g = 1 + 0.1 * rand(H, seed=48)
+    eps = 1e-5
+    wp = mfma.pack_weight(w) if packed else w
+    want_x = (x0.double() + a.double() @ w.double().T).float()
+    x = x0.clone()
+    y = torch.full((M, H), 7.0, dtype=torch.bfloat16, device=dev())
+    mfma.gemm(a, wp, x, accumulate=True, packed=packed, leave=(g, y, None, eps))
+    assert float((x - want_x).abs().max()) <= 2e-6 * K ** 0.5 * float(want_x.abs().max()) + 1e-4
+    plain = x0.clone()
+    mfma.gemm(a, wp, plain, accumulate=True, packed=packed)
+    assert torch.equal(x, plain)                     # the same slices, added in the same order
+    exact = (x.double() * torch.rsqrt((x.double() ** 2).mean(-1, keepdim=True) + eps) * g.double()).float()
+    assert float(((y.float() - exact).abs() / exact.abs().clamp_min(1e-3)).max()) <= 2 ** -8 + 1e-4
+
+
 def test_gemm_mfma_refuses_a_handed_norm_it_cannot_do():
     from herbert_rs_amd.errors import BackendError
     from herbert_rs_amd.kernels import mfma
+    assert mfma.norm_handoff(16, 64, 32) == "half" and mfma.norm_handoff(17, 64, 32) is None
+    assert mfma.norm_handoff(64, 8192, 512) == "whole" and mfma.norm_handoff(65, 8192, 512) is None
+    assert mfma.norm_handoff(64, 8196, 512) is None and mfma.norm_handoff(20, 64, 448) is None
     M, H = 17, 64
     a = rand(M, 32, seed=1, dtype=torch.bfloat16)
     w = rand(H, 32, seed=2, dtype=torch.bfloat16)
@@ -496,10 +524,13 @@ def test_gemm_mfma_refuses_a_handed_norm_it_cannot_do():
     g = torch.ones(H, device=dev())
     xg = torch.empty(M, H, dtype=torch.bfloat16, device=dev())
     squares = torch.empty(4, 4, device=dev())
+    eps = 1e-6
     with pytest.raises(BackendError):
-        mfma.gemm(a, w, x, accumulate=True, leave=(g, xg, squares))                 # more than 16 rows
+        mfma.gemm(a, w, x, accumulate=True, leave=(g, xg, squares, eps))            # more than 16 rows
     with pytest.raises(BackendError):
-        mfma.gemm(a[:4], w, x[:4], accumulate=False, leave=(g, xg[:4], squares))    # nothing is added
+        mfma.gemm(a, w, x, accumulate=True, leave=(g, xg, None, eps))               # K too short to cut
+    with pytest.raises(BackendError):
+        mfma.gemm(a[:4], w, x[:4], accumulate=False, leave=(g, xg[:4], squares, eps))    # nothing is added
     with pytest.raises(BackendError):
         mfma.gemm(xg[:4], rand(32, H, seed=3, dtype=torch.bfloat16), torch.zeros(4, 32, device=dev()),
                   accumulate=True, row_scale=(squares, 1e-6))
