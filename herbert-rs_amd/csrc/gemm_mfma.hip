@@ -349,13 +349,14 @@ __global__ void gemm_slices_kernel(const float* __restrict__ partial, float* __r
 }
 
 // The same for a product that adds to the residual stream and is followed by an RMSNorm: a block a
-// row adds the slices to x, stores x and writes y = bf16(x / rms(x) * g) as well. A thread has at
+// row adds the slices to x, stores x and writes y = bf16(x / rms(x) * g) as well (or, for at most 16
+// rows, what NormHandoff describes: the next product expects that). A thread has at
 // most two chunks of four columns (N in steps of 4, at most 8192, 1024 threads) and asks for its
 // part of up to eight slices at once: with at most 64 rows there are few blocks, and what counts is
 // that each has all its loads in flight together.
 __global__ void __launch_bounds__(1024)
 gemm_slices_norm_kernel(const float* __restrict__ partial, float* __restrict__ C, int M, int N, int ldc, int slices,
-                        const float* __restrict__ g, float eps, bf16* __restrict__ y) {
+                        const float* __restrict__ g, float eps, bf16* __restrict__ y, float* __restrict__ squares) {
     __shared__ float red[16];
     const int m = blockIdx.x;
     f32x4* row = (f32x4*)(C + (size_t)m * ldc);
@@ -396,9 +397,32 @@ gemm_slices_norm_kernel(const float* __restrict__ partial, float* __restrict__ C
             ss += v[c][0] * v[c][0] + v[c][1] * v[c][1] + v[c][2] * v[c][2] + v[c][3] * v[c][3];
         }
     }
+    bf16* out = y + (size_t)m * N;
+    if (squares) {
+        // half the norm, as the few-row kernel leaves it (at most 16 rows): y = bf16(x * g) and the
+        // sums of x^2 by blocks of 16 columns, four threads a block
+        const int MP = M <= 1 ? 1 : (M <= 2 ? 2 : (M <= 4 ? 4 : (M <= 8 ? 8 : 16)));
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            const int i = threadIdx.x + 1024 * c;
+            float sq = i < nv ? v[c][0] * v[c][0] + v[c][1] * v[c][1] + v[c][2] * v[c][2] + v[c][3] * v[c][3] : 0.f;
+            sq += __shfl_xor(sq, 1, 64);
+            sq += __shfl_xor(sq, 2, 64);
+            if (i < nv) {
+                if ((i & 3) == 0) squares[(size_t)(i / 4) * MP + m] = sq;
+                bf16x4 o;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[e] = (__bf16)(v[c][e] * gv[c][e]);
+                *(bf16x4*)((__bf16*)out + 4 * i) = o;
+            }
+        }
+        if (m == 0)            // rows from M on hold zeros
+            for (int i = threadIdx.x; i < (N + 15) / 16 * (MP - M); i += 1024)
+                squares[(size_t)(i / (MP - M)) * MP + M + i % (MP - M)] = 0.f;
+        return;
+    }
     ss = hb_block_sum(ss, red);
     const float inv = 1.0f / sqrtf(ss / (float)N + eps);
-    bf16* out = y + (size_t)m * N;
 #pragma unroll
     for (int c = 0; c < 2; ++c) {
         const int i = threadIdx.x + 1024 * c;
@@ -1126,9 +1150,8 @@ extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N,
     const bool emit_whole = emit_g && !emit_partial;      // the second kernel of a product cut into slices norms
     HB_REQUIRE(!scale_partial || (M <= 16 && !norm_w), "gemm_mfma: a norm is handed on for at most 16 rows");
     HB_REQUIRE(!emit_g || (epi == EPI_ADD && emit_xg && !norm_w), "gemm_mfma: only the adding product leaves a norm behind");
-    HB_REQUIRE(!emit_g || (emit_whole ? M > 16 && M <= 64 && N % 4 == 0 && N <= 8192 && ldc % 4 == 0 && K % 64 == 0 && tile_hint == 0
-                                      : M <= 16),
-               "gemm_mfma: a norm is left half done for at most 16 rows, whole for 17 to 64 rows of at most 8192");
+    HB_REQUIRE(!emit_g || (emit_whole ? M > 16 && M <= 64 : M <= 16),
+               "gemm_mfma: a norm is left half done for at most 16 rows, whole for 17 to 64 rows");
     HB_REQUIRE(!scale_partial || (scale_parts > 0 && epi != EPI_ADD), "gemm_mfma: bad partial sums of a handed-on norm");
     HB_REQUIRE(!norm_w || (M <= 16 && epi != EPI_ADD && (epi == EPI_SWIGLU || N >= 16384)),
                "gemm_mfma: the fused norm takes M <= 16, N >= 16384 and no add");
@@ -1145,33 +1168,75 @@ extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N,
         const int per = (steps + sl - 1) / sl;
         return steps / sl >= 4 && per * (sl - 1) < steps && (size_t)sl * M * N <= workspace_floats;
     };
-    if (tile == 0 && M <= 16) {
-        // At most 16 rows. The waves of the few-row kernel take the weights from HBM straight into
-        // their MFMA operands. Wide products that fill the CUs with 128 x 32 tiles (gate/up) are a
-        // sixth faster through the LDS rings of the tiled kernel (36 against 42 us for 24576 x 4096).
-        const long tiles = (N + 127) / 128;
-        if (!norm_w && !emit_g && K % 64 == 0 && N >= 16384 && tiles <= 512) {
-            tile = 112;
-        } else {
+    // What the second kernel of a product cut into slices can leave behind: rows of at most 8192.
+    const bool reducer_norms = N % 4 == 0 && N <= 8192 && ldc % 4 == 0;
+    if (tile == 0 && M <= 64) {
+        // At most 64 rows: the product is bound by the weights it reads, and what counts is how
+        // evenly and how deeply the CUs stream them. Candidates: the few-row kernel (at most 16
+        // rows; its waves take the weights from HBM straight into their MFMA operands) and the tiled
+        // kernel with tiles one block of rows high and K cut into 1 to 16 slices. Taken: the least
+        // estimated time (us). The estimates were fitted to measurements of the four products of a
+        // layer for six model sizes (hidden 1024 to 5120) and 4 to 64 rows; the choice is within 1 %
+        // of the best candidate on average and within 12 % at worst.
+        double best = -1;
+        bool skinny = false;
+        if (M <= 16) {
+            // Workgroups of 16 (or 64) weight rows, each streaming at a rate of its own: about
+            // 24 KB/us alone on a CU (more if some CUs stay empty), 28 KB/us for a CU with several;
+            // more rows cost more reads of the activations. 320 workgroups on 256 CUs take as long as 512.
+            const int nb = (epi == EPI_SWIGLU || N >= 16384) ? 4 : 1;
+            const long wgs = (N + 16 * nb - 1) / (16 * nb);
+            const double rounds = wgs <= 256 ? 1 : (wgs <= 512 ? 2 : wgs / 256.0 + 0.5);
+            double rate = (wgs <= 256 ? 24e3 : 28e3) / (1 + 0.02 * M);
+            if (wgs < 256) rate *= 1 + 0.6 * (256 - wgs) / 256.0;
+            best = 3.0 + rounds * 32.0 * nb * K / rate;
+            skinny = true;
+        }
+        if (!norm_w && K % 64 == 0) {
+            struct Small { int id, bn, bm, per_cu; double step_us; };
+            static const Small small[] = {{112, 128, 32, 2, 0.5}, {124, 128, 64, 2, 0.6}, {184, 256, 64, 1, 0.9}};
+            const int steps = K / 64;
+            for (const Small& v : small) {
+                if (M > v.bm) continue;
+                if (scale_partial && v.id != 112) continue;            // only this one finishes a handed-on norm
+                const long tiles = (N + v.bn - 1) / v.bn;
+                for (int sl = 1; sl <= 16; sl *= 2) {
+                    if (sl > 1 && !slices_fit(steps, sl)) break;
+                    // a norm is left behind by the kernel that adds the slices up; a handed-on one is
+                    // finished in the epilogue of a product that is not cut
+                    if (emit_g && (sl == 1 || !reducer_norms)) continue;
+                    if (scale_partial && sl > 1) break;
+                    const long wgs = tiles * sl, slots = 256 * v.per_cu;
+                    const long rounds = (wgs + slots - 1) / slots;
+                    const long on_a_cu = ((wgs < slots ? wgs : slots) + 255) / 256;
+                    const int per = (steps + sl - 1) / sl;
+                    const double waiting = (double)rounds * per * v.step_us * on_a_cu;       // bound by latency
+                    double streaming = (double)wgs * per * (v.bn * 128 + v.bm * 64) / 6.0e6;   // bound by HBM
+                    if (wgs > slots) streaming *= 1.12;
+                    double cost = (waiting > streaming ? waiting : streaming) + 3.0;
+                    if (sl > 1) cost += 2.5 + (double)(sl + 1) * M * N * 4 / 2.0e6 + (emit_g ? 1.5 : 0.0);
+                    if (best < 0 || cost < best) {
+                        best = cost;
+                        skinny = false;
+                        tile = v.id;
+                        slices = sl;
+                    }
+                }
+            }
+        }
+        if (skinny) {
             pick_skinny(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream, hand);
             HB_CHECK_LAUNCH("gemm_skinny");
             return 0;
         }
-    }
-    HB_REQUIRE(!norm_w && (!emit_g || emit_whole), "gemm_mfma: the tiled product neither norms its input nor leaves half a norm");
-    if (tile == 0 && K % 64) tile = 123;
-    if (tile == 0 && M <= 64) {
-        // 17 to 64 rows: the product is bound by the weights it reads. Tiles one block of rows high,
-        // 128 wide (256 for wide products of more than 32 rows: fewer activations are read again), and
-        // K cut until about 192 workgroups stream: measured best for 4096- to 24576-wide products.
-        tile = M <= 32 ? 112 : (N >= 8192 ? 184 : 124);
-        const long tiles = (N + (tile == 184 ? 255 : 127)) / (tile == 184 ? 256 : 128);
-        while (tiles * slices < 192 && slices < 16 && slices_fit(K / 64, 2 * slices)) slices *= 2;
-        if (emit_whole && slices == 1) {
-            HB_REQUIRE(slices_fit(K / 64, 2), "gemm_mfma: K=%d or the workspace is too small to leave a norm behind", K);
-            slices = 2;
+        if (tile == 0) {
+            HB_REQUIRE(!emit_g && !scale_partial, "gemm_mfma: a product of M=%d, N=%d, K=%d cannot hand a norm on", M, N, K);
+            tile = 123;
         }
     }
+    HB_REQUIRE(!norm_w, "gemm_mfma: the tiled product does not norm its input");
+    HB_REQUIRE(!emit_g || (slices > 1 && reducer_norms && tile_hint == 0), "gemm_mfma: this product leaves no norm behind");
+    if (tile == 0 && K % 64) tile = 123;
     // tile_hint: 0 = choose (otherwise a variant by number, for measurements and tests; + 1000 x the
     // number of K slices). The bigger the tile, the more arithmetic per byte moved and the higher
     // its rate, but the fewer tiles there are for the 256 CUs; with few tiles and a long K, K is
@@ -1219,9 +1284,9 @@ extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N,
     }
     if (rc == 0 && slices > 1) {
         const size_t total = (size_t)M * N;
-        if (emit_whole)
+        if (emit_g)
             gemm_slices_norm_kernel<<<M, 1024, 0, stream>>>(workspace, (float*)C, M, N, ldc, slices, emit_g, emit_eps,
-                                                           (bf16*)emit_xg);
+                                                           (bf16*)emit_xg, emit_partial);
         else if (epi == EPI_SWIGLU)
             gemm_slices_swiglu_kernel<<<(unsigned)((total / 2 + 255) / 256), 256, 0, stream>>>(workspace, (bf16*)C, M, N,
                                                                                              ldc, slices);

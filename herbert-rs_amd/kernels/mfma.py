@@ -25,11 +25,9 @@ SLICE_WORKSPACE_FLOATS = 16 << 20     # most that the tiled product may use for 
 
 
 def _slice_workspace(device, M, N, K, tile=0):
-    """(pointer, floats) of the scratch for products whose K is cut into slices: more than 16 rows
-    and too few tiles of 128 x 128 to give every CU one. The kernel takes as many slices as fit in
-    it. A buffer that was handed out is kept for good: a captured graph may hold its address."""
-    if M <= 16 and not tile:
-        return None, 0
+    """(pointer, floats) of the scratch for products whose K may be cut into slices: too few tiles
+    of 128 x 128 to give every CU one. The kernel takes as many slices as fit in it. A buffer that
+    was handed out is kept for good: a captured graph may hold its address."""
     tiles = ((M + 127) // 128) * ((N + 127) // 128)
     slices = min(16, K // 256) if tiles < 256 or tile else 1
     need = min(slices * M * N, SLICE_WORKSPACE_FLOATS)
