@@ -1132,36 +1132,13 @@ extern "C" int hb_gemm_qkv_mfma(const void* X, const void* W, int M, int K, int 
                         m_tiles, n_tiles, stream, (float*)nullptr, e, RowScale{});
 }
 
-// C (+)= X @ W^T. X [M, K] bf16, W [N, K] bf16. epi 0: C f32 [M, N] stored; 1: added to;
-// 2: W's rows are gate/up interleaved in blocks of 16 and C is bf16 [M, N / 2] = silu(gate) * up.
-// packed != 0: W is stored as [K / 32][N / 16][64 lanes][8]: lane = 16 * (k / 8 % 4) + n % 16.
-// All blocks of one k-step lie together: workgroups that advance through K side by side read one
-// contiguous stretch of memory at a time, as a streaming copy would.
-// workspace: float scratch for K cut into slices (more than 16 rows); without it K is not cut.
-// norm_w != null: X is the float32 residual stream [M, K] and the product is RMSNorm(X; norm_w, eps) W^T
-// (M <= 16 only, never with the add epilogue).
-// hand_*: see NormHandoff (all null / 0 for a product that neither leaves nor takes a norm).
-extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N, int K, int ldc, int epi,
-                            int packed, const float* norm_w, float eps, int tile_hint, float* workspace,
-                            size_t workspace_floats, const float* emit_g, void* emit_xg, float* emit_partial,
-                            const float* scale_partial, int scale_parts, float scale_eps, float emit_eps,
-                            hipStream_t stream) {
-    const NormHandoff hand = {emit_g, (bf16*)emit_xg, emit_partial, scale_partial, scale_parts, scale_eps, emit_eps};
-    const bool emit_whole = emit_g && !emit_partial;      // the second kernel of a product cut into slices norms
-    HB_REQUIRE(!scale_partial || (M <= 16 && !norm_w), "gemm_mfma: a norm is handed on for at most 16 rows");
-    HB_REQUIRE(!emit_g || (epi == EPI_ADD && emit_xg && !norm_w), "gemm_mfma: only the adding product leaves a norm behind");
-    HB_REQUIRE(!emit_g || (emit_whole ? M > 16 && M <= 64 : M <= 16),
-               "gemm_mfma: a norm is left half done for at most 16 rows, whole for 17 to 64 rows");
-    HB_REQUIRE(!scale_partial || (scale_parts > 0 && epi != EPI_ADD), "gemm_mfma: bad partial sums of a handed-on norm");
-    HB_REQUIRE(!norm_w || (M <= 16 && epi != EPI_ADD && (epi == EPI_SWIGLU || N >= 16384)),
-               "gemm_mfma: the fused norm takes M <= 16, N >= 16384 and no add");
-    HB_REQUIRE(!packed || N % 16 == 0, "gemm_mfma: packed weights need N %% 16 == 0");
-    HB_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_mfma: empty problem (M=%d, N=%d, K=%d)", M, N, K);
-    HB_REQUIRE(epi >= 0 && epi <= 2, "gemm_mfma: unknown epilogue %d", epi);
-    HB_REQUIRE(K % 32 == 0, "gemm_mfma: K=%d is no multiple of 32", K);
-    HB_REQUIRE(epi != EPI_SWIGLU || N % 32 == 0, "gemm_mfma: the SwiGLU epilogue needs N %% 32 == 0");
-    HB_REQUIRE(ldc >= (epi == EPI_SWIGLU ? N / 2 : N), "gemm_mfma: output row stride %d too small", ldc);
-    const RowScale row_scale = {scale_partial, scale_parts, scale_eps};
+// Which kernel a product runs on: tile 0 = the few-row kernel, otherwise a tile variant by number and
+// the number of K slices; tile -1: nothing takes this product with what is asked of it. The flags
+// say whether the input is normed on the way (norm_w), a norm is left behind (emit_g) or a handed-on
+// one is finished (scale_partial).
+struct GemmPlan { int tile, slices; };
+static GemmPlan plan_gemm(int M, int N, int K, int ldc, int epi, bool norm_w, bool emit_g, bool scale_partial,
+                          int tile_hint, size_t workspace_floats) {
     int tile = tile_hint % 1000, slices = tile_hint >= 1000 ? tile_hint / 1000 : 1;
     // no slice of K may be empty, and each has at least four steps to run through its ring
     auto slices_fit = [&](int steps, int sl) {
@@ -1224,18 +1201,13 @@ extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N,
                 }
             }
         }
-        if (skinny) {
-            pick_skinny(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream, hand);
-            HB_CHECK_LAUNCH("gemm_skinny");
-            return 0;
-        }
+        if (skinny) return GemmPlan{0, 1};
         if (tile == 0) {
-            HB_REQUIRE(!emit_g && !scale_partial, "gemm_mfma: a product of M=%d, N=%d, K=%d cannot hand a norm on", M, N, K);
+            if (emit_g || scale_partial) return GemmPlan{-1, 0};
             tile = 123;
         }
     }
-    HB_REQUIRE(!norm_w, "gemm_mfma: the tiled product does not norm its input");
-    HB_REQUIRE(!emit_g || (slices > 1 && reducer_norms && tile_hint == 0), "gemm_mfma: this product leaves no norm behind");
+    if (norm_w || (emit_g && !(slices > 1 && reducer_norms && tile_hint == 0))) return GemmPlan{-1, 0};
     if (tile == 0 && K % 64) tile = 123;
     // tile_hint: 0 = choose (otherwise a variant by number, for measurements and tests; + 1000 x the
     // number of K slices). The bigger the tile, the more arithmetic per byte moved and the higher
@@ -1265,6 +1237,57 @@ extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N,
             }
         }
     }
+    return GemmPlan{tile, slices};
+}
+
+// The plan as a number for tests and measurements: tile + 1000 x slices (slices > 1), 0 for the
+// few-row kernel, -1 if the product is refused. emit: 0 none, 1 a norm is left behind.
+extern "C" int hb_gemm_mfma_plan(int M, int N, int K, int epi, int normed_input, int emit, int scaled,
+                                 size_t workspace_floats) {
+    const GemmPlan p = plan_gemm(M, N, K, epi == EPI_SWIGLU ? N / 2 : N, epi, normed_input != 0, emit != 0, scaled != 0, 0,
+                                 workspace_floats);
+    return p.tile <= 0 ? p.tile : p.tile + (p.slices > 1 ? 1000 * p.slices : 0);
+}
+
+// C (+)= X @ W^T. X [M, K] bf16, W [N, K] bf16. epi 0: C f32 [M, N] stored; 1: added to;
+// 2: W's rows are gate/up interleaved in blocks of 16 and C is bf16 [M, N / 2] = silu(gate) * up.
+// packed != 0: W is stored as [K / 32][N / 16][64 lanes][8]: lane = 16 * (k / 8 % 4) + n % 16.
+// All blocks of one k-step lie together: workgroups that advance through K side by side read one
+// contiguous stretch of memory at a time, as a streaming copy would.
+// workspace: float scratch for K cut into slices (more than 16 rows); without it K is not cut.
+// norm_w != null: X is the float32 residual stream [M, K] and the product is RMSNorm(X; norm_w, eps) W^T
+// (M <= 16 only, never with the add epilogue).
+// hand_*: see NormHandoff (all null / 0 for a product that neither leaves nor takes a norm).
+extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N, int K, int ldc, int epi,
+                            int packed, const float* norm_w, float eps, int tile_hint, float* workspace,
+                            size_t workspace_floats, const float* emit_g, void* emit_xg, float* emit_partial,
+                            const float* scale_partial, int scale_parts, float scale_eps, float emit_eps,
+                            hipStream_t stream) {
+    const NormHandoff hand = {emit_g, (bf16*)emit_xg, emit_partial, scale_partial, scale_parts, scale_eps, emit_eps};
+    const bool emit_whole = emit_g && !emit_partial;      // the second kernel of a product cut into slices norms
+    HB_REQUIRE(!scale_partial || (M <= 16 && !norm_w), "gemm_mfma: a norm is handed on for at most 16 rows");
+    HB_REQUIRE(!emit_g || (epi == EPI_ADD && emit_xg && !norm_w), "gemm_mfma: only the adding product leaves a norm behind");
+    HB_REQUIRE(!emit_g || (emit_whole ? M > 16 && M <= 64 : M <= 16),
+               "gemm_mfma: a norm is left half done for at most 16 rows, whole for 17 to 64 rows");
+    HB_REQUIRE(!scale_partial || (scale_parts > 0 && epi != EPI_ADD), "gemm_mfma: bad partial sums of a handed-on norm");
+    HB_REQUIRE(!norm_w || (M <= 16 && epi != EPI_ADD && (epi == EPI_SWIGLU || N >= 16384)),
+               "gemm_mfma: the fused norm takes M <= 16, N >= 16384 and no add");
+    HB_REQUIRE(!packed || N % 16 == 0, "gemm_mfma: packed weights need N %% 16 == 0");
+    HB_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_mfma: empty problem (M=%d, N=%d, K=%d)", M, N, K);
+    HB_REQUIRE(epi >= 0 && epi <= 2, "gemm_mfma: unknown epilogue %d", epi);
+    HB_REQUIRE(K % 32 == 0, "gemm_mfma: K=%d is no multiple of 32", K);
+    HB_REQUIRE(epi != EPI_SWIGLU || N % 32 == 0, "gemm_mfma: the SwiGLU epilogue needs N %% 32 == 0");
+    HB_REQUIRE(ldc >= (epi == EPI_SWIGLU ? N / 2 : N), "gemm_mfma: output row stride %d too small", ldc);
+    const RowScale row_scale = {scale_partial, scale_parts, scale_eps};
+    const GemmPlan plan = plan_gemm(M, N, K, ldc, epi, norm_w != nullptr, emit_g != nullptr, scale_partial != nullptr,
+                                    tile_hint, workspace_floats);
+    HB_REQUIRE(plan.tile >= 0, "gemm_mfma: no kernel takes M=%d, N=%d, K=%d with the norm asked of it", M, N, K);
+    if (plan.tile == 0) {
+        pick_skinny(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream, hand);
+        HB_CHECK_LAUNCH("gemm_skinny");
+        return 0;
+    }
+    const int tile = plan.tile, slices = plan.slices;
     HB_REQUIRE(slices == 1 || (size_t)slices * M * N <= workspace_floats, "gemm_mfma: no room for %d slices", slices);
     HB_REQUIRE(!scale_partial || tile == 112, "gemm_mfma: only the few-row kernels take a handed-on norm");
     int rc;

@@ -14,6 +14,7 @@ _F = ctypes.c_float
 lib.register_signatures("gemm_mfma", {
     "hb_gemm_mfma": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _F, _I, _P, ctypes.c_size_t, _P, _P, _P, _P, _I, _F,
                      _F, _P],
+    "hb_gemm_mfma_plan": [_I, _I, _I, _I, _I, _I, _I, ctypes.c_size_t],
     "hb_gemm_qkv_mfma": [_P, _P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _F, _I, _I, _I, _P],
 })
 
@@ -145,6 +146,14 @@ def _handoff_args(M, N, K, leave, row_scale, accumulate, norm):
         _check(squares, "squares", torch.float32, ((K + 15) // 16, padded_rows(M)))
         args[3:6] = [squares.data_ptr(), squares.shape[0], float(eps)]
     return args
+
+
+def gemm_plan(M, N, K, epi=EPI_STORE, normed_input=False, leaves_norm=False, finishes_norm=False, device="cuda"):
+    """Which kernel hb_gemm_mfma picks for a product, for tests and measurements: 0 = the few-row
+    kernel, otherwise the tile variant + 1000 x the K slices (if more than one), -1 = refused."""
+    _, ws_floats = _slice_workspace(torch.device(device), M, N, K)
+    return lib.load("gemm_mfma").hb_gemm_mfma_plan(M, N, K, epi, int(normed_input), int(leaves_norm),
+                                                   int(finishes_norm), ws_floats)
 
 
 def gemm(a, w, out, accumulate=False, packed=False, norm=None, tile=0, leave=None, row_scale=None):
