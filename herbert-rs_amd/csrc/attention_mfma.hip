@@ -286,7 +286,7 @@ attn_decode_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_cache, bf16*
                    float* __restrict__ partial_o, float* __restrict__ partial_ml,
                    const int* __restrict__ context_lens, const int* __restrict__ slots,
                    const int* __restrict__ page_table, int max_pages, int nq, int nkv, float c, int window,
-                   int pages_per_split, DecodeFusion fu) {
+                   int pages_per_split, DecodeFusion fu, bf16* __restrict__ out) {
     const int b = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z, splits = gridDim.z;
     const int G = nq / nkv;
     const int lane = threadIdx.x, c32 = lane & 31, g2 = lane >> 5;
@@ -483,6 +483,23 @@ attn_decode_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_cache, bf16*
 #undef LOAD_K
 #undef LOAD_V
     l += __shfl_xor(l, 32, 64);
+    if (out) {
+        // one range a sequence: nothing to merge, the output is O / l (zeros if no key was visible)
+        if (c32 < G) {
+            const float inv = l > 0.f ? 1.0f / l : 0.f;
+            bf16* dst = out + ((size_t)b * nq + kvh * G + c32) * HD;
+#pragma unroll
+            for (int d = 0; d < HD / 32; ++d)
+#pragma unroll
+                for (int qd = 0; qd < 4; ++qd) {
+                    bf16x4 v;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) v[j] = (__bf16)(oacc[d][4 * qd + j] * inv);
+                    *(bf16x4*)((__bf16*)dst + d * 32 + 8 * qd + 4 * g2) = v;
+                }
+        }
+        return;
+    }
     if (c32 < G) {
         const size_t base = ((size_t)b * nq + kvh * G + c32) * splits + split;
         if (g2 == 0) {
@@ -608,18 +625,20 @@ extern "C" int hb_attn_decode_mfma(const void* q, void* k_cache, void* v_cache, 
     dim3 grid(B, nkv, splits);
     const float c = scale * LOG2E;
     const DecodeFusion fu = {qkv, q_norm_w, k_norm_w, cos_t, sin_t, eps, write_kv};
+    bf16* const direct = splits == 1 ? (bf16*)out : nullptr;      // one range: the kernel writes the output itself
     HB_REQUIRE(qkv || q, "attn_decode: neither q nor the projection rows are given");
     HB_REQUIRE((cos_t == nullptr) == (sin_t == nullptr), "attn_decode: cos and sin tables come together");
 #define LAUNCH_DECODE(HDV) do {                                                                          \
     if (qkv)                                                                                             \
         attn_decode_kernel<HDV, true><<<grid, 64, 0, stream>>>(nullptr, (bf16*)k_cache, (bf16*)v_cache,  \
             partial_o, partial_ml, context_lens, slots, page_table, max_pages, nq, nkv, c, window,       \
-            pages_per_split, fu);                                                                        \
+            pages_per_split, fu, direct);                                                                \
     else                                                                                                 \
         attn_decode_kernel<HDV, false><<<grid, 64, 0, stream>>>((const bf16*)q, (bf16*)k_cache,          \
             (bf16*)v_cache, partial_o, partial_ml, context_lens, slots, page_table, max_pages, nq, nkv,  \
-            c, window, pages_per_split, fu);                                                             \
-    attn_decode_merge_kernel<HDV><<<B * nq, 256, 0, stream>>>(partial_o, partial_ml, (bf16*)out, splits, c); \
+            c, window, pages_per_split, fu, direct);                                                     \
+    if (!direct)                                                                                         \
+        attn_decode_merge_kernel<HDV><<<B * nq, 256, 0, stream>>>(partial_o, partial_ml, (bf16*)out, splits, c); \
     } while (0)
     if (hd == 32) LAUNCH_DECODE(32);
     else if (hd == 64) LAUNCH_DECODE(64);

@@ -285,12 +285,18 @@ def _prefill_tiles(meta):
     return tiles
 
 
+DECODE_WAVES = 1024       # waves the decode kernel is cut into at least, where the contexts are long enough
+
+
 def _decode_split(meta, nkv, window):
-    """(ranges, pages per range): enough waves for the 256 CUs, every range at least one page."""
+    """(ranges, pages per range): enough waves for the 256 CUs, every range at least one page. With
+    one range the kernel writes the output itself and no merge runs."""
     span = (meta.context_bucket + 63) // 64     # by bucket, so that a captured graph's grid stays right
     if window:
         span = min(span, (window + 63) // 64 + 1)
-    want = max(1, -(-1024 // (meta.num_seqs * nkv)))
+    want = max(1, -(-DECODE_WAVES // (meta.num_seqs * nkv)))
+    if 2 * meta.num_seqs * nkv >= DECODE_WAVES:      # two waves a CU already: a merge would cost more than it gains
+        want = 1
     splits = max(1, min(span, want, 32))      # the merge's cost grows with the ranges
     per = -(-span // splits)
     return -(-span // per), per

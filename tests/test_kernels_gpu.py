@@ -228,8 +228,11 @@ def test_attention_mfma_prefill(nq, nkv, hd, window):
 @pytest.mark.parametrize("nq,nkv,hd,window", [(4, 1, 128, 0), (32, 8, 128, 0), (6, 2, 32, 0), (5, 1, 64, 70),
                                               (3, 3, 128, 100), (64, 2, 64, 0)])
 @pytest.mark.parametrize("lengths", [[1, 64, 65, 700], [1000], [130, 3, 512, 999, 77, 640, 64, 128, 256]])
-def test_attention_mfma_decode(nq, nkv, hd, window, lengths):
+@pytest.mark.parametrize("waves", [1024, 1])
+def test_attention_mfma_decode(nq, nkv, hd, window, lengths, waves, monkeypatch):
+    """waves = 1: every sequence is one range, and the kernel writes the output without a merge."""
     from herbert_rs_amd.kernels import mfma
+    monkeypatch.setattr(mfma, "DECODE_WAVES", waves)
     meta, kv, dense = paged_case(lengths, [1] * len(lengths), nkv, hd, torch.bfloat16, seed=nq + hd,
                                  n_pages=80)
     q = rand(len(lengths), nq * hd, seed=22, dtype=torch.bfloat16)
@@ -337,11 +340,14 @@ def test_gemm_qkv_with_norm_rotation_and_cache_write(nq, nkv, norm, rope, packed
                                                         (6, 2, 32, 0, True, False), (5, 1, 64, 70, False, True),
                                                         (3, 3, 128, 100, True, True), (64, 2, 64, 0, False, False)])
 @pytest.mark.parametrize("lengths", [[1, 64, 65, 700], [1000], [130, 3, 512, 999, 77, 640, 64, 128, 256]])
-def test_attention_mfma_decode_fused_with_norm_rotation_and_cache_write(nq, nkv, hd, window, norm, rope, lengths):
+@pytest.mark.parametrize("waves", [1024, 1])
+def test_attention_mfma_decode_fused_with_norm_rotation_and_cache_write(nq, nkv, hd, window, norm, rope, lengths,
+                                                                        waves, monkeypatch):
     """The decode kernel that norms, rotates and writes the new key and value itself against the
-    separate kernels: same pages afterwards, same output."""
+    separate kernels: same pages afterwards, same output (waves = 1: without a merge)."""
     from herbert_rs_amd.cache.paged import LayerKV
     from herbert_rs_amd.kernels import mfma, ops
+    monkeypatch.setattr(mfma, "DECODE_WAVES", waves)
     B = len(lengths)
     meta, kv, _ = paged_case(lengths, [1] * B, nkv, hd, torch.bfloat16, seed=nq + hd, n_pages=80)
     kv2 = LayerKV(kv.k.clone(), kv.v.clone(), kv.page_table, 64, 0)
