@@ -270,6 +270,8 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache
 // given, over the whole head) itself: every wave for its query heads, and the one wave whose
 // range holds the new position also for the new key and value, which it writes to the pages
 // before it reads them (write_kv == 0: the keys and values are another layer's).
+// QS > 1: the projection was cut into QS slices of K whose sums lie slice_stride floats apart
+// behind qkv; the kernel adds them up in their order as it loads them (no kernel of its own does).
 struct DecodeFusion {
     const float* qkv;
     const float* q_norm_w;
@@ -278,9 +280,10 @@ struct DecodeFusion {
     const float* sin_t;
     float eps;
     int write_kv;
+    size_t slice_stride;
 };
 
-template <int HD, bool FUSED>
+template <int HD, bool FUSED, int QS = 1>
 __global__ void __launch_bounds__(64)
 attn_decode_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_cache, bf16* __restrict__ v_cache,
                    float* __restrict__ partial_o, float* __restrict__ partial_ml,
@@ -332,19 +335,29 @@ attn_decode_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_cache, bf16*
             qw0 = fu.q_norm_w[j];
             qw1 = fu.q_norm_w[j + HALF];
         }
+        // (all slices of a value are asked for together and added in their order)
+        auto summed = [&](const float* p) {
+            float part[QS];
+#pragma unroll
+            for (int i = 0; i < QS; ++i) part[i] = p[(size_t)i * fu.slice_stride];
+            float sum = part[0];
+#pragma unroll
+            for (int i = 1; i < QS; ++i) sum += part[i];
+            return sum;
+        };
 #pragma unroll
         for (int it = 0; it < PRE; ++it) {
             const int hl = it * PER + sub < G ? it * PER + sub : G - 1;
-            xq0[it] = qin[hl * HD + j];
-            xq1[it] = qin[hl * HD + j + HALF];
+            xq0[it] = summed(qin + hl * HD + j);
+            xq1[it] = summed(qin + hl * HD + j + HALF);
         }
         if (writer) {
             const float* kin = row + (size_t)(nq + kvh) * HD;
             const float* vin = row + (size_t)(nq + nkv + kvh) * HD;
-            k0 = kin[j];
-            k1 = kin[j + HALF];
-            v0 = vin[j];
-            v1 = vin[j + HALF];
+            k0 = summed(kin + j);
+            k1 = summed(kin + j + HALF);
+            v0 = summed(vin + j);
+            v1 = summed(vin + j + HALF);
             if (fu.k_norm_w) {
                 kw0 = fu.k_norm_w[j];
                 kw1 = fu.k_norm_w[j + HALF];
@@ -424,7 +437,13 @@ attn_decode_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_cache, bf16*
         for (int it = PRE; it * PER < G; ++it) {
             const int hl = it * PER + sub;
             const int hs = hl < G ? hl : G - 1;
-            finish_head(hl, qin[hs * HD + j], qin[hs * HD + j + HALF]);
+            float x0 = 0.f, x1 = 0.f;
+#pragma unroll
+            for (int i = 0; i < QS; ++i) {
+                x0 += qin[(size_t)i * fu.slice_stride + hs * HD + j];
+                x1 += qin[(size_t)i * fu.slice_stride + hs * HD + j + HALF];
+            }
+            finish_head(hl, x0, x1);
         }
     };
     // The first page's operands go out before that work, so that it hides their way from memory,
@@ -610,43 +629,56 @@ extern "C" int hb_attn_prefill_mfma(const void* q, const void* k_cache, const vo
     return 0;
 }
 
-// qkv != null: the fused form (see DecodeFusion); q is then not read.
+// qkv != null: the fused form (see DecodeFusion); q is then not read. qkv_slices > 1 (2, 4 or 8, heads
+// of 128 only): qkv is the first of that many slices of the projection's sums, slice_stride floats apart.
 extern "C" int hb_attn_decode_mfma(const void* q, void* k_cache, void* v_cache, void* out,
                                    float* partial_o, float* partial_ml, const int* context_lens,
                                    const int* slots, const int* page_table, int max_pages, int page_size,
                                    int B, int nq, int nkv, int hd, float scale, int window, int splits,
                                    int pages_per_split, const float* qkv, const float* q_norm_w,
                                    const float* k_norm_w, const float* cos_t, const float* sin_t, float eps,
-                                   int write_kv, hipStream_t stream) {
+                                   int write_kv, int qkv_slices, size_t slice_stride, hipStream_t stream) {
     HB_REQUIRE(B > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attn_decode: bad sizes");
     HB_REQUIRE(page_size == PAGE, "attn_decode: pages must hold %d tokens", PAGE);
     HB_REQUIRE(nq / nkv <= 32, "attn_decode: more than 32 query heads share a kv head");
     HB_REQUIRE(splits > 0 && splits <= 1024 && pages_per_split > 0 && nkv <= 65535, "attn_decode: bad split");
     HB_REQUIRE(window >= 0, "attn_decode: bad window");
     HB_REQUIRE(scale > 0.f, "attn_decode: the score scale must be positive");
+    HB_REQUIRE(qkv_slices == 1 || (qkv && hd == 128 && (qkv_slices == 2 || qkv_slices == 4 || qkv_slices == 8) &&
+                                   slice_stride >= (size_t)B * (nq + 2 * nkv) * hd),
+               "attn_decode: %d slices of the projection are not taken here", qkv_slices);
     dim3 grid(B, nkv, splits);
     const float c = scale * LOG2E;
-    const DecodeFusion fu = {qkv, q_norm_w, k_norm_w, cos_t, sin_t, eps, write_kv};
+    const DecodeFusion fu = {qkv, q_norm_w, k_norm_w, cos_t, sin_t, eps, write_kv, slice_stride};
     bf16* const direct = splits == 1 ? (bf16*)out : nullptr;      // one range: the kernel writes the output itself
     HB_REQUIRE(qkv || q, "attn_decode: neither q nor the projection rows are given");
     HB_REQUIRE((cos_t == nullptr) == (sin_t == nullptr), "attn_decode: cos and sin tables come together");
+#define DECODE_ARGS(QPTR) QPTR, (bf16*)k_cache, (bf16*)v_cache, partial_o, partial_ml, context_lens, slots, \
+                          page_table, max_pages, nq, nkv, c, window, pages_per_split, fu, direct
 #define LAUNCH_DECODE(HDV) do {                                                                          \
     if (qkv)                                                                                             \
-        attn_decode_kernel<HDV, true><<<grid, 64, 0, stream>>>(nullptr, (bf16*)k_cache, (bf16*)v_cache,  \
-            partial_o, partial_ml, context_lens, slots, page_table, max_pages, nq, nkv, c, window,       \
-            pages_per_split, fu, direct);                                                                \
+        attn_decode_kernel<HDV, true><<<grid, 64, 0, stream>>>(DECODE_ARGS(nullptr));                    \
     else                                                                                                 \
-        attn_decode_kernel<HDV, false><<<grid, 64, 0, stream>>>((const bf16*)q, (bf16*)k_cache,          \
-            (bf16*)v_cache, partial_o, partial_ml, context_lens, slots, page_table, max_pages, nq, nkv,  \
-            c, window, pages_per_split, fu, direct);                                                     \
-    if (!direct)                                                                                         \
-        attn_decode_merge_kernel<HDV><<<B * nq, 256, 0, stream>>>(partial_o, partial_ml, (bf16*)out, splits, c); \
+        attn_decode_kernel<HDV, false><<<grid, 64, 0, stream>>>(DECODE_ARGS((const bf16*)q));            \
     } while (0)
+    if (qkv_slices == 2) attn_decode_kernel<128, true, 2><<<grid, 64, 0, stream>>>(DECODE_ARGS(nullptr));
+    else if (qkv_slices == 4) attn_decode_kernel<128, true, 4><<<grid, 64, 0, stream>>>(DECODE_ARGS(nullptr));
+    else if (qkv_slices == 8) attn_decode_kernel<128, true, 8><<<grid, 64, 0, stream>>>(DECODE_ARGS(nullptr));
+    else
     if (hd == 32) LAUNCH_DECODE(32);
     else if (hd == 64) LAUNCH_DECODE(64);
     else if (hd == 128) LAUNCH_DECODE(128);
     else HB_REQUIRE(false, "attn_decode: head_dim %d is not one of 32, 64, 128", hd);
 #undef LAUNCH_DECODE
+#undef DECODE_ARGS
     HB_CHECK_LAUNCH("attn_decode");
+    if (!direct) {
+#define LAUNCH_MERGE(HDV) attn_decode_merge_kernel<HDV><<<B * nq, 256, 0, stream>>>(partial_o, partial_ml, (bf16*)out, splits, c)
+        if (hd == 32) LAUNCH_MERGE(32);
+        else if (hd == 64) LAUNCH_MERGE(64);
+        else LAUNCH_MERGE(128);
+#undef LAUNCH_MERGE
+        HB_CHECK_LAUNCH("attn_decode_merge");
+    }
     return 0;
 }

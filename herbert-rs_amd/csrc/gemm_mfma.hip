@@ -1083,7 +1083,8 @@ static int launch_tile64(const void* X, const void* W, void* C, int M, int N, in
     const bf16* x = (const bf16*)X;
     const bf16* w = (const bf16*)W;
     HB_REQUIRE(slices >= 1 && (slices == 1 || partial), "gemm_mfma: bad slices");
-    HB_REQUIRE(!scale.partial || (M <= 16 && slices == 1 && epi != EPI_ADD), "gemm_mfma: this product takes no handed-on norm");
+    // (a handed-on norm and K slices go together: every slice's sums are scaled, and so is their sum)
+    HB_REQUIRE(!scale.partial || (M <= 16 && epi != EPI_ADD), "gemm_mfma: this product takes no handed-on norm");
     HB_REQUIRE((K / 64 + slices - 1) / slices * (slices - 1) < K / 64, "gemm_mfma: a slice of K would be empty");
 #define EXTRA , partial, QkvEpilogue{}, scale
     TILE_DISPATCH(gemm_tile_kernel, TNB, TMB, WNW, WMW, WST, XST);
@@ -1138,7 +1139,7 @@ extern "C" int hb_gemm_qkv_mfma(const void* X, const void* W, int M, int K, int 
 // one is finished (scale_partial).
 struct GemmPlan { int tile, slices; };
 static GemmPlan plan_gemm(int M, int N, int K, int ldc, int epi, bool norm_w, bool emit_g, bool scale_partial,
-                          int tile_hint, size_t workspace_floats) {
+                          int tile_hint, size_t workspace_floats, bool deferred = false) {
     int tile = tile_hint % 1000, slices = tile_hint >= 1000 ? tile_hint / 1000 : 1;
     // no slice of K may be empty, and each has at least four steps to run through its ring
     auto slices_fit = [&](int steps, int sl) {
@@ -1179,10 +1180,9 @@ static GemmPlan plan_gemm(int M, int N, int K, int ldc, int epi, bool norm_w, bo
                 const long tiles = (N + v.bn - 1) / v.bn;
                 for (int sl = 1; sl <= 16; sl *= 2) {
                     if (sl > 1 && !slices_fit(steps, sl)) break;
-                    // a norm is left behind by the kernel that adds the slices up; a handed-on one is
-                    // finished in the epilogue of a product that is not cut
+                    // a norm is left behind by the kernel that adds the slices up
                     if (emit_g && (sl == 1 || !reducer_norms)) continue;
-                    if (scale_partial && sl > 1) break;
+                    if (deferred && sl > 8) break;                 // whoever adds the slices up takes 2, 4 or 8
                     const long wgs = tiles * sl, slots = 256 * v.per_cu;
                     const long rounds = (wgs + slots - 1) / slots;
                     const long on_a_cu = ((wgs < slots ? wgs : slots) + 255) / 256;
@@ -1191,7 +1191,7 @@ static GemmPlan plan_gemm(int M, int N, int K, int ldc, int epi, bool norm_w, bo
                     double streaming = (double)wgs * per * (v.bn * 128 + v.bm * 64) / 6.0e6;   // bound by HBM
                     if (wgs > slots) streaming *= 1.12;
                     double cost = (waiting > streaming ? waiting : streaming) + 3.0;
-                    if (sl > 1) cost += 2.5 + (double)(sl + 1) * M * N * 4 / 2.0e6 + (emit_g ? 1.5 : 0.0);
+                    if (sl > 1) cost += deferred ? 0.3 * sl : 2.5 + (double)(sl + 1) * M * N * 4 / 2.0e6 + (emit_g ? 1.5 : 0.0);
                     if (best < 0 || cost < best) {
                         best = cost;
                         skinny = false;
@@ -1241,11 +1241,12 @@ static GemmPlan plan_gemm(int M, int N, int K, int ldc, int epi, bool norm_w, bo
 }
 
 // The plan as a number for tests and measurements: tile + 1000 x slices (slices > 1), 0 for the
-// few-row kernel, -1 if the product is refused. emit: 0 none, 1 a norm is left behind.
+// few-row kernel, -1 if the product is refused. emit: 0 none, 1 a norm is left behind. deferred:
+// the slices are left for the next kernel to add up.
 extern "C" int hb_gemm_mfma_plan(int M, int N, int K, int epi, int normed_input, int emit, int scaled,
-                                 size_t workspace_floats) {
+                                 size_t workspace_floats, int deferred) {
     const GemmPlan p = plan_gemm(M, N, K, epi == EPI_SWIGLU ? N / 2 : N, epi, normed_input != 0, emit != 0, scaled != 0, 0,
-                                 workspace_floats);
+                                 workspace_floats, deferred != 0);
     return p.tile <= 0 ? p.tile : p.tile + (p.slices > 1 ? 1000 * p.slices : 0);
 }
 
@@ -1257,12 +1258,12 @@ extern "C" int hb_gemm_mfma_plan(int M, int N, int K, int epi, int normed_input,
 // workspace: float scratch for K cut into slices (more than 16 rows); without it K is not cut.
 // norm_w != null: X is the float32 residual stream [M, K] and the product is RMSNorm(X; norm_w, eps) W^T
 // (M <= 16 only, never with the add epilogue).
-// hand_*: see NormHandoff (all null / 0 for a product that neither leaves nor takes a norm).
+// emit_*, scale_*: see NormHandoff (all null / 0 for a product that neither leaves nor takes a norm).
 extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N, int K, int ldc, int epi,
                             int packed, const float* norm_w, float eps, int tile_hint, float* workspace,
                             size_t workspace_floats, const float* emit_g, void* emit_xg, float* emit_partial,
                             const float* scale_partial, int scale_parts, float scale_eps, float emit_eps,
-                            hipStream_t stream) {
+                            int* deferred_slices, hipStream_t stream) {
     const NormHandoff hand = {emit_g, (bf16*)emit_xg, emit_partial, scale_partial, scale_parts, scale_eps, emit_eps};
     const bool emit_whole = emit_g && !emit_partial;      // the second kernel of a product cut into slices norms
     HB_REQUIRE(!scale_partial || (M <= 16 && !norm_w), "gemm_mfma: a norm is handed on for at most 16 rows");
@@ -1279,8 +1280,13 @@ extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N,
     HB_REQUIRE(epi != EPI_SWIGLU || N % 32 == 0, "gemm_mfma: the SwiGLU epilogue needs N %% 32 == 0");
     HB_REQUIRE(ldc >= (epi == EPI_SWIGLU ? N / 2 : N), "gemm_mfma: output row stride %d too small", ldc);
     const RowScale row_scale = {scale_partial, scale_parts, scale_eps};
+    // deferred_slices != null (plain store only): if K is cut into slices, they are left in the
+    // workspace [slice][M][N] for the caller's next kernel to add up, and their number is written
+    // there; 1 means C holds the product as usual.
+    HB_REQUIRE(!deferred_slices || (epi == EPI_STORE && !emit_g && tile_hint == 0), "gemm_mfma: only a plain product leaves its slices");
+    if (deferred_slices) *deferred_slices = 1;
     const GemmPlan plan = plan_gemm(M, N, K, ldc, epi, norm_w != nullptr, emit_g != nullptr, scale_partial != nullptr,
-                                    tile_hint, workspace_floats);
+                                    tile_hint, workspace_floats, deferred_slices != nullptr);
     HB_REQUIRE(plan.tile >= 0, "gemm_mfma: no kernel takes M=%d, N=%d, K=%d with the norm asked of it", M, N, K);
     if (plan.tile == 0) {
         pick_skinny(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream, hand);
@@ -1304,6 +1310,10 @@ extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N,
             HB_REQUIRE(slices == 1, "gemm_mfma: this tile does not cut K");
             return launch_tile32<4, 4, 2, 2, 4>(X, W, C, M, N, K, ldc, epi, packed, stream);
         default: HB_REQUIRE(false, "gemm_mfma: unknown tile %d", tile);
+    }
+    if (rc == 0 && slices > 1 && deferred_slices) {
+        *deferred_slices = slices;
+        return 0;
     }
     if (rc == 0 && slices > 1) {
         const size_t total = (size_t)M * N;

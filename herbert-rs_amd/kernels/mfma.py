@@ -13,8 +13,8 @@ _I = ctypes.c_int
 _F = ctypes.c_float
 lib.register_signatures("gemm_mfma", {
     "hb_gemm_mfma": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _F, _I, _P, ctypes.c_size_t, _P, _P, _P, _P, _I, _F,
-                     _F, _P],
-    "hb_gemm_mfma_plan": [_I, _I, _I, _I, _I, _I, _I, ctypes.c_size_t],
+                     _F, _P, _P],
+    "hb_gemm_mfma_plan": [_I, _I, _I, _I, _I, _I, _I, ctypes.c_size_t, _I],
     "hb_gemm_qkv_mfma": [_P, _P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _F, _I, _I, _I, _P],
 })
 
@@ -148,18 +148,23 @@ def _handoff_args(M, N, K, leave, row_scale, accumulate, norm):
     return args
 
 
-def gemm_plan(M, N, K, epi=EPI_STORE, normed_input=False, leaves_norm=False, finishes_norm=False, device="cuda"):
+def gemm_plan(M, N, K, epi=EPI_STORE, normed_input=False, leaves_norm=False, finishes_norm=False, device="cuda",
+              defer_slices=False):
     """Which kernel hb_gemm_mfma picks for a product, for tests and measurements: 0 = the few-row
     kernel, otherwise the tile variant + 1000 x the K slices (if more than one), -1 = refused."""
     _, ws_floats = _slice_workspace(torch.device(device), M, N, K)
     return lib.load("gemm_mfma").hb_gemm_mfma_plan(M, N, K, epi, int(normed_input), int(leaves_norm),
-                                                   int(finishes_norm), ws_floats)
+                                                   int(finishes_norm), ws_floats, int(defer_slices))
 
 
-def gemm(a, w, out, accumulate=False, packed=False, norm=None, tile=0, leave=None, row_scale=None):
+def gemm(a, w, out, accumulate=False, packed=False, norm=None, tile=0, leave=None, row_scale=None,
+         defer_slices=False):
     """out f32 [M, N] (+)= a bf16 [M, K] @ w bf16 [N, K]^T (w as stored, or as pack_weight gives it).
     norm = (weight f32 [K], eps): a is the float32 residual stream and is RMS-normed on the way.
-    leave, row_scale: see _handoff_args."""
+    leave, row_scale: see _handoff_args.
+    defer_slices: if the kernel cuts K into slices it leaves their sums for the caller's next kernel
+    to add up; returns (slices, pointer to the first, floats between two): with slices == 1 `out`
+    holds the product as usual, otherwise `out` is not written."""
     M, K = a.shape
     norm_ptr, eps = _norm_args(a, norm, K)
     _check(w, "w", torch.bfloat16, (None, K))
@@ -171,9 +176,15 @@ def gemm(a, w, out, accumulate=False, packed=False, norm=None, tile=0, leave=Non
     if tile and leave is not None and leave[2] is None:
         raise BackendError("the whole norm is left behind by the product's own choice of tile")
     ws_ptr, ws_floats = _slice_workspace(a.device, M, N, K, tile)
+    if defer_slices and (accumulate or leave is not None or tile):
+        raise BackendError("only a plain product leaves its slices to the next kernel")
+    deferred = ctypes.c_int(1) if defer_slices else None
     lib.call("gemm_mfma", "hb_gemm_mfma", a.data_ptr(), w.data_ptr(), out.data_ptr(), M, N, K, N,
              EPI_ADD if accumulate else EPI_STORE, 1 if packed else 0, norm_ptr, eps, int(tile), ws_ptr,
-             ws_floats, *hand, _stream())
+             ws_floats, *hand, ctypes.byref(deferred) if defer_slices else None, _stream())
+    if defer_slices:
+        return (deferred.value, ws_ptr, M * N) if deferred.value > 1 else (1, out.data_ptr(), 0)
+    return None
 
 
 QKV_FUSE_MIN_M = 1024      # below that the plain product picks smaller tiles or cuts K, and wins
@@ -243,13 +254,14 @@ def gemm_swiglu(a, w_interleaved, out, packed=False, norm=None, tile=0, row_scal
     hand = _handoff_args(M, N, K, None, row_scale, False, norm)
     ws_ptr, ws_floats = _slice_workspace(a.device, M, N, K, tile)
     lib.call("gemm_mfma", "hb_gemm_mfma", a.data_ptr(), w_interleaved.data_ptr(), out.data_ptr(), M, N, K,
-             N // 2, EPI_SWIGLU, 1 if packed else 0, norm_ptr, eps, int(tile), ws_ptr, ws_floats, *hand, _stream())
+             N // 2, EPI_SWIGLU, 1 if packed else 0, norm_ptr, eps, int(tile), ws_ptr, ws_floats, *hand, None,
+             _stream())
 
 
 lib.register_signatures("attention_mfma", {
     "hb_attn_prefill_mfma": [_P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P],
     "hb_attn_decode_mfma": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I,
-                            _P, _P, _P, _P, _P, _F, _I, _P],
+                            _P, _P, _P, _P, _P, _F, _I, _I, ctypes.c_size_t, _P],
 })
 
 ATTENTION_HEAD_DIMS = (32, 64, 128)
@@ -322,10 +334,14 @@ def decode_fusable(meta, kv, nq, nkv, hd, rot_dims, dtype):
             and nq % nkv == 0 and nq // nkv <= 32 and rot_dims in (0, hd))
 
 
-def attention_decode_fused(qkv, q_norm_w, k_norm_w, cos, sin, meta, kv, out, nq, nkv, hd, eps, scale, window):
+def attention_decode_fused(qkv, q_norm_w, k_norm_w, cos, sin, meta, kv, out, nq, nkv, hd, eps, scale, window,
+                           qkv_slices=None):
     """One token a sequence: per-head norm (if weights are given), rotation (if tables are given),
     the new key and value written to the pages, and attention over them, in one kernel (+ merge).
-    qkv f32 [B, (nq + 2 nkv) hd]; cos / sin f32 [max_pos, hd / 2]; out bf16 [B, nq hd]."""
+    qkv f32 [B, (nq + 2 nkv) hd]; cos / sin f32 [max_pos, hd / 2]; out bf16 [B, nq hd].
+    qkv_slices = (slices, pointer, floats between two), as gemm(..., defer_slices=True) returns it:
+    the projection's sums are still in that many slices, which the kernel adds up as it loads them
+    (qkv itself is then not read)."""
     B = meta.num_seqs
     _check(qkv, "qkv", torch.float32, (B, (nq + 2 * nkv) * hd))
     _check(out, "out", torch.bfloat16, (B, nq * hd))
@@ -350,12 +366,18 @@ def attention_decode_fused(qkv, q_norm_w, k_norm_w, cos, sin, meta, kv, out, nq,
     window = int(window or 0)
     splits, per = _decode_split(meta, nkv, window)
     po, pml = _partial_buffers(qkv.device, B * nq, splits, hd)
+    n_slices, src, stride = qkv_slices if qkv_slices is not None else (1, qkv.data_ptr(), 0)
+    if n_slices > 1 and (n_slices not in DEFERRED_SLICES or hd != 128 or stride < qkv.numel()):
+        raise BackendError(f"fused decode attention does not add up {n_slices} slices of the projection")
     lib.call("attention_mfma", "hb_attn_decode_mfma", None, kv.k.data_ptr(), kv.v.data_ptr(), out.data_ptr(),
              po.data_ptr(), pml.data_ptr(), meta.context_lens.data_ptr(), meta.slots.data_ptr(),
              kv.page_table.data_ptr(), kv.page_table.shape[1], kv.page_size, B, nq, nkv, hd, float(scale),
-             window, splits, per, qkv.data_ptr(), None if q_norm_w is None else q_norm_w.data_ptr(),
+             window, splits, per, src, None if q_norm_w is None else q_norm_w.data_ptr(),
              None if k_norm_w is None else k_norm_w.data_ptr(), None if cos is None else cos.data_ptr(),
-             None if sin is None else sin.data_ptr(), float(eps), 1, _stream())
+             None if sin is None else sin.data_ptr(), float(eps), 1, n_slices, stride, _stream())
+
+
+DEFERRED_SLICES = (2, 4, 8)     # numbers of slices of the projection that the decode kernel adds up itself
 
 
 def attention(q, meta, kv, out, nq, nkv, hd, scale, window):
@@ -381,7 +403,7 @@ def attention(q, meta, kv, out, nq, nkv, hd, scale, window):
         lib.call("attention_mfma", "hb_attn_decode_mfma", q.data_ptr(), kv.k.data_ptr(), kv.v.data_ptr(),
                  out.data_ptr(), po.data_ptr(), pml.data_ptr(), meta.context_lens.data_ptr(),
                  meta.slots.data_ptr(), kv.page_table.data_ptr(), kv.page_table.shape[1], kv.page_size,
-                 T, nq, nkv, hd, float(scale), window, splits, per, None, None, None, None, None, 0.0, 0,
+                 T, nq, nkv, hd, float(scale), window, splits, per, None, None, None, None, None, 0.0, 0, 1, 0,
                  _stream())
         return
     _check(meta.positions, "positions", torch.int32, (T,))

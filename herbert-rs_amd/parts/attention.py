@@ -124,19 +124,24 @@ class Attention(Part):
                 self.project_out(ctx, attn, x)
                 return
         qkv = rt.buffer("qkv", (T, width), torch.float32)
+        fused_decode = False
+        if write_kv and rt.dtype == torch.bfloat16:
+            from ..kernels import mfma
+            fused_decode = mfma.decode_fusable(ctx.meta, kv, self.nq, self.nkv, self.hd, rot_dims, rt.dtype)
+        slices = None
         if fused_norm is not None:
             self.qkv.forward_normed(x, fused_norm.w, fused_norm.eps, qkv)
         else:
-            self.qkv.forward(y, qkv, row_scale=row_scale)
+            # (the fused decode kernel of heads of 128 adds up slices of K itself)
+            slices = self.qkv.forward(y, qkv, row_scale=row_scale, defer_slices=fused_decode and self.hd == 128)
         attn = rt.buffer("attn", (T, self.q_dim))
-        if write_kv and rt.dtype == torch.bfloat16:
-            from ..kernels import mfma
-            if mfma.decode_fusable(ctx.meta, kv, self.nq, self.nkv, self.hd, rot_dims, rt.dtype):
-                # one token a sequence: norm, rotation, cache write and attention in one kernel
-                mfma.attention_decode_fused(qkv, self.q_norm_w, self.k_norm_w, cos, sin, ctx.meta, kv, attn,
-                                            self.nq, self.nkv, self.hd, self.eps, self.scale, self.window)
-                self.project_out(ctx, attn, x)
-                return
+        if fused_decode:
+            # one token a sequence: norm, rotation, cache write and attention in one kernel
+            mfma.attention_decode_fused(qkv, self.q_norm_w, self.k_norm_w, cos, sin, ctx.meta, kv, attn,
+                                        self.nq, self.nkv, self.hd, self.eps, self.scale, self.window,
+                                        qkv_slices=slices)
+            self.project_out(ctx, attn, x)
+            return
         q = rt.buffer("q", (T, self.q_dim))
         ops.qk_norm_rope_write(qkv, self.q_norm_w, self.k_norm_w, cos, sin, rot_dims, ctx.meta, kv, q,
                                self.nq, self.nkv, self.hd, self.eps, write_kv=write_kv)

@@ -23,17 +23,20 @@ class Linear:
             self.packed = True
         self.weight = weight
 
-    def forward(self, a, out, accumulate=False, leave=None, row_scale=None):
+    def forward(self, a, out, accumulate=False, leave=None, row_scale=None, defer_slices=False):
         """out[M, N] (+)= a[M, K] @ W^T. leave and row_scale hand an RMSNorm from one product to the
-        next (see norm_handoff); they go to the MFMA kernel as kernels.mfma.gemm describes them."""
+        next (see norm_handoff); they go to the MFMA kernel as kernels.mfma.gemm describes them.
+        defer_slices: the caller's next kernel can add up slices of K; returns what kernels.mfma.gemm
+        returns for it, (1, pointer to out, 0) if the product is whole."""
         if self.weight.dtype == torch.bfloat16 and a.dtype == torch.bfloat16:
             from ..kernels import mfma
             if self.packed or mfma.gemm_supported(a, self.weight, out):
-                mfma.gemm(a, self.weight, out, accumulate, packed=self.packed, leave=leave, row_scale=row_scale)
-                return
+                return mfma.gemm(a, self.weight, out, accumulate, packed=self.packed, leave=leave,
+                                 row_scale=row_scale, defer_slices=defer_slices)
         if leave is not None or row_scale is not None:
             raise ValueError("this product cannot hand a norm on (ask norm_handoff first)")
         ops.gemm_plain(a, self.weight, out, accumulate)
+        return (1, out.data_ptr(), 0) if defer_slices else None
 
     def norm_handoff(self, rows):
         """How this product, for that many rows, can prepare the RMSNorm of the rows it adds to: "half"

@@ -351,6 +351,7 @@ def test_attention_mfma_decode_fused_with_norm_rotation_and_cache_write(nq, nkv,
     B = len(lengths)
     meta, kv, _ = paged_case(lengths, [1] * B, nkv, hd, torch.bfloat16, seed=nq + hd, n_pages=80)
     kv2 = LayerKV(kv.k.clone(), kv.v.clone(), kv.page_table, 64, 0)
+    before_k, before_v = kv.k.clone(), kv.v.clone()
     qkv = rand(B, (nq + 2 * nkv) * hd, seed=23, scale=1.5)
     qw = (1 + rand(hd, seed=24, scale=0.3)) if norm else None
     kw = (1 + rand(hd, seed=25, scale=0.3)) if norm else None
@@ -366,6 +367,20 @@ def test_attention_mfma_decode_fused_with_norm_rotation_and_cache_write(nq, nkv,
     mfma.attention(q, meta, kv, want, nq, nkv, hd, scale, window)
     got = torch.full_like(q, 7.0)
     mfma.attention_decode_fused(qkv, qw, kw, cos, sin, meta, kv2, got, nq, nkv, hd, eps, scale, window)
+    if hd == 128:
+        # the same projection rows in 2, 4 or 8 slices that sum to them exactly: the kernel adds them up
+        for n in mfma.DEFERRED_SLICES:
+            parts = torch.zeros(n, *qkv.shape, device=dev())
+            coarse = (qkv * 8).round() / 8                  # leaves a remainder that float32 adds back exactly
+            parts[0], parts[n - 1] = coarse / 2, coarse / 2
+            parts[n // 2] += qkv - coarse
+            assert torch.equal(parts.sum(0), qkv)
+            kv3 = LayerKV(kv2.k.clone().fill_(0), kv2.v.clone().fill_(0), kv.page_table, 64, 0)
+            kv3.k.copy_(before_k), kv3.v.copy_(before_v)
+            sliced = torch.full_like(q, 5.0)
+            mfma.attention_decode_fused(torch.empty_like(qkv), qw, kw, cos, sin, meta, kv3, sliced, nq, nkv, hd, eps,
+                                        scale, window, qkv_slices=(n, parts.data_ptr(), qkv.numel()))
+            assert torch.equal(sliced, got) and torch.equal(kv3.k, kv2.k) and torch.equal(kv3.v, kv2.v), n
     assert torch.equal(kv.v, kv2.v)
     # the two kernels sum the squares in another order: a key element may round the other way
     dk = (kv.k.float() - kv2.k.float()).abs()
