@@ -1141,6 +1141,7 @@ struct GemmPlan { int tile, slices; };
 static GemmPlan plan_gemm(int M, int N, int K, int ldc, int epi, bool norm_w, bool emit_g, bool scale_partial,
                           int tile_hint, size_t workspace_floats, bool deferred = false) {
     int tile = tile_hint % 1000, slices = tile_hint >= 1000 ? tile_hint / 1000 : 1;
+    if (tile_hint == 1) return M <= 16 ? GemmPlan{0, 1} : GemmPlan{-1, 0};      // the few-row kernel, asked for by name
     // no slice of K may be empty, and each has at least four steps to run through its ring
     auto slices_fit = [&](int steps, int sl) {
         const int per = (steps + sl - 1) / sl;
@@ -1207,7 +1208,7 @@ static GemmPlan plan_gemm(int M, int N, int K, int ldc, int epi, bool norm_w, bo
             tile = 123;
         }
     }
-    if (norm_w || (emit_g && !(slices > 1 && reducer_norms && tile_hint == 0))) return GemmPlan{-1, 0};
+    if (norm_w || (emit_g && !(slices > 1 && reducer_norms))) return GemmPlan{-1, 0};
     if (tile == 0 && K % 64) tile = 123;
     // tile_hint: 0 = choose (otherwise a variant by number, for measurements and tests; + 1000 x the
     // number of K slices). The bigger the tile, the more arithmetic per byte moved and the higher
@@ -1283,7 +1284,7 @@ extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N,
     // deferred_slices != null (plain store only): if K is cut into slices, they are left in the
     // workspace [slice][M][N] for the caller's next kernel to add up, and their number is written
     // there; 1 means C holds the product as usual.
-    HB_REQUIRE(!deferred_slices || (epi == EPI_STORE && !emit_g && tile_hint == 0), "gemm_mfma: only a plain product leaves its slices");
+    HB_REQUIRE(!deferred_slices || (epi == EPI_STORE && !emit_g), "gemm_mfma: only a plain product leaves its slices");
     if (deferred_slices) *deferred_slices = 1;
     const GemmPlan plan = plan_gemm(M, N, K, ldc, epi, norm_w != nullptr, emit_g != nullptr, scale_partial != nullptr,
                                     tile_hint, workspace_floats, deferred_slices != nullptr);

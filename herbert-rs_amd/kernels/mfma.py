@@ -173,10 +173,8 @@ def gemm(a, w, out, accumulate=False, packed=False, norm=None, tile=0, leave=Non
     if K % 32 or (norm is not None and accumulate):
         raise BackendError(f"gemm_mfma refuses M={M}, N={N}, K={K}")
     hand = _handoff_args(M, N, K, leave, row_scale, accumulate, norm)
-    if tile and leave is not None and leave[2] is None:
-        raise BackendError("the whole norm is left behind by the product's own choice of tile")
     ws_ptr, ws_floats = _slice_workspace(a.device, M, N, K, tile)
-    if defer_slices and (accumulate or leave is not None or tile):
+    if defer_slices and (accumulate or leave is not None):
         raise BackendError("only a plain product leaves its slices to the next kernel")
     deferred = ctypes.c_int(1) if defer_slices else None
     lib.call("gemm_mfma", "hb_gemm_mfma", a.data_ptr(), w.data_ptr(), out.data_ptr(), M, N, K, N,

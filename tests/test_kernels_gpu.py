@@ -533,6 +533,27 @@ def test_gemm_mfma_leaves_the_whole_norm_for_17_to_64_rows(M, H, K, packed):
     assert float(((y.float() - exact).abs() / exact.abs().clamp_min(1e-3)).max()) <= 2 ** -8 + 1e-4
 
 
+@pytest.mark.parametrize("tile", [1, 4112, 8112])
+def test_gemm_mfma_kernels_by_name_leave_the_same_norm(tile):
+    """The few-row kernel (1) and the tiled kernel with K slices, asked for by name, leave the same
+    half-done norm behind a product of 8 rows."""
+    from herbert_rs_amd.kernels import mfma
+    M, H, K = 8, 2048, 2048
+    a = rand(M, K, seed=81, dtype=torch.bfloat16)
+    w = mfma.pack_weight(rand(H, K, seed=82, dtype=torch.bfloat16, scale=0.1))
+    x0 = rand(M, H, seed=83, scale=2.0)
+    g = 1 + 0.1 * rand(H, seed=84)
+    x = x0.clone()
+    xg = torch.empty(M, H, dtype=torch.bfloat16, device=dev())
+    squares = torch.empty(H // 16, 8, device=dev())
+    mfma.gemm(a, w, x, accumulate=True, packed=True, leave=(g, xg, squares, 1e-6), tile=tile)
+    want_x = (x0.double() + a.double() @ rand(H, K, seed=82, dtype=torch.bfloat16, scale=0.1).double().T).float()
+    assert float((x - want_x).abs().max()) <= 2e-6 * K ** 0.5 * float(want_x.abs().max()) + 1e-4
+    assert torch.equal(xg, (x * g).to(torch.bfloat16))
+    want_squares = (x.double() ** 2).view(M, H // 16, 16).sum(-1).T
+    assert torch.allclose(squares.double(), want_squares, rtol=1e-6, atol=0)
+
+
 def test_gemm_mfma_refuses_a_handed_norm_it_cannot_do():
     from herbert_rs_amd.errors import BackendError
     from herbert_rs_amd.kernels import mfma
