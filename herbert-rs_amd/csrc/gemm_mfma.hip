@@ -1161,12 +1161,12 @@ static GemmPlan plan_gemm(int M, int N, int K, int ldc, int epi, bool norm_w, bo
         bool skinny = false;
         if (M <= 16) {
             // Workgroups of 16 (or 64) weight rows, each streaming at a rate of its own: about
-            // 24 KB/us alone on a CU (more if some CUs stay empty), 28 KB/us for a CU with several;
+            // 24 KB/us alone on a CU (more if some CUs stay empty), 28 KB/us for a CU with several of 16 rows;
             // more rows cost more reads of the activations. 320 workgroups on 256 CUs take as long as 512.
             const int nb = (epi == EPI_SWIGLU || N >= 16384) ? 4 : 1;
             const long wgs = (N + 16 * nb - 1) / (16 * nb);
             const double rounds = wgs <= 256 ? 1 : (wgs <= 512 ? 2 : wgs / 256.0 + 0.5);
-            double rate = (wgs <= 256 ? 24e3 : 28e3) / (1 + 0.02 * M);
+            double rate = (wgs <= 256 || nb == 4 ? 24e3 : 28e3) / (1 + 0.02 * M);
             if (wgs < 256) rate *= 1 + 0.6 * (256 - wgs) / 256.0;
             best = 3.0 + rounds * 32.0 * nb * K / rate;
             skinny = true;
