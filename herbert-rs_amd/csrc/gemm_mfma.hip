@@ -128,6 +128,20 @@ gemm_skinny_kernel(const void* __restrict__ Xv, const bf16* __restrict__ W, void
     float sumsq[MB];
 #pragma unroll
     for (int b = 0; b < MB; ++b) sumsq[b] = 0.f;
+    // What wave 0 adds its sums to, and the norm weights it needs to leave a norm behind, are asked
+    // for now: by the epilogue they have long arrived.
+    float c_before[NB][4], g_ahead[NB][4];
+    if (EPI == EPI_ADD && MB == 1 && wave == 0) {
+#pragma unroll
+        for (int a = 0; a < NB; ++a)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int n = n0 + a * 16 + g4 * 4 + i;
+                const bool in = r16 < M && n < N;
+                c_before[a][i] = in ? ((const float*)Cv)[(size_t)r16 * ldc + n] : 0.f;
+                g_ahead[a][i] = in && hand.emit_g ? hand.emit_g[n] : 0.f;
+            }
+    }
     const int mine = wave < nsteps ? (nsteps - wave + WAVES - 1) / WAVES : 0;   // this wave's steps
     const int groups = mine / U;
     SkinnyOperands<MB, NB, NORM> cur[U], nxt[U];
@@ -318,11 +332,11 @@ gemm_skinny_kernel(const void* __restrict__ Xv, const bf16* __restrict__ W, void
                     if (n < N) {
                         const size_t idx = (size_t)m * ldc + n;
                         float x = acc[a][b][i];
-                        if (EPI == EPI_ADD) x += C[idx];
+                        if (EPI == EPI_ADD) x += MB == 1 ? c_before[a][i] : C[idx];
                         C[idx] = x;
                         if (emit) {
                             squares = fmaf(x, x, squares);
-                            hand.emit_xg[(size_t)m * N + n] = hb_from_float<bf16>(x * hand.emit_g[n]);
+                            hand.emit_xg[(size_t)m * N + n] = hb_from_float<bf16>(x * g_ahead[a][i]);
                         }
                     }
                 }
