@@ -1,11 +1,15 @@
 // bfloat16 matrix products on the gfx950 matrix cores, float32 accumulation:
 //   C[m, n] (+)= sum_k X[m, k] * W[n, k]        X [M, K], W [N, K], both k-contiguous
-//   skinny (M <= 64, decoding): HBM-bound. The weights stream from memory straight into
+//   few rows (M <= 16, decoding): HBM-bound. The weights stream from memory straight into
 //     16x16x32 MFMA operands (each is used once), the waves of a workgroup split K between
 //     them and add their parts through LDS in a fixed order.
-//   tiled (M > 64, prompts): 32x32x16 MFMA; tiles of 256 x 256, 256 x 128 or 128 x 128 loaded
-//     from global memory straight into rings of LDS stages, a step of 64 k ahead of the MFMAs
-//     that consume them; with few tiles K is cut into slices over further workgroups.
+//   tiled: 32x32x16 MFMA; tiles loaded from global memory straight into rings of LDS stages, a
+//     step of 64 k ahead of the MFMAs that consume them; with few tiles K is cut into slices
+//     over further workgroups, whose sums a second kernel (or the caller's next kernel) adds up.
+//     256 x 256, 256 x 128 or 128 x 128 for prompts; one block of rows high (128 x 32, 128 x 64,
+//     256 x 64) for at most 64 rows, where it competes with the few-row kernel (see plan_gemm).
+// Between a product that adds to the residual stream and the next one an RMSNorm can be handed
+// on instead of run (see NormHandoff).
 // In both the weight rows are the MFMA's first operand, so a lane ends up with runs of four
 // consecutive n of one m: row-major stores of C are vector stores.
 // Epilogues: 0 store float32, 1 add to float32 (the residual stream), 2 SwiGLU to bfloat16
@@ -30,8 +34,9 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 __device__ __forceinline__ float silu_mul(float g, float u) { return g / (1.0f + __expf(-g)) * u; }
 
-// ------------------------------------------------------------------ skinny
-// Workgroup: WAVES waves, NB blocks of 16 weight rows, MB blocks of 16 activation rows.
+// ---------------------------------------------------------------- few rows
+// Workgroup: WAVES waves, NB blocks of 16 weight rows, MB blocks of 16 activation rows (built for
+// MB = 1: products of more than 16 rows go to the tiled kernel).
 // Wave w takes the k-steps (32 wide) s = w, w + WAVES, ...; it loads U steps ahead of the
 // ones it multiplies, so that enough bytes are in flight to keep HBM busy.
 // x * g of 8 consecutive k as an MFMA operand; the squares of x are added to ss.
