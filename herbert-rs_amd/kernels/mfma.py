@@ -313,15 +313,18 @@ def _decode_split(meta, nkv, window):
 
 
 def _partial_buffers(device, n_rows, splits, hd):
-    """(partial outputs, partial max / sum) of the decode kernel's ranges."""
-    key = str(device)
-    need_o = n_rows * splits * hd
-    buf = _partials.get(key)
-    if buf is None or buf[0].numel() < need_o or buf[1].numel() < n_rows * splits * 2:
-        buf = (torch.empty(need_o, dtype=torch.float32, device=device),
-               torch.empty(n_rows * splits * 2, dtype=torch.float32, device=device))
-        _partials[key] = buf
-    return buf
+    """(partial outputs, partial max / sum) of the decode kernel's ranges. Buffers that were handed
+    out are kept for good, also when larger ones replace them: a captured graph may hold their
+    addresses."""
+    kept = _partials.setdefault(str(device), [])
+    need_o, need_ml = n_rows * splits * hd, n_rows * splits * 2
+    if not kept or kept[-1][0].numel() < need_o or kept[-1][1].numel() < need_ml:
+        grow = 2 if kept else 1
+        kept.append((torch.empty(max(need_o, grow * (kept[-1][0].numel() if kept else 0)), dtype=torch.float32,
+                                 device=device),
+                     torch.empty(max(need_ml, grow * (kept[-1][1].numel() if kept else 0)), dtype=torch.float32,
+                                 device=device)))
+    return kept[-1]
 
 
 def decode_fusable(meta, kv, nq, nkv, hd, rot_dims, dtype):

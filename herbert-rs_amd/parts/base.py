@@ -49,6 +49,7 @@ class Runtime:
         self.dtype = dtype
         self.device = torch.device(device)
         self._buffers = {}
+        self._outgrown = []      # never freed: a captured graph may hold their addresses
 
     @property
     def exact(self):
@@ -56,7 +57,9 @@ class Runtime:
         return self.dtype == torch.float32
 
     def buffer(self, name, shape, dtype=None):
-        """A scratch tensor of at least this size, reused from call to call under its name."""
+        """A scratch tensor of at least this size, reused from call to call under its name. A
+        buffer that has become too small is replaced by one at least twice as large and kept all
+        the same (a captured graph may still write to it): what is kept is less than what is in use."""
         dtype = dtype or self.dtype
         n = 1
         for s in shape:
@@ -64,7 +67,12 @@ class Runtime:
         key = (name, dtype)
         buf = self._buffers.get(key)
         if buf is None or buf.numel() < n:
-            buf = torch.empty(max(n, 1), dtype=dtype, device=self.device)
+            if buf is not None:
+                self._outgrown.append(buf)
+                n_new = max(n, 2 * buf.numel())
+            else:
+                n_new = max(n, 1)
+            buf = torch.empty(n_new, dtype=dtype, device=self.device)
             self._buffers[key] = buf
         return buf[:n].view(*shape)
 

@@ -457,3 +457,41 @@ def test_norms_handed_from_product_to_product(name, batch, model_root, monkeypat
             assert ok, (i, hands_on, err)
     if batch <= 16 or name == "D":
         assert float(np.abs(got[True] - got[False]).max()) <= 2 ** -7 * float(np.abs(got[False]).max())
+
+
+def test_graphs_survive_larger_batches_that_outgrow_the_scratch_buffers(model_root):
+    """A graph captured for two sequences keeps writing to the scratch buffers of its time. A later
+    batch of nine needs larger ones: the old ones must stay allocated. Here other tensors are
+    allocated and filled in between, which would land in freed memory and be overwritten by the
+    graph of two when it is replayed afterwards; and that graph must still give what eager steps give."""
+    folder = make_folder(model_root, "D", "bfloat16")
+    vocab = CONFIGS["D"][0]["vocab_size"]
+    seqs = [random_tokens(vocab, 40, 700 + i) for i in range(9)]
+    outs = {}
+    for graphs in (False, True):
+        engine = hb.Engine.from_folder(folder, dtype="bfloat16", max_tokens=64 * 12, use_graphs=graphs)
+        two = [engine.alloc_slot() for _ in range(2)]
+        engine.step([StepEntry(s, seqs[i][:2], []) for i, s in enumerate(two)])          # prompts smaller than the batches
+        got = [engine.step([StepEntry(s, [seqs[i][p]], [0]) for i, s in enumerate(two)]).cpu().numpy()
+               for p in range(2, 8)]                                                      # captured on the second step
+        more = [engine.alloc_slot() for _ in range(7)]
+        engine.step([StepEntry(s, seqs[2 + i][:2], []) for i, s in enumerate(more)])
+        for p in range(2, 6):
+            engine.step([StepEntry(s, [seqs[2 + i][p]], [0]) for i, s in enumerate(more)] +
+                        [StepEntry(s, [seqs[i][6 + p]], [0]) for i, s in enumerate(two)])   # nine rows: larger buffers
+        # tensors of many small sizes: whatever was freed when the buffers grew is handed out again here
+        junk = [torch.full((128 << (i % 10),), float("nan"), device="cuda") for i in range(3000)]
+        torch.cuda.synchronize()
+        for s in more:
+            engine.free_slot(s)
+        got += [engine.step([StepEntry(s, [seqs[i][p]], [0]) for i, s in enumerate(two)]).cpu().numpy()
+                for p in range(12, 24)]                                                   # the graph of two again
+        torch.cuda.synchronize()
+        assert all(bool(torch.isnan(t).all()) for t in junk), "a replayed graph wrote into memory that was freed"
+        del junk
+        outs[graphs] = np.stack(got)
+        if graphs:
+            assert any(st.graphs for st in engine._decode.values())
+        engine.cache.check()
+    assert np.isfinite(outs[True]).all()
+    assert np.array_equal(outs[True], outs[False])
