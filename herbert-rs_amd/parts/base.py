@@ -132,7 +132,6 @@ class StepContext:
         if how is None:
             return None
         rows, width = x.shape
-        import torch
         squares = None
         xg = self.rt.buffer("handed_rows", (rows, width), torch.bfloat16)
         if how == "half":

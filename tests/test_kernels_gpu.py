@@ -554,6 +554,41 @@ def test_gemm_mfma_kernels_by_name_leave_the_same_norm(tile):
     assert torch.allclose(squares.double(), want_squares, rtol=1e-6, atol=0)
 
 
+@pytest.mark.parametrize("M,scaled", [(12, False), (8, True), (16, True), (40, False)])
+def test_gemm_mfma_leaves_its_slices_to_the_next_kernel(M, scaled):
+    """A plain product whose K is cut leaves the slices' sums in the workspace and says how many
+    there are: added up in their order they are the product, bit for bit what the second kernel
+    makes of them; a handed-on norm is finished in every slice."""
+    from herbert_rs_amd.kernels import mfma
+    N, K = 6144, 4096
+    a = rand(M, K, seed=90, dtype=torch.bfloat16)
+    w = rand(N, K, seed=91, dtype=torch.bfloat16, scale=0.05)
+    wp = mfma.pack_weight(w)
+    MP = mfma.padded_rows(M)
+    squares = (rand(K // 16, MP, seed=92).abs() + 0.5) * 16 if scaled else None
+    eps = 1e-6
+    row_scale = (squares, eps) if scaled else None
+    assert mfma.gemm_plan(M, N, K, finishes_norm=scaled, defer_slices=True) > 1000
+    out = torch.full((M, N), 7.0, device=dev())
+    n, ptr, stride = mfma.gemm(a, wp, out, packed=True, row_scale=row_scale, defer_slices=True)
+    assert n in mfma.DEFERRED_SLICES and stride == M * N and float(out.min()) == 7.0      # out is not written
+    parts = torch.empty(n, M, N, device=dev())
+    ws = mfma._workspaces[str(dev())][-1]
+    assert ws.data_ptr() == ptr
+    parts.copy_(ws[:n * M * N].view(n, M, N))
+    whole = torch.empty(M, N, device=dev())
+    mfma.gemm(a, wp, whole, packed=True, row_scale=row_scale)
+    summed = parts[0].clone()
+    for i in range(1, n):
+        summed += parts[i]
+    want = a.double() @ w.double().T
+    if scaled:
+        want = want * torch.rsqrt(squares.double().sum(0)[:M, None] / K + eps)
+    assert float((summed - want.float()).abs().max()) <= 2e-6 * K ** 0.5 * float(want.abs().max()) + 1e-4
+    if mfma.gemm_plan(M, N, K, finishes_norm=scaled) == mfma.gemm_plan(M, N, K, finishes_norm=scaled, defer_slices=True):
+        assert torch.equal(summed, whole)
+
+
 def test_gemm_mfma_refuses_a_handed_norm_it_cannot_do():
     from herbert_rs_amd.errors import BackendError
     from herbert_rs_amd.kernels import mfma
