@@ -185,14 +185,15 @@ def gemm(a, w, out, accumulate=False, packed=False, norm=None, tile=0, leave=Non
     return None
 
 
-QKV_FUSE_MIN_M = 1024      # below that the plain product picks smaller tiles or cuts K, and wins
+QKV_FUSE_MIN_TILES = 136   # of 256 x 256; with fewer (measured: 120 lose, 144 win) the plain product's smaller tiles or K slices fill the CUs better
 
 
 def gemm_qkv_fusable(a, w, meta, kv, nq, nkv, hd, rot_dims):
     """True if the q/k/v projection of this step should norm, rotate and write the cache itself:
     a long bfloat16 prompt step, heads of 128 rotated whole or not at all, pages of 64 tokens."""
     return (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and kv.k.dtype == torch.bfloat16
-            and a.shape[0] >= QKV_FUSE_MIN_M and a.shape[1] % 64 == 0 and hd == 128 and kv.page_size == 64
+            and -(-a.shape[0] // 256) * -(-w.shape[0] // 256) >= QKV_FUSE_MIN_TILES
+            and a.shape[1] % 64 == 0 and hd == 128 and kv.page_size == 64
             and rot_dims in (0, hd) and w.shape[0] == (nq + 2 * nkv) * hd and meta.num_tokens == a.shape[0])
 
 

@@ -87,10 +87,16 @@ def test_chunks_of_a_prompt_and_slots_used_again(dtype, model_root):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_long_prompts_with_heads_of_128(dtype, model_root):
+def test_long_prompts_with_heads_of_128(dtype, model_root, monkeypatch):
     """Heads of 128 and prompts of more than a thousand tokens: in bfloat16 the q/k/v projection
-    then norms, rotates and writes the cache itself, and decoding does so inside its attention
-    kernel. Whole, in a batch with a short prompt, in pieces, and decoded on: the plain logits."""
+    then norms, rotates and writes the cache itself (for a product whose tiles fill the GPU; this
+    small model's are let in by hand), and decoding does so inside its attention kernel. Whole, in
+    a batch with a short prompt, in pieces, and decoded on: the plain logits."""
+    from herbert_rs_amd.kernels import mfma
+    monkeypatch.setattr(mfma, "QKV_FUSE_MIN_TILES", 16)
+    fused = []
+    real = mfma.gemm_qkv
+    monkeypatch.setattr(mfma, "gemm_qkv", lambda *a, **k: (fused.append(1), real(*a, **k))[1])
     folder = make_folder(model_root, "D", dtype)
     vocab = CONFIGS["D"][0]["vocab_size"]
     a, b = random_tokens(vocab, 1100, 30), random_tokens(vocab, 45, 31)
@@ -117,6 +123,7 @@ def test_long_prompts_with_heads_of_128(dtype, model_root):
     assert close(piece, ref_a[1099], dtype)[0]
     engine.free_slot(s3)
     engine.cache.check()
+    assert (len(fused) > 0) == (dtype == "bfloat16")
 
 
 def test_a_batch_of_more_than_64_decodes_like_each_sequence_alone(model_root):

@@ -322,12 +322,12 @@ def test_gemm_qkv_with_norm_rotation_and_cache_write(nq, nkv, norm, rope, packed
     want_q = torch.full((T, nq * hd), 9.0, dtype=torch.bfloat16, device=dev())
     ops.qk_norm_rope_write(qkv, qw, kw, cos, sin, hd if rope else 0, meta, kv, want_q, nq, nkv, hd, eps)
     got_q = torch.full((T, nq * hd), 7.0, dtype=torch.bfloat16, device=dev())
-    old = mfma.QKV_FUSE_MIN_M
-    mfma.QKV_FUSE_MIN_M = 64
+    old = mfma.QKV_FUSE_MIN_TILES
+    mfma.QKV_FUSE_MIN_TILES = 1          # (the engine takes this path only when its tiles fill the GPU)
     try:
         assert mfma.gemm_qkv_fusable(a, wp, meta, kv2, nq, nkv, hd, hd if rope else 0)
     finally:
-        mfma.QKV_FUSE_MIN_M = old
+        mfma.QKV_FUSE_MIN_TILES = old
     mfma.gemm_qkv(a, wp, packed, qw, kw, cos, sin, meta, kv2, got_q, nq, nkv, hd, eps)
     # the two paths add the squares and the products in other orders: an element may round the other way
     for got, want in ((got_q, want_q), (kv2.k, kv.k), (kv2.v, kv.v)):
