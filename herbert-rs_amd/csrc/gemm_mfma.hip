@@ -1229,6 +1229,42 @@ static GemmPlan plan_gemm(int M, int N, int K, int ldc, int epi, bool norm_w, bo
     }
     if (norm_w || (emit_g && !(slices > 1 && reducer_norms))) return GemmPlan{-1, 0};
     if (tile == 0 && K % 64) tile = 123;
+    if (tile == 0 && M <= 1024 && K % 64 == 0) {
+        // 65 to 1024 rows: neither the arithmetic nor the weights alone decide. All tiles from 128 x 64
+        // to 256 x 256 with 1 to 16 K slices are candidates; a candidate takes as long as the slowest
+        // of: its workgroups' steps one after another (a step's time alone on a CU, about twice that
+        // with two on a CU), what all workgroups move out of the L2s (16 TB/s), what comes from
+        // HBM once (7 TB/s); plus a start and, for slices, the second kernel. Fitted to the four
+        // products of a layer for three model sizes and 96 to 1024 rows (the choice is then 1 % from
+        // the best candidate on average, 12 % at worst), checked on three other sizes (2 %, 13 %).
+        struct Mid { int id, bn, bm, per_cu; double step_us; };
+        static const Mid mid[] = {{188, 256, 256, 1, 1.26}, {142, 256, 128, 1, 0.77}, {122, 128, 128, 2, 0.95},
+                                  {124, 128, 64, 2, 0.48}, {184, 256, 64, 1, 0.67}};
+        const int steps = K / 64;
+        double best = -1;
+        for (const Mid& v : mid) {
+            const long tiles = (long)((M + v.bm - 1) / v.bm) * ((N + v.bn - 1) / v.bn);
+            for (int sl = 1; sl <= 16; sl *= 2) {
+                if (sl > 1 && !slices_fit(steps, sl)) break;
+                const long wgs = tiles * sl, slots = 256 * v.per_cu;
+                const long rounds = (wgs + slots - 1) / slots;
+                const long on_a_cu = ((wgs < slots ? wgs : slots) + 255) / 256;
+                const int per = (steps + sl - 1) / sl;
+                const double stepping = (double)rounds * per * v.step_us * (1 + 1.06 * (on_a_cu - 1));
+                const double moving = (double)wgs * per * (v.bn + v.bm) * 128 / 16.3e6;
+                const double fetching = ((double)N + M) * K * 2 / 7.1e6;
+                double cost = stepping > moving ? stepping : moving;
+                if (fetching > cost) cost = fetching;
+                cost += 2.3;
+                if (sl > 1) cost += 1.5 + (double)(sl + 1) * M * N * 4 / 2.3e6;
+                if (best < 0 || cost < best) {
+                    best = cost;
+                    tile = v.id;
+                    slices = sl;
+                }
+            }
+        }
+    }
     // tile_hint: 0 = choose (otherwise a variant by number, for measurements and tests; + 1000 x the
     // number of K slices). The bigger the tile, the more arithmetic per byte moved and the higher
     // its rate, but the fewer tiles there are for the 256 CUs; with few tiles and a long K, K is
