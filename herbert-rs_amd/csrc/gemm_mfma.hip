@@ -1229,14 +1229,15 @@ static GemmPlan plan_gemm(int M, int N, int K, int ldc, int epi, bool norm_w, bo
     }
     if (norm_w || (emit_g && !(slices > 1 && reducer_norms))) return GemmPlan{-1, 0};
     if (tile == 0 && K % 64) tile = 123;
-    if (tile == 0 && M <= 1024 && K % 64 == 0) {
-        // 65 to 1024 rows: neither the arithmetic nor the weights alone decide. All tiles from 128 x 64
+    if (tile == 0 && K % 64 == 0) {
+        // More than 64 rows: neither the arithmetic nor the weights alone decide. All tiles from 128 x 64
         // to 256 x 256 with 1 to 16 K slices are candidates; a candidate takes as long as the slowest
         // of: its workgroups' steps one after another (a step's time alone on a CU, about twice that
         // with two on a CU), what all workgroups move out of the L2s (16 TB/s), what comes from
         // HBM once (7 TB/s); plus a start and, for slices, the second kernel. Fitted to the four
         // products of a layer for three model sizes and 96 to 1024 rows (the choice is then 1 % from
-        // the best candidate on average, 12 % at worst), checked on three other sizes (2 %, 13 %).
+        // the best candidate on average, 12 % at worst), checked on three other sizes (2 %, 13 %) and
+        // on 1280 to 4096 rows (under 1 %, 7 %).
         struct Mid { int id, bn, bm, per_cu; double step_us; };
         static const Mid mid[] = {{188, 256, 256, 1, 1.26}, {142, 256, 128, 1, 0.77}, {122, 128, 128, 2, 0.95},
                                   {124, 128, 64, 2, 0.48}, {184, 256, 64, 1, 0.67}};
@@ -1265,34 +1266,8 @@ static GemmPlan plan_gemm(int M, int N, int K, int ldc, int epi, bool norm_w, bo
             }
         }
     }
-    // tile_hint: 0 = choose (otherwise a variant by number, for measurements and tests; + 1000 x the
-    // number of K slices). The bigger the tile, the more arithmetic per byte moved and the higher
-    // its rate, but the fewer tiles there are for the 256 CUs; with few tiles and a long K, K is
-    // cut into slices over further workgroups, whose sums a second kernel adds in their order.
-    // Taken: the variant and the slices with the least estimated time (us): rounds of workgroups
-    // over the CUs x steps x the time of a step as measured, + what the second pass moves.
-    struct Variant { int id, bn, bm, per_cu; double step_us; };
-    static const Variant variants[] = {{188, 256, 256, 1, 1.69}, {142, 256, 128, 1, 0.98}, {122, 128, 128, 2, 0.55}};
-    if (tile == 0) {
-        const int steps = K / 64;
-        double best = 0;
-        for (const Variant& v : variants) {
-            const long tiles = (long)((M + v.bm - 1) / v.bm) * ((N + v.bn - 1) / v.bn);
-            for (int sl = 1; sl <= 16; sl *= 2) {
-                if (sl > 1 && !slices_fit(steps, sl)) break;
-                const long wgs = tiles * sl;
-                const long rounds = (wgs + 256 * v.per_cu - 1) / (256 * v.per_cu);
-                const int share = wgs > 256 ? v.per_cu : 1;
-                double cost = (double)rounds * share * ((steps + sl - 1) / sl) * v.step_us + 5.0;
-                if (sl > 1) cost += 4.0 + (double)(sl + 2) * M * N * 4 / 2.5e6;
-                if (tile == 0 || cost < best) {
-                    tile = v.id;
-                    slices = sl;
-                    best = cost;
-                }
-            }
-        }
-    }
+    // (tile_hint: 0 = choose; otherwise a variant by number, for measurements and tests, + 1000 x
+    // the number of K slices; 1 = the few-row kernel)
     return GemmPlan{tile, slices};
 }
 
