@@ -71,8 +71,8 @@ struct SkinnyOperands {
 // for every block of 16 columns, the sum of x^2 over the block (emit_*); the product that follows
 // reads xg as its input and scales its sums by inv, which it gets by adding up those partial
 // sums in a fixed order (scale_*). No norm kernel runs in between.
-// With 17 to 64 rows K is cut into slices and a second kernel adds them up: it sees whole rows and
-// does the whole norm (emit_partial null, emit_eps its eps; emit_xg is then the normed rows).
+// With more than 16 rows K is (often) cut into slices and a second kernel adds them up: it sees whole
+// rows and does the whole norm (emit_partial null, emit_eps its eps; emit_xg is then the normed rows).
 struct NormHandoff {
     const float* emit_g;         // weight of the norm that follows, [N]; null: nothing is left behind
     bf16* emit_xg;               // [M, N]
@@ -1227,7 +1227,7 @@ static GemmPlan plan_gemm(int M, int N, int K, int ldc, int epi, bool norm_w, bo
             tile = 123;
         }
     }
-    if (norm_w || (emit_g && !(slices > 1 && reducer_norms))) return GemmPlan{-1, 0};
+    if (norm_w) return GemmPlan{-1, 0};
     if (tile == 0 && K % 64) tile = 123;
     if (tile == 0 && K % 64 == 0) {
         // More than 64 rows: neither the arithmetic nor the weights alone decide. All tiles from 128 x 64
@@ -1247,6 +1247,7 @@ static GemmPlan plan_gemm(int M, int N, int K, int ldc, int epi, bool norm_w, bo
             const long tiles = (long)((M + v.bm - 1) / v.bm) * ((N + v.bn - 1) / v.bn);
             for (int sl = 1; sl <= 16; sl *= 2) {
                 if (sl > 1 && !slices_fit(steps, sl)) break;
+                if (emit_g && (sl == 1 || !reducer_norms)) continue;      // the kernel that adds the slices up norms
                 const long wgs = tiles * sl, slots = 256 * v.per_cu;
                 const long rounds = (wgs + slots - 1) / slots;
                 const long on_a_cu = ((wgs < slots ? wgs : slots) + 255) / 256;
@@ -1268,6 +1269,7 @@ static GemmPlan plan_gemm(int M, int N, int K, int ldc, int epi, bool norm_w, bo
     }
     // (tile_hint: 0 = choose; otherwise a variant by number, for measurements and tests, + 1000 x
     // the number of K slices; 1 = the few-row kernel)
+    if (emit_g && !(slices > 1 && reducer_norms)) return GemmPlan{-1, 0};
     return GemmPlan{tile, slices};
 }
 
@@ -1299,8 +1301,8 @@ extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N,
     const bool emit_whole = emit_g && !emit_partial;      // the second kernel of a product cut into slices norms
     HB_REQUIRE(!scale_partial || (M <= 16 && !norm_w), "gemm_mfma: a norm is handed on for at most 16 rows");
     HB_REQUIRE(!emit_g || (epi == EPI_ADD && emit_xg && !norm_w), "gemm_mfma: only the adding product leaves a norm behind");
-    HB_REQUIRE(!emit_g || (emit_whole ? M > 16 && M <= 64 : M <= 16),
-               "gemm_mfma: a norm is left half done for at most 16 rows, whole for 17 to 64 rows");
+    HB_REQUIRE(!emit_g || (emit_whole ? M > 16 : M <= 16),
+               "gemm_mfma: a norm is left half done for at most 16 rows, whole for more");
     HB_REQUIRE(!scale_partial || (scale_parts > 0 && epi != EPI_ADD), "gemm_mfma: bad partial sums of a handed-on norm");
     HB_REQUIRE(!norm_w || (M <= 16 && epi != EPI_ADD && (epi == EPI_SWIGLU || N >= 16384)),
                "gemm_mfma: the fused norm takes M <= 16, N >= 16384 and no add");

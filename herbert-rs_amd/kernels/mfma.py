@@ -29,6 +29,9 @@ def _slice_workspace(device, M, N, K, tile=0):
     """(pointer, floats) of the scratch for products whose K may be cut into slices: too few tiles
     of 128 x 128 to give every CU one. The kernel takes as many slices as fit in it. A buffer that
     was handed out is kept for good: a captured graph may hold its address."""
+    device = torch.device(device)
+    if device.index is None:
+        device = torch.device(device.type, torch.cuda.current_device())
     tiles = ((M + 127) // 128) * ((N + 127) // 128)
     slices = min(16, K // 256) if tiles < 256 or tile else 1
     need = min(slices * M * N, SLICE_WORKSPACE_FLOATS)
@@ -98,20 +101,22 @@ def padded_rows(M):
     return 1 << max(0, int(M) - 1).bit_length()
 
 
-NORM_WHOLE_MAX_M = 64         # rows of a product whose second kernel (the sum of its K slices) can norm as well
+NORM_WHOLE_MAX_M = 64         # up to here a product that leaves a norm behind is cut into K slices for it
 NORM_WHOLE_MAX_N = 8192
 
 
 def norm_handoff(M, N, K):
     """How a product of these sizes that adds to the residual stream can prepare the RMSNorm that
     follows: "half" (at most 16 rows: bf16(x * g) and sums of squares, finished by the next product),
-    "whole" (17 to 64 rows: the kernel that adds up the K slices norms the rows too) or None."""
+    "whole" (more rows: the kernel that adds up the K slices norms the rows too; beyond 64 rows only
+    if the product is cut into slices anyway) or None."""
     if K % 32:
         return None
     if M <= NORM_HANDOFF_MAX_M:
         return "half"
-    if M <= NORM_WHOLE_MAX_M and K % 64 == 0 and K >= 512 and N % 4 == 0 and N <= NORM_WHOLE_MAX_N:
-        return "whole"
+    if K % 64 == 0 and K >= 512 and N % 4 == 0 and N <= NORM_WHOLE_MAX_N:
+        if M <= NORM_WHOLE_MAX_M or gemm_plan(M, N, K, EPI_ADD) >= 2000:
+            return "whole"
     return None
 
 

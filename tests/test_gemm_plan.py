@@ -1,0 +1,90 @@
+"""The choice of kernel for a matrix product is made on the host: its invariants are checked
+here without a GPU, over a grid of sizes (the library is compiled if it is not there yet)."""
+import itertools
+
+import pytest
+
+from herbert_rs_amd.kernels import lib
+
+EPI_STORE, EPI_ADD, EPI_SWIGLU = 0, 1, 2
+TILES = {112: (128, 32), 124: (128, 64), 184: (256, 64), 122: (128, 128), 142: (256, 128), 188: (256, 256), 123: (128, 128)}
+
+
+@pytest.fixture(scope="module")
+def plan():
+    from herbert_rs_amd.kernels import mfma  # noqa: F401  (registers the signatures)
+    fn = lib.load("gemm_mfma").hb_gemm_mfma_plan
+
+    def ask(M, N, K, epi=EPI_STORE, normed=False, emit=False, scaled=False, workspace=1 << 24, deferred=False):
+        return fn(M, N, K, epi, int(normed), int(emit), int(scaled), workspace, int(deferred))
+    return ask
+
+
+ROWS = [1, 2, 7, 8, 16, 17, 32, 33, 64, 65, 100, 256, 700, 1024, 2048, 5000]
+WIDTHS = [64, 1024, 2048, 4096, 5120, 6144, 12288, 24576, 151936]
+DEPTHS = [64, 128, 512, 2048, 2112, 4096, 12288, 25600]
+
+
+def test_every_plan_is_a_kernel_that_takes_the_product(plan):
+    for M, N, K in itertools.product(ROWS, WIDTHS, DEPTHS):
+        for epi in (EPI_STORE, EPI_ADD, EPI_SWIGLU):
+            p = plan(M, N, K, epi)
+            assert p >= 0, (M, N, K, epi)
+            if p == 0:
+                assert M <= 16
+                continue
+            tile, slices = p % 1000, max(1, p // 1000)
+            assert tile in TILES and (tile != 112 or M <= 32), (M, N, K, p)
+            steps = K // 64
+            if slices > 1:
+                per = -(-steps // slices)
+                assert per * (slices - 1) < steps, (M, N, K, p)            # no slice of K is empty
+                assert steps // slices >= 4 and slices * M * N <= 1 << 24, (M, N, K, p)
+                assert slices in (2, 4, 8, 16)
+
+
+def test_without_a_workspace_k_is_never_cut(plan):
+    for M, N, K in itertools.product(ROWS, WIDTHS, DEPTHS):
+        assert plan(M, N, K, EPI_ADD, workspace=0) < 1000
+
+
+def test_k_in_steps_of_32_only_goes_to_the_kernel_built_for_it(plan):
+    for M in (1, 16, 17, 64, 300):
+        p = plan(M, 4096, 4096 + 32)
+        assert p == (0 if M <= 16 else 123)
+
+
+def test_a_norm_is_left_behind_by_the_few_row_kernel_or_by_the_kernel_that_adds_slices(plan):
+    for M, N, K in itertools.product([1, 8, 16, 17, 40, 64, 128, 512], [192, 2048, 4096, 5120, 8192], [512, 4096, 25600]):
+        p = plan(M, N, K, EPI_ADD, emit=True)
+        if M <= 16:
+            assert p == 0 or p >= 2000, (M, N, K, p)
+        else:
+            assert p >= 2000 or p == -1, (M, N, K, p)          # -1: nothing fits; the caller then norms by itself
+            if M <= 64:
+                assert p >= 2000, (M, N, K, p)
+    assert plan(40, 8196, 4096, EPI_ADD, emit=True) == -1      # rows too wide for the adding kernel
+    assert plan(40, 4096, 4096, EPI_ADD, emit=True, workspace=0) == -1
+
+
+def test_a_handed_on_norm_is_finished_by_the_few_row_kernel_or_the_128x32_tile(plan):
+    for M, N, K in itertools.product([1, 8, 16], [1024, 6144, 24576, 51200], [1024, 4096, 5120]):
+        for epi in (EPI_STORE, EPI_SWIGLU):
+            p = plan(M, N, K, epi, scaled=True)
+            assert p == 0 or p % 1000 == 112, (M, N, K, epi, p)
+
+
+def test_slices_left_to_the_next_kernel_are_2_4_or_8(plan):
+    for M, N, K in itertools.product([1, 8, 16, 40], [4096, 6144, 10240], [2048, 4096, 8192]):
+        p = plan(M, N, K, deferred=True)
+        assert p // 1000 in (0, 2, 4, 8), (M, N, K, p)
+
+
+def test_known_choices(plan):
+    """A few choices that measurements decided: decoding 8 rows of the 8B shape, its prompt of 2048."""
+    assert plan(8, 4096, 4096, EPI_ADD, emit=True) == 0                # o: the few-row kernel
+    assert plan(8, 24576, 4096, EPI_SWIGLU, scaled=True) == 112        # gate/up: 128 x 32 tiles, no slices
+    assert plan(8, 5120, 25600, EPI_ADD, emit=True) >= 2000            # hidden 5120: 320 workgroups would not spread
+    assert plan(2048, 24576, 4096, EPI_SWIGLU) == 188
+    assert plan(2048, 4096, 12288, EPI_ADD) == 142
+    assert plan(64, 24576, 4096, EPI_SWIGLU) % 1000 in (124, 184)

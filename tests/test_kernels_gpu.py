@@ -512,10 +512,11 @@ def test_gemm_mfma_hands_a_norm_to_the_next_product(M, H, K1, N2, packed):
 
 
 @pytest.mark.parametrize("M,H,K,packed", [(17, 64, 512, True), (64, 4096, 4096, True), (40, 1028, 576, False),
-                                          (33, 8192, 1024, True)])
-def test_gemm_mfma_leaves_the_whole_norm_for_17_to_64_rows(M, H, K, packed):
+                                          (33, 8192, 1024, True), (128, 4096, 4096, True), (300, 2048, 6144, False)])
+def test_gemm_mfma_leaves_the_whole_norm_for_more_than_16_rows(M, H, K, packed):
     """K is cut into slices and the kernel that adds them to x norms the rows too: x is the product
-    added to what was there, and y the bfloat16 nearest to the norm of that x (or its neighbour)."""
+    added to what was there, and y the bfloat16 nearest to the norm of that x (or its neighbour).
+    Beyond 64 rows this is offered where the product is cut into slices anyway."""
     from herbert_rs_amd.kernels import mfma
     assert mfma.norm_handoff(M, H, K) == "whole"
     a = rand(M, K, seed=45, dtype=torch.bfloat16)
@@ -593,7 +594,7 @@ def test_gemm_mfma_refuses_a_handed_norm_it_cannot_do():
     from herbert_rs_amd.errors import BackendError
     from herbert_rs_amd.kernels import mfma
     assert mfma.norm_handoff(16, 64, 32) == "half" and mfma.norm_handoff(17, 64, 32) is None
-    assert mfma.norm_handoff(64, 8192, 512) == "whole" and mfma.norm_handoff(65, 8192, 512) is None
+    assert mfma.norm_handoff(64, 8192, 512) == "whole" and mfma.norm_handoff(2048, 4096, 4096) is None
     assert mfma.norm_handoff(64, 8196, 512) is None and mfma.norm_handoff(20, 64, 448) is None
     M, H = 17, 64
     a = rand(M, 32, seed=1, dtype=torch.bfloat16)
