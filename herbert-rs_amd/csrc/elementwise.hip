@@ -203,10 +203,12 @@ __global__ void qk_norm_rope_write_kernel(
 // a wave per token, lane = the pair (j, j + hd/2), rows read and written whole. Value heads go
 // through LDS, so that the transposed pages are written along the tokens: lane = token, 64
 // consecutive tokens of a page are one 128-byte line.
+// QS > 1: the projection was cut into QS slices of K whose sums lie slice_stride floats apart
+// behind qkv; they are added up in their order as they are loaded.
 #define HB_TILED_HEAD_DIM 128
-template <class TQ, class TC>
+template <class TQ, class TC, int QS>
 __global__ void __launch_bounds__(256) qk_norm_rope_write_tiled_kernel(
-    const float* __restrict__ qkv, int ld_qkv, const float* __restrict__ q_norm_w,
+    const float* __restrict__ qkv, int ld_qkv, size_t slice_stride, const float* __restrict__ q_norm_w,
     const float* __restrict__ k_norm_w, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
     const int* __restrict__ positions, const int* __restrict__ seq_of, const int* __restrict__ slots,
     const int* __restrict__ page_table, int max_pages, int page_size, TQ* __restrict__ q_out,
@@ -216,12 +218,21 @@ __global__ void __launch_bounds__(256) qk_norm_rope_write_tiled_kernel(
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const bool is_q = h < nq, is_v = h >= nq + nkv;
     const int half = hd / 2;
+    auto summed = [&](const float* p) {
+        float part[QS];
+#pragma unroll
+        for (int i = 0; i < QS; ++i) part[i] = p[(size_t)i * slice_stride];
+        float sum = part[0];
+#pragma unroll
+        for (int i = 1; i < QS; ++i) sum += part[i];
+        return sum;
+    };
     if (is_v) {
         const int kvh = h - nq - nkv;
         for (int idx = tid; idx < 64 * hd; idx += 256) {
             const int r = idx / hd, c = idx - r * hd;
             const int t = t0 + r;
-            vt[r][c] = t < T ? qkv[(size_t)t * ld_qkv + (size_t)h * hd + c] : 0.f;
+            vt[r][c] = t < T ? summed(qkv + (size_t)t * ld_qkv + (size_t)h * hd + c) : 0.f;
         }
         __syncthreads();
         const int t = t0 + lane;
@@ -247,8 +258,8 @@ __global__ void __launch_bounds__(256) qk_norm_rope_write_tiled_kernel(
             const int tc = t < T ? t : T - 1;
             const float* src = qkv + (size_t)tc * ld_qkv + (size_t)h * hd;
             pos[u] = positions[tc];
-            x0[u] = mine ? src[j] : 0.f;
-            x1[u] = mine ? src[j + half] : 0.f;
+            x0[u] = mine ? summed(src + j) : 0.f;
+            x1[u] = mine ? summed(src + j + half) : 0.f;
         }
         if (cos_t) {
 #pragma unroll
@@ -293,7 +304,7 @@ extern "C" int hb_qk_norm_rope_write(const float* qkv, int ld_qkv, const float* 
                                      const int* slots, const int* page_table, int max_pages,
                                      int page_size, void* q_out, void* k_cache, void* v_cache, int dtype,
                                      int T, int nq, int nkv, int hd, float eps, int write_kv,
-                                     hipStream_t stream) {
+                                     int qkv_slices, size_t slice_stride, hipStream_t stream) {
     HB_REQUIRE(T > 0 && nq > 0 && nkv > 0, "qk_norm_rope_write: empty input");
     HB_REQUIRE(hd > 0 && hd <= HB_MAX_HEAD_DIM, "qk_norm_rope_write: head_dim %d not in 1..%d", hd,
                HB_MAX_HEAD_DIM);
@@ -306,12 +317,21 @@ extern "C" int hb_qk_norm_rope_write(const float* qkv, int ld_qkv, const float* 
     if (dtype == HB_BF16 && write_kv && T >= 64 && hd <= HB_TILED_HEAD_DIM && hd % 2 == 0 &&
         (cos_t == nullptr || rot_dims == hd) && (T + 63) / 64 <= 0x7fffffff) {
         dim3 tiles((T + 63) / 64, heads);
-        qk_norm_rope_write_tiled_kernel<bf16, bf16><<<tiles, 256, 0, stream>>>(
-            qkv, ld_qkv, q_norm_w, k_norm_w, cos_t, sin_t, positions, seq_of, slots, page_table, max_pages,
-            page_size, (bf16*)q_out, (bf16*)k_cache, (bf16*)v_cache, T, nq, nkv, hd, eps);
+        HB_REQUIRE(qkv_slices == 1 || slice_stride >= (size_t)T * ld_qkv, "qk_norm_rope_write: slices overlap");
+#define TILED_GO(QSV)                                                                                          \
+    qk_norm_rope_write_tiled_kernel<bf16, bf16, QSV><<<tiles, 256, 0, stream>>>(                              \
+        qkv, ld_qkv, slice_stride, q_norm_w, k_norm_w, cos_t, sin_t, positions, seq_of, slots, page_table,    \
+        max_pages, page_size, (bf16*)q_out, (bf16*)k_cache, (bf16*)v_cache, T, nq, nkv, hd, eps)
+        if (qkv_slices == 1) TILED_GO(1);
+        else if (qkv_slices == 2) TILED_GO(2);
+        else if (qkv_slices == 4) TILED_GO(4);
+        else if (qkv_slices == 8) TILED_GO(8);
+        else HB_REQUIRE(false, "qk_norm_rope_write: %d slices of the projection are not taken", qkv_slices);
+#undef TILED_GO
         HB_CHECK_LAUNCH("qk_norm_rope_write_tiled");
         return 0;
     }
+    HB_REQUIRE(qkv_slices == 1, "qk_norm_rope_write: only the kernel for bfloat16 prompts of 64 tokens or more adds up slices");
     dim3 grid(T, heads);
     if (dtype == HB_F32)
         qk_norm_rope_write_kernel<float, float><<<grid, HB_WAVE, 0, stream>>>(

@@ -1248,6 +1248,7 @@ static GemmPlan plan_gemm(int M, int N, int K, int ldc, int epi, bool norm_w, bo
             for (int sl = 1; sl <= 16; sl *= 2) {
                 if (sl > 1 && !slices_fit(steps, sl)) break;
                 if (emit_g && (sl == 1 || !reducer_norms)) continue;      // the kernel that adds the slices up norms
+                if (deferred && sl > 8) break;                            // whoever adds the slices up takes 2, 4 or 8
                 const long wgs = tiles * sl, slots = 256 * v.per_cu;
                 const long rounds = (wgs + slots - 1) / slots;
                 const long on_a_cu = ((wgs < slots ? wgs : slots) + 255) / 256;
@@ -1258,7 +1259,7 @@ static GemmPlan plan_gemm(int M, int N, int K, int ldc, int epi, bool norm_w, bo
                 double cost = stepping > moving ? stepping : moving;
                 if (fetching > cost) cost = fetching;
                 cost += 2.3;
-                if (sl > 1) cost += 1.5 + (double)(sl + 1) * M * N * 4 / 2.3e6;
+                if (sl > 1) cost += deferred ? (double)sl * M * N * 4 / 2.3e6 : 1.5 + (double)(sl + 1) * M * N * 4 / 2.3e6;
                 if (best < 0 || cost < best) {
                     best = cost;
                     tile = v.id;

@@ -23,7 +23,7 @@ SIGNATURES = {
         "hb_embed": [_P, _P, _I, _P, _I, _I, _I, _I, _P],
         "hb_rmsnorm": [_P, _P, _P, _I, _P, _I, _I, _F, _P],
         "hb_qk_norm_rope_write": [_P, _I, _P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _P, _P, _P, _I,
-                                  _I, _I, _I, _I, _F, _I, _P],
+                                  _I, _I, _I, _I, _F, _I, _I, ctypes.c_size_t, _P],
         "hb_swiglu": [_P, _P, _I, _I, _I, _P],
         "hb_fill_u32": [_P, _U32, _SZ, _P],
     },

@@ -93,12 +93,25 @@ def _check_paged(meta, cache, T):
     _check(cache.v, "value pages", cache.k.dtype, (pages, nkv, hd, page))
 
 
+ROPE_WRITE_SLICES = (2, 4, 8)
+
+
+def rope_write_adds_slices(T, hd, rot_dims, dtype, write_kv, has_rotation):
+    """True if qk_norm_rope_write can add up K slices of the projection itself for such a step: the
+    kernel for bfloat16 prompts of 64 tokens or more does."""
+    return (dtype == torch.bfloat16 and write_kv and T >= 64 and hd <= 128 and hd % 2 == 0
+            and (not has_rotation or rot_dims == hd))
+
+
 def qk_norm_rope_write(qkv, q_norm_w, k_norm_w, cos, sin, rot_dims, meta, cache, q_out, nq, nkv, hd, eps,
-                       write_kv=True):
+                       write_kv=True, qkv_slices=None):
     """Per-head norm (if weights given), rotation (if tables given), q to q_out, k / v to the pages.
 
     qkv f32 [T, (nq + 2 nkv) hd] (query heads only when write_kv is false); cos / sin f32 [max_pos, rot_dims / 2]; q_out [T, nq hd] in the
     cache's dtype; cache.k / cache.v [pages, nkv, page_size, hd].
+    qkv_slices = (slices, pointer, floats between two), as kernels.mfma.gemm(..., defer_slices=True)
+    returns it: the projection's sums still lie in that many slices (see rope_write_adds_slices),
+    and qkv itself is not read.
     """
     T = qkv.shape[0]
     _check(qkv, "qkv", torch.float32, (T, (nq + (2 * nkv if write_kv else 0)) * hd))
@@ -115,12 +128,16 @@ def qk_norm_rope_write(qkv, q_norm_w, k_norm_w, cos, sin, rot_dims, meta, cache,
         if meta.max_position >= cos.shape[0]:
             raise BackendError(f"position {meta.max_position} beyond the rotation table "
                                f"({cos.shape[0]} rows)")
-    lib.call("elementwise", "hb_qk_norm_rope_write", qkv.data_ptr(), qkv.shape[1], _ptr(q_norm_w),
+    n_slices, src, stride = qkv_slices if qkv_slices is not None else (1, qkv.data_ptr(), 0)
+    if n_slices > 1 and (n_slices not in ROPE_WRITE_SLICES or stride < qkv.numel() or not rope_write_adds_slices(
+            T, hd, rot_dims, q_out.dtype, write_kv, cos is not None)):
+        raise BackendError(f"qk_norm_rope_write does not add up {n_slices} slices of the projection here")
+    lib.call("elementwise", "hb_qk_norm_rope_write", src, qkv.shape[1], _ptr(q_norm_w),
              _ptr(k_norm_w), _ptr(cos), _ptr(sin), rot_dims, meta.positions.data_ptr(),
              meta.seq_of.data_ptr(), meta.slots.data_ptr(), cache.page_table.data_ptr(),
              cache.page_table.shape[1], cache.page_size, q_out.data_ptr(), cache.k.data_ptr(),
              cache.v.data_ptr(), dtype_code(q_out), T, nq, nkv, hd, float(eps), 1 if write_kv else 0,
-             _stream())
+             n_slices, stride, _stream())
 
 
 def attention_plain(q, meta, cache, out, nq, nkv, hd, scale, window):

@@ -132,8 +132,11 @@ class Attention(Part):
         if fused_norm is not None:
             self.qkv.forward_normed(x, fused_norm.w, fused_norm.eps, qkv)
         else:
-            # (the fused decode kernel of heads of 128 adds up slices of K itself)
-            slices = self.qkv.forward(y, qkv, row_scale=row_scale, defer_slices=fused_decode and self.hd == 128)
+            # (the fused decode kernel of heads of 128 and the rotation kernel of bfloat16 prompts add
+            # up slices of K themselves)
+            defer = (fused_decode and self.hd == 128) or (not fused_decode and ops.rope_write_adds_slices(
+                T, self.hd, rot_dims, rt.dtype, write_kv, cos is not None))
+            slices = self.qkv.forward(y, qkv, row_scale=row_scale, defer_slices=defer)
         attn = rt.buffer("attn", (T, self.q_dim))
         if fused_decode:
             # one token a sequence: norm, rotation, cache write and attention in one kernel
@@ -144,7 +147,7 @@ class Attention(Part):
             return
         q = rt.buffer("q", (T, self.q_dim))
         ops.qk_norm_rope_write(qkv, self.q_norm_w, self.k_norm_w, cos, sin, rot_dims, ctx.meta, kv, q,
-                               self.nq, self.nkv, self.hd, self.eps, write_kv=write_kv)
+                               self.nq, self.nkv, self.hd, self.eps, write_kv=write_kv, qkv_slices=slices)
         self.attend(ctx, q, kv, attn)
         self.project_out(ctx, attn, x)
 

@@ -75,7 +75,7 @@ def test_a_handed_on_norm_is_finished_by_the_few_row_kernel_or_the_128x32_tile(p
 
 
 def test_slices_left_to_the_next_kernel_are_2_4_or_8(plan):
-    for M, N, K in itertools.product([1, 8, 16, 40], [4096, 6144, 10240], [2048, 4096, 8192]):
+    for M, N, K in itertools.product([1, 8, 16, 40, 100, 256, 700], [1024, 4096, 6144, 10240], [2048, 4096, 8192, 25600]):
         p = plan(M, N, K, deferred=True)
         assert p // 1000 in (0, 2, 4, 8), (M, N, K, p)
 

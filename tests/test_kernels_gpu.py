@@ -264,6 +264,20 @@ def test_qk_norm_rope_write(nq, nkv, hd, rot, norm, dtype):
         eps = 1e-5
         q = torch.full((T, nq * hd), 9.0, dtype=dtype, device=dev())
         ops.qk_norm_rope_write(qkv, qw, kw, cos, sin, rot, meta, kv, q, nq, nkv, hd, eps)
+        if ops.rope_write_adds_slices(T, hd, rot, dtype, True, cos is not None):
+            # the same rows in 2, 4 or 8 slices that sum to them exactly: the kernel adds them up
+            from herbert_rs_amd.cache.paged import LayerKV
+            for n in ops.ROPE_WRITE_SLICES:
+                parts = torch.zeros(n, *qkv.shape, device=dev())
+                coarse = (qkv * 8).round() / 8
+                parts[0], parts[n - 1] = coarse / 2, coarse / 2
+                parts[n // 2] += qkv - coarse
+                assert torch.equal(parts.sum(0), qkv)
+                kv_s = LayerKV(before_k.clone(), before_v.clone(), kv.page_table, kv.page_size, 0)
+                q_s = torch.full_like(q, 5.0)
+                ops.qk_norm_rope_write(torch.empty_like(qkv), qw, kw, cos, sin, rot, meta, kv_s, q_s, nq, nkv, hd, eps,
+                                       qkv_slices=(n, parts.data_ptr(), qkv.numel()))
+                assert torch.equal(q_s, q) and torch.equal(kv_s.k, kv.k) and torch.equal(kv_s.v, kv.v), n
 
         x = qkv.double().cpu().view(T, nq + 2 * nkv, hd)
         pos = meta.positions.cpu().long()
