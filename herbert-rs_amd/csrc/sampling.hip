@@ -118,6 +118,9 @@ __device__ __forceinline__ float key_float(uint32_t k) {
 
 #define SAMPLE_THREADS 1024
 #define SAMPLE_MAX_K 1024
+#define SAMPLE_AHEAD 8           // logits a thread asks for at once when it walks a row
+#define SAMPLE_LIST 4096         // keys of one first byte that the kernel keeps in LDS
+#define SAMPLE_CHUNK 8192        // logits of a row that one block sifts when a row is shared out over blocks
 
 // (key descending, index ascending) "a before b"
 __device__ __forceinline__ bool cand_before(uint32_t ka, int ia, uint32_t kb, int ib) {
@@ -147,14 +150,140 @@ __device__ void bitonic_sort_lds(uint32_t* keys, int* idx, int n_pow2) {
     __syncthreads();
 }
 
+// The bin of the `remaining`-th largest key, counted from the top of a histogram of 256 bins, by
+// the first 256 threads of the block: bin b is it if fewer than `remaining` keys lie above it and
+// at least `remaining` in it and above. Writes the chosen bin into the prefix and what is still
+// to be found inside that bin. (A single thread walking the bins costs 7 us a byte.)
+__device__ __forceinline__ void choose_bin(const int* hist, int* wave_totals, int shift, uint32_t prefix,
+                                           int remaining, uint32_t* sel_prefix, int* sel_remaining) {
+    const int tid = threadIdx.x, lane = tid & (HB_WAVE - 1);
+    int mine = 0, here_and_above = 0;
+    if (tid < 256) {
+        mine = hist[tid];
+        here_and_above = mine;                 // over the lanes from this one up
+        for (int d = 1; d < HB_WAVE; d <<= 1) {
+            const int other = __shfl_down(here_and_above, d, HB_WAVE);
+            if (lane + d < HB_WAVE) here_and_above += other;
+        }
+        if (lane == 0) wave_totals[tid / HB_WAVE] = here_and_above;
+    }
+    __syncthreads();
+    if (tid < 256) {
+        for (int w = tid / HB_WAVE + 1; w < 256 / HB_WAVE; ++w) here_and_above += wave_totals[w];
+        const int above = here_and_above - mine;
+        if (above < remaining && here_and_above >= remaining) {
+            *sel_prefix = prefix | ((uint32_t)tid << shift);
+            *sel_remaining = remaining - above;
+        }
+    }
+    __syncthreads();
+}
+
+// The first of two kernels when a row is long: block (chunk, row) keeps the keys of its SAMPLE_CHUNK
+// logits in LDS, finds its own top_k among them (ties: lower index first) and leaves them, in any
+// order, in pre_key / pre_idx [row][chunk][top_k]. A single block walks a row at about 24 GB/s
+// only; shared out over the CUs the 600 KB of a row of 151936 logits are read in a few us.
+__global__ void __launch_bounds__(SAMPLE_THREADS)
+sample_chunk_topk_kernel(const float* __restrict__ logits, int ld, int V, float temperature, int top_k,
+                         uint32_t* __restrict__ pre_key, int* __restrict__ pre_idx) {
+    __shared__ uint32_t ck[SAMPLE_CHUNK];
+    __shared__ int hist[256];
+    __shared__ int wave_counts[SAMPLE_THREADS / HB_WAVE];
+    __shared__ uint32_t sel_prefix;
+    __shared__ int sel_remaining, n_out, eq_taken;
+    const int tid = threadIdx.x, lane = tid & (HB_WAVE - 1), wave = tid / HB_WAVE;
+    const int c = blockIdx.x, first = c * SAMPLE_CHUNK;
+    const int len = V - first < SAMPLE_CHUNK ? V - first : SAMPLE_CHUNK;
+    const float* row = logits + (size_t)blockIdx.y * ld + first;
+    const size_t base = ((size_t)blockIdx.y * gridDim.x + c) * top_k;
+    constexpr int PER = SAMPLE_CHUNK / SAMPLE_THREADS;
+    float v[PER];
+#pragma unroll
+    for (int u = 0; u < PER; ++u) {
+        const int j = tid + u * SAMPLE_THREADS;
+        v[u] = j < len ? row[j] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < PER; ++u) {
+        const int j = tid + u * SAMPLE_THREADS;
+        if (j < len) ck[j] = float_key(v[u] / temperature);
+    }
+    if (tid == 0) {
+        sel_prefix = 0;
+        sel_remaining = top_k;
+        n_out = 0;
+        eq_taken = 0;
+    }
+    __syncthreads();
+    if (len <= top_k) {                       // all of a short chunk
+        for (int j = tid; j < len; j += SAMPLE_THREADS) {
+            pre_key[base + j] = ck[j];
+            pre_idx[base + j] = first + j;
+        }
+        return;
+    }
+    for (int shift = 24; shift >= 0; shift -= 8) {
+        if (tid < 256) hist[tid] = 0;
+        __syncthreads();
+        const uint32_t prefix = sel_prefix;
+        const int remaining = sel_remaining;
+        const uint32_t mask = shift == 24 ? 0u : (0xffffffffu << (shift + 8));
+        int run_bin = -1, run = 0;
+        for (int j = tid; j < len; j += SAMPLE_THREADS) {
+            const uint32_t k = ck[j];
+            if ((k & mask) != prefix) continue;
+            const int bin = (k >> shift) & 0xff;
+            if (bin == run_bin) {
+                ++run;
+            } else {
+                if (run) atomicAdd(&hist[run_bin], run);
+                run_bin = bin;
+                run = 1;
+            }
+        }
+        if (run) atomicAdd(&hist[run_bin], run);
+        __syncthreads();
+        choose_bin(hist, wave_counts, shift, prefix, remaining, &sel_prefix, &sel_remaining);
+    }
+    const uint32_t kth = sel_prefix;
+    const int need_eq = sel_remaining;
+    // the keys lie in LDS in the order of their indices: the equal ones are ranked stretch by stretch
+    for (int start = 0; start < len; start += SAMPLE_THREADS) {
+        const int j = start + tid;
+        const uint32_t k = j < len ? ck[j] : 0u;
+        const bool above = j < len && k > kth, equal = j < len && k == kth;
+        const unsigned long long bal = __ballot(equal);
+        const int before_lane = __popcll(bal & ((1ull << lane) - 1ull));
+        if (lane == 0) wave_counts[wave] = __popcll(bal);
+        __syncthreads();
+        int before = eq_taken;
+        for (int w = 0; w < wave; ++w) before += wave_counts[w];
+        if (above || (equal && before + before_lane < need_eq)) {
+            const int at = atomicAdd(&n_out, 1);
+            pre_key[base + at] = k;
+            pre_idx[base + at] = first + j;
+        }
+        __syncthreads();
+        if (tid == 0) {
+            int total = 0;
+            for (int w = 0; w < SAMPLE_THREADS / HB_WAVE; ++w) total += wave_counts[w];
+            eq_taken += total;
+        }
+        __syncthreads();
+    }
+}
+
 // One block per row, 0 < top_k <= SAMPLE_MAX_K and top_k < V.
 //  1. scaled = logit / temperature; the top_k largest (ties: lower index first) by a
 //     radix select over the keys, gathered and sorted in LDS;
 //  2. softmax over them; 3. top-p cut and renormalisation; 4. the draw.
+// pre_key != null: the row was cut into chunks of SAMPLE_CHUNK logits and sample_chunk_topk_kernel
+// has left the top_k of each chunk in pre_key / pre_idx [row][chunk][top_k] (a chunk shorter than
+// top_k: all of it); the top_k of the row are among them, and only they are walked.
 __global__ void __launch_bounds__(SAMPLE_THREADS)
 sample_topk_kernel(const float* __restrict__ logits, int ld, int V, float temperature, int top_k,
                    float top_p, unsigned long long* __restrict__ rng, const int* __restrict__ rng_index,
-                   int* __restrict__ out) {
+                   int* __restrict__ out, const uint32_t* __restrict__ pre_key, const int* __restrict__ pre_idx) {
     __shared__ uint32_t keys[SAMPLE_MAX_K];
     __shared__ int idx[SAMPLE_MAX_K];
     __shared__ float prob[SAMPLE_MAX_K];
@@ -168,77 +297,168 @@ sample_topk_kernel(const float* __restrict__ logits, int ld, int V, float temper
     const float* row = logits + (size_t)blockIdx.x * ld;
     const int tid = threadIdx.x;
 
-    // ---- radix select: the key of the top_k-th largest scaled logit
-    if (tid == 0) {
-        sel_prefix = 0;
-        sel_remaining = top_k;
-    }
-    for (int shift = 24; shift >= 0; shift -= 8) {
+    // ---- radix select: the key of the top_k-th largest scaled logit.
+    // One block reads a row at about 24 GB/s, so what counts is how often the row is walked:
+    // once for the histogram of the keys' first byte (sign and exponent), once more to collect
+    // what lies in the chosen bin into LDS (everything above it belongs to the top k anyway);
+    // the other three bytes are then decided on that list. A list that does not fit (flat
+    // logits) sends the kernel back to walking the row for every byte.
+    __shared__ uint32_t cand_key[SAMPLE_LIST];
+    __shared__ int cand_idx[SAMPLE_LIST];
+    __shared__ int eq_idx[SAMPLE_MAX_K];
+    __shared__ int cand_count, eq_count;
+    const int lane = tid & (HB_WAVE - 1), wave = tid / HB_WAVE;
+    // f(key, index) for every element of the row, SAMPLE_AHEAD loads of a thread in flight at once
+    const int chunks = (V + SAMPLE_CHUNK - 1) / SAMPLE_CHUNK;
+    auto walk_row = [&](auto&& f) {
+        if (pre_key) {
+            const size_t first = (size_t)blockIdx.x * chunks * top_k;
+            for (int t = tid; t < chunks * top_k; t += SAMPLE_THREADS) {
+                const int c = t / top_k, j = t - c * top_k;
+                const int len = V - c * SAMPLE_CHUNK < SAMPLE_CHUNK ? V - c * SAMPLE_CHUNK : SAMPLE_CHUNK;
+                if (j < (len < top_k ? len : top_k)) f(pre_key[first + t], pre_idx[first + t]);
+            }
+            return;
+        }
+        for (int base = tid; base < V; base += SAMPLE_AHEAD * SAMPLE_THREADS) {
+            float v[SAMPLE_AHEAD];
+#pragma unroll
+            for (int u = 0; u < SAMPLE_AHEAD; ++u) {
+                const int i = base + u * SAMPLE_THREADS;
+                v[u] = i < V ? row[i] : 0.f;
+            }
+#pragma unroll
+            for (int u = 0; u < SAMPLE_AHEAD; ++u) {
+                const int i = base + u * SAMPLE_THREADS;
+                if (i < V) f(float_key(v[u] / temperature), i);
+            }
+        }
+    };
+    // counts the byte at `shift` of the keys that f hands to count(key), runs of one bin at a time
+    auto choose_byte = [&](int shift, auto&& walk) {
         if (tid < 256) hist[tid] = 0;
         __syncthreads();
         const uint32_t prefix = sel_prefix;
+        const int remaining = sel_remaining;
         const uint32_t mask = shift == 24 ? 0u : (0xffffffffu << (shift + 8));
-        for (int i = tid; i < V; i += blockDim.x) {
-            const uint32_t k = float_key(row[i] / temperature);
-            if ((k & mask) == prefix) atomicAdd(&hist[(k >> shift) & 0xff], 1);
-        }
-        __syncthreads();
-        if (tid == 0) {
-            int remaining = sel_remaining;
-            int b = 255;
-            for (; b > 0; --b) {
-                if (hist[b] >= remaining) break;
-                remaining -= hist[b];
+        int run_bin = -1, run = 0;
+        walk([&](uint32_t k, int) {
+            if ((k & mask) != prefix) return;
+            const int bin = (k >> shift) & 0xff;
+            if (bin == run_bin) {
+                ++run;
+            } else {
+                if (run) atomicAdd(&hist[run_bin], run);
+                run_bin = bin;
+                run = 1;
             }
-            sel_prefix = prefix | ((uint32_t)b << shift);
-            sel_remaining = remaining;
-        }
+        });
+        if (run) atomicAdd(&hist[run_bin], run);
         __syncthreads();
+        choose_bin(hist, wave_counts, shift, prefix, remaining, &sel_prefix, &sel_remaining);
+    };
+    if (tid == 0) {
+        sel_prefix = 0;
+        sel_remaining = top_k;
+        n_gathered = 0;
+        eq_taken = 0;
+        eq_count = 0;
+        cand_count = 0;
+    }
+    choose_byte(24, walk_row);
+    {
+        const uint32_t first = sel_prefix >> 24;
+        walk_row([&](uint32_t k, int i) {
+            const uint32_t byte = k >> 24;
+            if (byte > first) {                       // above the chosen bin: one of the top k
+                const int at = atomicAdd(&n_gathered, 1);
+                keys[at] = k;
+                idx[at] = i;
+            } else if (byte == first) {
+                const int at = atomicAdd(&cand_count, 1);
+                if (at < SAMPLE_LIST) {
+                    cand_key[at] = k;
+                    cand_idx[at] = i;
+                }
+            }
+        });
+    }
+    __syncthreads();
+    const int listed = cand_count;
+    const bool from_list = listed <= SAMPLE_LIST;
+    auto walk_list = [&](auto&& f) {
+        for (int c = tid; c < listed; c += SAMPLE_THREADS) f(cand_key[c], cand_idx[c]);
+    };
+    for (int shift = 16; shift >= 0; shift -= 8) {
+        if (from_list) choose_byte(shift, walk_list);
+        else choose_byte(shift, walk_row);
     }
     const uint32_t kth = sel_prefix;        // key of the k-th largest
     const int need_eq = sel_remaining;      // how many of the equal keys belong to the top k
 
-    // ---- gather: all keys above kth in any order, the first need_eq equal ones by index
-    if (tid == 0) {
-        n_gathered = 0;
-        eq_taken = 0;
+    // ---- gather: the keys above kth in any order (the sort that follows orders them), and of the
+    // equal ones the need_eq with the lowest indices. The equal ones are listed first; only a
+    // list that overflows is walked in index order.
+    auto take = [&](uint32_t k, int i) {
+        if (k > kth) {
+            if (from_list && (k >> 24) > (kth >> 24)) return;      // gathered before
+            const int at = atomicAdd(&n_gathered, 1);
+            keys[at] = k;
+            idx[at] = i;
+        } else if (k == kth) {
+            const int e = atomicAdd(&eq_count, 1);
+            if (e < SAMPLE_MAX_K) eq_idx[e] = i;
+        }
+    };
+    if (from_list) {
+        walk_list(take);
+    } else {
+        __syncthreads();
+        if (tid == 0) n_gathered = 0;                  // (what the first walk gathered is gathered again)
+        __syncthreads();
+        walk_row(take);
     }
     __syncthreads();
-    const int lane = tid & (HB_WAVE - 1), wave = tid / HB_WAVE;
-    for (int base = 0; base < V; base += blockDim.x) {
-        const int i = base + tid;
-        uint32_t k = 0;
-        bool above = false, equal = false;
-        if (i < V) {
-            k = float_key(row[i] / temperature);
-            above = k > kth;
-            equal = k == kth;
-        }
-        if (above) {
-            const int at = atomicAdd(&n_gathered, 1);
-            keys[at] = k;
-            idx[at] = i;
-        }
-        // ordered rank of the equal ones within this stretch of the row
-        const unsigned long long bal = __ballot(equal);
-        const int before_lane = __popcll(bal & ((1ull << lane) - 1ull));
-        if (lane == 0) wave_counts[wave] = __popcll(bal);
-        __syncthreads();
-        int before = eq_taken;
-        for (int w = 0; w < wave; ++w) before += wave_counts[w];
-        const int rank = before + before_lane;
-        if (equal && rank < need_eq) {
-            const int at = atomicAdd(&n_gathered, 1);
-            keys[at] = k;
-            idx[at] = i;
+    const int total_eq = eq_count;
+    if (total_eq <= SAMPLE_MAX_K) {
+        // rank of an equal key = how many of the listed ones have a lower index
+        for (int e = tid; e < total_eq; e += blockDim.x) {
+            const int mine = eq_idx[e];
+            int rank = 0;
+            if (total_eq > need_eq)
+                for (int o = 0; o < total_eq; ++o) rank += eq_idx[o] < mine;
+            if (rank < need_eq) {
+                const int at = atomicAdd(&n_gathered, 1);
+                keys[at] = kth;
+                idx[at] = mine;
+            }
         }
         __syncthreads();
-        if (tid == 0) {
-            int total = 0;
-            for (int w = 0; w < SAMPLE_THREADS / HB_WAVE; ++w) total += wave_counts[w];
-            eq_taken += total;
+    } else {
+        for (int base = 0; base < V; base += blockDim.x) {
+            const int i = base + tid;
+            const bool equal = i < V && float_key(row[i] / temperature) == kth;
+            // ordered rank of the equal ones within this stretch of the row
+            const unsigned long long bal = __ballot(equal);
+            const int before_lane = __popcll(bal & ((1ull << lane) - 1ull));
+            if (lane == 0) wave_counts[wave] = __popcll(bal);
+            __syncthreads();
+            int before = eq_taken;
+            for (int w = 0; w < wave; ++w) before += wave_counts[w];
+            const int rank = before + before_lane;
+            if (equal && rank < need_eq) {
+                const int at = atomicAdd(&n_gathered, 1);
+                keys[at] = kth;
+                idx[at] = i;
+            }
+            __syncthreads();
+            if (tid == 0) {
+                int total = 0;
+                for (int w = 0; w < SAMPLE_THREADS / HB_WAVE; ++w) total += wave_counts[w];
+                eq_taken += total;
+            }
+            __syncthreads();
         }
-        __syncthreads();
     }
     const int n = n_gathered;   // == top_k
     int n_pow2 = 1;
@@ -482,16 +702,27 @@ sample_finish_kernel(const uint32_t* __restrict__ keys, const int* __restrict__ 
 // Sample one token per row. temperature > 0. top_k == 0 means no top-k; top_p >= 1 none.
 // scratch_keys / scratch_idx: [R, P2] each, P2 = the power of two >= V, used by the general
 // path only (top_k == 0, top_k >= V or top_k > 1024).
+// pre_key / pre_idx: [R, ceil(V / 8192), top_k] each, optional: with them a long row (more than two
+// chunks of 8192) is first sifted by a block a chunk.
 extern "C" int hb_sample(const float* logits, int ld, int R, int V, float temperature, int top_k,
                          float top_p, unsigned long long* rng, const int* rng_index, int* out,
-                         uint32_t* scratch_keys, int* scratch_idx, int P2, hipStream_t stream) {
+                         uint32_t* scratch_keys, int* scratch_idx, int P2, uint32_t* pre_key, int* pre_idx,
+                         hipStream_t stream) {
     HB_REQUIRE(R > 0 && V > 0 && ld >= V, "sample: bad sizes (R=%d, V=%d, ld=%d)", R, V, ld);
     HB_REQUIRE(temperature > 0.f, "sample: temperature must be > 0 (0 is argmax)");
     HB_REQUIRE(top_k >= 0, "sample: top_k must be >= 0");
     const bool k_active = top_k > 0 && top_k < V;
     if (k_active && top_k <= SAMPLE_MAX_K) {
-        sample_topk_kernel<<<R, SAMPLE_THREADS, 0, stream>>>(logits, ld, V, temperature, top_k, top_p,
-                                                           rng, rng_index, out);
+        const int chunks = (V + SAMPLE_CHUNK - 1) / SAMPLE_CHUNK;
+        const bool sift = pre_key && pre_idx && chunks > 2 && R <= 65535;
+        if (sift) {
+            sample_chunk_topk_kernel<<<dim3(chunks, R), SAMPLE_THREADS, 0, stream>>>(logits, ld, V, temperature,
+                                                                                    top_k, pre_key, pre_idx);
+            HB_CHECK_LAUNCH("sample_chunk_topk");
+        }
+        sample_topk_kernel<<<R, SAMPLE_THREADS, 0, stream>>>(logits, ld, V, temperature, top_k, top_p, rng,
+                                                           rng_index, out, sift ? pre_key : nullptr,
+                                                           sift ? pre_idx : nullptr);
         HB_CHECK_LAUNCH("sample_topk");
         return 0;
     }

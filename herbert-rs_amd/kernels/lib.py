@@ -35,7 +35,7 @@ SIGNATURES = {
     },
     "sampling": {
         "hb_argmax": [_P, _I, _I, _I, _P, _P, _P, _I, _P],
-        "hb_sample": [_P, _I, _I, _I, _F, _I, _F, _P, _P, _P, _P, _P, _I, _P],
+        "hb_sample": [_P, _I, _I, _I, _F, _I, _F, _P, _P, _P, _P, _P, _I, _P, _P, _P],
     },
 }
 

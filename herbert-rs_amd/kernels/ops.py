@@ -189,11 +189,16 @@ def argmax(logits, out):
              chunks, _stream())
 
 
-def sample(logits, temperature, top_k, top_p, rng_states, rng_index, out, scratch=None):
+SAMPLE_CHUNK = 8192
+
+
+def sample(logits, temperature, top_k, top_p, rng_states, rng_index, out, scratch=None, sifted=None):
     """One token per row by temperature / top-k / top-p; rng_states int64 [n], advanced in place.
 
     `scratch` = (keys int32 [R, P2], idx int32 [R, P2]) with P2 the power of two >= V; needed
     unless 0 < top_k <= 1024 and top_k < V.
+    `sifted` = (keys int32, idx int32), each of at least R * ceil(V / 8192) * top_k elements, optional:
+    with them a long row is first sifted by a block for every 8192 logits (same result, sooner).
     """
     _check(logits, "logits", torch.float32, (None, None))
     R, V = logits.shape
@@ -212,6 +217,14 @@ def sample(logits, temperature, top_k, top_p, rng_states, rng_index, out, scratc
         _check(idx, "scratch idx", torch.int32, tuple(keys.shape))
         if keys.shape[0] < R:
             raise BackendError("sample: scratch has fewer rows than the logits")
+    pre_key = pre_idx = None
+    if sifted is not None:
+        pre_key, pre_idx = sifted
+        need = R * (-(-V // SAMPLE_CHUNK)) * max(int(top_k), 1)
+        _check(pre_key, "sifted keys", torch.int32, (None,))
+        _check(pre_idx, "sifted idx", torch.int32, (None,))
+        if pre_key.numel() < need or pre_idx.numel() < need:
+            raise BackendError(f"sample: the buffers for sifted candidates hold fewer than {need} elements")
     lib.call("sampling", "hb_sample", logits.data_ptr(), V, R, V, float(temperature), int(top_k),
              float(top_p), rng_states.data_ptr(), _ptr(rng_index), out.data_ptr(), _ptr(keys),
-             _ptr(idx), p2, _stream())
+             _ptr(idx), p2, _ptr(pre_key), _ptr(pre_idx), _stream())

@@ -28,6 +28,18 @@ class Sampler:
         states = [_signed64(xorshift.sequence_seed(seed, i)) for i in range(num_sequences)]
         self.states = torch.tensor(states, dtype=torch.int64, device=device)
         self._scratch = None
+        self._sifted = None
+
+    def _sifted_for(self, rows):
+        """Buffers for the candidates that a block a chunk sifts out of a long row (top-k up to 1024)."""
+        p = self.params
+        if not (0 < p.top_k < self.vocab_size and p.top_k <= 1024) or self.vocab_size <= 2 * ops.SAMPLE_CHUNK:
+            return None
+        need = rows * (-(-self.vocab_size // ops.SAMPLE_CHUNK)) * p.top_k
+        if self._sifted is None or self._sifted[0].numel() < need:
+            self._sifted = (torch.empty(need, dtype=torch.int32, device=self.device),
+                            torch.empty(need, dtype=torch.int32, device=self.device))
+        return self._sifted
 
     def _scratch_for(self, rows):
         p = self.params
@@ -50,5 +62,5 @@ class Sampler:
         else:
             index = torch.tensor(list(sequence_indices), dtype=torch.int32, device=self.device)
             ops.sample(logits, self.params.temperature, self.params.top_k, self.params.top_p,
-                       self.states, index, out, self._scratch_for(rows))
+                       self.states, index, out, self._scratch_for(rows), self._sifted_for(rows))
         return out.tolist()

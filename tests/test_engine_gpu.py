@@ -367,6 +367,48 @@ def test_sampler_matches_the_plain_sampler(top_k, top_p):
     assert [int(s) & ((1 << 64) - 1) for s in states.tolist()] == [r.state for r in rngs]
 
 
+@pytest.mark.parametrize("sift", [False, True])
+@pytest.mark.parametrize("V,levels,top_k", [(3000, 3, 40), (5000, 2, 1000), (151936, 40, 64), (2000, 1, 7),
+                                            (17000, 5, 1000), (20000, 1000, 300), (151936, 100000, 1024)])
+def test_sampler_with_many_equal_logits(V, levels, top_k, sift):
+    """Logits that take few values: the k-th largest is then one of hundreds or thousands of equal
+    ones (more than the kernel lists at once when V / levels exceeds 1024), and those with the
+    lowest indices belong to the candidates. Same tokens as the host formulation, also when a
+    block for every 8192 logits sifts the row first (17000: the last chunk is shorter than top_k)."""
+    from herbert_rs_amd.kernels import ops
+    from herbert_rs_amd.sampling import xorshift
+    R, temperature, top_p = 3, 0.9, 1.0
+    g = torch.Generator().manual_seed(V + top_k)
+    logits = torch.randint(0, levels, (R, V), generator=g).float() * 0.5
+    dev_logits = logits.cuda()
+    seeds = [xorshift.sequence_seed(11, i) for i in range(R)]
+    states = torch.tensor([s - (1 << 64) if s >= (1 << 63) else s for s in seeds], dtype=torch.int64, device="cuda")
+    index = torch.arange(R, dtype=torch.int32, device="cuda")
+    rngs = [plain_sampler.XorShift64(s) for s in seeds]
+    out = torch.empty(R, dtype=torch.int32, device="cuda")
+    works = [plain_sampler.candidates(logits[r].numpy(), temperature, top_k, top_p) for r in range(R)]
+    for r in range(R):                 # the candidates are the top_k first indices of the highest level(s)
+        assert len(works[r]) == top_k
+    sifted = None
+    if sift:
+        need = R * -(-V // ops.SAMPLE_CHUNK) * top_k
+        sifted = (torch.full((need,), -1, dtype=torch.int32, device="cuda"),
+                  torch.full((need,), -1, dtype=torch.int32, device="cuda"))
+    for draw in range(10):
+        ops.sample(dev_logits, temperature, top_k, top_p, states, index, out, None, sifted)
+        got = out.tolist()
+        for r in range(R):
+            u = rngs[r].next_f32()
+            want = plain_sampler.pick(works[r], u)
+            if got[r] != want:
+                cum, near = np.float32(0), False
+                for _, p in works[r]:
+                    cum = np.float32(cum + p)
+                    if abs(float(cum) - float(u)) < 1e-5:
+                        near = True
+                assert near and got[r] in [i for i, _ in works[r]], (draw, r, got[r], want)
+
+
 def test_sampling_through_generate_is_reproducible(model_root):
     folder = make_folder(model_root, "B", "float32")
     prompts = [random_tokens(384, n, 70 + n) for n in (1, 17, 33, 9)]
