@@ -571,18 +571,83 @@ __global__ void sample_bitonic_stage_kernel(uint32_t* __restrict__ keys, int* __
     }
 }
 
-// finish: one block per row over its first n candidates (sorted when sorted != 0, else
-// in index order). Values pass through LDS in stretches; thread 0 adds them in order.
+// finish: one block per row over its first n candidates (sorted when sorted != 0, else in index
+// order). The sums that decide a cut or a draw run over the candidates in their order, a stretch
+// of FINISH_CHUNK at a time: a thread adds up four neighbours, the threads' sums are scanned in
+// a fixed order (within a wave, then over the waves), and the thread in whose four the sum first
+// passes the mark walks them one by one. The order of additions is fixed; it is not the order of
+// a single running sum, whose rounding may put a draw that falls within an ulp of a boundary on
+// the other side of it.
 #define FINISH_CHUNK 4096
+// Adds value(i) for i in [0, n) in order. MARK 0: no mark; 1: stops at the first i whose running
+// sum is >= mark; 2: at the first whose running sum is > mark. Returns the sum over all (MARK 0)
+// or up to and including the marked one; *marked = its i, or -1.
+template <int MARK, class Value>
+__device__ float ordered_sum(int n, float mark, int* marked, float* buf, float* wave_totals, int* s_found,
+                             float* s_total, Value&& value) {
+    const int tid = threadIdx.x, lane = tid & (HB_WAVE - 1), wave = tid / HB_WAVE;
+    const int waves = blockDim.x / HB_WAVE;
+    float carry = 0.f;
+    __syncthreads();                       // nobody is still reading what an earlier call found
+    if (tid == 0) *s_found = -1;
+    for (int c = 0; c < n; c += FINISH_CHUNK) {
+        const int m = n - c < FINISH_CHUNK ? n - c : FINISH_CHUNK;
+        __syncthreads();
+        for (int i = tid; i < m; i += blockDim.x) buf[i] = value(c + i);
+        __syncthreads();
+        float part = 0.f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            if (4 * tid + e < m) part += buf[4 * tid + e];
+        float incl = part;                                   // over the threads of this wave up to this one
+        for (int d = 1; d < HB_WAVE; d <<= 1) {
+            const float other = __shfl_up(incl, d, HB_WAVE);
+            if (lane >= d) incl += other;
+        }
+        float excl = __shfl_up(incl, 1, HB_WAVE);            // the lane before: its sum is where this one starts
+        if (lane == 0) excl = 0.f;
+        if (lane == HB_WAVE - 1) wave_totals[wave] = incl;
+        __syncthreads();
+        float before = carry;                                // everything before this wave
+        for (int w = 0; w < wave; ++w) before += wave_totals[w];
+        float chunk_total = 0.f;
+        for (int w = 0; w < waves; ++w) chunk_total += wave_totals[w];
+        if (MARK) {
+            const float upto = before + incl, until = before + excl;    // with and without this thread's four
+            const bool passes = MARK == 1 ? upto >= mark : upto > mark;
+            const bool passed = MARK == 1 ? until >= mark : until > mark;
+            if (passes && !passed && 4 * tid < m) {
+                // the first thread whose sum passes the mark: the scan is monotonic, so there is one
+                float cum = until;
+                int at = 4 * tid;
+                for (int e = 0; e < 4 && 4 * tid + e < m; ++e) {
+                    cum += buf[4 * tid + e];
+                    at = 4 * tid + e;
+                    if (MARK == 1 ? cum >= mark : cum > mark) break;
+                }
+                *s_found = c + at;
+                *s_total = cum;
+            }
+            __syncthreads();
+            if (*s_found >= 0) {
+                *marked = *s_found;
+                return *s_total;
+            }
+        }
+        carry += chunk_total;
+    }
+    if (MARK) *marked = -1;
+    return carry;
+}
+
 __global__ void __launch_bounds__(1024)
 sample_finish_kernel(const uint32_t* __restrict__ keys, const int* __restrict__ idx, int P2, int n,
                      int sorted, float top_p, unsigned long long* __restrict__ rng,
                      const int* __restrict__ rng_index, int* __restrict__ out) {
     __shared__ float buf[FINISH_CHUNK];
     __shared__ float red[16];
-    __shared__ float s_max, s_inv, s_inv2, s_r;
-    __shared__ int s_kept, s_chosen, s_done;
-    __shared__ float s_cum;
+    __shared__ float s_max, s_r, s_total;
+    __shared__ int s_found;
     const uint32_t* k = keys + (size_t)blockIdx.x * P2;
     const int* x = idx + (size_t)blockIdx.x * P2;
     const int tid = threadIdx.x;
@@ -601,102 +666,33 @@ sample_finish_kernel(const uint32_t* __restrict__ keys, const int* __restrict__ 
             s_max = mv;
         }
     }
-    __syncthreads();
-    const float max_val = s_max;
-
-    // pass 1: the softmax denominator
-    float sum = 0.f;
-    for (int c = 0; c < n; c += FINISH_CHUNK) {
-        const int m = n - c < FINISH_CHUNK ? n - c : FINISH_CHUNK;
-        __syncthreads();
-        for (int i = tid; i < m; i += blockDim.x) buf[i] = expf(key_float(k[c + i]) - max_val);
-        __syncthreads();
-        if (tid == 0)
-            for (int i = 0; i < m; ++i) sum += buf[i];
-    }
-    if (tid == 0) {
-        s_inv = 1.0f / sum;
-        s_kept = n;
-        s_inv2 = 1.0f;
-    }
-    __syncthreads();
-    const float inv = s_inv;
-
-    // pass 2: the top-p cut (candidates are sorted then) and the sum of the kept ones
-    if (top_p < 1.0f) {
-        if (tid == 0) {
-            s_cum = 0.f;
-            s_done = 0;
-        }
-        float cum = 0.f;
-        for (int c = 0; c < n; c += FINISH_CHUNK) {
-            __syncthreads();
-            if (s_done) break;
-            const int m = n - c < FINISH_CHUNK ? n - c : FINISH_CHUNK;
-            for (int i = tid; i < m; i += blockDim.x) buf[i] = expf(key_float(k[c + i]) - max_val) * inv;
-            __syncthreads();
-            if (tid == 0) {
-                for (int i = 0; i < m; ++i) {
-                    cum += buf[i];
-                    if (cum >= top_p) {
-                        s_kept = c + i + 1;
-                        s_done = 1;
-                        break;
-                    }
-                }
-            }
-        }
-        __syncthreads();
-        const int kept = s_kept;
-        float sum2 = 0.f;
-        for (int c = 0; c < kept; c += FINISH_CHUNK) {
-            const int m = kept - c < FINISH_CHUNK ? kept - c : FINISH_CHUNK;
-            __syncthreads();
-            for (int i = tid; i < m; i += blockDim.x) buf[i] = expf(key_float(k[c + i]) - max_val) * inv;
-            __syncthreads();
-            if (tid == 0)
-                for (int i = 0; i < m; ++i) sum2 += buf[i];
-        }
-        if (tid == 0) s_inv2 = 1.0f / sum2;
-        __syncthreads();
-    }
-
-    // pass 3: the draw
     if (tid == 0) {
         unsigned long long* st = rng + (rng_index ? rng_index[blockIdx.x] : blockIdx.x);
         s_r = xorshift_next_f32(st);
-        s_done = 0;
-        s_chosen = x[s_kept - 1];
     }
     __syncthreads();
-    const int kept = s_kept;
-    const float inv2 = s_inv2;
-    const float r = s_r;
+    const float max_val = s_max, r = s_r;
+    int marked;
+
+    // the softmax denominator
+    const float inv = 1.0f / ordered_sum<0>(n, 0.f, &marked, buf, red, &s_found, &s_total,
+                                            [&](int i) { return expf(key_float(k[i]) - max_val); });
+    // the top-p cut (candidates are sorted then) and the sum of the kept ones
+    int kept = n;
+    float inv2 = 1.0f;
+    if (top_p < 1.0f) {
+        const float sum2 = ordered_sum<1>(n, top_p, &marked, buf, red, &s_found, &s_total,
+                                          [&](int i) { return expf(key_float(k[i]) - max_val) * inv; });
+        if (marked >= 0) kept = marked + 1;
+        inv2 = 1.0f / sum2;
+    }
+    // the draw: the first candidate whose running probability exceeds r, else the last one kept
     const bool renorm = top_p < 1.0f;
-    float cum = 0.f;
-    for (int c = 0; c < kept; c += FINISH_CHUNK) {
-        __syncthreads();
-        if (s_done) break;
-        const int m = kept - c < FINISH_CHUNK ? kept - c : FINISH_CHUNK;
-        for (int i = tid; i < m; i += blockDim.x) {
-            float p = expf(key_float(k[c + i]) - max_val) * inv;
-            if (renorm) p *= inv2;
-            buf[i] = p;
-        }
-        __syncthreads();
-        if (tid == 0) {
-            for (int i = 0; i < m; ++i) {
-                cum += buf[i];
-                if (r < cum) {
-                    s_chosen = x[c + i];
-                    s_done = 1;
-                    break;
-                }
-            }
-        }
-    }
-    __syncthreads();
-    if (tid == 0) out[blockIdx.x] = s_chosen;
+    ordered_sum<2>(kept, r, &marked, buf, red, &s_found, &s_total, [&](int i) {
+        const float p = expf(key_float(k[i]) - max_val) * inv;
+        return renorm ? p * inv2 : p;
+    });
+    if (tid == 0) out[blockIdx.x] = x[marked >= 0 ? marked : kept - 1];
 }
 
 // Sample one token per row. temperature > 0. top_k == 0 means no top-k; top_p >= 1 none.
