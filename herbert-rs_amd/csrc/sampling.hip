@@ -571,6 +571,49 @@ __global__ void sample_bitonic_stage_kernel(uint32_t* __restrict__ keys, int* __
     }
 }
 
+// The stages of a bitonic sort whose stride is below SORT_BLOCK / 2, on one stretch of SORT_BLOCK
+// elements in LDS: every step from first_size up to last_size, and within the first one only the
+// strides from first_stride down (the larger ones were done in global memory). With first_size = 2
+// and last_size = SORT_BLOCK this sorts the stretch from scratch.
+#define SORT_BLOCK 4096
+__global__ void __launch_bounds__(1024)
+sample_bitonic_local_kernel(uint32_t* __restrict__ keys, int* __restrict__ idx, int P2, int first_size,
+                            int last_size, int first_stride) {
+    __shared__ uint32_t lk[SORT_BLOCK];
+    __shared__ int lx[SORT_BLOCK];
+    const int block = P2 < SORT_BLOCK ? P2 : SORT_BLOCK;
+    const size_t base = (size_t)blockIdx.y * P2 + (size_t)blockIdx.x * block;
+    for (int i = threadIdx.x; i < block; i += blockDim.x) {
+        lk[i] = keys[base + i];
+        lx[i] = idx[base + i];
+    }
+    const int offset = blockIdx.x * block;          // position of this stretch in its row: decides the direction
+    for (int size = first_size; size <= last_size; size <<= 1) {
+        for (int stride = size == first_size ? first_stride : size >> 1; stride > 0; stride >>= 1) {
+            __syncthreads();
+            for (int i = threadIdx.x; i < block / 2; i += blockDim.x) {
+                const int lo = 2 * i - (i & (stride - 1));
+                const int hi = lo + stride;
+                const bool up = ((offset + lo) & size) == 0;
+                const bool hi_first = cand_before(lk[hi], lx[hi], lk[lo], lx[lo]);
+                if (hi_first == up) {
+                    const uint32_t tk = lk[lo];
+                    lk[lo] = lk[hi];
+                    lk[hi] = tk;
+                    const int ti = lx[lo];
+                    lx[lo] = lx[hi];
+                    lx[hi] = ti;
+                }
+            }
+        }
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < block; i += blockDim.x) {
+        keys[base + i] = lk[i];
+        idx[base + i] = lx[i];
+    }
+}
+
 // finish: one block per row over its first n candidates (sorted when sorted != 0, else in index
 // order). The sums that decide a cut or a draw run over the candidates in their order, a stretch
 // of FINISH_CHUNK at a time: a thread adds up four neighbours, the threads' sums are scanned in
@@ -731,11 +774,18 @@ extern "C" int hb_sample(const float* logits, int ld, int R, int V, float temper
     HB_CHECK_LAUNCH("sample_prepare");
     const int sorted = (k_active || top_p < 1.0f) ? 1 : 0;
     if (sorted) {
-        dim3 sgrid((P2 / 2 + 255) / 256, R);
-        for (int size = 2; size <= P2; size <<= 1)
-            for (int stride = size >> 1; stride > 0; stride >>= 1)
+        // stretches of SORT_BLOCK are sorted in LDS; a larger step does its wide strides in global
+        // memory, one kernel each, and the rest again in LDS
+        const int block = P2 < SORT_BLOCK ? P2 : SORT_BLOCK;
+        dim3 lgrid(P2 / block, R), sgrid((P2 / 2 + 255) / 256, R);
+        sample_bitonic_local_kernel<<<lgrid, 1024, 0, stream>>>(scratch_keys, scratch_idx, P2, 2, block, 1);
+        for (int size = 2 * block; size <= P2; size <<= 1) {
+            for (int stride = size >> 1; stride >= block; stride >>= 1)
                 sample_bitonic_stage_kernel<<<sgrid, 256, 0, stream>>>(scratch_keys, scratch_idx, P2, size,
                                                                        stride);
+            sample_bitonic_local_kernel<<<lgrid, 1024, 0, stream>>>(scratch_keys, scratch_idx, P2, size, size,
+                                                                    block / 2);
+        }
         HB_CHECK_LAUNCH("sample_sort");
     }
     const int n = k_active ? top_k : V;
