@@ -313,7 +313,8 @@ def _decode_split(meta, nkv, window):
     want = max(1, -(-DECODE_WAVES // (meta.num_seqs * nkv)))
     if 2 * meta.num_seqs * nkv >= DECODE_WAVES:      # two waves a CU already: a merge would cost more than it gains
         want = 1
-    splits = max(1, min(span, want, 32))      # the merge's cost grows with the ranges
+    # the merge's cost grows with the ranges: more than 32 only where each still has four pages
+    splits = max(1, min(span, want, max(32, min(128, span // 4))))
     per = -(-span // splits)
     return -(-span // per), per
 
