@@ -126,6 +126,68 @@ def test_long_prompts_with_heads_of_128(dtype, model_root, monkeypatch):
     assert (len(fused) > 0) == (dtype == "bfloat16")
 
 
+ODD_SIZES = {
+    # a vocabulary and a width that no kernel's block divides, seven heads on one kv head
+    "odd_vocab": dict(vocab_size=323, hidden_size=72, intermediate_size=100, num_attention_heads=7,
+                      num_key_value_heads=1, head_dim=16, eos_token_id=1),
+    # widths in steps of 32 (the matrix-core products) with a vocabulary that is not one of 16
+    "mfma_odd_vocab": dict(vocab_size=1001, hidden_size=160, intermediate_size=352, num_attention_heads=6,
+                           num_key_value_heads=3, head_dim=64, eos_token_id=1),
+    # head sizes in steps of 16 that the matrix-core attention does not take
+    "head_80": dict(vocab_size=400, hidden_size=128, intermediate_size=192, num_attention_heads=4,
+                    num_key_value_heads=2, head_dim=80, eos_token_id=1),
+    "head_112": dict(vocab_size=272, hidden_size=96, intermediate_size=160, num_attention_heads=3,
+                     num_key_value_heads=3, head_dim=112, eos_token_id=1),
+    # the largest head the attention kernels take
+    "head_512": dict(vocab_size=256, hidden_size=64, intermediate_size=96, num_attention_heads=2,
+                     num_key_value_heads=1, head_dim=512, eos_token_id=1),
+    # forty query heads to one kv head: more than the matrix-core attention shares a key among
+    "group_40": dict(vocab_size=256, hidden_size=64, intermediate_size=96, num_attention_heads=40,
+                     num_key_value_heads=1, head_dim=32, eos_token_id=1),
+}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", sorted(ODD_SIZES))
+def test_sizes_that_fit_no_kernels_blocks(name, dtype, model_root):
+    """Sizes that the configuration allows and that the fast kernels' blocks do not divide: the
+    engine takes another kernel for them (never a wrong result): a prompt whole, a batch of
+    unequal prompts, and tokens decoded on, against the plain logits."""
+    folder = make_folder(model_root, "A", dtype, overrides=ODD_SIZES[name])
+    vocab = ODD_SIZES[name]["vocab_size"]
+    a, b = random_tokens(vocab, 100, 40), random_tokens(vocab, 13, 41)
+    ref_a, ref_b = plain_logits(folder, a), plain_logits(folder, b)
+    engine = hb.load(folder, dtype=dtype, cache_tokens=64 * 6)
+    s1, s2 = engine.alloc_slot(), engine.alloc_slot()
+    got = engine.step([StepEntry(s1, a[:90], [0, 63, 64, 89]), StepEntry(s2, b[:9], [0, 8])]).cpu().numpy()
+    for row, (ref, p) in enumerate(((ref_a, 0), (ref_a, 63), (ref_a, 64), (ref_a, 89), (ref_b, 0), (ref_b, 8))):
+        ok, err = close(got[row], ref[p], dtype)
+        assert ok, f"prompt row {row} position {p}: err {err}"
+    for k in range(10):
+        entries = [StepEntry(s1, [a[90 + k]], [0])] + ([StepEntry(s2, [b[9 + k]], [0])] if k < 4 else [])
+        got = engine.step(entries).cpu().numpy()
+        ok, err = close(got[0], ref_a[90 + k], dtype)
+        assert ok, f"decoded {90 + k}: err {err}"
+        if k < 4:
+            ok, err = close(got[1], ref_b[9 + k], dtype)
+            assert ok, f"decoded {9 + k} of the short one: err {err}"
+    engine.free_slot(s1)
+    engine.free_slot(s2)
+    engine.cache.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_head_too_large_is_refused(dtype, model_root):
+    """Heads of more than 512 are beyond every attention kernel: a clear error, no result."""
+    from herbert_rs_amd.errors import BackendError
+    folder = make_folder(model_root, "A", dtype, overrides=dict(head_dim=528, num_attention_heads=2,
+                                                                num_key_value_heads=1))
+    with pytest.raises(BackendError, match="head"):
+        engine = hb.load(folder, dtype=dtype, cache_tokens=128)
+        slot = engine.alloc_slot()
+        engine.step([StepEntry(slot, [1, 2, 3], [2])])
+
+
 def test_a_batch_of_more_than_64_decodes_like_each_sequence_alone(model_root):
     """With more than 64 sequences a decode step is no longer a skinny product: the tiled kernels
     (and, in bfloat16, HIP graphs of them) take over. Every sequence must still get the logits
