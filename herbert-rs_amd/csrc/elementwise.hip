@@ -199,10 +199,10 @@ __global__ void qk_norm_rope_write_kernel(
 }
 
 // The same for many tokens (prompts), bfloat16 output, rotation over the whole head or none,
-// head size up to 128: a workgroup takes 64 consecutive tokens of one head. Query and key heads:
-// a wave per token, lane = the pair (j, j + hd/2), rows read and written whole. Value heads go
-// through LDS, so that the transposed pages are written along the tokens: lane = token, 64
-// consecutive tokens of a page are one 128-byte line.
+// head size in steps of 8 up to 128, rows of the projection 16-byte aligned: a workgroup takes 64
+// consecutive tokens of one head. Query and key heads: half a wave a token, 16 bytes a lane.
+// Value heads go through LDS, so that the transposed pages are written along the tokens: lane =
+// token, 64 consecutive tokens of a page are one 128-byte line.
 // QS > 1: the projection was cut into QS slices of K whose sums lie slice_stride floats apart
 // behind qkv; they are added up in their order as they are loaded.
 #define HB_TILED_HEAD_DIM 128
@@ -218,21 +218,25 @@ __global__ void __launch_bounds__(256) qk_norm_rope_write_tiled_kernel(
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const bool is_q = h < nq, is_v = h >= nq + nkv;
     const int half = hd / 2;
-    auto summed = [&](const float* p) {
-        float part[QS];
+    auto summed4 = [&](const float* p) {
+        hb_f4 part[QS];
 #pragma unroll
-        for (int i = 0; i < QS; ++i) part[i] = p[(size_t)i * slice_stride];
-        float sum = part[0];
+        for (int i = 0; i < QS; ++i) part[i] = *(const hb_f4*)(p + (size_t)i * slice_stride);
+        hb_f4 sum = part[0];
 #pragma unroll
         for (int i = 1; i < QS; ++i) sum += part[i];
         return sum;
     };
     if (is_v) {
         const int kvh = h - nq - nkv;
-        for (int idx = tid; idx < 64 * hd; idx += 256) {
-            const int r = idx / hd, c = idx - r * hd;
+        const int q4 = hd / 4;                       // 16-byte chunks of a row
+        for (int idx = tid; idx < 64 * q4; idx += 256) {
+            const int r = idx / q4, c = (idx - r * q4) * 4;
             const int t = t0 + r;
-            vt[r][c] = t < T ? summed(qkv + (size_t)t * ld_qkv + (size_t)h * hd + c) : 0.f;
+            hb_f4 v = {0.f, 0.f, 0.f, 0.f};
+            if (t < T) v = summed4(qkv + (size_t)t * ld_qkv + (size_t)h * hd + c);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) vt[r][c + e] = v[e];
         }
         __syncthreads();
         const int t = t0 + lane;
@@ -243,56 +247,71 @@ __global__ void __launch_bounds__(256) qk_norm_rope_write_tiled_kernel(
         for (int d = wave; d < hd; d += 4) dst[(size_t)d * page_size] = hb_from_float<TC>(vt[lane][d]);
         return;
     }
+    // Query and key heads: half a wave a token, a lane four consecutive elements (16 bytes in, 8
+    // out); the lanes l < hd / 8 hold the first half of the head, their partners l + hd / 8 the
+    // elements they are rotated with. A wave's 16 tokens go in two rounds of 8 (4 passes of 2
+    // tokens): all loads of a round go out before anything waits for them.
     const float* norm_w = is_q ? q_norm_w : k_norm_w;
-    const bool mine = lane < half;
-    const int j = mine ? lane : 0;
-    const float w0 = norm_w ? norm_w[j] : 1.f, w1 = norm_w ? norm_w[j + half] : 1.f;
-    // a wave's 16 tokens in two rounds of 8: all loads of a round go out before anything waits for them
+    const int l = lane & 31, sub = lane >> 5;
+    const int eighth = hd / 8;
+    const bool mine = l < 2 * eighth;
+    const bool first = l < eighth;
+    const int d0 = mine ? 4 * l : 0;
+    const int j0 = mine && !first ? d0 - half : d0;              // where this lane's angles lie
+    const int partner = (lane & 32) + (mine ? (first ? l + eighth : l - eighth) : l);
+    hb_f4 w = {1.f, 1.f, 1.f, 1.f};
+    if (norm_w && mine) w = *(const hb_f4*)(norm_w + d0);
 #pragma unroll
     for (int round = 0; round < 2; ++round) {
-        float x0[8], x1[8], c[8], sn[8];
-        int pos[8];
+        hb_f4 x[4], c[4], sn[4];
+        int pos[4];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            const int t = t0 + wave + 4 * (round * 8 + u);
+        for (int u = 0; u < 4; ++u) {
+            const int t = t0 + 16 * wave + 8 * round + 2 * u + sub;
             const int tc = t < T ? t : T - 1;
-            const float* src = qkv + (size_t)tc * ld_qkv + (size_t)h * hd;
             pos[u] = positions[tc];
-            x0[u] = mine ? summed(src + j) : 0.f;
-            x1[u] = mine ? summed(src + j + half) : 0.f;
+            x[u] = hb_f4{0.f, 0.f, 0.f, 0.f};
+            if (mine) x[u] = summed4(qkv + (size_t)tc * ld_qkv + (size_t)h * hd + d0);
         }
         if (cos_t) {
 #pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                c[u] = cos_t[(size_t)pos[u] * half + j];
-                sn[u] = sin_t[(size_t)pos[u] * half + j];
+            for (int u = 0; u < 4; ++u) {
+                c[u] = *(const hb_f4*)(cos_t + (size_t)pos[u] * half + j0);
+                sn[u] = *(const hb_f4*)(sin_t + (size_t)pos[u] * half + j0);
             }
         }
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            const int t = t0 + wave + 4 * (round * 8 + u);
-            float a0 = x0[u], a1 = x1[u];
+        for (int u = 0; u < 4; ++u) {
+            const int t = t0 + 16 * wave + 8 * round + 2 * u + sub;
+            hb_f4 a = x[u];
             if (norm_w) {
-                const float ss = hb_wave_sum(a0 * a0 + a1 * a1);
+                float ss = a[0] * a[0] + a[1] * a[1] + a[2] * a[2] + a[3] * a[3];
+#pragma unroll
+                for (int d = 1; d < 32; d <<= 1) ss += __shfl_xor(ss, d, 64);
                 const float inv = 1.0f / sqrtf(ss / (float)hd + eps);
-                a0 = a0 * inv * w0;
-                a1 = a1 * inv * w1;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) a[e] = a[e] * inv * w[e];
             }
             if (cos_t) {
-                const float r0 = a0 * c[u] - a1 * sn[u], r1 = a0 * sn[u] + a1 * c[u];
-                a0 = r0;
-                a1 = r1;
+                hb_f4 o;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float other = __shfl(a[e], partner, 64);
+                    // first half: x0 c - x1 s; second half: x0 s + x1 c (x0 the partner's element)
+                    o[e] = first ? a[e] * c[u][e] - other * sn[u][e] : other * sn[u][e] + a[e] * c[u][e];
+                }
+                a = o;
             }
             if (!mine || t >= T) continue;
+            TQ packed[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) packed[e] = hb_from_float<TQ>(a[e]);
             if (is_q) {
-                TQ* dst = q_out + ((size_t)t * nq + h) * hd;
-                dst[j] = hb_from_float<TQ>(a0);
-                dst[j + half] = hb_from_float<TQ>(a1);
+                *(uint2*)(q_out + ((size_t)t * nq + h) * hd + d0) = *(const uint2*)packed;
             } else {
                 const int page = page_table[(size_t)slots[seq_of[t]] * max_pages + pos[u] / page_size];
-                TC* dst = k_cache + (((size_t)page * nkv + (h - nq)) * page_size + pos[u] % page_size) * hd;
-                dst[j] = hb_from_float<TC>(a0);
-                dst[j + half] = hb_from_float<TC>(a1);
+                *(uint2*)(k_cache + (((size_t)page * nkv + (h - nq)) * page_size + pos[u] % page_size) * hd + d0) =
+                    *(const uint2*)packed;
             }
         }
     }
@@ -314,7 +333,8 @@ extern "C" int hb_qk_norm_rope_write(const float* qkv, int ld_qkv, const float* 
     const int heads = nq + (write_kv ? 2 * nkv : 0);
     HB_REQUIRE(ld_qkv >= heads * hd, "qk_norm_rope_write: row stride %d too small", ld_qkv);
     HB_REQUIRE(heads <= 65535, "qk_norm_rope_write: too many heads for the grid");
-    if (dtype == HB_BF16 && write_kv && T >= 64 && hd <= HB_TILED_HEAD_DIM && hd % 2 == 0 &&
+    if (dtype == HB_BF16 && write_kv && T >= 64 && hd <= HB_TILED_HEAD_DIM && hd % 8 == 0 && ld_qkv % 4 == 0 &&
+        slice_stride % 4 == 0 && ((uintptr_t)qkv & 15) == 0 &&
         (cos_t == nullptr || rot_dims == hd) && (T + 63) / 64 <= 0x7fffffff) {
         dim3 tiles((T + 63) / 64, heads);
         HB_REQUIRE(qkv_slices == 1 || slice_stride >= (size_t)T * ld_qkv, "qk_norm_rope_write: slices overlap");

@@ -370,10 +370,12 @@ __global__ void gemm_slices_kernel(const float* __restrict__ partial, float* __r
 // The same for a product that adds to the residual stream and is followed by an RMSNorm: a block a
 // row adds the slices to x, stores x and writes y = bf16(x / rms(x) * g) as well (or, for at most 16
 // rows, what NormHandoff describes: the next product expects that). A thread has at
-// most two chunks of four columns (N in steps of 4, at most 8192, 1024 threads) and asks for its
-// part of up to eight slices at once: with at most 64 rows there are few blocks, and what counts is
-// that each has all its loads in flight together.
-__global__ void __launch_bounds__(1024)
+// most CHUNKS chunks of four columns (N in steps of 4, at most 8192 = 4 THREADS CHUNKS) and asks for
+// its part of up to FLY slices at once: with at most 64 rows there are few blocks, and what counts is
+// that each has all its loads in flight together (1024 threads, eight slices); with many rows
+// there are blocks enough, of 256 threads.
+template <int THREADS, int CHUNKS, int FLY>
+__global__ void __launch_bounds__(THREADS)
 gemm_slices_norm_kernel(const float* __restrict__ partial, float* __restrict__ C, int M, int N, int ldc, int slices,
                         const float* __restrict__ g, float eps, bf16* __restrict__ y, float* __restrict__ squares) {
     __shared__ float red[16];
@@ -381,36 +383,36 @@ gemm_slices_norm_kernel(const float* __restrict__ partial, float* __restrict__ C
     f32x4* row = (f32x4*)(C + (size_t)m * ldc);
     const f32x4* g4 = (const f32x4*)g;
     const int nv = N / 4;
-    f32x4 v[2], gv[2];
+    f32x4 v[CHUNKS], gv[CHUNKS];
 #pragma unroll
-    for (int c = 0; c < 2; ++c) {
-        const int i = threadIdx.x + 1024 * c;
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int i = threadIdx.x + THREADS * c;
         const int at = i < nv ? i : nv - 1;              // past the end: the last chunk again, never stored
         v[c] = row[at];
         gv[c] = g4[at];
     }
-    for (int s0 = 0; s0 < slices; s0 += 8) {
-        f32x4 p[2][8];
+    for (int s0 = 0; s0 < slices; s0 += FLY) {
+        f32x4 p[CHUNKS][FLY];
 #pragma unroll
-        for (int c = 0; c < 2; ++c) {
-            const int i = threadIdx.x + 1024 * c;
+        for (int c = 0; c < CHUNKS; ++c) {
+            const int i = threadIdx.x + THREADS * c;
             const int at = i < nv ? i : nv - 1;
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
+            for (int j = 0; j < FLY; ++j) {
                 const int sl = s0 + j < slices ? s0 + j : slices - 1;
                 p[c][j] = ((const f32x4*)(partial + ((size_t)sl * M + m) * N))[at];
             }
         }
 #pragma unroll
-        for (int c = 0; c < 2; ++c)
+        for (int c = 0; c < CHUNKS; ++c)
 #pragma unroll
-            for (int j = 0; j < 8; ++j)
+            for (int j = 0; j < FLY; ++j)
                 if (s0 + j < slices) v[c] += p[c][j];     // in the order of the slices
     }
     float ss = 0.f;
 #pragma unroll
-    for (int c = 0; c < 2; ++c) {
-        const int i = threadIdx.x + 1024 * c;
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int i = threadIdx.x + THREADS * c;
         if (i < nv) {
             row[i] = v[c];
             ss += v[c][0] * v[c][0] + v[c][1] * v[c][1] + v[c][2] * v[c][2] + v[c][3] * v[c][3];
@@ -422,8 +424,8 @@ gemm_slices_norm_kernel(const float* __restrict__ partial, float* __restrict__ C
         // sums of x^2 by blocks of 16 columns, four threads a block
         const int MP = M <= 1 ? 1 : (M <= 2 ? 2 : (M <= 4 ? 4 : (M <= 8 ? 8 : 16)));
 #pragma unroll
-        for (int c = 0; c < 2; ++c) {
-            const int i = threadIdx.x + 1024 * c;
+        for (int c = 0; c < CHUNKS; ++c) {
+            const int i = threadIdx.x + THREADS * c;
             float sq = i < nv ? v[c][0] * v[c][0] + v[c][1] * v[c][1] + v[c][2] * v[c][2] + v[c][3] * v[c][3] : 0.f;
             sq += __shfl_xor(sq, 1, 64);
             sq += __shfl_xor(sq, 2, 64);
@@ -436,15 +438,15 @@ gemm_slices_norm_kernel(const float* __restrict__ partial, float* __restrict__ C
             }
         }
         if (m == 0)            // rows from M on hold zeros
-            for (int i = threadIdx.x; i < (N + 15) / 16 * (MP - M); i += 1024)
+            for (int i = threadIdx.x; i < (N + 15) / 16 * (MP - M); i += THREADS)
                 squares[(size_t)(i / (MP - M)) * MP + M + i % (MP - M)] = 0.f;
         return;
     }
     ss = hb_block_sum(ss, red);
     const float inv = 1.0f / sqrtf(ss / (float)N + eps);
 #pragma unroll
-    for (int c = 0; c < 2; ++c) {
-        const int i = threadIdx.x + 1024 * c;
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int i = threadIdx.x + THREADS * c;
         if (i < nv) {
             bf16x4 o;
 #pragma unroll
@@ -1352,8 +1354,15 @@ extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N,
     if (rc == 0 && slices > 1) {
         const size_t total = (size_t)M * N;
         if (emit_g)
-            gemm_slices_norm_kernel<<<M, 1024, 0, stream>>>(workspace, (float*)C, M, N, ldc, slices, emit_g, emit_eps,
-                                                           (bf16*)emit_xg, emit_partial);
+            if (M <= 64)
+                gemm_slices_norm_kernel<1024, 2, 8><<<M, 1024, 0, stream>>>(workspace, (float*)C, M, N, ldc, slices, emit_g,
+                                                                             emit_eps, (bf16*)emit_xg, emit_partial);
+            else if (N <= 4096)   // many rows: smaller blocks, several to a CU, that hide each other's waits
+                gemm_slices_norm_kernel<256, 4, 2><<<M, 256, 0, stream>>>(workspace, (float*)C, M, N, ldc, slices, emit_g,
+                                                                           emit_eps, (bf16*)emit_xg, emit_partial);
+            else
+                gemm_slices_norm_kernel<256, 8, 2><<<M, 256, 0, stream>>>(workspace, (float*)C, M, N, ldc, slices, emit_g,
+                                                                           emit_eps, (bf16*)emit_xg, emit_partial);
         else if (epi == EPI_SWIGLU)
             gemm_slices_swiglu_kernel<<<(unsigned)((total / 2 + 255) / 256), 256, 0, stream>>>(workspace, (bf16*)C, M, N,
                                                                                              ldc, slices);

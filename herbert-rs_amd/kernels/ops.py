@@ -99,7 +99,7 @@ ROPE_WRITE_SLICES = (2, 4, 8)
 def rope_write_adds_slices(T, hd, rot_dims, dtype, write_kv, has_rotation):
     """True if qk_norm_rope_write can add up K slices of the projection itself for such a step: the
     kernel for bfloat16 prompts of 64 tokens or more does."""
-    return (dtype == torch.bfloat16 and write_kv and T >= 64 and hd <= 128 and hd % 2 == 0
+    return (dtype == torch.bfloat16 and write_kv and T >= 64 and hd <= 128 and hd % 8 == 0
             and (not has_rotation or rot_dims == hd))
 
 

@@ -245,7 +245,8 @@ def test_attention_mfma_decode(nq, nkv, hd, window, lengths, waves, monkeypatch)
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("nq,nkv,hd,rot,norm", [(4, 2, 128, 128, True), (3, 1, 64, 64, False), (2, 2, 96, 0, True),
-                                                (5, 1, 32, 32, True), (2, 1, 80, 40, True), (1, 1, 256, 256, True)])
+                                                (5, 1, 32, 32, True), (2, 1, 80, 40, True), (1, 1, 256, 256, True),
+                                                (6, 2, 48, 48, True), (2, 1, 112, 112, True), (3, 1, 16, 16, True)])
 def test_qk_norm_rope_write(nq, nkv, hd, rot, norm, dtype):
     """Per-head norm, rotation and the write into the pages, for prompts that cross pages and a
     step that is no multiple of 64 tokens (the tiled kernel), and for a few tokens (the plain one)."""
