@@ -19,6 +19,13 @@
 //          partial (reference, sum, O) per range are merged by a second kernel in the fixed
 //          order of the ranges. The kernel can also norm and rotate q and k and write the new
 //          token's key and value itself.
+// In xigh/herbert-rs the same sums are crates/backends/backend_common/src/generic_attention/prefill/kernel_f32.rs:39-113
+// (prompts: causal by count, online softmax) and crates/backends/backend_common/src/attention_common.rs:20-124
+// (decoding over a bfloat16 cache); the split of a long context into ranges whose partial (max, sum,
+// output) a second kernel merges is crates/backends/backend_metal/shaders/attention_decode_flash.metal:30-198
+// (tiles of 256 positions there), a key row shared by the query heads of its kv head as in
+// crates/backends/backend_common/src/avx512_attn_dot8_bf16.S. The new key's norm, rotation and cache write inside the
+// decode kernel: crates/backends/backend_metal/shaders/head_norm_rope_kv_append.metal:37-110.
 #include "common.h"
 #include <math.h>
 

@@ -5,6 +5,11 @@
 // chunks of 64 that start at multiples of 64 of the absolute position, with an
 // online softmax: the chunking, and so the rounding, depends on the positions only,
 // not on how the tokens were cut into steps or batches.
+// In xigh/herbert-rs: scores q . k / sqrt(hd), query head h on kv head h / (nq / nkv)
+// (crates/backends/backend_common/src/generic_attention/decode.rs:126), causal by count
+// (crates/backends/backend_common/src/generic_attention/prefill/kernel_f32.rs:65-67), online softmax and
+// sum of p v (kernel_f32.rs:83-110; decoding: crates/backends/backend_common/src/attention_common.rs:141-178),
+// all float32. The window is not in the reference, which never reads those keys.
 #include "common.h"
 #include <math.h>
 

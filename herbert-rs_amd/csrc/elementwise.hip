@@ -1,6 +1,17 @@
 // Row-wise kernels of the decoder: embedding gather, RMSNorm, the fused
 // per-head norm + rotation + cache write, and SwiGLU. All arithmetic is float32;
 // the template parameters are the storage types of inputs and outputs.
+// What each computes, in xigh/herbert-rs:
+//   embedding        crates/backends/backend_common/src/generic_model.rs:104-111 (no multiplier; an id >= V is an error);
+//                    crates/backends/backend_vulkan/shaders/embedding.comp:20-27
+//   RMSNorm          crates/backends/backend_common/src/kernels.rs:54-64: x * 1 / sqrt(sum(x^2) / dim + eps) * w, eps inside
+//                    the root, plain weight; crates/backends/backend_vulkan/shaders/rms_norm_batch.comp:25-41
+//   per-head norm    crates/backends/backend_common/src/generic_attention/mod.rs:62-76 (before the rotation, the same eps,
+//                    one weight [hd] for all heads, values untouched); backend_vulkan/shaders/head_rms_norm.comp:24-41
+//   rotation         crates/backends/backend_common/src/kernels.rs:739-759 (pairs (j, j + R/2): x0 c - x1 s, x0 s + x1 c;
+//                    elements from R on unchanged); tables crates/backends/backend_common/src/loader_common.rs:179-202
+//   the three fused  crates/backends/backend_metal/shaders/head_norm_rope_kv_append.metal:37-110 (norm, rotation, append)
+//   SwiGLU           crates/backends/backend_common/src/kernels.rs:676-687: g / (1 + exp(-g)) * u
 #include "common.h"
 
 HB_MODULE_ERROR_SLOT()

@@ -16,6 +16,12 @@
 // (weight rows interleaved in blocks of 16: gate rows, then the up rows of the same outputs),
 // 3 (tiled, an entry point of its own) the q/k/v projection with per-head norm, rotation and
 // cache write.
+// In xigh/herbert-rs: crates/backends/backend_bf16/src/kernels.rs:154-164 is the product; the inputs are rounded to
+// bfloat16 before they are multiplied, as crates/backends/backend_bf16_avx512/src/avx512_bf16_matvec.S:1-12 does
+// (float32 sums); SwiGLU in the epilogue as crates/backends/backend_metal/shaders/fused_gate_up_swiglu.metal:27-83;
+// the residual added in the epilogue as the Metal backend's down projection
+// (crates/backends/backend_metal/src/backend.rs:488-507); the norm that follows a residual sum prepared with it as
+// crates/backends/backend_metal/shaders/rms_norm_residual.metal:31-78 fuses the two.
 #include "common.h"
 #include <mutex>
 #include <unordered_set>

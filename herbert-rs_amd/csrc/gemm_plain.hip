@@ -4,6 +4,8 @@
 // mode for shapes its MFMA kernels refuse. Each output is summed over k ascending by
 // one thread with fused multiply-adds, so its value does not depend on M, on the tile
 // it falls in, or on what else is in the batch.
+// In xigh/herbert-rs: crates/backends/backend_bf16/src/kernels.rs:154-164 (float32 sums over k ascending of
+// x[m, k] * float(w[n, k]), no bias); crates/backends/backend_vulkan/shaders/bf16_matmul.comp:31-60.
 #include "common.h"
 
 HB_MODULE_ERROR_SLOT()

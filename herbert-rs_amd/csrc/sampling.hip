@@ -2,6 +2,11 @@
 // The order of candidates is value descending, index ascending among equals; sums that
 // decide a cut or a draw are added one value after the other in that order by one
 // thread, so that a seed gives the same token as the step-by-step host formulation.
+// In xigh/herbert-rs: crates/core/src/sampler.rs:72-145 (logits / temperature, the top_k largest,
+// softmax with the maximum taken off, the shortest prefix by probability whose sum reaches top_p,
+// a draw r in [0, 1) against the running sum, the last candidate if none), :244-254 (argmax: the
+// first of equals); the random numbers are the host's (xorshift64, :30-34, 50-62). On the GPU there:
+// crates/backends/backend_metal/shaders/argmax.metal:14-149 (two stages, strict >).
 #include "common.h"
 #include <math.h>
 

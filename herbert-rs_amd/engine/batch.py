@@ -1,5 +1,10 @@
 """The tokens of one step, packed over the sequences of the batch, with what kernels need
-to find each token's sequence, position and pages."""
+to find each token's sequence, position and pages.
+
+The reference steps one sequence at a time (crates/backends/backend_common/src/generic_model.rs:131 prompts with a
+start position, :524 one token); a batch of unequal sequences in one step has no counterpart
+there. Its checks are kept: no empty sequence, ids below the vocabulary, positions below
+max_position_embeddings (crates/backends/backend_common/src/generic_model.rs:139-152, 165-171, 531-537)."""
 from dataclasses import dataclass
 from typing import List
 

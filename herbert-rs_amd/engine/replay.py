@@ -9,6 +9,10 @@ one JSON object per line on standard input:
 For a step that wants something, `<out>/<step>.f32` holds the float32 logits
 [wanted, vocab] (little-endian) in the order of the entries and of `want`.
 After each step a line `done <step>` is printed and flushed.
+
+The reference has no replay program; its nearest hooks are token ids given as the prompt
+(crates/cli/src/token_parser.rs:13-26) and logits at every fed position
+(crates/backends/backend_common/src/generic_model.rs:808-826).
 """
 import argparse
 import json

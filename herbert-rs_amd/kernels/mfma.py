@@ -1,5 +1,10 @@
 """Host side of the bfloat16 MFMA kernels (matrix products and attention): which shapes they
-take, operand checks, launches. What they refuse goes to the plain kernels."""
+take, operand checks, launches. What they refuse goes to the plain kernels.
+
+The reference rounds the inputs of its bfloat16 product to bfloat16 and sums in float32 as well
+(crates/backends/backend_bf16_avx512/src/avx512_bf16_matvec.S:1-12); its GPU backend chooses between a
+single-pass and a split decode attention by the context's length
+(crates/backends/backend_metal/src/kernels/attention.rs:73-91), as _decode_split does here."""
 import ctypes
 
 import torch

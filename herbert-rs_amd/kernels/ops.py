@@ -3,6 +3,11 @@
 Each function checks on the host that shapes, dtypes, devices and layouts are
 what the kernel and its grid assume, and only then launches on the current
 HIP stream. There is no fallback of any kind behind them.
+
+The operations are those of the reference's op trait (crates/backends/backend_common/src/linear_ops.rs:68-437:
+matmul, rms_norm, swiglu, rotation) and of its GPU command buffer
+(crates/backends/backend_vulkan/src/backend.rs:182-281: embedding, norms, per-head norms, rotation, cache
+append, attention, residual sums), several of them to a kernel here.
 """
 import torch
 
