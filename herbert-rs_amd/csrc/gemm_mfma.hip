@@ -1164,10 +1164,11 @@ extern "C" int hb_gemm_qkv_mfma(const void* X, const void* W, int M, int K, int 
 // the number of K slices; tile -1: nothing takes this product with what is asked of it. The flags
 // say whether the input is normed on the way (norm_w), a norm is left behind (emit_g) or a handed-on
 // one is finished (scale_partial).
-struct GemmPlan { int tile, slices; };
+struct GemmPlan { int tile, slices; double cost = -1; };      // cost: the estimated time in us where the plan was chosen by one
 static GemmPlan plan_gemm(int M, int N, int K, int ldc, int epi, bool norm_w, bool emit_g, bool scale_partial,
                           int tile_hint, size_t workspace_floats, bool deferred = false) {
     int tile = tile_hint % 1000, slices = tile_hint >= 1000 ? tile_hint / 1000 : 1;
+    double low_cost = -1, mid_cost = -1;
     if (tile_hint == 1) return M <= 16 ? GemmPlan{0, 1} : GemmPlan{-1, 0};      // the few-row kernel, asked for by name
     // no slice of K may be empty, and each has at least four steps to run through its ring
     auto slices_fit = [&](int steps, int sl) {
@@ -1229,7 +1230,8 @@ static GemmPlan plan_gemm(int M, int N, int K, int ldc, int epi, bool norm_w, bo
                 }
             }
         }
-        if (skinny) return GemmPlan{0, 1};
+        if (skinny) return GemmPlan{0, 1, best};
+        low_cost = best;
         if (tile == 0) {
             if (emit_g || scale_partial) return GemmPlan{-1, 0};
             tile = 123;
@@ -1275,11 +1277,12 @@ static GemmPlan plan_gemm(int M, int N, int K, int ldc, int epi, bool norm_w, bo
                 }
             }
         }
+        mid_cost = best;
     }
     // (tile_hint: 0 = choose; otherwise a variant by number, for measurements and tests, + 1000 x
     // the number of K slices; 1 = the few-row kernel)
     if (emit_g && !(slices > 1 && reducer_norms)) return GemmPlan{-1, 0};
-    return GemmPlan{tile, slices};
+    return GemmPlan{tile, slices, mid_cost >= 0 ? mid_cost : low_cost};
 }
 
 // The plan as a number for tests and measurements: tile + 1000 x slices (slices > 1), 0 for the
@@ -1290,6 +1293,14 @@ extern "C" int hb_gemm_mfma_plan(int M, int N, int K, int epi, int normed_input,
     const GemmPlan p = plan_gemm(M, N, K, epi == EPI_SWIGLU ? N / 2 : N, epi, normed_input != 0, emit != 0, scaled != 0, 0,
                                  workspace_floats, deferred != 0);
     return p.tile <= 0 ? p.tile : p.tile + (p.slices > 1 ? 1000 * p.slices : 0);
+}
+
+// The estimated time in us of the plan that hb_gemm_mfma_plan gives, or a negative number where the
+// plan is not chosen by an estimate (the few products that only one kernel takes).
+extern "C" double hb_gemm_mfma_plan_cost(int M, int N, int K, int epi, int normed_input, int emit, int scaled,
+                                         size_t workspace_floats, int deferred) {
+    return plan_gemm(M, N, K, epi == EPI_SWIGLU ? N / 2 : N, epi, normed_input != 0, emit != 0, scaled != 0, 0,
+                     workspace_floats, deferred != 0).cost;
 }
 
 // C (+)= X @ W^T. X [M, K] bf16, W [N, K] bf16. epi 0: C f32 [M, N] stored; 1: added to;

@@ -20,6 +20,7 @@ lib.register_signatures("gemm_mfma", {
     "hb_gemm_mfma": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _F, _I, _P, ctypes.c_size_t, _P, _P, _P, _P, _I, _F,
                      _F, _P, _P],
     "hb_gemm_mfma_plan": [_I, _I, _I, _I, _I, _I, _I, ctypes.c_size_t, _I],
+    "hb_gemm_mfma_plan_cost": [_I, _I, _I, _I, _I, _I, _I, ctypes.c_size_t, _I],
     "hb_gemm_qkv_mfma": [_P, _P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _F, _I, _I, _I, _P],
 })
 
@@ -31,14 +32,14 @@ SLICE_WORKSPACE_FLOATS = 16 << 20     # most that the tiled product may use for 
 
 
 def _slice_workspace(device, M, N, K, tile=0):
-    """(pointer, floats) of the scratch for products whose K may be cut into slices: too few tiles
-    of 128 x 128 to give every CU one. The kernel takes as many slices as fit in it. A buffer that
+    """(pointer, floats) of the scratch for products whose K may be cut into slices: those with few
+    tiles (whether it is cut, and how, is the kernel's estimate). It takes as many slices as fit in it. A buffer that
     was handed out is kept for good: a captured graph may hold its address."""
     device = torch.device(device)
     if device.index is None:
         device = torch.device(device.type, torch.cuda.current_device())
-    tiles = ((M + 127) // 128) * ((N + 127) // 128)
-    slices = min(16, K // 256) if tiles < 256 or tile else 1
+    tiles = ((M + 255) // 256) * ((N + 255) // 256)       # of the largest kind: under two rounds of them on 256 CUs
+    slices = min(16, K // 256) if tiles < 512 or tile else 1
     need = min(slices * M * N, SLICE_WORKSPACE_FLOATS)
     if slices < 2 or need < 2 * M * N:
         return None, 0
@@ -122,6 +123,11 @@ def norm_handoff(M, N, K):
     if K % 64 == 0 and K >= 512 and N % 4 == 0 and N <= NORM_WHOLE_MAX_N:
         if M <= NORM_WHOLE_MAX_M or gemm_plan(M, N, K, EPI_ADD) >= 2000:
             return "whole"
+        # Not cut by itself: cut it for the norm's sake if that is estimated to take less time than the
+        # uncut product and a norm kernel (one read of the float32 rows, one write of bfloat16 ones).
+        alone, cut = gemm_plan_cost(M, N, K, EPI_ADD), gemm_plan_cost(M, N, K, EPI_ADD, leaves_norm=True)
+        if alone > 0 and cut > 0 and cut < alone + 2.3 + M * N * 6 / 5.0e6:
+            return "whole"
     return None
 
 
@@ -165,6 +171,15 @@ def gemm_plan(M, N, K, epi=EPI_STORE, normed_input=False, leaves_norm=False, fin
     _, ws_floats = _slice_workspace(torch.device(device), M, N, K)
     return lib.load("gemm_mfma").hb_gemm_mfma_plan(M, N, K, epi, int(normed_input), int(leaves_norm),
                                                    int(finishes_norm), ws_floats, int(defer_slices))
+
+
+def gemm_plan_cost(M, N, K, epi=EPI_STORE, normed_input=False, leaves_norm=False, finishes_norm=False, device="cuda",
+                   defer_slices=False):
+    """The estimated time in us of the plan gemm_plan gives; negative where no estimate chose it."""
+    _, ws_floats = _slice_workspace(torch.device(device), M, N, K)
+    fn = lib.load("gemm_mfma").hb_gemm_mfma_plan_cost
+    fn.restype = ctypes.c_double
+    return fn(M, N, K, epi, int(normed_input), int(leaves_norm), int(finishes_norm), ws_floats, int(defer_slices))
 
 
 def gemm(a, w, out, accumulate=False, packed=False, norm=None, tile=0, leave=None, row_scale=None,
