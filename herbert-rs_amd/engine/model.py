@@ -7,6 +7,7 @@ run the schedule's entries in order on the packed rows, then the final norm
 and the head on the wanted rows only.
 """
 from ..errors import ConfigError
+from ..kernels import ops
 from ..parts import StepContext, build
 from ..parts.spec import ScheduleEntry
 
@@ -96,6 +97,10 @@ class Model:
     # ---- one step
     def forward(self, rt, meta, cache):
         """float32 logits [wanted rows, vocab] (None when nothing is wanted)."""
+        with ops.stream_scope():
+            return self._forward(rt, meta, cache)
+
+    def _forward(self, rt, meta, cache):
         ctx = StepContext(rt=rt, meta=meta, cache=cache)
         x = self.embedding.forward(ctx, meta.token_ids)
         for i, e in enumerate(self.schedule):

@@ -69,9 +69,13 @@ def loaded_modules():
     return sorted(_loaded)
 
 
+_functions = {}
+
+
 def call(module, fname, *args):
     """Call a C entry point; a non-zero return becomes BackendError with its text."""
-    lib = load(module)
-    rc = getattr(lib, fname)(*args)
-    if rc != 0:
-        raise BackendError(lib.hb_last_error().decode(errors="replace"))
+    fn = _functions.get((module, fname))
+    if fn is None:
+        fn = _functions[(module, fname)] = getattr(load(module), fname)
+    if fn(*args) != 0:
+        raise BackendError(load(module).hb_last_error().decode(errors="replace"))

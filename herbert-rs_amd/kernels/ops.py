@@ -26,8 +26,28 @@ def dtype_code(t):
         raise BackendError(f"dtype {t.dtype} is not supported by the kernels") from None
 
 
+_scoped_stream = None
+
+
+class stream_scope:
+    """While a forward pass runs, the launches go to the stream that was current when it began:
+    looking the stream up costs as much as a launch does."""
+
+    def __enter__(self):
+        global _scoped_stream
+        self.outer = _scoped_stream
+        _scoped_stream = torch.cuda.current_stream().cuda_stream
+        return self
+
+    def __exit__(self, *exc):
+        global _scoped_stream
+        _scoped_stream = self.outer
+        return False
+
+
 def _stream():
-    return torch.cuda.current_stream().cuda_stream
+    s = _scoped_stream
+    return s if s is not None else torch.cuda.current_stream().cuda_stream
 
 
 def _check(t, name, dtype=None, shape=None):
@@ -38,8 +58,15 @@ def _check(t, name, dtype=None, shape=None):
     if dtype is not None and t.dtype != dtype:
         raise BackendError(f"{name} must be {dtype}, got {t.dtype}")
     if shape is not None:
-        if len(shape) != t.dim() or any(s is not None and s != d for s, d in zip(shape, t.shape)):
-            raise BackendError(f"{name} must have shape {list(shape)}, got {list(t.shape)}")
+        got = t.shape
+        bad = len(shape) != len(got)
+        if not bad:
+            for s, d in zip(shape, got):
+                if s is not None and s != d:
+                    bad = True
+                    break
+        if bad:
+            raise BackendError(f"{name} must have shape {list(shape)}, got {list(got)}")
 
 
 def _ptr(t):
