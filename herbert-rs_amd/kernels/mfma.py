@@ -26,6 +26,7 @@ lib.register_signatures("gemm_mfma", {
 
 EPI_STORE, EPI_ADD, EPI_SWIGLU = 0, 1, 2
 _workspaces = {}
+_workspace_of = {}
 
 
 SLICE_WORKSPACE_FLOATS = 16 << 20     # most that the tiled product may use for its K slices (64 MB)
@@ -35,6 +36,17 @@ def _slice_workspace(device, M, N, K, tile=0):
     """(pointer, floats) of the scratch for products whose K may be cut into slices: those with few
     tiles (whether it is cut, and how, is the kernel's estimate). It takes as many slices as fit in it. A buffer that
     was handed out is kept for good: a captured graph may hold its address."""
+    if not isinstance(device, torch.device) or device.index is None:      # "the current device": not remembered
+        return _new_slice_workspace(device, M, N, K, tile)
+    key = (device, M, N, K, tile)
+    found = _workspace_of.get(key)           # (a buffer that was handed out stays valid: see above)
+    if found is not None:
+        return found
+    found = _workspace_of[key] = _new_slice_workspace(device, M, N, K, tile)
+    return found
+
+
+def _new_slice_workspace(device, M, N, K, tile):
     device = torch.device(device)
     if device.index is None:
         device = torch.device(device.type, torch.cuda.current_device())
@@ -111,7 +123,19 @@ NORM_WHOLE_MAX_M = 64         # up to here a product that leaves a norm behind i
 NORM_WHOLE_MAX_N = 8192
 
 
+_handoffs = {}
+
+
 def norm_handoff(M, N, K):
+    """See _norm_handoff; the answer for a size is worked out once."""
+    key = (M, N, K)
+    how = _handoffs.get(key, 0)
+    if how == 0:
+        how = _handoffs[key] = _norm_handoff(M, N, K)
+    return how
+
+
+def _norm_handoff(M, N, K):
     """How a product of these sizes that adds to the residual stream can prepare the RMSNorm that
     follows: "half" (at most 16 rows: bf16(x * g) and sums of squares, finished by the next product),
     "whole" (more rows: the kernel that adds up the K slices norms the rows too; beyond 64 rows only
