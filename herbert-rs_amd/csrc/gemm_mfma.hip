@@ -609,6 +609,60 @@ __device__ __forceinline__ void store_wave_tile(const f32x16 (&acc)[TN32][TM32],
     }
 }
 
+// The same through LDS, for float32 outputs of the large tiles: a lane's sums are runs of four
+// columns of 32 different rows, so a store instruction of the direct way touches 32 lines in
+// pieces of 32 bytes, and reading C back for the add does the same (a round of 256 x 256 tiles
+// spent 45 us beside its products with the store and 68 us with the add, against 19 us with the
+// bfloat16 SwiGLU output). Here a wave first lays PB x 32 rows of its tile into LDS of its own
+// (`stage`, rows of TN32 x 32 floats, the 16-byte chunk c of row r at chunk c ^ (r mod chunks)),
+// then reads them back along the rows: an instruction then moves whole rows, 512 contiguous
+// bytes for a tile 128 wide. Needs ldc and N in steps of 4 and C aligned to 16 bytes.
+template <int EPI, int TN32, int TM32, int PB>
+__device__ __forceinline__ void store_wave_tile_lds(const f32x16 (&acc)[TN32][TM32], float* C, int M, int N, int ldc,
+                                                    int m_base, int n_base, int lane, float* stage) {
+    static_assert(TM32 % PB == 0, "the passes divide the wave's tile");
+    constexpr int CH = TN32 * 8;            // 16-byte chunks of a row
+    constexpr int RPI = 64 / CH;            // rows an instruction moves
+    constexpr int ITER = PB * 32 / RPI;
+    constexpr int GROUP = ITER < 8 ? ITER : 8;
+    const int c32 = lane & 31, g2 = lane >> 5;
+    const int rrow = lane / CH, rchunk = lane % CH;
+#pragma unroll
+    for (int b0 = 0; b0 < TM32; b0 += PB) {
+#pragma unroll
+        for (int bb = 0; bb < PB; ++bb)
+#pragma unroll
+            for (int a = 0; a < TN32; ++a)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int row = 32 * bb + c32, chunk = 8 * a + 2 * q + g2;
+                    const f32x4 v = {acc[a][b0 + bb][4 * q], acc[a][b0 + bb][4 * q + 1], acc[a][b0 + bb][4 * q + 2],
+                                     acc[a][b0 + bb][4 * q + 3]};
+                    *(f32x4*)(stage + row * (CH * 4) + ((chunk ^ (row & (CH - 1))) * 4)) = v;
+                }
+#pragma unroll
+        for (int i0 = 0; i0 < ITER; i0 += GROUP) {
+            f32x4 before[GROUP];
+            if (EPI == EPI_ADD) {
+#pragma unroll
+                for (int u = 0; u < GROUP; ++u) {
+                    const int row = (i0 + u) * RPI + rrow;
+                    const int m = m_base + 32 * b0 + row, n = n_base + 4 * rchunk;
+                    before[u] = (m < M && n < N) ? *(const f32x4*)(C + (size_t)m * ldc + n) : f32x4{0.f, 0.f, 0.f, 0.f};
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < GROUP; ++u) {
+                const int row = (i0 + u) * RPI + rrow;
+                const int m = m_base + 32 * b0 + row, n = n_base + 4 * rchunk;
+                f32x4 v = *(const f32x4*)(stage + row * (CH * 4) + ((rchunk ^ (row & (CH - 1))) * 4));
+                if (EPI == EPI_ADD) v += before[u];
+                if (m < M && n < N) *(f32x4*)(C + (size_t)m * ldc + n) = v;
+            }
+        }
+    }
+}
+
 // The q/k/v projection of prompts with what follows it, for heads of 128 (a wave's tile is 128
 // columns wide: one head): per-head RMSNorm (if weights are given), rotation over the whole head
 // (if tables are given), queries to q_out [M, nq 128] and keys and values into the pages (values
@@ -936,11 +990,31 @@ gemm_tile_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* _
     }
     if constexpr (EPI == EPI_QKV)
         store_wave_tile_qkv<TN32, TM32>(acc, qkv, M, N, m0 + wm * TMB * 16, n0 + wn * TNB * 16, c32, g2);
-    else if (gridDim.y > 1)
-        store_wave_tile<EPI_STORE, TN32, TM32>(acc, partial + (size_t)blockIdx.y * M * N, M, N, N,
-                                               m0 + wm * TMB * 16, n0 + wn * TNB * 16, c32, g2);
-    else
-        store_wave_tile<EPI, TN32, TM32>(acc, Cv, M, N, ldc, m0 + wm * TMB * 16, n0 + wn * TNB * 16, c32, g2);
+    else {
+        // float32 outputs of the large tiles go through LDS (see store_wave_tile_lds): each wave has a
+        // quarter of what the rings held, once every wave's loads have landed and its reads are done
+        constexpr int REGION = (WST * W_STAGE + XST * X_STAGE) * (int)sizeof(bf16) / NW;       // bytes
+        constexpr int PB_FIT = REGION / (32 * TN32 * 128);
+        constexpr int PB = PB_FIT >= TM32 ? TM32 : (PB_FIT >= 2 && TM32 % 2 == 0 ? 2 : 1);
+        constexpr bool VIA_LDS = (EPI == EPI_STORE || EPI == EPI_ADD) && BM >= 128 && PB_FIT >= 1;
+        const bool sliced = gridDim.y > 1;
+        float* const dst = sliced ? partial + (size_t)blockIdx.y * M * N : (float*)Cv;
+        const int ld = sliced ? N : ldc;
+        if (VIA_LDS && (ld & 3) == 0 && (N & 3) == 0 && ((size_t)dst & 15) == 0) {
+            hb_workgroup_barrier();
+            float* const stage = (float*)((char*)lds + wave * REGION);
+            if (sliced || EPI == EPI_STORE)
+                store_wave_tile_lds<EPI_STORE, TN32, TM32, PB>(acc, dst, M, N, ld, m0 + wm * TMB * 16,
+                                                               n0 + wn * TNB * 16, lane, stage);
+            else
+                store_wave_tile_lds<EPI_ADD, TN32, TM32, PB>(acc, dst, M, N, ld, m0 + wm * TMB * 16,
+                                                             n0 + wn * TNB * 16, lane, stage);
+        } else if (sliced) {
+            store_wave_tile<EPI_STORE, TN32, TM32>(acc, dst, M, N, N, m0 + wm * TMB * 16, n0 + wn * TNB * 16, c32, g2);
+        } else {
+            store_wave_tile<EPI, TN32, TM32>(acc, Cv, M, N, ldc, m0 + wm * TMB * 16, n0 + wn * TNB * 16, c32, g2);
+        }
+    }
 }
 
 // K in steps of 32 only: one k-step a stage, everything in 1 KB blocks (the activations too: a
