@@ -99,6 +99,31 @@ def test_gemm_mfma_store_and_add(M, N, K):
     assert float((c2 - (base + want)).abs().max()) <= tol
 
 
+@pytest.mark.parametrize("tile", [188, 142, 122, 2188, 4142])
+@pytest.mark.parametrize("M,N,K", [(300, 520, 1024), (257, 1028, 1024), (640, 330, 1024), (129, 257, 1024)])
+def test_gemm_mfma_large_tiles_with_ragged_edges(M, N, K, tile):
+    """The large tiles by name, whole and with K cut, for sizes that end inside a tile: their
+    float32 outputs leave through LDS a row at a time where N is a multiple of 4, lane by lane
+    otherwise, and rows and columns past the end are never written."""
+    from herbert_rs_amd.kernels import mfma
+    a = rand(M, K, seed=17, dtype=torch.bfloat16)
+    w = rand(N, K, seed=18, dtype=torch.bfloat16)
+    want = (a.double() @ w.double().T).float()
+    tol = 2e-6 * K ** 0.5 * float(want.abs().max()) + 1e-4
+    for packed in (False, True):
+        if packed and N % 16:
+            continue
+        wt = mfma.pack_weight(w) if packed else w
+        c = torch.full((M + 1, N), 7.0, device=dev())          # a row behind the last one
+        mfma.gemm(a, wt, c[:M], packed=packed, tile=tile)
+        assert float((c[:M] - want).abs().max()) <= tol
+        assert float((c[M] - 7.0).abs().max()) == 0.0
+        base = rand(M, N, seed=19)
+        c2 = base.clone()
+        mfma.gemm(a, wt, c2, accumulate=True, packed=packed, tile=tile)
+        assert float((c2 - (base + want)).abs().max()) <= tol
+
+
 @pytest.mark.parametrize("M,I,K", [(1, 16, 32), (8, 12288, 4096), (40, 48, 96), (64, 1024, 64),
                                    (100, 176, 128), (300, 256, 64)])
 def test_gemm_mfma_swiglu(M, I, K):
