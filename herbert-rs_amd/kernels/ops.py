@@ -9,6 +9,8 @@ matmul, rms_norm, swiglu, rotation) and of its GPU command buffer
 (crates/backends/backend_vulkan/src/backend.rs:182-281: embedding, norms, per-head norms, rotation, cache
 append, attention, residual sums), several of them to a kernel here.
 """
+import threading
+
 import torch
 
 from ..errors import BackendError
@@ -26,27 +28,25 @@ def dtype_code(t):
         raise BackendError(f"dtype {t.dtype} is not supported by the kernels") from None
 
 
-_scoped_stream = None
+_scoped = threading.local()      # .stream: the stream of the forward pass that this thread is in
 
 
 class stream_scope:
     """While a forward pass runs, the launches go to the stream that was current when it began:
-    looking the stream up costs as much as a launch does."""
+    looking the stream up costs as much as a launch does. A thread has its own."""
 
     def __enter__(self):
-        global _scoped_stream
-        self.outer = _scoped_stream
-        _scoped_stream = torch.cuda.current_stream().cuda_stream
+        self.outer = getattr(_scoped, "stream", None)
+        _scoped.stream = torch.cuda.current_stream().cuda_stream
         return self
 
     def __exit__(self, *exc):
-        global _scoped_stream
-        _scoped_stream = self.outer
+        _scoped.stream = self.outer
         return False
 
 
 def _stream():
-    s = _scoped_stream
+    s = getattr(_scoped, "stream", None)
     return s if s is not None else torch.cuda.current_stream().cuda_stream
 
 
