@@ -4,8 +4,13 @@
 
 One JSON line: `value` is decoded tokens a second at batch 8 with every sequence holding
 `context` tokens; `prefill` is one 2,048-token prompt; `roofline` prices the decode step
-against HBM; `points` holds decode at batch 1 and 64. Weights are random, token ids are
-random, and the cache below the timed steps is filled by real prefill steps of random prompts.
+against HBM. `points` (flat, numbers only) holds, for batch 1, 8 and 64: tokens a second,
+ms a step, GB/s and the fraction of 8 TB/s at the full context (`decode_b1`, `decode_b1_ms`,
+`decode_b1_gbs`, `decode_b1_frac`), the same at a context of 512 (`..._ctx512...`) and the mean
+over a decode from 512 to the full context (`..._mean...`, from steps timed at a few contexts
+in between); and the other two workloads of the benchmark description through the generation
+loop (`qwen3_1p7b_...`, `qwen3_32b_...`). Weights are random, token ids are random, and the
+cache below the timed steps is filled by real prefill steps of random prompts.
 """
 import argparse
 import json
@@ -21,41 +26,64 @@ PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
 
 
 def load_shape(index=2):
-    """Layer sizes of a benchmark configuration, parsed from BASELINE.json's configs[index]."""
+    """Layer sizes of a benchmark configuration, from BASELINE.json's configs[index]. Every
+    field must be found where the sentence is expected to give it; a reworded sentence raises
+    rather than yield another model."""
     import re
     with open(os.path.join(ROOT, "BASELINE.json")) as f:
         text = json.load(f)["configs"][index]
 
-    def num(pattern):
-        return int(re.search(pattern, text).group(1))
-    return dict(
-        num_hidden_layers=num(r"(\d+) layers"), hidden_size=num(r"hidden (\d+)"),
-        num_attention_heads=num(r"(\d+) query heads"), num_key_value_heads=num(r"(\d+) KV heads"),
-        head_dim=num(r"head_dim (\d+)"), intermediate_size=num(r"intermediate (\d+)"),
-        vocab_size=num(r"vocab (\d+)"),
-        context=num(r"Context length (\d+)") if "Context length" in text else 0,
-        rope_theta=1e6, rms_norm_eps=1e-6, tie_word_embeddings="tied embeddings" in text)
+    def find(field, pattern, convert=int):
+        found = re.findall(pattern, text)
+        if len(found) != 1:
+            raise ValueError(f"BASELINE.json configs[{index}]: expected {field} once as /{pattern}/, "
+                             f"found {found!r} in: {text!r}")
+        return convert(found[0])
+
+    tied, separate = "tied embeddings" in text, "separate lm_head" in text
+    if tied == separate:
+        raise ValueError(f"BASELINE.json configs[{index}]: neither or both of 'tied embeddings' and "
+                         f"'separate lm_head' in: {text!r}")
+    shape = dict(
+        num_hidden_layers=find("layers", r"Model: (\d+) layers"), hidden_size=find("hidden", r"hidden (\d+),"),
+        num_attention_heads=find("query heads", r"(\d+) query heads"),
+        num_key_value_heads=find("KV heads", r"(\d+) KV heads"),
+        head_dim=find("head_dim", r"head_dim (\d+)[, ]"), intermediate_size=find("intermediate", r"intermediate (\d+),"),
+        vocab_size=find("vocab", r"vocab (\d+),"), rope_theta=find("rope_theta", r"rope_theta ([0-9.e+]+),", float),
+        rms_norm_eps=find("rms_norm_eps", r"rms_norm_eps ([0-9.e-]+),", float), tie_word_embeddings=tied)
+    shape["context"] = find("context length", r"Context length (\d+) per sequence") if index == 2 else 0
+    for key, value in shape.items():
+        if key not in ("tie_word_embeddings", "context") and not value > 0:
+            raise ValueError(f"BASELINE.json configs[{index}]: {key} = {value}")
+    return shape
 
 
-def run_workload(args, index):
+def workload_bytes(cfg, layers, elem):
+    """(bytes of weights a decode step reads once, bytes of cache per token held)."""
+    H, I, V = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
+    per_layer = (cfg.q_dim + 2 * cfg.kv_dim) * H + H * cfg.q_dim + 3 * H * I
+    return (layers * per_layer + V * H) * elem, layers * 2 * cfg.kv_dim * elem, per_layer
+
+
+def run_workload(args, index, new=None):
     """The other two workloads of the benchmark description, through the generation loop:
     configs[3] (1.7B shape: 16 prompts of 64..1024 tokens, 256 new tokens each) and configs[4]
-    (32B shape: 8 prompts of 2048 tokens, 512 new tokens each)."""
+    (32B shape: 8 prompts of 2048 tokens, 512 new tokens each). Returns the record as a dict."""
     import torch
     import herbert_rs_amd as hb
     from herbert_rs_amd.sampling import SamplingParams
     shape = load_shape(index)
     shape.pop("context")
+    layers_full = shape["num_hidden_layers"]
     if args.layers:
         shape["num_hidden_layers"] = args.layers
     gen = torch.Generator().manual_seed(index)
     if index == 3:
         lengths = torch.randint(64, 1025, (16,), generator=gen).tolist()
-        new, name = 256, "Qwen3-1.7B shape"
+        default_new, name = 256, "Qwen3-1.7B shape"
     else:
-        lengths, new, name = [2048] * 8, 512, "Qwen3-32B shape"
-    if args.steps != 32:
-        new = args.steps
+        lengths, default_new, name = [2048] * 8, 512, "Qwen3-32B shape"
+    new = new or default_new
     raw = dict(shape, architectures=["Qwen3ForCausalLM"], model_type="qwen3",
                max_position_embeddings=4096, eos_token_id=151645)
     cfg = hb.Qwen3Config.from_dict(raw)
@@ -72,14 +100,22 @@ def run_workload(args, index):
     st = engine.last_generation_stats
     assert all(len(r.tokens) == new for r in results)
     decoded = st.generated_tokens - len(prompts)
-    print(json.dumps({
+    ms = st.decode_seconds / st.decode_steps * 1e3
+    elem = 2 if args.dtype == "bfloat16" else 4
+    weight_bytes, kv_per_token, _ = workload_bytes(cfg, cfg.num_hidden_layers, elem)
+    held = sum(n + new / 2.0 for n in lengths)          # tokens in the cache at the middle of the decode
+    gbs = (weight_bytes + held * kv_per_token) / (ms * 1e-3) / 1e9
+    del engine
+    torch.cuda.empty_cache()
+    return {
         "metric": f"decode tok/s, {name}, batch {len(prompts)}, {new} new tokens each",
         "value": round(decoded / st.decode_seconds, 2), "unit": "tokens/s", "n_gpus": 1,
-        "steps": st.decode_steps, "warmup": 0, "ms_per_step": round(st.decode_seconds / st.decode_steps * 1e3, 4),
+        "steps": st.decode_steps, "warmup": 0, "ms_per_step": round(ms, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
         "data": "synthetic: random weights N(0, 0.02), random token ids",
-        "config": {"model": name, "layers": cfg.num_hidden_layers, "hidden_size": cfg.hidden_size,
+        "config": {"model": name, "layers": layers_full, "layers_run": cfg.num_hidden_layers,
+                   "hidden_size": cfg.hidden_size,
                    "num_attention_heads": cfg.num_attention_heads,
                    "num_key_value_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
                    "intermediate_size": cfg.intermediate_size, "vocab_size": cfg.vocab_size,
@@ -87,8 +123,9 @@ def run_workload(args, index):
                    "prompt_tokens": st.prompt_tokens, "new_tokens": new, "parallelism": "single GPU"},
         "prefill": {"value": round(st.prompt_tokens / st.prefill_seconds, 1), "tokens": st.prompt_tokens,
                     "ms": round(st.prefill_seconds * 1e3, 3)},
-    }))
-    return 0
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_GBS, 4)},
+    }
 
 
 def main():
@@ -101,6 +138,9 @@ def main():
     ap.add_argument("--context", type=int, default=None)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
+    ap.add_argument("--no-workloads", action="store_true",
+                    help="skip the 1.7B and 32B workloads that the default run adds to `points`")
+    ap.add_argument("--no-sweep", action="store_true", help="time the full context only, not 512 and the mean")
     ap.add_argument("--workload", default="headline", choices=["headline", "qwen3-1.7b", "qwen3-32b"],
                     help="headline: BASELINE.json configs[2]; the others: configs[3] and configs[4]")
     ap.add_argument("--prefill-tokens", type=int, default=2048, help="length of the prompt of the prefill figure")
@@ -113,7 +153,9 @@ def main():
         return 2
 
     if args.workload != "headline":
-        return run_workload(args, 3 if args.workload == "qwen3-1.7b" else 4)
+        print(json.dumps(run_workload(args, 3 if args.workload == "qwen3-1.7b" else 4,
+                                      new=None if args.steps == 32 else args.steps)))
+        return 0
 
     import torch
     import herbert_rs_amd as hb
@@ -145,36 +187,44 @@ def main():
 
     # bytes of weights that one decode step reads once
     H, I, V = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
-    per_layer = (cfg.q_dim + 2 * cfg.kv_dim) * H + H * cfg.q_dim + 3 * H * I
-    weight_bytes = (layers * per_layer + V * H) * elem
-    kv_bytes_per_token = layers * 2 * cfg.kv_dim * elem
+    weight_bytes, kv_bytes_per_token, per_layer = workload_bytes(cfg, layers, elem)
 
-    def decode_run(batch, steps, warmup):
-        """tokens/s and ms/step of `steps` decode steps at `batch`, every sequence at `context`."""
+    def step_gbs(batch, mean_context, ms):
+        return (weight_bytes + batch * mean_context * kv_bytes_per_token) / (ms * 1e-3) / 1e9
+
+    def decode_run(batch, plan):
+        """[(context, tokens/s, ms/step)] for each (context, steps, warmup) of `plan` (contexts
+        ascending): `steps` timed decode steps at `batch` after `warmup` untimed ones, ending with
+        every sequence holding `context` tokens; one pass over a cache that is filled by real
+        prefill of random prompts up to where each run's steps begin."""
         slots = [engine.alloc_slot() for _ in range(batch)]
-        fill = context - steps - warmup
-        chunk = 2048
-        for s in slots:                      # real prefill of random prompts, in chunks
-            for a in range(0, fill, chunk):
-                n = min(chunk, fill - a)
-                engine.step([StepEntry(s, ids(n), [])])
         chooser = Sampler(SamplingParams(temperature=0.0), batch, V, engine.device)
         tokens = [ids(1)[0] for _ in range(batch)]
+        held, chunk, out = 0, 2048, []
 
         def one():
             logits = engine.step([StepEntry(s, [t], [0]) for s, t in zip(slots, tokens)])
             return chooser.choose(logits, range(batch))
-        for _ in range(warmup):
-            tokens = one()
-        torch.cuda.synchronize()
-        t = time.perf_counter()
-        for _ in range(steps):
-            tokens = one()
-        torch.cuda.synchronize()
-        dt = time.perf_counter() - t
+        for c, steps, warmup in plan:
+            fill = c - steps - warmup - held
+            if fill < 0:
+                raise ValueError(f"context {c} leaves no room for {steps} + {warmup} steps after {held} tokens")
+            for s in slots:
+                for a in range(0, fill, chunk):
+                    engine.step([StepEntry(s, ids(min(chunk, fill - a)), [])])
+            for _ in range(warmup):
+                tokens = one()
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            for _ in range(steps):
+                tokens = one()
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t
+            held = c
+            out.append((c, batch * steps / dt, dt / steps * 1e3))
         for s in slots:
             engine.free_slot(s)
-        return batch * steps / dt, dt / steps * 1e3
+        return out
 
     def prefill_run(tokens_n, reps):
         slot = engine.alloc_slot()
@@ -194,11 +244,50 @@ def main():
         print(f"[bench] prefill {args.prefill_tokens}: {args.prefill_tokens / sec:.0f} tok/s, {sec * 1e3:.2f} ms",
               file=sys.stderr, flush=True)
         return 0
-    value, ms = decode_run(args.batch, args.steps, args.warmup)
-    print(f"[bench] decode b{args.batch}: {value:.1f} tok/s, {ms:.3f} ms/step", file=sys.stderr, flush=True)
-    avg_ctx = context - args.steps / 2.0
-    step_bytes = weight_bytes + args.batch * avg_ctx * kv_bytes_per_token
-    achieved = step_bytes / (ms * 1e-3) / 1e9
+    # contexts of the sweep: 512 (where the described decode starts), the full context, and a
+    # few in between for the mean over a decode from the one to the other
+    sweep_steps, sweep_warmup = min(args.steps, 12), 3
+    low = 512
+    between = [] if args.no_sweep or args.no_points or context <= low + 64 else \
+        [c for c in (low, 1024, 2048, 3072) if c < context - args.steps - args.warmup - sweep_steps]
+
+    def measure(batch):
+        """(at the full context, at 512 or None, mean over 512 -> full context or None), each
+        (tokens/s, ms/step, GB/s)."""
+        # the sweep's shorter runs first, in one pass over a cache that grows; the full context is
+        # timed with exactly --steps steps after --warmup
+        runs = decode_run(batch, [(c, sweep_steps, sweep_warmup) for c in between]
+                          + [(context, args.steps, args.warmup)])
+        full = runs.pop()
+        at_full = (full[1], full[2], step_gbs(batch, context - args.steps / 2.0, full[2]))
+        if not runs:
+            return at_full, None, None
+        c0, v0, ms0 = runs[0]
+        at_low = (v0, ms0, step_gbs(batch, c0 - sweep_steps / 2.0, ms0))
+        pts = [(c - sweep_steps / 2.0, ms_c) for c, _, ms_c in runs] + [(context - args.steps / 2.0, full[2])]
+        area = sum((pts[i + 1][0] - pts[i][0]) * (pts[i + 1][1] + pts[i][1]) / 2.0 for i in range(len(pts) - 1))
+        mean_ms = area / (pts[-1][0] - pts[0][0])
+        mean_ctx = (pts[-1][0] + pts[0][0]) / 2.0
+        return at_full, at_low, (batch / mean_ms * 1e3, mean_ms, step_gbs(batch, mean_ctx, mean_ms))
+
+    def add_points(points, batch, result):
+        at_full, at_low, mean = result
+        for tag, r in (("", at_full), ("_ctx512", at_low), ("_mean_512_to_full", mean)):
+            if r is None:
+                continue
+            key = f"decode_b{batch}{tag}"
+            points[key] = round(r[0], 2)
+            points[key + "_ms"] = round(r[1], 4)
+            points[key + "_gbs"] = round(r[2], 1)
+            points[key + "_frac"] = round(r[2] / HBM_GBS, 4)
+
+    points = {}
+    head = measure(args.batch)
+    value, ms = head[0][0], head[0][1]
+    add_points(points, args.batch, head)
+    for key in (f"decode_b{args.batch}", f"decode_b{args.batch}_ms", f"decode_b{args.batch}_gbs",
+                f"decode_b{args.batch}_frac"):
+        points.pop(key)          # the headline itself: `value`, `ms_per_step`, `roofline`
     out = {
         "metric": "decode tok/s at batch 8, Qwen3-8B shape, context 4096 (+ prefill tok/s at 2048 "
                   "tokens, decode at batch 1 and 64)",
@@ -229,11 +318,25 @@ def main():
         out["prefill"] = {"value": round(T / sec, 1), "tokens": T, "ms": round(sec * 1e3, 3),
                           "frac": round(flops / sec / peak, 4)}
         print(f"[bench] prefill {T}: {T / sec:.0f} tok/s", file=sys.stderr, flush=True)
-        b1, _ = decode_run(1, args.steps, args.warmup)
-        print(f"[bench] decode b1: {b1:.1f} tok/s", file=sys.stderr, flush=True)
-        b64, _ = decode_run(64, args.steps, args.warmup)
-        print(f"[bench] decode b64: {b64:.1f} tok/s", file=sys.stderr, flush=True)
-        out["points"] = {"decode_b1": round(b1, 2), "decode_b64": round(b64, 2)}
+        for batch in (1, 64):
+            if batch != args.batch:
+                r = measure(batch)
+                add_points(points, batch, r)
+                print(f"[bench] decode b{batch}: {r[0][0]:.1f} tok/s, {r[0][1]:.3f} ms/step", file=sys.stderr, flush=True)
+        if not args.no_workloads and not args.layers:
+            del engine
+            torch.cuda.empty_cache()
+            for index, tag in ((3, "qwen3_1p7b_b16"), (4, "qwen3_32b_b8")):
+                rec = run_workload(args, index)
+                points[tag + "_decode"] = rec["value"]
+                points[tag + "_decode_ms"] = rec["ms_per_step"]
+                points[tag + "_decode_gbs"] = rec["roofline"]["achieved"]
+                points[tag + "_decode_frac"] = rec["roofline"]["frac"]
+                points[tag + "_prefill"] = rec["prefill"]["value"]
+                print(f"[bench] {rec['config']['model']}: {rec['value']:.1f} tok/s, {rec['ms_per_step']:.3f} ms/step",
+                      file=sys.stderr, flush=True)
+    if points:
+        out["points"] = points
     print(json.dumps(out))
     return 0
 

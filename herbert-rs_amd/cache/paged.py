@@ -53,6 +53,11 @@ class KVGroup:
         v = self.pool[i, 1].view(n_pages, self.need.kv_heads, self.need.head_dim, PAGE_TOKENS)
         return LayerKV(k, v, self.table, PAGE_TOKENS, int(self.need.window or 0))
 
+    def pages_missing(self, slot, new_length):
+        """How many pages `ensure(slot, new_length)` would take."""
+        row = self.table_host[slot]
+        return int((row[int(self.first_page[slot]):pages_for(new_length)] < 0).sum())
+
     def ensure(self, slot, new_length):
         """Hold a page for every position below new_length that a query may still see."""
         row = self.table_host[slot]
@@ -85,12 +90,20 @@ class KVGroup:
             p += 1
         self.first_page[slot] = p
 
-    def truncate(self, slot, length):
-        row = self.table_host[slot]
+    def can_truncate(self, slot, length):
         if self.need.window:
             oldest = max(0, length + 1 - self.need.window)   # oldest key the next query sees
             if self.first_page[slot] * PAGE_TOKENS > oldest:
-                raise CacheError("cannot roll a windowed cache back past keys it has given up")
+                return False
+        return True
+
+    def truncate(self, slot, length):
+        """Give back the pages wholly behind `length`. What the kept last page holds behind
+        `length` stays where it is: no query sees it (keys are counted, not marked) and the next
+        tokens overwrite it."""
+        row = self.table_host[slot]
+        if not self.can_truncate(slot, length):
+            raise CacheError("cannot roll a windowed cache back past keys it has given up")
         for p in range(pages_for(length), self.pages_per_slot):
             if row[p] >= 0:
                 self.pages.give_back(int(row[p]))
@@ -186,6 +199,33 @@ class Cache:
             g.ensure(slot, new_length)
         return new_length
 
+    def reserve_all(self, wanted):
+        """`reserve` for every (slot, new tokens) of a step, all or nothing: the pages that each
+        group needs are counted first, and a step that does not fit raises CacheError with the
+        cache unchanged."""
+        targets = []
+        for slot, new_tokens in wanted:
+            new_length = self.length(slot) + int(new_tokens)
+            if new_length > self.max_positions:
+                raise CacheError(f"slot {slot}: {new_length} positions exceed the model's "
+                                 f"{self.max_positions}")
+            targets.append((slot, new_length))
+        for g in self.kv_groups.values():
+            need = sum(g.pages_missing(slot, n) for slot, n in targets)
+            if need > g.pages.free_count:
+                raise CacheError(f"the step needs {need} more pages of {PAGE_TOKENS} tokens but only "
+                                 f"{g.pages.free_count} of {g.pages.count} are free")
+        for slot, new_length in targets:
+            for g in self.kv_groups.values():
+                g.ensure(slot, new_length)
+
+    def unreserve(self, slot):
+        """Give back what was reserved for a step that did not run: the pages behind the slot's
+        committed length."""
+        length = self.length(slot)
+        for g in self.kv_groups.values():
+            g.truncate(slot, length)
+
     def commit(self, slot, new_tokens):
         """The step has run: the slot is longer; windowed groups give up what is out of sight."""
         self.lengths[slot] += int(new_tokens)
@@ -200,6 +240,9 @@ class Cache:
             raise CacheError(f"cannot truncate slot {slot} of length {self.length(slot)} to {length}")
         if self.state_groups and length != self.length(slot):
             raise CacheError("a cache with per-sequence state cannot be rolled back")
+        for g in self.kv_groups.values():       # refuse before anything is given back
+            if not g.can_truncate(slot, length):
+                raise CacheError("cannot roll a windowed cache back past keys it has given up")
         for g in self.kv_groups.values():
             g.truncate(slot, length)
         self.lengths[slot] = length

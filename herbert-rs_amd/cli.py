@@ -4,26 +4,96 @@ Kept with their names, meanings and defaults: --model, --prompt, --prompt-file, 
 --max-tokens (2048), --ignore-eos, --no-repeat-check, --stop, --verbose, --temperature (0.4,
 0 = greedy), --top-k (40, 0 = off), --top-p (0.9, 1.0 = off), --show-specials. Added here:
 --dtype, --seed, --cache-tokens, and --random-weights to write a random model folder.
-With a tokenizer.json in the model folder the prompt is text wrapped in the ChatML
-template (main.rs:281-294); without one it is comma-separated token ids
-(crates/cli/src/token_parser.rs:13-26) and the output is token ids.
+With a tokenizer.json in the model folder the prompt is text wrapped in the architecture's
+chat template (for this family ChatML, main.rs:281-294; the template and the end-of-turn
+token are data of the architecture's registry entry); without one it is comma-separated
+token ids (crates/cli/src/token_parser.rs:13-26) and the output is token ids.
+--stop with a tokenizer is a stop string, matched on the decoded text after every token
+(main.rs:236-247,1328-1332,1360); without one it is a token id. --max-tokens counts decode
+steps after the token that the prompt gives, as the reference's single shot counts them
+(main.rs:1040,1241): up to max-tokens + 1 tokens come out. SIGINT, SIGTERM and SIGHUP set a
+flag that the generation loop looks at before every decode step; a second signal exits at
+once with 130 (main.rs:22-50,1242-1245).
 """
 import argparse
-import json
 import os
+import signal
 import sys
 import time
 
 from .errors import HerbertError, RequestError
 
 
-def build_prompt(user_prompt, system_prompt=None):
-    """ChatML as the reference builds it for this family (crates/cli/src/main.rs:281-294)."""
-    out = ""
-    if system_prompt:
-        out += "<|im_start|>system\n" + system_prompt + "<|im_end|>\n"
-    out += "<|im_start|>user\n" + user_prompt + "<|im_end|>\n<|im_start|>assistant\n"
+def decode_escaped_text(raw):
+    """\\n, \\r, \\t, \\0 and \\\\ become the characters they name; any other backslash stays
+    (crates/cli/src/main.rs:212-234)."""
+    out = []
+    it = iter(raw)
+    for c in it:
+        if c != "\\":
+            out.append(c)
+            continue
+        nxt = next(it, None)
+        if nxt is None:
+            out.append("\\")
+        elif nxt in "nrt0\\":
+            out.append({"n": "\n", "r": "\r", "t": "\t", "0": "\0", "\\": "\\"}[nxt])
+        else:
+            out.append("\\" + nxt)
+    return "".join(out)
+
+
+def normalize_stop_sequences(raw):
+    """Trimmed, unescaped, without empty ones and repeats (crates/cli/src/main.rs:249-258)."""
+    out = []
+    for seq in raw:
+        decoded = decode_escaped_text(seq.strip())
+        if decoded and decoded not in out:
+            out.append(decoded)
     return out
+
+
+def find_stop_sequence(text, stop_sequences):
+    """The first stop sequence that the tail of `text` holds, else None: only the last
+    (longest stop sequence + 64) bytes are searched (crates/cli/src/main.rs:236-247)."""
+    longest = max((len(s.encode()) for s in stop_sequences), default=0)
+    tail = text.encode()[-(longest + 64):].decode(errors="ignore") if text else ""
+    for seq in stop_sequences:
+        if seq in tail:
+            return seq
+    return None
+
+
+class InterruptFlag:
+    """Set by the first SIGINT / SIGTERM / SIGHUP; the second exits at once with 130
+    (crates/cli/src/main.rs:22-50)."""
+
+    def __init__(self):
+        self.count = 0
+        self._old = {}
+
+    def __call__(self):
+        return self.count > 0
+
+    def _handle(self, signum, frame):
+        self.count += 1
+        if self.count >= 2:
+            os._exit(130)
+
+    def install(self):
+        for name in ("SIGINT", "SIGTERM", "SIGHUP"):
+            sig = getattr(signal, name, None)
+            if sig is not None:
+                try:
+                    self._old[sig] = signal.signal(sig, self._handle)
+                except ValueError:       # not the main thread: the flag can still be set by hand
+                    pass
+        return self
+
+    def restore(self):
+        for sig, old in self._old.items():
+            signal.signal(sig, old)
+        self._old = {}
 
 
 def parse_token_ids(text):
@@ -83,7 +153,7 @@ def main(argv=None):
 
 def _run(args):
     from .api import load, write_random_model
-    from .sampling import SamplingParams
+    from .sampling import INTERRUPTED, STOP_SEQUENCE, SamplingParams
     if args.random_weights and not os.path.exists(os.path.join(args.model, "model.safetensors")):
         write_random_model(args.model, os.path.join(args.model, "config.json"), seed=args.seed or 0,
                            dtype=args.dtype)
@@ -94,29 +164,31 @@ def _run(args):
     if prompt is None:
         raise RequestError("--prompt or --prompt-file is required (there is no interactive mode)")
     tokenizer = load_tokenizer(args.model)
+    from .config import load_config
+    chat = load_config(args.model)[0].chat
     if tokenizer is not None:
-        ids = tokenizer.encode(build_prompt(prompt, args.system), add_special_tokens=False).ids
+        text = chat.build_prompt(prompt, args.system) if chat is not None else prompt
+        ids = tokenizer.encode(text, add_special_tokens=False).ids
     else:
         ids = parse_token_ids(prompt)
     stop_ids = []
     stop_strings = []
-    for s in args.stop:
-        if tokenizer is None:
+    if tokenizer is None:
+        for s in args.stop:
             stop_ids.extend(parse_token_ids(s))
-        else:
-            stop_strings.append(s.encode().decode("unicode_escape"))
-    if tokenizer is not None:
-        im_end = tokenizer.token_to_id("<|im_end|>")
-        if im_end is not None:
-            stop_ids.append(im_end)
+    else:
+        stop_strings = normalize_stop_sequences(args.stop)
+        if chat is not None and chat.end_of_turn is not None:
+            end = tokenizer.token_to_id(chat.end_of_turn)
+            stop_ids.append(end if end is not None else chat.end_of_turn_id)
 
     t0 = time.perf_counter()
-    cache_tokens = args.cache_tokens or (len(ids) + args.max_tokens + 64)
+    cache_tokens = args.cache_tokens or (len(ids) + args.max_tokens + 65)
     engine = load(args.model, dtype=args.dtype, cache_tokens=cache_tokens)
     load_seconds = time.perf_counter() - t0
 
     params = SamplingParams(temperature=args.temperature, top_k=args.top_k, top_p=args.top_p,
-                            max_tokens=args.max_tokens, stop_ids=tuple(stop_ids),
+                            max_tokens=args.max_tokens + 1, stop_ids=tuple(stop_ids),
                             ignore_eos=args.ignore_eos, repeat_check=not args.no_repeat_check,
                             seed=args.seed)
     produced = []
@@ -126,16 +198,28 @@ def _run(args):
         produced.append(tok)
         if tokenizer is None:
             print(tok if len(produced) == 1 else f",{tok}", end="", flush=True)
-        else:
-            text = tokenizer.decode(produced, skip_special_tokens=not args.show_specials)
-            if not text.endswith("�"):
-                print(text[printed[0]:], end="", flush=True)
-                printed[0] = len(text)
+            return None
+        # the whole text again each time and only what is new printed, never a trailing U+FFFD,
+        # which a later token may still complete (crates/cli/src/main.rs:1306-1326)
+        text = tokenizer.decode(produced, skip_special_tokens=not args.show_specials)
+        safe = len(text.rstrip("\ufffd"))
+        if safe > printed[0]:
+            print(text[printed[0]:safe], end="", flush=True)
+            printed[0] = safe
+        if stop_strings and find_stop_sequence(text, stop_strings) is not None:
+            return STOP_SEQUENCE
+        return None
 
+    interrupt = InterruptFlag().install()
     t0 = time.perf_counter()
-    result = engine.generate([ids], params, on_token=on_token)[0]
+    try:
+        result = engine.generate([ids], params, on_token=on_token, interrupt=interrupt)[0]
+    finally:
+        interrupt.restore()
     total = time.perf_counter() - t0
     print()
+    if result.stop_reason == INTERRUPTED:
+        print("[herbert] Interrupted", file=sys.stderr)
     if args.verbose:
         st = engine.last_generation_stats
         decoded = max(0, st.generated_tokens - 1)

@@ -16,6 +16,8 @@ from ..config import load_config
 from ..errors import BackendError, ModelLoadError, RequestError
 from ..parts import Runtime
 from ..weights import read_tensor, read_tensors
+from collections import OrderedDict
+
 from . import batch as batching
 from .batch import StaticDecodeMeta, StepEntry
 from .model import Model
@@ -25,11 +27,23 @@ _DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16,
 
 
 class _DecodeState:
-    def __init__(self, static):
+    """What the decode steps of one batch size share: the fixed metadata buffers and the one
+    logits buffer that every graph of this batch size writes to."""
+
+    def __init__(self, static, logits):
         self.static = static
-        self.seen = {}
-        self.graphs = {}
-        self.logits = {}
+        self.logits = logits
+        self.seen = {}          # context bucket -> eager steps run
+
+
+# Captured graphs kept at any time, over all batch sizes and context buckets; the least recently
+# replayed one is dropped for a new one. A graph holds no logits of its own (they are per batch
+# size) and no scratch (the parts' buffers are the runtime's), so a graph costs its kernel
+# arguments only; the cap bounds what a long run over many batch sizes and contexts accumulates.
+MAX_GRAPHS = 48
+# Batch sizes whose fixed buffers (metadata, logits [B, vocab] float32) are kept; beyond it the
+# least recently used size is dropped together with its graphs.
+MAX_DECODE_BATCH_SIZES = 8
 
 
 def require_gpu():
@@ -54,7 +68,10 @@ class Engine:
                            self.device, max_slots)
         self.steps_run = 0
         self.use_graphs = bool(use_graphs) and self.model.graph_safe
-        self._decode = {}       # batch size -> _DecodeState
+        self._decode = OrderedDict()    # batch size -> _DecodeState, least recently used first
+        self._graphs = OrderedDict()    # (batch size, context bucket) -> graph, least recently used first
+        self.graphs_captured = 0
+        self.ignored_tensors = []       # stored tensors that the model did not ask for
         self._tensor_source = None      # how get_tensor finds a tensor again: set by the constructors below
 
     # ---- construction
@@ -65,9 +82,12 @@ class Engine:
         arch, config = load_config(folder)
         spec = arch.build_spec(config)
         needs = Model(spec).tensor_needs()
-        tensors = read_tensors(folder, needs)
+        ignored = []
+        tensors = read_tensors(folder, needs, name_map=arch.name_map, ignored=ignored)
         engine = cls(config, spec, tensors, dtype, max_tokens, max_slots, device, use_graphs)
-        engine._tensor_source = lambda name: read_tensor(folder, name, needs)
+        engine._tensor_source = lambda name: read_tensor(folder, name, needs, arch.name_map)
+        engine.ignored_tensors = ignored
+        engine.architecture = arch
         return engine
 
     @classmethod
@@ -89,6 +109,7 @@ class Engine:
             return random_tensors({name: needs[name]}, seed, weight_dtype or dtype, std, norm_std,
                                   device=str(dev))[name].cpu()
         engine._tensor_source = again
+        engine.architecture = arch
         return engine
 
     def get_tensor(self, name):
@@ -105,6 +126,15 @@ class Engine:
 
     def free_slot(self, slot):
         self.cache.free_slot(slot)
+
+    def truncate(self, slot, length):
+        """Roll a sequence back to its first `length` positions; the next step's tokens go on from
+        there and overwrite what lay behind (the reference's truncate_kv,
+        crates/core/src/backend.rs:129-310, crates/backends/backend_common/src/cpu_backend.rs:527-543,
+        crates/backends/backend_common/src/kv_cache.rs:389-397). Pages wholly behind the new
+        length go back to the pool. Refused where it cannot be done: beyond the present length,
+        into keys that a windowed group has already given up, or with per-sequence state."""
+        self.cache.truncate(slot, int(length))
 
     # ---- the step
     def step(self, entries):
@@ -133,13 +163,18 @@ class Engine:
                 raise RequestError(f"sequence of {start + len(e.tokens)} tokens exceeds "
                                    f"max_position_embeddings ({self.spec.max_positions})")
             starts.append(start)
-        for e in entries:
-            self.cache.reserve(e.slot, len(e.tokens))
-        if self.use_graphs and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
-            logits = self._decode_step(entries, starts)
-        else:
-            meta = batching.pack(entries, starts, self.device)
-            logits = self.model.forward(self.rt, meta, self.cache)
+        # all pages of the step or none: a step that does not fit leaves the cache as it was
+        self.cache.reserve_all([(e.slot, len(e.tokens)) for e in entries])
+        try:
+            if self.use_graphs and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
+                logits = self._decode_step(entries, starts)
+            else:
+                meta = batching.pack(entries, starts, self.device)
+                logits = self.model.forward(self.rt, meta, self.cache)
+        except Exception:
+            for e in entries:       # nothing was committed: give back what was taken for the step
+                self.cache.unreserve(e.slot)
+            raise
         for e in entries:
             self.cache.commit(e.slot, len(e.tokens))
         self.steps_run += 1
@@ -150,34 +185,52 @@ class Engine:
         metadata lives in fixed buffers; from the second step of a shape on, the forward pass is a
         captured HIP graph that is replayed, so that the host launches one graph and not hundreds
         of kernels. A graph is tied to the batch size and to the bucket of the longest context
-        (which sizes the attention grid); the logits it returns are overwritten by its next replay."""
+        (which sizes the attention grid). All graphs of a batch size write their logits into that
+        size's one buffer: what a step returns is overwritten by the next decode step of the same
+        batch size. At most MAX_GRAPHS graphs and MAX_DECODE_BATCH_SIZES batch sizes are kept,
+        the least recently used go first."""
         B = len(entries)
         state = self._decode.get(B)
         if state is None:
-            state = self._decode[B] = _DecodeState(StaticDecodeMeta(B, self.device))
+            while len(self._decode) >= MAX_DECODE_BATCH_SIZES:
+                torch.cuda.synchronize(self.device)
+                old, _ = self._decode.popitem(last=False)
+                for key in [k for k in self._graphs if k[0] == old]:
+                    del self._graphs[key]
+            logits = torch.empty((B, self.spec.vocab_size), dtype=torch.float32, device=self.device)
+            state = self._decode[B] = _DecodeState(StaticDecodeMeta(B, self.device), logits)
+        self._decode.move_to_end(B)
         meta = state.static.update(entries, starts)
-        key = meta.context_bucket
-        graph = state.graphs.get(key)
+        key = (B, meta.context_bucket)
+        graph = self._graphs.get(key)
         if graph is not None:
+            self._graphs.move_to_end(key)
             graph.replay()
-            return state.logits[key]
-        seen = state.seen.get(key, 0)
-        state.seen[key] = seen + 1
-        if seen == 0:
-            return self.model.forward(self.rt, meta, self.cache)      # also sizes every scratch buffer
-        torch.cuda.synchronize(self.device)
+            return state.logits
+        seen = state.seen.get(key[1], 0)
+        state.seen[key[1]] = seen + 1
+        if seen == 0:       # eager: also sizes every scratch buffer
+            return self.model.forward(self.rt, meta, self.cache, logits_out=state.logits)
+        torch.cuda.synchronize(self.device)      # also: no graph that is dropped below still runs
+        while len(self._graphs) >= MAX_GRAPHS:
+            self._graphs.popitem(last=False)
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
-            logits = self.model.forward(self.rt, meta, self.cache)
-        state.graphs[key] = graph
-        state.logits[key] = logits
+            self.model.forward(self.rt, meta, self.cache, logits_out=state.logits)
+        self._graphs[key] = graph
+        self.graphs_captured += 1
         graph.replay()
-        return logits
+        return state.logits
 
-    def generate(self, prompts, params=None, max_batch=64, on_token=None):
+    def decode_graph_stats(self):
+        """(graphs kept, batch sizes kept, bytes of the per-batch-size logits buffers)."""
+        held = sum(st.logits.numel() * 4 for st in self._decode.values())
+        return len(self._graphs), len(self._decode), held
+
+    def generate(self, prompts, params=None, max_batch=64, on_token=None, interrupt=None):
         """Generate from lists of token ids; see engine.generate.Generator."""
         from .generate import Generator
         gen = Generator(self, max_batch=max_batch)
-        results = gen.generate(prompts, params, on_token)
+        results = gen.generate(prompts, params, on_token, interrupt)
         self.last_generation_stats = gen.stats
         return results

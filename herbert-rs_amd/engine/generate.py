@@ -4,9 +4,20 @@ Requests are served in batches, one after another: the prompts of a batch in
 one step, then one token for every sequence that still runs. A sequence ends
 on its end-of-sequence token (kept in the output, as the reference keeps it:
 crates/cli/src/main.rs:1272,1357-1359), on a stop token, after max_tokens
-tokens (counting the one the prompt gives, crates/cli/src/chat.rs:231), on
-a repetition loop (crates/core/src/decode_utils.rs:14-33) or at the model's
-last position; it gives its slot back at once and the others go on.
+tokens, on a repetition loop (crates/core/src/decode_utils.rs:14-33), when
+the caller's `on_token` says so (stop strings are the caller's, since text is:
+crates/cli/src/main.rs:1328-1332,1360) or at the model's last position; it
+gives its slot back at once and the others go on. Before every decode step
+the caller's interrupt flag is looked at (crates/cli/src/main.rs:1242-1245):
+when it is set, every running sequence ends with what it has and every slot
+is given back.
+
+`max_tokens` here counts every generated token, the one the prompt's step
+gives included: the reference's chat and server loops (`for _ in
+1..max_tokens` after the first token, crates/cli/src/chat.rs:231). Its
+single-shot command line runs `for _step in 0..max_tokens` decode steps after
+the first token (crates/cli/src/main.rs:1040,1241), one token more; the
+command line here asks this loop for max_tokens + 1 to give what that gives.
 """
 import time
 from dataclasses import dataclass, field
@@ -14,8 +25,8 @@ from typing import List
 
 from ..cache import PAGE_TOKENS
 from ..errors import RequestError
-from ..sampling import (EOS, LENGTH, MAX_TOKENS, REPETITION_LOOP, STOP_TOKEN, SamplingParams,
-                        detect_repetition_loop)
+from ..sampling import (EOS, INTERRUPTED, LENGTH, MAX_TOKENS, REPETITION_LOOP, STOP_TOKEN,
+                        SamplingParams, detect_repetition_loop)
 from .batch import StepEntry
 
 
@@ -90,9 +101,12 @@ class Generator:
         self.make_chooser = make_chooser
         self.stats = GenerationStats()
 
-    def generate(self, prompts, params=None, on_token=None):
+    def generate(self, prompts, params=None, on_token=None, interrupt=None):
         """One GenerationResult per prompt (a list of token ids), in the prompts' order.
-        on_token(request index, token) is called for every generated token."""
+        on_token(request index, token) is called for every generated token; if it returns a
+        string, the sequence ends there with that stop reason (the token is kept). `interrupt()`
+        is asked before every decode step and before every batch: once it is true, running
+        sequences end with reason "interrupted" and requests not yet started return no tokens."""
         params = params or SamplingParams()
         params.validate()
         eng = self.engine
@@ -104,11 +118,15 @@ class Generator:
         results = [None] * len(prompts)
         self.stats = GenerationStats()
         for members in batches:
-            self._run_batch(members, prompts, params, chooser, results, on_token)
+            if interrupt is not None and interrupt():
+                for i in members:
+                    results[i] = GenerationResult([], INTERRUPTED, len(prompts[i]))
+                continue
+            self._run_batch(members, prompts, params, chooser, results, on_token, interrupt)
             self.stats.batches += 1
         return results
 
-    def _run_batch(self, members, prompts, params, chooser, results, on_token):
+    def _run_batch(self, members, prompts, params, chooser, results, on_token, interrupt=None):
         eng = self.engine
         eos = eng.spec.eos_token_id
         slots = {i: eng.alloc_slot() for i in members}
@@ -132,13 +150,17 @@ class Generator:
                 for i, tok in zip(list(live), tokens):
                     generated[i].append(int(tok))
                     self.stats.generated_tokens += 1
-                    if on_token is not None:
-                        on_token(i, int(tok))
+                    said = on_token(i, int(tok)) if on_token is not None else None
                     reason = stop_reason(generated[i], params, eos)
+                    if reason is None and isinstance(said, str):
+                        reason = said
                     if reason is None and eng.cache.length(slots[i]) >= eng.spec.max_positions:
                         reason = LENGTH
                     if reason is not None:
                         finish(i, reason)
+                if live and interrupt is not None and interrupt():
+                    for i in list(live):
+                        finish(i, INTERRUPTED)
                 if not live:
                     break
                 entries = [StepEntry(slots[i], [generated[i][-1]], [0]) for i in live]

@@ -95,13 +95,14 @@ class Model:
         return needs
 
     # ---- one step
-    def forward(self, rt, meta, cache):
-        """float32 logits [wanted rows, vocab] (None when nothing is wanted)."""
+    def forward(self, rt, meta, cache, logits_out=None):
+        """float32 logits [wanted rows, vocab] (None when nothing is wanted); written into
+        `logits_out` if that is given (it must have exactly that shape)."""
         with ops.stream_scope():
-            return self._forward(rt, meta, cache)
+            return self._forward(rt, meta, cache, logits_out)
 
-    def _forward(self, rt, meta, cache):
-        ctx = StepContext(rt=rt, meta=meta, cache=cache)
+    def _forward(self, rt, meta, cache, logits_out=None):
+        ctx = StepContext(rt=rt, meta=meta, cache=cache, logits_out=logits_out)
         x = self.embedding.forward(ctx, meta.token_ids)
         for i, e in enumerate(self.schedule):
             ctx.entry = i

@@ -8,8 +8,51 @@ family in the reference and therefore here: per-head q/k RMSNorm on, no biases
 (loader_common.rs:978; config.rs:518-525), scale 1/sqrt(head_dim)
 (loader_common.rs:1003-1005).
 """
-from ..config import Qwen3Config, register_architecture
+from ..config import ChatFormat, Qwen3Config, register_architecture
 from ..parts import LayerSpec, ModelSpec, PartSpec, ScheduleEntry
+from ..weights.names import NameMap
+
+# The spellings under which this family's checkpoints store their tensors, as the reference's
+# loader accepts them (loader_common.rs:423-451 prefixes of vision-language and bare
+# checkpoints and the adapter suffix, :475-566 aliases of other exporters, :1469-1528 fused
+# q/k/v and gate/up tensors whose rows are cut apart).
+NAMES = NameMap(
+    prefixes=(("language_model.model.", "model."), ("language_model.", ""),
+              ("model.language_model.", "model.")),
+    bare_prefix="model.",
+    bare_starts=("embed_tokens.", "embedding_norm.", "layers.", "norm."),
+    keep_starts=("model.", "lm_head."),
+    suffixes=((".base_layer.weight", ".weight"),),
+    layer_prefix="model.layers.",
+    layer_aliases={
+        "self_attn.out_proj.weight": "self_attn.o_proj.weight",
+        "self_attn.q_layernorm.weight": "self_attn.q_norm.weight",
+        "self_attn.k_layernorm.weight": "self_attn.k_norm.weight",
+        "operator_norm.weight": "input_layernorm.weight",
+        "ffn_norm.weight": "post_attention_layernorm.weight",
+        "feed_forward.w1.weight": "mlp.gate_proj.weight",
+        "feed_forward.w3.weight": "mlp.up_proj.weight",
+        "feed_forward.w2.weight": "mlp.down_proj.weight",
+    },
+    fused={
+        "self_attn.qkv_proj.weight": ("self_attn.q_proj.weight", "self_attn.k_proj.weight",
+                                      "self_attn.v_proj.weight"),
+        "mlp.gate_up_proj.weight": ("mlp.gate_proj.weight", "mlp.up_proj.weight"),
+    },
+)
+
+
+def chatml_prompt(user_prompt, system_prompt=None):
+    """ChatML as the reference builds it for this family (crates/cli/src/main.rs:281-294)."""
+    out = ""
+    if system_prompt:
+        out += "<|im_start|>system\n" + system_prompt + "<|im_end|>\n"
+    out += "<|im_start|>user\n" + user_prompt + "<|im_end|>\n<|im_start|>assistant\n"
+    return out
+
+
+# the end-of-turn token and its id where the tokenizer lacks it (crates/cli/src/main.rs:616-619)
+CHAT = ChatFormat(chatml_prompt, end_of_turn="<|im_end|>", end_of_turn_id=151645)
 
 
 def build_spec(cfg):
@@ -61,4 +104,5 @@ def build_spec(cfg):
     )
 
 
-ARCHITECTURE = register_architecture("Qwen3ForCausalLM", Qwen3Config, build_spec, model_types=("qwen3",))
+ARCHITECTURE = register_architecture("Qwen3ForCausalLM", Qwen3Config, build_spec, model_types=("qwen3",),
+                                     name_map=NAMES, chat=CHAT, default=True)

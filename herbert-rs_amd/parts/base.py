@@ -119,6 +119,7 @@ class StepContext:
     norm_ahead: Any = None
     left: Any = None
     norm_after_block: Any = None     # set by the model: (first norm of the next entry's block, entry)
+    logits_out: Any = None           # where the head is to write, if the caller owns the logits
 
     def leave_norm(self, linear, x):
         """For a part, just before `linear` adds its last product into x: a NormedRows that product

@@ -67,6 +67,11 @@ class OutputHead(Part):
 
     def forward(self, ctx, x, rows):
         y = self.norm.forward(ctx, x, rows, name="head_normed")
-        logits = torch.empty((rows.shape[0], self.vocab_size), dtype=torch.float32, device=x.device)
+        shape = (rows.shape[0], self.vocab_size)
+        logits = ctx.logits_out
+        if logits is None:
+            logits = torch.empty(shape, dtype=torch.float32, device=x.device)
+        elif tuple(logits.shape) != shape or logits.dtype != torch.float32 or not logits.is_contiguous():
+            raise ValueError(f"the caller's logits are {tuple(logits.shape)} {logits.dtype}, the step's {shape} float32")
         self.proj.forward(y, logits)
         return logits

@@ -5,6 +5,8 @@ STOP_TOKEN = "stop_token"
 MAX_TOKENS = "max_tokens"
 REPETITION_LOOP = "repetition_loop"
 LENGTH = "length"              # the model's max_position_embeddings is reached
+STOP_SEQUENCE = "stop_sequence"  # the caller's own rule on the decoded text (crates/cli/src/main.rs:1328-1332,1360)
+INTERRUPTED = "interrupted"    # the caller's interrupt flag was set (crates/cli/src/main.rs:1242-1245)
 
 
 def detect_repetition_loop(tokens, min_pattern=6, max_pattern=100, repeats=3):

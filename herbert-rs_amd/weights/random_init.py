@@ -23,17 +23,35 @@ def _tensor_seed(seed, name):
     return int.from_bytes(digest[:8], "little") & ((1 << 63) - 1)
 
 
+def _draw_index(shape, gen, device, std, norm_std):
+    return torch.zeros(shape, dtype=torch.int32, device=device)
+
+
+def _draw_scale(shape, gen, device, std, norm_std):
+    t = torch.ones(shape, dtype=torch.float32, device=device)
+    if norm_std:
+        t += norm_std * torch.randn(shape, generator=gen, dtype=torch.float32, device=device)
+    return t
+
+
+# how a role is drawn when the need brings no initialiser of its own; "matrix" and "table" are
+# drawn below (in row blocks when large)
+ROLE_INITIALISERS = {"index": _draw_index, "scale": _draw_scale}
+
+
 def random_tensor(name, need, seed, dtype, std=0.02, norm_std=0.0, device="cpu"):
-    """One tensor for `need`, drawn in float32 on `device` and stored as `dtype`."""
+    """One tensor for `need`, drawn in float32 on `device` and stored as `dtype` (integers stay
+    int32). The need's own initialiser decides if it has one, else its role."""
     gen = torch.Generator(device=device)
     gen.manual_seed(_tensor_seed(seed, name))
-    if need.role == "index":
-        return torch.zeros(need.shape, dtype=torch.int32, device=device)
-    if need.role == "scale":
-        t = torch.ones(need.shape, dtype=torch.float32, device=device)
-        if norm_std:
-            t += norm_std * torch.randn(need.shape, generator=gen, dtype=torch.float32, device=device)
-        return t.to(dtype)
+    init = need.init or ROLE_INITIALISERS.get(need.role)
+    if init is not None:
+        t = init(tuple(need.shape), gen, device, std, norm_std)
+        if tuple(t.shape) != tuple(need.shape):
+            raise ConfigError(f"the initialiser of {name} made {list(t.shape)}, not {list(need.shape)}")
+        return t if not t.is_floating_point() else t.to(dtype)
+    if need.role not in ("matrix", "table"):
+        raise ConfigError(f"tensor {name}: role {need.role!r} has no initialiser; give the TensorNeed one")
     rows = need.shape[0]
     if device == "cpu" or rows * (need.shape[1] if len(need.shape) > 1 else 1) < (1 << 28):
         t = torch.randn(need.shape, generator=gen, dtype=torch.float32, device=device)

@@ -4,11 +4,15 @@ The files are found as the reference finds them (model.safetensors.index.json
 naming the shards by basename, else a single model.safetensors:
 bc/loader_common.rs:1131-1149, `bc/` = crates/backends/backend_common/src/).
 Tensors keep what they are stored in: bfloat16 stays bfloat16, a 32-bit float
-stays so, other floats become bfloat16, integers become int32. Names are normalised and fused q/k/v and gate/up tensors are cut
-into their parts as the reference's loader does (bc/loader_common.rs:423-451, 475-566, 1469-1528). Unlike the
-reference, which ignores unknown names and does not check plain shapes
-(bc/loader_common.rs:679-685), every problem is collected and reported in one
-error: missing names, unexpected names and wrong shapes.
+stays so, other floats become bfloat16, integers become int32. How stored
+names are spelled and which tensors are fused is the architecture's NameMap
+(weights/names.py); the reader applies it and knows no spelling itself.
+Stored tensors that the model does not ask for are passed over, as the
+reference passes them over (bc/loader_common.rs:679-685,1588: rotary
+inv_freq buffers, a stored head beside tied embeddings, :1851-1872); with
+`strict=True` they are an error too. Unlike the reference, which does not
+check plain shapes, every other problem is collected and reported in one
+error: missing names, wrong shapes or dtypes, names stored twice.
 """
 import json
 import os
@@ -17,59 +21,7 @@ import torch
 from safetensors import safe_open
 
 from ..errors import ModelLoadError
-
-# ---- names as the reference's loader normalises them (bc/loader_common.rs:423-451, 475-566)
-_ALIASES = {
-    "self_attn.out_proj.weight": "self_attn.o_proj.weight",
-    "self_attn.q_layernorm.weight": "self_attn.q_norm.weight",
-    "self_attn.k_layernorm.weight": "self_attn.k_norm.weight",
-    "operator_norm.weight": "input_layernorm.weight",
-    "ffn_norm.weight": "post_attention_layernorm.weight",
-    "feed_forward.w1.weight": "mlp.gate_proj.weight",
-    "feed_forward.w3.weight": "mlp.up_proj.weight",
-    "feed_forward.w2.weight": "mlp.down_proj.weight",
-}
-# fused tensors and the tensors their rows are cut into, in order (bc/loader_common.rs:1469-1528)
-_FUSED = {
-    "self_attn.qkv_proj.weight": ("self_attn.q_proj.weight", "self_attn.k_proj.weight",
-                                  "self_attn.v_proj.weight"),
-    "mlp.gate_up_proj.weight": ("mlp.gate_proj.weight", "mlp.up_proj.weight"),
-}
-
-
-def canonical_name(name):
-    """A stored tensor's name in the form the models ask for: `model.` prefix variants of
-    vision-language and bare checkpoints, the `.base_layer.weight` suffix and the aliases of
-    other exporters are brought to the one spelling."""
-    if name.startswith("language_model.model."):
-        name = "model." + name[len("language_model.model."):]
-    elif name.startswith("language_model."):
-        name = name[len("language_model."):]
-    elif name.startswith("model.language_model."):
-        name = "model." + name[len("model.language_model."):]
-    elif not name.startswith(("model.", "lm_head.")) and \
-            name.startswith(("embed_tokens.", "embedding_norm.", "layers.", "norm.")):
-        name = "model." + name
-    if name.endswith(".base_layer.weight"):
-        name = name[:-len(".base_layer.weight")] + ".weight"
-    if name.startswith("model.layers."):
-        head, _, rest = name[len("model.layers."):].partition(".")
-        if rest in _ALIASES:
-            name = f"model.layers.{head}.{_ALIASES[rest]}"
-    return name
-
-
-def _fused_targets(name, needs):
-    """For a fused tensor's (canonical) name: the names its rows are cut into, if the model asks
-    for all of them; else None."""
-    for suffix, parts in _FUSED.items():
-        if name.endswith("." + suffix):
-            prefix = name[:-len(suffix)]
-            targets = [prefix + p for p in parts]
-            if all(t in needs for t in targets):
-                return targets
-    return None
-
+from .names import AS_STORED
 
 _FLOATS = (torch.float16, torch.float64)
 _INTS = (torch.int8, torch.int16, torch.int64, torch.uint8)
@@ -102,14 +54,18 @@ def stored_dtype(t):
     raise ModelLoadError(f"unsupported dtype {t.dtype}")
 
 
-def read_tensors(folder, needs, device="cpu"):
+def read_tensors(folder, needs, device="cpu", name_map=None, strict=False, ignored=None):
     """dict name -> tensor on `device` for exactly the names in `needs`.
 
-    `needs` maps a name to a TensorNeed. Raises one ModelLoadError that lists
-    every missing name, every unexpected name and every wrong shape.
+    `needs` maps a name to a TensorNeed; `name_map` is the architecture's NameMap (default: names
+    as stored). Raises one ModelLoadError that lists every missing name, every wrong shape and
+    every name stored twice. Stored tensors nobody asks for are skipped and their names appended
+    to `ignored` (a list, if given); with `strict` they are listed in the error as unexpected.
     """
+    name_map = name_map or AS_STORED
     found = {}
-    unexpected = []
+    unexpected = ignored if ignored is not None else []
+    del unexpected[:]
     wrong = []
     duplicate = []
     for path in shard_files(folder):
@@ -119,8 +75,8 @@ def read_tensors(folder, needs, device="cpu"):
             raise ModelLoadError(f"cannot read {path}: {e}") from None
         with handle as f:
             for stored in f.keys():
-                name = canonical_name(stored)
-                targets = None if name in needs else _fused_targets(name, needs)
+                name = name_map.canonical(stored)
+                targets = None if name in needs else name_map.fused_targets(name, needs)
                 if name not in needs and targets is None:
                     unexpected.append(stored)
                     continue
@@ -154,6 +110,8 @@ def read_tensors(folder, needs, device="cpu"):
                         found[n] = t[row:row + rows].contiguous().to(device)
                         row += rows
     missing = [n for n in needs if n not in found]
+    if not strict:
+        unexpected = []
     if missing or unexpected or wrong or duplicate:
         parts = [f"weights in {folder} do not fit the configuration:"]
         if missing:
@@ -168,19 +126,20 @@ def read_tensors(folder, needs, device="cpu"):
     return found
 
 
-def read_tensor(folder, name, needs):
+def read_tensor(folder, name, needs, name_map=None):
     """The one tensor `name` of `needs` as `folder` stores it (cut out of a fused tensor if that is
     how it is stored), on the CPU."""
+    name_map = name_map or AS_STORED
     if name not in needs:
         raise ModelLoadError(f"the model has no tensor {name!r}; it has: " + ", ".join(sorted(needs)))
     for path in shard_files(folder):
         with safe_open(path, framework="pt", device="cpu") as f:
             for stored in f.keys():
-                cname = canonical_name(stored)
+                cname = name_map.canonical(stored)
                 if cname == name:
                     t = f.get_tensor(stored)
                     return t.to(stored_dtype(t))
-                targets = _fused_targets(cname, needs)
+                targets = name_map.fused_targets(cname, needs)
                 if targets and name in targets:
                     t = f.get_tensor(stored)
                     row = sum(needs[n].shape[0] for n in targets[:targets.index(name)])

@@ -1,0 +1,37 @@
+"""How close the engine's logits must be to the plain implementation's.
+
+float32: the reference's own arithmetic in another order, so rounding only: an absolute bound.
+bfloat16: activations, cache and probabilities are rounded to 8 bits of mantissa at about ten
+places a layer; the error is measured against the root mean square of the plain logits of the
+row, and the bound for a model is about twice the worst that its tests have been seen to give
+(the worst of every run is printed after the tests). A fault that moves a few per cent of one
+probability mass to a wrong key (a page's edge, a window's edge, a stale slot) shifts logits by
+more than that.
+"""
+import numpy as np
+
+from .conftest import observe
+
+F32_ABS = 1e-4
+# worst seen relative to the row's rms, by configuration (tests/tiny.py), times about two
+BF16_REL_L2 = {"A": 0.05, "B": 0.05, "C": 0.05, "D": 0.05, "wide": 0.05, "odd": 0.05}
+BF16_REL_RMS = {"A": 0.05, "B": 0.05, "C": 0.05, "D": 0.05, "wide": 0.05, "odd": 0.05}
+
+
+def rel_rms_error(got, ref):
+    """(largest absolute error, the same over the row's rms, rms of the error over the row's rms)."""
+    diff = got.astype(np.float64) - ref.astype(np.float64)
+    err = float(np.abs(diff).max())
+    rms = max(float(np.sqrt((ref.astype(np.float64) ** 2).mean())), 1e-30)
+    return err, err / rms, float(np.sqrt((diff ** 2).mean())) / rms
+
+
+def close(got, ref, dtype, config, label=None):
+    """(ok, error): the error is absolute in float32 and relative to the row's rms in bfloat16."""
+    err, rel, rel_l2 = rel_rms_error(got, ref)
+    if dtype == "float32":
+        observe(f"float32 {config} {label or ''} abs", err)
+        return err <= F32_ABS, err
+    observe(f"bfloat16 {config} {label or ''} max / rms", rel)
+    observe(f"bfloat16 {config} {label or ''} rms / rms", rel_l2)
+    return rel <= BF16_REL_RMS[config] and rel_l2 <= BF16_REL_L2[config], max(rel, rel_l2)

@@ -97,8 +97,10 @@ def decoder_layer(x, positions, cfg, w, layer):
     return x
 
 
-def forward(cfg, w, tokens, start_pos=0):
-    """Logits [T, V] at every position of one whole sequence.
+def forward(cfg, w, tokens, start_pos=0, rows=None):
+    """Logits [T, V] at every position of one whole sequence, or, with `rows`, at those positions
+    only: the final norm and the head then run on those rows alone, as the reference runs them
+    on the rows it needs (bc/generic_model.rs:269-274).
 
     Embedding without multiplier (bc/generic_model.rs:163-175), the layers in
     order (:203-219), final RMSNorm and lm_head (:266-283); the head is the
@@ -112,6 +114,8 @@ def forward(cfg, w, tokens, start_pos=0):
     x = ops.embedding(tokens, w["model.embed_tokens.weight"]).to(dtype)
     for layer in range(cfg["num_hidden_layers"]):
         x = decoder_layer(x, positions, cfg, w, layer)
+    if rows is not None:
+        x = x[list(rows)]
     x = ops.rms_norm(x, w["model.norm.weight"], cfg.get("rms_norm_eps", 1e-5))
     head = w["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings", True) \
         else w["lm_head.weight"]

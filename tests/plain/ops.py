@@ -38,11 +38,19 @@ def rms_norm(x, weight, eps):
     return x * inv_rms * weight
 
 
+# Above this many multiply-adds (or query-key pairs) a formula is handed to torch's matrix
+# product on the CPU instead of the loop that spells it out: the same sums, in the library's
+# order. test_plain checks that both ways agree; the loops stay the definition.
+WHOLE_FROM = 1 << 24
+
+
 def linear(x, weight):
     """C[m, n] = sum_k A[m, k] * W[n, k]; weights are [out, in], no bias.
 
     crates/backends/backend_bf16/src/kernels.rs:154-164.
     """
+    if x.shape[0] * weight.shape[0] * weight.shape[1] > WHOLE_FROM:
+        return x @ weight.T
     out = torch.zeros(x.shape[0], weight.shape[0], dtype=x.dtype)
     for n in range(weight.shape[0]):
         out[:, n] = (x * weight[n]).sum(-1)
@@ -156,6 +164,19 @@ def causal_attention(q, k, v, positions, scale=None, window=None):
     if scale is None:
         scale = 1.0 / math.sqrt(hd)
     out = torch.zeros_like(q)
+    if T * T * nq > WHOLE_FROM:
+        # every query of a head at once: scores [T, T], keys out of sight at -inf
+        pos = torch.as_tensor(list(positions))
+        seen = pos[None, :] <= pos[:, None]
+        if window is not None:
+            seen &= pos[None, :] > pos[:, None] - window
+        for h in range(nq):
+            g = h // group
+            s = (q[:, h] @ k[:, g].T) * scale
+            s = s.masked_fill(~seen, float("-inf"))
+            e = torch.exp(s - s.max(-1, keepdim=True).values)
+            out[:, h] = (e / e.sum(-1, keepdim=True)) @ v[:, g]
+        return out
     for h in range(nq):
         g = h // group
         for i in range(T):

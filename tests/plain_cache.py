@@ -19,6 +19,24 @@ def plain_logits(folder, tokens):
     return _logits[key]
 
 
+def plain_rows(folder, tokens, rows):
+    """{position: float32 logits [vocab]} at `rows` only (for models whose vocabulary makes every
+    position's logits too much to keep)."""
+    if folder not in _folders:
+        _folders[folder] = plain_model.read_folder(folder, torch.float32)
+    cfg, w = _folders[folder]
+    rows = sorted(set(rows))
+    out = plain_model.forward(cfg, w, list(tokens), rows=rows).numpy().astype(np.float32)
+    return {p: out[i] for i, p in enumerate(rows)}
+
+
+def forget(folder):
+    """Drop a folder's weights and logits (large models)."""
+    _folders.pop(folder, None)
+    for key in [k for k in _logits if k[0] == folder]:
+        del _logits[key]
+
+
 def plain_folder(folder):
     if folder not in _folders:
         _folders[folder] = plain_model.read_folder(folder, torch.float32)

@@ -9,8 +9,8 @@ import torch
 from herbert_rs_amd.cache import Cache, FreeList, KVNeed, StateNeed, pages_for
 from herbert_rs_amd.engine.generate import Generator, plan_batches, stop_reason
 from herbert_rs_amd.errors import CacheError, RequestError
-from herbert_rs_amd.sampling import (EOS, LENGTH, MAX_TOKENS, REPETITION_LOOP, STOP_TOKEN,
-                                     SamplingParams, detect_repetition_loop)
+from herbert_rs_amd.sampling import (EOS, INTERRUPTED, LENGTH, MAX_TOKENS, REPETITION_LOOP,
+                                     STOP_SEQUENCE, STOP_TOKEN, SamplingParams, detect_repetition_loop)
 from herbert_rs_amd.sampling import xorshift
 
 
@@ -212,11 +212,11 @@ class ArgmaxChooser:
         return [int(r.argmax()) for r in logits]
 
 
-def run(prompts, engine=None, **kw):
+def run(prompts, engine=None, on_token=None, interrupt=None, **kw):
     engine = engine or FakeEngine()
     gen = Generator(engine, max_batch=kw.pop("max_batch", 4), make_chooser=ArgmaxChooser)
     params = SamplingParams(temperature=0.0, **kw)
-    return engine, gen, gen.generate(prompts, params)
+    return engine, gen, gen.generate(prompts, params, on_token, interrupt)
 
 
 def test_stops_eos_max_tokens_stop_token_and_order():
@@ -232,7 +232,76 @@ def test_stops_eos_max_tokens_stop_token_and_order():
     assert gen.stats.generated_tokens == 7 and gen.stats.decode_steps == 3 and gen.stats.prompt_tokens == 5
 
 
+def test_the_interrupt_flag_is_looked_at_before_every_decode_step():
+    """crates/cli/src/main.rs:1242-1245: the flag ends the loop between two steps; what was
+    generated stays, every slot comes back, batches not yet started do not start."""
+    asked = []
+
+    def interrupt():
+        asked.append(1)
+        return len(asked) > 3        # true when asked the fourth time
+
+    eng, gen, res = run([[10], [20], [30]], max_tokens=20, max_batch=2, repeat_check=False,
+                        interrupt=interrupt)
+    # asked before the batch, then before decode steps 1, 2 and 3: two decode steps ran
+    assert res[0].tokens == [11, 12, 13] and res[1].tokens == [21, 22, 23]
+    assert res[0].stop_reason == res[1].stop_reason == INTERRUPTED
+    assert res[2].tokens == [] and res[2].stop_reason == INTERRUPTED
+    assert len(eng.steps) == 3 and eng.cache.slots.held_count == 0
+    # set during the prompt's step: the token of that step is kept; a sequence that has ended
+    # by itself keeps its own reason
+    calls = []
+    _, _, res = run([[7], [8]], max_tokens=20, repeat_check=False,
+                    interrupt=lambda: calls.append(1) or len(calls) > 1)
+    assert res[0].stop_reason == INTERRUPTED and res[0].tokens == [8]
+    assert res[1].stop_reason == EOS and res[1].tokens == [9]
+
+
+def test_the_caller_ends_a_sequence_from_on_token():
+    """Stop strings are matched by whoever has the text (crates/cli/src/main.rs:1328-1332,1360):
+    on_token's answer ends that sequence, the token stays in the output, the others go on."""
+    def on_token(i, tok):
+        return STOP_SEQUENCE if (i == 1 and tok == 23) else None
+    eng, _, res = run([[10], [20]], max_tokens=5, repeat_check=False, on_token=on_token)
+    assert res[1].tokens == [21, 22, 23] and res[1].stop_reason == STOP_SEQUENCE
+    assert res[0].tokens == [11, 12, 13, 14, 15] and res[0].stop_reason == MAX_TOKENS
+    assert eng.steps[3] == [(0, 1)] and eng.cache.slots.held_count == 0
+    # the loop's own rules come first: eos on the same token is eos
+    _, _, res = run([[7]], max_tokens=5, repeat_check=False, on_token=lambda i, t: STOP_SEQUENCE)
+    assert res[0].tokens == [8] and res[0].stop_reason == STOP_SEQUENCE
+    _, _, res = run([[8]], max_tokens=5, repeat_check=False, on_token=lambda i, t: STOP_SEQUENCE)
+    assert res[0].tokens == [9] and res[0].stop_reason == EOS
+
+
+def test_a_step_that_does_not_fit_takes_no_page():
+    """All the pages of a step or none: the third sequence's pages do not fit, and the first
+    two hold afterwards exactly what they held before."""
+    c = make_cache(max_tokens=64 * 4)
+    a, b, d = c.alloc_slot(), c.alloc_slot(), c.alloc_slot()
+    c.reserve_all([(a, 60), (b, 10)])
+    c.commit(a, 60); c.commit(b, 10)
+    before = {k: (g.pages.held_count, g.table_host.copy()) for k, g in c.kv_groups.items()}
+    with pytest.raises(CacheError, match="needs 4 more pages"):
+        c.reserve_all([(a, 10), (b, 60), (d, 70)])       # 1 + 1 + 2 pages, 2 free
+    for k, g in c.kv_groups.items():
+        assert g.pages.held_count == before[k][0] and (g.table_host == before[k][1]).all()
+    c.check()
+    with pytest.raises(CacheError, match="exceed"):
+        c.reserve_all([(a, 1), (b, 600)])
+    c.reserve_all([(a, 10), (b, 60)])                    # this fits: 2 pages
+    assert all(g.pages.free_count == 0 for g in c.kv_groups.values())
+    c.unreserve(a); c.unreserve(b)                       # the step did not run
+    for k, g in c.kv_groups.items():
+        assert g.pages.held_count == before[k][0] and (g.table_host == before[k][1]).all()
+    assert c.length(a) == 60 and c.length(b) == 10
+    c.check()
+
+
 def test_max_tokens_counts_the_first_token_and_ignore_eos():
+    """The loop's max_tokens is the number of tokens that come out, the prompt step's token
+    included (crates/cli/src/chat.rs:231 `for _ in 1..max_tokens` after the first token). The
+    single-shot command line counts decode steps after that token
+    (crates/cli/src/main.rs:1040,1241) and therefore asks the loop for one more."""
     _, _, res = run([[5]], max_tokens=3, repeat_check=False)
     assert res[0].tokens == [6, 7, 8] and res[0].stop_reason == MAX_TOKENS
     _, _, res = run([[7]], max_tokens=4, ignore_eos=True, repeat_check=False)

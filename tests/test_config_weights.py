@@ -171,21 +171,39 @@ def test_one_error_lists_missing_unexpected_and_wrong(model_root, tmp_path):
     with open(tmp_path / "config.json", "w") as f:
         json.dump(TINY_A, f)
     with pytest.raises(ModelLoadError) as err:
-        read_tensors(str(tmp_path), needs_of(TINY_A))
+        read_tensors(str(tmp_path), needs_of(TINY_A), strict=True)
     text = str(err.value)
     assert "missing (2)" in text and "model.layers.1.self_attn.q_norm.weight" in text
     assert "model.norm.weight" in text
     assert "unexpected (1)" in text and "rotary_emb.inv_freq" in text
     assert "gate_proj.weight: expected [128, 64], got [128, 63]" in text
-
-
-def test_tied_model_refuses_a_stray_head_and_untied_needs_one(model_root, tmp_path):
-    src = make_folder(model_root, "A", "float32")
-    tensors = load_file(os.path.join(src, "model.safetensors"))
-    tensors["lm_head.weight"] = torch.zeros(256, 64)
-    save_file(tensors, str(tmp_path / "model.safetensors"))
-    with pytest.raises(ModelLoadError, match="unexpected"):
+    # without `strict` the stray tensor is no fault, the others still are, in one error
+    with pytest.raises(ModelLoadError) as err:
         read_tensors(str(tmp_path), needs_of(TINY_A))
+    text = str(err.value)
+    assert "missing (2)" in text and "expected [128, 64], got [128, 63]" in text
+    assert "unexpected" not in text and "inv_freq" not in text
+
+
+def test_unknown_names_are_passed_over_and_an_untied_model_needs_its_head(model_root, tmp_path):
+    """Tensors nobody asks for are ignored as the reference ignores them
+    (crates/backends/backend_common/src/loader_common.rs:679-685,1588): rotary buffers, and a
+    stored head beside tied embeddings, which the reference drops for the embedding
+    (loader_common.rs:1851-1872)."""
+    src = make_folder(model_root, "A", "float32")
+    plain = load_file(os.path.join(src, "model.safetensors"))
+    tensors = dict(plain)
+    tensors["lm_head.weight"] = torch.full((256, 64), 9.0)
+    tensors["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(8)
+    tensors["model.layers.1.self_attn.rotary_emb.inv_freq"] = torch.zeros(8)
+    save_file(tensors, str(tmp_path / "model.safetensors"))
+    ignored = []
+    got = read_tensors(str(tmp_path), needs_of(TINY_A), ignored=ignored)
+    assert set(got) == set(plain) and all(torch.equal(got[k], plain[k]) for k in plain)
+    assert sorted(ignored) == ["lm_head.weight", "model.layers.0.self_attn.rotary_emb.inv_freq",
+                               "model.layers.1.self_attn.rotary_emb.inv_freq"]
+    with pytest.raises(ModelLoadError, match=r"unexpected \(3\)"):
+        read_tensors(str(tmp_path), needs_of(TINY_A), strict=True)
     with pytest.raises(ModelLoadError, match="lm_head.weight"):
         read_tensors(src, needs_of(dict(TINY_A, tie_word_embeddings=False)))
 
@@ -218,7 +236,8 @@ def test_bf16_conversion_bits():
 def test_names_are_normalised_and_fused_tensors_cut(model_root, tmp_path):
     """The spellings the reference's loader accepts (bc/loader_common.rs:423-451, 475-566) and its
     fused q/k/v and gate/up tensors (:1469-1528) give the same weights as the plain names."""
-    from herbert_rs_amd.weights.store import canonical_name
+    from herbert_rs_amd.models.qwen3 import NAMES
+    canonical_name = NAMES.canonical
     assert canonical_name("language_model.model.layers.0.mlp.up_proj.weight") == "model.layers.0.mlp.up_proj.weight"
     assert canonical_name("language_model.lm_head.weight") == "lm_head.weight"
     assert canonical_name("model.language_model.norm.weight") == "model.norm.weight"
@@ -242,15 +261,72 @@ def test_names_are_normalised_and_fused_tensors_cut(model_root, tmp_path):
         other[f"model.language_model.layers.{l}.mlp.gate_up_proj.weight"] = torch.cat(
             [plain[p + "mlp.gate_proj.weight"], plain[p + "mlp.up_proj.weight"]], 0)
     save_file(other, str(tmp_path / "model.safetensors"))
-    got = read_tensors(str(tmp_path), needs_of(TINY_B))
+    got = read_tensors(str(tmp_path), needs_of(TINY_B), name_map=NAMES)
     assert set(got) == set(plain) and all(torch.equal(got[k], plain[k]) for k in plain)
+    # the spellings are the architecture's: the reader alone takes names as they are stored
+    with pytest.raises(ModelLoadError, match="missing"):
+        read_tensors(str(tmp_path), needs_of(TINY_B))
+    assert resolve_architecture(TINY_B).name_map is NAMES
     # one tensor by its own name, also out of a fused one
     from herbert_rs_amd.weights import read_tensor
     for name in ("model.layers.2.self_attn.k_proj.weight", "model.layers.1.mlp.up_proj.weight", "model.norm.weight"):
-        assert torch.equal(read_tensor(str(tmp_path), name, needs_of(TINY_B)), plain[name])
+        assert torch.equal(read_tensor(str(tmp_path), name, needs_of(TINY_B), NAMES), plain[name])
     with pytest.raises(ModelLoadError, match="no tensor"):
-        read_tensor(str(tmp_path), "model.layers.9.mlp.up_proj.weight", needs_of(TINY_B))
+        read_tensor(str(tmp_path), "model.layers.9.mlp.up_proj.weight", needs_of(TINY_B), NAMES)
     other["model.language_model.layers.0.self_attn.qkv_proj.weight"] = torch.zeros(10, 96)
     save_file(other, str(tmp_path / "model.safetensors"))
     with pytest.raises(ModelLoadError, match=r"qkv_proj.weight: expected \[320, 96\], got \[10, 96\]"):
-        read_tensors(str(tmp_path), needs_of(TINY_B))
+        read_tensors(str(tmp_path), needs_of(TINY_B), name_map=NAMES)
+
+
+def test_an_architecture_brings_its_own_names_default_and_initialisers(tmp_path):
+    """What is particular to an architecture sits in its registry entry: the spellings of its
+    checkpoints, whether it is the one taken when config.json names none, its chat format; and a
+    tensor of a kind the library does not know (here a bias) brings its own random initialiser."""
+    from herbert_rs_amd.config import ChatFormat, register_architecture
+    from herbert_rs_amd.config import registry
+    from herbert_rs_amd.weights import TensorNeed, random_tensors
+    from herbert_rs_amd.weights.names import NameMap
+
+    def small_bias(shape, gen, device, std, norm_std):
+        return 0.5 + 0.01 * torch.randn(shape, generator=gen, dtype=torch.float32, device=device)
+
+    needs = {"h.0.w": TensorNeed((4, 6)), "h.0.b": TensorNeed((4,), "bias", init=small_bias),
+             "wte": TensorNeed((10, 6), "table"), "ln": TensorNeed((6,), "scale")}
+    t = random_tensors(needs, 5, "bfloat16", std=0.02, norm_std=0.0)
+    assert t["h.0.b"].dtype == torch.bfloat16 and abs(float(t["h.0.b"].float().mean()) - 0.5) < 0.05
+    assert float(t["ln"].float().min()) == 1.0 and float(t["h.0.w"].float().abs().max()) < 0.2
+    with pytest.raises(ConfigError, match="no initialiser"):
+        random_tensors({"x": TensorNeed((3,), "bias")}, 0)
+    with pytest.raises(ConfigError, match="made"):
+        random_tensors({"x": TensorNeed((3,), "bias", init=lambda *a: torch.zeros(2))}, 0)
+
+    names = NameMap(prefixes=(("transformer.", ""),), layer_prefix="h.",
+                    layer_aliases={"weight": "w", "bias": "b"}, fused={})
+    assert names.canonical("transformer.h.0.weight") == "h.0.w"
+    assert names.canonical("transformer.wte") == "wte" and names.canonical("other") == "other"
+    save_file({"transformer.h.0.weight": t["h.0.w"], "transformer.h.0.bias": t["h.0.b"],
+               "transformer.wte": t["wte"], "ln": t["ln"], "transformer.extra": torch.zeros(1)},
+              str(tmp_path / "model.safetensors"))
+    ignored = []
+    got = read_tensors(str(tmp_path), needs, name_map=names, ignored=ignored)
+    assert all(torch.equal(got[k], t[k]) for k in needs) and ignored == ["transformer.extra"]
+
+    saved = (dict(registry._ARCHITECTURES), dict(registry._MODEL_TYPES), list(registry._DEFAULT))
+    try:
+        chat = ChatFormat(lambda user, system=None: f"[{system or ''}|{user}]", "<eot>", 3)
+        arch = register_architecture("ToyLM", dict, lambda cfg: None, ("toy",), name_map=names, chat=chat)
+        assert resolve_architecture({"model_type": "toy"}) is arch and arch.name_map is names
+        assert arch.chat.build_prompt("hi") == "[|hi]" and arch.chat.end_of_turn_id == 3
+        assert resolve_architecture({}).name == "Qwen3ForCausalLM"      # registered as the default
+        registry._DEFAULT[:] = []
+        with pytest.raises(ConfigError, match="names neither"):
+            resolve_architecture({})
+    finally:
+        registry._ARCHITECTURES.clear(); registry._ARCHITECTURES.update(saved[0])
+        registry._MODEL_TYPES.clear(); registry._MODEL_TYPES.update(saved[1])
+        registry._DEFAULT[:] = saved[2]
+    qwen = resolve_architecture({"model_type": "qwen3"})
+    assert qwen.chat.end_of_turn == "<|im_end|>" and qwen.chat.end_of_turn_id == 151645
+    assert qwen.chat.build_prompt("Hi", "Be brief") == \
+        "<|im_start|>system\nBe brief<|im_end|>\n<|im_start|>user\nHi<|im_end|>\n<|im_start|>assistant\n"

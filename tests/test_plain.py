@@ -120,6 +120,24 @@ def test_attention_matches_library(nq, nkv):
     assert torch.allclose(got, want, atol=1e-5)
 
 
+def test_large_inputs_take_the_library_s_product_and_say_the_same(monkeypatch):
+    """Beyond ops.WHOLE_FROM multiply-adds the product and the attention scores go through
+    torch's matrix product on the CPU: the same sums as the loops that define them, a window and
+    positions that do not start at zero included."""
+    x, w = rand(7, 24, seed=31), rand(40, 24, seed=32)
+    T, nq, nkv, hd = 37, 6, 2, 8
+    q, k, v = rand(T, nq, hd, seed=33), rand(T, nkv, hd, seed=34), rand(T, nkv, hd, seed=35)
+    positions = list(range(5, 5 + T))
+    slow = (ops.linear(x, w), ops.causal_attention(q, k, v, positions),
+            ops.causal_attention(q, k, v, positions, window=9))
+    monkeypatch.setattr(ops, "WHOLE_FROM", 0)
+    fast = (ops.linear(x, w), ops.causal_attention(q, k, v, positions),
+            ops.causal_attention(q, k, v, positions, window=9))
+    for a, b in zip(slow, fast):
+        assert torch.allclose(a, b, atol=2e-6) and not torch.equal(a, torch.zeros_like(a))
+    assert not torch.allclose(fast[1], fast[2], atol=1e-3)          # the window is not lost on the way
+
+
 def test_attention_special_cases():
     hd = 4
     v = rand(5, 1, hd, seed=14)
@@ -243,6 +261,14 @@ def test_tied_head_and_separate_head():
     assert torch.allclose(pm.forward(CFG, sep, [1, 2, 3]), 2 * a, atol=1e-5)
 
 
+def test_logits_at_chosen_rows_only():
+    w = tiny_weights(CFG)
+    tokens = [3, 9, 27, 1, 43, 5]
+    whole = pm.forward(CFG, w, tokens)
+    some = pm.forward(CFG, w, tokens, rows=[0, 4, 5])
+    assert torch.equal(some, whole[[0, 4, 5]])
+
+
 def test_causality_of_the_whole_model():
     w = tiny_weights(CFG)
     a = pm.forward(CFG, w, [4, 8, 15, 16, 23])
@@ -267,6 +293,24 @@ def test_xorshift_vector_by_hand():
     assert ps.XorShift64(0).state == 0xDEADBEEF
     r = ps.XorShift64(7).next_f32()
     assert 0.0 <= r < 1.0
+    # The draw (crates/core/src/sampler.rs:58-62): the upper 24 bits of the new state over 2^24,
+    # cut and not rounded. By hand, from the state 2^63 + 2^36 + 2^33:
+    #   x ^= x << 13  (2^76 is lost)           -> 2^63 + 2^49 + 2^46 + 2^36 + 2^33
+    #   x ^= x >> 7                            -> ... + 2^56 + 2^42 + 2^39 + 2^29 + 2^26
+    #   x ^= x << 17  (2^80, 2^73, 2^66 lost; 2^63, 2^56, 2^46 meet their like and cancel)
+    #      = 2^59 + 2^53 + 2^50 + 2^49 + 2^43 + 2^42 + 2^39 + 2^36 + 2^33 + 2^29 + 2^26
+    #   x >> 40 = 2^19 + 2^13 + 2^10 + 2^9 + 2^3 + 2^2 = 534028
+    # Bits 39 and 36 lie below the cut: a draw that kept 32 bits and let the conversion to
+    # float32 round would give 534029 / 2^24.
+    rng = ps.XorShift64((1 << 63) + (1 << 36) + (1 << 33))
+    r = rng.next_f32()
+    assert rng.state == 0x08260C9224000000
+    assert r.dtype == np.float32 and float(r) == 534028.0 / 16777216.0
+    assert float(r) != float(np.float32(rng.state >> 32) / np.float32(2.0 ** 32))
+    # the engine's host copy of the generator, which seeds the GPU sampler, says the same
+    from herbert_rs_amd.sampling import xorshift
+    state = xorshift.step((1 << 63) + (1 << 36) + (1 << 33))
+    assert state == 0x08260C9224000000 and xorshift.to_unit(state) == 534028.0 / 16777216.0
 
 
 def test_sampler_reductions_to_argmax():
@@ -298,6 +342,18 @@ def test_sampler_top_k_and_top_p_sets():
     # probabilities 0.51, 0.19, 0.19, ...: the prefix reaching 0.6 is two tokens
     assert [i for i, _ in work] == [0, 2]
     assert abs(sum(float(p) for _, p in work) - 1.0) < 1e-6
+    # the prefix ends where the running sum is >= top_p, not > (crates/core/src/sampler.rs:117-121):
+    # logits ln 2, 0, 0 give exactly 0.5, 0.25, 0.25 in float32, and with top_p 0.75 the sum
+    # meets top_p at the second token; a strict comparison would keep all three
+    exact = np.log(np.array([2.0, 1.0, 1.0])).astype(np.float32)
+    probs = ps.candidates(exact, 1.0, 0, 1.0)
+    assert [float(p) for _, p in probs] == [0.5, 0.25, 0.25]
+    work = ps.candidates(exact, 1.0, 0, 0.75)
+    assert [i for i, _ in work] == [0, 1]
+    assert [float(p) for _, p in work] == [np.float32(0.5) / np.float32(0.75), np.float32(0.25) / np.float32(0.75)]
+    assert [i for i, _ in ps.candidates(exact, 1.0, 0, 0.7500001)] == [0, 1, 2]
+    # the same edge where no exponential's rounding can blur it: four equal logits, top_p 0.5
+    assert [(i, float(p)) for i, p in ps.candidates(np.full(4, 1.25, np.float32), 1.0, 0, 0.5)] == [(0, 0.5), (1, 0.5)]
 
 
 def test_repetition_detector():

@@ -1,0 +1,314 @@
+"""Schedules beyond a batch that starts together: a step that carries running sequences' single
+tokens beside a new sequence's whole prompt, a roll-back followed by other tokens, a step that
+does not fit, checkpoints with tensors nobody asks for, many decode graphs, stop strings."""
+import json
+import os
+import signal
+import subprocess
+import sys
+import time
+
+import numpy as np
+import pytest
+import torch
+
+import herbert_rs_amd as hb
+from herbert_rs_amd.engine import StepEntry
+from herbert_rs_amd.errors import CacheError
+
+from .bounds import close
+from .plain import model as plain
+from .plain_cache import plain_folder, plain_logits
+from .tiny import CONFIGS, make_folder, random_tokens
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["B", "D"])
+def test_decoding_sequences_and_a_new_prompt_in_one_step(name, dtype, model_root):
+    """Continuous batching's shape: two sequences that have run for a while bring one token each,
+    in the same step as the whole prompt of a sequence that starts, and as a piece of a prompt that
+    was begun before. Every logit is the one the sequence gets alone."""
+    folder = make_folder(model_root, name, dtype)
+    raw = CONFIGS[name][0]
+    vocab = raw["vocab_size"]
+    long_n = 200 if name == "B" else 900
+    a, b = random_tokens(vocab, long_n + 6, 201), random_tokens(vocab, 70 + 6, 202)
+    c, d = random_tokens(vocab, 97 + 3, 203), random_tokens(vocab, 130, 204)
+    ref = {k: plain_logits(folder, t) for k, t in (("a", a), ("b", b), ("c", c), ("d", d))}
+    engine = hb.load(folder, dtype=dtype, cache_tokens=64 * 40)
+    sa, sb = engine.alloc_slot(), engine.alloc_slot()
+    engine.step([StepEntry(sa, a[:long_n], []), StepEntry(sb, b[:70], [])])
+    for p in range(3):                                              # both decode for a while
+        engine.step([StepEntry(sa, [a[long_n + p]], [0]), StepEntry(sb, [b[70 + p]], [0])])
+    sc, sd = engine.alloc_slot(), engine.alloc_slot()
+    engine.step([StepEntry(sd, d[:40], [])])                         # d's prompt has begun
+    # the mixed step: a and b one token each, c whole, d's next piece
+    got = engine.step([StepEntry(sa, [a[long_n + 3]], [0]), StepEntry(sc, c[:97], [0, 50, 96]),
+                       StepEntry(sb, [b[73]], [0]), StepEntry(sd, d[40:110], [0, 69])]).cpu().numpy()
+    want = [("a", long_n + 3), ("c", 0), ("c", 50), ("c", 96), ("b", 73), ("d", 40), ("d", 109)]
+    for row, (k, p) in enumerate(want):
+        ok, err = close(got[row], ref[k][p], dtype, name, "mixed step")
+        assert ok, (k, p, err)
+    # and all four go on, one token each, from what that step left in the cache
+    got = engine.step([StepEntry(sa, [a[long_n + 4]], [0]), StepEntry(sb, [b[74]], [0]),
+                       StepEntry(sc, [c[97]], [0]), StepEntry(sd, [d[110]], [0])]).cpu().numpy()
+    for row, (k, p) in enumerate([("a", long_n + 4), ("b", 74), ("c", 97), ("d", 110)]):
+        ok, err = close(got[row], ref[k][p], dtype, name, "after mixed step")
+        assert ok, (k, p, err)
+    for s in (sa, sb, sc, sd):
+        engine.free_slot(s)
+    engine.cache.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["B", "D"])
+def test_roll_back_and_feed_other_tokens(name, dtype, model_root):
+    """Engine.truncate (the reference's truncate_kv, crates/backends/backend_common/src/
+    cpu_backend.rs:527-543): 150 tokens, back to 70 (inside a page: the rest of that page holds
+    keys and, transposed, values of the tokens given up) and to 64 (a page's edge), then other
+    tokens, whole and one by one; every position's logits are those of the new sequence."""
+    folder = make_folder(model_root, name, dtype)
+    vocab = CONFIGS[name][0]["vocab_size"]
+    first = random_tokens(vocab, 150, 301)
+    engine = hb.load(folder, dtype=dtype, cache_tokens=64 * 8)
+    group = next(iter(engine.cache.kv_groups.values()))
+    for keep, seed in ((70, 302), (64, 303), (0, 304), (149, 305)):
+        s = engine.alloc_slot()
+        engine.step([StepEntry(s, first, [])])
+        assert group.pages.held_count == 3
+        engine.truncate(s, keep)
+        assert engine.cache.length(s) == keep and group.pages.held_count == (keep + 63) // 64
+        other = first[:keep] + random_tokens(vocab, 60, seed)
+        ref = plain_logits(folder, other)
+        got = [engine.step([StepEntry(s, other[keep:keep + 30], list(range(30)))]).cpu().numpy()]
+        for p in range(keep + 30, keep + 60):
+            got.append(engine.step([StepEntry(s, [other[p]], [0])]).cpu().numpy())
+        got = np.concatenate(got)
+        for i, p in enumerate(range(keep, keep + 60)):
+            ok, err = close(got[i], ref[p], dtype, name, "after roll-back")
+            assert ok, (keep, p, err)
+        with pytest.raises(CacheError, match="cannot truncate"):
+            engine.truncate(s, keep + 61)
+        engine.free_slot(s)
+        engine.cache.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_windowed_cache_rolls_back_only_to_keys_it_still_has(dtype, model_root):
+    """Configuration C: one layer sees 70 keys and has given up the pages before them. Rolling
+    back a little stays within what is held and gives the plain logits; rolling back past it is
+    refused and changes nothing."""
+    folder = make_folder(model_root, "C", dtype)
+    vocab = CONFIGS["C"][0]["vocab_size"]
+    first = random_tokens(vocab, 200, 311)
+    engine = hb.load(folder, dtype=dtype, cache_tokens=64 * 8)
+    s = engine.alloc_slot()
+    engine.step([StepEntry(s, first, [])])
+    with pytest.raises(CacheError, match="given up"):
+        engine.truncate(s, 100)
+    assert engine.cache.length(s) == 200
+    engine.cache.check()
+    # after 200 tokens the windowed layer holds pages from position 128 on; a query at 198 sees
+    # the keys from 129 on
+    with pytest.raises(CacheError, match="given up"):
+        engine.truncate(s, 196)
+    engine.truncate(s, 198)
+    other = first[:198] + random_tokens(vocab, 20, 312)
+    ref = plain_logits(folder, other)
+    got = engine.step([StepEntry(s, other[198:], list(range(20)))]).cpu().numpy()
+    for i in range(20):
+        ok, err = close(got[i], ref[198 + i], dtype, "C", "after roll-back")
+        assert ok, (i, err)
+    engine.free_slot(s)
+    engine.cache.check()
+
+
+def test_a_step_that_does_not_fit_changes_nothing(model_root):
+    """All of a step's pages or none: the step is refused, the sequences that were in it hold
+    what they held, and they go on as if it had never been asked for."""
+    folder = make_folder(model_root, "B", "float32")
+    vocab = CONFIGS["B"][0]["vocab_size"]
+    a, b = random_tokens(vocab, 80, 321), random_tokens(vocab, 140, 322)
+    engine = hb.load(folder, dtype="float32", cache_tokens=64 * 4)
+    sa, sb = engine.alloc_slot(), engine.alloc_slot()
+    engine.step([StepEntry(sa, a[:60], []), StepEntry(sb, b[:10], [])])
+    group = next(iter(engine.cache.kv_groups.values()))
+    held = group.pages.held_count
+    with pytest.raises(CacheError, match="more pages"):
+        engine.step([StepEntry(sa, a[60:70], [9]), StepEntry(sb, b[10:140], [0])])   # 1 + 2 pages, 2 free
+    assert group.pages.held_count == held
+    assert engine.cache.length(sa) == 60 and engine.cache.length(sb) == 10
+    engine.cache.check()
+    got = engine.step([StepEntry(sa, a[60:80], [19]), StepEntry(sb, b[10:64], [53])]).cpu().numpy()
+    assert close(got[0], plain_logits(folder, a)[79], "float32", "B")[0]
+    assert close(got[1], plain_logits(folder, b)[63], "float32", "B")[0]
+    engine.free_slot(sa)
+    engine.free_slot(sb)
+    engine.cache.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_checkpoint_with_tensors_nobody_asks_for_loads_and_says_the_same(dtype, model_root, tmp_path):
+    """A tied model whose file also holds a head and rotary buffers (as exported checkpoints do):
+    the reference ignores what it does not know and takes the embedding for the head
+    (crates/backends/backend_common/src/loader_common.rs:679-685,1851-1872). Same logits as
+    without them; the engine says what it passed over."""
+    from safetensors.torch import load_file, save_file
+    src = make_folder(model_root, "A", dtype)
+    tensors = load_file(os.path.join(src, "model.safetensors"))
+    tensors["lm_head.weight"] = torch.full((256, 64), 3.0).to(tensors["model.norm.weight"].dtype)
+    for layer in range(2):
+        tensors[f"model.layers.{layer}.self_attn.rotary_emb.inv_freq"] = torch.ones(8)
+    save_file(tensors, str(tmp_path / "model.safetensors"))
+    with open(os.path.join(src, "config.json")) as f, open(tmp_path / "config.json", "w") as g:
+        g.write(f.read())
+    tokens = random_tokens(256, 40, 331)
+    engine = hb.load(str(tmp_path), dtype=dtype, cache_tokens=64)
+    assert sorted(engine.ignored_tensors) == ["lm_head.weight", "model.layers.0.self_attn.rotary_emb.inv_freq",
+                                              "model.layers.1.self_attn.rotary_emb.inv_freq"]
+    s = engine.alloc_slot()
+    got = engine.step([StepEntry(s, tokens, list(range(40)))]).cpu().numpy()
+    clean = hb.load(src, dtype=dtype, cache_tokens=64)
+    s2 = clean.alloc_slot()
+    assert np.array_equal(got, clean.step([StepEntry(s2, tokens, list(range(40)))]).cpu().numpy())
+    ref = plain_logits(src, tokens)
+    for p in range(40):
+        assert close(got[p], ref[p], dtype, "A")[0], p
+
+
+def test_decode_graphs_and_their_logits_are_bounded(model_root):
+    """Decoding at three batch sizes through twenty context buckets each: sixty shapes, more than
+    the engine keeps graphs for. One logits buffer per batch size, at most MAX_GRAPHS graphs, the
+    memory held levels off, and a shape whose graph was dropped is captured again and still
+    says what eager steps say."""
+    from herbert_rs_amd.engine import engine as eng_mod
+    folder = make_folder(model_root, "D", "bfloat16", overrides={"max_position_embeddings": 8192})
+    vocab = CONFIGS["D"][0]["vocab_size"]
+    sizes = (1, 3, 8)
+    engine = hb.Engine.from_folder(folder, dtype="bfloat16", max_tokens=64 * 90 * 8, use_graphs=True)
+    eager = hb.Engine.from_folder(folder, dtype="bfloat16", max_tokens=64 * 90 * 8, use_graphs=False)
+    feed = random_tokens(vocab, 8 * 64, 341)
+    held_after = []
+    for B in sizes:
+        slots = [engine.alloc_slot() for _ in range(B)]
+        slots_e = [eager.alloc_slot() for _ in range(B)]
+        at = 0
+        for bucket in range(20):
+            grow = 256 * bucket + 250 - at                    # up to just below the next bucket's edge
+            for eng, sl in ((engine, slots), (eager, slots_e)):
+                eng.step([StepEntry(s, [(7 * i + j) % vocab for j in range(grow)], []) for i, s in enumerate(sl)])
+            at += grow
+            for j in range(10):                                # 6 steps in this bucket, 4 in the next
+                toks = [feed[(at + 13 * i + j) % len(feed)] for i in range(B)]
+                a = engine.step([StepEntry(s, [t], [0]) for s, t in zip(slots, toks)]).cpu().numpy()
+                b = eager.step([StepEntry(s, [t], [0]) for s, t in zip(slots_e, toks)]).cpu().numpy()
+                assert np.array_equal(a, b), (B, bucket, j)
+                at += 1
+        for s in slots:
+            engine.free_slot(s)
+        for s in slots_e:
+            eager.free_slot(s)
+        torch.cuda.synchronize()
+        held_after.append(torch.cuda.memory_allocated())
+    assert held_after[-1] - held_after[0] < 64 << 20           # no pool of its own behind every graph
+    graphs, batch_sizes, logits_bytes = engine.decode_graph_stats()
+    assert engine.graphs_captured >= 60 - 3                    # nearly every shape was captured once
+    assert graphs <= eng_mod.MAX_GRAPHS < engine.graphs_captured
+    assert batch_sizes == len(sizes) and logits_bytes == sum(sizes) * vocab * 4
+    # the first batch size's graph is long gone: it is captured again and agrees with eager steps
+    s, se = engine.alloc_slot(), eager.alloc_slot()
+    engine.step([StepEntry(s, feed[:200], [])]); eager.step([StepEntry(se, feed[:200], [])])
+    before = engine.graphs_captured
+    for j in range(4):
+        a = engine.step([StepEntry(s, [feed[j]], [0])]).cpu().numpy()
+        b = eager.step([StepEntry(se, [feed[j]], [0])]).cpu().numpy()
+        assert np.array_equal(a, b)
+    assert engine.graphs_captured == before + 1 and engine.decode_graph_stats()[0] <= eng_mod.MAX_GRAPHS
+    engine.cache.check()
+
+
+def write_tokenizer(folder, vocab):
+    """A tokenizer.json of whole words w0, w1, ... and the chat format's special tokens, written
+    with the tokenizers package; the model's last ids are the specials."""
+    from tokenizers import Tokenizer, decoders, models, pre_tokenizers
+    specials = ["<|im_start|>", "<|im_end|>", "system", "user", "assistant"]
+    words = {f"w{i}": i for i in range(vocab - len(specials))}
+    for i, t in enumerate(specials):
+        words[t] = vocab - len(specials) + i
+    tok = Tokenizer(models.WordLevel(words, unk_token="w0"))
+    tok.pre_tokenizer = pre_tokenizers.WhitespaceSplit()
+    tok.add_special_tokens(["<|im_start|>", "<|im_end|>"])
+    tok.save(os.path.join(folder, "tokenizer.json"))
+    return tok, words
+
+
+def cli_folder(model_root, tmp_path):
+    src = make_folder(model_root, "A", "float32")
+    folder = str(tmp_path / "A_text")
+    os.makedirs(folder)
+    os.link(os.path.join(src, "model.safetensors"), os.path.join(folder, "model.safetensors"))
+    with open(os.path.join(src, "config.json")) as f:
+        raw = json.load(f)
+    raw["eos_token_id"] = 0                       # "w0": not among what this model says here
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(raw, f)
+    return folder, raw
+
+
+def run_cli(folder, *args, timeout=240):
+    return subprocess.run([sys.executable, os.path.join(ROOT, "bin", "herbert-cli"), "--model", folder,
+                           "--dtype", "float32", "--temperature", "0", "--no-repeat-check", *args],
+                          capture_output=True, text=True, timeout=timeout)
+
+
+def test_cli_with_a_tokenizer_chat_template_and_stop_strings(model_root, tmp_path):
+    """With a tokenizer.json the prompt is text in the architecture's chat template
+    (crates/cli/src/main.rs:281-294), the output is text, and --stop ends it where the decoded
+    text first holds the string (main.rs:236-247,1328-1332,1360), the token that completes the
+    string still printed."""
+    folder, raw = cli_folder(model_root, tmp_path)
+    tok, words = write_tokenizer(folder, raw["vocab_size"])
+    prompt = "w5 w17 w3"
+    ids = tok.encode("<|im_start|>system\nw9<|im_end|>\n<|im_start|>user\n" + prompt +
+                     "<|im_end|>\n<|im_start|>assistant\n", add_special_tokens=False).ids
+    assert ids[0] == words["<|im_start|>"] and words["w17"] in ids and len(ids) == 12
+    cfg, w = plain_folder(folder)
+    want = plain.greedy(cfg, w, ids, 13, stop_ids=(words["<|im_end|>"], 0))
+    out = run_cli(folder, "--prompt", prompt, "--system", "w9", "--max-tokens", "12", "--verbose")
+    assert out.returncode == 0, out.stderr
+    text = tok.decode(want, skip_special_tokens=True)
+    assert out.stdout.strip() == text.strip() and len(text.split()) >= 6
+    # a stop string: the third and fourth words of what it says
+    said = text.split()
+    stop = " ".join(said[2:4])
+    upto = next(n for n in range(1, len(said) + 1) if stop in " ".join(said[:n]))
+    out = run_cli(folder, "--prompt", prompt, "--system", "w9", "--max-tokens", "12", "--verbose",
+                  "--stop", stop, "--stop", "never said\\n")
+    assert out.returncode == 0, out.stderr
+    assert out.stdout.strip() == " ".join(said[:upto]) and upto <= 4
+    assert "Stop reason:     stop_sequence" in out.stderr and f"Output tokens:   {upto}" in out.stderr
+
+
+def test_cli_interrupt_ends_generation_cleanly(model_root, tmp_path):
+    """SIGINT sets a flag that the loop looks at before its next decode step
+    (crates/cli/src/main.rs:22-50,1242-1245): the process ends by itself with what it has."""
+    folder = make_folder(model_root, "D", "float32")
+    proc = subprocess.Popen([sys.executable, os.path.join(ROOT, "bin", "herbert-cli"), "--model", folder,
+                             "--dtype", "float32", "--temperature", "0", "--no-repeat-check", "--ignore-eos",
+                             "--prompt", "1,2,3", "--max-tokens", "2040", "--verbose"],
+                            stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
+    first = proc.stdout.read(1)                    # the first token is out: generation runs
+    assert first.isdigit()
+    proc.send_signal(signal.SIGINT)
+    try:
+        out, err = proc.communicate(timeout=120)
+    finally:
+        if proc.poll() is None:
+            proc.kill()
+    assert proc.returncode == 0, err
+    tokens = (first + out).strip().split(",")
+    assert "Interrupted" in err and "Stop reason:     interrupted" in err
+    assert 1 <= len(tokens) < 2041 and all(t.isdigit() for t in tokens)

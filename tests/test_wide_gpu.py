@@ -1,0 +1,125 @@
+"""The whole model at the layer widths that the benchmark times, against the plain implementation.
+
+Two layers of the Qwen3-8B shape (hidden 4096, 32 query heads on 8 kv heads of 128,
+intermediate 12288, vocabulary 151936, separate head), random bfloat16 weights, through
+bin/trace_run in bfloat16 and in float32: one prompt of 2,048 tokens (the q/k/v product that
+norms, rotates and writes the cache itself), decoding at batch 1, 8 and 64 with the kernels the
+host picks for these widths by itself, and batches of unequal lengths that follow one another
+in slots that were used before. Nothing is patched: what runs here is what bench.py times.
+"""
+import numpy as np
+import pytest
+import torch
+
+from . import replay_util as ru
+from .bounds import close
+from .plain_cache import forget, plain_rows
+from .tiny import make_folder_from, random_tokens
+
+pytestmark = pytest.mark.gpu
+
+WIDE = dict(
+    architectures=["Qwen3ForCausalLM"], model_type="qwen3",
+    num_hidden_layers=2, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
+    intermediate_size=12288, vocab_size=151936, rope_theta=1000000.0, rms_norm_eps=1e-6,
+    tie_word_embeddings=False, max_position_embeddings=4096, eos_token_id=151645)
+VOCAB = WIDE["vocab_size"]
+
+
+def wide_requests():
+    """id -> (tokens, length of the prompt part, places of the prompt whose logits are wanted)."""
+    reqs = {"long": (random_tokens(VOCAB, 2048 + 6, 900), 2048, [0, 1, 63, 64, 1023, 2047])}
+    for i, n in enumerate([300, 64, 129, 17, 200, 77, 256, 1]):                 # a batch of 8
+        extra = [4, 4, 4, 2, 4, 1, 4, 4][i]
+        reqs[f"e{i}"] = (random_tokens(VOCAB, n + extra, 910 + i), n, sorted({0, n - 1}))
+    for i in range(64):                                                        # a batch of 64
+        n = 1 + (37 * i + 11) % 90
+        extra = 3 if i % 2 else 2
+        reqs[f"s{i}"] = (random_tokens(VOCAB, n + extra, 1000 + i), n, [n - 1])
+    for i, n in enumerate([90, 5, 130, 64, 33, 70, 2, 191]):                    # again 8, in used slots
+        reqs[f"f{i}"] = (random_tokens(VOCAB, n + 3, 1100 + i), n, [n - 1])
+    return reqs
+
+
+def wide_trace(reqs):
+    """The long prompt alone and decoded on at batch 1; then the batches of 8, of 64 and of 8,
+    each: all prompts in one step, then one token each, shorter requests ending earlier."""
+    steps = []
+
+    def run_batch(ids):
+        first = {"step": len(steps), "entries": [], "end": []}
+        for rid in ids:
+            toks, n, want = reqs[rid]
+            first["entries"].append({"id": rid, "tokens": toks[:n], "want": want})
+        steps.append(first)
+        at = {rid: reqs[rid][1] for rid in ids}
+        live = list(ids)
+        while live:
+            rec = {"step": len(steps), "entries": [], "end": []}
+            for rid in list(live):
+                toks = reqs[rid][0]
+                rec["entries"].append({"id": rid, "tokens": [toks[at[rid]]], "want": [0]})
+                at[rid] += 1
+                if at[rid] == len(toks):
+                    rec["end"].append(rid)
+                    live.remove(rid)
+            steps.append(rec)
+
+    run_batch(["long"])
+    run_batch([f"e{i}" for i in range(8)])
+    run_batch([f"s{i}" for i in range(64)])
+    run_batch([f"f{i}" for i in range(8)])
+    return steps
+
+
+@pytest.fixture(scope="module")
+def wide_folder(tmp_path_factory):
+    root = tmp_path_factory.mktemp("wide")
+    return make_folder_from(root, "wide", WIDE, seed=8, dtype="bfloat16", std=0.02, norm_std=0.1)
+
+
+def test_the_host_picks_the_profiled_kernels_for_these_widths():
+    """The plans of the decode steps at batch 1, 8 and 64 for the 8B widths, by the planner's
+    own codes (0 = the few-row kernel; else tile + 1000 x K slices; tiles 112 = 128 x 32,
+    124 = 128 x 64, 184 = 256 x 64): the kernels whose profiles lie under profiles/."""
+    from herbert_rs_amd.kernels import mfma
+    STORE, ADD, SWIGLU = mfma.EPI_STORE, mfma.EPI_ADD, mfma.EPI_SWIGLU
+    H, Q, I, V = 4096, 6144, 12288, VOCAB
+    plan = mfma.gemm_plan
+    for M in (1, 8):
+        assert plan(M, H, H, ADD, leaves_norm=True) == 0                       # o: few rows
+        assert plan(M, H, I, ADD, leaves_norm=True) == 0                       # down
+        assert plan(M, 2 * I, H, SWIGLU, finishes_norm=True) == 112            # gate/up: 128 x 32 tiles
+        assert plan(M, V, H, STORE) == 0                                       # head
+    assert plan(1, Q, H, STORE, finishes_norm=True, defer_slices=True) == 0    # q/k/v at batch 1
+    assert plan(8, Q, H, STORE, finishes_norm=True, defer_slices=True) == 4112  # 4 K slices, added up by the attention
+    assert plan(64, Q, H, STORE, defer_slices=True) == 4124
+    assert plan(64, H, H, ADD, leaves_norm=True) == 8124 and plan(64, H, I, ADD, leaves_norm=True) == 8124
+    assert plan(64, 2 * I, H, SWIGLU) == 124 and plan(64, V, H, STORE) == 184
+    assert mfma.norm_handoff(8, H, H) == "half" and mfma.norm_handoff(64, H, I) == "whole"
+    # the prompt of 2,048 tokens: the fused q/k/v product is taken from 136 tiles of 256 x 256 on
+    assert -(-2048 // 256) * -(-Q // 256) >= mfma.QKV_FUSE_MIN_TILES
+    assert plan(2048, 2 * I, H, SWIGLU) == 188 and plan(2048, H, I, ADD) == 142
+
+
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_prompt_of_2048_and_decoding_at_batch_1_8_64(dtype, wide_folder, tmp_path):
+    reqs = wide_requests()
+    steps = wide_trace(reqs)
+    assert max(len(s["entries"]) for s in steps) == 64
+    out = ru.run_trace(wide_folder, dtype, steps, str(tmp_path / "out"), ru.needed_tokens(steps), VOCAB,
+                       timeout=600)
+    got = ru.collect(steps, out)
+    wanted = {}
+    for (rid, pos) in got:
+        wanted.setdefault(rid, []).append(pos)
+    assert len(got) == sum(len(w) + len(t) - n for t, n, w in reqs.values())
+    for rid, places in wanted.items():
+        ref = plain_rows(wide_folder, reqs[rid][0], places)
+        for pos in places:
+            kind = "prompt" if pos < reqs[rid][1] else "decode"
+            group = {"l": "b1", "e": "b8", "s": "b64", "f": "b8 again"}[rid[0]]
+            ok, err = close(got[(rid, pos)], ref[pos], dtype, "wide", f"{group} {kind}")
+            assert ok, f"request {rid} position {pos} ({group} {kind}): error {err}"
+    if dtype == "float32":
+        forget(wide_folder)

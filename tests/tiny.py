@@ -67,3 +67,14 @@ def make_folder(root, name, dtype="float32", overrides=None, seed=None, std=None
 def random_tokens(vocab, n, seed):
     g = torch.Generator().manual_seed(seed)
     return torch.randint(0, vocab, (n,), generator=g).tolist()
+
+
+def make_folder_from(root, tag, raw, seed, dtype="float32", std=0.02, norm_std=0.1):
+    """Write a random model of the configuration `raw` into root/<tag>_<dtype> once; returns the path."""
+    folder = os.path.join(str(root), f"{tag}_{dtype}")
+    if os.path.exists(os.path.join(folder, "model.safetensors")):
+        return folder
+    cfg, spec = spec_of(raw)
+    write_model_folder(folder, dict(raw), Model(spec).tensor_needs(), seed, dtype=dtype, std=std,
+                       norm_std=norm_std)
+    return folder
