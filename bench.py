@@ -283,7 +283,7 @@ def main():
 
     points = {}
     head = measure(args.batch)
-    value, ms = head[0][0], head[0][1]
+    value, ms, achieved = head[0]
     add_points(points, args.batch, head)
     for key in (f"decode_b{args.batch}", f"decode_b{args.batch}_ms", f"decode_b{args.batch}_gbs",
                 f"decode_b{args.batch}_frac"):
