@@ -8,7 +8,9 @@
 // first of equals); the random numbers are the host's (xorshift64, :30-34, 50-62). On the GPU there:
 // crates/backends/backend_metal/shaders/argmax.metal:14-149 (two stages, strict >).
 #include "common.h"
+#include "noalloc.h"
 #include <math.h>
+#include <mutex>
 
 HB_MODULE_ERROR_SLOT()
 
@@ -98,6 +100,65 @@ extern "C" int hb_argmax(const float* logits, int ld, int R, int V, int* out, fl
                                                      scratch_i);
     }
     HB_CHECK_LAUNCH("argmax");
+    return 0;
+}
+
+// ---- argmax without a workspace of the caller's (see noalloc.h) ----
+// The partial results live in this array: values [MAX_PAIRS] floats, then indices [MAX_PAIRS]
+// ints. In host code its name is only a handle for hipGetSymbolAddress: every GPU has a copy
+// of its own at an address of its own, looked up once per device and kept below.
+static __device__ __align__(256) unsigned char scratch[HB_ARGMAX_NOALLOC_MAX_PAIRS * (sizeof(float) + sizeof(int))];
+
+#define HB_MAX_DEVICES 64
+static void* scratch_on_device[HB_MAX_DEVICES] = {nullptr};
+static std::mutex scratch_lock;
+
+// The device address of `scratch` on the current device.
+static int scratch_address(void** ptr) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    HB_REQUIRE(e == hipSuccess, "argmax (no allocation): hipGetDevice failed: %s", hipGetErrorString(e));
+    HB_REQUIRE(dev >= 0 && dev < HB_MAX_DEVICES, "argmax (no allocation): device %d is beyond the %d this library keeps",
+               dev, HB_MAX_DEVICES);
+    std::lock_guard<std::mutex> guard(scratch_lock);
+    if (!scratch_on_device[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        HB_REQUIRE(e == hipSuccess && p, "argmax (no allocation): hipGetSymbolAddress failed on device %d: %s", dev,
+                   hipGetErrorString(e));
+        scratch_on_device[dev] = p;
+    }
+    *ptr = scratch_on_device[dev];
+    return 0;
+}
+
+extern "C" int hb_argmax_noalloc_setup(void) {
+    void* p = nullptr;
+    return scratch_address(&p);
+}
+
+extern "C" int hb_argmax_noalloc(const float* logits, int ld, int R, int V, int* out, hipStream_t stream) {
+    HB_REQUIRE(R > 0 && V > 0 && ld >= V, "argmax (no allocation): bad sizes (R=%d, V=%d, ld=%d)", R, V, ld);
+    HB_REQUIRE(logits && out, "argmax (no allocation): null logits or out");
+    int chunks = V / 8192;
+    chunks = chunks > 64 ? 64 : chunks;
+    if (chunks <= 1) {
+        argmax_kernel<<<dim3(R, 1), 1024, 0, stream>>>(logits, ld, V, out, nullptr, nullptr, nullptr, nullptr);
+        HB_CHECK_LAUNCH("argmax (no allocation)");
+        return 0;
+    }
+    HB_REQUIRE((long long)R * chunks <= HB_ARGMAX_NOALLOC_MAX_PAIRS,
+               "argmax (no allocation): %d rows x %d stretches = %lld partial results, the library's scratch holds %d; "
+               "use hb_argmax with a workspace of your own", R, chunks, (long long)R * chunks,
+               HB_ARGMAX_NOALLOC_MAX_PAIRS);
+    void* base = nullptr;
+    if (scratch_address(&base)) return 1;
+    float* part_v = (float*)base;
+    int* part_i = (int*)((unsigned char*)base + HB_ARGMAX_NOALLOC_MAX_PAIRS * sizeof(float));
+    // every pair the second kernel reads is written by the first: nothing has to be cleared
+    argmax_kernel<<<dim3(R, chunks), 1024, 0, stream>>>(logits, ld, V, out, part_v, part_i, nullptr, nullptr);
+    argmax_kernel<<<dim3(R, 1), 64, 0, stream>>>(nullptr, 0, chunks, out, nullptr, nullptr, part_v, part_i);
+    HB_CHECK_LAUNCH("argmax (no allocation)");
     return 0;
 }
 

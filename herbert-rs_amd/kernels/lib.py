@@ -35,6 +35,8 @@ SIGNATURES = {
     },
     "sampling": {
         "hb_argmax": [_P, _I, _I, _I, _P, _P, _P, _I, _P],
+        "hb_argmax_noalloc": [_P, _I, _I, _I, _P, _P],
+        "hb_argmax_noalloc_setup": [],
         "hb_sample": [_P, _I, _I, _I, _F, _I, _F, _P, _P, _P, _P, _P, _I, _P, _P, _P],
     },
 }
