@@ -122,8 +122,13 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache
     constexpr int KRPB = 128 / HD > 0 ? 128 / HD : 1;   // key rows in 256 bytes
     constexpr int KROWS = 512 / HD;               // key rows a load instruction brings (1 KB)
     constexpr int LOADS = HD / 32;                // a wave's load instructions for the keys of a page; as many for the values
-    __shared__ __attribute__((aligned(1024))) bf16 Ks[2][PAGE * HD];
-    __shared__ __attribute__((aligned(1024))) bf16 Vs[2][HD * PAGE];
+    // The LDS is the launch's (extern), not arrays of this kernel: for an array of its own the
+    // compiler knows which loads-to-LDS may alias a read and waits for every load in flight
+    // (s_waitcnt vmcnt(0)) before the first read that follows, which undoes the ring: the loads of
+    // the next pages would be waited for at once. What has to have landed is waited for by hand.
+    extern __shared__ __attribute__((aligned(1024))) bf16 attn_lds[];     // keys [2][PAGE * HD], then values [2][HD * PAGE]
+    bf16 (*Ks)[PAGE * HD] = (bf16 (*)[PAGE * HD])attn_lds;
+    bf16 (*Vs)[HD * PAGE] = (bf16 (*)[HD * PAGE])(attn_lds + 2 * PAGE * HD);
 
     int w = blockIdx.x;
     {
@@ -623,7 +628,7 @@ extern "C" int hb_attn_prefill_mfma(const void* q, const void* k_cache, const vo
     const int total = num_tiles * per_tile;
     const float c = scale * LOG2E;
 #define LAUNCH_PREFILL(HDV)                                                                              \
-    attn_prefill_kernel<HDV><<<total, 256, 0, stream>>>((const bf16*)q, (const bf16*)k_cache,            \
+    attn_prefill_kernel<HDV><<<total, 256, 4 * PAGE * HDV * sizeof(bf16), stream>>>((const bf16*)q, (const bf16*)k_cache, \
                                                        (const bf16*)v_cache, (bf16*)out, tile_seq, tile_row0, \
                                                        tile_rows, positions, slots, page_table, max_pages, nq, \
                                                        nkv, c, window, per_tile, total)
