@@ -144,6 +144,8 @@ def main():
     ap.add_argument("--workload", default="headline", choices=["headline", "qwen3-1.7b", "qwen3-32b"],
                     help="headline: BASELINE.json configs[2]; the others: configs[3] and configs[4]")
     ap.add_argument("--prefill-tokens", type=int, default=2048, help="length of the prompt of the prefill figure")
+    ap.add_argument("--prefill-chunk", type=int, default=0,
+                    help="feed the prompt of the prefill figure in steps of this many tokens (0: in one step)")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run the 2,048-token prefill alone (for profiles); prints no JSON line")
     args = ap.parse_args()
@@ -169,12 +171,12 @@ def main():
     layers_full = shape["num_hidden_layers"]
     layers = args.layers or layers_full
     raw = dict(shape, architectures=["Qwen3ForCausalLM"], model_type="qwen3",
-               num_hidden_layers=layers, max_position_embeddings=max(context, 4096) + 64,
+               num_hidden_layers=layers, max_position_embeddings=max(context, 4096, args.prefill_tokens) + 64,
                eos_token_id=151645)
     cfg = hb.Qwen3Config.from_dict(raw)
     torch.cuda.set_device(0)
     max_batch = args.batch if args.no_points else max(args.batch, 64)
-    cache_tokens = max_batch * (context + 64)
+    cache_tokens = max(max_batch * (context + 64), args.prefill_tokens + 64)
     t0 = time.time()
     engine = hb.Engine.from_config(cfg, seed=2, dtype=args.dtype, std=0.02, norm_std=0.0,
                                    max_tokens=cache_tokens, max_slots=max_batch)
@@ -226,16 +228,22 @@ def main():
             engine.free_slot(s)
         return out
 
-    def prefill_run(tokens_n, reps):
+    def prefill_once(tokens_n):
+        """One prompt of tokens_n tokens, whole or in chunks; the last token's logits are asked for."""
         slot = engine.alloc_slot()
-        engine.step([StepEntry(slot, ids(tokens_n), [tokens_n - 1])])
+        chunk = args.prefill_chunk or tokens_n
+        prompt = ids(tokens_n)
+        for a in range(0, tokens_n, chunk):
+            part = prompt[a:a + chunk]
+            engine.step([StepEntry(slot, part, [len(part) - 1] if a + chunk >= tokens_n else [])])
         engine.free_slot(slot)
+
+    def prefill_run(tokens_n, reps):
+        prefill_once(tokens_n)
         torch.cuda.synchronize()
         t = time.perf_counter()
         for _ in range(reps):
-            slot = engine.alloc_slot()
-            engine.step([StepEntry(slot, ids(tokens_n), [tokens_n - 1])])
-            engine.free_slot(slot)
+            prefill_once(tokens_n)
         torch.cuda.synchronize()
         return (time.perf_counter() - t) / reps
 

@@ -28,6 +28,7 @@
 // decode kernel: crates/backends/backend_metal/shaders/head_norm_rope_kv_append.metal:37-110.
 #include "common.h"
 #include <math.h>
+#include <type_traits>
 
 HB_MODULE_ERROR_SLOT()
 
@@ -57,6 +58,13 @@ __device__ __forceinline__ int acc_key(int kb, int g2, int i) { return kb * 32 +
 // far scaled by corr < 1) only when a score exceeds it by more than 8 / c, that is when a
 // probability would exceed 2^8 times the largest so far; till then corr is 1 and the caller
 // need not touch its sums. Any reference gives the same quotient in the end.
+__device__ __forceinline__ float max_with_other_half(float v) {
+    // lanes i and i ^ 32 exchange their values without a trip through LDS
+    const unsigned u = __float_as_uint(v);
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+
 #define RESCALE_LOG2 8.0f
 template <bool MASKED>
 __device__ __forceinline__ void softmax_page(f32x16 st[2], int g2, int page0, int lo, int hi, float c,
@@ -72,7 +80,7 @@ __device__ __forceinline__ void softmax_page(f32x16 st[2], int g2, int page0, in
             }
             mx = fmaxf(mx, st[kb][i]);
         }
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    mx = max_with_other_half(mx);
     corr = 1.0f;
     if ((mx - m) * c > RESCALE_LOG2 || m == -INFINITY) {       // (-inf) - (-inf) is NaN: compares false
         const float m_new = (mx == -INFINITY) ? m : mx;
@@ -102,46 +110,75 @@ __device__ __forceinline__ void rescale(f32x16 (&oacc)[NACC], float corr) {
         for (int i = 0; i < 16; ++i) oacc[d][i] *= corr;
 }
 
+// The first half of softmax_page alone: mask, the page's largest score, the reference moved up if
+// need be. Returns m * c (what is taken off the scaled scores), corr as softmax_page does.
+template <bool MASKED>
+__device__ __forceinline__ float softmax_reference(f32x16 st[2], int g2, int page0, int lo, int hi, float c,
+                                                   float& m, float& corr) {
+    float mx = -INFINITY;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            if (MASKED) {
+                const int key = page0 + acc_key(kb, g2, i);
+                st[kb][i] = (key >= lo && key <= hi) ? st[kb][i] : -INFINITY;
+            }
+            mx = fmaxf(mx, st[kb][i]);
+        }
+    mx = max_with_other_half(mx);
+    corr = 1.0f;
+    if ((mx - m) * c > RESCALE_LOG2 || m == -INFINITY) {
+        const float m_new = (mx == -INFINITY) ? m : mx;
+        corr = (m == -INFINITY) ? 0.f : fast_exp2((m - m_new) * c);
+        m = m_new;
+    }
+    return (m == -INFINITY) ? 0.f : m * c;
+}
+
 // ----------------------------------------------------------------- prefill
-// A workgroup: 32 queries x up to 4 query heads of one kv head (a wave a head). The pages go
-// from global memory straight into a ring of two LDS stages, the next page's loads in flight
-// while this page is worked on. Rows lie unpadded; the 16-byte chunk c of row r sits at chunk
-// c ^ (r / rows in 256 bytes), so that the operand reads of 16 rows at one chunk fall into 16
-// different bank groups.
-// Workgroups are numbered by falling work (the host sorts the tiles) and every other round of
-// 256 backwards: with one round per CU the heaviest tiles then share a CU with the lightest.
+// A workgroup: 32 queries x up to 4 query heads of one kv head, by eight waves in two groups of
+// four (a wave a head in each group). The groups take the tile's pages in turn, the first the
+// even ones and the second the odd ones, each with a reference, a sum and an output of its
+// own, which are added up through LDS at the end: the tile with the most pages, which decides
+// how long a prompt of a few thousand tokens takes, is done in half as many steps, and a CU
+// holds one workgroup whose eight waves (two a SIMD) are busy from its first page to its last.
+// Each group's pages go from global memory straight into a ring of two LDS stages of its own,
+// the next page's loads in flight while this page is worked on. Rows lie unpadded; the
+// 16-byte chunk c of row r sits at chunk c ^ (r / rows in 256 bytes), so that the operand
+// reads of 16 rows at one chunk fall into 16 different bank groups.
+// Workgroups are numbered by falling work (the host sorts the tiles): a CU that is done takes
+// the heaviest tile left.
 template <int HD>
-__global__ void __launch_bounds__(256, 2)
+__global__ void __launch_bounds__(512, 1)
 attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache,
                     const bf16* __restrict__ v_cache, bf16* __restrict__ out,
                     const int* __restrict__ tile_seq, const int* __restrict__ tile_row0,
                     const int* __restrict__ tile_rows, const int* __restrict__ positions,
                     const int* __restrict__ slots, const int* __restrict__ page_table, int max_pages, int nq,
-                    int nkv, float c, int window, int per_tile, int total) {
+                    int nkv, float c, int window, int per_tile) {
     constexpr int KCH = HD / 8;                   // 16-byte chunks of a key row
     constexpr int KRPB = 128 / HD > 0 ? 128 / HD : 1;   // key rows in 256 bytes
     constexpr int KROWS = 512 / HD;               // key rows a load instruction brings (1 KB)
     constexpr int LOADS = HD / 32;                // a wave's load instructions for the keys of a page; as many for the values
+    constexpr int STAGE = PAGE * HD;              // elements of one stage of keys, or of values
     // The LDS is the launch's (extern), not arrays of this kernel: for an array of its own the
     // compiler knows which loads-to-LDS may alias a read and waits for every load in flight
     // (s_waitcnt vmcnt(0)) before the first read that follows, which undoes the ring: the loads of
     // the next pages would be waited for at once. What has to have landed is waited for by hand.
-    extern __shared__ __attribute__((aligned(1024))) bf16 attn_lds[];     // keys [2][PAGE * HD], then values [2][HD * PAGE]
-    bf16 (*Ks)[PAGE * HD] = (bf16 (*)[PAGE * HD])attn_lds;
-    bf16 (*Vs)[HD * PAGE] = (bf16 (*)[HD * PAGE])(attn_lds + 2 * PAGE * HD);
+    extern __shared__ __attribute__((aligned(1024))) bf16 attn_lds[];     // [group][keys [2][STAGE], values [2][STAGE]]
 
-    int w = blockIdx.x;
-    {
-        const int round = w / 256, base = round * 256;
-        const int count = total - base < 256 ? total - base : 256;
-        if (round & 1) w = base + count - 1 - (w - base);
-    }
+    const int w = blockIdx.x;
     const int tile = w / per_tile, y = w % per_tile;
     const int G = nq / nkv;
     const int chunks = (G + 3) / 4;
     const int kvh = y / chunks;
     const int chunk = y % chunks;
-    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave8 = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int grp = wave8 >> 2, wave = wave8 & 3;
+    bf16* const Ks = attn_lds + grp * 4 * STAGE;
+    bf16* const Vs = Ks + 2 * STAGE;
     const int c32 = lane & 31, g2 = lane >> 5;
     const int head_in_group = chunk * 4 + wave;
     const bool active = head_in_group < G;
@@ -158,6 +195,10 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache
     const int hi_tile = pos0 + rows - 1;                                     // last visible key
     const int lo_tile = (window > 0 && pos0 + 1 > window) ? pos0 + 1 - window : 0;
     const int first_page = lo_tile / PAGE, last_page = hi_tile / PAGE;
+    // this group's pages: first_page + grp, + 2, ...; the first group has as many as the second or one more
+    const int steps = (last_page - first_page) / 2 + 1;                      // of the first group: every wave loops so often
+    const int mine = last_page - first_page - grp >= 0 ? (last_page - first_page - grp) / 2 + 1 : 0;
+    auto page_of = [&](int i) { return first_page + grp + 2 * i; };
 
     // this lane's part of the loads of a page: element offsets within the page's keys and values
     int k_off[LOADS], v_off[LOADS];
@@ -169,21 +210,23 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache
         const int vr = instr * 8 + lane / 8;
         v_off[i] = vr * PAGE + (((lane & 7) ^ ((vr >> 1) & 7)) * 8);
     }
-    auto issue_keys = [&](int page_idx, int stage) {
-        const bf16* kp = k_cache + ((size_t)pt[page_idx] * nkv + kvh) * PAGE * HD;
+    auto issue_keys = [&](int i, int stage) {
+        const bf16* kp = k_cache + ((size_t)pt[page_of(i)] * nkv + kvh) * PAGE * HD;
 #pragma unroll
-        for (int i = 0; i < LOADS; ++i) hb_load_to_lds(kp + k_off[i], &Ks[stage][(wave * LOADS + i) * 512]);
+        for (int j = 0; j < LOADS; ++j) hb_load_to_lds(kp + k_off[j], Ks + stage * STAGE + (wave * LOADS + j) * 512);
     };
-    auto issue_values = [&](int page_idx, int stage) {
-        const bf16* vp = v_cache + ((size_t)pt[page_idx] * nkv + kvh) * HD * PAGE;
+    auto issue_values = [&](int i, int stage) {
+        const bf16* vp = v_cache + ((size_t)pt[page_of(i)] * nkv + kvh) * HD * PAGE;
 #pragma unroll
-        for (int i = 0; i < LOADS; ++i) hb_load_to_lds(vp + v_off[i], &Vs[stage][(wave * LOADS + i) * 512]);
+        for (int j = 0; j < LOADS; ++j) hb_load_to_lds(vp + v_off[j], Vs + stage * STAGE + (wave * LOADS + j) * 512);
     };
-    // The keys run one page ahead of the values: the scores of page p + 1 are on the matrix cores
-    // while the softmax of page p runs on the vector units.
-    issue_keys(first_page, 0);
-    issue_values(first_page, 0);
-    if (first_page < last_page) issue_keys(first_page + 1, 1);
+    // The keys run one page ahead of the values: the scores of the group's next page are on the
+    // matrix cores while the softmax of this one runs on the vector units.
+    if (mine > 0) {
+        issue_keys(0, 0);
+        issue_values(0, 0);
+    }
+    if (mine > 1) issue_keys(1, 1);
 
     bf16x8 qreg[HD / 16];
     {
@@ -215,52 +258,142 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache
         for (int s = 0; s < HD / 16; ++s)
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb) {
-                const bf16x8 ka = *(const bf16x8*)(&Ks[stage][(kb * 32 + krow) * HD + (((2 * s + g2) ^ k_read[kb]) * 8)]);
+                const bf16x8 ka = *(const bf16x8*)(Ks + stage * STAGE + (kb * 32 + krow) * HD + (((2 * s + g2) ^ k_read[kb]) * 8));
                 st[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qreg[s], st[kb], 0, 0, 0);
             }
     };
-    hb_wait_vmcnt<0>();
-    hb_workgroup_barrier();
-    f32x16 st[2];
-    if (active) scores(0, st);
-    for (int page_idx = first_page; page_idx <= last_page; ++page_idx) {
-        const int it = page_idx - first_page;
+    // The matrix products of one step, in the order in which they are issued: the scores of the next
+    // page S (HD / 8 of them: k-step j / 2 of key block j % 2) and this page's P V (four groups of 8
+    // probabilities x HD / 32 blocks of the output). Between them go the exponentials, one group of
+    // 8 ahead of the P V products that use it, so that the vector units work in the shadow of the
+    // matrix cores within the wave itself: a wave issues in order, and a run of MFMAs followed by a
+    // run of exponentials would leave each unit idle in turn.
+    //   phase 0:        S[0, Q)                              exp of group 0
+    //   phase g = 1..3: S[g Q, (g + 1) Q), P V of group g - 1   exp of group g
+    //   phase 4:        P V of group 3
+    // with Q = HD / 32. The LDS operand of a product is read AHEAD products before it is used.
+    // (The parity of the step is known where the code is written out, twice a round: the stage of an
+    // operand is then a constant offset of its read and costs no register.)
+    constexpr int Q = HD / 32, NM = 8 * Q, AHEAD = 2;
+    auto step_products = [&](auto parity_tag, auto next_tag, f32x16 (&st)[2], f32x16 (&nxt)[2], float mc, float corr) {
+        constexpr int PAR = decltype(parity_tag)::value;
+        constexpr bool NEXT = decltype(next_tag)::value;
+        const bf16* const kst = Ks + ((PAR + 1) & 1) * STAGE;    // the next page's keys
+        const bf16* const vst = Vs + PAR * STAGE;                // this page's values
+        // product n of the step: is it a score product, and which
+        auto is_s = [](int n) { return n < Q || (n < 7 * Q && (n - Q) % (2 * Q) < Q); };
+        auto s_index = [](int n) { return n < Q ? n : ((n - Q) / (2 * Q) + 1) * Q + (n - Q) % (2 * Q); };
+        auto pv_group = [](int n) { return n < 7 * Q ? (n - Q) / (2 * Q) : 3; };
+        auto pv_block = [](int n) { return n < 7 * Q ? (n - Q) % (2 * Q) - Q : n - 7 * Q; };
+        auto operand = [&](int n) -> bf16x8 {
+            if (is_s(n)) {
+                const int j = s_index(n), ks = j / 2, kb = j % 2;
+                return *(const bf16x8*)(kst + (kb * 32 + krow) * HD + (((2 * ks + g2) ^ k_read[kb]) * 8));
+            }
+            const int g = pv_group(n), d = pv_block(n), kb = g >> 1, h2 = g & 1;
+            return *(const bf16x8*)(vst + (d * 32 + c32) * PAGE + (((kb * 4 + h2 * 2 + g2) ^ v_swz) * 8));
+        };
+        if (NEXT) {
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) nxt[kb][e] = 0.f;
+        }
+        bf16x8 ops[NM];
+        bf16x8 pb[4];
+        float sum = 0.f;
+        // exponential e (0..7) of group g: element 8 * (g & 1) + e of key block g >> 1
+        auto exponential = [&](int g, int e) {
+            const float p = fast_exp2(fmaf(st[g >> 1][8 * (g & 1) + e], c, -mc));
+            sum += p;
+            pb[g][e] = (__bf16)p;
+        };
+#pragma unroll
+        for (int n = 0; n < AHEAD; ++n)
+            if (NEXT || !is_s(n)) ops[n] = operand(n);
+#pragma unroll
+        for (int n = 0; n < NM; ++n) {
+            if (n + AHEAD < NM && (NEXT || !is_s(n + AHEAD))) ops[n + AHEAD] = operand(n + AHEAD);
+            if (is_s(n)) {
+                if (NEXT) {
+                    const int j = s_index(n);
+                    nxt[j % 2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ops[n], qreg[j / 2], nxt[j % 2], 0, 0, 0);
+                }
+            } else {
+                const int d = pv_block(n);
+                oacc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ops[n], pb[pv_group(n)], oacc[d], 0, 0, 0);
+            }
+            // the exponentials that go with this product: those of phase g are dealt out over the
+            // phase's products (phase 0 has Q of them, the others 2 Q)
+            if (n < 7 * Q) {
+                const int g = n < Q ? 0 : (n - Q) / (2 * Q) + 1;
+                const int in_phase = n < Q ? n : (n - Q) % (2 * Q), of = n < Q ? Q : 2 * Q;
+#pragma unroll
+                for (int e = in_phase * 8 / of; e < (in_phase + 1) * 8 / of; ++e) exponential(g, e);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        l = l * corr + sum;      // this lane's keys only; the two halves are added at the end
+    };
+    // One step of the group: its page i, whose scores are in `st`; the scores of page i + 1 go to `nxt`.
+    auto step = [&](auto parity_tag, int i, f32x16 (&st)[2], f32x16 (&nxt)[2]) {
         // landed, for every wave after the barrier: the values of this page and the keys of the
-        // next; and nobody reads any more the key stage of this page (its scores are done, those of
-        // the first page too) nor the value stage of the page before, which the next loads fill
+        // next; and nobody reads any more the key stage of this page (its scores are done) nor
+        // the value stage of the page before, which the next loads fill
         hb_wait_vmcnt<0>();
         hb_workgroup_barrier();
-        if (page_idx + 2 <= last_page) issue_keys(page_idx + 2, it & 1);
-        if (page_idx + 1 <= last_page) issue_values(page_idx + 1, (it + 1) & 1);
-        if (!active) continue;
-
-        f32x16 st_next[2];
-        if (page_idx < last_page) scores((it + 1) & 1, st_next);
-        float corr;
-        bf16x8 pb[2][2];
+        if (i + 2 < mine) issue_keys(i + 2, i & 1);
+        if (i + 1 < mine) issue_values(i + 1, (i + 1) & 1);
+        if (!active || i >= mine) return;
+        float corr, mc;
         // a page that every query of the tile sees whole needs no mask
-        const int page0 = page_idx * PAGE;
+        const int page0 = page_of(i) * PAGE;
         if (page0 + PAGE - 1 <= pos0 && (window == 0 || page0 >= hi_tile + 1 - window))
-            softmax_page<false>(st, g2, page0, lo_q, pos_q, c, m, l, corr, pb);
+            mc = softmax_reference<false>(st, g2, page0, lo_q, pos_q, c, m, corr);
         else
-            softmax_page<true>(st, g2, page0, lo_q, pos_q, c, m, l, corr, pb);
-        rescale(oacc, corr);
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-            for (int h2 = 0; h2 < 2; ++h2)
-#pragma unroll
-                for (int d = 0; d < HD / 32; ++d) {
-                    const bf16x8 va = *(const bf16x8*)(&Vs[it & 1][(d * 32 + c32) * PAGE +
-                                                                 (((kb * 4 + h2 * 2 + g2) ^ v_swz) * 8)]);
-                    oacc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb[kb][h2], oacc[d], 0, 0, 0);
-                }
-        if (page_idx < last_page) {
-            st[0] = st_next[0];
-            st[1] = st_next[1];
-        }
+            mc = softmax_reference<true>(st, g2, page0, lo_q, pos_q, c, m, corr);
+        rescale(oacc, corr);          // rarely: the reference moves lazily
+        // (After the group's last page the scores "of the next" are worked out all the same, from
+        // whatever the other key stage holds, and never looked at: a second copy of the code
+        // without them costs more registers than a wave has.)
+        step_products(parity_tag, std::true_type{}, st, nxt, mc, corr);
+    };
+    hb_wait_vmcnt<0>();
+    hb_workgroup_barrier();
+    f32x16 sa[2], sb[2];
+    if (active && mine > 0) scores(0, sa);
+    for (int i = 0; i < steps; i += 2) {           // two steps a round: the scores change places, nothing is copied
+        step(std::integral_constant<int, 0>{}, i, sa, sb);
+        if (i + 1 < steps) step(std::integral_constant<int, 1>{}, i + 1, sb, sa);
     }
-    if (!active || c32 >= rows) return;
+    // The second group hands over what it has: reference, sum and output of every lane, through
+    // the LDS that held the rings (nobody reads those any more after the barrier, and no load
+    // is in flight), [wave][value][lane].
+    hb_wait_vmcnt<0>();
+    hb_workgroup_barrier();
+    float* const hand = (float*)attn_lds + (size_t)wave * (HD / 2 + 2) * 64 + lane;
+    if (grp == 1 && active) {
+        hand[0] = m;
+        hand[64] = l;
+#pragma unroll
+        for (int d = 0; d < HD / 32; ++d)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) hand[(2 + d * 16 + i) * 64] = oacc[d][i];
+    }
+    __syncthreads();
+    if (grp == 1 || !active || c32 >= rows) return;
+    {
+        const float m1 = hand[0], l1 = hand[64];
+        const float mm = fmaxf(m, m1);
+        // (a group without a visible key has the reference -inf, the sum 0 and the output 0)
+        const float a0 = m == -INFINITY ? 0.f : fast_exp2((m - mm) * c);
+        const float a1 = m1 == -INFINITY ? 0.f : fast_exp2((m1 - mm) * c);
+        l = l * a0 + l1 * a1;
+#pragma unroll
+        for (int d = 0; d < HD / 32; ++d)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) oacc[d][i] = oacc[d][i] * a0 + hand[(2 + d * 16 + i) * 64] * a1;
+    }
     l += __shfl_xor(l, 32, 64);
     const float inv = l > 0.f ? 1.0f / l : 0.f;
     bf16* orow = out + ((size_t)(row0 + c32) * nq + h) * HD;
@@ -627,11 +760,22 @@ extern "C" int hb_attn_prefill_mfma(const void* q, const void* k_cache, const vo
     HB_REQUIRE((long)num_tiles * per_tile < (1l << 30), "attn_prefill: too many tiles");
     const int total = num_tiles * per_tile;
     const float c = scale * LOG2E;
+    // two groups of waves, each with two stages of keys and two of values
+    const size_t lds = (size_t)8 * PAGE * hd * sizeof(bf16);
 #define LAUNCH_PREFILL(HDV)                                                                              \
-    attn_prefill_kernel<HDV><<<total, 256, 4 * PAGE * HDV * sizeof(bf16), stream>>>((const bf16*)q, (const bf16*)k_cache, \
-                                                       (const bf16*)v_cache, (bf16*)out, tile_seq, tile_row0, \
-                                                       tile_rows, positions, slots, page_table, max_pages, nq, \
-                                                       nkv, c, window, per_tile, total)
+    do {                                                                                                 \
+        static bool allowed_##HDV = false;      /* once a process (and a device: the attribute is the function's) */ \
+        if (lds > 64 * 1024 && !allowed_##HDV) {                                                         \
+            hipError_t e_ = hipFuncSetAttribute((const void*)attn_prefill_kernel<HDV>,                   \
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);   \
+            HB_REQUIRE(e_ == hipSuccess, "attn_prefill: cannot have %zu bytes of LDS: %s", lds, hipGetErrorString(e_)); \
+            allowed_##HDV = true;                                                                        \
+        }                                                                                                \
+        attn_prefill_kernel<HDV><<<total, 512, lds, stream>>>((const bf16*)q, (const bf16*)k_cache,      \
+                                                             (const bf16*)v_cache, (bf16*)out, tile_seq, tile_row0, \
+                                                             tile_rows, positions, slots, page_table, max_pages, nq, \
+                                                             nkv, c, window, per_tile);                  \
+    } while (0)
     if (hd == 32) LAUNCH_PREFILL(32);
     else if (hd == 64) LAUNCH_PREFILL(64);
     else if (hd == 128) LAUNCH_PREFILL(128);
