@@ -64,6 +64,7 @@ class Engine:
         self.rt = Runtime(_DTYPES[dtype], self.device)
         self.model = Model(spec)
         self.model.load(tensors, self.rt)
+        self._check_cache_fits(max_tokens)
         self.cache = Cache(self.model.cache_needs(), max_tokens, spec.max_positions, self.rt.dtype,
                            self.device, max_slots)
         self.steps_run = 0
@@ -73,6 +74,25 @@ class Engine:
         self.graphs_captured = 0
         self.ignored_tensors = []       # stored tensors that the model did not ask for
         self._tensor_source = None      # how get_tensor finds a tensor again: set by the constructors below
+
+    def _check_cache_fits(self, max_tokens):
+        """Refuse a cache that the GPU's free memory cannot hold, in the library's own words,
+        before the allocator fails on it."""
+        from ..cache import KVNeed, PAGE_TOKENS
+        if self.device.type != "cuda":
+            return
+        pages = (max(int(max_tokens), 1) + PAGE_TOKENS - 1) // PAGE_TOKENS
+        element = 4 if self.rt.exact else 2
+        needed = 0
+        for need in self.model.cache_needs().values():
+            for one in (need if isinstance(need, (tuple, list)) else (need,)):
+                if isinstance(one, KVNeed):
+                    needed += 2 * pages * PAGE_TOKENS * one.kv_heads * one.head_dim * element
+        free, _ = torch.cuda.mem_get_info(self.device)
+        if needed > free:
+            from ..errors import CacheError
+            raise CacheError(f"a cache of {max_tokens} tokens needs {needed / 2**30:.1f} GiB of keys and values, "
+                             f"{free / 2**30:.1f} GiB of GPU memory are free")
 
     # ---- construction
     @classmethod
