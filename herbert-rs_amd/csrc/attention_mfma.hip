@@ -137,6 +137,84 @@ __device__ __forceinline__ float softmax_reference(f32x16 st[2], int g2, int pag
 }
 
 // ----------------------------------------------------------------- prefill
+// What a lane needs to find its operands in the LDS stages of a page's keys and values.
+struct PrefillLane {
+    int c32, g2, krow, k_read[2], v_swz;
+};
+
+// The matrix products of one step of the prompt kernels, in the order in which they are issued:
+// the scores of the next page S (HD / 8 of them: k-step j / 2 of key block j % 2) and this page's
+// P V (four groups of 8 probabilities x HD / 32 blocks of the output). Between them go the
+// exponentials, one group of 8 ahead of the P V products that use it, so that the vector units
+// work in the shadow of the matrix cores within the wave itself: a wave issues in order, and a
+// run of MFMAs followed by a run of exponentials would leave each unit idle in turn.
+//   phase 0:        S[0, Q)                                 exp of group 0
+//   phase g = 1..3: S[g Q, (g + 1) Q), P V of group g - 1   exp of group g
+//   phase 4:        P V of group 3
+// with Q = HD / 32. The LDS operand of a product is read AHEAD products before it is used.
+// kst: the stage of the next page's keys; vst: the stage of this page's values. After the last
+// page the scores "of the next" are worked out all the same, from whatever that stage holds,
+// and never looked at: a second copy of the code without them costs more registers than a wave has.
+template <int HD>
+__device__ __forceinline__ void prefill_step_products(const bf16* kst, const bf16* vst, f32x16 (&st)[2],
+                                                      f32x16 (&nxt)[2], f32x16 (&oacc)[HD / 32],
+                                                      const bf16x8 (&qreg)[HD / 16], const PrefillLane& ln, float c,
+                                                      float mc, float corr, float& l) {
+    constexpr int Q = HD / 32, NM = 8 * Q, AHEAD = 3;
+    const int c32 = ln.c32, g2 = ln.g2, krow = ln.krow, v_swz = ln.v_swz;
+    // product n of the step: is it a score product, and which
+    auto is_s = [](int n) { return n < Q || (n < 7 * Q && (n - Q) % (2 * Q) < Q); };
+    auto s_index = [](int n) { return n < Q ? n : ((n - Q) / (2 * Q) + 1) * Q + (n - Q) % (2 * Q); };
+    auto pv_group = [](int n) { return n < 7 * Q ? (n - Q) / (2 * Q) : 3; };
+    auto pv_block = [](int n) { return n < 7 * Q ? (n - Q) % (2 * Q) - Q : n - 7 * Q; };
+    constexpr int KRPB = 128 / HD > 0 ? 128 / HD : 1;
+    auto operand = [&](int n) -> bf16x8 {
+        if (is_s(n)) {
+            const int j = s_index(n), ks = j / 2, kb = j % 2;
+            return *(const bf16x8*)(kst + (kb * 32 + krow) * HD + (((2 * ks + g2) ^ ln.k_read[kb]) * 8));
+        }
+        const int g = pv_group(n), d = pv_block(n), kb = g >> 1, h2 = g & 1;
+        return *(const bf16x8*)(vst + (d * 32 + c32) * PAGE + (((kb * 4 + h2 * 2 + g2) ^ v_swz) * 8));
+    };
+    (void)KRPB;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) nxt[kb][e] = 0.f;
+    bf16x8 ops[NM];
+    bf16x8 pb[4];
+    float sum = 0.f;
+    // exponential e (0..7) of group g: element 8 * (g & 1) + e of key block g >> 1
+    auto exponential = [&](int g, int e) {
+        const float p = fast_exp2(fmaf(st[g >> 1][8 * (g & 1) + e], c, -mc));
+        sum += p;
+        pb[g][e] = (__bf16)p;
+    };
+#pragma unroll
+    for (int n = 0; n < AHEAD; ++n) ops[n] = operand(n);
+#pragma unroll
+    for (int n = 0; n < NM; ++n) {
+        if (n + AHEAD < NM) ops[n + AHEAD] = operand(n + AHEAD);
+        if (is_s(n)) {
+            const int j = s_index(n);
+            nxt[j % 2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ops[n], qreg[j / 2], nxt[j % 2], 0, 0, 0);
+        } else {
+            const int d = pv_block(n);
+            oacc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ops[n], pb[pv_group(n)], oacc[d], 0, 0, 0);
+        }
+        // the exponentials that go with this product: those of phase g are dealt out over the
+        // phase's products (phase 0 has Q of them, the others 2 Q)
+        if (n < 7 * Q) {
+            const int g = n < Q ? 0 : (n - Q) / (2 * Q) + 1;
+            const int in_phase = n < Q ? n : (n - Q) % (2 * Q), of = n < Q ? Q : 2 * Q;
+#pragma unroll
+            for (int e = in_phase * 8 / of; e < (in_phase + 1) * 8 / of; ++e) exponential(g, e);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    l = l * corr + sum;      // this lane's keys only; the two halves are added at the end
+}
+
 // A workgroup: 32 queries x up to 4 query heads of one kv head, by eight waves in two groups of
 // four (a wave a head in each group). The groups take the tile's pages in turn, the first the
 // even ones and the second the odd ones, each with a reference, a sum and an output of its
@@ -247,6 +325,7 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) k_read[kb] = ((kb * 32 + krow) / KRPB) % KCH;
     const int v_swz = (c32 >> 1) & 7;            // of rows d * 32 + c32
+    const PrefillLane ln = {c32, g2, krow, {k_read[0], k_read[1]}, v_swz};
     // raw scores of the page in a key stage; the two key blocks alternate, so that no MFMA waits
     // for the one before it
     auto scores = [&](int stage, f32x16 (&st)[2]) {
@@ -261,79 +340,6 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache
                 const bf16x8 ka = *(const bf16x8*)(Ks + stage * STAGE + (kb * 32 + krow) * HD + (((2 * s + g2) ^ k_read[kb]) * 8));
                 st[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qreg[s], st[kb], 0, 0, 0);
             }
-    };
-    // The matrix products of one step, in the order in which they are issued: the scores of the next
-    // page S (HD / 8 of them: k-step j / 2 of key block j % 2) and this page's P V (four groups of 8
-    // probabilities x HD / 32 blocks of the output). Between them go the exponentials, one group of
-    // 8 ahead of the P V products that use it, so that the vector units work in the shadow of the
-    // matrix cores within the wave itself: a wave issues in order, and a run of MFMAs followed by a
-    // run of exponentials would leave each unit idle in turn.
-    //   phase 0:        S[0, Q)                              exp of group 0
-    //   phase g = 1..3: S[g Q, (g + 1) Q), P V of group g - 1   exp of group g
-    //   phase 4:        P V of group 3
-    // with Q = HD / 32. The LDS operand of a product is read AHEAD products before it is used.
-    // (The parity of the step is known where the code is written out, twice a round: the stage of an
-    // operand is then a constant offset of its read and costs no register.)
-    constexpr int Q = HD / 32, NM = 8 * Q, AHEAD = 2;
-    auto step_products = [&](auto parity_tag, auto next_tag, f32x16 (&st)[2], f32x16 (&nxt)[2], float mc, float corr) {
-        constexpr int PAR = decltype(parity_tag)::value;
-        constexpr bool NEXT = decltype(next_tag)::value;
-        const bf16* const kst = Ks + ((PAR + 1) & 1) * STAGE;    // the next page's keys
-        const bf16* const vst = Vs + PAR * STAGE;                // this page's values
-        // product n of the step: is it a score product, and which
-        auto is_s = [](int n) { return n < Q || (n < 7 * Q && (n - Q) % (2 * Q) < Q); };
-        auto s_index = [](int n) { return n < Q ? n : ((n - Q) / (2 * Q) + 1) * Q + (n - Q) % (2 * Q); };
-        auto pv_group = [](int n) { return n < 7 * Q ? (n - Q) / (2 * Q) : 3; };
-        auto pv_block = [](int n) { return n < 7 * Q ? (n - Q) % (2 * Q) - Q : n - 7 * Q; };
-        auto operand = [&](int n) -> bf16x8 {
-            if (is_s(n)) {
-                const int j = s_index(n), ks = j / 2, kb = j % 2;
-                return *(const bf16x8*)(kst + (kb * 32 + krow) * HD + (((2 * ks + g2) ^ k_read[kb]) * 8));
-            }
-            const int g = pv_group(n), d = pv_block(n), kb = g >> 1, h2 = g & 1;
-            return *(const bf16x8*)(vst + (d * 32 + c32) * PAGE + (((kb * 4 + h2 * 2 + g2) ^ v_swz) * 8));
-        };
-        if (NEXT) {
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) nxt[kb][e] = 0.f;
-        }
-        bf16x8 ops[NM];
-        bf16x8 pb[4];
-        float sum = 0.f;
-        // exponential e (0..7) of group g: element 8 * (g & 1) + e of key block g >> 1
-        auto exponential = [&](int g, int e) {
-            const float p = fast_exp2(fmaf(st[g >> 1][8 * (g & 1) + e], c, -mc));
-            sum += p;
-            pb[g][e] = (__bf16)p;
-        };
-#pragma unroll
-        for (int n = 0; n < AHEAD; ++n)
-            if (NEXT || !is_s(n)) ops[n] = operand(n);
-#pragma unroll
-        for (int n = 0; n < NM; ++n) {
-            if (n + AHEAD < NM && (NEXT || !is_s(n + AHEAD))) ops[n + AHEAD] = operand(n + AHEAD);
-            if (is_s(n)) {
-                if (NEXT) {
-                    const int j = s_index(n);
-                    nxt[j % 2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ops[n], qreg[j / 2], nxt[j % 2], 0, 0, 0);
-                }
-            } else {
-                const int d = pv_block(n);
-                oacc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ops[n], pb[pv_group(n)], oacc[d], 0, 0, 0);
-            }
-            // the exponentials that go with this product: those of phase g are dealt out over the
-            // phase's products (phase 0 has Q of them, the others 2 Q)
-            if (n < 7 * Q) {
-                const int g = n < Q ? 0 : (n - Q) / (2 * Q) + 1;
-                const int in_phase = n < Q ? n : (n - Q) % (2 * Q), of = n < Q ? Q : 2 * Q;
-#pragma unroll
-                for (int e = in_phase * 8 / of; e < (in_phase + 1) * 8 / of; ++e) exponential(g, e);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        l = l * corr + sum;      // this lane's keys only; the two halves are added at the end
     };
     // One step of the group: its page i, whose scores are in `st`; the scores of page i + 1 go to `nxt`.
     auto step = [&](auto parity_tag, int i, f32x16 (&st)[2], f32x16 (&nxt)[2]) {
@@ -353,10 +359,10 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache
         else
             mc = softmax_reference<true>(st, g2, page0, lo_q, pos_q, c, m, corr);
         rescale(oacc, corr);          // rarely: the reference moves lazily
-        // (After the group's last page the scores "of the next" are worked out all the same, from
-        // whatever the other key stage holds, and never looked at: a second copy of the code
-        // without them costs more registers than a wave has.)
-        step_products(parity_tag, std::true_type{}, st, nxt, mc, corr);
+        // (the parity of the step is known where the code is written out, twice a round: the stage
+        // of an operand is then a constant offset of its read and costs no register)
+        constexpr int PAR = decltype(parity_tag)::value;
+        prefill_step_products<HD>(Ks + ((PAR + 1) & 1) * STAGE, Vs + PAR * STAGE, st, nxt, oacc, qreg, ln, c, mc, corr, l);
     };
     hb_wait_vmcnt<0>();
     hb_workgroup_barrier();
@@ -394,6 +400,179 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache
 #pragma unroll
             for (int i = 0; i < 16; ++i) oacc[d][i] = oacc[d][i] * a0 + hand[(2 + d * 16 + i) * 64] * a1;
     }
+    l += __shfl_xor(l, 32, 64);
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    bf16* orow = out + ((size_t)(row0 + c32) * nq + h) * HD;
+#pragma unroll
+    for (int d = 0; d < HD / 32; ++d)
+#pragma unroll
+        for (int qd = 0; qd < 4; ++qd) {
+            bf16x4 v;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) v[r] = (__bf16)(oacc[d][4 * qd + r] * inv);
+            *(bf16x4*)(orow + d * 32 + 8 * qd + 4 * g2) = v;
+        }
+}
+
+// The prompt kernel for long prompts (many tiles, all of them long): a workgroup is 64 consecutive
+// tokens x up to 4 query heads of one kv head; its eight waves are two halves of 32 tokens (a wave
+// a head in each) that share the pages: one ring of three LDS stages for the keys and one for the
+// values, every page loaded once for both halves, so that half as many bytes go into LDS for a
+// product and a page's loads have two steps to land instead of one (the kernel above waits for
+// its loads for a third of its time). No merge at the end: a half owns its rows.
+// Every wave issues the same number of loads in every step (past the last page: that page again,
+// into a stage nobody reads any more), so that the wait before the barrier can count: all but
+// the loads of the step before have landed.
+template <int HD>
+__global__ void __launch_bounds__(512, 1)
+attn_prefill_long_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_cache,
+                         const bf16* __restrict__ v_cache, bf16* __restrict__ out,
+                         const int* __restrict__ tile_seq, const int* __restrict__ tile_row0,
+                         const int* __restrict__ tile_rows, const int* __restrict__ positions,
+                         const int* __restrict__ slots, const int* __restrict__ page_table, int max_pages,
+                         int nq, int nkv, float c, int window, int per_tile) {
+    constexpr int KCH = HD / 8;
+    constexpr int KRPB = 128 / HD > 0 ? 128 / HD : 1;
+    constexpr int KROWS = 512 / HD;
+    constexpr int INSTRS = HD / 8;                // load instructions (1 KB each) for the keys of a page; as many for the values
+    constexpr int PL = INSTRS >= 8 ? INSTRS / 8 : 1;   // of which a wave issues (with fewer than 8, the first waves one each)
+    constexpr int STAGE = PAGE * HD;
+    extern __shared__ __attribute__((aligned(1024))) bf16 attn_lds[];     // keys [3][STAGE], values [3][STAGE]
+    bf16* const Ks = attn_lds;
+    bf16* const Vs = attn_lds + 3 * STAGE;
+
+    const int w = blockIdx.x;
+    const int tile = w / per_tile, y = w % per_tile;
+    const int G = nq / nkv;
+    const int chunks = (G + 3) / 4;
+    const int kvh = y / chunks;
+    const int chunk = y % chunks;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave8 = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int half = wave8 >> 2, wave = wave8 & 3;
+    const int c32 = lane & 31, g2 = lane >> 5;
+    const int head_in_group = chunk * 4 + wave;
+
+    const int tile_row = tile_row0[tile], tile_n = tile_rows[tile];          // up to 64 rows
+    const int rows = tile_n - 32 * half < 32 ? tile_n - 32 * half : 32;      // of this half; <= 0: it has none
+    const bool active = head_in_group < G && rows > 0;
+    const int h = kvh * G + (head_in_group < G ? head_in_group : G - 1);
+    const int row0 = tile_row + (rows > 0 ? 32 * half : 0);
+    const int slot = slots[tile_seq[tile]];
+    const int* pt = page_table + (size_t)slot * max_pages;
+    const int tile_pos0 = positions[tile_row];
+    const int pos0 = tile_pos0 + (rows > 0 ? 32 * half : 0);
+    const int my_row = rows > 0 ? (c32 < rows ? c32 : rows - 1) : 0;
+    const int pos_q = pos0 + my_row;
+    const int lo_q = (window > 0 && pos_q + 1 > window) ? pos_q + 1 - window : 0;
+    const int hi_half = pos0 + (rows > 0 ? rows : 1) - 1;                     // last key this half sees
+    // the workgroup's pages: from the first a row of the tile sees to the last
+    const int lo_tile = (window > 0 && tile_pos0 + 1 > window) ? tile_pos0 + 1 - window : 0;
+    const int first_page = lo_tile / PAGE, last_page = (tile_pos0 + tile_n - 1) / PAGE;
+    const int steps = last_page - first_page + 1;
+    const int mine = active ? hi_half / PAGE - first_page + 1 : 0;            // this half's steps: pages up to its own last
+    auto page_of = [&](int i) { return first_page + (i < steps ? i : steps - 1); };   // past the end: the last page again
+
+    int k_off[PL], v_off[PL];
+    const bool loads = INSTRS >= 8 || wave8 < INSTRS;
+#pragma unroll
+    for (int i = 0; i < PL; ++i) {
+        const int instr = (INSTRS >= 8 ? wave8 * PL + i : wave8) % INSTRS;
+        const int kr = instr * KROWS + lane / KCH;
+        k_off[i] = kr * HD + (((lane % KCH) ^ ((kr / KRPB) % KCH)) * 8);
+        const int vr = instr * 8 + lane / 8;
+        v_off[i] = vr * PAGE + (((lane & 7) ^ ((vr >> 1) & 7)) * 8);
+    }
+    auto issue_keys = [&](int i) {
+        if (!loads) return;
+        const bf16* kp = k_cache + ((size_t)pt[page_of(i)] * nkv + kvh) * PAGE * HD;
+#pragma unroll
+        for (int j = 0; j < PL; ++j) {
+            const int instr = (INSTRS >= 8 ? wave8 * PL + j : wave8) % INSTRS;
+            hb_load_to_lds(kp + k_off[j], Ks + (i % 3) * STAGE + instr * 512);
+        }
+    };
+    auto issue_values = [&](int i) {
+        if (!loads) return;
+        const bf16* vp = v_cache + ((size_t)pt[page_of(i)] * nkv + kvh) * HD * PAGE;
+#pragma unroll
+        for (int j = 0; j < PL; ++j) {
+            const int instr = (INSTRS >= 8 ? wave8 * PL + j : wave8) % INSTRS;
+            hb_load_to_lds(vp + v_off[j], Vs + (i % 3) * STAGE + instr * 512);
+        }
+    };
+    // in flight before the first step: the keys of pages 0, 1, 2 and the values of pages 0, 1; the
+    // last two of these five are what a step leaves in flight
+    issue_keys(0);
+    issue_values(0);
+    issue_keys(1);
+    issue_values(1);
+    issue_keys(2);
+
+    bf16x8 qreg[HD / 16];
+    {
+        const bf16* qrow = q + ((size_t)(row0 + my_row) * nq + h) * HD + g2 * 8;
+#pragma unroll
+        for (int s2 = 0; s2 < HD / 16; ++s2) qreg[s2] = *(const bf16x8*)(qrow + s2 * 16);
+    }
+    f32x16 oacc[HD / 32];
+#pragma unroll
+    for (int d = 0; d < HD / 32; ++d)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) oacc[d][i] = 0.f;
+    float m = -INFINITY, l = 0.f;
+    const int krow = perm(c32);
+    PrefillLane ln;
+    ln.c32 = c32;
+    ln.g2 = g2;
+    ln.krow = krow;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) ln.k_read[kb] = ((kb * 32 + krow) / KRPB) % KCH;
+    ln.v_swz = (c32 >> 1) & 7;
+
+    auto step = [&](int i, f32x16 (&st)[2], f32x16 (&nxt)[2]) {
+        // landed, for every wave after the barrier: all but what the step before asked for, that is
+        // the keys of page i + 1 and the values of page i; and nobody reads any more the stages that
+        // this step's loads fill (the keys of page i, the values of page i - 1)
+        if (loads) hb_wait_vmcnt<2 * PL>();
+        hb_workgroup_barrier();
+        issue_values(i + 2);
+        issue_keys(i + 3);
+        if (i >= mine) return;
+        float corr, mc;
+        const int page0 = page_of(i) * PAGE;
+        if (page0 + PAGE - 1 <= pos0 && (window == 0 || page0 >= hi_half + 1 - window))
+            mc = softmax_reference<false>(st, g2, page0, lo_q, pos_q, c, m, corr);
+        else
+            mc = softmax_reference<true>(st, g2, page0, lo_q, pos_q, c, m, corr);
+        rescale(oacc, corr);
+        prefill_step_products<HD>(Ks + ((i + 1) % 3) * STAGE, Vs + (i % 3) * STAGE, st, nxt, oacc, qreg, ln, c, mc,
+                                  corr, l);
+    };
+    // the first page's scores: its keys are the oldest of the five sets of loads (and of the
+    // query's own loads behind them)
+    if (loads) hb_wait_vmcnt<3 * PL>();
+    hb_workgroup_barrier();
+    f32x16 sa[2], sb[2];
+    if (mine > 0) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) sa[kb][i] = 0.f;
+#pragma unroll
+        for (int s2 = 0; s2 < HD / 16; ++s2)
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+                const bf16x8 ka = *(const bf16x8*)(Ks + (kb * 32 + krow) * HD + (((2 * s2 + g2) ^ ln.k_read[kb]) * 8));
+                sa[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qreg[s2], sa[kb], 0, 0, 0);
+            }
+    }
+    for (int i = 0; i < steps; i += 2) {
+        step(i, sa, sb);
+        if (i + 1 < steps) step(i + 1, sb, sa);
+    }
+    hb_wait_vmcnt<0>();          // nothing of this workgroup's is in flight when it ends
+    if (!active || c32 >= rows) return;
     l += __shfl_xor(l, 32, 64);
     const float inv = l > 0.f ? 1.0f / l : 0.f;
     bf16* orow = out + ((size_t)(row0 + c32) * nq + h) * HD;
@@ -750,36 +929,44 @@ extern "C" int hb_attn_prefill_mfma(const void* q, const void* k_cache, const vo
                                     const int* tile_seq, const int* tile_row0, const int* tile_rows,
                                     int num_tiles, const int* positions, const int* slots,
                                     const int* page_table, int max_pages, int page_size, int nq, int nkv,
-                                    int hd, float scale, int window, hipStream_t stream) {
+                                    int hd, float scale, int window, int tile_height, hipStream_t stream) {
     HB_REQUIRE(num_tiles > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attn_prefill: bad sizes");
     HB_REQUIRE(page_size == PAGE, "attn_prefill: pages must hold %d tokens", PAGE);
     HB_REQUIRE(window >= 0, "attn_prefill: bad window");
     HB_REQUIRE(scale > 0.f, "attn_prefill: the score scale must be positive");
+    HB_REQUIRE(tile_height == 32 || tile_height == 64, "attn_prefill: tiles are 32 or 64 tokens high");
     const int G = nq / nkv;
     const int per_tile = nkv * ((G + 3) / 4);
     HB_REQUIRE((long)num_tiles * per_tile < (1l << 30), "attn_prefill: too many tiles");
     const int total = num_tiles * per_tile;
     const float c = scale * LOG2E;
-    // two groups of waves, each with two stages of keys and two of values
-    const size_t lds = (size_t)8 * PAGE * hd * sizeof(bf16);
-#define LAUNCH_PREFILL(HDV)                                                                              \
+    // tiles of 32 tokens: two groups of waves, each with two stages of keys and two of values;
+    // tiles of 64: one ring of three stages of keys and three of values
+    const size_t lds = (size_t)(tile_height == 64 ? 6 : 8) * PAGE * hd * sizeof(bf16);
+#define LAUNCH_PREFILL(KERNEL, HDV)                                                                      \
     do {                                                                                                 \
-        static bool allowed_##HDV = false;      /* once a process (and a device: the attribute is the function's) */ \
-        if (lds > 64 * 1024 && !allowed_##HDV) {                                                         \
-            hipError_t e_ = hipFuncSetAttribute((const void*)attn_prefill_kernel<HDV>,                   \
+        static bool allowed = false;            /* once a process (the attribute is the function's) */   \
+        if (lds > 64 * 1024 && !allowed) {                                                               \
+            hipError_t e_ = hipFuncSetAttribute((const void*)KERNEL<HDV>,                                \
                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);   \
             HB_REQUIRE(e_ == hipSuccess, "attn_prefill: cannot have %zu bytes of LDS: %s", lds, hipGetErrorString(e_)); \
-            allowed_##HDV = true;                                                                        \
+            allowed = true;                                                                              \
         }                                                                                                \
-        attn_prefill_kernel<HDV><<<total, 512, lds, stream>>>((const bf16*)q, (const bf16*)k_cache,      \
-                                                             (const bf16*)v_cache, (bf16*)out, tile_seq, tile_row0, \
-                                                             tile_rows, positions, slots, page_table, max_pages, nq, \
-                                                             nkv, c, window, per_tile);                  \
+        KERNEL<HDV><<<total, 512, lds, stream>>>((const bf16*)q, (const bf16*)k_cache, (const bf16*)v_cache, \
+                                                 (bf16*)out, tile_seq, tile_row0, tile_rows, positions, slots, \
+                                                 page_table, max_pages, nq, nkv, c, window, per_tile);   \
     } while (0)
-    if (hd == 32) LAUNCH_PREFILL(32);
-    else if (hd == 64) LAUNCH_PREFILL(64);
-    else if (hd == 128) LAUNCH_PREFILL(128);
-    else HB_REQUIRE(false, "attn_prefill: head_dim %d is not one of 32, 64, 128", hd);
+    if (tile_height == 64) {
+        if (hd == 32) LAUNCH_PREFILL(attn_prefill_long_kernel, 32);
+        else if (hd == 64) LAUNCH_PREFILL(attn_prefill_long_kernel, 64);
+        else if (hd == 128) LAUNCH_PREFILL(attn_prefill_long_kernel, 128);
+        else HB_REQUIRE(false, "attn_prefill: head_dim %d is not one of 32, 64, 128", hd);
+    } else {
+        if (hd == 32) LAUNCH_PREFILL(attn_prefill_kernel, 32);
+        else if (hd == 64) LAUNCH_PREFILL(attn_prefill_kernel, 64);
+        else if (hd == 128) LAUNCH_PREFILL(attn_prefill_kernel, 128);
+        else HB_REQUIRE(false, "attn_prefill: head_dim %d is not one of 32, 64, 128", hd);
+    }
 #undef LAUNCH_PREFILL
     HB_CHECK_LAUNCH("attn_prefill");
     return 0;

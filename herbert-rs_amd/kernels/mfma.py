@@ -307,7 +307,7 @@ def gemm_swiglu(a, w_interleaved, out, packed=False, norm=None, tile=0, row_scal
 
 
 lib.register_signatures("attention_mfma", {
-    "hb_attn_prefill_mfma": [_P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P],
+    "hb_attn_prefill_mfma": [_P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I, _P],
     "hb_attn_decode_mfma": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I,
                             _P, _P, _P, _P, _P, _F, _I, _I, ctypes.c_size_t, _P],
 })
@@ -324,24 +324,35 @@ def attention_supported(q, kv, nq, nkv, hd):
             and hd in ATTENTION_HEAD_DIMS and nq % nkv == 0 and nq // nkv <= 32)
 
 
-def _prefill_tiles(meta):
-    """Device arrays (sequence, first packed row, rows) of the 32-token query tiles of a step,
-    those that see the most keys first: the kernel deals them out heaviest first."""
-    tiles = meta.derived.get("prefill_tiles")
+PREFILL_LONG_MIN_WORKGROUPS = 512      # from so many workgroups of 64-token tiles on (measured: 4 K tokens of 8 kv heads 200 -> 176 us, 2 K 57 -> 70): the kernel for long prompts
+
+
+def _prefill_tile_height(meta, nkv, group):
+    """32, or 64 where the step has so many tokens that tiles of 64 still make several rounds of
+    workgroups: the kernel for those loads every page once for 64 tokens and has its loads two
+    steps ahead; with fewer, tiles of 32 whose pages two groups of waves take in turn end sooner."""
+    tiles = sum(-(-(int(meta.host_starts[i + 1]) - int(meta.host_starts[i])) // 64) for i in range(meta.num_seqs))
+    return 64 if tiles * nkv * -(-group // 4) >= PREFILL_LONG_MIN_WORKGROUPS else 32
+
+
+def _prefill_tiles(meta, height=QUERY_TILE):
+    """Device arrays (sequence, first packed row, rows) of the query tiles of a step (`height` tokens
+    each), those that see the most keys first: the kernel deals them out heaviest first."""
+    tiles = meta.derived.get(("prefill_tiles", height))
     if tiles is None:
         items = []
         starts, context = meta.host_starts, meta.host_context
         for i in range(meta.num_seqs):
             a, b = int(starts[i]), int(starts[i + 1])
-            for r in range(a, b, QUERY_TILE):
-                n = min(QUERY_TILE, b - r)
+            for r in range(a, b, height):
+                n = min(height, b - r)
                 last_position = int(context[i]) - (b - (r + n)) - 1
                 items.append((-last_position, i, r, n))
         items.sort()
         seq, row0, rows = [it[1] for it in items], [it[2] for it in items], [it[3] for it in items]
         packed = torch.tensor([seq, row0, rows], dtype=torch.int32).to(meta.positions.device)
         tiles = (packed[0], packed[1], packed[2], len(seq))
-        meta.derived["prefill_tiles"] = tiles
+        meta.derived[("prefill_tiles", height)] = tiles
     return tiles
 
 
@@ -440,9 +451,10 @@ def attention_decode_fused(qkv, q_norm_w, k_norm_w, cos, sin, meta, kv, out, nq,
 DEFERRED_SLICES = (2, 4, 8)     # numbers of slices of the projection that the decode kernel adds up itself
 
 
-def attention(q, meta, kv, out, nq, nkv, hd, scale, window):
+def attention(q, meta, kv, out, nq, nkv, hd, scale, window, tile_height=None):
     """Causal (and windowed) attention of the step's tokens over their slots' pages.
-    One token a sequence: the split decode kernel; otherwise the tiled prefill kernel."""
+    One token a sequence: the split decode kernel; otherwise one of the two tiled prompt kernels
+    (tile_height 32 or 64 asks for one by name; None: the host's choice, see _prefill_tile_height)."""
     T = q.shape[0]
     _check(q, "q", torch.bfloat16, (T, nq * hd))
     _check(out, "out", torch.bfloat16, (T, nq * hd))
@@ -467,8 +479,11 @@ def attention(q, meta, kv, out, nq, nkv, hd, scale, window):
                  _stream())
         return
     _check(meta.positions, "positions", torch.int32, (T,))
-    tile_seq, tile_row0, tile_rows, n_tiles = _prefill_tiles(meta)
+    height = tile_height or _prefill_tile_height(meta, nkv, nq // nkv)
+    if height not in (32, 64):
+        raise BackendError("prompt attention has tiles of 32 or of 64 tokens")
+    tile_seq, tile_row0, tile_rows, n_tiles = _prefill_tiles(meta, height)
     lib.call("attention_mfma", "hb_attn_prefill_mfma", q.data_ptr(), kv.k.data_ptr(), kv.v.data_ptr(),
              out.data_ptr(), tile_seq.data_ptr(), tile_row0.data_ptr(), tile_rows.data_ptr(), n_tiles,
              meta.positions.data_ptr(), meta.slots.data_ptr(), kv.page_table.data_ptr(),
-             kv.page_table.shape[1], kv.page_size, nq, nkv, hd, float(scale), window, _stream())
+             kv.page_table.shape[1], kv.page_size, nq, nkv, hd, float(scale), window, height, _stream())

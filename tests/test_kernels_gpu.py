@@ -234,17 +234,21 @@ def test_attention_plain(nq, nkv, hd, window, dtype):
     assert float((out.float().cpu() - want).abs().max()) <= tol * float(want.abs().max())
 
 
+@pytest.mark.parametrize("tile_height", [32, 64])
 @pytest.mark.parametrize("nq,nkv,hd,window", [(4, 1, 128, 0), (8, 2, 64, 0), (6, 2, 32, 0), (5, 1, 64, 70),
                                               (3, 3, 128, 100), (16, 2, 128, 0), (2, 2, 32, 0)])
-def test_attention_mfma_prefill(nq, nkv, hd, window):
+def test_attention_mfma_prefill(nq, nkv, hd, window, tile_height):
+    """Both prompt kernels, each asked for by name: tiles of 32 tokens (two groups of waves take a
+    tile's pages in turn) and tiles of 64 (two halves share the pages). Sequences that start in
+    the cache at positions that no tile height divides, tiles of 1 to 64 rows, windows."""
     from herbert_rs_amd.kernels import mfma
-    lengths, new = [5, 200, 64, 129, 33, 300], [5, 70, 2, 129, 32, 300]
+    lengths, new = [5, 200, 64, 129, 33, 300, 450], [5, 70, 2, 129, 32, 300, 97]
     meta, kv, dense = paged_case(lengths, new, nkv, hd, torch.bfloat16, seed=nq + hd)
     q = rand(sum(new), nq * hd, seed=21, dtype=torch.bfloat16)
     out = torch.full_like(q, 9.0)
     scale = hd ** -0.5
     assert mfma.attention_supported(q, kv, nq, nkv, hd)
-    mfma.attention(q, meta, kv, out, nq, nkv, hd, scale, window)
+    mfma.attention(q, meta, kv, out, nq, nkv, hd, scale, window, tile_height=tile_height)
     want = attention_reference(q, meta, dense, nq, nkv, hd, scale, window)
     # probabilities and the output are rounded to bfloat16 (2^-9 each)
     assert float((out.float().cpu() - want).abs().max()) <= 2 ** -7 * float(want.abs().max())
@@ -655,14 +659,18 @@ def test_gemm_mfma_refuses_a_handed_norm_it_cannot_do():
                   accumulate=True, row_scale=(squares, 1e-6))
 
 
-@pytest.mark.parametrize("tile", [0, 188, 142, 122, 123, 112, 124, 184])
-@pytest.mark.parametrize("M,N,K,packed", [(65, 128, 64, True), (200, 336, 192, True), (300, 530, 96, False),
-                                          (513, 1040, 256, True), (2300, 528, 128, True), (17, 272, 64, True),
-                                          (40, 530, 320, False), (64, 1040, 128, True)])
+# every tile with every size it takes (K in steps of 32 goes to the host's own choice and to tile 123 only)
+TILE_CASES = [(tile, M, N, K, packed)
+              for tile in (0, 188, 142, 122, 123, 112, 124, 184)
+              for M, N, K, packed in [(65, 128, 64, True), (200, 336, 192, True), (300, 530, 96, False),
+                                      (513, 1040, 256, True), (2300, 528, 128, True), (17, 272, 64, True),
+                                      (40, 530, 320, False), (64, 1040, 128, True)]
+              if K % 64 == 0 or tile in (0, 123)]
+
+
+@pytest.mark.parametrize("tile,M,N,K,packed", TILE_CASES)
 def test_gemm_mfma_tile_variants(tile, M, N, K, packed):
     from herbert_rs_amd.kernels import mfma
-    if K % 64 and tile not in (0, 123):
-        pytest.skip("this tile takes K in steps of 64")
     a = rand(M, K, seed=7, dtype=torch.bfloat16)
     w = rand(N, K, seed=8, dtype=torch.bfloat16)
     want = (a.double() @ w.double().T).float()
@@ -685,18 +693,26 @@ def test_gemm_mfma_tile_variants(tile, M, N, K, packed):
         assert float((out.float() - wanted).abs().max()) <= 2 ** -7 * float(wanted.abs().max()) + 1e-4
 
 
-@pytest.mark.parametrize("tile", [0, 2122, 4188, 3142, 8122, 4112, 16124, 2184])
-@pytest.mark.parametrize("M,N,K,packed", [(200, 336, 512, True), (513, 1040, 768, True), (128, 1024, 4096, True),
-                                          (300, 530, 1024, False), (24, 1056, 2112, True), (64, 8192, 1024, True),
-                                          (33, 336, 4096, False)])
+def _slices_fit(tile, K):
+    """A tile number's slices (its thousands) are no more than the workspace is sized for and leave no slice empty."""
+    slices, steps = tile // 1000, K // 64
+    return slices <= 1 or (slices <= min(16, K // 256) and -(-steps // slices) * (slices - 1) < steps)
+
+
+SLICE_CASES = [(tile, M, N, K, packed)
+               for tile in (0, 2122, 4188, 3142, 8122, 4112, 16124, 2184)
+               for M, N, K, packed in [(200, 336, 512, True), (513, 1040, 768, True), (128, 1024, 4096, True),
+                                       (300, 530, 1024, False), (24, 1056, 2112, True), (64, 8192, 1024, True),
+                                       (33, 336, 4096, False)]
+               if _slices_fit(tile, K)]
+
+
+@pytest.mark.parametrize("tile,M,N,K,packed", SLICE_CASES)
 def test_gemm_mfma_tiled_with_k_slices(tile, M, N, K, packed):
     """Few tiles: K is cut into slices over workgroups (thousands of the tile number = slices), the
     sums added in order by a second kernel, also under the SwiGLU epilogue; tile 0 chooses by
     itself (K = 2112 = 33 steps: eight slices of five steps would leave the last one empty)."""
     from herbert_rs_amd.kernels import mfma
-    slices, steps = tile // 1000, K // 64
-    if slices > 1 and (slices > min(16, K // 256) or -(-steps // slices) * (slices - 1) >= steps):
-        pytest.skip("more slices than the workspace is sized for, or than K has steps for")
     a = rand(M, K, seed=60, dtype=torch.bfloat16)
     w = rand(N, K, seed=61, dtype=torch.bfloat16, scale=0.05)
     want = (a.double() @ w.double().T).float()

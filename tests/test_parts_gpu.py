@@ -1,7 +1,8 @@
 """Each part alone against the plain formulas, models put together from parts in other ways
 (a layer run twice, a layer that reads another's cache, no rotation), and a toy mixer with state
-of its own, a toy feed-forward with routing and a toy position encoding that are registered here,
-outside the framework's files."""
+of its own, a toy feed-forward with routing and two toy position encodings (another rotation
+table; learned rows added to the embedding, no rotation at all) that are registered here, outside
+the framework's files."""
 import numpy as np
 import pytest
 import torch
@@ -429,3 +430,65 @@ def test_toy_routed_feed_forward_and_toy_position_encoding():
     want = pops.linear(pops.rms_norm(x, w["fn"], 1e-6), w["emb"])
     assert torch.allclose(run_engine(spec, w, tokens), want, atol=1e-4)
     assert torch.allclose(run_engine(spec, w, tokens, cut=4), want, atol=1e-4)
+
+
+def _small_positions(shape, gen, device, std, norm_std):
+    return 0.3 * torch.randn(shape, generator=gen, dtype=torch.float32, device=device)
+
+
+@register("embedding", "toy_table_with_learned_positions")
+class ToyLearnedPositions(Part):
+    """A position encoding that is no rotation: a learned row for every position, added to the
+    token's embedding (the mixers then take the position "none"). It is an embedding part of its
+    own: what it needs of the step, each token's absolute position, is in ctx.meta. Its table is
+    a tensor of a kind the library does not know and brings its own random initialiser."""
+    graph_safe = True
+
+    def __init__(self, vocab_size, hidden_size, max_positions, weight, positions_weight, shared=None):
+        from herbert_rs_amd.parts.io import TokenEmbedding
+        self.tokens = TokenEmbedding(vocab_size, hidden_size, weight)
+        self.max_positions, self.hidden_size, self.positions_name = max_positions, hidden_size, positions_weight
+
+    def tensor_needs(self):
+        needs = dict(self.tokens.tensor_needs())
+        needs[self.positions_name] = TensorNeed((self.max_positions, self.hidden_size), "learned_positions",
+                                                init=_small_positions)
+        return needs
+
+    def load(self, tensors, rt, shared_with_head=False):
+        self.tokens.load(tensors, rt, shared_with_head=shared_with_head)
+        self.linear = self.tokens.linear           # what a tied head multiplies with
+        self.rows = tensors[self.positions_name].to(rt.device).float()
+
+    def forward(self, ctx, token_ids):
+        x = self.tokens.forward(ctx, token_ids)
+        x += self.rows[ctx.meta.positions.long()]
+        return x
+
+
+def test_toy_position_encoding_that_is_no_rotation():
+    base = small_spec(2, [ScheduleEntry(0), ScheduleEntry(1)], rope=False)
+    emb = PartSpec("toy_table_with_learned_positions",
+                   {"vocab_size": 60, "hidden_size": 40, "max_positions": 256, "weight": "emb", "positions_weight": "pos"})
+    spec = ModelSpec(hidden_size=40, vocab_size=60, max_positions=256, embedding=emb, layers=base.layers,
+                     schedule=base.schedule, final_norm=base.final_norm, head=base.head)
+    w = weights_for(spec, seed=9)
+    assert tuple(w["pos"].shape) == (256, 40) and 0.2 < float(w["pos"].std()) < 0.4
+    tokens = [5, 9, 33, 2, 41, 17, 8, 11, 3]
+    positions = list(range(len(tokens)))
+    x = pops.embedding(tokens, w["emb"]) + w["pos"][positions]
+    for p in ("L0.", "L1."):
+        x, _ = plain_layer(w, p, x, positions, rope=False)
+    want = pops.linear(pops.rms_norm(x, w["fn"], 1e-6), w["emb"])
+    assert torch.allclose(run_engine(spec, w, tokens), want, atol=1e-4)
+    assert torch.allclose(run_engine(spec, w, tokens, cut=4), want, atol=1e-4)      # positions go on from the cache's length
+    # In one layer without rotation the last token sees the set of earlier tokens, not their order:
+    # its logits stay when two earlier tokens change places. With the learned rows they move.
+    swapped = [9, 5] + tokens[2:]
+    one = small_spec(1, [ScheduleEntry(0)], rope=False)
+    w1 = weights_for(one, seed=9)
+    assert torch.allclose(run_engine(one, w1, swapped)[-1], run_engine(one, w1, tokens)[-1], atol=1e-4)
+    toy_one = ModelSpec(hidden_size=40, vocab_size=60, max_positions=256, embedding=emb, layers=one.layers,
+                        schedule=one.schedule, final_norm=one.final_norm, head=one.head)
+    w3 = weights_for(toy_one, seed=9)
+    assert not torch.allclose(run_engine(toy_one, w3, swapped)[-1], run_engine(toy_one, w3, tokens)[-1], atol=1e-3)

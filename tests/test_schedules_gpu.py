@@ -126,6 +126,74 @@ def test_a_windowed_cache_rolls_back_only_to_keys_it_still_has(dtype, model_root
     engine.cache.check()
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_window_with_heads_of_128(dtype, model_root):
+    """Configuration D with a window of 100 keys on its first layer: in bfloat16 the window goes
+    through the matrix-core attention of prompts (tiles whose first pages are out of sight) and
+    through the decode kernel that norms, rotates and writes the cache itself, while the windowed
+    layer's cache gives pages back; prompts of unequal lengths in one step, then one token each
+    across page edges."""
+    over = {"sliding_window": 100, "layer_types": ["sliding_attention", "full_attention"]}
+    folder = make_folder(model_root, "D", dtype, overrides=over)
+    vocab = CONFIGS["D"][0]["vocab_size"]
+    seqs = [random_tokens(vocab, n + 70, 400 + n) for n in (300, 31, 130)]
+    cuts = [300, 31, 130]
+    refs = [plain_logits(folder, t) for t in seqs]
+    engine = hb.load(folder, dtype=dtype, cache_tokens=64 * 12)
+    windowed = [g for need, g in engine.cache.kv_groups.items() if need.window][0]
+    slots = [engine.alloc_slot() for _ in seqs]
+    got = engine.step([StepEntry(s, t[:c], [0, c // 2, c - 1]) for s, t, c in zip(slots, seqs, cuts)]).cpu().numpy()
+    for i, c in enumerate(cuts):
+        for j, p in enumerate((0, c // 2, c - 1)):
+            ok, err = close(got[3 * i + j], refs[i][p], dtype, "D", "window")
+            assert ok, (i, p, err)
+    for k in range(70):
+        got = engine.step([StepEntry(s, [t[c + k]], [0]) for s, t, c in zip(slots, seqs, cuts)]).cpu().numpy()
+        for i, c in enumerate(cuts):
+            ok, err = close(got[i], refs[i][c + k], dtype, "D", "window")
+            assert ok, (i, c + k, err)
+    assert windowed.first_page[slots[0]] == (370 + 1 - 100) // 64       # pages out of every later query's sight are back
+    for s in slots:
+        engine.free_slot(s)
+    engine.cache.check()
+
+
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_long_prompts_take_the_kernel_for_them_by_themselves(dtype, model_root):
+    """Configuration F (eight kv heads): a step of 4,100 prompt tokens has 520 attention workgroups
+    of 64-token tiles, from which on the host takes the kernel for long prompts (two halves of 32
+    tokens share a tile's pages); nothing is asked for by name. Two prompts of unequal lengths in
+    the step, one of them going on from 37 tokens already in the cache (its tiles start at
+    positions that 64 does not divide, and its last tile has 27 rows: one half is short), then
+    single tokens."""
+    from herbert_rs_amd.kernels import mfma
+    folder = make_folder(model_root, "F", dtype)
+    vocab = CONFIGS["F"][0]["vocab_size"]
+    a, b = random_tokens(vocab, 2600 + 4, 501), random_tokens(vocab, 37 + 1500 + 4, 502)
+    ref_a, ref_b = plain_logits(folder, a), plain_logits(folder, b)
+    engine = hb.load(folder, dtype=dtype, cache_tokens=64 * 70)
+    sa, sb = engine.alloc_slot(), engine.alloc_slot()
+    engine.step([StepEntry(sb, b[:37], [])])
+    entries = [StepEntry(sa, a[:2600], [0, 31, 32, 63, 64, 1300, 2559, 2560, 2599]),
+               StepEntry(sb, b[37:1537], [0, 26, 27, 700, 1472, 1473, 1499])]
+    meta_tiles = -(-2600 // 64) + -(-1500 // 64)
+    assert meta_tiles * 8 >= mfma.PREFILL_LONG_MIN_WORKGROUPS
+    got = engine.step(entries).cpu().numpy()
+    row = 0
+    for ref, base, e in ((ref_a, 0, entries[0]), (ref_b, 37, entries[1])):
+        for p in e.want:
+            ok, err = close(got[row], ref[base + p], dtype, "F", "long prompt")
+            assert ok, (base + p, err)
+            row += 1
+    for k in range(4):
+        got = engine.step([StepEntry(sa, [a[2600 + k]], [0]), StepEntry(sb, [b[1537 + k]], [0])]).cpu().numpy()
+        assert close(got[0], ref_a[2600 + k], dtype, "F", "long prompt")[0]
+        assert close(got[1], ref_b[1537 + k], dtype, "F", "long prompt")[0]
+    engine.free_slot(sa)
+    engine.free_slot(sb)
+    engine.cache.check()
+
+
 def test_a_step_that_does_not_fit_changes_nothing(model_root):
     """All of a step's pages or none: the step is refused, the sequences that were in it hold
     what they held, and they go on as if it had never been asked for."""

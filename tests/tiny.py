@@ -37,7 +37,15 @@ TINY_D = dict(
     intermediate_size=320, vocab_size=512, rope_theta=1000000.0, rms_norm_eps=1e-6,
     tie_word_embeddings=True, max_position_embeddings=2048, eos_token_id=511)
 
-CONFIGS = {"A": (TINY_A, 0, 0.02), "B": (TINY_B, 1, 0.05), "C": (TINY_C, 2, 0.04), "D": (TINY_D, 3, 0.05)}
+# eight kv heads of 64: a step of a few thousand prompt tokens has enough attention tiles for the
+# kernel that long prompts take
+TINY_F = dict(
+    architectures=["Qwen3ForCausalLM"], model_type="qwen3",
+    num_hidden_layers=1, hidden_size=128, num_attention_heads=8, num_key_value_heads=8, head_dim=64,
+    intermediate_size=160, vocab_size=288, rope_theta=1000000.0, rms_norm_eps=1e-6,
+    tie_word_embeddings=True, max_position_embeddings=4096, eos_token_id=1)
+
+CONFIGS = {"A": (TINY_A, 0, 0.02), "B": (TINY_B, 1, 0.05), "C": (TINY_C, 2, 0.04), "D": (TINY_D, 3, 0.05), "F": (TINY_F, 5, 0.05)}
 
 
 def spec_of(raw):
@@ -53,7 +61,8 @@ def make_folder(root, name, dtype="float32", overrides=None, seed=None, std=None
     tag = f"{name}_{dtype}"
     if overrides:
         raw.update(overrides)
-        tag += "_" + "_".join(f"{k}{v}" for k, v in sorted(overrides.items()))
+        tag += "_" + "".join(c if c.isalnum() or c in "._-" else "-" for c in
+                             "_".join(f"{k}{v}" for k, v in sorted(overrides.items())))
     folder = os.path.join(str(root), tag)
     if os.path.exists(os.path.join(folder, "model.safetensors")):
         return folder
