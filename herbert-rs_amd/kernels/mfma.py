@@ -330,9 +330,17 @@ PREFILL_LONG_MIN_WORKGROUPS = 512      # from so many workgroups of 64-token til
 def _prefill_tile_height(meta, nkv, group):
     """32, or 64 where the step has so many tokens that tiles of 64 still make several rounds of
     workgroups: the kernel for those loads every page once for 64 tokens and has its loads two
-    steps ahead; with fewer, tiles of 32 whose pages two groups of waves take in turn end sooner."""
-    tiles = sum(-(-(int(meta.host_starts[i + 1]) - int(meta.host_starts[i])) // 64) for i in range(meta.num_seqs))
-    return 64 if tiles * nkv * -(-group // 4) >= PREFILL_LONG_MIN_WORKGROUPS else 32
+    steps ahead; with fewer, tiles of 32 whose pages two groups of waves take in turn end sooner.
+    Tiles of 64 must be worth their eight waves: those of at most 32 tokens (single tokens of
+    running sequences beside a prompt, a prompt's short end) leave one half idle and walk their
+    pages alone, so a step made mostly of them keeps tiles of 32."""
+    tiles = full = 0
+    for i in range(meta.num_seqs):
+        n = int(meta.host_starts[i + 1]) - int(meta.host_starts[i])
+        tiles += -(-n // 64)
+        full += n // 64 + (1 if n % 64 > 32 else 0)
+    per_tile = nkv * -(-group // 4)
+    return 64 if full * per_tile >= PREFILL_LONG_MIN_WORKGROUPS and 4 * full >= 3 * tiles else 32
 
 
 def _prefill_tiles(meta, height=QUERY_TILE):
