@@ -9,6 +9,7 @@ prefill_with_token, decode_step and verify_draft_tokens
 cases are kept: empty input (:139-152), token id >= vocab (:165-171), position
 beyond max_position_embeddings (:531-537).
 """
+import numpy as np
 import torch
 
 from ..cache import Cache
@@ -171,9 +172,12 @@ class Engine:
             seen.add(e.slot)
             if len(e.tokens) == 0:
                 raise RequestError("a sequence of a step has no tokens")
-            for t in e.tokens:
-                if not 0 <= int(t) < vocab:
-                    raise RequestError(f"token id {t} out of range (vocab_size {vocab})")
+            ids = np.asarray(e.tokens)
+            if ids.dtype.kind not in "iu":
+                raise RequestError("token ids must be integers")
+            low, high = int(ids.min()), int(ids.max())
+            if low < 0 or high >= vocab:
+                raise RequestError(f"token id {low if low < 0 else high} out of range (vocab_size {vocab})")
             for j in e.want:
                 if not 0 <= int(j) < len(e.tokens):
                     raise RequestError(f"wanted place {j} is outside the sequence's "
