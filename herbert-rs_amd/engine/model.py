@@ -114,6 +114,8 @@ class Model:
                 first_norm = getattr(self.blocks[self.schedule[i + 1].layer], "first_norm", None)
                 if first_norm is not None:
                     ctx.norm_after_block = (first_norm(), i + 1)
+            # a block that knows nothing of norms handed from part to part must meet none
+            ctx.handed = ctx.norm_ahead = None
             self.blocks[e.layer].forward(ctx, x)
         if meta.want_rows.shape[0] == 0:
             return None

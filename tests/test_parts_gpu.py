@@ -1,8 +1,8 @@
 """Each part alone against the plain formulas, models put together from parts in other ways
 (a layer run twice, a layer that reads another's cache, no rotation), and a toy mixer with state
 of its own, a toy feed-forward with routing and two toy position encodings (another rotation
-table; learned rows added to the embedding, no rotation at all) that are registered here, outside
-the framework's files."""
+table; learned rows added to the embedding, no rotation at all), a toy arrangement of a layer and a
+toy norm that are registered here, outside the framework's files."""
 import numpy as np
 import pytest
 import torch
@@ -492,3 +492,113 @@ def test_toy_position_encoding_that_is_no_rotation():
                         schedule=one.schedule, final_norm=one.final_norm, head=one.head)
     w3 = weights_for(toy_one, seed=9)
     assert not torch.allclose(run_engine(toy_one, w3, swapped)[-1], run_engine(toy_one, w3, tokens)[-1], atol=1e-3)
+
+
+# ---- a toy arrangement of a layer and a toy norm, between the library's own blocks
+@register("norm", "toy_centred_norm")
+class ToyCentredNorm(Part):
+    """y = (x - mean) / sqrt(var + eps) * w: not of the form x * w / rms(x), so no product can
+    finish it; it has its own (library) arithmetic and knows nothing of norms handed on."""
+
+    def __init__(self, size, eps, weight):
+        self.size, self.eps, self.weight_name = size, eps, weight
+
+    def tensor_needs(self):
+        return {self.weight_name: TensorNeed((self.size,), "scale")}
+
+    def load(self, tensors, rt):
+        self.w = tensors[self.weight_name].to(rt.device).float()
+        self.dtype = rt.dtype
+
+    def forward(self, ctx, x, rows=None, name="normed"):
+        x = x.float() if rows is None else x.float()[rows.long()]
+        c = x - x.mean(-1, keepdim=True)
+        return (c / torch.sqrt((c * c).mean(-1, keepdim=True) + self.eps) * self.w).to(self.dtype)
+
+
+@register("block", "toy_parallel")
+class ToyParallelBlock(Part):
+    """x += mixer(norm(x)) + feed_forward(norm(x)): both parts read the same normed rows."""
+
+    def __init__(self, mixer, feed_forward, norms):
+        self.mixer, self.feed_forward, self.norm = mixer, feed_forward, norms["input"]
+
+    def parts(self):
+        return [self.norm, self.mixer, self.feed_forward]
+
+    def forward(self, ctx, x):
+        y = self.norm.forward(ctx, x).clone()
+        self.mixer.forward(ctx, y, x)
+        self.feed_forward.forward(ctx, y, x)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_block_and_toy_norm_between_the_library_s_blocks(dtype):
+    from .bounds import close
+    hidden, inter, vocab = 64, 96, 90
+    pos = PartSpec("rope", {"theta": 1e4, "rotary_dims": 16, "max_positions": 256})
+
+    def layer(i, block, norms):
+        p = f"L{i}."
+        names = {k: p + k for k in ("q", "k", "v", "o", "q_norm", "k_norm")}
+        return LayerSpec(PartSpec(block),
+                         PartSpec("attention", dict(hidden_size=hidden, num_heads=4, num_kv_heads=2, head_dim=16,
+                                                    eps=1e-6, position=pos, names=names)),
+                         PartSpec("swiglu", {"hidden_size": hidden, "intermediate_size": inter,
+                                             "names": {"gate": p + "g", "up": p + "u", "down": p + "d"}}), norms)
+
+    def rms(i, k):
+        return PartSpec("rmsnorm", {"size": hidden, "eps": 1e-6, "weight": f"L{i}.{k}"})
+
+    layers = [layer(0, "prenorm", {"input": rms(0, "n1"), "post_mixer": rms(0, "n2")}),
+              layer(1, "toy_parallel", {"input": PartSpec("toy_centred_norm", {"size": hidden, "eps": 1e-3,
+                                                                               "weight": "L1.n1"})}),
+              layer(2, "prenorm", {"input": rms(2, "n1"), "post_mixer": rms(2, "n2")})]
+    spec = ModelSpec(hidden_size=hidden, vocab_size=vocab, max_positions=256,
+                     embedding=PartSpec("table", {"vocab_size": vocab, "hidden_size": hidden, "weight": "emb"}),
+                     layers=layers, schedule=[ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(2)],
+                     final_norm=rms(3, "fn"),
+                     head=PartSpec("linear", {"vocab_size": vocab, "hidden_size": hidden, "weight": "head",
+                                              "tied_to_embedding": True}))
+    # (weights of the tiny configurations' scale, whose bounds are used below; matrices that
+    # bfloat16 holds exactly, so that both dtypes run the same model)
+    from herbert_rs_amd.engine.model import Model
+    from herbert_rs_amd.weights import random_tensors
+    w = random_tensors(Model(spec).tensor_needs(), 12, "float32", std=0.05, norm_std=0.1)
+    w = {k: v.to(torch.bfloat16).float() if v.dim() == 2 else v for k, v in w.items()}
+    tokens = [5, 9, 33, 2, 41, 17, 8, 11, 3, 50, 27, 64, 80, 1]
+    positions = list(range(len(tokens)))
+
+    x = pops.embedding(tokens, w["emb"])
+    x, _ = plain_layer_of(w, "L0.", x, positions, inter)
+    c = x - x.mean(-1, keepdim=True)
+    y = c / torch.sqrt((c * c).mean(-1, keepdim=True) + 1e-3) * w["L1.n1"]
+    x = x + plain_mixer(w, "L1.", y, positions) + pops.swiglu_mlp(y, w["L1.g"], w["L1.u"], w["L1.d"])
+    x, _ = plain_layer_of(w, "L2.", x, positions, inter)
+    want = pops.linear(pops.rms_norm(x, w["L3.fn"], 1e-6), w["emb"]).numpy()
+
+    engine = Engine(None, spec, w, dtype=dtype, max_tokens=256)
+    for cut in (len(tokens), 6):             # whole, then a prompt of 6 and one token at a time
+        s = engine.alloc_slot()
+        got = [engine.step([StepEntry(s, tokens[:cut], list(range(cut)))]).cpu()]
+        got += [engine.step([StepEntry(s, [t], [0])]).cpu() for t in tokens[cut:]]
+        engine.free_slot(s)
+        got = torch.cat(got).numpy()
+        for t in positions:
+            ok, err = close(got[t], want[t], dtype, "A", f"toy block cut {cut}")
+            assert ok, (cut, t, err)
+
+
+def plain_mixer(w, p, y, positions):
+    q = pops.apply_rope(pops.head_rms_norm(pops.split_heads(pops.linear(y, w[p + "q"]), 4, 16), w[p + "q_norm"], 1e-6),
+                        positions, 1e4)
+    k = pops.apply_rope(pops.head_rms_norm(pops.split_heads(pops.linear(y, w[p + "k"]), 2, 16), w[p + "k_norm"], 1e-6),
+                        positions, 1e4)
+    v = pops.split_heads(pops.linear(y, w[p + "v"]), 2, 16)
+    return pops.linear(pops.causal_attention(q, k, v, positions).reshape(len(positions), 64), w[p + "o"])
+
+
+def plain_layer_of(w, p, x, positions, inter):
+    x = x + plain_mixer(w, p, pops.rms_norm(x, w[p + "n1"], 1e-6), positions)
+    y = pops.rms_norm(x, w[p + "n2"], 1e-6)
+    return x + pops.swiglu_mlp(y, w[p + "g"], w[p + "u"], w[p + "d"]), None
