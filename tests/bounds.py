@@ -19,8 +19,9 @@ F32_ABS = 1e-4
 #    fault that shifts a row coherently shows here first;
 #  - the largest error: the maximum of V noisy values grows with V (about sqrt(2 ln V) times the
 #    rms: 0.017 to 0.033 for vocabularies of 256 to 512, 0.043 to 0.051 for 151936).
-BF16_REL_L2 = {"A": 0.012, "B": 0.018, "C": 0.018, "D": 0.02, "F": 0.02, "wide": 0.02, "odd": 0.02}
-BF16_REL_RMS = {"A": 0.04, "B": 0.05, "C": 0.05, "D": 0.05, "F": 0.05, "wide": 0.08, "odd": 0.04}
+# ("random": the drawn configurations of test_random_configs_gpu, worst seen 0.011 and 0.036)
+BF16_REL_L2 = {"A": 0.012, "B": 0.018, "C": 0.018, "D": 0.02, "F": 0.02, "wide": 0.02, "odd": 0.02, "random": 0.02}
+BF16_REL_RMS = {"A": 0.04, "B": 0.05, "C": 0.05, "D": 0.05, "F": 0.05, "wide": 0.08, "odd": 0.04, "random": 0.06}
 
 
 def rel_rms_error(got, ref):
