@@ -249,10 +249,15 @@ __device__ __forceinline__ void choose_bin(const int* hist, int* wave_totals, in
 // logits in LDS, finds its own top_k among them (ties: lower index first) and leaves them, in any
 // order, in pre_key / pre_idx [row][chunk][top_k]. A single block walks a row at about 24 GB/s
 // only; shared out over the CUs the 600 KB of a row of 151936 logits are read in a few us.
+// chunk_ms != null: it also leaves, in chunk_ms [row][chunk][2], the largest scaled logit of the
+// chunk and the sum of exp(scaled - that) over the chunk, added up in a fixed order (a thread's
+// eight in their order, the lanes of a wave by a tree, the waves one after the other).
 __global__ void __launch_bounds__(SAMPLE_THREADS)
 sample_chunk_topk_kernel(const float* __restrict__ logits, int ld, int V, float temperature, int top_k,
-                         uint32_t* __restrict__ pre_key, int* __restrict__ pre_idx) {
+                         uint32_t* __restrict__ pre_key, int* __restrict__ pre_idx,
+                         float* __restrict__ chunk_ms) {
     __shared__ uint32_t ck[SAMPLE_CHUNK];
+    __shared__ float wave_vals[SAMPLE_THREADS / HB_WAVE];
     __shared__ int hist[256];
     __shared__ int wave_counts[SAMPLE_THREADS / HB_WAVE];
     __shared__ uint32_t sel_prefix;
@@ -279,6 +284,34 @@ sample_chunk_topk_kernel(const float* __restrict__ logits, int ld, int V, float 
         sel_remaining = top_k;
         n_out = 0;
         eq_taken = 0;
+    }
+    if (chunk_ms) {
+        float mv = -INFINITY;
+#pragma unroll
+        for (int u = 0; u < PER; ++u)
+            if (tid + u * SAMPLE_THREADS < len) mv = fmaxf(mv, v[u] / temperature);
+        mv = hb_wave_max(mv);
+        if (lane == 0) wave_vals[wave] = mv;
+        __syncthreads();
+        float cmax = wave_vals[0];
+        for (int w = 1; w < SAMPLE_THREADS / HB_WAVE; ++w) cmax = fmaxf(cmax, wave_vals[w]);
+        __syncthreads();
+        float part = 0.f;
+        if (cmax != -INFINITY) {
+#pragma unroll
+            for (int u = 0; u < PER; ++u)
+                if (tid + u * SAMPLE_THREADS < len) part += expf(v[u] / temperature - cmax);
+        }
+        for (int d = HB_WAVE / 2; d > 0; d >>= 1) part += __shfl_down(part, d, HB_WAVE);
+        if (lane == 0) wave_vals[wave] = part;
+        __syncthreads();
+        if (tid == 0) {
+            float sum = 0.f;
+            for (int w = 0; w < SAMPLE_THREADS / HB_WAVE; ++w) sum += wave_vals[w];
+            float* ms = chunk_ms + ((size_t)blockIdx.y * gridDim.x + c) * 2;
+            ms[0] = cmax;
+            ms[1] = sum;
+        }
     }
     __syncthreads();
     if (len <= top_k) {                       // all of a short chunk
@@ -349,7 +382,8 @@ sample_chunk_topk_kernel(const float* __restrict__ logits, int ld, int V, float 
 __global__ void __launch_bounds__(SAMPLE_THREADS)
 sample_topk_kernel(const float* __restrict__ logits, int ld, int V, float temperature, int top_k,
                    float top_p, unsigned long long* __restrict__ rng, const int* __restrict__ rng_index,
-                   int* __restrict__ out, const uint32_t* __restrict__ pre_key, const int* __restrict__ pre_idx) {
+                   int* __restrict__ out, const uint32_t* __restrict__ pre_key, const int* __restrict__ pre_idx,
+                   const float* __restrict__ chunk_ms) {
     __shared__ uint32_t keys[SAMPLE_MAX_K];
     __shared__ int idx[SAMPLE_MAX_K];
     __shared__ float prob[SAMPLE_MAX_K];
@@ -542,7 +576,14 @@ sample_topk_kernel(const float* __restrict__ logits, int ld, int V, float temper
     __shared__ float inv_sum_s;
     if (tid == 0) {
         float sum = 0.f;
-        for (int i = 0; i < n; ++i) sum += prob[i];
+        if (chunk_ms) {
+            // every logit of the row counts in the softmax: the chunks' sums, in the order of the chunks
+            const float* ms = chunk_ms + (size_t)blockIdx.x * chunks * 2;
+            for (int c = 0; c < chunks; ++c)
+                if (ms[2 * c] != -INFINITY) sum += ms[2 * c + 1] * expf(ms[2 * c] - max_val);
+        } else {
+            for (int i = 0; i < n; ++i) sum += prob[i];
+        }
         inv_sum_s = 1.0f / sum;
     }
     __syncthreads();
@@ -572,12 +613,21 @@ sample_topk_kernel(const float* __restrict__ logits, int ld, int V, float temper
             for (int i = 0; i < cutoff; ++i) sum += prob[i];
             inv_sum_s = 1.0f / sum;
             n_kept = cutoff;
+            // The candidates are the largest of a longer row: the prefix is the row's own only if
+            // the sum has reached top_p and everything kept is more probable than the last
+            // candidate (what was left out is at most as probable as that one, and among equals
+            // the index decides).
+            if (chunk_ms && !(cum >= top_p && prob[cutoff - 1] > prob[n - 1])) n_kept = -1;
         }
         __syncthreads();
         const int kept = n_kept;
         for (int i = tid; i < kept; i += blockDim.x) prob[i] *= inv_sum_s;
     }
     __syncthreads();
+    if (n_kept < 0) {                 // undecided: no draw is taken, the caller sees -1
+        if (tid == 0) out[blockIdx.x] = -1;
+        return;
+    }
 
     if (tid == 0) {
         unsigned long long* st = rng + (rng_index ? rng_index[blockIdx.x] : blockIdx.x);
@@ -822,12 +872,12 @@ extern "C" int hb_sample(const float* logits, int ld, int R, int V, float temper
         const bool sift = pre_key && pre_idx && chunks > 2 && R <= 65535;
         if (sift) {
             sample_chunk_topk_kernel<<<dim3(chunks, R), SAMPLE_THREADS, 0, stream>>>(logits, ld, V, temperature,
-                                                                                    top_k, pre_key, pre_idx);
+                                                                                    top_k, pre_key, pre_idx, nullptr);
             HB_CHECK_LAUNCH("sample_chunk_topk");
         }
         sample_topk_kernel<<<R, SAMPLE_THREADS, 0, stream>>>(logits, ld, V, temperature, top_k, top_p, rng,
                                                            rng_index, out, sift ? pre_key : nullptr,
-                                                           sift ? pre_idx : nullptr);
+                                                           sift ? pre_idx : nullptr, nullptr);
         HB_CHECK_LAUNCH("sample_topk");
         return 0;
     }
@@ -858,5 +908,29 @@ extern "C" int hb_sample(const float* logits, int ld, int R, int V, float temper
     sample_finish_kernel<<<R, 1024, 0, stream>>>(scratch_keys, scratch_idx, P2, n, sorted, top_p, rng,
                                                  rng_index, out);
     HB_CHECK_LAUNCH("sample_finish");
+    return 0;
+}
+
+// Top-p without top-k on a long row, the quick way: the prefix by descending probability whose
+// sum reaches top_p nearly always lies among the SAMPLE_MAX_K largest logits, so only those are
+// found and sorted (as for top_k = SAMPLE_MAX_K), while the softmax runs over the whole row (the
+// chunks' sums). A row whose prefix does not end inside those candidates gets out[r] = -1 and its
+// generator is left as it was: the caller samples that row with hb_sample.
+// pre_key / pre_idx: [R, ceil(V / 8192), 1024] each; chunk_ms: float [R, ceil(V / 8192), 2].
+extern "C" int hb_sample_nucleus(const float* logits, int ld, int R, int V, float temperature, float top_p,
+                                 unsigned long long* rng, const int* rng_index, int* out, uint32_t* pre_key,
+                                 int* pre_idx, float* chunk_ms, hipStream_t stream) {
+    HB_REQUIRE(R > 0 && R <= 65535 && V > SAMPLE_MAX_K && ld >= V,
+               "sample (top-p first): bad sizes (R=%d, V=%d, ld=%d); rows must be longer than %d", R, V, ld,
+               SAMPLE_MAX_K);
+    HB_REQUIRE(temperature > 0.f && top_p < 1.0f, "sample (top-p first): needs temperature > 0 and top_p < 1");
+    HB_REQUIRE(pre_key && pre_idx && chunk_ms, "sample (top-p first): needs its three buffers");
+    const int chunks = (V + SAMPLE_CHUNK - 1) / SAMPLE_CHUNK;
+    sample_chunk_topk_kernel<<<dim3(chunks, R), SAMPLE_THREADS, 0, stream>>>(logits, ld, V, temperature,
+                                                                            SAMPLE_MAX_K, pre_key, pre_idx, chunk_ms);
+    HB_CHECK_LAUNCH("sample_chunk_topk (top-p first)");
+    sample_topk_kernel<<<R, SAMPLE_THREADS, 0, stream>>>(logits, ld, V, temperature, SAMPLE_MAX_K, top_p, rng,
+                                                       rng_index, out, pre_key, pre_idx, chunk_ms);
+    HB_CHECK_LAUNCH("sample_topk (top-p first)");
     return 0;
 }

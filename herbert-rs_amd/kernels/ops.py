@@ -260,3 +260,39 @@ def sample(logits, temperature, top_k, top_p, rng_states, rng_index, out, scratc
     lib.call("sampling", "hb_sample", logits.data_ptr(), V, R, V, float(temperature), int(top_k),
              float(top_p), rng_states.data_ptr(), _ptr(rng_index), out.data_ptr(), _ptr(keys),
              _ptr(idx), p2, _ptr(pre_key), _ptr(pre_idx), _stream())
+
+
+NUCLEUS_CANDIDATES = 1024
+
+
+def nucleus_buffers(rows, vocab, device):
+    """(keys int32, idx int32, sums float32) that sample_nucleus needs for `rows` rows of `vocab` logits."""
+    chunks = -(-vocab // SAMPLE_CHUNK)
+    return (torch.empty(rows * chunks * NUCLEUS_CANDIDATES, dtype=torch.int32, device=device),
+            torch.empty(rows * chunks * NUCLEUS_CANDIDATES, dtype=torch.int32, device=device),
+            torch.empty(rows * chunks * 2, dtype=torch.float32, device=device))
+
+
+def sample_nucleus(logits, temperature, top_p, rng_states, rng_index, out, buffers):
+    """Top-p without top-k on rows of more than 1024 logits, the quick way: a row's prefix is looked
+    for among its 1024 largest logits only (the softmax still runs over the whole row). A row whose
+    prefix does not end among them gets out[r] = -1 and keeps its generator state: sample it with
+    `sample`. `buffers` as `nucleus_buffers` makes them."""
+    _check(logits, "logits", torch.float32, (None, None))
+    R, V = logits.shape
+    _check(out, "out", torch.int32, (R,))
+    _check(rng_states, "rng_states", torch.int64, (None,))
+    if rng_index is not None:
+        _check(rng_index, "rng_index", torch.int32, (R,))
+    elif rng_states.shape[0] < R:
+        raise BackendError("sample: fewer generator states than rows")
+    keys, idx, sums = buffers
+    chunks = -(-V // SAMPLE_CHUNK)
+    _check(keys, "candidate keys", torch.int32, (None,))
+    _check(idx, "candidate idx", torch.int32, (None,))
+    _check(sums, "chunk sums", torch.float32, (None,))
+    if min(keys.numel(), idx.numel()) < R * chunks * NUCLEUS_CANDIDATES or sums.numel() < R * chunks * 2:
+        raise BackendError("sample: the buffers of the quick top-p are too small for these logits")
+    lib.call("sampling", "hb_sample_nucleus", logits.data_ptr(), V, R, V, float(temperature), float(top_p),
+             rng_states.data_ptr(), _ptr(rng_index), out.data_ptr(), keys.data_ptr(), idx.data_ptr(),
+             sums.data_ptr(), _stream())

@@ -29,6 +29,7 @@ class Sampler:
         self.states = torch.tensor(states, dtype=torch.int64, device=device)
         self._scratch = None
         self._sifted = None
+        self._nucleus = None
 
     def _sifted_for(self, rows):
         """Buffers for the candidates that a block a chunk sifts out of a long row (top-k up to 1024)."""
@@ -61,6 +62,29 @@ class Sampler:
             ops.argmax(logits, out)
         else:
             index = torch.tensor(list(sequence_indices), dtype=torch.int32, device=self.device)
-            ops.sample(logits, self.params.temperature, self.params.top_k, self.params.top_p,
+            p = self.params
+            vocab = logits.shape[1]
+            if not 0 < p.top_k < vocab and p.top_p < 1.0 and vocab > ops.NUCLEUS_CANDIDATES:
+                return self._top_p_only(logits, index, out)
+            ops.sample(logits, p.temperature, p.top_k, p.top_p,
                        self.states, index, out, self._scratch_for(rows), self._sifted_for(rows))
         return out.tolist()
+
+    def _top_p_only(self, logits, index, out):
+        """Top-p without top-k: first among each row's 1024 largest logits, where the prefix that
+        reaches top_p nearly always ends (no sort of the whole vocabulary); the rows where it does
+        not (flat distributions) then go the general way, with the same draw."""
+        rows, p = logits.shape[0], self.params
+        if self._nucleus is None or self._nucleus[2].numel() < rows * (-(-logits.shape[1] // ops.SAMPLE_CHUNK)) * 2:
+            self._nucleus = ops.nucleus_buffers(rows, logits.shape[1], self.device)
+        ops.sample_nucleus(logits, p.temperature, p.top_p, self.states, index, out, self._nucleus)
+        tokens = out.tolist()
+        rest = [r for r, t in enumerate(tokens) if t < 0]
+        if rest:
+            at = torch.tensor(rest, dtype=torch.long, device=self.device)
+            sub_out = torch.empty(len(rest), dtype=torch.int32, device=self.device)
+            ops.sample(logits[at].contiguous(), p.temperature, p.top_k, p.top_p, self.states,
+                       index[at].contiguous(), sub_out, self._scratch_for(len(rest)), None)
+            for r, t in zip(rest, sub_out.tolist()):
+                tokens[r] = t
+        return tokens

@@ -427,6 +427,57 @@ def test_sampler_matches_the_plain_sampler(top_k, top_p, V):
     assert [int(s) & ((1 << 64) - 1) for s in states.tolist()] == [r.state for r in rngs]
 
 
+@pytest.mark.parametrize("V", [1500, 20000, 151936])
+def test_top_p_without_top_k_looks_among_the_largest_first(V):
+    """Top-p without top-k through the Sampler: a steep row is decided among its 1024 largest
+    logits, a flat row and a row whose 1024th largest is one of 1990 equal ones are not (they get
+    -1 from the quick kernel) and go the general way; all three give the plain sampler's tokens,
+    draw after draw, and every generator advances once a draw."""
+    from herbert_rs_amd.kernels import ops
+    from herbert_rs_amd.sampling import SamplingParams, xorshift
+    from herbert_rs_amd.sampling.sampler import Sampler
+    temperature, top_p = 0.8, 0.85
+    g = torch.Generator().manual_seed(V)
+    steep = torch.randn(V, generator=g) * 6.0
+    flat = torch.randn(V, generator=g) * 0.2
+    level = torch.randn(V, generator=g) * 0.5 - 8.0
+    # (1990 or V - 10 equal ones: top_p of them ends well inside a probability, not at its edge)
+    level[torch.randperm(V, generator=g)[:min(1990, V - 10)]] = 3.0
+    steep_tail = torch.randn(V, generator=g) * 5.0
+    logits = torch.stack([steep, flat, level, steep_tail])
+    R = logits.shape[0]
+    dev_logits = logits.cuda()
+    params = SamplingParams(temperature=temperature, top_k=0, top_p=top_p, max_tokens=4, seed=21)
+    sampler = Sampler(params, R, V, torch.device("cuda"))
+    rngs = [plain_sampler.XorShift64(xorshift.sequence_seed(21, i)) for i in range(R)]
+    works = [plain_sampler.candidates(logits[r].numpy(), temperature, 0, top_p) for r in range(R)]
+    assert len(works[0]) < 1024 < len(works[1])
+
+    # which rows the quick kernel decides (on copies of the states: a row it leaves keeps its state)
+    states = sampler.states.clone()
+    out = torch.empty(R, dtype=torch.int32, device="cuda")
+    ops.sample_nucleus(dev_logits, temperature, top_p, states, torch.arange(R, dtype=torch.int32, device="cuda"),
+                       out, ops.nucleus_buffers(R, V, "cuda"))
+    quick = [t >= 0 for t in out.tolist()]
+    assert quick[:3] == [True, False, False]
+    kept = [a == b for a, b in zip(states.tolist(), sampler.states.tolist())]
+    assert kept == [not q for q in quick]
+
+    for draw in range(10):
+        got = sampler.choose(dev_logits, list(range(R)))
+        for r in range(R):
+            u = rngs[r].next_f32()
+            want = plain_sampler.pick(works[r], u)
+            if got[r] != want:
+                cum, near = np.float32(0), False
+                for idx, p in works[r]:
+                    cum = np.float32(cum + p)
+                    if abs(float(cum) - float(u)) < 1e-5:
+                        near = True
+                assert near and got[r] in [i for i, _ in works[r]], (draw, r, got[r], want)
+    assert [int(s) & ((1 << 64) - 1) for s in sampler.states.tolist()] == [r.state for r in rngs]
+
+
 def test_sampler_draw_and_top_p_edge_on_exact_probabilities():
     """Equal logits give probabilities that are exact in float32 whatever the exponential's
     rounding (exp(0) = 1), so two rules show without a tolerance. (1) The draw is the upper bits
