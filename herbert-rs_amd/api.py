@@ -19,20 +19,24 @@ def load(model, dtype="bfloat16", cache_tokens=4096, max_slots=None):
 
 
 def generate(model, prompts, temperature=0.4, top_k=40, top_p=0.9, max_tokens=2048, stop_ids=(),
-             ignore_eos=False, no_repeat_check=False, seed=None, dtype="bfloat16", max_batch=64):
+             ignore_eos=False, no_repeat_check=False, seed=None, dtype="bfloat16", max_batch=64,
+             prefill_chunk=None, think_budget=0, think_tokens=None):
     """Generate from token-id prompts. `model` is a folder or an Engine; `prompts` one list of
-    ids or a list of them. Returns the generated ids (one list, or a list of lists)."""
+    ids or a list of them. Returns the generated ids (one list, or a list of lists).
+    `prefill_chunk`: prompts go through the engine in pieces of that many tokens. `think_budget`
+    with `think_tokens` (sampling.ThinkTokens): a cap on the tokens of a think block."""
     single = bool(prompts) and isinstance(prompts[0], int)
     plist = [list(prompts)] if single else [list(p) for p in prompts]
     params = SamplingParams(temperature=temperature, top_k=top_k, top_p=top_p, max_tokens=max_tokens,
                             stop_ids=tuple(stop_ids), ignore_eos=ignore_eos,
-                            repeat_check=not no_repeat_check, seed=seed)
+                            repeat_check=not no_repeat_check, seed=seed, think_budget=think_budget,
+                            think_tokens=think_tokens)
     if isinstance(model, Engine):
         engine = model
     else:
         room = sum((len(p) + max_tokens + 127) // 64 * 64 for p in plist[:max_batch])
         engine = load(model, dtype=dtype, cache_tokens=room)
-    results = engine.generate(plist, params, max_batch=max_batch)
+    results = engine.generate(plist, params, max_batch=max_batch, prefill_chunk=prefill_chunk)
     tokens = [r.tokens for r in results]
     return tokens[0] if single else tokens
 

@@ -117,12 +117,29 @@ def load_tokenizer(model_dir):
     return Tokenizer.from_file(path)
 
 
+def print_arch():
+    """What --arch shows: the reference prints the CPU's features there (crates/cli/src/arch.rs);
+    here it is the GPU the kernels are built for and the one that is present."""
+    import torch
+    print("herbert-cli: kernels for gfx950 (MI355X), wave64, MFMA bf16")
+    if not torch.cuda.is_available():
+        print("no GPU visible to this process")
+        return 0
+    for i in range(torch.cuda.device_count()):
+        p = torch.cuda.get_device_properties(i)
+        print(f"GPU {i}: {p.name} ({getattr(p, 'gcnArchName', '?')}), {p.multi_processor_count} CUs, "
+              f"{p.total_memory / 2**30:.0f} GiB")
+    return 0
+
+
 def make_parser():
     ap = argparse.ArgumentParser(prog="herbert-cli", description="Herbert - local LLM inference on MI355X")
-    ap.add_argument("--model", required=True, help="Model directory")
+    ap.add_argument("--arch", action="store_true", help="Show the GPU this would run on and exit")
+    ap.add_argument("--model", help="Model directory")
     ap.add_argument("--prompt", help="Input prompt (text with a tokenizer, else comma-separated ids)")
     ap.add_argument("--prompt-file", help="Read prompt from a file")
     ap.add_argument("--system", help="System prompt (prepended with chat template)")
+    ap.add_argument("--system-file", help="Read system prompt from a file")
     ap.add_argument("--max-tokens", type=int, default=2048, help="Max tokens to generate")
     ap.add_argument("--ignore-eos", action="store_true", help="Ignore EOS token")
     ap.add_argument("--no-repeat-check", action="store_true", help="Disable repetition loop detection")
@@ -132,7 +149,12 @@ def make_parser():
     ap.add_argument("--temperature", type=float, default=0.4, help="Sampling temperature (0 = greedy argmax)")
     ap.add_argument("--top-k", type=int, default=40, help="Top-k sampling (0 = disabled)")
     ap.add_argument("--top-p", type=float, default=0.9, help="Top-p / nucleus sampling (1.0 = disabled)")
+    ap.add_argument("--think-budget", type=int, default=0,
+                    help="Max tokens in <think> before forcing </think> (0 = unlimited)")
+    ap.add_argument("--nothink", action="store_true", help="Disable thinking (a think block is closed at once)")
     ap.add_argument("--show-specials", action="store_true", help="Show special tokens in output")
+    ap.add_argument("--prefill-chunk-size", type=int, default=None,
+                    help="Process the prompt in chunks of N tokens (default: HERBERT_PREFILL_CHUNK_SIZE, else whole)")
     ap.add_argument("--seed", type=int, default=None, help="Sampler seed (default: from the clock)")
     ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
     ap.add_argument("--cache-tokens", type=int, default=None,
@@ -153,7 +175,11 @@ def main(argv=None):
 
 def _run(args):
     from .api import load, write_random_model
-    from .sampling import INTERRUPTED, STOP_SEQUENCE, SamplingParams
+    from .sampling import INTERRUPTED, STOP_SEQUENCE, SamplingParams, ThinkTokens
+    if args.arch:
+        return print_arch()
+    if not args.model:
+        raise RequestError("--model is required")
     if args.random_weights and not os.path.exists(os.path.join(args.model, "model.safetensors")):
         write_random_model(args.model, os.path.join(args.model, "config.json"), seed=args.seed or 0,
                            dtype=args.dtype)
@@ -163,11 +189,26 @@ def _run(args):
             prompt = f.read()
     if prompt is None:
         raise RequestError("--prompt or --prompt-file is required (there is no interactive mode)")
+    # --system wins over --system-file (crates/cli/src/main.rs:390-397)
+    system = args.system
+    if system is None and args.system_file:
+        try:
+            with open(args.system_file) as f:
+                system = f.read()
+        except OSError as e:
+            raise RequestError(f"Failed to read system file {args.system_file!r}: {e}") from None
+    # the flag, else the environment, else the prompt whole (crates/cli/src/main.rs:400-408)
+    prefill_chunk = args.prefill_chunk_size
+    if prefill_chunk is None:
+        env = os.environ.get("HERBERT_PREFILL_CHUNK_SIZE", "")
+        prefill_chunk = int(env) if env.isdigit() else None
+    if prefill_chunk is not None and prefill_chunk <= 0:
+        prefill_chunk = None
     tokenizer = load_tokenizer(args.model)
     from .config import load_config
     chat = load_config(args.model)[0].chat
     if tokenizer is not None:
-        text = chat.build_prompt(prompt, args.system) if chat is not None else prompt
+        text = chat.build_prompt(prompt, system) if chat is not None else prompt
         ids = tokenizer.encode(text, add_special_tokens=False).ids
     else:
         ids = parse_token_ids(prompt)
@@ -182,6 +223,23 @@ def _run(args):
             end = tokenizer.token_to_id(chat.end_of_turn)
             stop_ids.append(end if end is not None else chat.end_of_turn_id)
 
+    # --nothink is a budget of one token (crates/cli/src/main.rs:685-687); the ids come from the
+    # tokenizer, else from the architecture's entry (:671-684)
+    think_budget = 1 if args.nothink else max(0, args.think_budget)
+    think_tokens = None
+    if think_budget > 0:
+        if chat is None or chat.think_open_id is None or chat.think_close_id is None or chat.newline_id is None:
+            raise RequestError("--think-budget / --nothink: this architecture names no think tokens")
+        open_id, close_id, newline_id = chat.think_open_id, chat.think_close_id, chat.newline_id
+        if tokenizer is not None:
+            found = tokenizer.token_to_id(chat.think_open)
+            open_id = found if found is not None else open_id
+            found = tokenizer.token_to_id(chat.think_close)
+            close_id = found if found is not None else close_id
+            line = tokenizer.encode("\n", add_special_tokens=False).ids
+            newline_id = line[0] if len(line) == 1 else newline_id
+        think_tokens = ThinkTokens(open_id, close_id, newline_id)
+
     t0 = time.perf_counter()
     cache_tokens = args.cache_tokens or (len(ids) + args.max_tokens + 65)
     engine = load(args.model, dtype=args.dtype, cache_tokens=cache_tokens)
@@ -190,7 +248,12 @@ def _run(args):
     params = SamplingParams(temperature=args.temperature, top_k=args.top_k, top_p=args.top_p,
                             max_tokens=args.max_tokens + 1, stop_ids=tuple(stop_ids),
                             ignore_eos=args.ignore_eos, repeat_check=not args.no_repeat_check,
-                            seed=args.seed)
+                            seed=args.seed, think_budget=think_budget, think_tokens=think_tokens)
+    vocab = engine.spec.vocab_size
+    if think_tokens is not None and not all(0 <= t < vocab for t in (think_tokens.open_id, think_tokens.close_id,
+                                                                     think_tokens.newline_id)):
+        raise RequestError(f"--think-budget / --nothink: the think tokens {think_tokens} lie outside the "
+                           f"model's vocabulary of {vocab}")
     produced = []
     printed = [0]
 
@@ -213,7 +276,8 @@ def _run(args):
     interrupt = InterruptFlag().install()
     t0 = time.perf_counter()
     try:
-        result = engine.generate([ids], params, on_token=on_token, interrupt=interrupt)[0]
+        result = engine.generate([ids], params, on_token=on_token, interrupt=interrupt,
+                                 prefill_chunk=prefill_chunk)[0]
     finally:
         interrupt.restore()
     total = time.perf_counter() - t0

@@ -27,6 +27,13 @@ class ChatFormat:
     build_prompt: Callable          # (user text, system text or None) -> str
     end_of_turn: Optional[str] = None
     end_of_turn_id: Optional[int] = None
+    # the tokens that open and close a think block, for a cap on its length
+    # (crates/cli/src/main.rs:671-684: looked up in the tokenizer, else these ids)
+    think_open: Optional[str] = None
+    think_close: Optional[str] = None
+    think_open_id: Optional[int] = None
+    think_close_id: Optional[int] = None
+    newline_id: Optional[int] = None
 
 
 @dataclass(frozen=True)

@@ -934,3 +934,22 @@ extern "C" int hb_sample_nucleus(const float* logits, int ld, int R, int V, floa
     HB_CHECK_LAUNCH("sample_topk (top-p first)");
     return 0;
 }
+
+// Leaves one token a row to choose from: every other logit of row rows[i] becomes -inf
+// (crates/core/src/sampler.rs:234-243 of the reference). rows, tokens: int32 [n], device memory.
+__global__ void force_token_kernel(float* __restrict__ logits, int ld, int V, const int* __restrict__ rows,
+                                   const int* __restrict__ tokens) {
+    const int j = blockIdx.x * blockDim.x + threadIdx.x;
+    const int keep = tokens[blockIdx.y];
+    if (j < V && j != keep) logits[(size_t)rows[blockIdx.y] * ld + j] = -INFINITY;
+}
+
+extern "C" int hb_force_tokens(float* logits, int ld, int R, int V, const int* rows, const int* tokens, int n,
+                               hipStream_t stream) {
+    HB_REQUIRE(R > 0 && V > 0 && ld >= V && n > 0 && n <= 65535, "force_tokens: bad sizes (R=%d, V=%d, ld=%d, n=%d)",
+               R, V, ld, n);
+    HB_REQUIRE(rows && tokens, "force_tokens: needs the rows and their tokens");
+    force_token_kernel<<<dim3((V + 255) / 256, n), 256, 0, stream>>>(logits, ld, V, rows, tokens);
+    HB_CHECK_LAUNCH("force_tokens");
+    return 0;
+}

@@ -251,10 +251,10 @@ class Engine:
         held = sum(st.logits.numel() * 4 for st in self._decode.values())
         return len(self._graphs), len(self._decode), held
 
-    def generate(self, prompts, params=None, max_batch=64, on_token=None, interrupt=None):
+    def generate(self, prompts, params=None, max_batch=64, on_token=None, interrupt=None, prefill_chunk=None):
         """Generate from lists of token ids; see engine.generate.Generator."""
         from .generate import Generator
-        gen = Generator(self, max_batch=max_batch)
+        gen = Generator(self, max_batch=max_batch, prefill_chunk=prefill_chunk)
         results = gen.generate(prompts, params, on_token, interrupt)
         self.last_generation_stats = gen.stats
         return results

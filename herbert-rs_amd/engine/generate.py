@@ -92,9 +92,14 @@ class Generator:
     """Runs requests through an engine. `make_chooser(params, n, vocab, device)` builds the object
     whose `choose(logits, sequence_indices)` picks tokens (the GPU sampler by default)."""
 
-    def __init__(self, engine, max_batch=64, make_chooser=None):
+    def __init__(self, engine, max_batch=64, make_chooser=None, prefill_chunk=None):
         self.engine = engine
         self.max_batch = int(max_batch)
+        # prompts longer than this many tokens are fed in pieces of that size, one step a piece
+        # (the reference's prefill_chunk_size: crates/cli/src/main.rs:400-408)
+        self.prefill_chunk = int(prefill_chunk) if prefill_chunk else None
+        if self.prefill_chunk is not None and self.prefill_chunk <= 0:
+            raise RequestError("prefill_chunk must be > 0")
         if make_chooser is None:
             from ..sampling.sampler import Sampler
             make_chooser = Sampler
@@ -126,6 +131,33 @@ class Generator:
             self.stats.batches += 1
         return results
 
+    def _prompts(self, live, prompts, slots, chooser):
+        """The prompts of a batch through the engine; the first token of each sequence, in the
+        order of `live`. Whole in one step, or, with a prefill chunk, in steps that carry the
+        next piece of every prompt that still has one: a sequence's token is chosen in the step
+        that brings its last piece."""
+        eng, chunk = self.engine, self.prefill_chunk
+        if chunk is None or all(len(prompts[i]) <= chunk for i in live):
+            entries = [StepEntry(slots[i], list(prompts[i]), [len(prompts[i]) - 1]) for i in live]
+            return chooser.choose(eng.step(entries), list(live))
+        fed = {i: 0 for i in live}
+        first = {}
+        while len(first) < len(live):
+            entries, ending = [], []
+            for i in live:
+                left = len(prompts[i]) - fed[i]
+                if left <= 0:
+                    continue
+                n = min(chunk, left)
+                entries.append(StepEntry(slots[i], list(prompts[i][fed[i]:fed[i] + n]), [n - 1] if n == left else []))
+                if n == left:
+                    ending.append(i)
+                fed[i] += n
+            logits = eng.step(entries)
+            if ending:
+                first.update(zip(ending, chooser.choose(logits, ending)))
+        return [first[i] for i in live]
+
     def _run_batch(self, members, prompts, params, chooser, results, on_token, interrupt=None):
         eng = self.engine
         eos = eng.spec.eos_token_id
@@ -140,9 +172,7 @@ class Generator:
 
         try:
             t0 = time.perf_counter()
-            entries = [StepEntry(slots[i], list(prompts[i]), [len(prompts[i]) - 1]) for i in live]
-            logits = eng.step(entries)
-            tokens = chooser.choose(logits, list(live))
+            tokens = self._prompts(live, prompts, slots, chooser)
             self.stats.prefill_seconds += time.perf_counter() - t0
             self.stats.prompt_tokens += sum(len(prompts[i]) for i in live)
             t0 = time.perf_counter()

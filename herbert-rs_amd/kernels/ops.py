@@ -296,3 +296,18 @@ def sample_nucleus(logits, temperature, top_p, rng_states, rng_index, out, buffe
     lib.call("sampling", "hb_sample_nucleus", logits.data_ptr(), V, R, V, float(temperature), float(top_p),
              rng_states.data_ptr(), _ptr(rng_index), out.data_ptr(), keys.data_ptr(), idx.data_ptr(),
              sums.data_ptr(), _stream())
+
+
+def force_tokens(logits, rows, tokens):
+    """Every logit of row rows[i] but that of tokens[i] becomes -inf, in place: the next choice in
+    that row can only be that token. rows, tokens: lists of ints (checked here against the shape)."""
+    _check(logits, "logits", torch.float32, (None, None))
+    R, V = logits.shape
+    if len(rows) != len(tokens) or not rows:
+        raise BackendError("force_tokens: needs as many tokens as rows, at least one")
+    for r, t in zip(rows, tokens):
+        if not (0 <= int(r) < R and 0 <= int(t) < V):
+            raise BackendError(f"force_tokens: row {r} or token {t} outside logits of shape {R} x {V}")
+    both = torch.tensor([list(map(int, rows)), list(map(int, tokens))], dtype=torch.int32, device=logits.device)
+    lib.call("sampling", "hb_force_tokens", logits.data_ptr(), V, R, V, both[0].data_ptr(), both[1].data_ptr(),
+             len(rows), _stream())

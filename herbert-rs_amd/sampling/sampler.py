@@ -10,6 +10,7 @@ import torch
 
 from ..kernels import ops
 from . import xorshift
+from .think import ThinkBudget
 
 
 def _signed64(v):
@@ -30,6 +31,10 @@ class Sampler:
         self._scratch = None
         self._sifted = None
         self._nucleus = None
+        # a cap on think blocks: one counter a sequence, fed with every token chosen for it
+        self.think = None
+        if params.think_budget > 0:
+            self.think = [ThinkBudget(params.think_budget, params.think_tokens) for _ in range(num_sequences)]
 
     def _sifted_for(self, rows):
         """Buffers for the candidates that a block a chunk sifts out of a long row (top-k up to 1024)."""
@@ -55,7 +60,23 @@ class Sampler:
         return self._scratch
 
     def choose(self, logits, sequence_indices):
-        """Token for each row of `logits`; row r belongs to sequence sequence_indices[r]."""
+        """Token for each row of `logits`; row r belongs to sequence sequence_indices[r]. Where a
+        sequence's think block has used its budget, the row is first left with the one token that
+        may follow (the logits are changed in place), then chosen from as every row is: a draw
+        is taken for it as for any other."""
+        if self.think is None:
+            return self._choose(logits, sequence_indices)
+        sequence_indices = list(sequence_indices)
+        forced = [(r, self.think[s].forced()) for r, s in enumerate(sequence_indices)]
+        forced = [(r, t) for r, t in forced if t is not None]
+        if forced:
+            ops.force_tokens(logits, [r for r, _ in forced], [t for _, t in forced])
+        tokens = self._choose(logits, sequence_indices)
+        for s, t in zip(sequence_indices, tokens):
+            self.think[s].track(t)
+        return tokens
+
+    def _choose(self, logits, sequence_indices):
         rows = logits.shape[0]
         out = torch.empty(rows, dtype=torch.int32, device=self.device)
         if self.params.greedy:

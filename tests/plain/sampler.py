@@ -128,3 +128,26 @@ def f32_to_bf16_bits(value):
 def bf16_bits_to_f32(bits):
     """Upper 16 bits of a float32; crates/core/src/tensor.rs:7-9."""
     return np.uint32((bits & 0xFFFF) << 16).view(np.float32)
+
+
+def think_forced(history, budget, open_id, close_id, newline_id):
+    """The token that the think budget forces after the generated tokens `history`, or None.
+
+    crates/core/src/sampler.rs:200-231, from the whole history instead of a running state: a
+    block is open if an opening token came after the last closing one; the count is the number
+    of tokens since the last opening token (the opening token itself not counted; a forced
+    line break counts like any token). count + 1 == budget forces the line break, count + 1 >
+    budget the closing token; a budget of 0 forces nothing.
+    """
+    if budget == 0:
+        return None
+    last_open = max((i for i, t in enumerate(history) if t == open_id), default=-1)
+    last_close = max((i for i, t in enumerate(history) if t == close_id), default=-1)
+    if last_open < 0 or last_close > last_open:
+        return None
+    count = len(history) - 1 - last_open
+    if count + 1 == budget:
+        return newline_id
+    if count + 1 > budget:
+        return close_id
+    return None

@@ -200,7 +200,7 @@ class FakeEngine:
                 row = np.zeros(self.spec.vocab_size, dtype=np.float32)
                 row[(e.tokens[j] + 1) % self.spec.vocab_size] = 1.0
                 rows.append(row)
-        return np.stack(rows)
+        return np.stack(rows) if rows else None
 
 
 class ArgmaxChooser:
@@ -368,3 +368,63 @@ def test_params_are_checked_and_seeds_give_streams():
     assert xorshift.initial_state(0) == 0xDEADBEEF and xorshift.step(1) == 1082269761
     assert xorshift.sequence_seed(7, 0) == 7
     assert len({xorshift.sequence_seed(7, i) for i in range(16)}) == 16
+
+
+def test_prompts_in_pieces_give_the_same_tokens():
+    """With a prefill chunk the prompts go through the engine in steps that carry the next piece
+    of every prompt that still has one; a sequence's first token is chosen in the step of its
+    last piece, and decoding goes on as without pieces."""
+    prompts = [[1, 2, 3, 4, 5], [20, 21], [30, 31, 32, 33, 34, 35, 36, 37, 38]]
+    _, _, whole = run(prompts, max_tokens=3, repeat_check=False)
+    eng = FakeEngine()
+    gen = Generator(eng, max_batch=4, make_chooser=ArgmaxChooser, prefill_chunk=4)
+    res = gen.generate(prompts, SamplingParams(temperature=0.0, max_tokens=3, repeat_check=False))
+    assert [r.tokens for r in res] == [r.tokens for r in whole]
+    assert eng.steps[:3] == [[(0, 4), (1, 2), (2, 4)], [(0, 1), (2, 4)], [(2, 1)]]
+    assert eng.steps[3] == [(0, 1), (1, 1), (2, 1)]                  # then one token each
+    assert gen.stats.prompt_tokens == 16 and eng.cache.slots.held_count == 0
+    # prompts no longer than the chunk: one step as before
+    eng2 = FakeEngine()
+    Generator(eng2, make_chooser=ArgmaxChooser, prefill_chunk=16).generate(
+        prompts, SamplingParams(temperature=0.0, max_tokens=1))
+    assert eng2.steps == [[(0, 5), (1, 2), (2, 9)]]
+    with pytest.raises(RequestError):
+        Generator(FakeEngine(), prefill_chunk=-1)
+
+
+def test_think_budget_follows_the_plain_rule():
+    from herbert_rs_amd.sampling import ThinkBudget, ThinkTokens
+    from .plain.sampler import think_forced
+    ids = ThinkTokens(open_id=5, close_id=6, newline_id=7)
+    # by hand: budget 3: after <think> a b the line break is forced, then </think>, then nothing
+    tb, seen = ThinkBudget(3, ids), []
+    for tok in (1, 5, 2, 2, 7, 6, 2):
+        seen.append(tb.forced())
+        tb.track(tok)
+    assert seen == [None, None, None, None, 7, 6, None]
+    # a budget of one (the command line's --nothink): line break, then the closing token
+    tb, seen = ThinkBudget(1, ids), []
+    for tok in (5, 7, 6, 3):
+        seen.append(tb.forced())
+        tb.track(tok)
+    assert seen == [None, 7, 6, None]
+    # a model that ignores nothing is forced nothing; a block opened by the prompt counts from there
+    tb = ThinkBudget(2, ids)
+    tb.set_in_think()
+    assert tb.forced() is None
+    tb.track(9)
+    assert tb.forced() == 7
+    # random streams, every prefix, against the rule written over the whole history
+    rng = np.random.default_rng(3)
+    for budget in (0, 1, 2, 5):
+        for _ in range(40):
+            stream = rng.choice([1, 2, 3, 5, 6, 7], size=30, p=[0.25, 0.25, 0.2, 0.12, 0.08, 0.1]).tolist()
+            tb, history = ThinkBudget(budget, ids), []
+            for tok in stream:
+                want = think_forced(history, budget, 5, 6, 7)
+                assert tb.forced() == want, (budget, history)
+                tok = want if want is not None else tok
+                tb.track(tok)
+                history.append(tok)
+    with pytest.raises(RequestError, match="think_tokens"):
+        SamplingParams(think_budget=3).validate()

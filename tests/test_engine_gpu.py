@@ -478,6 +478,43 @@ def test_top_p_without_top_k_looks_among_the_largest_first(V):
     assert [int(s) & ((1 << 64) - 1) for s in sampler.states.tolist()] == [r.state for r in rngs]
 
 
+@pytest.mark.parametrize("temperature", [0.0, 0.8])
+def test_sampler_caps_a_think_block(temperature):
+    """The Sampler with a think budget of 3: sequence 0 opens a block (its logits say so), then
+    wants token 11 for ever: it gets 11, 11, the line break, the closing token, then 11 again;
+    sequence 1 never opens one and is left alone. A forced row keeps one finite logit, and a
+    draw is taken for it as for any row (crates/core/src/sampler.rs:72-145 runs on the forced
+    logits), so the generators stay in step with the plain ones."""
+    from herbert_rs_amd.sampling import SamplingParams, ThinkTokens, xorshift
+    from herbert_rs_amd.sampling.sampler import Sampler
+    V, ids = 3000, ThinkTokens(open_id=5, close_id=6, newline_id=7)
+    params = SamplingParams(temperature=temperature, top_k=4, top_p=0.9, max_tokens=9, seed=3, think_budget=3,
+                            think_tokens=ids)
+    sampler = Sampler(params, 2, V, torch.device("cuda"))
+
+    def logits_for(a, b):
+        rows = torch.full((2, V), -4.0)
+        rows[0, a] = rows[1, b] = 30.0
+        return rows.cuda()
+
+    got = []
+    for step in range(7):
+        logits = logits_for(5 if step == 0 else 11, 12)
+        got.append(sampler.choose(logits, [0, 1]))
+        if step in (3, 4):
+            row = logits[0].cpu()
+            assert torch.isfinite(row).sum() == 1 and torch.isfinite(row[7 if step == 3 else 6])
+            assert torch.isfinite(logits[1]).all()
+    assert [g[0] for g in got] == [5, 11, 11, 7, 6, 11, 11]
+    assert [g[1] for g in got] == [12] * 7
+    if temperature > 0:
+        rngs = [plain_sampler.XorShift64(xorshift.sequence_seed(3, i)) for i in range(2)]
+        for r in rngs:
+            for _ in range(7):
+                r.next_f32()
+        assert [int(s) & ((1 << 64) - 1) for s in sampler.states.tolist()] == [r.state for r in rngs]
+
+
 def test_sampler_draw_and_top_p_edge_on_exact_probabilities():
     """Equal logits give probabilities that are exact in float32 whatever the exponential's
     rounding (exp(0) = 1), so two rules show without a tolerance. (1) The draw is the upper bits

@@ -298,12 +298,13 @@ def test_decode_graphs_and_their_logits_are_bounded(model_root):
     engine.cache.check()
 
 
-def write_tokenizer(folder, vocab):
+def write_tokenizer(folder, vocab, renamed=None):
     """A tokenizer.json of whole words w0, w1, ... and the chat format's special tokens, written
-    with the tokenizers package; the model's last ids are the specials."""
+    with the tokenizers package; the model's last ids are the specials. `renamed`: {id: word} for
+    ids that are to be other words than w<id>."""
     from tokenizers import Tokenizer, decoders, models, pre_tokenizers
     specials = ["<|im_start|>", "<|im_end|>", "system", "user", "assistant"]
-    words = {f"w{i}": i for i in range(vocab - len(specials))}
+    words = {(renamed or {}).get(i, f"w{i}"): i for i in range(vocab - len(specials))}
     for i, t in enumerate(specials):
         words[t] = vocab - len(specials) + i
     tok = Tokenizer(models.WordLevel(words, unk_token="w0"))
@@ -313,9 +314,9 @@ def write_tokenizer(folder, vocab):
     return tok, words
 
 
-def cli_folder(model_root, tmp_path):
-    src = make_folder(model_root, "A", "float32")
-    folder = str(tmp_path / "A_text")
+def cli_folder(model_root, tmp_path, name="A"):
+    src = make_folder(model_root, name, "float32")
+    folder = str(tmp_path / f"{name}_text")
     os.makedirs(folder)
     os.link(os.path.join(src, "model.safetensors"), os.path.join(folder, "model.safetensors"))
     with open(os.path.join(src, "config.json")) as f:
@@ -358,6 +359,56 @@ def test_cli_with_a_tokenizer_chat_template_and_stop_strings(model_root, tmp_pat
     assert out.returncode == 0, out.stderr
     assert out.stdout.strip() == " ".join(said[:upto]) and upto <= 4
     assert "Stop reason:     stop_sequence" in out.stderr and f"Output tokens:   {upto}" in out.stderr
+
+
+def test_cli_think_budget_system_file_and_prompt_in_pieces(model_root, tmp_path):
+    """--think-budget caps a think block as the reference's sampler does
+    (crates/core/src/sampler.rs:200-243): the tokenizer here calls an ordinary word that the model
+    says once <think>, so the block opens by itself; after budget - 1 tokens the line break's id (the
+    architecture's own, the tokenizer has none) is forced, then </think>, then the model goes on
+    freely. --nothink is a budget of one. The system prompt comes from a file and the prompt goes
+    through the engine in pieces of 5 tokens; neither changes a token."""
+    from .plain.sampler import think_forced
+    folder, raw = cli_folder(model_root, tmp_path, "C")      # (a model that says many different words)
+    tok, words = write_tokenizer(folder, raw["vocab_size"])
+    prompt = "w5 w17 w3"
+    text = "<|im_start|>system\nw9<|im_end|>\n<|im_start|>user\n" + prompt + "<|im_end|>\n<|im_start|>assistant\n"
+    ids = tok.encode(text, add_special_tokens=False).ids
+    cfg, w = plain_folder(folder)
+    free = plain.greedy(cfg, w, ids, 12)
+    newline_id = 198
+    # an ordinary word that the model says once becomes <think> (said again it would open a new block)
+    at = next((j for j, t in enumerate(free[:6]) if t < raw["vocab_size"] - 5 and t not in ids and t != newline_id
+               and free.count(t) == 1), None)
+    assert at is not None, free
+    open_id = free[at]
+    close_id = next(i for i in range(20, 200) if i not in free and i not in ids and i != newline_id)
+    tok, words = write_tokenizer(folder, raw["vocab_size"], {open_id: "<think>", close_id: "</think>"})
+    assert tok.encode(text, add_special_tokens=False).ids == ids and tok.token_to_id("<think>") == open_id
+
+    def capped(budget, n):
+        out = []
+        for _ in range(n):
+            logits = plain.forward(cfg, w, ids + out)[-1]
+            forced = think_forced(out, budget, open_id, close_id, newline_id)
+            out.append(forced if forced is not None else plain.argmax(logits))
+        return out
+
+    system = tmp_path / "system.txt"
+    system.write_text("w9")
+    for flags, budget in ((["--think-budget", "3"], 3), (["--nothink"], 1)):
+        n = at + budget + 4
+        want = capped(budget, n)
+        assert want[at] == open_id and want[at + budget] == newline_id and want[at + budget + 1] == close_id
+        assert close_id not in capped(0, n)
+        out = run_cli(folder, "--prompt", prompt, "--system-file", str(system), "--max-tokens", str(n - 1),
+                      "--ignore-eos", "--prefill-chunk-size", "5", "--show-specials", *flags)
+        assert out.returncode == 0, out.stderr
+        assert out.stdout.strip() == tok.decode(want, skip_special_tokens=False).strip(), (out.stdout, want)
+    # think tokens that the model's vocabulary does not hold are refused, not sampled
+    write_tokenizer(folder, raw["vocab_size"])
+    out = run_cli(folder, "--prompt", prompt, "--max-tokens", "4", "--nothink")
+    assert out.returncode == 1 and "outside the model's vocabulary" in out.stderr
 
 
 def test_cli_interrupt_ends_generation_cleanly(model_root, tmp_path):
