@@ -245,6 +245,40 @@ __device__ __forceinline__ void choose_bin(const int* hist, int* wave_totals, in
     __syncthreads();
 }
 
+// The largest scaled logit of a chunk of SAMPLE_CHUNK logits (thread t holds elements t, t + 1024, ...
+// in v) and the sum of exp(scaled - that), added up in a fixed order: a thread's eight in their
+// order, the lanes of a wave by a tree, the waves one after the other. Thread 0 writes both to ms.
+__device__ __forceinline__ void chunk_max_and_sum(const float (&v)[SAMPLE_CHUNK / SAMPLE_THREADS], int len,
+                                                  float temperature, float* wave_vals, float* ms) {
+    constexpr int PER = SAMPLE_CHUNK / SAMPLE_THREADS;
+    const int tid = threadIdx.x, lane = tid & (HB_WAVE - 1), wave = tid / HB_WAVE;
+    float mv = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < PER; ++u)
+        if (tid + u * SAMPLE_THREADS < len) mv = fmaxf(mv, v[u] / temperature);
+    mv = hb_wave_max(mv);
+    if (lane == 0) wave_vals[wave] = mv;
+    __syncthreads();
+    float cmax = wave_vals[0];
+    for (int w = 1; w < SAMPLE_THREADS / HB_WAVE; ++w) cmax = fmaxf(cmax, wave_vals[w]);
+    __syncthreads();
+    float part = 0.f;
+    if (cmax != -INFINITY) {
+#pragma unroll
+        for (int u = 0; u < PER; ++u)
+            if (tid + u * SAMPLE_THREADS < len) part += expf(v[u] / temperature - cmax);
+    }
+    for (int d = HB_WAVE / 2; d > 0; d >>= 1) part += __shfl_down(part, d, HB_WAVE);
+    if (lane == 0) wave_vals[wave] = part;
+    __syncthreads();
+    if (tid == 0) {
+        float sum = 0.f;
+        for (int w = 0; w < SAMPLE_THREADS / HB_WAVE; ++w) sum += wave_vals[w];
+        ms[0] = cmax;
+        ms[1] = sum;
+    }
+}
+
 // The first of two kernels when a row is long: block (chunk, row) keeps the keys of its SAMPLE_CHUNK
 // logits in LDS, finds its own top_k among them (ties: lower index first) and leaves them, in any
 // order, in pre_key / pre_idx [row][chunk][top_k]. A single block walks a row at about 24 GB/s
@@ -285,34 +319,8 @@ sample_chunk_topk_kernel(const float* __restrict__ logits, int ld, int V, float 
         n_out = 0;
         eq_taken = 0;
     }
-    if (chunk_ms) {
-        float mv = -INFINITY;
-#pragma unroll
-        for (int u = 0; u < PER; ++u)
-            if (tid + u * SAMPLE_THREADS < len) mv = fmaxf(mv, v[u] / temperature);
-        mv = hb_wave_max(mv);
-        if (lane == 0) wave_vals[wave] = mv;
-        __syncthreads();
-        float cmax = wave_vals[0];
-        for (int w = 1; w < SAMPLE_THREADS / HB_WAVE; ++w) cmax = fmaxf(cmax, wave_vals[w]);
-        __syncthreads();
-        float part = 0.f;
-        if (cmax != -INFINITY) {
-#pragma unroll
-            for (int u = 0; u < PER; ++u)
-                if (tid + u * SAMPLE_THREADS < len) part += expf(v[u] / temperature - cmax);
-        }
-        for (int d = HB_WAVE / 2; d > 0; d >>= 1) part += __shfl_down(part, d, HB_WAVE);
-        if (lane == 0) wave_vals[wave] = part;
-        __syncthreads();
-        if (tid == 0) {
-            float sum = 0.f;
-            for (int w = 0; w < SAMPLE_THREADS / HB_WAVE; ++w) sum += wave_vals[w];
-            float* ms = chunk_ms + ((size_t)blockIdx.y * gridDim.x + c) * 2;
-            ms[0] = cmax;
-            ms[1] = sum;
-        }
-    }
+    if (chunk_ms)
+        chunk_max_and_sum(v, len, temperature, wave_vals, chunk_ms + ((size_t)blockIdx.y * gridDim.x + c) * 2);
     __syncthreads();
     if (len <= top_k) {                       // all of a short chunk
         for (int j = tid; j < len; j += SAMPLE_THREADS) {
@@ -908,6 +916,95 @@ extern "C" int hb_sample(const float* logits, int ld, int R, int V, float temper
     sample_finish_kernel<<<R, 1024, 0, stream>>>(scratch_keys, scratch_idx, P2, n, sorted, top_p, rng,
                                                  rng_index, out);
     HB_CHECK_LAUNCH("sample_finish");
+    return 0;
+}
+
+// Temperature sampling over a whole long row (no top-k, no top-p), in two kernels: a block for every
+// SAMPLE_CHUNK logits leaves the chunk's largest scaled logit and its sum of exponentials; a block a
+// row then adds up the chunks in their order for the softmax's denominator, takes the draw, finds
+// the chunk in which the running probability passes it and walks that chunk (ordered_sum). The
+// candidates stay in index order, as the reference has them here (crates/core/src/sampler.rs:84-144).
+__global__ void __launch_bounds__(SAMPLE_THREADS)
+sample_chunk_sums_kernel(const float* __restrict__ logits, int ld, int V, float temperature,
+                         float* __restrict__ chunk_ms) {
+    __shared__ float wave_vals[SAMPLE_THREADS / HB_WAVE];
+    constexpr int PER = SAMPLE_CHUNK / SAMPLE_THREADS;
+    const int tid = threadIdx.x, c = blockIdx.x, first = c * SAMPLE_CHUNK;
+    const int len = V - first < SAMPLE_CHUNK ? V - first : SAMPLE_CHUNK;
+    const float* row = logits + (size_t)blockIdx.y * ld + first;
+    float v[PER];
+#pragma unroll
+    for (int u = 0; u < PER; ++u) {
+        const int j = tid + u * SAMPLE_THREADS;
+        v[u] = j < len ? row[j] : 0.f;
+    }
+    chunk_max_and_sum(v, len, temperature, wave_vals, chunk_ms + ((size_t)blockIdx.y * gridDim.x + c) * 2);
+}
+
+__global__ void __launch_bounds__(1024)
+sample_all_finish_kernel(const float* __restrict__ logits, int ld, int V, float temperature,
+                         const float* __restrict__ chunk_ms, unsigned long long* __restrict__ rng,
+                         const int* __restrict__ rng_index, int* __restrict__ out) {
+    __shared__ float buf[FINISH_CHUNK];
+    __shared__ float red[16];
+    __shared__ float s_max, s_inv, s_r, s_before, s_total;
+    __shared__ int s_chunk, s_found;
+    const int tid = threadIdx.x;
+    const int chunks = (V + SAMPLE_CHUNK - 1) / SAMPLE_CHUNK;
+    const float* row = logits + (size_t)blockIdx.x * ld;
+    if (tid == 0) {
+        const float* ms = chunk_ms + (size_t)blockIdx.x * chunks * 2;
+        float mx = -INFINITY;
+        for (int c = 0; c < chunks; ++c) mx = fmaxf(mx, ms[2 * c]);
+        float z = 0.f;
+        for (int c = 0; c < chunks; ++c)
+            if (ms[2 * c] != -INFINITY) z += ms[2 * c + 1] * expf(ms[2 * c] - mx);
+        const float inv = 1.0f / z;
+        unsigned long long* st = rng + (rng_index ? rng_index[blockIdx.x] : blockIdx.x);
+        const float r = xorshift_next_f32(st);
+        // the chunk in which the running probability first exceeds the draw
+        float before = 0.f;
+        int chosen = -1;
+        for (int c = 0; c < chunks; ++c) {
+            const float mass = ms[2 * c] != -INFINITY ? ms[2 * c + 1] * expf(ms[2 * c] - mx) * inv : 0.f;
+            if (r < before + mass) {
+                chosen = c;
+                break;
+            }
+            before += mass;
+        }
+        s_max = mx;
+        s_inv = inv;
+        s_r = r;
+        s_before = before;
+        s_chunk = chosen;
+    }
+    __syncthreads();
+    if (s_chunk < 0) {                      // the draw lies beyond the last running sum: the last token
+        if (tid == 0) out[blockIdx.x] = V - 1;
+        return;
+    }
+    const int first = s_chunk * SAMPLE_CHUNK;
+    const int len = V - first < SAMPLE_CHUNK ? V - first : SAMPLE_CHUNK;
+    const float max_val = s_max, inv = s_inv;
+    int marked;
+    ordered_sum<2>(len, s_r - s_before, &marked, buf, red, &s_found, &s_total,
+                   [&](int i) { return expf(row[first + i] / temperature - max_val) * inv; });
+    // (a chunk whose own walk ends just short of the mark, by rounding: its last token)
+    if (tid == 0) out[blockIdx.x] = first + (marked >= 0 ? marked : len - 1);
+}
+
+// chunk_ms: float [R, ceil(V / 8192), 2].
+extern "C" int hb_sample_all(const float* logits, int ld, int R, int V, float temperature, unsigned long long* rng,
+                             const int* rng_index, int* out, float* chunk_ms, hipStream_t stream) {
+    HB_REQUIRE(R > 0 && R <= 65535 && V > 0 && ld >= V, "sample (whole row): bad sizes (R=%d, V=%d, ld=%d)", R, V, ld);
+    HB_REQUIRE(temperature > 0.f, "sample (whole row): temperature must be > 0 (0 is argmax)");
+    HB_REQUIRE(chunk_ms, "sample (whole row): needs its buffer");
+    const int chunks = (V + SAMPLE_CHUNK - 1) / SAMPLE_CHUNK;
+    sample_chunk_sums_kernel<<<dim3(chunks, R), SAMPLE_THREADS, 0, stream>>>(logits, ld, V, temperature, chunk_ms);
+    HB_CHECK_LAUNCH("sample_chunk_sums");
+    sample_all_finish_kernel<<<R, 1024, 0, stream>>>(logits, ld, V, temperature, chunk_ms, rng, rng_index, out);
+    HB_CHECK_LAUNCH("sample_all_finish");
     return 0;
 }
 

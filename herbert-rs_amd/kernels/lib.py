@@ -40,6 +40,7 @@ SIGNATURES = {
         "hb_sample": [_P, _I, _I, _I, _F, _I, _F, _P, _P, _P, _P, _P, _I, _P, _P, _P],
         "hb_sample_nucleus": [_P, _I, _I, _I, _F, _F, _P, _P, _P, _P, _P, _P, _P],
         "hb_force_tokens": [_P, _I, _I, _I, _P, _P, _I, _P],
+        "hb_sample_all": [_P, _I, _I, _I, _F, _P, _P, _P, _P, _P],
     },
 }
 

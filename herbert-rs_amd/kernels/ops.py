@@ -298,6 +298,25 @@ def sample_nucleus(logits, temperature, top_p, rng_states, rng_index, out, buffe
              sums.data_ptr(), _stream())
 
 
+def sample_all(logits, temperature, rng_states, rng_index, out, sums):
+    """Temperature sampling over whole rows (no top-k, no top-p): a block for every 8192 logits adds
+    up its part of the softmax, a block a row takes the draw and walks the chunk it falls into.
+    `sums`: float32 of at least R * ceil(V / 8192) * 2 elements."""
+    _check(logits, "logits", torch.float32, (None, None))
+    R, V = logits.shape
+    _check(out, "out", torch.int32, (R,))
+    _check(rng_states, "rng_states", torch.int64, (None,))
+    if rng_index is not None:
+        _check(rng_index, "rng_index", torch.int32, (R,))
+    elif rng_states.shape[0] < R:
+        raise BackendError("sample: fewer generator states than rows")
+    _check(sums, "chunk sums", torch.float32, (None,))
+    if sums.numel() < R * (-(-V // SAMPLE_CHUNK)) * 2:
+        raise BackendError("sample: the buffer of the chunks' sums is too small for these logits")
+    lib.call("sampling", "hb_sample_all", logits.data_ptr(), V, R, V, float(temperature), rng_states.data_ptr(),
+             _ptr(rng_index), out.data_ptr(), sums.data_ptr(), _stream())
+
+
 def force_tokens(logits, rows, tokens):
     """Every logit of row rows[i] but that of tokens[i] becomes -inf, in place: the next choice in
     that row can only be that token. rows, tokens: lists of ints (checked here against the shape)."""

@@ -31,6 +31,7 @@ class Sampler:
         self._scratch = None
         self._sifted = None
         self._nucleus = None
+        self._sums = None
         # a cap on think blocks: one counter a sequence, fed with every token chosen for it
         self.think = None
         if params.think_budget > 0:
@@ -87,6 +88,13 @@ class Sampler:
             vocab = logits.shape[1]
             if not 0 < p.top_k < vocab and p.top_p < 1.0 and vocab > ops.NUCLEUS_CANDIDATES:
                 return self._top_p_only(logits, index, out)
+            if not 0 < p.top_k < vocab and p.top_p >= 1.0 and vocab > ops.SAMPLE_CHUNK:
+                # the whole row, no cut: nothing is sorted, the chunks of a long row are added up side by side
+                need = rows * (-(-vocab // ops.SAMPLE_CHUNK)) * 2
+                if self._sums is None or self._sums.numel() < need:
+                    self._sums = torch.empty(need, dtype=torch.float32, device=self.device)
+                ops.sample_all(logits, p.temperature, self.states, index, out, self._sums)
+                return out.tolist()
             ops.sample(logits, p.temperature, p.top_k, p.top_p,
                        self.states, index, out, self._scratch_for(rows), self._sifted_for(rows))
         return out.tolist()

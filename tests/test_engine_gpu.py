@@ -478,6 +478,45 @@ def test_top_p_without_top_k_looks_among_the_largest_first(V):
     assert [int(s) & ((1 << 64) - 1) for s in sampler.states.tolist()] == [r.state for r in rngs]
 
 
+@pytest.mark.parametrize("V", [8193, 20000, 151936])
+def test_temperature_sampling_over_whole_long_rows(V):
+    """No top-k, no top-p on rows of more than 8192 logits through the Sampler: the chunks of a row
+    are added up side by side and the draw is looked for in the chunk it falls into; the plain
+    sampler's tokens, draw after draw (either neighbour where the draw lies within rounding of a
+    boundary), and the generators in step."""
+    from herbert_rs_amd.sampling import SamplingParams, xorshift
+    from herbert_rs_amd.sampling.sampler import Sampler
+    temperature = 0.9
+    g = torch.Generator().manual_seed(V + 1)
+    logits = torch.stack([torch.randn(V, generator=g) * 3.0, torch.randn(V, generator=g) * 0.5,
+                          torch.randn(V, generator=g) * 8.0, torch.randn(V, generator=g)])
+    logits[3, 5000:] = -float("inf")                   # whole chunks without a finite logit
+    R = logits.shape[0]
+    dev_logits = logits.cuda()
+    sampler = Sampler(SamplingParams(temperature=temperature, top_k=0, top_p=1.0, max_tokens=4, seed=5), R, V,
+                      torch.device("cuda"))
+    rngs = [plain_sampler.XorShift64(xorshift.sequence_seed(5, i)) for i in range(R)]
+    works = [plain_sampler.candidates(logits[r].numpy(), temperature, 0, 1.0) for r in range(R)]
+    # the same probabilities summed in float64: where the exact running sum passes a draw
+    exact = [np.cumsum(np.array([p for _, p in w], dtype=np.float64)) for w in works]
+    for draw in range(12):
+        got = sampler.choose(dev_logits, list(range(R)))
+        for r in range(R):
+            u = rngs[r].next_f32()
+            want = plain_sampler.pick(works[r], u)
+            if got[r] != want:
+                # A running sum of V float32 terms drifts by about sqrt(V) half-ulps, the plain sampler's
+                # single one and the kernel's chunk by chunk differently, and so do their denominators:
+                # among tokens of negligible probability the draw then falls on another one. What must
+                # hold is that the token's stretch of the exact running sum lies within that drift of
+                # the draw (a wrong chunk or an edge missed would be off by a chunk's share, per cents).
+                drift = 8.0 * np.sqrt(V) * 2.0 ** -24
+                g_ = got[r]
+                assert exact[r][g_] >= u - drift and (g_ == 0 or exact[r][g_ - 1] <= u + drift), \
+                    (draw, r, g_, want, float(exact[r][g_]), float(u))
+    assert [int(s) & ((1 << 64) - 1) for s in sampler.states.tolist()] == [r.state for r in rngs]
+
+
 @pytest.mark.parametrize("temperature", [0.0, 0.8])
 def test_sampler_caps_a_think_block(temperature):
     """The Sampler with a think budget of 3: sequence 0 opens a block (its logits say so), then
