@@ -204,9 +204,18 @@ def main():
         tokens = [ids(1)[0] for _ in range(batch)]
         held, chunk, out = 0, 2048, []
 
+        ahead = [None]
+
         def one():
-            logits = engine.step([StepEntry(s, [t], [0]) for s, t in zip(slots, tokens)])
-            return chooser.choose(logits, range(batch))
+            """A decode step as the generation loop runs it: put on the stream with the tokens of the
+            step before still on the GPU, whose copy the host reads while this step runs."""
+            before = ahead[0]
+            if before is None:
+                logits = engine.step([StepEntry(s, [t], [0]) for s, t in zip(slots, tokens)])
+            else:
+                logits = engine.step([StepEntry(s, [0], [0]) for s in slots], tokens_on_device=before.device)
+            ahead[0] = chooser.choose_ahead(logits, range(batch))
+            return tokens if before is None else chooser.read(before)
         for c, steps, warmup in plan:
             fill = c - steps - warmup - held
             if fill < 0:

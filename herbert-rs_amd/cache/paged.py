@@ -44,7 +44,10 @@ class KVGroup:
         # entries of the device table that are not held point at page 0: a kernel never reads
         # them for a valid position, and an index that is always in range cannot fault
         self.table = torch.zeros((n_slots, self.pages_per_slot), dtype=torch.int32, device=device)
-        self.first_page = np.zeros(n_slots, dtype=np.int64)   # first logical page still held
+        # a slot holds the logical pages [first_page, held_end): it fills from the front as it grows,
+        # a window gives pages back at the front, a roll-back at the end
+        self.first_page = np.zeros(n_slots, dtype=np.int64)
+        self.held_end = [0] * n_slots
 
     def view(self, entry):
         i = self.entries.index(entry)
@@ -55,21 +58,19 @@ class KVGroup:
 
     def pages_missing(self, slot, new_length):
         """How many pages `ensure(slot, new_length)` would take."""
-        row = self.table_host[slot]
-        return int((row[int(self.first_page[slot]):pages_for(new_length)] < 0).sum())
+        return max(0, pages_for(new_length) - max(self.held_end[slot], int(self.first_page[slot])))
 
     def ensure(self, slot, new_length):
         """Hold a page for every position below new_length that a query may still see."""
-        row = self.table_host[slot]
-        first_new = None
         last = pages_for(new_length)
-        for p in range(int(self.first_page[slot]), last):
-            if row[p] < 0:
-                row[p] = self.pages.take()
-                if first_new is None:
-                    first_new = p
-        if first_new is not None:
-            self._upload(slot, first_new, last)
+        first_new = max(self.held_end[slot], int(self.first_page[slot]))
+        if first_new >= last:
+            return
+        row = self.table_host[slot]
+        for p in range(first_new, last):
+            row[p] = self.pages.take()
+        self.held_end[slot] = last
+        self._upload(slot, first_new, last)
 
     def _upload(self, slot, a, b):
         self.table[slot, a:b] = torch.from_numpy(np.maximum(self.table_host[slot, a:b], 0)).to(
@@ -104,10 +105,11 @@ class KVGroup:
         row = self.table_host[slot]
         if not self.can_truncate(slot, length):
             raise CacheError("cannot roll a windowed cache back past keys it has given up")
-        for p in range(pages_for(length), self.pages_per_slot):
+        for p in range(pages_for(length), self.held_end[slot]):
             if row[p] >= 0:
                 self.pages.give_back(int(row[p]))
                 row[p] = -1
+        self.held_end[slot] = min(self.held_end[slot], pages_for(length))
 
     def free_slot(self, slot):
         row = self.table_host[slot]
@@ -115,6 +117,7 @@ class KVGroup:
             self.pages.give_back(int(row[p]))
         row[:] = -1
         self.first_page[slot] = 0
+        self.held_end[slot] = 0
 
 
 class StateGroup:
@@ -267,3 +270,8 @@ class Cache:
             for slot in range(self.n_slots):
                 if not self.slots.is_held(slot) and (g.table_host[slot] >= 0).any():
                     raise CacheError(f"free slot {slot} still holds pages")
+                has = np.nonzero(g.table_host[slot] >= 0)[0].tolist()
+                first, end = int(g.first_page[slot]), g.held_end[slot]
+                if has != list(range(first, end)):
+                    raise CacheError(f"slot {slot} holds the pages {has}, not the stretch [{first}, {end}) "
+                                     "it keeps count of")

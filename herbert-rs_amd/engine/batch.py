@@ -100,7 +100,7 @@ class StaticDecodeMeta:
         self.host = torch.empty(7 * B + 1, dtype=torch.int32, pin_memory=True)
         self.copied = None       # event after the last copy out of `host`
         self.dev = torch.zeros(7 * B + 1, dtype=torch.int32, device=device)
-        h = self.host.numpy()
+        h = self.host_array = self.host.numpy()
         h[2 * B:3 * B] = np.arange(B)            # seq_of
         h[4 * B:5 * B + 1] = np.arange(B + 1)    # seq_starts
         h[6 * B + 1:7 * B + 1] = np.arange(B)    # want_rows
@@ -116,19 +116,20 @@ class StaticDecodeMeta:
         B = self.batch_size
         if self.copied is not None:
             self.copied.synchronize()        # the pinned buffer is free to be written again
-        h = self.host.numpy()
-        for i, e in enumerate(entries):
-            h[i] = e.tokens[0]
-            h[B + i] = start_lengths[i]
-            h[3 * B + i] = e.slot
-            h[5 * B + 1 + i] = start_lengths[i] + 1
+        h = self.host_array
+        h[0:B] = [e.tokens[0] for e in entries]
+        h[B:2 * B] = start_lengths
+        h[3 * B:4 * B] = [e.slot for e in entries]
+        context = h[5 * B + 1:6 * B + 1]
+        np.add(h[B:2 * B], 1, out=context)
         self.dev.copy_(self.host, non_blocking=True)
         if self.dev.is_cuda:
-            self.copied = torch.cuda.Event()
+            if self.copied is None:
+                self.copied = torch.cuda.Event()
             self.copied.record()
         m = self.meta
-        m.host_context = h[5 * B + 1:6 * B + 1].copy()
-        m.max_context = int(m.host_context.max())
+        m.host_context = context.copy()
+        m.max_context = int(max(start_lengths)) + 1
         m.max_position = m.max_context - 1
         m.context_bucket = bucket(m.max_context)
         return m

@@ -158,11 +158,22 @@ class Engine:
         self.cache.truncate(slot, int(length))
 
     # ---- the step
-    def step(self, entries):
+    accepts_device_tokens = True
+
+    def step(self, entries, tokens_on_device=None):
         """Run the entries' tokens; returns float32 logits [wanted, vocab] on the GPU
-        (rows in the order of the entries and of their `want`), or None if nothing is wanted."""
+        (rows in the order of the entries and of their `want`), or None if nothing is wanted.
+        `tokens_on_device` (int32 [entries] on the GPU, every entry bringing one token): the
+        tokens are taken from there, in the stream's order, and the entries' own are only
+        placeholders; so a step can be put on the stream before the host has seen the tokens
+        that the step before it chose."""
         if not entries:
             raise RequestError("a step needs at least one sequence")
+        if tokens_on_device is not None:
+            if (tokens_on_device.dtype != torch.int32 or tuple(tokens_on_device.shape) != (len(entries),)
+                    or not tokens_on_device.is_cuda or any(len(e.tokens) != 1 for e in entries)):
+                raise RequestError("tokens_on_device must be int32 [entries] on the engine's GPU, for entries "
+                                   "of one token each")
         vocab = self.spec.vocab_size
         seen = set()
         starts = []
@@ -172,10 +183,15 @@ class Engine:
             seen.add(e.slot)
             if len(e.tokens) == 0:
                 raise RequestError("a sequence of a step has no tokens")
-            ids = np.asarray(e.tokens)
-            if ids.dtype.kind not in "iu":
-                raise RequestError("token ids must be integers")
-            low, high = int(ids.min()), int(ids.max())
+            if len(e.tokens) == 1:              # decoding: no array for one number
+                low = high = e.tokens[0]
+                if not isinstance(low, (int, np.integer)) or isinstance(low, bool):
+                    raise RequestError("token ids must be integers")
+            else:
+                ids = np.asarray(e.tokens)
+                if ids.dtype.kind not in "iu":
+                    raise RequestError("token ids must be integers")
+                low, high = int(ids.min()), int(ids.max())
             if low < 0 or high >= vocab:
                 raise RequestError(f"token id {low if low < 0 else high} out of range (vocab_size {vocab})")
             for j in e.want:
@@ -191,9 +207,11 @@ class Engine:
         self.cache.reserve_all([(e.slot, len(e.tokens)) for e in entries])
         try:
             if self.use_graphs and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
-                logits = self._decode_step(entries, starts)
+                logits = self._decode_step(entries, starts, tokens_on_device)
             else:
                 meta = batching.pack(entries, starts, self.device)
+                if tokens_on_device is not None:
+                    meta.token_ids.copy_(tokens_on_device)
                 logits = self.model.forward(self.rt, meta, self.cache)
         except Exception:
             for e in entries:       # nothing was committed: give back what was taken for the step
@@ -204,7 +222,7 @@ class Engine:
         self.steps_run += 1
         return logits
 
-    def _decode_step(self, entries, starts):
+    def _decode_step(self, entries, starts, tokens_on_device=None):
         """One token for each sequence, every logit wanted: the launch-bound case. The step's
         metadata lives in fixed buffers; from the second step of a shape on, the forward pass is a
         captured HIP graph that is replayed, so that the host launches one graph and not hundreds
@@ -225,6 +243,8 @@ class Engine:
             state = self._decode[B] = _DecodeState(StaticDecodeMeta(B, self.device), logits)
         self._decode.move_to_end(B)
         meta = state.static.update(entries, starts)
+        if tokens_on_device is not None:
+            meta.token_ids.copy_(tokens_on_device)      # behind the copy from the host, before the graph
         key = (B, meta.context_bucket)
         graph = self._graphs.get(key)
         if graph is not None:

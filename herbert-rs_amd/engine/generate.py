@@ -92,9 +92,11 @@ class Generator:
     """Runs requests through an engine. `make_chooser(params, n, vocab, device)` builds the object
     whose `choose(logits, sequence_indices)` picks tokens (the GPU sampler by default)."""
 
-    def __init__(self, engine, max_batch=64, make_chooser=None, prefill_chunk=None):
+    def __init__(self, engine, max_batch=64, make_chooser=None, prefill_chunk=None, run_ahead=True):
         self.engine = engine
         self.max_batch = int(max_batch)
+        # decode steps are put on the GPU's stream one ahead of the host where engine and chooser can
+        self.run_ahead = bool(run_ahead)
         # prompts longer than this many tokens are fed in pieces of that size, one step a piece
         # (the reference's prefill_chunk_size: crates/cli/src/main.rs:400-408)
         self.prefill_chunk = int(prefill_chunk) if prefill_chunk else None
@@ -158,6 +160,41 @@ class Generator:
                 first.update(zip(ending, chooser.choose(logits, ending)))
         return [first[i] for i in live]
 
+    def _decode_ahead(self, live, slots, generated, params, chooser, take):
+        """Decoding with the host one step behind the GPU. The tokens that a step chooses stay on
+        the GPU, and the next step is put on the stream with them at once, before the host has
+        seen them; the host reads a step's tokens while the next one runs, so the GPU does not
+        wait for the host's share of a step. A sequence whose newest token turns out to end it
+        (end of sequence, a stop token, the caller's word) has then already been through one step
+        more: that step's work on it is thrown away, its slot is given back as always, and every
+        other sequence's tokens are what they would have been. Sequences that end for a reason the
+        host knows beforehand (max_tokens, the model's last position) are not taken ahead."""
+        eng = self.engine
+
+        def launch(order, device_tokens):
+            entries = [StepEntry(slots[i], [generated[i][-1]] if device_tokens is None else [0], [0])
+                       for i in order]
+            logits = eng.step(entries, tokens_on_device=device_tokens)
+            self.stats.decode_steps += 1
+            return chooser.choose_ahead(logits, order), {i: eng.cache.length(slots[i]) for i in order}
+
+        if not live:
+            return
+        order = list(live)
+        pending, held = launch(order, None)
+        while True:
+            # the step after the one in flight, for the sequences that its token cannot end by count
+            ahead = [i for i in order if i in slots and len(generated[i]) + 2 <= params.max_tokens
+                     and eng.cache.length(slots[i]) < eng.spec.max_positions]
+            following = None
+            if ahead:
+                rows = [order.index(i) for i in ahead]
+                following = launch(ahead, chooser.rows_of(pending, rows))
+            take(order, chooser.read(pending), held)
+            if not live or following is None:
+                break
+            order, (pending, held) = ahead, following
+
     def _run_batch(self, members, prompts, params, chooser, results, on_token, interrupt=None):
         eng = self.engine
         eos = eng.spec.eos_token_id
@@ -176,27 +213,39 @@ class Generator:
             self.stats.prefill_seconds += time.perf_counter() - t0
             self.stats.prompt_tokens += sum(len(prompts[i]) for i in live)
             t0 = time.perf_counter()
-            while True:
-                for i, tok in zip(list(live), tokens):
+
+            def take(order, tokens, held=None):
+                """The newest tokens of the sequences `order` (those that have ended since are
+                skipped). `held`: the positions each sequence held when the step that chose these
+                tokens had been put on the stream, if a later step has been since."""
+                for i, tok in zip(order, tokens):
+                    if i not in slots:
+                        continue
                     generated[i].append(int(tok))
                     self.stats.generated_tokens += 1
                     said = on_token(i, int(tok)) if on_token is not None else None
                     reason = stop_reason(generated[i], params, eos)
                     if reason is None and isinstance(said, str):
                         reason = said
-                    if reason is None and eng.cache.length(slots[i]) >= eng.spec.max_positions:
+                    length = eng.cache.length(slots[i]) if held is None else held[i]
+                    if reason is None and length >= eng.spec.max_positions:
                         reason = LENGTH
                     if reason is not None:
                         finish(i, reason)
                 if live and interrupt is not None and interrupt():
                     for i in list(live):
                         finish(i, INTERRUPTED)
-                if not live:
-                    break
-                entries = [StepEntry(slots[i], [generated[i][-1]], [0]) for i in live]
-                logits = eng.step(entries)
-                tokens = chooser.choose(logits, list(live))
-                self.stats.decode_steps += 1
+
+            take(list(live), tokens)
+            if self.run_ahead and getattr(chooser, "can_run_ahead", False) and \
+                    getattr(eng, "accepts_device_tokens", False):
+                self._decode_ahead(live, slots, generated, params, chooser, take)
+            else:
+                while live:
+                    order = list(live)
+                    logits = eng.step([StepEntry(slots[i], [generated[i][-1]], [0]) for i in order])
+                    self.stats.decode_steps += 1
+                    take(order, chooser.choose(logits, order))
             self.stats.decode_seconds += time.perf_counter() - t0
         finally:
             for i in list(slots):

@@ -207,14 +207,31 @@ def fill_u32(t, value):
     lib.call("elementwise", "hb_fill_u32", t.data_ptr(), int(value), nbytes // 4, _stream())
 
 
-def argmax(logits, out):
-    """out[r] = first index of the largest value of logits[r]; logits f32 [R, V], out int32 [R]."""
+ARGMAX_MAX_CHUNKS = 64
+
+
+def argmax_scratch(rows, device):
+    """The partial results of the first of argmax's two stages for up to `rows` rows, to be kept
+    and handed to `argmax` again and again."""
+    return (torch.empty((rows, ARGMAX_MAX_CHUNKS), dtype=torch.float32, device=device),
+            torch.empty((rows, ARGMAX_MAX_CHUNKS), dtype=torch.int32, device=device))
+
+
+def argmax(logits, out, scratch=None):
+    """out[r] = first index of the largest value of logits[r]; logits f32 [R, V], out int32 [R].
+    `scratch` as `argmax_scratch` makes it (for at least R rows), else it is allocated here."""
     _check(logits, "logits", torch.float32, (None, None))
     R, V = logits.shape
     _check(out, "out", torch.int32, (R,))
-    chunks = max(1, min(64, V // 8192, 1024 // R if R <= 1024 else 1))
+    chunks = max(1, min(ARGMAX_MAX_CHUNKS, V // 8192, 1024 // R if R <= 1024 else 1))
     sv = si = None
-    if chunks > 1:
+    if chunks > 1 and scratch is not None:
+        sv, si = scratch
+        _check(sv, "argmax scratch values", torch.float32, (None, ARGMAX_MAX_CHUNKS))
+        _check(si, "argmax scratch indices", torch.int32, tuple(sv.shape))
+        if sv.shape[0] < R:
+            raise BackendError("argmax: the scratch has fewer rows than the logits")
+    elif chunks > 1:
         sv = torch.empty((R, chunks), dtype=torch.float32, device=logits.device)
         si = torch.empty((R, chunks), dtype=torch.int32, device=logits.device)
     lib.call("sampling", "hb_argmax", logits.data_ptr(), V, R, V, out.data_ptr(), _ptr(sv), _ptr(si),

@@ -17,6 +17,14 @@ def _signed64(v):
     return v - (1 << 64) if v >= (1 << 63) else v
 
 
+class PendingTokens:
+    """Tokens that have been chosen on the GPU and are on their way to the host: `device` (int32
+    [rows]) can feed the next step at once, `Sampler.read` waits for the copy and gives the list."""
+
+    def __init__(self, device, host, event):
+        self.device, self.host, self.event = device, host, event
+
+
 class Sampler:
     """One generator stream per sequence, kept on the GPU and advanced by the kernel."""
 
@@ -32,6 +40,10 @@ class Sampler:
         self._sifted = None
         self._nucleus = None
         self._sums = None
+        self._argmax_scratch = None
+        self._host_ring = []            # pinned buffers that tokens on their way to the host land in
+        self._host_next = 0
+        self._index = None
         # a cap on think blocks: one counter a sequence, fed with every token chosen for it
         self.think = None
         if params.think_budget > 0:
@@ -77,27 +89,90 @@ class Sampler:
             self.think[s].track(t)
         return tokens
 
-    def _choose(self, logits, sequence_indices):
+    def _needs_host(self, vocab):
+        """True where the choice of a token takes a decision of the host in between: a think
+        budget (the forced token depends on the one before), top-p without top-k (rows that the
+        quick kernel leaves go the general way)."""
+        p = self.params
+        return self.think is not None or (not p.greedy and not 0 < p.top_k < vocab and p.top_p < 1.0
+                                          and vocab > ops.NUCLEUS_CANDIDATES)
+
+    @property
+    def can_run_ahead(self):
+        """Whether `choose_ahead` may be used: the tokens then stay on the GPU, where the next
+        step can take them from, and the host reads them later."""
+        return not self._needs_host(self.vocab_size)
+
+    def choose_ahead(self, logits, sequence_indices):
+        """Like `choose`, without waiting: the kernels are put on the stream, the tokens are copied
+        to the host behind them, and a PendingTokens is returned at once."""
+        if self._needs_host(logits.shape[1]):
+            raise RuntimeError("these sampling parameters need the host between two choices")
+        out = self._on_device(logits, sequence_indices)
+        rows = out.shape[0]
+        ring = self._host_ring
+        if not ring or ring[0].shape[0] < rows:
+            ring[:] = [torch.empty(max(rows, 64), dtype=torch.int32, pin_memory=True) for _ in range(4)]
+        host = ring[self._host_next % len(ring)][:rows]
+        self._host_next += 1
+        host.copy_(out, non_blocking=True)
+        event = torch.cuda.Event()
+        event.record()
+        return PendingTokens(out, host, event)
+
+    @staticmethod
+    def read(pending):
+        """The tokens of a `choose_ahead`, once they have arrived."""
+        pending.event.synchronize()
+        return pending.host.tolist()
+
+    @staticmethod
+    def rows_of(pending, rows):
+        """The device tokens of some rows of a `choose_ahead`, in the given order."""
+        if list(rows) == list(range(pending.device.shape[0])):
+            return pending.device
+        return pending.device[torch.tensor(list(rows), dtype=torch.long, device=pending.device.device)]
+
+    def _index_of(self, sequence_indices):
+        """The rows' sequences as a tensor on the GPU; the one of the step before is kept, since a
+        batch keeps its sequences for many steps (and a copy from the host would wait for the GPU)."""
+        key = tuple(sequence_indices)
+        if self._index is None or self._index[0] != key:
+            self._index = (key, torch.tensor(key, dtype=torch.int32, device=self.device))
+        return self._index[1]
+
+    def _on_device(self, logits, sequence_indices):
+        """The choice for every row as an int32 tensor on the GPU; only where no decision of the
+        host is needed in between."""
         rows = logits.shape[0]
         out = torch.empty(rows, dtype=torch.int32, device=self.device)
-        if self.params.greedy:
-            ops.argmax(logits, out)
-        else:
+        p = self.params
+        if p.greedy:
+            if self._argmax_scratch is None or self._argmax_scratch[0].shape[0] < rows:
+                self._argmax_scratch = ops.argmax_scratch(rows, self.device)
+            ops.argmax(logits, out, self._argmax_scratch)
+            return out
+        index = self._index_of(sequence_indices)
+        vocab = logits.shape[1]
+        if not 0 < p.top_k < vocab and p.top_p >= 1.0 and vocab > ops.SAMPLE_CHUNK:
+            # the whole row, no cut: nothing is sorted, the chunks of a long row are added up side by side
+            need = rows * (-(-vocab // ops.SAMPLE_CHUNK)) * 2
+            if self._sums is None or self._sums.numel() < need:
+                self._sums = torch.empty(need, dtype=torch.float32, device=self.device)
+            ops.sample_all(logits, p.temperature, self.states, index, out, self._sums)
+            return out
+        ops.sample(logits, p.temperature, p.top_k, p.top_p,
+                   self.states, index, out, self._scratch_for(rows), self._sifted_for(rows))
+        return out
+
+    def _choose(self, logits, sequence_indices):
+        p = self.params
+        vocab = logits.shape[1]
+        if not p.greedy and not 0 < p.top_k < vocab and p.top_p < 1.0 and vocab > ops.NUCLEUS_CANDIDATES:
             index = torch.tensor(list(sequence_indices), dtype=torch.int32, device=self.device)
-            p = self.params
-            vocab = logits.shape[1]
-            if not 0 < p.top_k < vocab and p.top_p < 1.0 and vocab > ops.NUCLEUS_CANDIDATES:
-                return self._top_p_only(logits, index, out)
-            if not 0 < p.top_k < vocab and p.top_p >= 1.0 and vocab > ops.SAMPLE_CHUNK:
-                # the whole row, no cut: nothing is sorted, the chunks of a long row are added up side by side
-                need = rows * (-(-vocab // ops.SAMPLE_CHUNK)) * 2
-                if self._sums is None or self._sums.numel() < need:
-                    self._sums = torch.empty(need, dtype=torch.float32, device=self.device)
-                ops.sample_all(logits, p.temperature, self.states, index, out, self._sums)
-                return out.tolist()
-            ops.sample(logits, p.temperature, p.top_k, p.top_p,
-                       self.states, index, out, self._scratch_for(rows), self._sifted_for(rows))
-        return out.tolist()
+            out = torch.empty(logits.shape[0], dtype=torch.int32, device=self.device)
+            return self._top_p_only(logits, index, out)
+        return self._on_device(logits, sequence_indices).tolist()
 
     def _top_p_only(self, logits, index, out):
         """Top-p without top-k: first among each row's 1024 largest logits, where the prefix that

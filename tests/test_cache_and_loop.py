@@ -428,3 +428,68 @@ def test_think_budget_follows_the_plain_rule():
                 history.append(tok)
     with pytest.raises(RequestError, match="think_tokens"):
         SamplingParams(think_budget=3).validate()
+
+
+class AheadEngine(FakeEngine):
+    """A stand-in engine that takes a step's tokens from "the device" (here: an array)."""
+    accepts_device_tokens = True
+
+    def step(self, entries, tokens_on_device=None):
+        if tokens_on_device is not None:
+            assert len(tokens_on_device) == len(entries) and all(e.tokens == [0] for e in entries)
+            entries = [type(e)(e.slot, [int(t)], e.want) for e, t in zip(entries, tokens_on_device)]
+        return super().step(entries)
+
+
+class AheadChooser(ArgmaxChooser):
+    can_run_ahead = True
+    unread = 0
+
+    def choose_ahead(self, logits, sequence_indices):
+        type(self).unread += 1
+        assert type(self).unread <= 2               # the host is never more than one step behind
+        return np.array(self.choose(logits, sequence_indices))
+
+    def read(self, pending):
+        type(self).unread -= 1
+        return pending.tolist()
+
+    def rows_of(self, pending, rows):
+        return pending[list(rows)]
+
+
+@pytest.mark.parametrize("kw", [dict(max_tokens=6, stop_ids=(23,)), dict(max_tokens=1), dict(max_tokens=2),
+                                dict(max_tokens=40, ignore_eos=True), dict(max_tokens=3, ignore_eos=True)])
+def test_decoding_one_step_ahead_of_the_host_gives_the_same(kw):
+    """With an engine that takes tokens from the device and a chooser that leaves them there, the
+    loop puts every decode step on the stream before it has read the tokens of the one before.
+    Same tokens and stop reasons as step by step; a sequence that ends on a token's value has
+    been through one step more (thrown away), one that ends by count or at the model's last
+    position has not; every slot comes back."""
+    prompts = [[5], [20, 21], [7, 8], [30, 31, 32]]
+    params = SamplingParams(temperature=0.0, repeat_check=False, **kw)
+    eng0 = FakeEngine()
+    want = Generator(eng0, max_batch=4, make_chooser=ArgmaxChooser).generate(prompts, params)
+    eng = AheadEngine()
+    AheadChooser.unread = 0
+    gen = Generator(eng, max_batch=4, make_chooser=AheadChooser)
+    got = gen.generate(prompts, params)
+    assert [(r.tokens, r.stop_reason) for r in got] == [(r.tokens, r.stop_reason) for r in want]
+    assert eng.cache.slots.held_count == 0 and AheadChooser.unread == 0
+    # what ran ahead for nothing: at most one step for every sequence that ended on a token's value
+    by_value = sum(r.stop_reason in (EOS, STOP_TOKEN) for r in got)
+    fed0 = sum(n for step in eng0.steps for _, n in step)
+    fed = sum(n for step in eng.steps for _, n in step)
+    assert fed0 <= fed <= fed0 + by_value
+    if kw.get("ignore_eos"):
+        assert fed == fed0                   # ends by count or position only: nothing is thrown away
+    # the caller's word and the interrupt flag work one step behind as well
+    eng = AheadEngine()
+    AheadChooser.unread = 0
+    res = Generator(eng, max_batch=4, make_chooser=AheadChooser).generate(
+        prompts, SamplingParams(temperature=0.0, max_tokens=30, ignore_eos=True, repeat_check=False),
+        on_token=lambda i, tok: "enough" if (i == 1 and tok == 25) else None,
+        interrupt=lambda: len(eng.steps) >= 8)
+    assert res[1].tokens == [22, 23, 24, 25] and res[1].stop_reason == "enough"
+    assert all(r.stop_reason == INTERRUPTED for j, r in enumerate(res) if j != 1)
+    assert eng.cache.slots.held_count == 0

@@ -318,6 +318,50 @@ def test_generation_stops_on_eos_and_other_sequences_go_on(model_root):
     assert engine.cache.slots.held_count == 0
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decoding_ahead_of_the_host_gives_what_step_by_step_gives(model_root, dtype):
+    """The generation loop puts every decode step on the stream before it has read the tokens of
+    the one before (they go from the sampler to the next step on the GPU). Same tokens and stop
+    reasons as with the host in between, greedy and sampled, with sequences that end on a token's
+    value in the middle of a batch (so that a step has run ahead for them and the batch shrinks),
+    through pages' edges; in float32 the greedy tokens are the plain implementation's."""
+    from herbert_rs_amd.engine.generate import Generator
+    from herbert_rs_amd.sampling import SamplingParams
+    folder = make_folder(model_root, "C", dtype)
+    cfg, w = plain_folder(folder)
+    prompts = [random_tokens(320, n, 80 + n) for n in (60, 9, 130, 3)]
+    engine = hb.load(folder, dtype=dtype, cache_tokens=64 * 12)
+    free = Generator(engine, run_ahead=False).generate(
+        prompts, SamplingParams(temperature=0.0, max_tokens=24, ignore_eos=True, repeat_check=False))
+    if dtype == "float32":
+        assert [r.tokens for r in free] == [plain.greedy(cfg, w, p, 24) for p in prompts]
+    stop = free[1].tokens[7]                          # request 1 ends at its 8th token, if not before
+    for params in (SamplingParams(temperature=0.0, max_tokens=24, ignore_eos=True, repeat_check=False, stop_ids=(stop,)),
+                   SamplingParams(temperature=0.9, top_k=12, top_p=0.95, seed=4, max_tokens=30, repeat_check=False),
+                   SamplingParams(temperature=1.1, top_k=0, top_p=1.0, seed=9, max_tokens=17, repeat_check=False)):
+        a = Generator(engine, run_ahead=False)
+        b = Generator(engine, run_ahead=True)
+        want = a.generate(prompts, params)
+        got = b.generate(prompts, params)
+        assert [(r.tokens, r.stop_reason) for r in got] == [(r.tokens, r.stop_reason) for r in want]
+        assert b.stats.decode_steps >= a.stats.decode_steps
+        engine.cache.check()
+        assert engine.cache.slots.held_count == 0
+    # the step function itself: tokens from the device give the logits that tokens from the host give
+    s1, s2 = engine.alloc_slot(), engine.alloc_slot()
+    engine.step([StepEntry(s1, prompts[0], []), StepEntry(s2, prompts[1], [])])
+    host = engine.step([StepEntry(s1, [17], [0]), StepEntry(s2, [200], [0])]).clone()
+    engine.truncate(s1, len(prompts[0]))
+    engine.truncate(s2, len(prompts[1]))
+    dev = torch.tensor([17, 200], dtype=torch.int32, device="cuda")
+    fed = engine.step([StepEntry(s1, [0], [0]), StepEntry(s2, [0], [0])], tokens_on_device=dev)
+    assert torch.equal(fed, host)
+    with pytest.raises(RequestError, match="tokens_on_device"):
+        engine.step([StepEntry(s1, [1, 2], [0])], tokens_on_device=dev[:1])
+    engine.free_slot(s1)
+    engine.free_slot(s2)
+
+
 def test_get_tensor_gives_the_weights_as_stored(model_root):
     from safetensors.torch import load_file
     from herbert_rs_amd.errors import ModelLoadError
