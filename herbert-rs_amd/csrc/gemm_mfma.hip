@@ -1192,6 +1192,27 @@ static int launch_tile64(const void* X, const void* W, void* C, int M, int N, in
 #undef EXTRA
 }
 
+// Tiles whose width is no power of two (192 = three pieces of 32 a wave): for the SwiGLU epilogue
+// only, whose bfloat16 output goes to memory lane by lane (the float32 epilogues' way through LDS
+// counts on rows of a power of two of 16-byte chunks).
+template <int TNB, int TMB, int WNW, int WMW, int WST, int XST>
+static int launch_tile64_swiglu(const void* X, const void* W, void* C, int M, int N, int K, int ldc, int epi,
+                                int packed, hipStream_t stream, int slices) {
+    constexpr int BN = 16 * TNB * WNW, BM = 16 * TMB * WMW;
+    HB_REQUIRE(epi == EPI_SWIGLU && slices == 1, "gemm_mfma: this tile takes the SwiGLU product whole only");
+    HB_REQUIRE(K % 64 == 0, "gemm_mfma: K=%d is no multiple of 64", K);
+    const int m_tiles = (M + BM - 1) / BM, n_tiles = (N + BN - 1) / BN;
+    const long total = (long)m_tiles * n_tiles;
+    const size_t lds = (size_t)(WST * BN + XST * BM) * 64 * sizeof(bf16) + WNW * WMW * 16 * sizeof(float);
+    const bf16* x = (const bf16*)X;
+    const bf16* w = (const bf16*)W;
+    if (packed)
+        return launch_tiles(gemm_tile_kernel<EPI_SWIGLU, true, TNB, TMB, WNW, WMW, WST, XST>, lds, 64 * WNW * WMW, total, 1,
+                            x, w, C, M, N, K, ldc, m_tiles, n_tiles, stream, (float*)nullptr, QkvEpilogue{}, RowScale{});
+    return launch_tiles(gemm_tile_kernel<EPI_SWIGLU, false, TNB, TMB, WNW, WMW, WST, XST>, lds, 64 * WNW * WMW, total, 1,
+                        x, w, C, M, N, K, ldc, m_tiles, n_tiles, stream, (float*)nullptr, QkvEpilogue{}, RowScale{});
+}
+
 template <int TNB, int TMB, int WNW, int WMW, int STAGES>
 static int launch_tile32(const void* X, const void* W, void* C, int M, int N, int K, int ldc, int epi, int packed,
                          hipStream_t stream) {
@@ -1323,13 +1344,17 @@ static GemmPlan plan_gemm(int M, int N, int K, int ldc, int epi, bool norm_w, bo
         // the best candidate on average, 12 % at worst), checked on three other sizes (2 %, 13 %) and
         // on 1280 to 4096 rows (under 1 %, 7 %).
         struct Mid { int id, bn, bm, per_cu; double step_us; };
+        // (168: three quarters of the 256 x 256 tile's arithmetic a step, for the SwiGLU product whole:
+        // where that one's tiles fill the last round of 256 badly, 192 columns often fill it)
         static const Mid mid[] = {{188, 256, 256, 1, 1.26}, {142, 256, 128, 1, 0.77}, {122, 128, 128, 2, 0.95},
-                                  {124, 128, 64, 2, 0.48}, {184, 256, 64, 1, 0.67}};
+                                  {124, 128, 64, 2, 0.48}, {184, 256, 64, 1, 0.67}, {168, 192, 256, 1, 1.0}};
         const int steps = K / 64;
         double best = -1;
         for (const Mid& v : mid) {
+            if (v.id == 168 && epi != EPI_SWIGLU) continue;
             const long tiles = (long)((M + v.bm - 1) / v.bm) * ((N + v.bn - 1) / v.bn);
             for (int sl = 1; sl <= 16; sl *= 2) {
+                if (v.id == 168 && sl > 1) break;
                 if (sl > 1 && !slices_fit(steps, sl)) break;
                 if (emit_g && (sl == 1 || !reducer_norms)) continue;      // the kernel that adds the slices up norms
                 if (deferred && sl > 8) break;                            // whoever adds the slices up takes 2, 4 or 8
@@ -1433,6 +1458,7 @@ extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N,
         case 124: rc = launch_tile64<2, 4, 4, 1, 3, 2>(X, W, C, M, N, K, ldc, epi, packed, stream, slices, workspace); break;   // 128 (n) x 64 (m)
         case 112: rc = launch_tile64<2, 2, 4, 1, 3, 2>(X, W, C, M, N, K, ldc, epi, packed, stream, slices, workspace, row_scale); break;   // 128 (n) x 32 (m)
         case 184: rc = launch_tile64<4, 4, 4, 1, 3, 2>(X, W, C, M, N, K, ldc, epi, packed, stream, slices, workspace); break;   // 256 (n) x 64 (m)
+        case 168: rc = launch_tile64_swiglu<6, 8, 2, 2, 2, 2>(X, W, C, M, N, K, ldc, epi, packed, stream, slices); break;   // 192 (n) x 256 (m)
         case 123:                                                                                                           // 128 x 128, K in steps of 32
             HB_REQUIRE(slices == 1, "gemm_mfma: this tile does not cut K");
             return launch_tile32<4, 4, 2, 2, 4>(X, W, C, M, N, K, ldc, epi, packed, stream);

@@ -7,7 +7,8 @@ import pytest
 from herbert_rs_amd.kernels import lib
 
 EPI_STORE, EPI_ADD, EPI_SWIGLU = 0, 1, 2
-TILES = {112: (128, 32), 124: (128, 64), 184: (256, 64), 122: (128, 128), 142: (256, 128), 188: (256, 256), 123: (128, 128)}
+TILES = {112: (128, 32), 124: (128, 64), 184: (256, 64), 122: (128, 128), 142: (256, 128), 188: (256, 256), 123: (128, 128),
+         168: (192, 256)}
 
 
 @pytest.fixture(scope="module")
@@ -35,6 +36,7 @@ def test_every_plan_is_a_kernel_that_takes_the_product(plan):
                 continue
             tile, slices = p % 1000, max(1, p // 1000)
             assert tile in TILES and (tile != 112 or M <= 32), (M, N, K, p)
+            assert tile != 168 or (epi == EPI_SWIGLU and slices == 1), (M, N, K, p)
             steps = K // 64
             if slices > 1:
                 per = -(-steps // slices)

@@ -141,6 +141,30 @@ def test_gemm_mfma_swiglu(M, I, K):
     assert float((err - 2 ** -8 * want.abs()).max()) <= 1e-3 * float(want.abs().max()) + 1e-5
 
 
+@pytest.mark.parametrize("M,I,K", [(300, 256, 128), (257, 1040, 1024), (512, 96, 64), (70, 304, 256), (1024, 1536, 512)])
+def test_gemm_mfma_swiglu_tile_192_wide(M, I, K):
+    """The SwiGLU product on tiles of 192 columns (three pieces of 32 a wave), by name: sizes
+    that end inside a tile in both directions, weights as stored and packed; rows past the end
+    are not written."""
+    from herbert_rs_amd.kernels import mfma
+    a = rand(M, K, seed=20, dtype=torch.bfloat16, scale=0.5)
+    gate = rand(I, K, seed=21, dtype=torch.bfloat16, scale=0.3)
+    up = rand(I, K, seed=22, dtype=torch.bfloat16, scale=0.3)
+    w = mfma.interleave_gate_up(gate, up)
+    g = a.double() @ gate.double().T
+    u = a.double() @ up.double().T
+    want = (g / (1 + torch.exp(-g)) * u).float()
+    for packed in (False, True):
+        out = torch.full((M + 1, I), 3.0, dtype=torch.bfloat16, device=dev())
+        mfma.gemm_swiglu(a, mfma.pack_weight(w) if packed else w, out[:M], packed, tile=168)
+        err = (out[:M].float() - want).abs()
+        assert float((err - 2 ** -8 * want.abs()).max()) <= 1e-3 * float(want.abs().max()) + 1e-5
+        assert float((out[M].float() - 3.0).abs().max()) == 0.0
+    c = torch.zeros(M, 2 * I, device=dev())
+    with pytest.raises(Exception, match="SwiGLU product whole only"):
+        mfma.gemm(a, w, c, tile=168)
+
+
 def test_gemm_mfma_refuses_what_it_cannot_do():
     from herbert_rs_amd.kernels import mfma
     a = rand(4, 40, dtype=torch.bfloat16)
