@@ -1231,28 +1231,41 @@ static int launch_tile32(const void* X, const void* W, void* C, int M, int N, in
 #undef TILE_DISPATCH
 
 // The q/k/v projection of a step with many rows, fused with norm, rotation and cache write
-// (see QkvEpilogue). X [M, K] bf16; W [(nq + 2 nkv) 128, K] bf16, rows q | k | v; 256 x 256 tiles.
+// (see QkvEpilogue). X [M, K] bf16; W [(nq + 2 nkv) 128, K] bf16, rows q | k | v. A wave's tile is
+// one head wide; shape: 0 = tiles of 256 x 256 (waves 2 x 2, for long prompts), 1 = a head wide and 256
+// rows high (four waves one above the other, 64 rows each), 2 = a head wide and 128 rows high (32
+// rows a wave): more and smaller tiles for prompts whose 256 x 256 tiles would not fill the CUs.
+template <int TNB, int TMB, int WNW, int WMW, int WST, int XST>
+static int launch_qkv(const bf16* x, const bf16* w, int M, int N, int K, int packed, const QkvEpilogue& e,
+                      hipStream_t stream) {
+    constexpr int BN = 16 * TNB * WNW, BM = 16 * TMB * WMW;
+    const int m_tiles = (M + BM - 1) / BM, n_tiles = (N + BN - 1) / BN;
+    const long total = (long)m_tiles * n_tiles;
+    const size_t lds = (size_t)(WST * BN + XST * BM) * 64 * sizeof(bf16) + WNW * WMW * 16 * sizeof(float);
+    if (packed)
+        return launch_tiles(gemm_tile_kernel<EPI_QKV, true, TNB, TMB, WNW, WMW, WST, XST>, lds, 64 * WNW * WMW, total, 1, x,
+                            w, nullptr, M, N, K, N, m_tiles, n_tiles, stream, (float*)nullptr, e, RowScale{});
+    return launch_tiles(gemm_tile_kernel<EPI_QKV, false, TNB, TMB, WNW, WMW, WST, XST>, lds, 64 * WNW * WMW, total, 1, x, w,
+                        nullptr, M, N, K, N, m_tiles, n_tiles, stream, (float*)nullptr, e, RowScale{});
+}
+
 extern "C" int hb_gemm_qkv_mfma(const void* X, const void* W, int M, int K, int packed, void* q_out, void* k_cache,
                                 void* v_cache, const int* positions, const int* seq_of, const int* slots,
                                 const int* page_table, int max_pages, int page_size, const float* q_norm_w,
                                 const float* k_norm_w, const float* cos_t, const float* sin_t, float eps, int nq,
-                                int nkv, int hd, hipStream_t stream) {
+                                int nkv, int hd, int shape, hipStream_t stream) {
     HB_REQUIRE(hd == 128 && page_size == 64, "gemm_qkv: heads of 128 and pages of 64 tokens only");
     HB_REQUIRE(M > 0 && nq > 0 && nkv > 0 && K > 0 && K % 64 == 0, "gemm_qkv: bad sizes (M=%d, K=%d)", M, K);
     HB_REQUIRE((cos_t == nullptr) == (sin_t == nullptr), "gemm_qkv: cos and sin tables come together");
+    HB_REQUIRE(shape >= 0 && shape <= 2, "gemm_qkv: unknown tile shape %d", shape);
     const int N = (nq + 2 * nkv) * 128;
     const QkvEpilogue e = {(bf16*)q_out, (bf16*)k_cache, (bf16*)v_cache, positions, seq_of, slots, page_table,
                            max_pages, q_norm_w, k_norm_w, cos_t, sin_t, eps, nq, nkv};
-    const int m_tiles = (M + 255) / 256, n_tiles = (N + 255) / 256;
-    const long total = (long)m_tiles * n_tiles;
-    const size_t lds = (size_t)(2 * 256 + 2 * 256) * 64 * sizeof(bf16);
     const bf16* x = (const bf16*)X;
     const bf16* w = (const bf16*)W;
-    if (packed)
-        return launch_tiles(gemm_tile_kernel<EPI_QKV, true, 8, 8, 2, 2, 2, 2>, lds, 256, total, 1, x, w, nullptr, M, N, K,
-                            N, m_tiles, n_tiles, stream, (float*)nullptr, e, RowScale{});
-    return launch_tiles(gemm_tile_kernel<EPI_QKV, false, 8, 8, 2, 2, 2, 2>, lds, 256, total, 1, x, w, nullptr, M, N, K, N,
-                        m_tiles, n_tiles, stream, (float*)nullptr, e, RowScale{});
+    if (shape == 0) return launch_qkv<8, 8, 2, 2, 2, 2>(x, w, M, N, K, packed, e, stream);
+    if (shape == 1) return launch_qkv<8, 4, 1, 4, 3, 2>(x, w, M, N, K, packed, e, stream);
+    return launch_qkv<8, 2, 1, 4, 3, 2>(x, w, M, N, K, packed, e, stream);
 }
 
 // Which kernel a product runs on: tile 0 = the few-row kernel, otherwise a tile variant by number and

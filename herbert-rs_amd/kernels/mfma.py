@@ -21,7 +21,7 @@ lib.register_signatures("gemm_mfma", {
                      _F, _P, _P],
     "hb_gemm_mfma_plan": [_I, _I, _I, _I, _I, _I, _I, ctypes.c_size_t, _I],
     "hb_gemm_mfma_plan_cost": [_I, _I, _I, _I, _I, _I, _I, ctypes.c_size_t, _I],
-    "hb_gemm_qkv_mfma": [_P, _P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _F, _I, _I, _I, _P],
+    "hb_gemm_qkv_mfma": [_P, _P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _F, _I, _I, _I, _I, _P],
 })
 
 EPI_STORE, EPI_ADD, EPI_SWIGLU = 0, 1, 2
@@ -237,20 +237,37 @@ def gemm(a, w, out, accumulate=False, packed=False, norm=None, tile=0, leave=Non
 QKV_FUSE_MIN_TILES = 136   # of 256 x 256; with fewer (measured: 120 lose, 144 win) the plain product's smaller tiles or K slices fill the CUs better
 
 
+def qkv_tile_shape(M, N):
+    """The tiles on which a q/k/v projection of M rows and N = heads x 128 columns norms, rotates and
+    writes the cache itself, or None where it should not (too few tiles to fill the CUs: the plain
+    product's smaller tiles and K slices then do better, and a kernel of its own does the rest).
+    0: 256 x 256; 1: a head wide, 256 rows high; 2: a head wide, 128 rows high."""
+    if -(-M // 256) * -(-N // 256) >= QKV_FUSE_MIN_TILES:
+        return 0
+    heads = N // 128
+    for shape, rows in ((1, 256), (2, 128)):
+        if QKV_FUSE_MIN_TILES <= -(-M // rows) * heads <= 256:
+            return shape
+    return None
+
+
 def gemm_qkv_fusable(a, w, meta, kv, nq, nkv, hd, rot_dims):
     """True if the q/k/v projection of this step should norm, rotate and write the cache itself:
-    a long bfloat16 prompt step, heads of 128 rotated whole or not at all, pages of 64 tokens."""
+    a long enough bfloat16 prompt step, heads of 128 rotated whole or not at all, pages of 64 tokens."""
     return (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and kv.k.dtype == torch.bfloat16
-            and -(-a.shape[0] // 256) * -(-w.shape[0] // 256) >= QKV_FUSE_MIN_TILES
             and a.shape[1] % 64 == 0 and hd == 128 and kv.page_size == 64
-            and rot_dims in (0, hd) and w.shape[0] == (nq + 2 * nkv) * hd and meta.num_tokens == a.shape[0])
+            and rot_dims in (0, hd) and w.shape[0] == (nq + 2 * nkv) * hd and meta.num_tokens == a.shape[0]
+            and qkv_tile_shape(a.shape[0], w.shape[0]) is not None)
 
 
-def gemm_qkv(a, w, packed, q_norm_w, k_norm_w, cos, sin, meta, kv, q_out, nq, nkv, hd, eps):
+def gemm_qkv(a, w, packed, q_norm_w, k_norm_w, cos, sin, meta, kv, q_out, nq, nkv, hd, eps, shape=None):
     """q_out bf16 [M, nq hd] and the pages of kv from a bf16 [M, K] @ w[(nq + 2 nkv) hd, K]^T: the
     product, the per-head norm (if weights are given), the rotation (if tables are given) and the
-    cache write in one kernel."""
+    cache write in one kernel. `shape`: the tiles (see qkv_tile_shape), by default what that picks
+    or, where it picks none, the large ones."""
     M, K = a.shape
+    if shape is None:
+        shape = qkv_tile_shape(M, (nq + 2 * nkv) * hd) or 0
     _check(a, "a", torch.bfloat16, (M, K))
     _check(w, "w", torch.bfloat16, ((nq + 2 * nkv) * hd, K))
     _check(q_out, "q_out", torch.bfloat16, (M, nq * hd))
@@ -277,7 +294,7 @@ def gemm_qkv(a, w, packed, q_norm_w, k_norm_w, cos, sin, meta, kv, q_out, nq, nk
     lib.call("gemm_mfma", "hb_gemm_qkv_mfma", a.data_ptr(), w.data_ptr(), M, K, 1 if packed else 0, q_out.data_ptr(),
              kv.k.data_ptr(), kv.v.data_ptr(), meta.positions.data_ptr(), meta.seq_of.data_ptr(),
              meta.slots.data_ptr(), kv.page_table.data_ptr(), kv.page_table.shape[1], kv.page_size, ptr(q_norm_w),
-             ptr(k_norm_w), ptr(cos), ptr(sin), float(eps), nq, nkv, hd, _stream())
+             ptr(k_norm_w), ptr(cos), ptr(sin), float(eps), nq, nkv, hd, int(shape), _stream())
 
 
 def interleave_gate_up(gate, up):

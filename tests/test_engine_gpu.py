@@ -91,7 +91,8 @@ def test_long_prompts_with_heads_of_128(dtype, model_root, monkeypatch):
     monkeypatch.setattr(mfma, "QKV_FUSE_MIN_TILES", 16)
     fused = []
     real = mfma.gemm_qkv
-    monkeypatch.setattr(mfma, "gemm_qkv", lambda *a, **k: (fused.append(1), real(*a, **k))[1])
+    monkeypatch.setattr(mfma, "gemm_qkv", lambda *a, **k: (
+        fused.append(mfma.qkv_tile_shape(a[0].shape[0], a[1].shape[0])), real(*a, **k))[1])
     folder = make_folder(model_root, "D", dtype)
     vocab = CONFIGS["D"][0]["vocab_size"]
     a, b = random_tokens(vocab, 1100, 30), random_tokens(vocab, 45, 31)
@@ -117,8 +118,18 @@ def test_long_prompts_with_heads_of_128(dtype, model_root, monkeypatch):
     piece = engine.step([StepEntry(s3, a[70:], [1099 - 70])]).cpu().numpy()[0]
     assert close(piece, ref_a[1099], dtype, "D")[0]
     engine.free_slot(s3)
+    # shorter prompts: the projection's smaller tiles (a head wide, 256 and 128 rows high)
+    for n in (600, 250):
+        s4 = engine.alloc_slot()
+        rows = [p for p in (0, 127, 128, 255, 256) if p < n] + [n - 1]
+        got = engine.step([StepEntry(s4, a[:n], rows)]).cpu().numpy()
+        for row, p in enumerate(rows):
+            assert close(got[row], ref_a[p], dtype, "D")[0], (n, p)
+        engine.free_slot(s4)
     engine.cache.check()
     assert (len(fused) > 0) == (dtype == "bfloat16")
+    if dtype == "bfloat16":
+        assert set(fused) == {0, 1, 2}, fused           # every tile shape was taken by the host's own choice
 
 
 ODD_SIZES = {

@@ -362,9 +362,10 @@ def test_qk_norm_rope_write(nq, nkv, hd, rot, norm, dtype):
         assert float((kv.v.double().cpu() - exp_v).abs().max()) <= tol * float(exp_v.abs().max())
 
 
+@pytest.mark.parametrize("shape", [0, 1, 2])
 @pytest.mark.parametrize("packed", [True, False])
 @pytest.mark.parametrize("nq,nkv,norm,rope", [(4, 2, True, True), (3, 1, False, True), (2, 2, True, False), (1, 1, True, True)])
-def test_gemm_qkv_with_norm_rotation_and_cache_write(nq, nkv, norm, rope, packed):
+def test_gemm_qkv_with_norm_rotation_and_cache_write(nq, nkv, norm, rope, packed, shape):
     """The q/k/v projection that norms, rotates and writes the pages in its epilogue against the
     product followed by the kernel of its own: prompts that cross pages, rows that are no
     multiple of the tile, an odd number of heads (half a tile of columns is empty)."""
@@ -396,7 +397,7 @@ def test_gemm_qkv_with_norm_rotation_and_cache_write(nq, nkv, norm, rope, packed
         assert mfma.gemm_qkv_fusable(a, wp, meta, kv2, nq, nkv, hd, hd if rope else 0)
     finally:
         mfma.QKV_FUSE_MIN_TILES = old
-    mfma.gemm_qkv(a, wp, packed, qw, kw, cos, sin, meta, kv2, got_q, nq, nkv, hd, eps)
+    mfma.gemm_qkv(a, wp, packed, qw, kw, cos, sin, meta, kv2, got_q, nq, nkv, hd, eps, shape=shape)
     # the two paths add the squares and the products in other orders: an element may round the other way
     for got, want in ((got_q, want_q), (kv2.k, kv.k), (kv2.v, kv.v)):
         d = (got.float() - want.float()).abs()
