@@ -8,6 +8,7 @@ leaves the order of candidates open, it is value descending, index ascending amo
 """
 import torch
 
+from ..errors import RequestError
 from ..kernels import ops
 from . import xorshift
 from .think import ThinkBudget
@@ -107,7 +108,7 @@ class Sampler:
         """Like `choose`, without waiting: the kernels are put on the stream, the tokens are copied
         to the host behind them, and a PendingTokens is returned at once."""
         if self._needs_host(logits.shape[1]):
-            raise RuntimeError("these sampling parameters need the host between two choices")
+            raise RequestError("these sampling parameters need the host between two choices")
         out = self._on_device(logits, sequence_indices)
         rows = out.shape[0]
         ring = self._host_ring
