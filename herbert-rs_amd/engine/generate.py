@@ -12,6 +12,12 @@ the caller's interrupt flag is looked at (crates/cli/src/main.rs:1242-1245):
 when it is set, every running sequence ends with what it has and every slot
 is given back.
 
+Where engine and sampler allow it, decode steps are put on the GPU's stream
+one ahead of the host (`_decode_ahead`): a step takes its tokens from where
+the sampler left them on the GPU, and the host reads them, applies the stop
+rules and calls `on_token` while the next step already runs. The tokens and
+stop reasons are those of the step-by-step loop.
+
 `max_tokens` here counts every generated token, the one the prompt's step
 gives included: the reference's chat and server loops (`for _ in
 1..max_tokens` after the first token, crates/cli/src/chat.rs:231). Its
