@@ -371,6 +371,10 @@ def test_decoding_ahead_of_the_host_gives_what_step_by_step_gives(model_root, dt
         engine.step([StepEntry(s1, [1, 2], [0])], tokens_on_device=dev[:1])
     engine.free_slot(s1)
     engine.free_slot(s2)
+    # and without captured graphs (the step's metadata is then packed afresh every time)
+    plain_steps = hb.Engine.from_folder(folder, dtype=dtype, max_tokens=64 * 12, use_graphs=False)
+    got = Generator(plain_steps, run_ahead=True).generate(prompts, params)
+    assert [(r.tokens, r.stop_reason) for r in got] == [(r.tokens, r.stop_reason) for r in want]
 
 
 def test_get_tensor_gives_the_weights_as_stored(model_root):
