@@ -435,6 +435,8 @@ class AheadEngine(FakeEngine):
     accepts_device_tokens = True
 
     def step(self, entries, tokens_on_device=None):
+        if any(len(e.tokens) > 1 or e.want != [0] for e in entries) or self.cache.lengths[entries[0].slot] == 0:
+            AheadChooser.unread = 0          # a new batch: what ran ahead for nothing before it is forgotten
         if tokens_on_device is not None:
             assert len(tokens_on_device) == len(entries) and all(e.tokens == [0] for e in entries)
             entries = [type(e)(e.slot, [int(t)], e.want) for e, t in zip(entries, tokens_on_device)]
@@ -493,3 +495,22 @@ def test_decoding_one_step_ahead_of_the_host_gives_the_same(kw):
     assert res[1].tokens == [22, 23, 24, 25] and res[1].stop_reason == "enough"
     assert all(r.stop_reason == INTERRUPTED for j, r in enumerate(res) if j != 1)
     assert eng.cache.slots.held_count == 0
+
+
+def test_decoding_ahead_on_random_requests_gives_the_same():
+    """Random prompts, stop tokens, budgets and batch sizes: the loop that runs one step ahead of
+    the host and the step-by-step loop give the same results, and every slot comes back."""
+    rng = random.Random(11)
+    for trial in range(60):
+        n = rng.randint(1, 9)
+        prompts = [[rng.randrange(50) for _ in range(rng.randint(1, 6))] for _ in range(n)]
+        params = SamplingParams(temperature=0.0, max_tokens=rng.choice([1, 2, 3, 7, 20, 60]),
+                                stop_ids=tuple(rng.sample(range(50), rng.randint(0, 6))),
+                                ignore_eos=rng.random() < 0.3, repeat_check=rng.random() < 0.5)
+        max_batch = rng.choice([1, 2, 4, 16])
+        want = Generator(FakeEngine(), max_batch=max_batch, make_chooser=ArgmaxChooser).generate(prompts, params)
+        eng = AheadEngine()
+        AheadChooser.unread = 0
+        got = Generator(eng, max_batch=max_batch, make_chooser=AheadChooser).generate(prompts, params)
+        assert [(r.tokens, r.stop_reason) for r in got] == [(r.tokens, r.stop_reason) for r in want], trial
+        assert eng.cache.slots.held_count == 0 and AheadChooser.unread <= 1
