@@ -77,6 +77,14 @@ __global__ void rmsnorm_kernel(const float* __restrict__ x, const float* __restr
 // The same for rows that fit the registers of one block (H in steps of 4, at most 8192): every
 // element is loaded once, 16 bytes a lane, all loads in flight together.
 typedef float hb_f4 __attribute__((ext_vector_type(4)));
+// four neighbours of a row in one store (rows start at multiples of four elements)
+__device__ __forceinline__ void store_four(float* out, hb_f4 v) { *(hb_f4*)out = v; }
+__device__ __forceinline__ void store_four(bf16* out, hb_f4 v) {
+    // (two conversions a register, round to nearest even as hb_from_float)
+    typedef __bf16 hb_b2 __attribute__((ext_vector_type(2)));
+    const hb_b2 lo = {(__bf16)v[0], (__bf16)v[1]}, hi = {(__bf16)v[2], (__bf16)v[3]};
+    *(uint2*)out = uint2{__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi)};
+}
 template <class TOut>
 __global__ void __launch_bounds__(256)
 rmsnorm_row_kernel(const float* __restrict__ x, const float* __restrict__ w, TOut* __restrict__ y,
@@ -94,7 +102,7 @@ rmsnorm_row_kernel(const float* __restrict__ x, const float* __restrict__ w, TOu
             v[c] = in[i];
             g[c] = w4[i];
         } else {
-            v[c] = hb_f4{0.f, 0.f, 0.f, 0.f};
+            v[c] = g[c] = hb_f4{0.f, 0.f, 0.f, 0.f};
         }
     }
     float ss = 0.f;
@@ -107,8 +115,11 @@ rmsnorm_row_kernel(const float* __restrict__ x, const float* __restrict__ w, TOu
     for (int c = 0; c < 8; ++c) {
         const int i = threadIdx.x + 256 * c;
         if (i < nv) {
+            // (element by element: written as a product of vectors this took 380 registers)
+            hb_f4 r;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) out[4 * i + e] = hb_from_float<TOut>(v[c][e] * inv * g[c][e]);
+            for (int e = 0; e < 4; ++e) r[e] = v[c][e] * inv * g[c][e];
+            store_four(out + 4 * i, r);
         }
     }
 }
