@@ -33,6 +33,22 @@ __global__ void embed_kernel(const int* __restrict__ ids, const TW* __restrict__
             out[k] = hb_to_float(blk[(size_t)(k / 32) * plane + ((k / 8) % 4) * 128 + (k % 8)]);
     } else {
         const TW* row = table + (size_t)n * H;
+        if (sizeof(TW) == 2 && H % 8 == 0) {
+            // eight bfloat16 a load (rows of a table whose width is a multiple of 8 start at 16 bytes)
+            for (int i = threadIdx.x * 8; i < H; i += blockDim.x * 8) {
+                const uint4 raw = *(const uint4*)(row + i);
+                const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+                float v[8];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    v[2 * e] = __uint_as_float(w[e] << 16);
+                    v[2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u);
+                }
+                *(float4*)(out + i) = float4{v[0], v[1], v[2], v[3]};
+                *(float4*)(out + i + 4) = float4{v[4], v[5], v[6], v[7]};
+            }
+            return;
+        }
         for (int i = threadIdx.x; i < H; i += blockDim.x) out[i] = hb_to_float(row[i]);
     }
 }
