@@ -26,6 +26,12 @@ __global__ void embed_kernel(const int* __restrict__ ids, const TW* __restrict__
     const int t = blockIdx.x;
     const int n = ids[t];
     float* out = x + (size_t)t * H;
+    if ((unsigned)n >= (unsigned)V) {
+        // The host checks the ids it sees; ids that come from the GPU (a sampler's output fed to the
+        // next step) cannot be: a bad one reads nothing and makes its row NaN, which shows.
+        for (int i = threadIdx.x; i < H; i += blockDim.x) out[i] = __uint_as_float(0x7fc00000u);
+        return;
+    }
     if (PACKED) {
         const TW* blk = table + (size_t)(n / 16) * 512 + (n % 16) * 8;
         const size_t plane = (size_t)(V / 16) * 512;

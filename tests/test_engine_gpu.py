@@ -369,6 +369,13 @@ def test_decoding_ahead_of_the_host_gives_what_step_by_step_gives(model_root, dt
     assert torch.equal(fed, host)
     with pytest.raises(RequestError, match="tokens_on_device"):
         engine.step([StepEntry(s1, [1, 2], [0])], tokens_on_device=dev[:1])
+    # an id from the device that the vocabulary does not hold (the host cannot check it) reads nothing:
+    # its row comes out NaN, the other sequence's row is what it would have been
+    engine.truncate(s1, len(prompts[0]))
+    engine.truncate(s2, len(prompts[1]))
+    bad = torch.tensor([17, 1 << 20], dtype=torch.int32, device="cuda")
+    fed = engine.step([StepEntry(s1, [0], [0]), StepEntry(s2, [0], [0])], tokens_on_device=bad)
+    assert torch.equal(fed[0], host[0]) and bool(torch.isnan(fed[1]).all())
     engine.free_slot(s1)
     engine.free_slot(s2)
     # and without captured graphs (the step's metadata is then packed afresh every time)
