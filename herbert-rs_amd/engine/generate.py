@@ -117,7 +117,8 @@ class Generator:
     def generate(self, prompts, params=None, on_token=None, interrupt=None):
         """One GenerationResult per prompt (a list of token ids), in the prompts' order.
         on_token(request index, token) is called for every generated token; if it returns a
-        string, the sequence ends there with that stop reason (the token is kept). `interrupt()`
+        string, the sequence ends there with that stop reason (the token is kept). It must not
+        use the engine: the step after the token's may already be on the GPU. `interrupt()`
         is asked before every decode step and before every batch: once it is true, running
         sequences end with reason "interrupted" and requests not yet started return no tokens."""
         params = params or SamplingParams()
