@@ -2,8 +2,9 @@
 
 Two layers of the Qwen3-8B shape (hidden 4096, 32 query heads on 8 kv heads of 128,
 intermediate 12288, vocabulary 151936, separate head), random bfloat16 weights, through
-bin/trace_run in bfloat16 and in float32: one prompt of 2,048 tokens (the q/k/v product that
-norms, rotates and writes the cache itself), decoding at batch 1, 8 and 64 with the kernels the
+bin/trace_run in bfloat16 and in float32: prompts of 2,048, 1,024 and 512 tokens (the q/k/v product
+that norms, rotates and writes the cache itself, on each of its three tile shapes; gate/up on tiles
+of 256 and of 192 columns), decoding at batch 1, 8 and 64 with the kernels the
 host picks for these widths by itself, and batches of unequal lengths that follow one another
 in slots that were used before. Nothing is patched: what runs here is what bench.py times.
 """
@@ -28,7 +29,10 @@ VOCAB = WIDE["vocab_size"]
 
 def wide_requests():
     """id -> (tokens, length of the prompt part, places of the prompt whose logits are wanted)."""
-    reqs = {"long": (random_tokens(VOCAB, 2048 + 6, 900), 2048, [0, 1, 63, 64, 1023, 2047])}
+    reqs = {"long": (random_tokens(VOCAB, 2048 + 6, 900), 2048, [0, 1, 63, 64, 1023, 2047]),
+            # prompts for which the host picks the tiles of 192 columns and the q/k/v tiles a head wide
+            "m512": (random_tokens(VOCAB, 512 + 2, 901), 512, [0, 127, 128, 511]),
+            "n1024": (random_tokens(VOCAB, 1024 + 2, 902), 1024, [0, 255, 256, 1023])}
     for i, n in enumerate([300, 64, 129, 17, 200, 77, 256, 1]):                 # a batch of 8
         extra = [4, 4, 4, 2, 4, 1, 4, 4][i]
         reqs[f"e{i}"] = (random_tokens(VOCAB, n + extra, 910 + i), n, sorted({0, n - 1}))
@@ -66,6 +70,8 @@ def wide_trace(reqs):
             steps.append(rec)
 
     run_batch(["long"])
+    run_batch(["m512"])
+    run_batch(["n1024"])
     run_batch([f"e{i}" for i in range(8)])
     run_batch([f"s{i}" for i in range(64)])
     run_batch([f"f{i}" for i in range(8)])
@@ -100,6 +106,10 @@ def test_the_host_picks_the_profiled_kernels_for_these_widths():
     # the prompt of 2,048 tokens: the fused q/k/v product is taken from 136 tiles of 256 x 256 on
     assert -(-2048 // 256) * -(-Q // 256) >= mfma.QKV_FUSE_MIN_TILES
     assert plan(2048, 2 * I, H, SWIGLU) == 188 and plan(2048, H, I, ADD) == 142
+    # prompts of 512 and 1,024 tokens: gate/up on tiles of 192 columns, q/k/v fused on tiles a head
+    # wide and 128 or 256 rows high; 256 tokens are too few for a fused q/k/v product
+    assert plan(512, 2 * I, H, SWIGLU) == 168 and plan(1024, 2 * I, H, SWIGLU) == 168
+    assert [mfma.qkv_tile_shape(m, Q) for m in (256, 512, 1024, 2048)] == [None, 2, 1, 0]
 
 
 @pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
@@ -118,7 +128,7 @@ def test_prompt_of_2048_and_decoding_at_batch_1_8_64(dtype, wide_folder, tmp_pat
         ref = plain_rows(wide_folder, reqs[rid][0], places)
         for pos in places:
             kind = "prompt" if pos < reqs[rid][1] else "decode"
-            group = {"l": "b1", "e": "b8", "s": "b64", "f": "b8 again"}[rid[0]]
+            group = {"l": "b1", "m": "b1", "n": "b1", "e": "b8", "s": "b64", "f": "b8 again"}[rid[0]]
             ok, err = close(got[(rid, pos)], ref[pos], dtype, "wide", f"{group} {kind}")
             assert ok, f"request {rid} position {pos} ({group} {kind}): error {err}"
     if dtype == "float32":
