@@ -10,7 +10,10 @@ ms a step, GB/s and the fraction of 8 TB/s at the full context (`decode_b1`, `de
 over a decode from 512 to the full context (`..._mean...`, from steps timed at a few contexts
 in between); and the other two workloads of the benchmark description through the generation
 loop (`qwen3_1p7b_...`, `qwen3_32b_...`). Weights are random, token ids are random, and the
-cache below the timed steps is filled by real prefill steps of random prompts.
+cache below the timed steps is filled by real prefill steps of random prompts. A timed decode
+step is what the generation loop does for a token: the step function (a HIP-graph replay), the
+greedy choice on the GPU, and the chosen tokens read by the host, which as in that loop reads
+the tokens of a step while the next step, fed from the GPU, already runs.
 """
 import argparse
 import json
