@@ -9,7 +9,8 @@ ms a step, GB/s and the fraction of 8 TB/s at the full context (`decode_b1`, `de
 `decode_b1_gbs`, `decode_b1_frac`), the same at a context of 512 (`..._ctx512...`) and the mean
 over a decode from 512 to the full context (`..._mean...`, from steps timed at a few contexts
 in between); and the other two workloads of the benchmark description through the generation
-loop (`qwen3_1p7b_...`, `qwen3_32b_...`). Weights are random, token ids are random, and the
+loop (`qwen3_1p7b_...`, `qwen3_32b_...`); `decode_b8_host_between_steps` is the headline's step
+with the host reading each step's tokens before it starts the next. Weights are random, token ids are random, and the
 cache below the timed steps is filled by real prefill steps of random prompts. A timed decode
 step is what the generation loop does for a token: the step function (a HIP-graph replay), the
 greedy choice on the GPU, and the chosen tokens read by the host, which as in that loop reads
@@ -197,7 +198,7 @@ def main():
     def step_gbs(batch, mean_context, ms):
         return (weight_bytes + batch * mean_context * kv_bytes_per_token) / (ms * 1e-3) / 1e9
 
-    def decode_run(batch, plan):
+    def decode_run(batch, plan, run_ahead=True):
         """[(context, tokens/s, ms/step)] for each (context, steps, warmup) of `plan` (contexts
         ascending): `steps` timed decode steps at `batch` after `warmup` untimed ones, ending with
         every sequence holding `context` tokens; one pass over a cache that is filled by real
@@ -212,6 +213,9 @@ def main():
         def one():
             """A decode step as the generation loop runs it: put on the stream with the tokens of the
             step before still on the GPU, whose copy the host reads while this step runs."""
+            if not run_ahead:       # the host reads a step's tokens before it starts the next
+                logits = engine.step([StepEntry(s, [t], [0]) for s, t in zip(slots, tokens)])
+                return chooser.choose(logits, range(batch))
             before = ahead[0]
             if before is None:
                 logits = engine.step([StepEntry(s, [t], [0]) for s, t in zip(slots, tokens)])
@@ -305,6 +309,12 @@ def main():
     head = measure(args.batch)
     value, ms, achieved = head[0]
     add_points(points, args.batch, head)
+    if not args.no_points:
+        # for comparison: the same step with the host between two steps (it reads a step's tokens,
+        # then starts the next), as the loop runs where a sampler's choice needs the host
+        _, v_sync, ms_sync = decode_run(args.batch, [(context, min(args.steps, 16), 3)], run_ahead=False)[0]
+        points[f"decode_b{args.batch}_host_between_steps"] = round(v_sync, 2)
+        points[f"decode_b{args.batch}_host_between_steps_ms"] = round(ms_sync, 4)
     for key in (f"decode_b{args.batch}", f"decode_b{args.batch}_ms", f"decode_b{args.batch}_gbs",
                 f"decode_b{args.batch}_frac"):
         points.pop(key)          # the headline itself: `value`, `ms_per_step`, `roofline`
