@@ -137,6 +137,35 @@ __device__ __forceinline__ float softmax_reference(f32x16 st[2], int g2, int pag
 }
 
 // ----------------------------------------------------------------- prefill
+// A read of 16 bytes from LDS that the compiler does not follow: it neither waits for it nor
+// knows that it is in flight, so the caller waits by count (lds_wait<N>: at most N reads, in the
+// order in which they were issued, may still be on their way) before the value is used. The
+// compiler's own waits drain every read in flight (lgkmcnt(0)) each time a value is needed, the
+// one issued a moment ago included; with three reads ahead of their products a wave of the
+// prompt kernels then stood still for a read's whole way through LDS eleven times a page.
+template <int BYTES_ON>
+__device__ __forceinline__ bf16x8 lds_read_ahead(const bf16* p) {
+    bf16x8 v;
+    const uint32_t at = (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) bf16*)p;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(at), "n"(BYTES_ON));
+    return v;
+}
+// (the value that is about to be used goes through the wait, so that its use cannot be moved before it)
+template <int N>
+__device__ __forceinline__ void lds_wait(bf16x8& arrived) {
+    asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(arrived) : "n"(N));
+}
+
+// f(integral_constant<int, B>), ..., f(integral_constant<int, E - 1>): a loop whose index is a
+// constant inside the body
+template <int B, int E, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (B < E) {
+        f(std::integral_constant<int, B>{});
+        static_for<B + 1, E>(f);
+    }
+}
+
 // What a lane needs to find its operands in the LDS stages of a page's keys and values.
 struct PrefillLane {
     int c32, g2, krow, k_read[2], v_swz;
@@ -168,13 +197,17 @@ __device__ __forceinline__ void prefill_step_products(const bf16* kst, const bf1
     auto pv_group = [](int n) { return n < 7 * Q ? (n - Q) / (2 * Q) : 3; };
     auto pv_block = [](int n) { return n < 7 * Q ? (n - Q) % (2 * Q) - Q : n - 7 * Q; };
     constexpr int KRPB = 128 / HD > 0 ? 128 / HD : 1;
-    auto operand = [&](int n) -> bf16x8 {
-        if (is_s(n)) {
-            const int j = s_index(n), ks = j / 2, kb = j % 2;
-            return *(const bf16x8*)(kst + (kb * 32 + krow) * HD + (((2 * ks + g2) ^ ln.k_read[kb]) * 8));
+    // (an address is a lane's own part, shared by the two key blocks of a k-step and by the output
+    // blocks of a group of probabilities, plus a constant that goes into the instruction)
+    auto operand = [&](auto n_tag) -> bf16x8 {
+        constexpr int n = decltype(n_tag)::value;
+        if constexpr (is_s(n)) {
+            constexpr int j = s_index(n), ks = j / 2, kb = j % 2;
+            return lds_read_ahead<kb * 32 * HD * 2>(kst + krow * HD + (((2 * ks + g2) ^ ln.k_read[0]) * 8));
+        } else {
+            constexpr int g = pv_group(n), d = pv_block(n), kb = g >> 1, h2 = g & 1;
+            return lds_read_ahead<d * 32 * PAGE * 2>(vst + c32 * PAGE + (((kb * 4 + h2 * 2 + g2) ^ v_swz) * 8));
         }
-        const int g = pv_group(n), d = pv_block(n), kb = g >> 1, h2 = g & 1;
-        return *(const bf16x8*)(vst + (d * 32 + c32) * PAGE + (((kb * 4 + h2 * 2 + g2) ^ v_swz) * 8));
     };
     (void)KRPB;
 #pragma unroll
@@ -190,28 +223,29 @@ __device__ __forceinline__ void prefill_step_products(const bf16* kst, const bf1
         sum += p;
         pb[g][e] = (__bf16)p;
     };
-#pragma unroll
-    for (int n = 0; n < AHEAD; ++n) ops[n] = operand(n);
-#pragma unroll
-    for (int n = 0; n < NM; ++n) {
-        if (n + AHEAD < NM) ops[n + AHEAD] = operand(n + AHEAD);
-        if (is_s(n)) {
-            const int j = s_index(n);
+    static_for<0, AHEAD>([&](auto t) { ops[decltype(t)::value] = operand(t); });
+    static_for<0, NM>([&](auto t) {
+        constexpr int n = decltype(t)::value;
+        if constexpr (n + AHEAD < NM) ops[n + AHEAD] = operand(std::integral_constant<int, n + AHEAD>{});
+        // the reads behind product n's own may still be on their way: AHEAD of them, fewer at the end
+        lds_wait<(n + AHEAD < NM ? AHEAD : NM - 1 - n)>(ops[n]);
+        if constexpr (is_s(n)) {
+            constexpr int j = s_index(n);
             nxt[j % 2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ops[n], qreg[j / 2], nxt[j % 2], 0, 0, 0);
         } else {
-            const int d = pv_block(n);
+            constexpr int d = pv_block(n);
             oacc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ops[n], pb[pv_group(n)], oacc[d], 0, 0, 0);
         }
         // the exponentials that go with this product: those of phase g are dealt out over the
         // phase's products (phase 0 has Q of them, the others 2 Q)
-        if (n < 7 * Q) {
-            const int g = n < Q ? 0 : (n - Q) / (2 * Q) + 1;
-            const int in_phase = n < Q ? n : (n - Q) % (2 * Q), of = n < Q ? Q : 2 * Q;
+        if constexpr (n < 7 * Q) {
+            constexpr int g = n < Q ? 0 : (n - Q) / (2 * Q) + 1;
+            constexpr int in_phase = n < Q ? n : (n - Q) % (2 * Q), of = n < Q ? Q : 2 * Q;
 #pragma unroll
             for (int e = in_phase * 8 / of; e < (in_phase + 1) * 8 / of; ++e) exponential(g, e);
         }
         __builtin_amdgcn_sched_barrier(0);
-    }
+    });
     l = l * corr + sum;      // this lane's keys only; the two halves are added at the end
 }
 
