@@ -1309,14 +1309,19 @@ static GemmPlan plan_gemm(int M, int N, int K, int ldc, int epi, bool norm_w, bo
         }
         if (!norm_w && K % 64 == 0) {
             struct Small { int id, bn, bm, per_cu; double step_us; };
-            static const Small small[] = {{112, 128, 32, 2, 0.5}, {124, 128, 64, 2, 0.6}, {184, 256, 64, 1, 0.9}};
+            // (164: tiles of 96 columns for the SwiGLU product of 33 to 64 rows, whole: 256 of them where
+            // tiles of 128 are 192, e.g. 24576 x 4096 at 64 rows 43 -> 40 us, 19456 x 2560 29 -> 26 us;
+            // for fewer rows the tile of 32 rows stays ahead)
+            static const Small small[] = {{112, 128, 32, 2, 0.5}, {124, 128, 64, 2, 0.6}, {184, 256, 64, 1, 0.9},
+                                          {164, 96, 64, 2, 0.585}};
             const int steps = K / 64;
             for (const Small& v : small) {
                 if (M > v.bm) continue;
                 if (scale_partial && v.id != 112) continue;            // only this one finishes a handed-on norm
+                if (v.id == 164 && (epi != EPI_SWIGLU || M <= 32)) continue;
                 const long tiles = (N + v.bn - 1) / v.bn;
                 for (int sl = 1; sl <= 16; sl *= 2) {
-                    if (sl > 1 && !slices_fit(steps, sl)) break;
+                    if (sl > 1 && (v.id == 164 || !slices_fit(steps, sl))) break;
                     // a norm is left behind by the kernel that adds the slices up
                     if (emit_g && (sl == 1 || !reducer_norms)) continue;
                     if (deferred && sl > 8) break;                 // whoever adds the slices up takes 2, 4 or 8
@@ -1326,6 +1331,7 @@ static GemmPlan plan_gemm(int M, int N, int K, int ldc, int epi, bool norm_w, bo
                     const int per = (steps + sl - 1) / sl;
                     const double waiting = (double)rounds * per * v.step_us * on_a_cu;       // bound by latency
                     double streaming = (double)wgs * per * (v.bn * 128 + v.bm * 64) / 6.0e6;   // bound by HBM
+                    if (v.id == 164) streaming /= 1.2;         // (a round of 256 workgroups streams a fifth faster than one of 192)
                     if (wgs > slots) streaming *= 1.12;
                     double cost = (waiting > streaming ? waiting : streaming) + 3.0;
                     if (sl > 1) cost += deferred ? 0.3 * sl : 2.5 + (double)(sl + 1) * M * N * 4 / 2.0e6 + (emit_g ? 1.5 : 0.0);
@@ -1472,6 +1478,7 @@ extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N,
         case 112: rc = launch_tile64<2, 2, 4, 1, 3, 2>(X, W, C, M, N, K, ldc, epi, packed, stream, slices, workspace, row_scale); break;   // 128 (n) x 32 (m)
         case 184: rc = launch_tile64<4, 4, 4, 1, 3, 2>(X, W, C, M, N, K, ldc, epi, packed, stream, slices, workspace); break;   // 256 (n) x 64 (m)
         case 168: rc = launch_tile64_swiglu<6, 8, 2, 2, 2, 2>(X, W, C, M, N, K, ldc, epi, packed, stream, slices); break;   // 192 (n) x 256 (m)
+        case 164: rc = launch_tile64_swiglu<6, 2, 1, 2, 3, 2>(X, W, C, M, N, K, ldc, epi, packed, stream, slices); break;   // 96 (n) x 64 (m), two waves one above the other
         case 123:                                                                                                           // 128 x 128, K in steps of 32
             HB_REQUIRE(slices == 1, "gemm_mfma: this tile does not cut K");
             return launch_tile32<4, 4, 2, 2, 4>(X, W, C, M, N, K, ldc, epi, packed, stream);

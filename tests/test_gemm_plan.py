@@ -8,7 +8,7 @@ from herbert_rs_amd.kernels import lib
 
 EPI_STORE, EPI_ADD, EPI_SWIGLU = 0, 1, 2
 TILES = {112: (128, 32), 124: (128, 64), 184: (256, 64), 122: (128, 128), 142: (256, 128), 188: (256, 256), 123: (128, 128),
-         168: (192, 256)}
+         168: (192, 256), 164: (96, 64)}
 
 
 @pytest.fixture(scope="module")
@@ -36,7 +36,8 @@ def test_every_plan_is_a_kernel_that_takes_the_product(plan):
                 continue
             tile, slices = p % 1000, max(1, p // 1000)
             assert tile in TILES and (tile != 112 or M <= 32), (M, N, K, p)
-            assert tile != 168 or (epi == EPI_SWIGLU and slices == 1), (M, N, K, p)
+            assert tile not in (168, 164) or (epi == EPI_SWIGLU and slices == 1), (M, N, K, p)
+            assert tile != 164 or 32 < M <= 64, (M, N, K, p)
             steps = K // 64
             if slices > 1:
                 per = -(-steps // slices)
@@ -89,4 +90,5 @@ def test_known_choices(plan):
     assert plan(8, 5120, 25600, EPI_ADD, emit=True) >= 2000            # hidden 5120: 320 workgroups would not spread
     assert plan(2048, 24576, 4096, EPI_SWIGLU) == 188
     assert plan(2048, 4096, 12288, EPI_ADD) == 142
-    assert plan(64, 24576, 4096, EPI_SWIGLU) % 1000 in (124, 184)
+    assert plan(64, 24576, 4096, EPI_SWIGLU) == 164                    # 256 tiles of 96 columns, not 192 of 128
+    assert plan(32, 24576, 4096, EPI_SWIGLU) == 112 and plan(64, 51200, 5120, EPI_SWIGLU) % 1000 in (124, 184)

@@ -141,11 +141,13 @@ def test_gemm_mfma_swiglu(M, I, K):
     assert float((err - 2 ** -8 * want.abs()).max()) <= 1e-3 * float(want.abs().max()) + 1e-5
 
 
-@pytest.mark.parametrize("M,I,K", [(300, 256, 128), (257, 1040, 1024), (512, 96, 64), (70, 304, 256), (1024, 1536, 512)])
-def test_gemm_mfma_swiglu_tile_192_wide(M, I, K):
-    """The SwiGLU product on tiles of 192 columns (three pieces of 32 a wave), by name: sizes
-    that end inside a tile in both directions, weights as stored and packed; rows past the end
-    are not written."""
+@pytest.mark.parametrize("M,I,K,tile", [(300, 256, 128, 168), (257, 1040, 1024, 168), (512, 96, 64, 168), (70, 304, 256, 168),
+                                        (1024, 1536, 512, 168), (64, 480, 256, 164), (33, 1040, 1024, 164), (50, 96, 64, 164),
+                                        (130, 304, 128, 164)])
+def test_gemm_mfma_swiglu_tiles_with_three_pieces_a_wave(M, I, K, tile):
+    """The SwiGLU product on tiles whose waves hold three pieces of 32 columns (192 columns by
+    four waves, 96 by two), by name: sizes that end inside a tile in both directions, weights as
+    stored and packed; rows past the end are not written."""
     from herbert_rs_amd.kernels import mfma
     a = rand(M, K, seed=20, dtype=torch.bfloat16, scale=0.5)
     gate = rand(I, K, seed=21, dtype=torch.bfloat16, scale=0.3)
@@ -156,13 +158,13 @@ def test_gemm_mfma_swiglu_tile_192_wide(M, I, K):
     want = (g / (1 + torch.exp(-g)) * u).float()
     for packed in (False, True):
         out = torch.full((M + 1, I), 3.0, dtype=torch.bfloat16, device=dev())
-        mfma.gemm_swiglu(a, mfma.pack_weight(w) if packed else w, out[:M], packed, tile=168)
+        mfma.gemm_swiglu(a, mfma.pack_weight(w) if packed else w, out[:M], packed, tile=tile)
         err = (out[:M].float() - want).abs()
         assert float((err - 2 ** -8 * want.abs()).max()) <= 1e-3 * float(want.abs().max()) + 1e-5
         assert float((out[M].float() - 3.0).abs().max()) == 0.0
     c = torch.zeros(M, 2 * I, device=dev())
     with pytest.raises(Exception, match="SwiGLU product whole only"):
-        mfma.gemm(a, w, c, tile=168)
+        mfma.gemm(a, w, c, tile=tile)
 
 
 def test_gemm_mfma_refuses_what_it_cannot_do():
