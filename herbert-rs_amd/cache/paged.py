@@ -235,6 +235,12 @@ class Cache:
         for g in self.kv_groups.values():
             g.release_unseen(slot, int(self.lengths[slot]))
 
+    @property
+    def rolls_back_freely(self):
+        """True where `truncate` never refuses a length within the slot's own: no per-sequence
+        state, no group that gives keys up as a sequence grows."""
+        return not self.state_groups and all(not g.need.window for g in self.kv_groups.values())
+
     def truncate(self, slot, length):
         """Roll a slot back to its first `length` positions (the reference's truncate_kv,
         crates/backends/backend_common/src/cpu_backend.rs:527-543). Fixed-size state cannot be

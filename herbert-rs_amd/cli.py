@@ -13,7 +13,8 @@ token ids (crates/cli/src/token_parser.rs:13-26) and the output is token ids.
 steps after the token that the prompt gives, as the reference's single shot counts them
 (main.rs:1040,1241): up to max-tokens + 1 tokens come out. SIGINT, SIGTERM and SIGHUP set a
 flag that the generation loop looks at before every decode step; a second signal exits at
-once with 130 (main.rs:22-50,1242-1245).
+once with 130 (main.rs:22-50,1242-1245). Without --prompt and --prompt-file the conversation
+of `chat.py` starts (main.rs:70,718-757), which needs a tokenizer.
 """
 import argparse
 import os
@@ -132,6 +133,66 @@ def print_arch():
     return 0
 
 
+class StreamPrinter:
+    """Prints a sequence's text as its tokens come: the whole text is decoded again each time and
+    only what is new is printed, never a trailing U+FFFD, which a later token may still
+    complete (crates/cli/src/main.rs:1306-1326). `on_token` is the generation loop's callback;
+    it ends the sequence where the text holds a stop string."""
+
+    def __init__(self, tokenizer, show_specials=False, stop_strings=(), out=None):
+        self.tokenizer, self.show_specials, self.stop_strings = tokenizer, show_specials, list(stop_strings)
+        self.out = out if out is not None else sys.stdout
+        self.produced, self.printed = [], 0
+
+    def on_token(self, _, tok):
+        from .sampling import STOP_SEQUENCE
+        self.produced.append(tok)
+        if self.tokenizer is None:
+            print(tok if len(self.produced) == 1 else f",{tok}", end="", flush=True, file=self.out)
+            return None
+        text = self.tokenizer.decode(self.produced, skip_special_tokens=not self.show_specials)
+        safe = len(text.rstrip("\ufffd"))
+        if safe > self.printed:
+            print(text[self.printed:safe], end="", flush=True, file=self.out)
+            self.printed = safe
+        if self.stop_strings and find_stop_sequence(text, self.stop_strings) is not None:
+            return STOP_SEQUENCE
+        return None
+
+
+def end_of_turn_id(chat, tokenizer):
+    """The id of the token that ends the model's turn: the tokenizer's, else the architecture's
+    own (crates/cli/src/main.rs:616-619); None where the architecture names none."""
+    if chat is None or chat.end_of_turn is None:
+        return None
+    found = tokenizer.token_to_id(chat.end_of_turn) if tokenizer is not None else None
+    return found if found is not None else chat.end_of_turn_id
+
+
+def think_tokens_of(chat, tokenizer):
+    """The ids that open and close a think block and of a line break: from the tokenizer, else
+    from the architecture's entry (crates/cli/src/main.rs:671-684)."""
+    from .sampling import ThinkTokens
+    if chat is None or chat.think_open_id is None or chat.think_close_id is None or chat.newline_id is None:
+        raise RequestError("--think-budget / --nothink: this architecture names no think tokens")
+    open_id, close_id, newline_id = chat.think_open_id, chat.think_close_id, chat.newline_id
+    if tokenizer is not None:
+        found = tokenizer.token_to_id(chat.think_open)
+        open_id = found if found is not None else open_id
+        found = tokenizer.token_to_id(chat.think_close)
+        close_id = found if found is not None else close_id
+        line = tokenizer.encode("\n", add_special_tokens=False).ids
+        newline_id = line[0] if len(line) == 1 else newline_id
+    return ThinkTokens(open_id, close_id, newline_id)
+
+
+def check_think_tokens(think_tokens, vocab):
+    if think_tokens is not None and not all(0 <= t < vocab for t in (think_tokens.open_id, think_tokens.close_id,
+                                                                     think_tokens.newline_id)):
+        raise RequestError(f"--think-budget / --nothink: the think tokens {think_tokens} lie outside the "
+                           f"model's vocabulary of {vocab}")
+
+
 def make_parser():
     ap = argparse.ArgumentParser(prog="herbert-cli", description="Herbert - local LLM inference on MI355X")
     ap.add_argument("--arch", action="store_true", help="Show the GPU this would run on and exit")
@@ -175,7 +236,7 @@ def main(argv=None):
 
 def _run(args):
     from .api import load, write_random_model
-    from .sampling import INTERRUPTED, STOP_SEQUENCE, SamplingParams, ThinkTokens
+    from .sampling import INTERRUPTED, SamplingParams
     if args.arch:
         return print_arch()
     if not args.model:
@@ -187,8 +248,6 @@ def _run(args):
     if args.prompt_file:
         with open(args.prompt_file) as f:
             prompt = f.read()
-    if prompt is None:
-        raise RequestError("--prompt or --prompt-file is required (there is no interactive mode)")
     # --system wins over --system-file (crates/cli/src/main.rs:390-397)
     system = args.system
     if system is None and args.system_file:
@@ -207,6 +266,12 @@ def _run(args):
     tokenizer = load_tokenizer(args.model)
     from .config import load_config
     chat = load_config(args.model)[0].chat
+    if prompt is None:
+        if tokenizer is None or chat is None:
+            raise RequestError("--prompt or --prompt-file is required: the conversation needs a tokenizer.json "
+                               "and a chat template")
+        from .chat import run_from_args
+        return run_from_args(args, tokenizer, chat, system, prefill_chunk)
     if tokenizer is not None:
         text = chat.build_prompt(prompt, system) if chat is not None else prompt
         ids = tokenizer.encode(text, add_special_tokens=False).ids
@@ -219,26 +284,13 @@ def _run(args):
             stop_ids.extend(parse_token_ids(s))
     else:
         stop_strings = normalize_stop_sequences(args.stop)
-        if chat is not None and chat.end_of_turn is not None:
-            end = tokenizer.token_to_id(chat.end_of_turn)
-            stop_ids.append(end if end is not None else chat.end_of_turn_id)
+        end = end_of_turn_id(chat, tokenizer)
+        if end is not None:
+            stop_ids.append(end)
 
-    # --nothink is a budget of one token (crates/cli/src/main.rs:685-687); the ids come from the
-    # tokenizer, else from the architecture's entry (:671-684)
+    # --nothink is a budget of one token (crates/cli/src/main.rs:685-687)
     think_budget = 1 if args.nothink else max(0, args.think_budget)
-    think_tokens = None
-    if think_budget > 0:
-        if chat is None or chat.think_open_id is None or chat.think_close_id is None or chat.newline_id is None:
-            raise RequestError("--think-budget / --nothink: this architecture names no think tokens")
-        open_id, close_id, newline_id = chat.think_open_id, chat.think_close_id, chat.newline_id
-        if tokenizer is not None:
-            found = tokenizer.token_to_id(chat.think_open)
-            open_id = found if found is not None else open_id
-            found = tokenizer.token_to_id(chat.think_close)
-            close_id = found if found is not None else close_id
-            line = tokenizer.encode("\n", add_special_tokens=False).ids
-            newline_id = line[0] if len(line) == 1 else newline_id
-        think_tokens = ThinkTokens(open_id, close_id, newline_id)
+    think_tokens = think_tokens_of(chat, tokenizer) if think_budget > 0 else None
 
     t0 = time.perf_counter()
     cache_tokens = args.cache_tokens or (len(ids) + args.max_tokens + 65)
@@ -249,29 +301,8 @@ def _run(args):
                             max_tokens=args.max_tokens + 1, stop_ids=tuple(stop_ids),
                             ignore_eos=args.ignore_eos, repeat_check=not args.no_repeat_check,
                             seed=args.seed, think_budget=think_budget, think_tokens=think_tokens)
-    vocab = engine.spec.vocab_size
-    if think_tokens is not None and not all(0 <= t < vocab for t in (think_tokens.open_id, think_tokens.close_id,
-                                                                     think_tokens.newline_id)):
-        raise RequestError(f"--think-budget / --nothink: the think tokens {think_tokens} lie outside the "
-                           f"model's vocabulary of {vocab}")
-    produced = []
-    printed = [0]
-
-    def on_token(_, tok):
-        produced.append(tok)
-        if tokenizer is None:
-            print(tok if len(produced) == 1 else f",{tok}", end="", flush=True)
-            return None
-        # the whole text again each time and only what is new printed, never a trailing U+FFFD,
-        # which a later token may still complete (crates/cli/src/main.rs:1306-1326)
-        text = tokenizer.decode(produced, skip_special_tokens=not args.show_specials)
-        safe = len(text.rstrip("\ufffd"))
-        if safe > printed[0]:
-            print(text[printed[0]:safe], end="", flush=True)
-            printed[0] = safe
-        if stop_strings and find_stop_sequence(text, stop_strings) is not None:
-            return STOP_SEQUENCE
-        return None
+    check_think_tokens(think_tokens, engine.spec.vocab_size)
+    on_token = StreamPrinter(tokenizer, args.show_specials, stop_strings).on_token
 
     interrupt = InterruptFlag().install()
     t0 = time.perf_counter()

@@ -27,6 +27,9 @@ class ChatFormat:
     build_prompt: Callable          # (user text, system text or None) -> str
     end_of_turn: Optional[str] = None
     end_of_turn_id: Optional[int] = None
+    # what stands between the token that ends a turn and the next turn's text in a conversation
+    # (crates/cli/src/chat.rs:364-381)
+    between_turns: str = ""
     # the tokens that open and close a think block, for a cap on its length
     # (crates/cli/src/main.rs:671-684: looked up in the tokenizer, else these ids)
     think_open: Optional[str] = None

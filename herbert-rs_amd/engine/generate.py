@@ -202,16 +202,48 @@ class Generator:
                 break
             order, (pending, held) = ahead, following
 
-    def _run_batch(self, members, prompts, params, chooser, results, on_token, interrupt=None):
+    def extend(self, slot, tokens, params, chooser, on_token=None, interrupt=None):
+        """One more turn of a sequence whose slot the caller keeps (the reference's
+        continue_prefill and decode on a kept KvHandle, crates/cli/src/chat.rs:1060-1075,
+        164-352): `tokens` go on from what the slot holds (nothing, for a first turn), then
+        tokens are generated as in `generate`. The slot is not given back; when this returns it
+        holds everything up to the newest generated token, which itself has not been through
+        the model: the next turn's tokens begin with it. `chooser` is the caller's too (its
+        generator streams go on from turn to turn); sequence index 0 is used. Returns one
+        GenerationResult."""
+        params.validate()
+        if not tokens:
+            raise RequestError("a turn needs at least one token")
+        eng = self.engine
+        room = eng.spec.max_positions - eng.cache.length(slot)
+        if len(tokens) > room:
+            raise RequestError(f"a turn of {len(tokens)} tokens does not fit: the sequence holds "
+                               f"{eng.cache.length(slot)} of max_position_embeddings ({eng.spec.max_positions})")
+        results = [None]
+        self.stats = GenerationStats()
+        self._run_batch([0], [list(tokens)], params, chooser, results, on_token, interrupt, kept={0: slot})
+        self.stats.batches += 1
+        return results[0]
+
+    def _run_batch(self, members, prompts, params, chooser, results, on_token, interrupt=None, kept=None):
+        """`kept`: request index -> a slot of the caller's (see `extend`) instead of one taken
+        here and given back at the end."""
         eng = self.engine
         eos = eng.spec.eos_token_id
-        slots = {i: eng.alloc_slot() for i in members}
+        kept = kept or {}
+        slots = {i: kept[i] if i in kept else eng.alloc_slot() for i in members}
+        before = {i: eng.cache.length(kept[i]) for i in kept}
         generated = {i: [] for i in members}
         live = list(members)
 
         def finish(i, reason):
             results[i] = GenerationResult(generated[i], reason, len(prompts[i]))
-            eng.free_slot(slots.pop(i))
+            slot = slots.pop(i)
+            if i in kept:
+                # a step that ran ahead of the host has taken the newest token in already
+                eng.truncate(slot, before[i] + len(prompts[i]) + len(generated[i]) - 1)
+            else:
+                eng.free_slot(slot)
             live.remove(i)
 
         try:
@@ -244,8 +276,10 @@ class Generator:
                         finish(i, INTERRUPTED)
 
             take(list(live), tokens)
+            # (a kept slot is rolled back by the one step that ran ahead: only where the cache can)
             if self.run_ahead and getattr(chooser, "can_run_ahead", False) and \
-                    getattr(eng, "accepts_device_tokens", False):
+                    getattr(eng, "accepts_device_tokens", False) and \
+                    (not kept or getattr(eng.cache, "rolls_back_freely", False)):
                 self._decode_ahead(live, slots, generated, params, chooser, take)
             else:
                 while live:
@@ -256,4 +290,6 @@ class Generator:
             self.stats.decode_seconds += time.perf_counter() - t0
         finally:
             for i in list(slots):
-                eng.free_slot(slots.pop(i))
+                slot = slots.pop(i)
+                if i not in kept:
+                    eng.free_slot(slot)

@@ -52,7 +52,7 @@ def chatml_prompt(user_prompt, system_prompt=None):
 
 
 # the end-of-turn token and its id where the tokenizer lacks it (crates/cli/src/main.rs:616-619)
-CHAT = ChatFormat(chatml_prompt, end_of_turn="<|im_end|>", end_of_turn_id=151645,
+CHAT = ChatFormat(chatml_prompt, end_of_turn="<|im_end|>", end_of_turn_id=151645, between_turns="\n",
                   think_open="<think>", think_close="</think>", think_open_id=151667, think_close_id=151668,
                   newline_id=198)
 

@@ -50,6 +50,12 @@ class Sampler:
         if params.think_budget > 0:
             self.think = [ThinkBudget(params.think_budget, params.think_tokens) for _ in range(num_sequences)]
 
+    def new_turn(self):
+        """A conversation's next turn: its think blocks begin closed (crates/cli/src/chat.rs:1119);
+        the generator streams go on."""
+        for t in self.think or ():
+            t.reset()
+
     def _sifted_for(self, rows):
         """Buffers for the candidates that a block a chunk sifts out of a long row (top-k up to 1024)."""
         p = self.params

@@ -35,6 +35,10 @@ class ThinkBudget:
         """The block was opened by the prompt, not by a generated token (sampler.rs:181-186)."""
         self.in_think, self.count = True, 0
 
+    def reset(self):
+        """A new turn begins outside any block (sampler.rs:194-198)."""
+        self.in_think, self.count = False, 0
+
     def track(self, token):
         """After every chosen token (sampler.rs:200-212)."""
         if token == self.tokens.open_id:

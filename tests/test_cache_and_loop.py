@@ -514,3 +514,197 @@ def test_decoding_ahead_on_random_requests_gives_the_same():
         got = Generator(eng, max_batch=max_batch, make_chooser=AheadChooser).generate(prompts, params)
         assert [(r.tokens, r.stop_reason) for r in got] == [(r.tokens, r.stop_reason) for r in want], trial
         assert eng.cache.slots.held_count == 0 and AheadChooser.unread <= 1
+
+
+# ---- a conversation: turns on a kept slot
+class KeepingEngine(AheadEngine):
+    """Remembers the tokens every slot holds, and can roll a slot back."""
+
+    def __init__(self, ahead=True, rolls_back=True):
+        super().__init__()
+        self.accepts_device_tokens = ahead
+        self.cache.rolls_back_freely = rolls_back
+        self.held = {}
+        self.rolled_back = 0
+
+    def alloc_slot(self):
+        s = super().alloc_slot()
+        self.held[s] = []
+        return s
+
+    def step(self, entries, tokens_on_device=None):
+        if any(len(e.tokens) > 1 for e in entries):
+            AheadChooser.unread = 0          # a new turn: what ran ahead for nothing before it is forgotten
+        if tokens_on_device is not None:
+            entries = [type(e)(e.slot, [int(t)], e.want) for e, t in zip(entries, tokens_on_device)]
+        for e in entries:
+            self.held[e.slot].extend(e.tokens)
+        return FakeEngine.step(self, entries)
+
+    def truncate(self, slot, length):
+        assert 0 <= length <= self.cache.lengths[slot]
+        self.rolled_back += self.cache.lengths[slot] - length
+        self.cache.lengths[slot] = length
+        del self.held[slot][length:]
+
+
+@pytest.mark.parametrize("ahead,rolls_back", [(False, True), (True, True), (True, False)])
+def test_turns_on_a_kept_slot_go_on_from_what_it_holds(ahead, rolls_back):
+    """Generator.extend: the slot is the caller's and is kept; after a turn it holds the turn's
+    tokens and all generated ones but the newest, whether or not a step ran ahead of the host
+    (the extra step is rolled back; where the cache cannot roll back nothing runs ahead)."""
+    eng = KeepingEngine(ahead, rolls_back)
+    AheadChooser.unread = 0
+    gen = Generator(eng, max_batch=1, make_chooser=AheadChooser)
+    chooser = AheadChooser(None, 1, 50, "cpu")
+    slot = eng.alloc_slot()
+    r1 = gen.extend(slot, [30, 31], SamplingParams(temperature=0.0, max_tokens=4, repeat_check=False), chooser)
+    assert r1.tokens == [32, 33, 34, 35] and r1.stop_reason == MAX_TOKENS
+    assert eng.held[slot] == [30, 31, 32, 33, 34] and eng.cache.length(slot) == 5
+    # a turn that the model ends on a token's value: with a step ahead that token has been fed already
+    r2 = gen.extend(slot, [35, 5], SamplingParams(temperature=0.0, max_tokens=10, repeat_check=False), chooser)
+    assert r2.tokens == [6, 7, 8, 9] and r2.stop_reason == EOS
+    assert eng.held[slot] == [30, 31, 32, 33, 34, 35, 5, 6, 7, 8] and eng.cache.length(slot) == 10
+    assert eng.rolled_back == (1 if ahead and rolls_back else 0)
+    # the caller's word ends a turn as well; the slot is still the caller's
+    r3 = gen.extend(slot, [9, 40], SamplingParams(temperature=0.0, max_tokens=10, repeat_check=False), chooser,
+                    on_token=lambda i, tok: "enough" if tok == 42 else None)
+    assert r3.tokens == [41, 42] and r3.stop_reason == "enough" and eng.held[slot][-3:] == [9, 40, 41]
+    assert eng.cache.slots.held_count == 1
+    with pytest.raises(RequestError, match="does not fit"):
+        gen.extend(slot, list(range(30)), SamplingParams(temperature=0.0, max_tokens=2), chooser)
+    with pytest.raises(RequestError, match="at least one token"):
+        gen.extend(slot, [], SamplingParams(temperature=0.0, max_tokens=2), chooser)
+    eng.free_slot(slot)
+    assert eng.cache.slots.held_count == 0
+
+
+class WordTokenizer:
+    """Words and the specials of a chat template as tokens; ids grow as words are first seen."""
+    SPECIALS = ["<|im_start|>", "<|im_end|>", "\n"]
+
+    def __init__(self):
+        self.ids = {"<|im_start|>": 10, "<|im_end|>": 9, "\n": 11}
+
+    def token_to_id(self, token):
+        return self.ids.get(token)
+
+    def encode(self, text, add_special_tokens=False):
+        import re
+        pieces = [p for p in re.split(r"(<\|im_start\|>|<\|im_end\|>|\n| )", text) if p and p != " "]
+        for p in pieces:
+            self.ids.setdefault(p, 12 + len(self.ids))
+        return type("Encoding", (), {"ids": [self.ids[p] for p in pieces]})()
+
+    def decode(self, ids, skip_special_tokens=True):
+        names = {v: k for k, v in self.ids.items()}
+        words = [names.get(i, f"#{i}") for i in ids]
+        if skip_special_tokens:
+            words = [w for w in words if w not in ("<|im_start|>", "<|im_end|>")]
+        return " ".join(words)
+
+
+def test_a_conversation_keeps_its_slot_and_runs_its_commands():
+    """The chat loop with a stand-in engine (next token = last + 1, token 9 ends a turn) and a
+    word tokenizer: what each turn feeds, the slash commands, a line continued with a backslash,
+    /clear, the end of the input."""
+    import io
+    from herbert_rs_amd.chat import Chat, ChatSession
+    from herbert_rs_amd.models.qwen3 import CHAT
+    from herbert_rs_amd.sampling import ThinkTokens
+    import herbert_rs_amd.chat as chat_mod
+
+    class FakeSampler(AheadChooser):
+        made = 0
+
+        def __init__(self, params, n, vocab, device):
+            super().__init__(params, n, vocab, device)
+            type(self).made += 1
+            self.turns = 0
+
+        def new_turn(self):
+            self.turns += 1
+
+    import herbert_rs_amd.sampling.sampler as sampler_mod
+    eng = KeepingEngine(ahead=True)
+    eng.spec.max_positions = 200
+    tok = WordTokenizer()
+    params = SamplingParams(temperature=0.0, max_tokens=5, stop_ids=(9,), repeat_check=False)
+    session = ChatSession(eng, tok, CHAT, params, system="be brief", end_id=9)
+    lines = iter(["/config", "hello \\", "there", "/stats", "/temp 0.5", "/temp x", "/topk 7", "/topp 2", "/think 3",
+                  "again", "/nope", "/clear", "/stats", "once more", "/tools", "", "/quit", "never read"])
+
+    def read_line(prompt):
+        try:
+            return next(lines)
+        except StopIteration:
+            raise EOFError
+    out, err = io.StringIO(), io.StringIO()
+    real = sampler_mod.Sampler
+    sampler_mod.Sampler = FakeSampler
+    AheadChooser.unread = 0
+    try:
+        chat = Chat(session, think_tokens=lambda: ThinkTokens(20, 21, 11), read_line=read_line, out=out, err=err)
+        assert chat.run() == 0
+    finally:
+        sampler_mod.Sampler = real
+    said = err.getvalue()
+    assert "--- Config (greedy) ---" in said and "think_budget: unlimited" in said
+    assert "Usage: /temp <value>" in said and "Top-p must be between 0 and 1" in said
+    assert "think_budget: 3 tokens" in said and "Unknown command: /nope" in said
+    assert "[Conversation cleared]" in said and "KV cache tokens: 0 (cleared)" in said
+    assert "/tools is not available here" in said and "Turns:           1" in said
+    assert next(lines) == "never read"                       # /quit ended the loop
+    assert eng.cache.slots.held_count == 0                   # the slot went back at the end
+    # the first turn: the template with the system prompt, the two lines joined by a line break
+    first = tok.encode(CHAT.build_prompt("hello \nthere", "be brief")).ids
+    assert session.turns == 3 and FakeSampler.made == 2      # the commands that change parameters made a new sampler, /clear none
+    # what the slots held is gone with them; the turns' tokens are seen in the steps' sizes
+    sizes = [n for step in eng.steps for _, n in step]
+    assert sizes[0] == len(first)
+    # the model's text went to `out`, one line a turn
+    assert len(out.getvalue().strip().split("\n")) == 3
+
+
+def test_a_turn_begins_with_the_token_the_last_one_ended_on():
+    from herbert_rs_amd.chat import ChatSession
+    from herbert_rs_amd.models.qwen3 import CHAT
+    import herbert_rs_amd.sampling.sampler as sampler_mod
+
+    class FakeSampler(AheadChooser):
+        def new_turn(self):
+            pass
+    real = sampler_mod.Sampler
+    sampler_mod.Sampler = FakeSampler
+    AheadChooser.unread = 0
+    try:
+        eng = KeepingEngine(ahead=True)
+        eng.spec.max_positions = 300
+        tok = WordTokenizer()
+        tok.ids.update({"a": 5, "b": 30})
+        session = ChatSession(eng, tok, CHAT, SamplingParams(temperature=0.0, max_tokens=3, stop_ids=(9,),
+                                                              repeat_check=False), end_id=9)
+        # "assistant" and the line break that ends the template get ids 12.. ; the reply counts on from the last
+        r1 = session.say("a")
+        slot = session.slot
+        held1 = list(eng.held[slot])
+        assert held1[:-len(r1.tokens) + 1 or None][:len(tok.encode(CHAT.build_prompt("a", None)).ids)] == \
+            tok.encode(CHAT.build_prompt("a", None)).ids
+        assert r1.stop_reason == MAX_TOKENS and session.last_token == r1.tokens[-1]
+        assert held1 == tok.encode(CHAT.build_prompt("a", None)).ids + r1.tokens[:-1]
+        # cut short: the next turn brings the last token, the end-of-turn token, the line break, the template
+        r2 = session.say("b")
+        want = held1 + [r1.tokens[-1], 9, 11] + tok.encode(CHAT.build_prompt("b", None)).ids + r2.tokens[:-1]
+        assert eng.held[slot] == want
+        # a turn that the model ended itself: its last token is the end-of-turn token and is not doubled
+        session.last_token = 9
+        assert session.turn_tokens("b")[:3] == [9, 11, 10]
+        # no room: the turn is refused and the conversation is still there
+        eng.spec.max_positions = len(want) + 5
+        with pytest.raises(RequestError, match="no room left"):
+            session.say("b")
+        assert session.slot == slot
+        session.clear()
+        assert eng.cache.slots.held_count == 0
+    finally:
+        sampler_mod.Sampler = real

@@ -97,6 +97,46 @@ def test_roll_back_and_feed_other_tokens(name, dtype, model_root):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["C", "D"])
+def test_turns_on_a_kept_slot_leave_the_whole_conversation_in_the_cache(name, dtype, model_root):
+    """Generator.extend, the conversation's step (the reference's continue_prefill and decode on a
+    kept KvHandle, crates/cli/src/chat.rs:1060-1075): three turns on one slot, each ended by a
+    word of the caller's (where a step ran ahead of the host it is rolled back; the windowed
+    configuration C cannot roll back and runs nothing ahead). Afterwards the slot holds
+    every turn's tokens and all generated ones but the newest, and the logits of the next tokens
+    are those of the plain model on that whole sequence."""
+    from herbert_rs_amd.engine.generate import Generator
+    from herbert_rs_amd.sampling import SamplingParams
+    from herbert_rs_amd.sampling.sampler import Sampler
+    folder = make_folder(model_root, name, dtype)
+    vocab = CONFIGS[name][0]["vocab_size"]
+    engine = hb.load(folder, dtype=dtype, cache_tokens=64 * 8)
+    assert engine.cache.rolls_back_freely == (name == "D")
+    gen = Generator(engine, max_batch=1, prefill_chunk=40)
+    slot = engine.alloc_slot()
+    sequence, last = [], []
+    for turn, n in enumerate((70, 3, 58)):
+        tokens = last + random_tokens(vocab, n, 400 + turn)
+        # the caller ends the turn at its third token: nobody knew beforehand that it would end there
+        params = SamplingParams(temperature=0.0, max_tokens=6, ignore_eos=True, repeat_check=False)
+        said = []
+        r = gen.extend(slot, tokens, params, Sampler(params, 1, vocab, engine.device),
+                       on_token=lambda i, t: said.append(t) or ("enough" if len(said) == 3 else None))
+        assert r.tokens == said and len(said) == 3 and r.stop_reason == "enough"
+        sequence += tokens + r.tokens[:-1]
+        last = [r.tokens[-1]]
+        assert engine.cache.length(slot) == len(sequence)
+    more = last + random_tokens(vocab, 9, 410)
+    ref = plain_logits(folder, sequence + more)
+    got = engine.step([StepEntry(slot, more, list(range(len(more))))]).cpu().numpy()
+    for i in range(len(more)):
+        ok, err = close(got[i], ref[len(sequence) + i], dtype, name, "after three turns")
+        assert ok, (i, err)
+    engine.free_slot(slot)
+    engine.cache.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_a_windowed_cache_rolls_back_only_to_keys_it_still_has(dtype, model_root):
     """Configuration C: one layer sees 70 keys and has given up the pages before them. Rolling
     back a little stays within what is held and gives the plain logits; rolling back past it is
@@ -431,3 +471,53 @@ def test_cli_interrupt_ends_generation_cleanly(model_root, tmp_path):
     tokens = (first + out).strip().split(",")
     assert "Interrupted" in err and "Stop reason:     interrupted" in err
     assert 1 <= len(tokens) < 2041 and all(t.isdigit() for t in tokens)
+
+
+def test_cli_conversation_goes_on_in_its_slot(model_root, tmp_path):
+    """Without a prompt the command line is a conversation (crates/cli/src/main.rs:718-757,
+    crates/cli/src/chat.rs:601-1331): every turn goes on from what the cache holds. What the
+    model says in a turn is what the plain implementation says after the whole conversation so
+    far as one sequence: the earlier turns, each one's last token and end-of-turn token, the
+    new message in the template. A stop string cuts the turns short, so that each ends on a
+    token's value with the next step already run: that step is rolled back. /clear starts over
+    and gives the first turn's answer again."""
+    folder, raw = cli_folder(model_root, tmp_path, "C")      # (a model that says many different words)
+    tok, words = write_tokenizer(folder, raw["vocab_size"])
+    cfg, w = plain_folder(folder)
+    im_end = words["<|im_end|>"]
+    limit = 8
+
+    def template(message, system=None):
+        head = f"<|im_start|>system\n{system}<|im_end|>\n" if system else ""
+        return tok.encode(head + "<|im_start|>user\n" + message + "<|im_end|>\n<|im_start|>assistant\n",
+                          add_special_tokens=False).ids
+
+    def reply(sequence, stop=None):
+        said = plain.greedy(cfg, w, sequence, limit, stop_ids=(im_end, 0))
+        if stop is not None:
+            for n in range(1, len(said) + 1):
+                if stop in tok.decode(said[:n], skip_special_tokens=True):
+                    return said[:n]
+        return said
+
+    first = template("w5 w17 w3", "w9")
+    free = reply(first)
+    stop = tok.decode(free[2:3], skip_special_tokens=True).strip()     # the third word it says
+    r1 = reply(first, stop)
+    assert 1 <= len(r1) <= 3
+    second = first + r1 + [im_end] + template("w40 w41")
+    r2 = reply(second, stop)
+    third = second + r2 + ([] if r2[-1] == im_end else [im_end]) + template("w7")
+    r3 = reply(third, stop)
+    lines = ["w5 w17 \\", "w3", "/stats", "w40 w41", "w7", "/clear", "w5 w17 w3", "/stats", "/quit"]
+    out = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "herbert-cli"), "--model", folder, "--dtype", "float32",
+                          "--temperature", "0", "--no-repeat-check", "--system", "w9", "--max-tokens", str(limit),
+                          "--stop", stop, "--cache-tokens", "512"],
+                         input="\n".join(lines) + "\n", capture_output=True, text=True, timeout=240)
+    assert out.returncode == 0, out.stderr
+    said = [l.strip() for l in out.stdout.split("\n") if l.strip()]
+    want = [tok.decode(r, skip_special_tokens=True).strip() for r in (r1, r2, r3, r1)]
+    assert said == want, (out.stdout, want)
+    held = len(first) + len(r1) - 1
+    assert f"KV cache tokens: {held}" in out.stderr and "[Conversation cleared]" in out.stderr
+    assert out.stderr.count("Turns:") == 2 and "Turns:           4" in out.stderr
