@@ -38,7 +38,11 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 #define EPI_SWIGLU 2
 #define EPI_QKV 3
 
-__device__ __forceinline__ float silu_mul(float g, float u) { return g / (1.0f + __expf(-g)) * u; }
+// silu(g) u with the hardware's reciprocal (1 ulp; the result is rounded to bfloat16): a full division
+// is a dozen instructions, and the epilogue of a 256 x 256 tile does 128 of these a lane
+__device__ __forceinline__ float silu_mul(float g, float u) {
+    return g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)) * u;
+}
 
 // ---------------------------------------------------------------- few rows
 // Workgroup: WAVES waves, NB blocks of 16 weight rows, MB blocks of 16 activation rows (built for
@@ -663,6 +667,56 @@ __device__ __forceinline__ void store_wave_tile_lds(const f32x16 (&acc)[TN32][TM
     }
 }
 
+// The SwiGLU outputs of the large tiles through LDS as well. A lane holds runs of four outputs of
+// 32 different rows, 8 bytes each: a store instruction of the direct way touches 32 lines in pieces
+// of 16 bytes (a round of 256 x 256 tiles spent 15 us beside its products that way, for a quarter
+// of the bytes that the float32 store moves in 8). Here a wave lays its whole tile's outputs into
+// LDS of its own (rows of TN32 x 16 bfloat16, the 16-byte chunk c of row r at chunk c ^ (r mod
+// chunks), or (c + r) mod chunks where the chunks are no power of two), then reads them back
+// along the rows: an instruction stores whole rows, 128 contiguous bytes for a tile 128 wide.
+// n_base: the wave's first column among the interleaved gate/up columns. Needs ldc in steps of
+// 8 and C aligned to 16 bytes.
+template <int TN32, int TM32>
+__device__ __forceinline__ void store_wave_tile_swiglu_lds(const f32x16 (&acc)[TN32][TM32], bf16* C, int M, int N,
+                                                           int ldc, int m_base, int n_base, int lane, bf16* stage) {
+    constexpr int CH = 2 * TN32;            // 16-byte chunks of a row: 16 outputs a piece of 32 columns
+    constexpr int RPI = 64 / CH;            // rows an instruction moves
+    constexpr int ROWS = 32 * TM32;
+    constexpr bool POW2 = (CH & (CH - 1)) == 0;
+    auto place = [&](int row, int chunk) { return POW2 ? (chunk ^ (row & (CH - 1))) : (chunk + row) % CH; };
+    const int c32 = lane & 31, g2 = lane >> 5;
+#pragma unroll
+    for (int b = 0; b < TM32; ++b)
+#pragma unroll
+        for (int a = 0; a < TN32; ++a)
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+                // rows 0..15 of a piece are gate rows, 16..31 the up rows of the same outputs
+                const int row = 32 * b + c32;
+                bf16x4 v;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) v[j] = (__bf16)silu_mul(acc[a][b][4 * q + j], acc[a][b][4 * q + 8 + j]);
+                *(bf16x4*)((__bf16*)stage + row * (CH * 8) + place(row, 2 * a + q) * 8 + 4 * g2) = v;
+            }
+    const int rrow = lane / CH, rchunk = lane % CH;
+    if (lane >= RPI * CH) return;
+#pragma unroll
+    for (int i = 0; i < (ROWS + RPI - 1) / RPI; ++i) {
+        const int row = i * RPI + rrow;
+        if (row >= ROWS) break;
+        const int m = m_base + row, n = n_base / 2 + 8 * rchunk;
+        const bf16x8 v = *(const bf16x8*)((const __bf16*)stage + row * (CH * 8) + place(row, rchunk) * 8);
+        if (m >= M) continue;
+        if (n + 7 < N / 2) {
+            *(bf16x8*)((__bf16*)C + (size_t)m * ldc + n) = v;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                if (n + j < N / 2) ((__bf16*)C)[(size_t)m * ldc + n + j] = v[j];
+        }
+    }
+}
+
 // The q/k/v projection of prompts with what follows it, for heads of 128 (a wave's tile is 128
 // columns wide: one head): per-head RMSNorm (if weights are given), rotation over the whole head
 // (if tables are given), queries to q_out [M, nq 128] and keys and values into the pages (values
@@ -1000,7 +1054,12 @@ gemm_tile_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* _
         const bool sliced = gridDim.y > 1;
         float* const dst = sliced ? partial + (size_t)blockIdx.y * M * N : (float*)Cv;
         const int ld = sliced ? N : ldc;
-        if (VIA_LDS && (ld & 3) == 0 && (N & 3) == 0 && ((size_t)dst & 15) == 0) {
+        constexpr bool SWIGLU_VIA_LDS = EPI == EPI_SWIGLU && BM >= 128 && REGION >= 32 * TM32 * TN32 * 32;
+        if (SWIGLU_VIA_LDS && !sliced && (ldc & 7) == 0 && ((size_t)Cv & 15) == 0) {
+            hb_workgroup_barrier();
+            store_wave_tile_swiglu_lds<TN32, TM32>(acc, (bf16*)Cv, M, N, ldc, m0 + wm * TMB * 16, n0 + wn * TNB * 16, lane,
+                                                   (bf16*)((char*)lds + wave * REGION));
+        } else if (VIA_LDS && (ld & 3) == 0 && (N & 3) == 0 && ((size_t)dst & 15) == 0) {
             hb_workgroup_barrier();
             float* const stage = (float*)((char*)lds + wave * REGION);
             if (sliced || EPI == EPI_STORE)
