@@ -708,3 +708,45 @@ def test_a_turn_begins_with_the_token_the_last_one_ended_on():
         assert eng.cache.slots.held_count == 0
     finally:
         sampler_mod.Sampler = real
+
+
+def test_command_line_pieces_that_need_no_gpu(tmp_path, capsys):
+    """What the command line decides before it loads a model: stop strings unescaped and
+    searched in the text's tail (crates/cli/src/main.rs:212-258), token ids parsed
+    (crates/cli/src/token_parser.rs:13-26), no conversation without a tokenizer, the text of a
+    stream printed once and never with a trailing replacement character."""
+    import io
+    import json
+    from herbert_rs_amd import cli
+    from .tiny import TINY_A
+    assert cli.decode_escaped_text(r"a\nb\t\\c\q\0") == "a\nb\t\\c\\q\0"
+    assert cli.normalize_stop_sequences([" x ", "x", "", r"\n\n"]) == ["x", "\n\n"]
+    assert cli.find_stop_sequence("so it ends. END", ["never", "END"]) == "END"
+    assert cli.find_stop_sequence("END" + "." * 200, ["END"]) is None          # only the tail is searched
+    assert cli.parse_token_ids("5, 17,3") == [5, 17, 3]
+    with pytest.raises(RequestError, match="Invalid token ID"):
+        cli.parse_token_ids("5,x")
+    with pytest.raises(RequestError, match="Need tokenizer.json"):
+        cli.parse_token_ids("hello")
+    folder = tmp_path / "m"
+    folder.mkdir()
+    (folder / "config.json").write_text(json.dumps(TINY_A))
+    assert cli.main(["--model", str(folder)]) == 1
+    assert "the conversation needs a tokenizer.json" in capsys.readouterr().err
+    assert cli.main([]) == 1 and "--model is required" in capsys.readouterr().err
+
+    class Pieces:
+        """Token 1 is the first half of a character, token 2 its second half."""
+        def decode(self, ids, skip_special_tokens=True):
+            text = ""
+            for a, b in zip(ids[::2], ids[1::2] + [None]):
+                text += "é" if (a, b) == (1, 2) else ("�" if b is None and a == 1 else f"<{a}>" + (f"<{b}>" if b else ""))
+            return text
+    out = io.StringIO()
+    printer = cli.StreamPrinter(Pieces(), out=out, stop_strings=["é"])
+    assert printer.on_token(0, 1) is None and out.getvalue() == ""             # half a character: nothing yet
+    assert printer.on_token(0, 2) == STOP_SEQUENCE and out.getvalue() == "é"
+    ids_out = io.StringIO()
+    plain_printer = cli.StreamPrinter(None, out=ids_out)
+    plain_printer.on_token(0, 7), plain_printer.on_token(0, 8)
+    assert ids_out.getvalue() == "7,8"
