@@ -91,8 +91,7 @@ class ChatSession:
             from .sampling.sampler import Sampler
             self.sampler = Sampler(self.params, 1, eng.spec.vocab_size, eng.device)
         self.sampler.new_turn()
-        fresh = self.slot is None
-        if fresh:
+        if self.slot is None:
             self.slot = eng.alloc_slot()
         try:
             result = self.generator.extend(self.slot, tokens, params, self.sampler, on_token, interrupt)
