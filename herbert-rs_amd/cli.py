@@ -2,7 +2,8 @@
 
 Kept with their names, meanings and defaults: --model, --prompt, --prompt-file, --system,
 --max-tokens (2048), --ignore-eos, --no-repeat-check, --stop, --verbose, --temperature (0.4,
-0 = greedy), --top-k (40, 0 = off), --top-p (0.9, 1.0 = off), --show-specials. Added here:
+0 = greedy), --top-k (40, 0 = off), --top-p (0.9, 1.0 = off), --show-specials, --backend (one
+backend here; `help` lists it) and --gpu (an index, or `list`). Added here:
 --dtype, --seed, --cache-tokens, and --random-weights to write a random model folder.
 With a tokenizer.json in the model folder the prompt is text wrapped in the architecture's
 chat template (for this family ChatML, main.rs:281-294; the template and the end-of-turn
@@ -63,6 +64,9 @@ def find_stop_sequence(text, stop_sequences):
         if seq in tail:
             return seq
     return None
+
+
+BACKEND = "hip-gfx950"
 
 
 class InterruptFlag:
@@ -197,6 +201,9 @@ def make_parser():
     ap = argparse.ArgumentParser(prog="herbert-cli", description="Herbert - local LLM inference on MI355X")
     ap.add_argument("--arch", action="store_true", help="Show the GPU this would run on and exit")
     ap.add_argument("--model", help="Model directory")
+    ap.add_argument("--backend", default="auto", help="Backend name (default: auto; use --backend help to list options)")
+    ap.add_argument("--gpu", metavar="INDEX", default=None,
+                    help='GPU device index. Use "list" to show available GPUs.')
     ap.add_argument("--prompt", help="Input prompt (text with a tokenizer, else comma-separated ids)")
     ap.add_argument("--prompt-file", help="Read prompt from a file")
     ap.add_argument("--system", help="System prompt (prepended with chat template)")
@@ -239,6 +246,24 @@ def _run(args):
     from .sampling import INTERRUPTED, SamplingParams
     if args.arch:
         return print_arch()
+    # one backend here, under two names; `help` lists them, `--gpu list` the devices
+    # (crates/cli/src/main.rs:367-386)
+    if args.backend == "help":
+        print(f"Available backends:\n  auto        the one below\n  {BACKEND}  hand-written HIP kernels for MI355X",
+              file=sys.stderr)
+        return 0
+    if args.backend not in ("auto", BACKEND):
+        raise RequestError(f"unknown backend {args.backend!r}; available: auto, {BACKEND}")
+    if args.gpu == "list":
+        return print_arch()
+    if args.gpu is not None:
+        if not args.gpu.isdigit():
+            raise RequestError(f'--gpu must be a number or "list", got: {args.gpu}')
+        import torch
+        if int(args.gpu) >= max(1, torch.cuda.device_count()):
+            raise RequestError(f"--gpu {args.gpu}: this process sees {torch.cuda.device_count()} GPU(s)")
+        if torch.cuda.is_available():
+            torch.cuda.set_device(int(args.gpu))
     if not args.model:
         raise RequestError("--model is required")
     if args.random_weights and not os.path.exists(os.path.join(args.model, "model.safetensors")):
@@ -320,7 +345,7 @@ def _run(args):
         decoded = max(0, st.generated_tokens - 1)
         err = sys.stderr
         print("--- Stats ---", file=err)
-        print("Backend:         hip-gfx950", file=err)
+        print(f"Backend:         {BACKEND}", file=err)
         print(f"Model load:      {load_seconds:.3f}s", file=err)
         print(f"Input tokens:    {st.prompt_tokens}", file=err)
         print(f"Output tokens:   {st.generated_tokens}", file=err)

@@ -734,6 +734,14 @@ def test_command_line_pieces_that_need_no_gpu(tmp_path, capsys):
     assert cli.main(["--model", str(folder)]) == 1
     assert "the conversation needs a tokenizer.json" in capsys.readouterr().err
     assert cli.main([]) == 1 and "--model is required" in capsys.readouterr().err
+    # one backend under two names, as the reference lists its own (crates/cli/src/main.rs:367-386)
+    assert cli.main(["--backend", "help"]) == 0 and cli.BACKEND in capsys.readouterr().err
+    assert cli.main(["--backend", "metal", "--model", str(folder)]) == 1
+    assert "unknown backend 'metal'" in capsys.readouterr().err
+    assert cli.main(["--gpu", "x", "--model", str(folder)]) == 1
+    assert '--gpu must be a number or "list"' in capsys.readouterr().err
+    assert cli.main(["--gpu", "7", "--model", str(folder)]) == 1 and "--gpu 7" in capsys.readouterr().err
+    assert cli.main(["--gpu", "list"]) == 0
 
     class Pieces:
         """Token 1 is the first half of a character, token 2 its second half."""
