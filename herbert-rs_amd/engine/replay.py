@@ -34,19 +34,25 @@ class Replayer:
         os.makedirs(out_dir, exist_ok=True)
 
     def run_step(self, record):
-        step = record["step"]
+        try:
+            step = record["step"]
+            asked = [(e["id"], [int(t) for t in e["tokens"]], [int(j) for j in e.get("want", [])])
+                     for e in record.get("entries", [])]
+            ended = list(record.get("end", []))
+        except (KeyError, TypeError, ValueError) as e:
+            raise RequestError(f"a step is an object with \"step\", \"entries\" (each with \"id\", \"tokens\" "
+                               f"and \"want\") and \"end\": {type(e).__name__} {e}") from None
         entries = []
-        for e in record.get("entries", []):
-            rid = e["id"]
+        for rid, tokens, want in asked:
             if rid not in self.slots:
                 self.slots[rid] = self.engine.alloc_slot()
-            entries.append(StepEntry(self.slots[rid], list(e["tokens"]), list(e.get("want", []))))
+            entries.append(StepEntry(self.slots[rid], tokens, want))
         if entries:
             logits = self.engine.step(entries)
             if logits is not None:
                 arr = logits.detach().to("cpu").numpy().astype("<f4", copy=False)
                 arr.tofile(os.path.join(self.out_dir, f"{step}.f32"))
-        for rid in record.get("end", []):
+        for rid in ended:
             if rid not in self.slots:
                 raise RequestError(f"request {rid!r} ends but never started")
             self.engine.free_slot(self.slots.pop(rid))
@@ -64,11 +70,15 @@ def main(argv=None):
     try:
         engine = Engine.from_folder(args.model, dtype=args.dtype, max_tokens=args.max_tokens)
         replayer = Replayer(engine, args.out)
-        for line in sys.stdin:
+        for number, line in enumerate(sys.stdin, 1):
             line = line.strip()
             if not line:
                 continue
-            step = replayer.run_step(json.loads(line))
+            try:
+                record = json.loads(line)
+            except ValueError as e:
+                raise RequestError(f"line {number} of the input is not JSON: {e}") from None
+            step = replayer.run_step(record)
             print(f"done {step}", flush=True)
     except HerbertError as e:
         print(f"trace_run: {e}", file=sys.stderr, flush=True)

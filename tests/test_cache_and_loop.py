@@ -758,3 +758,44 @@ def test_command_line_pieces_that_need_no_gpu(tmp_path, capsys):
     plain_printer = cli.StreamPrinter(None, out=ids_out)
     plain_printer.on_token(0, 7), plain_printer.on_token(0, 8)
     assert ids_out.getvalue() == "7,8"
+
+
+def test_replay_reads_steps_and_names_what_is_wrong_with_them(tmp_path):
+    """The replay program's reading of its input, with a stand-in engine: slots by request id,
+    given back at "end", logits written for the steps that want some, clear errors for a step
+    that is no such object and for a request that ends without having started."""
+    from herbert_rs_amd.engine.replay import Replayer
+
+    class Rows:
+        def __init__(self, a):
+            self.a = a
+
+        def detach(self):
+            return self
+
+        def to(self, _):
+            return self
+
+        def numpy(self):
+            return self.a
+
+    class Eng(FakeEngine):
+        def step(self, entries):
+            out = super().step(entries)
+            return None if out is None else Rows(out)
+    eng = Eng()
+    rp = Replayer(eng, str(tmp_path / "out"))
+    assert rp.run_step({"step": 0, "entries": [{"id": "a", "tokens": [5, 6], "want": [1]},
+                                               {"id": "b", "tokens": [9], "want": []}], "end": []}) == 0
+    got = np.fromfile(tmp_path / "out" / "0.f32", dtype="<f4").reshape(1, -1)
+    assert got.shape == (1, 50) and got[0].argmax() == 7
+    assert rp.run_step({"step": 1, "entries": [{"id": "a", "tokens": [7]}], "end": ["b"]}) == 1
+    assert not (tmp_path / "out" / "1.f32").exists() and eng.cache.slots.held_count == 1
+    assert eng.steps == [[(0, 2), (1, 1)], [(0, 1)]]
+    with pytest.raises(RequestError, match="ends but never started"):
+        rp.run_step({"step": 2, "entries": [], "end": ["zz"]})
+    for bad in ({"entries": []}, {"step": 3, "entries": [{"tokens": [1]}]}, {"step": 3, "entries": [{"id": "c", "tokens": ["x"]}]},
+                {"step": 3, "entries": 7}):
+        with pytest.raises(RequestError, match="a step is an object"):
+            rp.run_step(bad)
+    assert rp.run_step({"step": 4, "entries": [], "end": ["a"]}) == 4 and eng.cache.slots.held_count == 0
