@@ -69,8 +69,29 @@ def registered_architectures():
     return sorted(_ARCHITECTURES)
 
 
+_plugins_loaded = []
+
+
+def load_plugins():
+    """Import, once, the modules that the environment variable HERBERT_PLUGINS names (separated by
+    commas): modules outside this package that register parts or an architecture of their own, so
+    that the programs (`bin/trace_run`, `bin/herbert-cli`) and `load` know them as they know the
+    library's. The reference's families are compiled in (crates/core/src/config.rs:95-101)."""
+    import importlib
+    import os
+    for name in os.environ.get("HERBERT_PLUGINS", "").split(","):
+        name = name.strip()
+        if name and name not in _plugins_loaded:
+            _plugins_loaded.append(name)
+            try:
+                importlib.import_module(name)
+            except ImportError as e:
+                raise ConfigError(f"HERBERT_PLUGINS names {name!r}, which cannot be imported: {e}") from None
+
+
 def resolve_architecture(raw):
     """The Architecture that a config dict names."""
+    load_plugins()
     archs = raw.get("architectures")
     if isinstance(archs, list) and archs:
         name = archs[0]

@@ -330,3 +330,24 @@ def test_an_architecture_brings_its_own_names_default_and_initialisers(tmp_path)
     assert qwen.chat.end_of_turn == "<|im_end|>" and qwen.chat.end_of_turn_id == 151645
     assert qwen.chat.build_prompt("Hi", "Be brief") == \
         "<|im_start|>system\nBe brief<|im_end|>\n<|im_start|>user\nHi<|im_end|>\n<|im_start|>assistant\n"
+
+
+def test_plugins_named_in_the_environment_are_imported_once(tmp_path, monkeypatch):
+    """HERBERT_PLUGINS names modules outside the package that register parts or architectures of
+    their own; they are imported before a config.json's architecture is looked up, once, and one
+    that cannot be imported is a clear error."""
+    import sys
+    from herbert_rs_amd.config import registry
+    (tmp_path / "counting_plugin.py").write_text("import os\nos.environ['COUNTING_PLUGIN'] = str(int(os.environ.get('COUNTING_PLUGIN', '0')) + 1)\n")
+    monkeypatch.syspath_prepend(str(tmp_path))
+    monkeypatch.setenv("HERBERT_PLUGINS", " counting_plugin ,")
+    monkeypatch.setenv("COUNTING_PLUGIN", "0")
+    monkeypatch.setattr(registry, "_plugins_loaded", [])
+    assert resolve_architecture({"model_type": "qwen3"}).name == "Qwen3ForCausalLM"
+    assert resolve_architecture({"model_type": "qwen3"}).name == "Qwen3ForCausalLM"
+    import os
+    assert os.environ["COUNTING_PLUGIN"] == "1"
+    monkeypatch.setenv("HERBERT_PLUGINS", "counting_plugin,no_such_plugin_module")
+    with pytest.raises(ConfigError, match="no_such_plugin_module"):
+        resolve_architecture({"model_type": "qwen3"})
+    sys.modules.pop("counting_plugin", None)
