@@ -95,8 +95,9 @@ class ChatSession:
             self.slot = eng.alloc_slot()
         try:
             result = self.generator.extend(self.slot, tokens, params, self.sampler, on_token, interrupt)
-        except HerbertError:
-            # what the slot holds is no longer known to fit a turn's end: start over
+        except BaseException:
+            # (an error of the engine's, or anything the caller's on_token raised) what the slot
+            # holds is no longer known to end where a turn ends: start over
             self.clear()
             raise
         st = self.generator.stats
