@@ -1462,6 +1462,36 @@ static GemmPlan plan_gemm(int M, int N, int K, int ldc, int epi, bool norm_w, bo
     return GemmPlan{tile, slices, mid_cost >= 0 ? mid_cost : low_cost};
 }
 
+// The rows of the first of two products that M rows are better cut into (see hb_gemm_mfma), or 0.
+static int split_rows(int M, int N, int K, int ldc, int epi, bool special, int tile_hint, size_t workspace_floats,
+                      const GemmPlan& whole) {
+    if (special || M <= 128 || (tile_hint != 0 && tile_hint != -128 && tile_hint != -256)) return 0;
+    int best_main = 0;
+    double best = whole.cost;
+    for (int bm = 128; bm <= 256; bm *= 2) {
+        const int main_rows = M / bm * bm, rest = M - main_rows;
+        if (rest == 0 || main_rows == 0) continue;
+        const GemmPlan a = plan_gemm(main_rows, N, K, ldc, epi, false, false, false, 0, workspace_floats);
+        const GemmPlan b = plan_gemm(rest, N, K, ldc, epi, false, false, false, 0, workspace_floats);
+        if (a.tile < 0 || b.tile < 0) continue;
+        if (tile_hint == -bm) return main_rows;
+        if (tile_hint != 0 || whole.cost < 0 || a.cost < 0 || b.cost < 0) continue;
+        // (a second launch and its start are in the estimates; a tenth is kept as a margin for their error)
+        if (a.cost + b.cost < 0.9 * best) {
+            best = (a.cost + b.cost) / 0.9;
+            best_main = main_rows;
+        }
+    }
+    return best_main;
+}
+
+// The rows that hb_gemm_mfma cuts off as a first product of their own, or 0 (for tests and measurements).
+extern "C" int hb_gemm_mfma_split(int M, int N, int K, int epi, size_t workspace_floats) {
+    const int ldc = epi == EPI_SWIGLU ? N / 2 : N;
+    const GemmPlan whole = plan_gemm(M, N, K, ldc, epi, false, false, false, 0, workspace_floats);
+    return whole.tile < 0 ? 0 : split_rows(M, N, K, ldc, epi, false, 0, workspace_floats, whole);
+}
+
 // The plan as a number for tests and measurements: tile + 1000 x slices (slices > 1), 0 for the
 // few-row kernel, -1 if the product is refused. emit: 0 none, 1 a norm is left behind. deferred:
 // the slices are left for the next kernel to add up.
@@ -1516,8 +1546,24 @@ extern "C" int hb_gemm_mfma(const void* X, const void* W, void* C, int M, int N,
     HB_REQUIRE(!deferred_slices || (epi == EPI_STORE && !emit_g), "gemm_mfma: only a plain product leaves its slices");
     if (deferred_slices) *deferred_slices = 1;
     const GemmPlan plan = plan_gemm(M, N, K, ldc, epi, norm_w != nullptr, emit_g != nullptr, scale_partial != nullptr,
-                                    tile_hint, workspace_floats, deferred_slices != nullptr);
+                                    tile_hint < 0 ? 0 : tile_hint, workspace_floats, deferred_slices != nullptr);
     HB_REQUIRE(plan.tile >= 0, "gemm_mfma: no kernel takes M=%d, N=%d, K=%d with the norm asked of it", M, N, K);
+    // Rows that end a little past a whole number of tiles pay a round of tiles for a few rows (a
+    // prompt of 2,049 tokens took a quarter longer than one of 2,048). Such a product is cut in
+    // two along its rows, the whole tiles and the rest as products of their own (the epilogues
+    // work row by row), where the estimates say that this is a good deal faster.
+    // tile_hint -128 / -256: cut there whatever the estimates say (for tests).
+    const int rows_main = split_rows(M, N, K, ldc, epi, norm_w || emit_g || scale_partial || deferred_slices, tile_hint,
+                                     workspace_floats, plan);
+    if (rows_main > 0) {
+        const size_t out_bytes = epi == EPI_SWIGLU ? sizeof(bf16) : sizeof(float);
+        const int rc = hb_gemm_mfma(X, W, C, rows_main, N, K, ldc, epi, packed, nullptr, eps, 0, workspace, workspace_floats,
+                                    nullptr, nullptr, nullptr, nullptr, 0, 0.f, 0.f, nullptr, stream);
+        if (rc != 0) return rc;
+        return hb_gemm_mfma((const bf16*)X + (size_t)rows_main * K, W, (char*)C + (size_t)rows_main * ldc * out_bytes,
+                            M - rows_main, N, K, ldc, epi, packed, nullptr, eps, 0, workspace, workspace_floats, nullptr,
+                            nullptr, nullptr, nullptr, 0, 0.f, 0.f, nullptr, stream);
+    }
     if (plan.tile == 0) {
         pick_skinny(X, W, C, M, N, K, ldc, epi, packed, norm_w, eps, stream, hand);
         HB_CHECK_LAUNCH("gemm_skinny");

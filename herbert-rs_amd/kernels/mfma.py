@@ -21,6 +21,7 @@ lib.register_signatures("gemm_mfma", {
                      _F, _P, _P],
     "hb_gemm_mfma_plan": [_I, _I, _I, _I, _I, _I, _I, ctypes.c_size_t, _I],
     "hb_gemm_mfma_plan_cost": [_I, _I, _I, _I, _I, _I, _I, ctypes.c_size_t, _I],
+    "hb_gemm_mfma_split": [_I, _I, _I, _I, ctypes.c_size_t],
     "hb_gemm_qkv_mfma": [_P, _P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _F, _I, _I, _I, _I, _P],
 })
 
@@ -197,6 +198,13 @@ def gemm_plan(M, N, K, epi=EPI_STORE, normed_input=False, leaves_norm=False, fin
                                                    int(finishes_norm), ws_floats, int(defer_slices))
 
 
+def gemm_split(M, N, K, epi=EPI_STORE, device="cuda"):
+    """The rows that hb_gemm_mfma cuts off as a first product of their own (whole tiles; the rest
+    follows as a second product), or 0 where it runs the product whole."""
+    _, ws_floats = _slice_workspace(torch.device(device), M, N, K)
+    return lib.load("gemm_mfma").hb_gemm_mfma_split(M, N, K, epi, ws_floats)
+
+
 def gemm_plan_cost(M, N, K, epi=EPI_STORE, normed_input=False, leaves_norm=False, finishes_norm=False, device="cuda",
                    defer_slices=False):
     """The estimated time in us of the plan gemm_plan gives; negative where no estimate chose it."""
@@ -242,7 +250,13 @@ def qkv_tile_shape(M, N):
     writes the cache itself, or None where it should not (too few tiles to fill the CUs: the plain
     product's smaller tiles and K slices then do better, and a kernel of its own does the rest).
     0: 256 x 256; 1: a head wide, 256 rows high; 2: a head wide, 128 rows high."""
-    if -(-M // 256) * -(-N // 256) >= QKV_FUSE_MIN_TILES:
+    tiles = -(-M // 256) * -(-N // 256)
+    if tiles >= QKV_FUSE_MIN_TILES:
+        # (rows that end a little past whole tiles, with a last round of tiles that is nearly empty:
+        # the plain product cuts such rows off as a product of their own and is then ahead, 3 % of a
+        # prompt of 2,600 tokens)
+        if tiles > 256 and tiles % 256 < 64 and 0 < M % 256 <= 64:
+            return None
         return 0
     heads = N // 128
     for shape, rows in ((1, 256), (2, 128)):

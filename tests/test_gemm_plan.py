@@ -92,3 +92,24 @@ def test_known_choices(plan):
     assert plan(2048, 4096, 12288, EPI_ADD) == 142
     assert plan(64, 24576, 4096, EPI_SWIGLU) == 164                    # 256 tiles of 96 columns, not 192 of 128
     assert plan(32, 24576, 4096, EPI_SWIGLU) == 112 and plan(64, 51200, 5120, EPI_SWIGLU) % 1000 in (124, 184)
+
+
+def test_rows_just_past_whole_tiles_are_cut_off_as_a_product_of_their_own():
+    """A product whose rows end a little past a whole number of large tiles would pay a round of
+    tiles for them: it is cut in two along its rows where the estimates say so, never where the
+    rows fill their tiles, and never for few rows."""
+    from herbert_rs_amd.kernels import mfma  # noqa: F401
+    split = lib.load("gemm_mfma").hb_gemm_mfma_split
+    W = 1 << 26
+    H, I = 4096, 12288
+    for M in (2049, 2064, 2112):
+        assert split(M, 2 * I, H, EPI_SWIGLU, W) == 2048 and split(M, H, I, EPI_ADD, W) == 2048, M
+    assert split(2049, 2 * I, H, EPI_SWIGLU, 0) == 2048           # (a rest of few rows needs no room for K slices)
+    for M in (1, 16, 64, 128, 1024, 2048, 2304, 4096):
+        for N, K, epi in ((2 * I, H, EPI_SWIGLU), (H, I, EPI_ADD), (H, H, EPI_ADD), (6144, H, EPI_STORE)):
+            assert split(M, N, K, epi, W) == 0, (M, N, K)
+    for M, N, K in itertools.product([130, 257, 300, 513, 700, 1025, 1500, 3000, 5000], WIDTHS, [512, 2048, 4096, 12288]):
+        for epi in (EPI_STORE, EPI_ADD, EPI_SWIGLU):
+            for ws in (0, W):
+                rows = split(M, N, K, epi, ws)
+                assert rows == 0 or (0 < rows < M and rows % 128 == 0 and M - rows < 256), (M, N, K, epi, rows)

@@ -167,6 +167,33 @@ def test_gemm_mfma_swiglu_tiles_with_three_pieces_a_wave(M, I, K, tile):
         mfma.gemm(a, w, c, tile=tile)
 
 
+@pytest.mark.parametrize("M,N,K,cut", [(300, 256, 128, -128), (257, 96, 64, -256), (530, 512, 256, -256), (129, 64, 64, -128),
+                                       (2049, 512, 128, 0)])
+def test_gemm_mfma_rows_cut_into_two_products(M, N, K, cut):
+    """A product cut in two along its rows (whole tiles, then the rest, each a product of its own;
+    by name, and at the last size by the kernel's own estimates): store, add and SwiGLU give what
+    the product whole gives, and nothing beyond the rows is written."""
+    from herbert_rs_amd.kernels import mfma
+    a = rand(M, K, seed=30, dtype=torch.bfloat16, scale=0.5)
+    w = rand(N, K, seed=31, dtype=torch.bfloat16, scale=0.3)
+    want = a.double() @ w.double().T
+    wp = mfma.pack_weight(w)
+    out = torch.full((M + 1, N), 3.0, device=dev())
+    mfma.gemm(a, wp, out[:M], False, True, tile=cut)
+    assert float((out[:M].double() - want).abs().max()) <= 1e-5 * float(want.abs().max()) + 1e-6
+    assert float((out[M] - 3.0).abs().max()) == 0.0
+    mfma.gemm(a, wp, out[:M], True, True, tile=cut)
+    assert float((out[:M].double() - 2 * want).abs().max()) <= 2e-5 * float(want.abs().max()) + 1e-6
+    gate, up = w[:N // 2], w[N // 2:]
+    g, u = a.double() @ gate.double().T, a.double() @ up.double().T
+    act = (g / (1 + torch.exp(-g)) * u).float()
+    half = torch.full((M + 1, N // 2), 3.0, dtype=torch.bfloat16, device=dev())
+    mfma.gemm_swiglu(a, mfma.pack_weight(mfma.interleave_gate_up(gate, up)), half[:M], True, tile=cut)
+    err = (half[:M].float() - act).abs()
+    assert float((err - 2 ** -8 * act.abs()).max()) <= 1e-3 * float(act.abs().max()) + 1e-5
+    assert float((half[M].float() - 3.0).abs().max()) == 0.0
+
+
 def test_gemm_mfma_refuses_what_it_cannot_do():
     from herbert_rs_amd.kernels import mfma
     a = rand(4, 40, dtype=torch.bfloat16)
