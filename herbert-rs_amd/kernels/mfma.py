@@ -54,7 +54,9 @@ def _new_slice_workspace(device, M, N, K, tile):
     tiles = ((M + 255) // 256) * ((N + 255) // 256)       # of the largest kind: under two rounds of them on 256 CUs
     slices = min(16, K // 256) if tiles < 512 or tile else 1
     need = min(slices * M * N, SLICE_WORKSPACE_FLOATS)
-    if slices < 2 or need < 2 * M * N:
+    # (a product too large to be cut even in two still gets the room: where its rows are cut into
+    # whole tiles and a rest, the rest's few rows are cut along K)
+    if slices < 2:
         return None, 0
     kept = _workspaces.setdefault(str(device), [])
     if not kept or kept[-1].numel() < need:
