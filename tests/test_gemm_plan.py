@@ -8,7 +8,7 @@ from herbert_rs_amd.kernels import lib
 
 EPI_STORE, EPI_ADD, EPI_SWIGLU = 0, 1, 2
 TILES = {112: (128, 32), 124: (128, 64), 184: (256, 64), 122: (128, 128), 142: (256, 128), 188: (256, 256), 123: (128, 128),
-         168: (192, 256), 164: (96, 64)}
+         168: (192, 256), 164: (96, 64), 186: (256, 192)}
 
 
 @pytest.fixture(scope="module")

@@ -168,12 +168,15 @@ def test_gemm_mfma_swiglu_tiles_with_three_pieces_a_wave(M, I, K, tile):
 
 
 @pytest.mark.parametrize("M,N,K,cut", [(300, 256, 128, -128), (257, 96, 64, -256), (530, 512, 256, -256), (129, 64, 64, -128),
-                                       (2049, 512, 128, 0)])
+                                       (2049, 512, 128, 0), (2060, 4096, 4096, 0)])
 def test_gemm_mfma_rows_cut_into_two_products(M, N, K, cut):
     """A product cut in two along its rows (whole tiles, then the rest, each a product of its own;
-    by name, and at the last size by the kernel's own estimates): store, add and SwiGLU give what
-    the product whole gives, and nothing beyond the rows is written."""
+    by name, and at the last sizes by the kernel's own estimates, which cut the 8B shape's products
+    of 2,060 rows at 2,048): store, add and SwiGLU give what the product whole gives, and nothing
+    beyond the rows is written."""
     from herbert_rs_amd.kernels import mfma
+    if (M, N, K) == (2060, 4096, 4096):
+        assert mfma.gemm_split(M, N, K, mfma.EPI_ADD) == 2048 and mfma.gemm_split(M, N, K, mfma.EPI_STORE) == 2048
     a = rand(M, K, seed=30, dtype=torch.bfloat16, scale=0.5)
     w = rand(N, K, seed=31, dtype=torch.bfloat16, scale=0.3)
     want = a.double() @ w.double().T
@@ -715,7 +718,7 @@ def test_gemm_mfma_refuses_a_handed_norm_it_cannot_do():
 
 # every tile with every size it takes (K in steps of 32 goes to the host's own choice and to tile 123 only)
 TILE_CASES = [(tile, M, N, K, packed)
-              for tile in (0, 188, 142, 122, 123, 112, 124, 184)
+              for tile in (0, 188, 142, 186, 122, 123, 112, 124, 184)
               for M, N, K, packed in [(65, 128, 64, True), (200, 336, 192, True), (300, 530, 96, False),
                                       (513, 1040, 256, True), (2300, 528, 128, True), (17, 272, 64, True),
                                       (40, 530, 320, False), (64, 1040, 128, True)]
@@ -754,7 +757,7 @@ def _slices_fit(tile, K):
 
 
 SLICE_CASES = [(tile, M, N, K, packed)
-               for tile in (0, 2122, 4188, 3142, 8122, 4112, 16124, 2184)
+               for tile in (0, 2122, 4188, 3142, 2186, 8122, 4112, 16124, 2184)
                for M, N, K, packed in [(200, 336, 512, True), (513, 1040, 768, True), (128, 1024, 4096, True),
                                        (300, 530, 1024, False), (24, 1056, 2112, True), (64, 8192, 1024, True),
                                        (33, 336, 4096, False)]

@@ -6,7 +6,7 @@ bin/trace_run in bfloat16 and in float32: prompts of 2,048, 1,024 and 512 tokens
 that norms, rotates and writes the cache itself, on each of its three tile shapes; gate/up on tiles
 of 256 and of 192 columns), decoding at batch 1, 8 and 64 with the kernels the
 host picks for these widths by itself, and batches of unequal lengths that follow one another
-in slots that were used before (the first brings 1,044 rows in one step: a product cut along its rows). Nothing is patched: what runs here is what bench.py times.
+in slots that were used before. Nothing is patched: what runs here is what bench.py times.
 """
 import numpy as np
 import pytest
@@ -110,9 +110,8 @@ def test_the_host_picks_the_profiled_kernels_for_these_widths():
     # wide and 128 or 256 rows high; 256 tokens are too few for a fused q/k/v product
     assert plan(512, 2 * I, H, SWIGLU) == 168 and plan(1024, 2 * I, H, SWIGLU) == 168
     assert [mfma.qkv_tile_shape(m, Q) for m in (256, 512, 1024, 2048)] == [None, 2, 1, 0]
-    # rows that end just past whole tiles are cut off as a product of their own: the batch of 8 prompts
-    # below brings 1,044 rows, of which the down product takes 1,024 first; 2,048 rows are never cut
-    assert mfma.gemm_split(1044, H, I, ADD) == 1024 and mfma.gemm_split(2048, H, I, ADD) == 0
+    # rows that end just past whole tiles are cut off as a product of their own; 2,048 rows are never cut
+    assert mfma.gemm_split(2048, H, I, ADD) == 0 and mfma.gemm_split(2048, 2 * I, H, SWIGLU) == 0
     assert mfma.gemm_split(2049, 2 * I, H, SWIGLU) == 2048 and mfma.gemm_split(2049, H, H, ADD) == 2048
 
 
