@@ -267,8 +267,17 @@ gemm_skinny_kernel(const void* __restrict__ Xv, const bf16* __restrict__ W, void
 #pragma unroll
         for (int j = 0; j < HP; ++j)     // past the end the last part was read once more: left out here
             handed += hp_first + j * hp_step < hand.scale_parts ? hp[j] : 0.f;
-        for (int p = hp_first + HP * hp_step; p < hand.scale_parts; p += hp_step)
-            handed += hand.scale_partial[(size_t)p * MP + (lane & (MP - 1))];
+        // (what lies beyond the first HP parts of a thread, for long rows: asked for HP at a time too)
+        for (int base = hp_first + HP * hp_step; base < hand.scale_parts; base += HP * hp_step) {
+            float more[HP];
+#pragma unroll
+            for (int j = 0; j < HP; ++j) {
+                const int p = base + j * hp_step;
+                more[j] = hand.scale_partial[(size_t)(p < hand.scale_parts ? p : hand.scale_parts - 1) * MP + (lane & (MP - 1))];
+            }
+#pragma unroll
+            for (int j = 0; j < HP; ++j) handed += base + j * hp_step < hand.scale_parts ? more[j] : 0.f;
+        }
         for (int d = 32; d >= MP; d >>= 1) handed += __shfl_xor(handed, d, 64);   // lanes of the same row
         if (lane < MP) handed_of_wave[wave * 16 + lane] = handed;    // read by wave 0 after the tree's barriers
     }
@@ -973,19 +982,21 @@ gemm_tile_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, void* _
     float* const row_sums = (float*)(xlds + XST * X_STAGE);       // [NW][16]
     const int MP = M <= 1 ? 1 : (M <= 2 ? 2 : (M <= 4 ? 4 : (M <= 8 ? 8 : 16)));
     if (scale.partial) {
-        constexpr int HP = 8;
-        float hp[HP];
+        // (asked for HP at a time: one after another, as a plain loop over the parts does it, every
+        // part costs a trip to the L2; with 16 rows and 256 parts that were eight trips, 8 us)
+        constexpr int HP = 16;
         const int first = tid / MP, stride = 64 * NW / MP;
-#pragma unroll
-        for (int j = 0; j < HP; ++j) {
-            const int p = first + j * stride;
-            hp[j] = scale.partial[(size_t)(p < scale.parts ? p : scale.parts - 1) * MP + (lane & (MP - 1))];
-        }
         float sum = 0.f;
+        for (int base = first; base < scale.parts; base += HP * stride) {
+            float hp[HP];
 #pragma unroll
-        for (int j = 0; j < HP; ++j) sum += first + j * stride < scale.parts ? hp[j] : 0.f;
-        for (int p = first + HP * stride; p < scale.parts; p += stride)
-            sum += scale.partial[(size_t)p * MP + (lane & (MP - 1))];
+            for (int j = 0; j < HP; ++j) {
+                const int p = base + j * stride;
+                hp[j] = scale.partial[(size_t)(p < scale.parts ? p : scale.parts - 1) * MP + (lane & (MP - 1))];
+            }
+#pragma unroll
+            for (int j = 0; j < HP; ++j) sum += base + j * stride < scale.parts ? hp[j] : 0.f;
+        }
         for (int d = 32; d >= MP; d >>= 1) sum += __shfl_xor(sum, d, 64);
         if (lane < MP) row_sums[wave * 16 + lane] = sum;
     }
