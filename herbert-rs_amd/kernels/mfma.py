@@ -410,7 +410,19 @@ def _decode_split(meta, nkv, window):
     if window:
         span = min(span, (window + 63) // 64 + 1)
     pairs = meta.num_seqs * nkv
-    if 2 * pairs >= DECODE_WAVES:      # two waves a CU already: a merge would cost more than it gains
+    if 2 * pairs >= DECODE_WAVES:
+        # Two waves a CU already: a merge costs more than it gains (5 to 8 % of a step), as long as
+        # the waves sit evenly. A wave that reads a whole context is a long job, and the time goes
+        # with the CU that has the most of them (three where most have two: 65 sequences took a
+        # quarter longer than 64) or, beyond what the GPU holds at a time, with the last round
+        # (160 sequences: two rounds for one and a quarter). Where the most is 1.3 times the mean
+        # or more, eight ranges (four for contexts under 2 K tokens, none under 1 K) even that out:
+        # 7 % off at 65 sequences, 10 to 12 % at 136 to 160.
+        unit = max(1, DECODE_WAVES // 4) if pairs <= DECODE_WAVES else DECODE_WAVES     # what fills evenly
+        fine = min(8, span // 4)
+        if -(-pairs // unit) >= 1.3 * pairs / unit and fine >= 4:
+            per = -(-span // fine)
+            return -(-span // per), per
         return 1, span
     # the merge's cost grows with the ranges: more than 32 only where each still has four pages
     most = max(1, min(span, max(32, min(128, span // 4))))

@@ -113,3 +113,27 @@ def test_rows_just_past_whole_tiles_are_cut_off_as_a_product_of_their_own():
             for ws in (0, W):
                 rows = split(M, N, K, epi, ws)
                 assert rows == 0 or (0 < rows < M and rows % 128 == 0 and M - rows < 256), (M, N, K, epi, rows)
+
+
+def test_decode_attention_ranges_by_how_evenly_the_waves_sit():
+    """One range a (sequence, kv head) from 512 of them on, unless the waves would sit unevenly on
+    the CUs (three on some where most have two, or a second round that is a quarter full): then
+    eight shorter ranges; below, as many ranges as fill one round of 1,024 waves."""
+    from herbert_rs_amd.kernels import mfma
+
+    class Meta:
+        def __init__(self, seqs, tokens):
+            self.num_seqs, self.context_bucket = seqs, tokens
+    split = lambda b, t=4096, nkv=8, window=0: mfma._decode_split(Meta(b, t), nkv, window)
+    assert split(1) == (32, 2) and split(8) == (16, 4) and split(32) == (4, 16) and split(48) == (2, 32)
+    for b in (64, 80, 96, 128, 200, 256):
+        assert split(b) == (1, 64), b
+    for b in (65, 72, 136, 160):
+        assert split(b) == (8, 8), b
+    assert split(65, 1024) == (4, 4) and split(65, 512) == (1, 8)
+    assert split(65, 4096, window=100) == (1, 3)
+    for b in range(1, 300, 7):
+        for t in (64, 700, 4096, 32768):
+            ranges, per = split(b, t)
+            span = -(-t // 64)
+            assert ranges >= 1 and per >= 1 and ranges * per >= span > (ranges - 1) * per, (b, t)

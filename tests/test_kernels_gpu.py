@@ -328,6 +328,24 @@ def test_attention_mfma_decode(nq, nkv, hd, window, lengths, waves, monkeypatch)
     assert float((out.float().cpu() - want).abs().max()) <= 2 ** -7 * float(want.abs().max())
 
 
+def test_attention_mfma_decode_of_many_sequences_in_shorter_ranges():
+    """70 sequences on 8 kv heads are 560 waves of one range each: three on some CUs where most have
+    two. The host then cuts every context into shorter ranges (here six) with a merge, as it does
+    for few sequences; with 64 sequences, which sit evenly, every sequence stays one range."""
+    from herbert_rs_amd.kernels import mfma
+    nq, nkv, hd = 16, 8, 128
+    lengths = [1100 + (37 * i) % 230 for i in range(70)]
+    meta, kv, dense = paged_case(lengths, [1] * len(lengths), nkv, hd, torch.bfloat16, seed=5, n_pages=70 * 21 + 8)
+    assert mfma._decode_split(meta, nkv, 0)[0] == 6
+    q = rand(len(lengths), nq * hd, seed=26, dtype=torch.bfloat16)
+    out = torch.full_like(q, 9.0)
+    mfma.attention(q, meta, kv, out, nq, nkv, hd, hd ** -0.5, 0)
+    want = attention_reference(q, meta, dense, nq, nkv, hd, hd ** -0.5, 0)
+    assert float((out.float().cpu() - want).abs().max()) <= 2 ** -7 * float(want.abs().max())
+    meta64, _, _ = paged_case(lengths[:64], [1] * 64, nkv, hd, torch.bfloat16, seed=5, n_pages=64 * 21 + 8)
+    assert mfma._decode_split(meta64, nkv, 0)[0] == 1
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("nq,nkv,hd,rot,norm", [(4, 2, 128, 128, True), (3, 1, 64, 64, False), (2, 2, 96, 0, True),
                                                 (5, 1, 32, 32, True), (2, 1, 80, 40, True), (1, 1, 256, 256, True),
