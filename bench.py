@@ -152,6 +152,9 @@ def main():
                     help="feed the prompt of the prefill figure in steps of this many tokens (0: in one step)")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run the 2,048-token prefill alone (for profiles); prints no JSON line")
+    ap.add_argument("--contexts", default=None,
+                    help="decode one batch whose sequences hold these numbers of tokens (comma-separated, "
+                         "e.g. 32768,1024,1024: unequal lengths); prints ms a step and GB/s, no JSON line")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU only: --gpus {args.gpus} is not supported (this library "
@@ -170,6 +173,9 @@ def main():
     from herbert_rs_amd.sampling.sampler import Sampler
 
     shape = load_shape()
+    unequal = [int(c) for c in args.contexts.split(",")] if args.contexts else None
+    if unequal:
+        args.context, args.batch, args.no_points = max(unequal), len(unequal), True
     context = args.context or shape.pop("context")
     shape.pop("context", None)
     layers_full = shape["num_hidden_layers"]
@@ -181,6 +187,8 @@ def main():
     torch.cuda.set_device(0)
     max_batch = args.batch if args.no_points else max(args.batch, 64)
     cache_tokens = max(max_batch * (context + 64), args.prefill_tokens + 64)
+    if unequal:
+        cache_tokens = sum((c + 127) // 64 * 64 for c in unequal)
     t0 = time.time()
     engine = hb.Engine.from_config(cfg, seed=2, dtype=args.dtype, std=0.02, norm_std=0.0,
                                    max_tokens=cache_tokens, max_slots=max_batch)
@@ -263,6 +271,33 @@ def main():
         torch.cuda.synchronize()
         return (time.perf_counter() - t) / reps
 
+    if unequal:
+        # one batch of sequences of these lengths (after the timed steps), decoded as the loop does
+        if min(unequal) <= args.steps + args.warmup:
+            raise ValueError(f"every sequence of --contexts needs more than {args.steps + args.warmup} tokens")
+        slots = [engine.alloc_slot() for _ in unequal]
+        for s, c in zip(slots, unequal):
+            fill = c - args.steps - args.warmup
+            for a in range(0, fill, 2048):
+                engine.step([StepEntry(s, ids(min(2048, fill - a)), [])])
+        chooser = Sampler(SamplingParams(temperature=0.0), len(slots), V, engine.device)
+        ahead = chooser.choose_ahead(engine.step([StepEntry(s, ids(1), [0]) for s in slots]), range(len(slots)))
+        for n in (args.warmup - 1, args.steps):
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            for _ in range(n):
+                logits = engine.step([StepEntry(s, [0], [0]) for s in slots], tokens_on_device=ahead.device)
+                before, ahead = ahead, chooser.choose_ahead(logits, range(len(slots)))
+                chooser.read(before)
+            torch.cuda.synchronize()
+            ms = (time.perf_counter() - t) / max(1, n) * 1e3
+        held = sum(unequal) - len(unequal) * args.steps / 2.0
+        gbs = (weight_bytes + held * kv_bytes_per_token) / (ms * 1e-3) / 1e9
+        print(f"[bench] decode of {len(unequal)} sequences holding {args.contexts} tokens: {ms:.3f} ms a step, "
+              f"{len(unequal) / ms * 1e3:.0f} tok/s, {gbs:.0f} GB/s of {HBM_GBS:.0f} "
+              f"(weights {weight_bytes / 1e9:.2f} GB + keys and values {held * kv_bytes_per_token / 1e9:.2f} GB)",
+              file=sys.stderr, flush=True)
+        return 0
     if args.prefill_only:
         sec = prefill_run(args.prefill_tokens, max(1, args.steps))
         print(f"[bench] prefill {args.prefill_tokens}: {args.prefill_tokens / sec:.0f} tok/s, {sec * 1e3:.2f} ms",

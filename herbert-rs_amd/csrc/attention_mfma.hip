@@ -647,10 +647,27 @@ attn_decode_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_cache, bf16*
                    float* __restrict__ partial_o, float* __restrict__ partial_ml,
                    const int* __restrict__ context_lens, const int* __restrict__ slots,
                    const int* __restrict__ page_table, int max_pages, int nq, int nkv, float c, int window,
-                   int pages_per_split, DecodeFusion fu, bf16* __restrict__ out) {
-    const int b = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z, splits = gridDim.z;
-    const int G = nq / nkv;
+                   int pages_per_split, DecodeFusion fu, bf16* __restrict__ out,
+                   const int* __restrict__ ranges, int n_seqs) {
+    // ranges == null: the grid is (sequence, kv head, range), every sequence cut into gridDim.z
+    // ranges of pages_per_split pages (those past a sequence's end hold nothing).
+    // ranges != null (sequences of unequal lengths, at most 64): the grid is (1, kv head, item);
+    // ranges[0 .. n_seqs] count the ranges of the sequences before each one, ranges[n_seqs + 1] is
+    // the pages of a range: item i is range i - ranges[b] of the sequence b whose count it falls
+    // into, and items from ranges[n_seqs] on are nothing. The partial results are then laid out
+    // [head, item]: those of one sequence and head lie side by side.
+    const int kvh = blockIdx.y, splits = gridDim.z;
     const int lane = threadIdx.x, c32 = lane & 31, g2 = lane >> 5;
+    int b = blockIdx.x, split = blockIdx.z;
+    if (ranges) {
+        const int item = blockIdx.z;
+        const int upto = lane < n_seqs ? ranges[lane + 1] : 0x7fffffff;
+        b = __builtin_amdgcn_readfirstlane(__popcll(__ballot(upto <= item)));     // sequences wholly before the item
+        if (b >= n_seqs) return;
+        split = item - ranges[b];
+        pages_per_split = ranges[n_seqs + 1];
+    }
+    const int G = nq / nkv;
     const int ctx = context_lens[b];                 // keys 0 .. ctx-1; the query sits at ctx-1
     const int hi = ctx - 1;
     const int lo = (window > 0 && ctx > window) ? ctx - window : 0;
@@ -878,7 +895,8 @@ attn_decode_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_cache, bf16*
         return;
     }
     if (c32 < G) {
-        const size_t base = ((size_t)b * nq + kvh * G + c32) * splits + split;
+        const size_t base = ranges ? (size_t)(kvh * G + c32) * splits + blockIdx.z
+                                   : ((size_t)b * nq + kvh * G + c32) * splits + split;
         if (g2 == 0) {
             partial_ml[base * 2] = m;        // -inf when this range held no visible key
             partial_ml[base * 2 + 1] = l;
@@ -901,7 +919,7 @@ attn_decode_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_cache, bf16*
 template <int HD>
 __global__ void __launch_bounds__(256)
 attn_decode_merge_kernel(const float* __restrict__ partial_o, const float* __restrict__ partial_ml,
-                         bf16* __restrict__ out, int splits, float c) {
+                         bf16* __restrict__ out, int splits, float c, const int* __restrict__ ranges, int nq) {
     // thread = (group of ranges, 4 consecutive d): it adds up the weighted partial sums of the ranges
     // g, g + GROUPS, ... once the first wave has worked out the weights; the groups are then added
     // in order through LDS. (Asking for the partial sums before the weights are known gains nothing:
@@ -913,8 +931,16 @@ attn_decode_merge_kernel(const float* __restrict__ partial_o, const float* __res
     __shared__ float s_inv;
     const int tid = threadIdx.x;
     const size_t bh = blockIdx.x;
-    const float* ml = partial_ml + bh * splits * 2;
     const int chunk = tid % CHUNKS, grp = tid / CHUNKS;
+    // the first partial result of this sequence and head (with a list of ranges, see
+    // attn_decode_kernel: [head, item], and the sequence has its own count of them)
+    size_t first = bh * splits;
+    if (ranges) {
+        const int b = bh / nq, h = bh % nq;
+        first = (size_t)h * splits + ranges[b];
+        splits = ranges[b + 1] - ranges[b];
+    }
+    const float* ml = partial_ml + first * 2;
 
     if (tid < 64) {
         float M = -INFINITY;
@@ -940,7 +966,7 @@ attn_decode_merge_kernel(const float* __restrict__ partial_o, const float* __res
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
     if (grp < GROUPS)
         for (int s = grp; s < splits; s += GROUPS) {
-            const f32x4 v = *(const f32x4*)(partial_o + (bh * splits + s) * HD + chunk * 4);
+            const f32x4 v = *(const f32x4*)(partial_o + (first + s) * HD + chunk * 4);
             acc += v * wgt[s];
         }
     if (grp < GROUPS) {
@@ -1014,7 +1040,12 @@ extern "C" int hb_attn_decode_mfma(const void* q, void* k_cache, void* v_cache, 
                                    int B, int nq, int nkv, int hd, float scale, int window, int splits,
                                    int pages_per_split, const float* qkv, const float* q_norm_w,
                                    const float* k_norm_w, const float* cos_t, const float* sin_t, float eps,
-                                   int write_kv, int qkv_slices, size_t slice_stride, hipStream_t stream) {
+                                   int write_kv, int qkv_slices, size_t slice_stride, const int* ranges,
+                                   hipStream_t stream) {
+    // ranges != null: see attn_decode_kernel; `splits` is then the number of items of the grid (the
+    // partial results are [nq, splits]), pages_per_split is not read
+    HB_REQUIRE(!ranges || (B >= 2 && B <= 64 && splits >= 2 && window == 0),
+               "attn_decode: a list of ranges is for 2 to 64 sequences, with a merge, without a window");
     HB_REQUIRE(B > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attn_decode: bad sizes");
     HB_REQUIRE(page_size == PAGE, "attn_decode: pages must hold %d tokens", PAGE);
     HB_REQUIRE(nq / nkv <= 32, "attn_decode: more than 32 query heads share a kv head");
@@ -1024,14 +1055,14 @@ extern "C" int hb_attn_decode_mfma(const void* q, void* k_cache, void* v_cache, 
     HB_REQUIRE(qkv_slices == 1 || (qkv && hd == 128 && (qkv_slices == 2 || qkv_slices == 4 || qkv_slices == 8) &&
                                    slice_stride >= (size_t)B * (nq + 2 * nkv) * hd),
                "attn_decode: %d slices of the projection are not taken here", qkv_slices);
-    dim3 grid(B, nkv, splits);
+    dim3 grid(ranges ? 1 : B, nkv, splits);
     const float c = scale * LOG2E;
     const DecodeFusion fu = {qkv, q_norm_w, k_norm_w, cos_t, sin_t, eps, write_kv, slice_stride};
     bf16* const direct = splits == 1 ? (bf16*)out : nullptr;      // one range: the kernel writes the output itself
     HB_REQUIRE(qkv || q, "attn_decode: neither q nor the projection rows are given");
     HB_REQUIRE((cos_t == nullptr) == (sin_t == nullptr), "attn_decode: cos and sin tables come together");
 #define DECODE_ARGS(QPTR) QPTR, (bf16*)k_cache, (bf16*)v_cache, partial_o, partial_ml, context_lens, slots, \
-                          page_table, max_pages, nq, nkv, c, window, pages_per_split, fu, direct
+                          page_table, max_pages, nq, nkv, c, window, pages_per_split, fu, direct, ranges, B
 #define LAUNCH_DECODE(HDV) do {                                                                          \
     if (qkv)                                                                                             \
         attn_decode_kernel<HDV, true><<<grid, 64, 0, stream>>>(DECODE_ARGS(nullptr));                    \
@@ -1050,7 +1081,7 @@ extern "C" int hb_attn_decode_mfma(const void* q, void* k_cache, void* v_cache, 
 #undef DECODE_ARGS
     HB_CHECK_LAUNCH("attn_decode");
     if (!direct) {
-#define LAUNCH_MERGE(HDV) attn_decode_merge_kernel<HDV><<<B * nq, 256, 0, stream>>>(partial_o, partial_ml, (bf16*)out, splits, c)
+#define LAUNCH_MERGE(HDV) attn_decode_merge_kernel<HDV><<<B * nq, 256, 0, stream>>>(partial_o, partial_ml, (bf16*)out, splits, c, ranges, nq)
         if (hd == 32) LAUNCH_MERGE(32);
         else if (hd == 64) LAUNCH_MERGE(64);
         else LAUNCH_MERGE(128);

@@ -39,6 +39,53 @@ class BatchMeta:
     host_context: np.ndarray
     derived: dict = None       # what kernels' host sides derive once a step (tile lists and the like)
     context_bucket: int = 0    # max_context rounded up to CONTEXT_BUCKET: sizes the decode kernels' grids
+    unequal: bool = False      # the contexts fill at most 0.55 of num_seqs x max_context (see is_unequal)
+    static: object = None      # the StaticDecodeMeta whose buffers these are, if any
+
+    def ranges_for(self, items, unit):
+        """The list that cuts this step's contexts into at most `items` ranges of equally many whole
+        units of `unit` positions (see range_list), as int32 [num_seqs + 2] on the GPU; None if a
+        step with fixed buffers has no room for another list. A step with fixed buffers refills the
+        lists it has handed out at every update."""
+        key = ("ranges", int(items), int(unit))
+        got = self.derived.get(key)
+        if got is None:
+            if self.static is not None:
+                got = self.static.add_range_list(int(items), int(unit))
+                if got is None:
+                    return None
+            else:
+                got = torch.from_numpy(range_list(self.host_context, items, unit)).to(self.token_ids.device)
+            self.derived[key] = got
+        return got
+
+
+def is_unequal(context):
+    """True where the sequences of a step together hold at most 0.55 of what they would if all were
+    as long as the longest: a kernel that gives every sequence the same share of the GPU then leaves
+    much of it idle. (Measured on decode steps of the 8B shape: dealing the attention's grid out by
+    a list takes 7 to 11 % off a step at 0.34 to 0.51 and 23 to 54 % at 0.08 to 0.18, nothing
+    from 0.56 on, and adds 2 to 4 % where all are equal.)"""
+    context = np.asarray(context, dtype=np.int64)
+    return len(context) > 1 and 20 * int(context.sum()) <= 11 * len(context) * int(context.max())
+
+
+def range_list(context, items, unit):
+    """Cut B sequences of unequal lengths into ranges of equally many whole units (pages), at most
+    `items` of them together (items > B): int32 [B + 2] with [0 .. B] the number of ranges of the
+    sequences before each one and [B + 1] the units of a range. Every sequence gets the ranges that
+    cover its units: sum ceil(p / per) < sum p / per + B <= items for per >= sum p / (items - B)."""
+    context = np.asarray(context, dtype=np.int64)
+    B = len(context)
+    if items <= B:
+        raise ValueError(f"{items} ranges cannot be dealt out to {B} sequences")
+    units = np.maximum(1, -(-context // unit))
+    per = max(1, int(-(-units.sum() // (items - B))))
+    out = np.empty(B + 2, dtype=np.int32)
+    out[0] = 0
+    np.cumsum(-(-units // per), out=out[1:B + 1])
+    out[B + 1] = per
+    return out
 
 
 CONTEXT_BUCKET = 256
@@ -88,18 +135,22 @@ def pack(entries, start_lengths, device, staging=None):
         context_lens=dev[o + 2 * B + 1:o + 3 * B + 1], want_rows=dev[o + 3 * B + 1:o + 3 * B + 1 + R],
         num_tokens=T, num_seqs=B, max_new=max(counts), max_context=int(ctx.max()),
         max_position=int(pos.max()), host_starts=starts.copy(), host_context=ctx.copy(), derived={},
-        context_bucket=bucket(int(ctx.max())))
+        context_bucket=bucket(int(ctx.max())), unequal=is_unequal(ctx))
 
 
 class StaticDecodeMeta:
     """The metadata of a step of B sequences with one token each, every logit wanted, in buffers
     that stay where they are: a captured graph reads them, `update` refills them."""
 
+    RANGE_LISTS = 4      # lists of ranges (BatchMeta.ranges_for) that the buffers have room for
+
     def __init__(self, batch_size, device):
         B = self.batch_size = batch_size
-        self.host = torch.empty(7 * B + 1, dtype=torch.int32, pin_memory=True)
+        size = 7 * B + 1 + self.RANGE_LISTS * (B + 2)
+        self.host = torch.zeros(size, dtype=torch.int32, pin_memory=torch.device(device).type == "cuda")
         self.copied = None       # event after the last copy out of `host`
-        self.dev = torch.zeros(7 * B + 1, dtype=torch.int32, device=device)
+        self.dev = torch.zeros(size, dtype=torch.int32, device=device)
+        self.range_lists = []    # (items, unit) of the lists handed out, in the order of their places
         h = self.host_array = self.host.numpy()
         h[2 * B:3 * B] = np.arange(B)            # seq_of
         h[4 * B:5 * B + 1] = np.arange(B + 1)    # seq_starts
@@ -110,7 +161,25 @@ class StaticDecodeMeta:
             seq_starts=d[4 * B:5 * B + 1], context_lens=d[5 * B + 1:6 * B + 1],
             want_rows=d[6 * B + 1:7 * B + 1], num_tokens=B, num_seqs=B, max_new=1, max_context=0,
             max_position=0, host_starts=np.arange(B + 1, dtype=np.int32),
-            host_context=np.zeros(B, dtype=np.int32), derived={}, context_bucket=0)
+            host_context=np.zeros(B, dtype=np.int32), derived={}, context_bucket=0, static=self)
+
+    def _range_place(self, i):
+        first = 7 * self.batch_size + 1 + i * (self.batch_size + 2)
+        return slice(first, first + self.batch_size + 2)
+
+    def add_range_list(self, items, unit):
+        """A place in the buffers for the list (items, unit), filled for the step at hand and from
+        now on at every update; None if all places are taken. Not under graph capture: the list is
+        copied to the GPU here, so a step's first, eager run has to be the one that asks."""
+        if len(self.range_lists) == self.RANGE_LISTS:
+            return None
+        if self.dev.is_cuda and torch.cuda.is_current_stream_capturing():
+            raise RuntimeError("a list of ranges is first asked for while a graph is captured")
+        place = self._range_place(len(self.range_lists))
+        self.range_lists.append((items, unit))
+        self.host_array[place] = range_list(self.meta.host_context, items, unit)
+        self.dev[place].copy_(self.host[place])
+        return self.dev[place]
 
     def update(self, entries, start_lengths):
         B = self.batch_size
@@ -122,6 +191,8 @@ class StaticDecodeMeta:
         h[3 * B:4 * B] = [e.slot for e in entries]
         context = h[5 * B + 1:6 * B + 1]
         np.add(h[B:2 * B], 1, out=context)
+        for i, (items, unit) in enumerate(self.range_lists):
+            h[self._range_place(i)] = range_list(context, items, unit)
         self.dev.copy_(self.host, non_blocking=True)
         if self.dev.is_cuda:
             if self.copied is None:
@@ -132,4 +203,5 @@ class StaticDecodeMeta:
         m.max_context = int(max(start_lengths)) + 1
         m.max_position = m.max_context - 1
         m.context_bucket = bucket(m.max_context)
+        m.unequal = is_unequal(context)
         return m

@@ -34,7 +34,7 @@ class _DecodeState:
     def __init__(self, static, logits):
         self.static = static
         self.logits = logits
-        self.seen = {}          # context bucket -> eager steps run
+        self.seen = {}          # (context bucket, unequal) -> eager steps run
 
 
 # Captured graphs kept at any time, over all batch sizes and context buckets; the least recently
@@ -71,7 +71,7 @@ class Engine:
         self.steps_run = 0
         self.use_graphs = bool(use_graphs) and self.model.graph_safe
         self._decode = OrderedDict()    # batch size -> _DecodeState, least recently used first
-        self._graphs = OrderedDict()    # (batch size, context bucket) -> graph, least recently used first
+        self._graphs = OrderedDict()    # (batch size, context bucket, unequal) -> graph, least recently used first
         self.graphs_captured = 0
         self.ignored_tensors = []       # stored tensors that the model did not ask for
         self._tensor_source = None      # how get_tensor finds a tensor again: set by the constructors below
@@ -226,8 +226,9 @@ class Engine:
         """One token for each sequence, every logit wanted: the launch-bound case. The step's
         metadata lives in fixed buffers; from the second step of a shape on, the forward pass is a
         captured HIP graph that is replayed, so that the host launches one graph and not hundreds
-        of kernels. A graph is tied to the batch size and to the bucket of the longest context
-        (which sizes the attention grid). All graphs of a batch size write their logits into that
+        of kernels. A graph is tied to the batch size, to the bucket of the longest context
+        (which sizes the attention grid) and to whether the contexts are of very unequal lengths
+        (the attention then deals its grid out by a list). All graphs of a batch size write their logits into that
         size's one buffer: what a step returns is overwritten by the next decode step of the same
         batch size. At most MAX_GRAPHS graphs and MAX_DECODE_BATCH_SIZES batch sizes are kept,
         the least recently used go first."""
@@ -245,14 +246,14 @@ class Engine:
         meta = state.static.update(entries, starts)
         if tokens_on_device is not None:
             meta.token_ids.copy_(tokens_on_device)      # behind the copy from the host, before the graph
-        key = (B, meta.context_bucket)
+        key = (B, meta.context_bucket, meta.unequal)
         graph = self._graphs.get(key)
         if graph is not None:
             self._graphs.move_to_end(key)
             graph.replay()
             return state.logits
-        seen = state.seen.get(key[1], 0)
-        state.seen[key[1]] = seen + 1
+        seen = state.seen.get(key[1:], 0)
+        state.seen[key[1:]] = seen + 1
         if seen == 0:       # eager: also sizes every scratch buffer
             return self.model.forward(self.rt, meta, self.cache, logits_out=state.logits)
         torch.cuda.synchronize(self.device)      # also: no graph that is dropped below still runs

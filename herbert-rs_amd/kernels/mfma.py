@@ -342,7 +342,7 @@ def gemm_swiglu(a, w_interleaved, out, packed=False, norm=None, tile=0, row_scal
 lib.register_signatures("attention_mfma", {
     "hb_attn_prefill_mfma": [_P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I, _P],
     "hb_attn_decode_mfma": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I,
-                            _P, _P, _P, _P, _P, _F, _I, _I, ctypes.c_size_t, _P],
+                            _P, _P, _P, _P, _P, _F, _I, _I, ctypes.c_size_t, _P, _P],
 })
 
 ATTENTION_HEAD_DIMS = (32, 64, 128)
@@ -435,6 +435,23 @@ def _decode_split(meta, nkv, window):
     return best
 
 
+def _decode_ranges(meta, nkv, window):
+    """(items of the grid, list of ranges on the GPU) for a step whose contexts are of very unequal
+    lengths, else None. Equal shares would leave the waves of the short sequences with nothing and
+    those of the long ones with all the work (one sequence of 32 K tokens beside seven of 1 K: 128 of
+    1,024 waves read 2 K tokens each); with the list every wave has a range of the same length of
+    whichever sequence, as many ranges as the GPU holds waves at a time. The list changes with
+    every step and is read by the kernel; the grid does not change."""
+    B = meta.num_seqs
+    if not meta.unequal or window or not 2 <= B <= 64 or meta.max_new != 1:
+        return None
+    items = min(1024, DECODE_WAVES // nkv)
+    if items < 2 * B:
+        return None
+    listed = meta.ranges_for(items, 64)
+    return None if listed is None else (items, listed)
+
+
 def _partial_buffers(device, n_rows, splits, hd):
     """(partial outputs, partial max / sum) of the decode kernel's ranges. Buffers that were handed
     out are kept for good, also when larger ones replace them: a captured graph may hold their
@@ -488,8 +505,13 @@ def attention_decode_fused(qkv, q_norm_w, k_norm_w, cos, sin, meta, kv, out, nq,
         if meta.max_position >= cos.shape[0]:
             raise BackendError(f"position {meta.max_position} beyond the rotation table ({cos.shape[0]} rows)")
     window = int(window or 0)
-    splits, per = _decode_split(meta, nkv, window)
-    po, pml = _partial_buffers(qkv.device, B * nq, splits, hd)
+    listed = _decode_ranges(meta, nkv, window)
+    if listed:
+        (splits, ranges), per = listed, 1
+        po, pml = _partial_buffers(qkv.device, nq, splits, hd)
+    else:
+        (splits, per), ranges = _decode_split(meta, nkv, window), None
+        po, pml = _partial_buffers(qkv.device, B * nq, splits, hd)
     n_slices, src, stride = qkv_slices if qkv_slices is not None else (1, qkv.data_ptr(), 0)
     if n_slices > 1 and (n_slices not in DEFERRED_SLICES or hd != 128 or stride < qkv.numel()):
         raise BackendError(f"fused decode attention does not add up {n_slices} slices of the projection")
@@ -498,7 +520,8 @@ def attention_decode_fused(qkv, q_norm_w, k_norm_w, cos, sin, meta, kv, out, nq,
              kv.page_table.data_ptr(), kv.page_table.shape[1], kv.page_size, B, nq, nkv, hd, float(scale),
              window, splits, per, src, None if q_norm_w is None else q_norm_w.data_ptr(),
              None if k_norm_w is None else k_norm_w.data_ptr(), None if cos is None else cos.data_ptr(),
-             None if sin is None else sin.data_ptr(), float(eps), 1, n_slices, stride, _stream())
+             None if sin is None else sin.data_ptr(), float(eps), 1, n_slices, stride,
+             None if ranges is None else ranges.data_ptr(), _stream())
 
 
 DEFERRED_SLICES = (2, 4, 8)     # numbers of slices of the projection that the decode kernel adds up itself
@@ -523,13 +546,18 @@ def attention(q, meta, kv, out, nq, nkv, hd, scale, window, tile_height=None):
         if T != meta.num_seqs:
             raise BackendError("decode attention needs one token for each sequence")
         _check(meta.context_lens, "context_lens", torch.int32, (T,))
-        splits, per = _decode_split(meta, nkv, window)
-        po, pml = _partial_buffers(q.device, T * nq, splits, hd)
+        listed = _decode_ranges(meta, nkv, window)
+        if listed:
+            (splits, ranges), per = listed, 1
+            po, pml = _partial_buffers(q.device, nq, splits, hd)
+        else:
+            (splits, per), ranges = _decode_split(meta, nkv, window), None
+            po, pml = _partial_buffers(q.device, T * nq, splits, hd)
         lib.call("attention_mfma", "hb_attn_decode_mfma", q.data_ptr(), kv.k.data_ptr(), kv.v.data_ptr(),
                  out.data_ptr(), po.data_ptr(), pml.data_ptr(), meta.context_lens.data_ptr(),
                  meta.slots.data_ptr(), kv.page_table.data_ptr(), kv.page_table.shape[1], kv.page_size,
                  T, nq, nkv, hd, float(scale), window, splits, per, None, None, None, None, None, 0.0, 0, 1, 0,
-                 _stream())
+                 None if ranges is None else ranges.data_ptr(), _stream())
         return
     _check(meta.positions, "positions", torch.int32, (T,))
     height = tile_height or _prefill_tile_height(meta, nkv, nq // nkv)

@@ -799,3 +799,48 @@ def test_replay_reads_steps_and_names_what_is_wrong_with_them(tmp_path):
         with pytest.raises(RequestError, match="a step is an object"):
             rp.run_step(bad)
     assert rp.run_step({"step": 4, "entries": [], "end": ["a"]}) == 4 and eng.cache.slots.held_count == 0
+
+
+def test_lists_of_ranges_cover_every_sequence_and_follow_the_steps():
+    """The list that deals a decode grid out over sequences of unequal lengths: every sequence's
+    ranges cover its pages, none has a range too many, all together fit the grid; a step with fixed
+    buffers makes its lists again at every update; what counts as unequal."""
+    from herbert_rs_amd.engine.batch import StaticDecodeMeta, StepEntry, is_unequal, pack, range_list
+    rng = random.Random(5)
+    for _ in range(300):
+        B = rng.randint(1, 64)
+        items = rng.randint(B + 1, 4 * B + 8)
+        unit = rng.choice([16, 64])
+        ctx = [rng.choice([1, unit - 1, unit, unit + 1, rng.randint(1, 40000)]) for _ in range(B)]
+        got = range_list(ctx, items, unit)
+        per, counts = int(got[B + 1]), np.diff(got[:B + 1])
+        assert got[0] == 0 and got[B] <= items and per >= 1 and (counts >= 1).all()
+        for n, c in zip(ctx, counts):
+            pages = -(-n // unit)
+            assert (c - 1) * per < pages <= c * per
+    with pytest.raises(ValueError):
+        range_list([5, 5], 2, 64)
+    assert not is_unequal([700]) and not is_unequal([500, 500, 501]) and not is_unequal([1000, 300])
+    assert is_unequal([1000, 1, 1]) and is_unequal([1000, 100]) and is_unequal([32768] + [1024] * 7) and not is_unequal([4096] + [2048] * 3)
+
+    static = StaticDecodeMeta(3, torch.device("cpu"))
+    entries = [StepEntry(4, [7], [0]), StepEntry(2, [8], [0]), StepEntry(9, [9], [0])]
+    meta = static.update(entries, [5000, 10, 63])
+    assert meta.unequal and list(meta.host_context) == [5001, 11, 64]
+    first = meta.ranges_for(16, 64)
+    assert first.tolist() == range_list([5001, 11, 64], 16, 64).tolist()
+    assert meta.ranges_for(16, 64) is first                  # one list for all who ask for the same
+    other = meta.ranges_for(8, 64)
+    meta = static.update(entries, [5055, 64, 64])            # a page more for each
+    assert first.tolist() == range_list([5056, 65, 65], 16, 64).tolist()
+    assert other.tolist() == range_list([5056, 65, 65], 8, 64).tolist()
+    assert meta.ranges_for(16, 64) is first
+    for items in (32, 64):
+        assert meta.ranges_for(items, 64) is not None
+    assert meta.ranges_for(128, 64) is None                  # no room for a fifth list: the caller does without
+    meta = static.update(entries, [70, 64, 64])
+    assert not meta.unequal and list(meta.slots) == [4, 2, 9]
+
+    packed = pack(entries, [5000, 10, 63], torch.device("cpu"))
+    assert packed.unequal and packed.ranges_for(16, 64).tolist() == range_list([5001, 11, 64], 16, 64).tolist()
+    assert not pack(entries, [64, 10, 63], torch.device("cpu")).unequal

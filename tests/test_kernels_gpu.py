@@ -253,8 +253,11 @@ def paged_case(lengths, new_counts, nkv, hd, dtype, seed=0, n_pages=64, shuffle=
     meta.host_starts = np.array(starts, dtype=np.int32)
     meta.host_context = np.array(lengths, dtype=np.int32)
     meta.derived = {}
-    from herbert_rs_amd.engine.batch import bucket
+    from herbert_rs_amd.engine.batch import BatchMeta, bucket, is_unequal
     meta.context_bucket = bucket(max(lengths))
+    # contexts of very unequal lengths: the decode kernel deals its grid out by a list of ranges
+    meta.unequal, meta.static, meta.token_ids = is_unequal(lengths), None, meta.positions
+    meta.ranges_for = lambda items, unit: BatchMeta.ranges_for(meta, items, unit)
     return meta, kv, dense
 
 
@@ -313,19 +316,58 @@ def test_attention_mfma_prefill(nq, nkv, hd, window, tile_height):
 @pytest.mark.parametrize("nq,nkv,hd,window", [(4, 1, 128, 0), (32, 8, 128, 0), (6, 2, 32, 0), (5, 1, 64, 70),
                                               (3, 3, 128, 100), (64, 2, 64, 0)])
 @pytest.mark.parametrize("lengths", [[1, 64, 65, 700], [1000], [130, 3, 512, 999, 77, 640, 64, 128, 256]])
-@pytest.mark.parametrize("waves", [1024, 1])
-def test_attention_mfma_decode(nq, nkv, hd, window, lengths, waves, monkeypatch):
-    """waves = 1: every sequence is one range, and the kernel writes the output without a merge."""
+@pytest.mark.parametrize("waves,by_list", [(1024, True), (1024, False), (1, False)])
+def test_attention_mfma_decode(nq, nkv, hd, window, lengths, waves, by_list, monkeypatch):
+    """waves = 1: every sequence is one range, and the kernel writes the output without a merge.
+    by_list: where the lengths are very unequal (and there is no window) the grid is dealt out by a
+    list of ranges; without it every sequence has the same number of ranges."""
     from herbert_rs_amd.kernels import mfma
     monkeypatch.setattr(mfma, "DECODE_WAVES", waves)
     meta, kv, dense = paged_case(lengths, [1] * len(lengths), nkv, hd, torch.bfloat16, seed=nq + hd,
                                  n_pages=80)
+    meta.unequal = meta.unequal and by_list
+    assert (mfma._decode_ranges(meta, nkv, window) is not None) == (by_list and len(lengths) > 1 and not window)
     q = rand(len(lengths), nq * hd, seed=22, dtype=torch.bfloat16)
     out = torch.full_like(q, 9.0)
     scale = hd ** -0.5
     mfma.attention(q, meta, kv, out, nq, nkv, hd, scale, window)
     want = attention_reference(q, meta, dense, nq, nkv, hd, scale, window)
     assert float((out.float().cpu() - want).abs().max()) <= 2 ** -7 * float(want.abs().max())
+
+
+@pytest.mark.parametrize("lengths", [[20000, 70, 1000, 64, 1, 65, 130, 900], [300] * 30 + [9000, 5000],
+                                     [64] * 63 + [4000], [8000, 1, 1]])
+def test_attention_mfma_decode_of_unequal_sequences_by_a_list(lengths):
+    """Sequences of very unequal lengths: the grid's items are dealt out by a list, every item a
+    range of the same number of pages of whichever sequence. In each sequence one key far back (in
+    its first page, at a page's edge, in its last range) scores far above the rest, so that a range
+    that is skipped, read twice or given to another sequence shows."""
+    from herbert_rs_amd.engine.batch import range_list
+    from herbert_rs_amd.kernels import mfma
+    nq, nkv, hd = 16, 8, 128
+    B = len(lengths)
+    pages = sum((n + 64) // 64 + 1 for n in lengths)
+    meta, kv, dense = paged_case(lengths, [1] * B, nkv, hd, torch.bfloat16, seed=B, n_pages=pages)
+    items, listed = mfma._decode_ranges(meta, nkv, 0)
+    assert items == 128
+    got = listed.cpu().numpy()
+    assert (got == range_list(lengths, items, 64)).all() and got[B] <= items
+    per = int(got[B + 1])
+    assert all((got[b + 1] - got[b]) * per >= -(-n // 64) > (got[b + 1] - got[b] - 1) * per for b, n in enumerate(lengths))
+    targets = [[0, 63, 64, n - 2, (n - 1) // 64 * 64, n // 2][b % 6] % max(1, n - 1) for b, n in enumerate(lengths)]
+    q = torch.zeros(B, nq * hd)
+    for b, t in enumerate(targets):
+        q[b] = (dense[b][0][t] * 8).repeat_interleave(nq // nkv, dim=0).reshape(-1)    # each head with its kv head's key
+    q = q.to(torch.bfloat16).to(dev())
+    out = torch.full_like(q, 9.0)
+    mfma.attention(q, meta, kv, out, nq, nkv, hd, 1.0, 0)
+    want = attention_reference(q, meta, dense, nq, nkv, hd, 1.0, 0)
+    assert float((out.float().cpu() - want).abs().max()) <= 2 ** -7 * float(want.abs().max())
+    res = out.float().cpu().view(B, nq, hd)
+    for b, t in enumerate(targets):
+        if lengths[b] > 1:
+            V = dense[b][1][t].repeat_interleave(nq // nkv, dim=0)
+            assert float((res[b] - V).abs().max()) < 0.05, (b, t)
 
 
 def test_attention_mfma_decode_of_many_sequences_in_shorter_ranges():
@@ -459,16 +501,18 @@ def test_gemm_qkv_with_norm_rotation_and_cache_write(nq, nkv, norm, rope, packed
                                                         (6, 2, 32, 0, True, False), (5, 1, 64, 70, False, True),
                                                         (3, 3, 128, 100, True, True), (64, 2, 64, 0, False, False)])
 @pytest.mark.parametrize("lengths", [[1, 64, 65, 700], [1000], [130, 3, 512, 999, 77, 640, 64, 128, 256]])
-@pytest.mark.parametrize("waves", [1024, 1])
+@pytest.mark.parametrize("waves,by_list", [(1024, True), (1024, False), (1, False)])
 def test_attention_mfma_decode_fused_with_norm_rotation_and_cache_write(nq, nkv, hd, window, norm, rope, lengths,
-                                                                        waves, monkeypatch):
+                                                                        waves, by_list, monkeypatch):
     """The decode kernel that norms, rotates and writes the new key and value itself against the
-    separate kernels: same pages afterwards, same output (waves = 1: without a merge)."""
+    separate kernels: same pages afterwards, same output (waves = 1: without a merge; by_list: very
+    unequal lengths by a list of ranges, in both kernels)."""
     from herbert_rs_amd.cache.paged import LayerKV
     from herbert_rs_amd.kernels import mfma, ops
     monkeypatch.setattr(mfma, "DECODE_WAVES", waves)
     B = len(lengths)
     meta, kv, _ = paged_case(lengths, [1] * B, nkv, hd, torch.bfloat16, seed=nq + hd, n_pages=80)
+    meta.unequal = meta.unequal and by_list
     kv2 = LayerKV(kv.k.clone(), kv.v.clone(), kv.page_table, 64, 0)
     before_k, before_v = kv.k.clone(), kv.v.clone()
     qkv = rand(B, (nq + 2 * nkv) * hd, seed=23, scale=1.5)

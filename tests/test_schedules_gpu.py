@@ -63,6 +63,38 @@ def test_decoding_sequences_and_a_new_prompt_in_one_step(name, dtype, model_root
     engine.cache.check()
 
 
+@pytest.mark.parametrize("name,lengths", [("D", [1780, 3, 70, 250, 64]), ("F", [3050, 10, 500, 64, 129, 1, 63, 700])])
+def test_decoding_a_batch_of_very_unequal_lengths(name, lengths, model_root):
+    """One long sequence beside short ones, decoded together for 40 steps: the attention deals its
+    grid out by a list of ranges that the host makes again at every step (sequences pass the ends
+    of pages and of context buckets on the way, the first step runs eagerly, the second is
+    captured, the rest are replays), and the shortest sequence ends earlier. Every logit is the one
+    the sequence gets alone."""
+    folder = make_folder(model_root, name, "bfloat16")
+    raw = CONFIGS[name][0]
+    vocab = raw["vocab_size"]
+    steps = 40
+    toks = [random_tokens(vocab, n + (steps if i != 1 else 9), 700 + i) for i, n in enumerate(lengths)]
+    ref = [plain_logits(folder, t) for t in toks]
+    engine = hb.load(folder, dtype="bfloat16", cache_tokens=64 * (sum(-(-(n + steps) // 64) for n in lengths) + 2))
+    slots = [engine.alloc_slot() for _ in lengths]
+    engine.step([StepEntry(s, t[:n], []) for s, t, n in zip(slots, toks, lengths)])
+    live = list(range(len(lengths)))
+    for j in range(steps):
+        live = [i for i in live if lengths[i] + j < len(toks[i])]
+        got = engine.step([StepEntry(slots[i], [toks[i][lengths[i] + j]], [0]) for i in live]).cpu().numpy()
+        for row, i in enumerate(live):
+            ok, err = close(got[row], ref[i][lengths[i] + j], "bfloat16", name, "unequal batch")
+            assert ok, (i, j, err)
+    items = 1024 // raw["num_key_value_heads"]
+    for B in (len(lengths), len(lengths) - 1):
+        assert engine._decode[B].static.range_lists == [(items, 64)]      # the list was what ran
+    assert engine.graphs_captured >= 3
+    for s in slots:
+        engine.free_slot(s)
+    engine.cache.check()
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["B", "D"])
 def test_roll_back_and_feed_other_tokens(name, dtype, model_root):
