@@ -46,7 +46,7 @@ class BatchMeta:
         """The list that cuts this step's contexts into at most `items` ranges of equally many whole
         units of `unit` positions (see range_list), as int32 [num_seqs + 2] on the GPU; None if a
         step with fixed buffers has no room for another list. A step with fixed buffers refills the
-        lists it has handed out at every update."""
+        lists it has handed out at every update whose sequences are `unequal`: ask only then."""
         key = ("ranges", int(items), int(unit))
         got = self.derived.get(key)
         if got is None:
@@ -191,8 +191,10 @@ class StaticDecodeMeta:
         h[3 * B:4 * B] = [e.slot for e in entries]
         context = h[5 * B + 1:6 * B + 1]
         np.add(h[B:2 * B], 1, out=context)
-        for i, (items, unit) in enumerate(self.range_lists):
-            h[self._range_place(i)] = range_list(context, items, unit)
+        unequal = is_unequal(context)
+        if unequal:                     # nobody reads the lists of a step whose sequences are alike
+            for i, (items, unit) in enumerate(self.range_lists):
+                h[self._range_place(i)] = range_list(context, items, unit)
         self.dev.copy_(self.host, non_blocking=True)
         if self.dev.is_cuda:
             if self.copied is None:
@@ -203,5 +205,5 @@ class StaticDecodeMeta:
         m.max_context = int(max(start_lengths)) + 1
         m.max_position = m.max_context - 1
         m.context_bucket = bucket(m.max_context)
-        m.unequal = is_unequal(context)
+        m.unequal = unequal
         return m

@@ -840,6 +840,8 @@ def test_lists_of_ranges_cover_every_sequence_and_follow_the_steps():
     assert meta.ranges_for(128, 64) is None                  # no room for a fifth list: the caller does without
     meta = static.update(entries, [70, 64, 64])
     assert not meta.unequal and list(meta.slots) == [4, 2, 9]
+    meta = static.update(entries, [900, 65, 65])               # unequal again: the lists follow
+    assert meta.unequal and first.tolist() == range_list([901, 66, 66], 16, 64).tolist()
 
     packed = pack(entries, [5000, 10, 63], torch.device("cpu"))
     assert packed.unequal and packed.ranges_for(16, 64).tolist() == range_list([5001, 11, 64], 16, 64).tolist()
