@@ -137,3 +137,28 @@ def test_decode_attention_ranges_by_how_evenly_the_waves_sit():
             ranges, per = split(b, t)
             span = -(-t // 64)
             assert ranges >= 1 and per >= 1 and ranges * per >= span > (ranges - 1) * per, (b, t)
+
+
+def test_decode_attention_takes_a_list_of_ranges_only_where_it_fits():
+    """The list that deals the decode grid out over sequences of unequal lengths: for 2 to 64
+    sequences without a window whose grid has at least two items a sequence; else equal shares."""
+    import torch
+    from herbert_rs_amd.engine.batch import StepEntry, pack, range_list
+    from herbert_rs_amd.kernels import mfma
+
+    def meta_of(contexts):
+        return pack([StepEntry(i, [1], [0]) for i in range(len(contexts))], [c - 1 for c in contexts],
+                    torch.device("cpu"))
+    unequal = [9000] + [100] * 7
+    items, listed = mfma._decode_ranges(meta_of(unequal), 8, 0)
+    assert items == 128 and listed.tolist() == range_list(unequal, 128, 64).tolist()
+    assert mfma._decode_ranges(meta_of(unequal), 2, 0)[0] == 512
+    assert mfma._decode_ranges(meta_of(unequal), 1, 0)[0] == 1024           # the grid's z has no more
+    assert mfma._decode_ranges(meta_of(unequal), 8, 70) is None             # a window
+    assert mfma._decode_ranges(meta_of([9000] * 4 + [8000] * 4), 8, 0) is None      # lengths alike
+    assert mfma._decode_ranges(meta_of([9000]), 8, 0) is None
+    assert mfma._decode_ranges(meta_of([9000] + [100] * 64), 8, 0) is None  # more sequences than a wave's lanes
+    assert mfma._decode_ranges(meta_of([9000] + [100] * 39), 16, 0) is None  # 64 items for 40 sequences
+    assert mfma._decode_ranges(meta_of([9000] + [100] * 31), 16, 0)[0] == 64
+    prompt = pack([StepEntry(0, [1, 2, 3], [2]), StepEntry(1, [4], [0])], [9000, 10], torch.device("cpu"))
+    assert prompt.unequal and mfma._decode_ranges(prompt, 8, 0) is None     # not one token a sequence
