@@ -28,23 +28,32 @@ _DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16,
 
 
 class _DecodeState:
-    """What the decode steps of one batch size share: the fixed metadata buffers and the one
-    logits buffer that every graph of this batch size writes to."""
+    """What the decode steps of one batch size share: the fixed metadata buffers and the logits
+    buffer that every graph of this batch size writes to (rows of the engine's one buffer for the
+    usual sizes, `own_logits` for a larger one)."""
 
-    def __init__(self, static, logits):
+    def __init__(self, static, logits, own_logits):
         self.static = static
         self.logits = logits
+        self.own_logits = own_logits
         self.seen = {}          # (context bucket, unequal) -> eager steps run
 
 
 # Captured graphs kept at any time, over all batch sizes and context buckets; the least recently
-# replayed one is dropped for a new one. A graph holds no logits of its own (they are per batch
-# size) and no scratch (the parts' buffers are the runtime's), so a graph costs its kernel
-# arguments only; the cap bounds what a long run over many batch sizes and contexts accumulates.
-MAX_GRAPHS = 48
-# Batch sizes whose fixed buffers (metadata, logits [B, vocab] float32) are kept; beyond it the
-# least recently used size is dropped together with its graphs.
-MAX_DECODE_BATCH_SIZES = 8
+# replayed one is dropped for a new one. A graph holds no logits of its own and no scratch (the
+# parts' buffers are the runtime's), so a graph costs its kernel arguments only; the cap bounds
+# what a long run over many batch sizes and contexts accumulates. A batch whose sequences end one
+# after another passes through every size below its first, and each (size, context bucket) is a
+# graph: the cap leaves room for a few such batches' graphs, so that the next batch finds them.
+MAX_GRAPHS = 192
+# Decode steps of up to this many sequences write their logits into the first rows of one buffer
+# [rows, vocab] float32 that the engine keeps (39 MB for a vocabulary of 151,936); what a decode
+# step returns is therefore overwritten by the next decode step, whatever its size.
+SHARED_LOGITS_ROWS = 64
+# Batch sizes whose fixed metadata buffers are kept, and, among them, sizes beyond the shared
+# logits buffer that keep one of their own; the least recently used goes, with its graphs.
+MAX_DECODE_BATCH_SIZES = 96
+MAX_OWN_LOGITS = 8
 
 
 def require_gpu():
@@ -72,6 +81,7 @@ class Engine:
         self.use_graphs = bool(use_graphs) and self.model.graph_safe
         self._decode = OrderedDict()    # batch size -> _DecodeState, least recently used first
         self._graphs = OrderedDict()    # (batch size, context bucket, unequal) -> graph, least recently used first
+        self._shared_logits = None      # [SHARED_LOGITS_ROWS at most, vocab], made by the first decode step
         self.graphs_captured = 0
         self.ignored_tensors = []       # stored tensors that the model did not ask for
         self._tensor_source = None      # how get_tensor finds a tensor again: set by the constructors below
@@ -228,20 +238,33 @@ class Engine:
         captured HIP graph that is replayed, so that the host launches one graph and not hundreds
         of kernels. A graph is tied to the batch size, to the bucket of the longest context
         (which sizes the attention grid) and to whether the contexts are of very unequal lengths
-        (the attention then deals its grid out by a list). All graphs of a batch size write their logits into that
-        size's one buffer: what a step returns is overwritten by the next decode step of the same
-        batch size. At most MAX_GRAPHS graphs and MAX_DECODE_BATCH_SIZES batch sizes are kept,
-        the least recently used go first."""
+        (the attention then deals its grid out by a list). All graphs write their logits into the
+        first rows of the engine's one buffer (batch sizes beyond SHARED_LOGITS_ROWS: into one of
+        their size's own): what a step returns is overwritten by the next decode step. At most
+        MAX_GRAPHS graphs and MAX_DECODE_BATCH_SIZES batch sizes are kept, the least recently used
+        go first."""
         B = len(entries)
         state = self._decode.get(B)
         if state is None:
-            while len(self._decode) >= MAX_DECODE_BATCH_SIZES:
+            rows = min(SHARED_LOGITS_ROWS, self.cache.n_slots)
+            own = B > rows
+            crowded = [b for b, st in self._decode.items() if st.own_logits] if own else []
+            drop = crowded[:1] if len(crowded) >= MAX_OWN_LOGITS else []
+            if not drop and len(self._decode) >= MAX_DECODE_BATCH_SIZES:
+                drop = [next(iter(self._decode))]
+            for old in drop:
                 torch.cuda.synchronize(self.device)
-                old, _ = self._decode.popitem(last=False)
+                del self._decode[old]
                 for key in [k for k in self._graphs if k[0] == old]:
                     del self._graphs[key]
-            logits = torch.empty((B, self.spec.vocab_size), dtype=torch.float32, device=self.device)
-            state = self._decode[B] = _DecodeState(StaticDecodeMeta(B, self.device), logits)
+            if own:
+                logits = torch.empty((B, self.spec.vocab_size), dtype=torch.float32, device=self.device)
+            else:
+                if self._shared_logits is None:
+                    self._shared_logits = torch.empty((rows, self.spec.vocab_size), dtype=torch.float32,
+                                                      device=self.device)
+                logits = self._shared_logits[:B]
+            state = self._decode[B] = _DecodeState(StaticDecodeMeta(B, self.device), logits, own)
         self._decode.move_to_end(B)
         meta = state.static.update(entries, starts)
         if tokens_on_device is not None:
@@ -268,8 +291,10 @@ class Engine:
         return state.logits
 
     def decode_graph_stats(self):
-        """(graphs kept, batch sizes kept, bytes of the per-batch-size logits buffers)."""
-        held = sum(st.logits.numel() * 4 for st in self._decode.values())
+        """(graphs kept, batch sizes kept, bytes of the decode steps' logits buffers)."""
+        held = sum(st.logits.numel() * 4 for st in self._decode.values() if st.own_logits)
+        if self._shared_logits is not None:
+            held += self._shared_logits.numel() * 4
         return len(self._graphs), len(self._decode), held
 
     def generate(self, prompts, params=None, max_batch=64, on_token=None, interrupt=None, prefill_chunk=None):
