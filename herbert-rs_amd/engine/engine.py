@@ -173,6 +173,8 @@ class Engine:
     def step(self, entries, tokens_on_device=None):
         """Run the entries' tokens; returns float32 logits [wanted, vocab] on the GPU
         (rows in the order of the entries and of their `want`), or None if nothing is wanted.
+        The logits of a step in which every sequence brings one token and wants its logits lie
+        in a buffer that the next such step writes again: copy what is to outlast it.
         `tokens_on_device` (int32 [entries] on the GPU, every entry bringing one token): the
         tokens are taken from there, in the stream's order, and the entries' own are only
         placeholders; so a step can be put on the stream before the host has seen the tokens
