@@ -651,7 +651,7 @@ attn_decode_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_cache, bf16*
                    const int* __restrict__ ranges, int n_seqs) {
     // ranges == null: the grid is (sequence, kv head, range), every sequence cut into gridDim.z
     // ranges of pages_per_split pages (those past a sequence's end hold nothing).
-    // ranges != null (sequences of unequal lengths, at most 64): the grid is (1, kv head, item);
+    // ranges != null (sequences of unequal lengths): the grid is (1, kv head, item);
     // ranges[0 .. n_seqs] count the ranges of the sequences before each one, ranges[n_seqs + 1] is
     // the pages of a range: item i is range i - ranges[b] of the sequence b whose count it falls
     // into, and items from ranges[n_seqs] on are nothing. The partial results are then laid out
@@ -661,8 +661,12 @@ attn_decode_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_cache, bf16*
     int b = blockIdx.x, split = blockIdx.z;
     if (ranges) {
         const int item = blockIdx.z;
-        const int upto = lane < n_seqs ? ranges[lane + 1] : 0x7fffffff;
-        b = __builtin_amdgcn_readfirstlane(__popcll(__ballot(upto <= item)));     // sequences wholly before the item
+        b = 0;                                              // sequences wholly before the item
+        for (int first = 0; first < n_seqs; first += 64) {
+            const int upto = first + lane < n_seqs ? ranges[first + lane + 1] : 0x7fffffff;
+            b += __popcll(__ballot(upto <= item));
+        }
+        b = __builtin_amdgcn_readfirstlane(b);
         if (b >= n_seqs) return;
         split = item - ranges[b];
         pages_per_split = ranges[n_seqs + 1];
@@ -1044,8 +1048,8 @@ extern "C" int hb_attn_decode_mfma(const void* q, void* k_cache, void* v_cache, 
                                    hipStream_t stream) {
     // ranges != null: see attn_decode_kernel; `splits` is then the number of items of the grid (the
     // partial results are [nq, splits]), pages_per_split is not read
-    HB_REQUIRE(!ranges || (B >= 2 && B <= 64 && splits >= 2 && window == 0),
-               "attn_decode: a list of ranges is for 2 to 64 sequences, with a merge, without a window");
+    HB_REQUIRE(!ranges || (B >= 2 && splits >= 2 && window == 0),
+               "attn_decode: a list of ranges is for two sequences or more, with a merge, without a window");
     HB_REQUIRE(B > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attn_decode: bad sizes");
     HB_REQUIRE(page_size == PAGE, "attn_decode: pages must hold %d tokens", PAGE);
     HB_REQUIRE(nq / nkv <= 32, "attn_decode: more than 32 query heads share a kv head");

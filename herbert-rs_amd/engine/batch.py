@@ -39,7 +39,7 @@ class BatchMeta:
     host_context: np.ndarray
     derived: dict = None       # what kernels' host sides derive once a step (tile lists and the like)
     context_bucket: int = 0    # max_context rounded up to CONTEXT_BUCKET: sizes the decode kernels' grids
-    unequal: bool = False      # the contexts fill at most 0.55 of num_seqs x max_context (see is_unequal)
+    unequal: int = 0           # how unequal the contexts' lengths are: 0 (alike), 1, 2 (see unequal_level)
     static: object = None      # the StaticDecodeMeta whose buffers these are, if any
 
     def ranges_for(self, items, unit):
@@ -60,14 +60,20 @@ class BatchMeta:
         return got
 
 
-def is_unequal(context):
-    """True where the sequences of a step together hold at most 0.55 of what they would if all were
-    as long as the longest: a kernel that gives every sequence the same share of the GPU then leaves
-    much of it idle. (Measured on decode steps of the 8B shape: dealing the attention's grid out by
-    a list takes 7 to 11 % off a step at 0.34 to 0.51 and 23 to 54 % at 0.08 to 0.18, nothing
-    from 0.56 on, and adds 2 to 4 % where all are equal.)"""
+def unequal_level(context):
+    """How unequal the lengths of a step's sequences are, by what they hold together of what they
+    would if all were as long as the longest: 0 above 0.55, 1 from there down, 2 from 0.45 down. A
+    kernel that gives every sequence the same share of the GPU leaves much of it idle where this
+    is not 0. (Measured on decode steps of the 8B shape: dealing the attention's grid out by a list
+    takes 7 to 11 % off a step of 8 to 64 sequences at 0.34 to 0.51 and 23 to 54 % at 0.08 to
+    0.18, nothing from 0.56 on, and adds 2 to 4 % where all are equal. 80 to 200 sequences, whose
+    lists need more than one round of waves: 9 to 36 % off at 0.17 to 0.40, 60 % at 0.07, between
+    9 % more and 7 % less at 0.5: these take the list from level 2 on.)"""
     context = np.asarray(context, dtype=np.int64)
-    return len(context) > 1 and 20 * int(context.sum()) <= 11 * len(context) * int(context.max())
+    if len(context) < 2:
+        return 0
+    held, room = 20 * int(context.sum()), len(context) * int(context.max())
+    return 2 if held <= 9 * room else 1 if held <= 11 * room else 0
 
 
 def range_list(context, items, unit):
@@ -135,7 +141,7 @@ def pack(entries, start_lengths, device, staging=None):
         context_lens=dev[o + 2 * B + 1:o + 3 * B + 1], want_rows=dev[o + 3 * B + 1:o + 3 * B + 1 + R],
         num_tokens=T, num_seqs=B, max_new=max(counts), max_context=int(ctx.max()),
         max_position=int(pos.max()), host_starts=starts.copy(), host_context=ctx.copy(), derived={},
-        context_bucket=bucket(int(ctx.max())), unequal=is_unequal(ctx))
+        context_bucket=bucket(int(ctx.max())), unequal=unequal_level(ctx))
 
 
 class StaticDecodeMeta:
@@ -191,7 +197,7 @@ class StaticDecodeMeta:
         h[3 * B:4 * B] = [e.slot for e in entries]
         context = h[5 * B + 1:6 * B + 1]
         np.add(h[B:2 * B], 1, out=context)
-        unequal = is_unequal(context)
+        unequal = unequal_level(context)
         if unequal:                     # nobody reads the lists of a step whose sequences are alike
             for i, (items, unit) in enumerate(self.range_lists):
                 h[self._range_place(i)] = range_list(context, items, unit)

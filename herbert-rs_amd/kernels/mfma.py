@@ -440,13 +440,16 @@ def _decode_ranges(meta, nkv, window):
     lengths, else None. Equal shares would leave the waves of the short sequences with nothing and
     those of the long ones with all the work (one sequence of 32 K tokens beside seven of 1 K: 128 of
     1,024 waves read 2 K tokens each); with the list every wave has a range of the same length of
-    whichever sequence, as many ranges as the GPU holds waves at a time. The list changes with
-    every step and is read by the kernel; the grid does not change."""
+    whichever sequence, as many ranges as the GPU holds waves at a time (more where that would be
+    fewer than two a sequence, and the lengths are unequal enough for more than a round to pay). The list changes with every step and is read by the kernel; the
+    grid does not change."""
     B = meta.num_seqs
-    if not meta.unequal or window or not 2 <= B <= 64 or meta.max_new != 1:
+    if not meta.unequal or window or B < 2 or meta.max_new != 1:
         return None
-    items = min(1024, DECODE_WAVES // nkv)
-    if items < 2 * B:
+    # at least two items a sequence, so that a range is no longer than the mean sequence: beyond
+    # half a round of sequences the grid is more than one round of waves (the kernel's limit: 1,024 items)
+    items = max(DECODE_WAVES // nkv, 2 * B)
+    if items > 1024 or items < 4 or (items * nkv > DECODE_WAVES and meta.unequal < 2):
         return None
     listed = meta.ranges_for(items, 64)
     return None if listed is None else (items, listed)

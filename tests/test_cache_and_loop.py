@@ -805,7 +805,7 @@ def test_lists_of_ranges_cover_every_sequence_and_follow_the_steps():
     """The list that deals a decode grid out over sequences of unequal lengths: every sequence's
     ranges cover its pages, none has a range too many, all together fit the grid; a step with fixed
     buffers makes its lists again at every update; what counts as unequal."""
-    from herbert_rs_amd.engine.batch import StaticDecodeMeta, StepEntry, is_unequal, pack, range_list
+    from herbert_rs_amd.engine.batch import StaticDecodeMeta, StepEntry, unequal_level, pack, range_list
     rng = random.Random(5)
     for _ in range(300):
         B = rng.randint(1, 64)
@@ -820,8 +820,9 @@ def test_lists_of_ranges_cover_every_sequence_and_follow_the_steps():
             assert (c - 1) * per < pages <= c * per
     with pytest.raises(ValueError):
         range_list([5, 5], 2, 64)
-    assert not is_unequal([700]) and not is_unequal([500, 500, 501]) and not is_unequal([1000, 300])
-    assert is_unequal([1000, 1, 1]) and is_unequal([1000, 100]) and is_unequal([32768] + [1024] * 7) and not is_unequal([4096] + [2048] * 3)
+    assert [unequal_level(c) for c in ([700], [500, 500, 501], [1000, 300], [4096] + [2048] * 3)] == [0, 0, 0, 0]
+    assert [unequal_level(c) for c in ([1000, 100], [1000, 50, 500], [4096] + [1024] * 7)] == [1, 1, 2]
+    assert [unequal_level(c) for c in ([1000, 1, 1], [32768] + [1024] * 7, [8192] + [512] * 127)] == [2, 2, 2]
 
     static = StaticDecodeMeta(3, torch.device("cpu"))
     entries = [StepEntry(4, [7], [0]), StepEntry(2, [8], [0]), StepEntry(9, [9], [0])]

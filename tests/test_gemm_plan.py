@@ -140,8 +140,9 @@ def test_decode_attention_ranges_by_how_evenly_the_waves_sit():
 
 
 def test_decode_attention_takes_a_list_of_ranges_only_where_it_fits():
-    """The list that deals the decode grid out over sequences of unequal lengths: for 2 to 64
-    sequences without a window whose grid has at least two items a sequence; else equal shares."""
+    """The list that deals the decode grid out over sequences of unequal lengths: for two sequences
+    or more without a window, a round of waves or two items a sequence, up to the kernel's 1,024
+    items; else equal shares."""
     import torch
     from herbert_rs_amd.engine.batch import StepEntry, pack, range_list
     from herbert_rs_amd.kernels import mfma
@@ -157,8 +158,14 @@ def test_decode_attention_takes_a_list_of_ranges_only_where_it_fits():
     assert mfma._decode_ranges(meta_of(unequal), 8, 70) is None             # a window
     assert mfma._decode_ranges(meta_of([9000] * 4 + [8000] * 4), 8, 0) is None      # lengths alike
     assert mfma._decode_ranges(meta_of([9000]), 8, 0) is None
-    assert mfma._decode_ranges(meta_of([9000] + [100] * 64), 8, 0) is None  # more sequences than a wave's lanes
-    assert mfma._decode_ranges(meta_of([9000] + [100] * 39), 16, 0) is None  # 64 items for 40 sequences
+    assert mfma._decode_ranges(meta_of([9000] + [100] * 64), 8, 0)[0] == 130   # two items a sequence
+    assert mfma._decode_ranges(meta_of([9000] + [100] * 39), 16, 0)[0] == 80
     assert mfma._decode_ranges(meta_of([9000] + [100] * 31), 16, 0)[0] == 64
+    assert mfma._decode_ranges(meta_of([9000] + [100] * 511), 8, 0)[0] == 1024
+    assert mfma._decode_ranges(meta_of([9000] + [100] * 512), 8, 0) is None     # more items than the kernel takes
+    half = [4000] * 40 + [200] * 40                             # holds 0.525 of 80 x 4000: level 1
+    assert meta_of(half).unequal == 1 and meta_of(half[8:72]).unequal == 1
+    assert mfma._decode_ranges(meta_of(half), 8, 0) is None     # more than a round of waves: from level 2 on
+    assert mfma._decode_ranges(meta_of(half[8:72]), 8, 0)[0] == 128
     prompt = pack([StepEntry(0, [1, 2, 3], [2]), StepEntry(1, [4], [0])], [9000, 10], torch.device("cpu"))
     assert prompt.unequal and mfma._decode_ranges(prompt, 8, 0) is None     # not one token a sequence

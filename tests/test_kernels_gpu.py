@@ -253,10 +253,10 @@ def paged_case(lengths, new_counts, nkv, hd, dtype, seed=0, n_pages=64, shuffle=
     meta.host_starts = np.array(starts, dtype=np.int32)
     meta.host_context = np.array(lengths, dtype=np.int32)
     meta.derived = {}
-    from herbert_rs_amd.engine.batch import BatchMeta, bucket, is_unequal
+    from herbert_rs_amd.engine.batch import BatchMeta, bucket, unequal_level
     meta.context_bucket = bucket(max(lengths))
     # contexts of very unequal lengths: the decode kernel deals its grid out by a list of ranges
-    meta.unequal, meta.static, meta.token_ids = is_unequal(lengths), None, meta.positions
+    meta.unequal, meta.static, meta.token_ids = unequal_level(lengths), None, meta.positions
     meta.ranges_for = lambda items, unit: BatchMeta.ranges_for(meta, items, unit)
     return meta, kv, dense
 
@@ -336,7 +336,7 @@ def test_attention_mfma_decode(nq, nkv, hd, window, lengths, waves, by_list, mon
 
 
 @pytest.mark.parametrize("lengths", [[20000, 70, 1000, 64, 1, 65, 130, 900], [300] * 30 + [9000, 5000],
-                                     [64] * 63 + [4000], [8000, 1, 1]])
+                                     [64] * 63 + [4000], [8000, 1, 1], [64] * 129 + [6000]])
 def test_attention_mfma_decode_of_unequal_sequences_by_a_list(lengths):
     """Sequences of very unequal lengths: the grid's items are dealt out by a list, every item a
     range of the same number of pages of whichever sequence. In each sequence one key far back (in
@@ -349,7 +349,7 @@ def test_attention_mfma_decode_of_unequal_sequences_by_a_list(lengths):
     pages = sum((n + 64) // 64 + 1 for n in lengths)
     meta, kv, dense = paged_case(lengths, [1] * B, nkv, hd, torch.bfloat16, seed=B, n_pages=pages)
     items, listed = mfma._decode_ranges(meta, nkv, 0)
-    assert items == 128
+    assert items == max(128, 2 * B)
     got = listed.cpu().numpy()
     assert (got == range_list(lengths, items, 64)).all() and got[B] <= items
     per = int(got[B + 1])
