@@ -10,7 +10,8 @@ ms a step, GB/s and the fraction of 8 TB/s at the full context (`decode_b1`, `de
 over a decode from 512 to the full context (`..._mean...`, from steps timed at a few contexts
 in between); and the other two workloads of the benchmark description through the generation
 loop (`qwen3_1p7b_...`, `qwen3_32b_...`); `decode_b8_host_between_steps` is the headline's step
-with the host reading each step's tokens before it starts the next. Weights are random, token ids are random, and the
+with the host reading each step's tokens before it starts the next; `decode_b16_unequal_lengths` is a batch of one
+sequence at the full context beside fifteen of a sixteenth of it. Weights are random, token ids are random, and the
 cache below the timed steps is filled by real prefill steps of random prompts. A timed decode
 step is what the generation loop does for a token: the step function (a HIP-graph replay), the
 greedy choice on the GPU, and the chosen tokens read by the host, which as in that loop reads
@@ -271,18 +272,19 @@ def main():
         torch.cuda.synchronize()
         return (time.perf_counter() - t) / reps
 
-    if unequal:
-        # one batch of sequences of these lengths (after the timed steps), decoded as the loop does
-        if min(unequal) <= args.steps + args.warmup:
-            raise ValueError(f"every sequence of --contexts needs more than {args.steps + args.warmup} tokens")
-        slots = [engine.alloc_slot() for _ in unequal]
-        for s, c in zip(slots, unequal):
-            fill = c - args.steps - args.warmup
+    def unequal_run(contexts, steps, warmup):
+        """(ms a step, GB/s) of one batch whose sequences hold `contexts` tokens after the timed
+        steps, decoded as the generation loop does (each step put on the stream one ahead)."""
+        if min(contexts) <= steps + warmup:
+            raise ValueError(f"every sequence of {contexts} needs more than {steps + warmup} tokens")
+        slots = [engine.alloc_slot() for _ in contexts]
+        for s, c in zip(slots, contexts):
+            fill = c - steps - warmup
             for a in range(0, fill, 2048):
                 engine.step([StepEntry(s, ids(min(2048, fill - a)), [])])
         chooser = Sampler(SamplingParams(temperature=0.0), len(slots), V, engine.device)
         ahead = chooser.choose_ahead(engine.step([StepEntry(s, ids(1), [0]) for s in slots]), range(len(slots)))
-        for n in (args.warmup - 1, args.steps):
+        for n in (warmup - 1, steps):
             torch.cuda.synchronize()
             t = time.perf_counter()
             for _ in range(n):
@@ -291,8 +293,13 @@ def main():
                 chooser.read(before)
             torch.cuda.synchronize()
             ms = (time.perf_counter() - t) / max(1, n) * 1e3
-        held = sum(unequal) - len(unequal) * args.steps / 2.0
-        gbs = (weight_bytes + held * kv_bytes_per_token) / (ms * 1e-3) / 1e9
+        for s in slots:
+            engine.free_slot(s)
+        held = sum(contexts) - len(contexts) * steps / 2.0
+        return ms, (weight_bytes + held * kv_bytes_per_token) / (ms * 1e-3) / 1e9, held
+
+    if unequal:
+        ms, gbs, held = unequal_run(unequal, args.steps, max(2, args.warmup))
         print(f"[bench] decode of {len(unequal)} sequences holding {args.contexts} tokens: {ms:.3f} ms a step, "
               f"{len(unequal) / ms * 1e3:.0f} tok/s, {gbs:.0f} GB/s of {HBM_GBS:.0f} "
               f"(weights {weight_bytes / 1e9:.2f} GB + keys and values {held * kv_bytes_per_token / 1e9:.2f} GB)",
@@ -350,6 +357,12 @@ def main():
         _, v_sync, ms_sync = decode_run(args.batch, [(context, min(args.steps, 16), 3)], run_ahead=False)[0]
         points[f"decode_b{args.batch}_host_between_steps"] = round(v_sync, 2)
         points[f"decode_b{args.batch}_host_between_steps_ms"] = round(ms_sync, 4)
+        # a batch of unequal lengths: one sequence at the full context beside fifteen of a sixteenth
+        mixed = [context] + [max(context // 16, 64)] * 15
+        ms_mixed, gbs_mixed, _ = unequal_run(mixed, min(args.steps, 16), 3)
+        points["decode_b16_unequal_lengths_ms"] = round(ms_mixed, 4)
+        points["decode_b16_unequal_lengths"] = round(len(mixed) / ms_mixed * 1e3, 2)
+        points["decode_b16_unequal_lengths_gbs"] = round(gbs_mixed, 1)
     for key in (f"decode_b{args.batch}", f"decode_b{args.batch}_ms", f"decode_b{args.batch}_gbs",
                 f"decode_b{args.batch}_frac"):
         points.pop(key)          # the headline itself: `value`, `ms_per_step`, `roofline`
