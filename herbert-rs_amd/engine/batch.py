@@ -79,18 +79,26 @@ def unequal_level(context):
 def range_list(context, items, unit):
     """Cut B sequences of unequal lengths into ranges of equally many whole units (pages), at most
     `items` of them together (items > B): int32 [B + 2] with [0 .. B] the number of ranges of the
-    sequences before each one and [B + 1] the units of a range. Every sequence gets the ranges that
-    cover its units: sum ceil(p / per) < sum p / per + B <= items for per >= sum p / (items - B)."""
+    sequences before each one and [B + 1] the units of a range, the fewest with which every
+    sequence's ranges, rounded up, still fit. (They do at sum p / (items - B) units: sum ceil(p / per)
+    < sum p / per + B <= items; and the number of ranges never grows with the units a range has.)"""
     context = np.asarray(context, dtype=np.int64)
     B = len(context)
     if items <= B:
         raise ValueError(f"{items} ranges cannot be dealt out to {B} sequences")
     units = np.maximum(1, -(-context // unit))
-    per = max(1, int(-(-units.sum() // (items - B))))
+    total = int(units.sum())
+    low, high = max(1, -(-total // items)), max(1, -(-total // (items - B)))      # high always fits
+    while low < high:
+        per = (low + high) // 2
+        if int((-(-units // per)).sum()) <= items:
+            high = per
+        else:
+            low = per + 1
     out = np.empty(B + 2, dtype=np.int32)
     out[0] = 0
-    np.cumsum(-(-units // per), out=out[1:B + 1])
-    out[B + 1] = per
+    np.cumsum(-(-units // high), out=out[1:B + 1])
+    out[B + 1] = high
     return out
 
 

@@ -803,7 +803,8 @@ def test_replay_reads_steps_and_names_what_is_wrong_with_them(tmp_path):
 
 def test_lists_of_ranges_cover_every_sequence_and_follow_the_steps():
     """The list that deals a decode grid out over sequences of unequal lengths: every sequence's
-    ranges cover its pages, none has a range too many, all together fit the grid; a step with fixed
+    ranges cover its pages, none has a range too many, all together fit the grid, with the shortest
+    ranges that do; a step with fixed
     buffers makes its lists again at every update; what counts as unequal."""
     from herbert_rs_amd.engine.batch import StaticDecodeMeta, StepEntry, unequal_level, pack, range_list
     rng = random.Random(5)
@@ -818,6 +819,8 @@ def test_lists_of_ranges_cover_every_sequence_and_follow_the_steps():
         for n, c in zip(ctx, counts):
             pages = -(-n // unit)
             assert (c - 1) * per < pages <= c * per
+        # and no shorter range would do
+        assert per == 1 or sum(-(-(-(-n // unit)) // (per - 1)) for n in ctx) > items
     with pytest.raises(ValueError):
         range_list([5, 5], 2, 64)
     assert [unequal_level(c) for c in ([700], [500, 500, 501], [1000, 300], [4096] + [2048] * 3)] == [0, 0, 0, 0]
