@@ -441,8 +441,8 @@ def _decode_ranges(meta, nkv, window):
     those of the long ones with all the work (one sequence of 32 K tokens beside seven of 1 K: 128 of
     1,024 waves read 2 K tokens each); with the list every wave has a range of the same length of
     whichever sequence, as many ranges as the GPU holds waves at a time (more where that would be
-    fewer than two a sequence, and the lengths are unequal enough for more than a round to pay). The list changes with every step and is read by the kernel; the
-    grid does not change."""
+    fewer than two a sequence, and the lengths are unequal enough for more than one round of waves
+    to pay). The list changes with every step and is read by the kernel; the grid does not change."""
     B = meta.num_seqs
     if not meta.unequal or window or B < 2 or meta.max_new != 1:
         return None
