@@ -106,7 +106,14 @@ CONTEXT_BUCKET = 256
 
 
 def bucket(context):
-    return (int(context) + CONTEXT_BUCKET - 1) // CONTEXT_BUCKET * CONTEXT_BUCKET
+    """The context rounded up to what sizes a decode kernel's grid (and names a captured graph):
+    multiples of 256 up to 4,096 tokens, of 512 up to 8,192, of 1,024 up to 16,384 and so on, so that
+    a sequence that grows long passes through 8 buckets for each doubling and a grid is never
+    more than an eighth too large."""
+    context, step = int(context), CONTEXT_BUCKET
+    while context > 16 * step:
+        step *= 2
+    return (context + step - 1) // step * step
 
 
 def pack(entries, start_lengths, device, staging=None):

@@ -850,3 +850,15 @@ def test_lists_of_ranges_cover_every_sequence_and_follow_the_steps():
     packed = pack(entries, [5000, 10, 63], torch.device("cpu"))
     assert packed.unequal and packed.ranges_for(16, 64).tolist() == range_list([5001, 11, 64], 16, 64).tolist()
     assert not pack(entries, [64, 10, 63], torch.device("cpu")).unequal
+
+
+def test_context_buckets_grow_with_the_context():
+    """What sizes the decode kernels' grids and names a captured graph: multiples of 256 up to
+    4,096 tokens, then eight buckets for every doubling; never below the context, never more than
+    an eighth above it beyond the first buckets."""
+    from herbert_rs_amd.engine.batch import bucket
+    assert [bucket(c) for c in (1, 256, 257, 4096, 4097, 4608, 4609, 8192, 8193, 16384, 16385, 32768)] == \
+        [256, 256, 512, 4096, 4608, 4608, 5120, 8192, 9216, 16384, 18432, 32768]
+    assert len({bucket(c) for c in range(1, 32769)}) == 16 + 8 + 8 + 8
+    for c in list(range(1, 10000, 37)) + [40000, 131072, 131073, 1000000]:
+        assert c <= bucket(c) < max(c + 256, c * 9 // 8)
