@@ -38,7 +38,7 @@ class BatchMeta:
     host_starts: np.ndarray    # host copies, for kernels' grids
     host_context: np.ndarray
     derived: dict = None       # what kernels' host sides derive once a step (tile lists and the like)
-    context_bucket: int = 0    # max_context rounded up to CONTEXT_BUCKET: sizes the decode kernels' grids
+    context_bucket: int = 0    # max_context rounded up (see bucket): sizes the decode kernels' grids
     unequal: int = 0           # how unequal the contexts' lengths are: 0 (alike), 1, 2 (see unequal_level)
     static: object = None      # the StaticDecodeMeta whose buffers these are, if any
 
