@@ -28,14 +28,12 @@ _DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16,
 
 
 class _DecodeState:
-    """What the decode steps of one batch size share: the fixed metadata buffers and the logits
-    buffer that every graph of this batch size writes to (rows of the engine's one buffer for the
-    usual sizes, `own_logits` for a larger one)."""
+    """What the decode steps of one batch size share: the fixed metadata buffers and the rows of
+    the engine's logits buffer that every graph of this batch size writes to."""
 
-    def __init__(self, static, logits, own_logits):
+    def __init__(self, static, logits):
         self.static = static
         self.logits = logits
-        self.own_logits = own_logits
         self.seen = {}          # (context bucket, unequal) -> eager steps run
 
 
@@ -46,14 +44,14 @@ class _DecodeState:
 # after another passes through every size below its first, and each (size, context bucket) is a
 # graph: the cap leaves room for a few such batches' graphs, so that the next batch finds them.
 MAX_GRAPHS = 192
-# Decode steps of up to this many sequences write their logits into the first rows of one buffer
-# [rows, vocab] float32 that the engine keeps (39 MB for a vocabulary of 151,936); what a decode
-# step returns is therefore overwritten by the next decode step, whatever its size.
+# Decode steps write their logits into the first rows of one buffer [rows, vocab] float32 that the
+# engine keeps: what a decode step returns is therefore overwritten by the next decode step,
+# whatever its size. The buffer starts with this many rows (39 MB for a vocabulary of 151,936) or
+# as many as the cache has slots, if fewer; a larger batch makes a larger one (twice the rows, or
+# what the batch needs) and every graph, which holds the old one's address, is dropped.
 SHARED_LOGITS_ROWS = 64
-# Batch sizes whose fixed metadata buffers are kept, and, among them, sizes beyond the shared
-# logits buffer that keep one of their own; the least recently used goes, with its graphs.
+# Batch sizes whose fixed metadata buffers are kept; the least recently used goes, with its graphs.
 MAX_DECODE_BATCH_SIZES = 96
-MAX_OWN_LOGITS = 8
 
 
 def require_gpu():
@@ -81,7 +79,7 @@ class Engine:
         self.use_graphs = bool(use_graphs) and self.model.graph_safe
         self._decode = OrderedDict()    # batch size -> _DecodeState, least recently used first
         self._graphs = OrderedDict()    # (batch size, context bucket, unequal) -> graph, least recently used first
-        self._shared_logits = None      # [SHARED_LOGITS_ROWS at most, vocab], made by the first decode step
+        self._shared_logits = None      # [rows, vocab], made by the first decode step, grown by a larger batch
         self.graphs_captured = 0
         self.ignored_tensors = []       # stored tensors that the model did not ask for
         self._tensor_source = None      # how get_tensor finds a tensor again: set by the constructors below
@@ -241,32 +239,27 @@ class Engine:
         of kernels. A graph is tied to the batch size, to the bucket of the longest context
         (which sizes the attention grid) and to whether the contexts are of very unequal lengths
         (the attention then deals its grid out by a list). All graphs write their logits into the
-        first rows of the engine's one buffer (batch sizes beyond SHARED_LOGITS_ROWS: into one of
-        their size's own): what a step returns is overwritten by the next decode step. At most
-        MAX_GRAPHS graphs and MAX_DECODE_BATCH_SIZES batch sizes are kept, the least recently used
-        go first."""
+        first rows of the engine's one buffer: what a step returns is overwritten by the next
+        decode step. At most MAX_GRAPHS graphs and MAX_DECODE_BATCH_SIZES batch sizes are kept,
+        the least recently used go first."""
         B = len(entries)
         state = self._decode.get(B)
         if state is None:
-            rows = min(SHARED_LOGITS_ROWS, self.cache.n_slots)
-            own = B > rows
-            crowded = [b for b, st in self._decode.items() if st.own_logits] if own else []
-            drop = crowded[:1] if len(crowded) >= MAX_OWN_LOGITS else []
-            if not drop and len(self._decode) >= MAX_DECODE_BATCH_SIZES:
-                drop = [next(iter(self._decode))]
-            for old in drop:
+            if len(self._decode) >= MAX_DECODE_BATCH_SIZES:
                 torch.cuda.synchronize(self.device)
-                del self._decode[old]
+                old, _ = self._decode.popitem(last=False)
                 for key in [k for k in self._graphs if k[0] == old]:
                     del self._graphs[key]
-            if own:
-                logits = torch.empty((B, self.spec.vocab_size), dtype=torch.float32, device=self.device)
-            else:
-                if self._shared_logits is None:
-                    self._shared_logits = torch.empty((rows, self.spec.vocab_size), dtype=torch.float32,
-                                                      device=self.device)
-                logits = self._shared_logits[:B]
-            state = self._decode[B] = _DecodeState(StaticDecodeMeta(B, self.device), logits, own)
+            held = 0 if self._shared_logits is None else self._shared_logits.shape[0]
+            if B > held:
+                torch.cuda.synchronize(self.device)     # nothing that writes the old buffer still runs
+                self._graphs.clear()
+                self._decode.clear()
+                rows = min(self.cache.n_slots, max(SHARED_LOGITS_ROWS, 2 * held, B))
+                self._shared_logits = None
+                self._shared_logits = torch.empty((rows, self.spec.vocab_size), dtype=torch.float32,
+                                                  device=self.device)
+            state = self._decode[B] = _DecodeState(StaticDecodeMeta(B, self.device), self._shared_logits[:B])
         self._decode.move_to_end(B)
         meta = state.static.update(entries, starts)
         if tokens_on_device is not None:
@@ -294,9 +287,7 @@ class Engine:
 
     def decode_graph_stats(self):
         """(graphs kept, batch sizes kept, bytes of the decode steps' logits buffers)."""
-        held = sum(st.logits.numel() * 4 for st in self._decode.values() if st.own_logits)
-        if self._shared_logits is not None:
-            held += self._shared_logits.numel() * 4
+        held = 0 if self._shared_logits is None else self._shared_logits.numel() * 4
         return len(self._graphs), len(self._decode), held
 
     def generate(self, prompts, params=None, max_batch=64, on_token=None, interrupt=None, prefill_chunk=None):

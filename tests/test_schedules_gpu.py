@@ -371,6 +371,34 @@ def test_decode_graphs_and_their_logits_are_bounded(model_root, monkeypatch):
     engine.cache.check()
 
 
+def test_a_larger_batch_makes_a_larger_logits_buffer(model_root):
+    """The decode steps' one logits buffer has 64 rows at first; a batch of 70 sequences makes one
+    of 128 (every graph is dropped with the old one), and steps of 3, of 70 and of 3 again say
+    what eager steps say."""
+    folder = make_folder(model_root, "A", "bfloat16")
+    vocab = CONFIGS["A"][0]["vocab_size"]
+    engine = hb.Engine.from_folder(folder, dtype="bfloat16", max_tokens=64 * 140, max_slots=130, use_graphs=True)
+    eager = hb.Engine.from_folder(folder, dtype="bfloat16", max_tokens=64 * 140, max_slots=130, use_graphs=False)
+    feed = random_tokens(vocab, 400, 77)
+    for B, rows in ((3, 64), (70, 128), (3, 128)):
+        slots, slots_e = [engine.alloc_slot() for _ in range(B)], [eager.alloc_slot() for _ in range(B)]
+        for eng, sl in ((engine, slots), (eager, slots_e)):
+            eng.step([StepEntry(s, feed[i:i + 5 + i % 7], []) for i, s in enumerate(sl)])
+        for j in range(4):
+            toks = [feed[(11 * i + j) % len(feed)] for i in range(B)]
+            a = engine.step([StepEntry(s, [t], [0]) for s, t in zip(slots, toks)]).cpu().numpy()
+            b = eager.step([StepEntry(s, [t], [0]) for s, t in zip(slots_e, toks)]).cpu().numpy()
+            assert a.shape == (B, vocab) and np.array_equal(a, b), (B, j)
+        assert engine.decode_graph_stats()[2] == rows * vocab * 4
+        for s in slots:
+            engine.free_slot(s)
+        for s in slots_e:
+            eager.free_slot(s)
+    # the first graph of 3 sequences went with the smaller buffer: 70 and 3 are kept, 3 was captured twice
+    assert engine.decode_graph_stats()[:2] == (2, 2) and engine.graphs_captured == 3
+    engine.cache.check()
+
+
 def write_tokenizer(folder, vocab, renamed=None):
     """A tokenizer.json of whole words w0, w1, ... and the chat format's special tokens, written
     with the tokenizers package; the model's last ids are the specials. `renamed`: {id: word} for
