@@ -371,6 +371,34 @@ def test_decode_graphs_and_their_logits_are_bounded(model_root, monkeypatch):
     engine.cache.check()
 
 
+def test_generation_of_an_unequal_batch_whose_sequences_end_one_after_another(model_root):
+    """The generation loop over one long prompt beside short ones, greedy, in bfloat16: the decode
+    steps run one ahead of the host, as graphs, with the attention's grid dealt out by a list, and
+    the caller ends the sequences at different counts, so that the batch shrinks step by step. Every
+    token is at or near the top of what the plain implementation says for its place."""
+    from herbert_rs_amd.sampling import SamplingParams
+    folder = make_folder(model_root, "D", "bfloat16")
+    vocab = CONFIGS["D"][0]["vocab_size"]
+    prompts = [random_tokens(vocab, n, 800 + n) for n in (1500, 20, 300, 64, 5)]
+    ends = [6, 25, 12, 30, 18]
+    engine = hb.load(folder, dtype="bfloat16", cache_tokens=64 * 40)
+    count = [0] * len(prompts)
+
+    def on_token(i, tok):
+        count[i] += 1
+        return "enough" if count[i] >= ends[i] else None
+    res = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=40, ignore_eos=True, repeat_check=False),
+                          on_token=on_token)
+    assert [len(r.tokens) for r in res] == ends and engine.graphs_captured >= 4
+    assert any(st.static.range_lists for st in engine._decode.values())           # the list was what ran
+    for p, r in zip(prompts, res):
+        ref = plain_logits(folder, p + r.tokens)
+        for k, tok in enumerate(r.tokens):
+            row = ref[len(p) + k - 1]
+            assert float(row.max() - row[tok]) <= 0.05 * float(row.std()), (len(p), k)
+    engine.cache.check()
+
+
 def test_a_larger_batch_makes_a_larger_logits_buffer(model_root):
     """The decode steps' one logits buffer has 64 rows at first; a batch of 70 sequences makes one
     of 128 (every graph is dropped with the old one), and steps of 3, of 70 and of 3 again say
