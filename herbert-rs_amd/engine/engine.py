@@ -80,6 +80,7 @@ class Engine:
         self._decode = OrderedDict()    # batch size -> _DecodeState, least recently used first
         self._graphs = OrderedDict()    # (batch size, context bucket, unequal) -> graph, least recently used first
         self._shared_logits = None      # [rows, vocab], made by the first decode step, grown by a larger batch
+        self._capture_stream = None     # the stream that graphs are captured on
         self.graphs_captured = 0
         self.ignored_tensors = []       # stored tensors that the model did not ask for
         self._tensor_source = None      # how get_tensor finds a tensor again: set by the constructors below
@@ -274,12 +275,25 @@ class Engine:
         state.seen[key[1:]] = seen + 1
         if seen == 0:       # eager: also sizes every scratch buffer
             return self.model.forward(self.rt, meta, self.cache, logits_out=state.logits)
-        torch.cuda.synchronize(self.device)      # also: no graph that is dropped below still runs
-        while len(self._graphs) >= MAX_GRAPHS:
-            self._graphs.popitem(last=False)
+        if len(self._graphs) >= MAX_GRAPHS:
+            torch.cuda.synchronize(self.device)      # no graph that is dropped here still runs
+            while len(self._graphs) >= MAX_GRAPHS:
+                self._graphs.popitem(last=False)
+        # Captured on a stream of its own behind what the step's stream holds, without waiting for
+        # the GPU: the host records the kernels while the steps before still run. (torch.cuda.graph
+        # as a context would first wait for the GPU and hand every cached block back to the driver.)
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            self.model.forward(self.rt, meta, self.cache, logits_out=state.logits)
+        if self._capture_stream is None:
+            self._capture_stream = torch.cuda.Stream(self.device)
+        step_stream = torch.cuda.current_stream(self.device)
+        self._capture_stream.wait_stream(step_stream)
+        with torch.cuda.stream(self._capture_stream):
+            graph.capture_begin()
+            try:
+                self.model.forward(self.rt, meta, self.cache, logits_out=state.logits)
+            finally:
+                graph.capture_end()
+        step_stream.wait_stream(self._capture_stream)
         self._graphs[key] = graph
         self.graphs_captured += 1
         graph.replay()
