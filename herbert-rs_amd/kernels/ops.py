@@ -51,22 +51,25 @@ def _stream():
 
 
 def _check(t, name, dtype=None, shape=None):
+    """Refuse what a kernel must not be given: not a contiguous GPU tensor, another dtype, another
+    shape (None in `shape`: any size). Called for every operand of every launch, hence the short
+    way through for what is right."""
+    try:
+        if t.is_cuda and t.is_contiguous() and (dtype is None or t.dtype == dtype):
+            if shape is None or t.shape == shape:
+                return
+            got = t.shape
+            if len(shape) == len(got) and all(s is None or s == d for s, d in zip(shape, got)):
+                return
+    except AttributeError:
+        pass
     if not isinstance(t, torch.Tensor) or not t.is_cuda:
         raise BackendError(f"{name} must be a tensor on the GPU")
     if not t.is_contiguous():
         raise BackendError(f"{name} must be contiguous")
     if dtype is not None and t.dtype != dtype:
         raise BackendError(f"{name} must be {dtype}, got {t.dtype}")
-    if shape is not None:
-        got = t.shape
-        bad = len(shape) != len(got)
-        if not bad:
-            for s, d in zip(shape, got):
-                if s is not None and s != d:
-                    bad = True
-                    break
-        if bad:
-            raise BackendError(f"{name} must have shape {list(shape)}, got {list(got)}")
+    raise BackendError(f"{name} must have shape {list(shape)}, got {list(t.shape)}")
 
 
 def _ptr(t):

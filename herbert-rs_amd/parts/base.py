@@ -49,6 +49,7 @@ class Runtime:
         self.dtype = dtype
         self.device = torch.device(device)
         self._buffers = {}
+        self._views = {}         # (name, dtype, shape) -> the view of the buffer that was handed out last
         self._outgrown = []      # never freed: a captured graph may hold their addresses
 
     @property
@@ -61,6 +62,10 @@ class Runtime:
         buffer that has become too small is replaced by one at least twice as large and kept all
         the same (a captured graph may still write to it): what is kept is less than what is in use."""
         dtype = dtype or self.dtype
+        shape = tuple(shape)
+        view = self._views.get((name, dtype, shape))      # the same request as before: the same tensor
+        if view is not None:
+            return view
         n = 1
         for s in shape:
             n *= int(s)
@@ -74,7 +79,12 @@ class Runtime:
                 n_new = max(n, 1)
             buf = torch.empty(n_new, dtype=dtype, device=self.device)
             self._buffers[key] = buf
-        return buf[:n].view(*shape)
+            for old in [k for k in self._views if k[0] == name and k[1] == dtype]:
+                del self._views[old]                       # views of the buffer that was replaced
+        if len(self._views) > 4096:
+            self._views.clear()
+        view = self._views[(name, dtype, shape)] = buf[:n].view(*shape)
+        return view
 
     def weight(self, t, matrix=True):
         """A stored tensor as the kernels read it: matrices in the compute dtype, scales in float32."""
