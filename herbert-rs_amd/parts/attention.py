@@ -17,7 +17,7 @@ import math
 import torch
 
 from ..cache import KVNeed
-from ..kernels import ops
+from ..kernels import mfma, ops
 from ..weights import TensorNeed
 from .base import Part
 from .linear import Linear
@@ -113,7 +113,6 @@ class Attention(Part):
         rot = self.position.rotation()
         cos, sin, rot_dims = rot if rot is not None else (None, None, 0)
         if write_kv and fused_norm is None and row_scale is None and rt.dtype == torch.bfloat16:
-            from ..kernels import mfma
             if mfma.gemm_qkv_fusable(y, self.qkv.weight, ctx.meta, kv, self.nq, self.nkv, self.hd, rot_dims):
                 # a long prompt: the projection norms, rotates and writes the cache in its epilogue
                 q = rt.buffer("q", (T, self.q_dim))
@@ -126,7 +125,6 @@ class Attention(Part):
         qkv = rt.buffer("qkv", (T, width), torch.float32)
         fused_decode = False
         if write_kv and rt.dtype == torch.bfloat16:
-            from ..kernels import mfma
             fused_decode = mfma.decode_fusable(ctx.meta, kv, self.nq, self.nkv, self.hd, rot_dims, rt.dtype)
         slices = None
         if fused_norm is not None:
@@ -153,7 +151,6 @@ class Attention(Part):
 
     def attend(self, ctx, q, kv, out):
         if q.dtype == torch.bfloat16:
-            from ..kernels import mfma
             if mfma.attention_supported(q, kv, self.nq, self.nkv, self.hd):
                 mfma.attention(q, ctx.meta, kv, out, self.nq, self.nkv, self.hd, self.scale, self.window)
                 return

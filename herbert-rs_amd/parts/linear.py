@@ -8,7 +8,7 @@ the plain kernel (same storage types, float32 arithmetic) does the rest from row
 """
 import torch
 
-from ..kernels import ops
+from ..kernels import mfma, ops
 
 
 class Linear:
@@ -18,7 +18,6 @@ class Linear:
         self.packed = False
         if pack and weight.dtype == torch.bfloat16 and weight.is_cuda \
                 and self.out_features % 16 == 0 and self.in_features % 32 == 0:
-            from ..kernels import mfma
             weight = mfma.pack_weight(weight)
             self.packed = True
         self.weight = weight
@@ -29,7 +28,6 @@ class Linear:
         defer_slices: the caller's next kernel can add up slices of K; returns what kernels.mfma.gemm
         returns for it, (1, pointer to out, 0) if the product is whole."""
         if self.weight.dtype == torch.bfloat16 and a.dtype == torch.bfloat16:
-            from ..kernels import mfma
             if self.packed or mfma.gemm_supported(a, self.weight, out):
                 return mfma.gemm(a, self.weight, out, accumulate, packed=self.packed, leave=leave,
                                  row_scale=row_scale, defer_slices=defer_slices)
@@ -43,35 +41,29 @@ class Linear:
         (the next product finishes it), "whole" or None; see kernels.mfma.norm_handoff."""
         if self.weight.dtype != torch.bfloat16:
             return None
-        from ..kernels import mfma
         return mfma.norm_handoff(rows, self.out_features, self.in_features)
 
     def finishes_norm(self, rows):
         """True if this product can take rows that are half normed (bf16(x * g) and sums of squares)."""
         if self.weight.dtype != torch.bfloat16 or self.in_features % 32:
             return False
-        from ..kernels import mfma
         return rows <= mfma.NORM_HANDOFF_MAX_M
 
     @staticmethod
     def handed_rows(rows):
         """Rows of the sums of squares that go with a handed-on norm of that many rows."""
-        from ..kernels import mfma
         return mfma.padded_rows(rows)
 
     def forward_swiglu(self, a, out, norm=None, row_scale=None):
         """out bf16 [M, N / 2] = silu(gate) * up for a weight whose rows are gate/up interleaved."""
-        from ..kernels import mfma
         mfma.gemm_swiglu(a, self.weight, out, packed=self.packed, norm=norm, row_scale=row_scale)
 
     def fuses_norm(self, x):
         """True if RMSNorm(x) @ W^T runs as one kernel for this input (few rows, bfloat16 weights)."""
         if self.weight.dtype != torch.bfloat16:
             return False
-        from ..kernels import mfma
         return mfma.norm_fusable(x, self.weight)
 
     def forward_normed(self, x, norm_weight, eps, out):
         """out[M, N] = RMSNorm(x; norm_weight, eps) @ W^T in one kernel (see fuses_norm)."""
-        from ..kernels import mfma
         mfma.gemm(x, self.weight, out, packed=self.packed, norm=(norm_weight, eps))

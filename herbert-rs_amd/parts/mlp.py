@@ -6,7 +6,7 @@ are read once.
 """
 import torch
 
-from ..kernels import ops
+from ..kernels import mfma, ops
 from ..weights import TensorNeed
 from .base import Part
 from .linear import Linear
@@ -36,7 +36,6 @@ class SwiGLU(Part):
         gate, up = rt.weight(tensors[n["gate"]]), rt.weight(tensors[n["up"]])
         # bfloat16 with sizes the MFMA kernel takes: gate and up rows interleaved so that the
         # product's epilogue applies silu(gate) * up and the float32 [T, 2I] never exists
-        from ..kernels import mfma
         self.fused_epilogue = (rt.dtype == torch.bfloat16 and self.intermediate_size % 16 == 0
                                and self.hidden_size % 32 == 0 and mfma.gemm_supported(
                                    gate[:1], gate, swiglu=True))
