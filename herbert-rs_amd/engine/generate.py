@@ -167,7 +167,7 @@ class Generator:
                 first.update(zip(ending, chooser.choose(logits, ending)))
         return [first[i] for i in live]
 
-    def _decode_ahead(self, live, slots, generated, params, chooser, take):
+    def _decode_ahead(self, live, slots, generated, params, chooser, take, kept=()):
         """Decoding with the host one step behind the GPU. The tokens that a step chooses stay on
         the GPU, and the next step is put on the stream with them at once, before the host has
         seen them; the host reads a step's tokens while the next one runs, so the GPU does not
@@ -175,8 +175,14 @@ class Generator:
         (end of sequence, a stop token, the caller's word) has then already been through one step
         more: that step's work on it is thrown away, its slot is given back as always, and every
         other sequence's tokens are what they would have been. Sequences that end for a reason the
-        host knows beforehand (max_tokens, the model's last position) are not taken ahead."""
+        host knows beforehand (max_tokens, the model's last position) are not taken ahead.
+        The step thrown away has also taken a draw from the sequence's generator stream: for a
+        sequence whose slot the caller keeps (`kept`: its chooser goes on into the next turn) the
+        streams are saved before every step that runs ahead (`chooser.save_streams`) and the
+        sequence's is put back when it ends, so that a seeded conversation draws what the
+        step-by-step loop draws, one draw a token."""
         eng = self.engine
+        saves = bool(kept) and hasattr(chooser, "save_streams")
 
         def launch(order, device_tokens):
             entries = [StepEntry(slots[i], [generated[i][-1]] if device_tokens is None else [0], [0])
@@ -193,11 +199,17 @@ class Generator:
             # the step after the one in flight, for the sequences that its token cannot end by count
             ahead = [i for i in order if i in slots and len(generated[i]) + 2 <= params.max_tokens
                      and eng.cache.length(slots[i]) < eng.spec.max_positions]
-            following = None
+            following = saved = None
             if ahead:
                 rows = [order.index(i) for i in ahead]
+                if saves:
+                    saved = chooser.save_streams()
                 following = launch(ahead, chooser.rows_of(pending, rows))
             take(order, chooser.read(pending), held)
+            if saved is not None:
+                for i in ahead:
+                    if i not in slots and i in kept:        # it ended on this token: the draw after it never was
+                        chooser.restore_stream(i, saved)
             if not live or following is None:
                 break
             order, (pending, held) = ahead, following
@@ -280,7 +292,7 @@ class Generator:
             if self.run_ahead and getattr(chooser, "can_run_ahead", False) and \
                     getattr(eng, "accepts_device_tokens", False) and \
                     (not kept or getattr(eng.cache, "rolls_back_freely", False)):
-                self._decode_ahead(live, slots, generated, params, chooser, take)
+                self._decode_ahead(live, slots, generated, params, chooser, take, kept)
             else:
                 while live:
                     order = list(live)

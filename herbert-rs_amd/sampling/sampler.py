@@ -56,6 +56,15 @@ class Sampler:
         for t in self.think or ():
             t.reset()
 
+    def save_streams(self):
+        """A copy of every sequence's generator state as it is at this point of the stream (no
+        waiting): for a caller that may have to take a draw back (`restore_stream`)."""
+        return self.states.clone()
+
+    def restore_stream(self, sequence, saved):
+        """Put sequence `sequence`'s generator state back to what `saved` (a `save_streams`) holds."""
+        self.states[sequence:sequence + 1].copy_(saved[sequence:sequence + 1])
+
     def _sifted_for(self, rows):
         """Buffers for the candidates that a block a chunk sifts out of a long row (top-k up to 1024)."""
         p = self.params

@@ -19,9 +19,14 @@ F32_ABS = 1e-4
 #    fault that shifts a row coherently shows here first;
 #  - the largest error: the maximum of V noisy values grows with V (about sqrt(2 ln V) times the
 #    rms: 0.017 to 0.033 for vocabularies of 256 to 512, 0.043 to 0.051 for 151936).
-# ("random": the drawn configurations of test_random_configs_gpu, worst seen 0.011 and 0.036)
-BF16_REL_L2 = {"A": 0.012, "B": 0.018, "C": 0.018, "D": 0.02, "F": 0.02, "wide": 0.02, "odd": 0.02, "random": 0.02}
-BF16_REL_RMS = {"A": 0.04, "B": 0.05, "C": 0.05, "D": 0.05, "F": 0.05, "wide": 0.08, "odd": 0.04, "random": 0.06}
+# ("random": the drawn configurations of test_random_configs_gpu, worst seen 0.011 and 0.036;
+#  "long": contexts of 9,000 to 17,000 tokens with scores scaled up so that a few far keys hold a
+#  query's weight, which also carries the rounding of those scores into the output: worst seen
+#  0.0146 and 0.050; "deep": 1 to 36 layers at a quarter of the 8B width, vocabulary 4096: 0.0084 and
+#  0.037 for one layer, 0.0114 and 0.050 for 36: the error hardly grows with depth, and in float32
+#  it goes from 9e-6 for one layer to 1.1e-5 for 36)
+BF16_REL_L2 = {"A": 0.012, "B": 0.018, "C": 0.018, "D": 0.02, "F": 0.02, "wide": 0.02, "odd": 0.02, "random": 0.02, "long": 0.025, "deep": 0.02}
+BF16_REL_RMS = {"A": 0.04, "B": 0.05, "C": 0.05, "D": 0.05, "F": 0.05, "wide": 0.08, "odd": 0.04, "random": 0.06, "long": 0.08, "deep": 0.08}
 
 
 def rel_rms_error(got, ref):

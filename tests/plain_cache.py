@@ -22,11 +22,14 @@ def plain_logits(folder, tokens):
 def plain_rows(folder, tokens, rows):
     """{position: float32 logits [vocab]} at `rows` only (for models whose vocabulary makes every
     position's logits too much to keep)."""
-    if folder not in _folders:
-        _folders[folder] = plain_model.read_folder(folder, torch.float32)
-    cfg, w = _folders[folder]
     rows = sorted(set(rows))
-    out = plain_model.forward(cfg, w, list(tokens), rows=rows).numpy().astype(np.float32)
+    key = (folder, tuple(tokens), tuple(rows))
+    if key not in _logits:
+        if folder not in _folders:
+            _folders[folder] = plain_model.read_folder(folder, torch.float32)
+        cfg, w = _folders[folder]
+        _logits[key] = plain_model.forward(cfg, w, list(tokens), rows=rows).numpy().astype(np.float32)
+    out = _logits[key]
     return {p: out[i] for i, p in enumerate(rows)}
 
 

@@ -579,6 +579,52 @@ def test_turns_on_a_kept_slot_go_on_from_what_it_holds(ahead, rolls_back):
     assert eng.cache.slots.held_count == 0
 
 
+class CountingChooser(AheadChooser):
+    """Counts the draws that each sequence's generator stream has given, as the GPU sampler's
+    states advance once a choice."""
+
+    def __init__(self, params, n, vocab, device):
+        super().__init__(params, n, vocab, device)
+        self.draws = [0] * n
+
+    def choose(self, logits, sequence_indices):
+        for i in sequence_indices:
+            self.draws[i] += 1
+        return super().choose(logits, sequence_indices)
+
+    def save_streams(self):
+        return list(self.draws)
+
+    def restore_stream(self, sequence, saved):
+        self.draws[sequence] = saved[sequence]
+
+
+@pytest.mark.parametrize("ahead", [False, True])
+def test_a_turn_on_a_kept_slot_takes_one_draw_a_token(ahead):
+    """A turn that ends on a token's value has been through one step more when the loop runs ahead
+    of the host, and that step has drawn from the sequence's generator: the draw is taken back,
+    so that the next turn of a seeded conversation draws what it draws step by step. A turn that
+    ends by count is not taken ahead and has nothing to take back."""
+    eng = KeepingEngine(ahead, True)
+    CountingChooser.unread = 0
+    gen = Generator(eng, max_batch=1, make_chooser=CountingChooser)
+    chooser = CountingChooser(None, 1, 50, "cpu")
+    slot = eng.alloc_slot()
+    r1 = gen.extend(slot, [35, 5], SamplingParams(temperature=0.0, max_tokens=10, repeat_check=False), chooser)
+    assert r1.tokens == [6, 7, 8, 9] and r1.stop_reason == EOS
+    assert eng.rolled_back == (1 if ahead else 0)
+    assert chooser.draws == [4]
+    CountingChooser.unread = 0           # (the step that ran ahead for nothing was never read)
+    r2 = gen.extend(slot, [9, 20], SamplingParams(temperature=0.0, max_tokens=3, repeat_check=False), chooser)
+    assert r2.tokens == [21, 22, 23] and r2.stop_reason == MAX_TOKENS and chooser.draws == [7]
+    # a batch of the loop's own slots does not save anything: those streams end with their sequences
+    CountingChooser.unread = 0
+    got = Generator(AheadEngine(), max_batch=2, make_chooser=CountingChooser).generate(
+        [[5], [30]], SamplingParams(temperature=0.0, max_tokens=6, repeat_check=False))
+    assert [r.stop_reason for r in got] == [EOS, MAX_TOKENS]
+    eng.free_slot(slot)
+
+
 class WordTokenizer:
     """Words and the specials of a chat template as tokens; ids grow as words are first seen."""
     SPECIALS = ["<|im_start|>", "<|im_end|>", "\n"]

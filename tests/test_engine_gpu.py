@@ -715,19 +715,30 @@ def test_sampling_through_generate_is_reproducible(model_root):
     b = hb.generate(folder, prompts, **kw)
     c = hb.generate(folder, prompts, **dict(kw, seed=8))
     assert a == b and a != c and all(len(t) == 12 for t in a)
-    # the first request's tokens are those of the reference's one sampler with that seed
+    # every request's tokens are those of the reference's sampler on the plain model's logits, each
+    # request with the stream of its own seed (the first with the seed itself): every token of all
+    # four; another token only where the draw lies within rounding of a boundary between two
+    # candidates, and the comparison then goes on from the engine's token
+    from herbert_rs_amd.sampling import xorshift
     cfg, w = plain_folder(folder)
-    rng = plain_sampler.XorShift64(7)
-    seq = list(prompts[0])
-    for tok in a[0]:
-        logits = plain.forward(cfg, w, seq)[-1].numpy()
-        work = plain_sampler.candidates(logits, 0.7, 20, 1.0)
-        u = rng.next_f32()
-        want = plain_sampler.pick(work, u)
-        if tok != want:                                       # only at a rounding-level tie
-            assert tok in [i for i, _ in work]
-            break
-        seq.append(tok)
+    excused = 0
+    for i, (prompt, tokens) in enumerate(zip(prompts, a)):
+        rng = plain_sampler.XorShift64(xorshift.sequence_seed(7, i))
+        seq = list(prompt)
+        for n, tok in enumerate(tokens):
+            logits = plain.forward(cfg, w, seq)[-1].numpy()
+            work = plain_sampler.candidates(logits, 0.7, 20, 1.0)
+            u = rng.next_f32()
+            want = plain_sampler.pick(work, u)
+            if tok != want:
+                cum, near = np.float32(0), False
+                for _, p in work:
+                    cum = np.float32(cum + p)
+                    near = near or abs(float(cum) - float(u)) < 1e-5
+                assert near and tok in [j for j, _ in work], (i, n, tok, want)
+                excused += 1
+            seq.append(tok)
+    assert excused <= 2
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
