@@ -11,7 +11,11 @@ over a decode from 512 to the full context (`..._mean...`, from steps timed at a
 in between); and the other two workloads of the benchmark description through the generation
 loop (`qwen3_1p7b_...`, `qwen3_32b_...`); `decode_b8_host_between_steps` is the headline's step
 with the host reading each step's tokens before it starts the next; `decode_b16_unequal_lengths` is a batch of one
-sequence at the full context beside fifteen of a sixteenth of it. Weights are random, token ids are random, and the
+sequence at the full context beside fifteen of a sixteenth of it; and, unless --no-long, further sizes and
+lengths: decode at batch 8 at 16,384 and 32,768 tokens of context, at batch 64 at 16,384 (155 GB of keys and
+values: 32,768 would not fit beside the weights), at batch 128 and 256 at the full context, and prompts of 8,192,
+16,384 and 32,768 tokens fed in chunks of 8,192 (`decode_b8_ctx16384...`, `decode_b128...`, `prefill_8192`,
+`prefill_8192_frac`, ...). Weights are random, token ids are random, and the
 cache below the timed steps is filled by real prefill steps of random prompts. A timed decode
 step is what the generation loop does for a token: the step function (a HIP-graph replay), the
 greedy choice on the GPU, and the chosen tokens read by the host, which as in that loop reads
@@ -146,6 +150,8 @@ def main():
     ap.add_argument("--no-workloads", action="store_true",
                     help="skip the 1.7B and 32B workloads that the default run adds to `points`")
     ap.add_argument("--no-sweep", action="store_true", help="time the full context only, not 512 and the mean")
+    ap.add_argument("--no-long", action="store_true",
+                    help="skip the further sizes and lengths (contexts of 16 K and 32 K, batch 128 and 256, long prompts)")
     ap.add_argument("--workload", default="headline", choices=["headline", "qwen3-1.7b", "qwen3-32b"],
                     help="headline: BASELINE.json configs[2]; the others: configs[3] and configs[4]")
     ap.add_argument("--prefill-tokens", type=int, default=2048, help="length of the prompt of the prefill figure")
@@ -181,13 +187,20 @@ def main():
     shape.pop("context", None)
     layers_full = shape["num_hidden_layers"]
     layers = args.layers or layers_full
+    long_points = not (args.no_points or args.no_long or unequal or args.prefill_only)
+    LONG_CONTEXTS, LONG_BATCHES, LONG_PROMPTS, LONG_CHUNK = (16384, 32768), (128, 256), (8192, 16384, 32768), 8192
+    longest = max(LONG_CONTEXTS + LONG_PROMPTS) if long_points else 0
     raw = dict(shape, architectures=["Qwen3ForCausalLM"], model_type="qwen3",
-               num_hidden_layers=layers, max_position_embeddings=max(context, 4096, args.prefill_tokens) + 64,
+               num_hidden_layers=layers, max_position_embeddings=max(context, 4096, args.prefill_tokens, longest) + 64,
                eos_token_id=151645)
     cfg = hb.Qwen3Config.from_dict(raw)
     torch.cuda.set_device(0)
     max_batch = args.batch if args.no_points else max(args.batch, 64)
     cache_tokens = max(max_batch * (context + 64), args.prefill_tokens + 64)
+    if long_points:
+        max_batch = max(max_batch, max(LONG_BATCHES))
+        cache_tokens = max(cache_tokens, max(LONG_BATCHES) * (context + 64), 64 * (LONG_CONTEXTS[0] + 64),
+                           args.batch * (LONG_CONTEXTS[1] + 64))
     if unequal:
         cache_tokens = sum((c + 127) // 64 * 64 for c in unequal)
     t0 = time.time()
@@ -207,7 +220,7 @@ def main():
     def step_gbs(batch, mean_context, ms):
         return (weight_bytes + batch * mean_context * kv_bytes_per_token) / (ms * 1e-3) / 1e9
 
-    def decode_run(batch, plan, run_ahead=True):
+    def decode_run(batch, plan, run_ahead=True, fill_chunk=2048):
         """[(context, tokens/s, ms/step)] for each (context, steps, warmup) of `plan` (contexts
         ascending): `steps` timed decode steps at `batch` after `warmup` untimed ones, ending with
         every sequence holding `context` tokens; one pass over a cache that is filled by real
@@ -215,7 +228,7 @@ def main():
         slots = [engine.alloc_slot() for _ in range(batch)]
         chooser = Sampler(SamplingParams(temperature=0.0), batch, V, engine.device)
         tokens = [ids(1)[0] for _ in range(batch)]
-        held, chunk, out = 0, 2048, []
+        held, chunk, out = 0, fill_chunk, []
 
         ahead = [None]
 
@@ -223,13 +236,13 @@ def main():
             """A decode step as the generation loop runs it: put on the stream with the tokens of the
             step before still on the GPU, whose copy the host reads while this step runs."""
             if not run_ahead:       # the host reads a step's tokens before it starts the next
-                logits = engine.step([StepEntry(s, [t], [0]) for s, t in zip(slots, tokens)])
+                logits = engine.step([StepEntry(s, [t], [0]) for s, t in zip(slots, tokens)], keep_logits=False)
                 return chooser.choose(logits, range(batch))
             before = ahead[0]
             if before is None:
-                logits = engine.step([StepEntry(s, [t], [0]) for s, t in zip(slots, tokens)])
+                logits = engine.step([StepEntry(s, [t], [0]) for s, t in zip(slots, tokens)], keep_logits=False)
             else:
-                logits = engine.step([StepEntry(s, [0], [0]) for s in slots], tokens_on_device=before.device)
+                logits = engine.step([StepEntry(s, [0], [0]) for s in slots], tokens_on_device=before.device, keep_logits=False)
             ahead[0] = chooser.choose_ahead(logits, range(batch))
             return tokens if before is None else chooser.read(before)
         for c, steps, warmup in plan:
@@ -253,24 +266,28 @@ def main():
             engine.free_slot(s)
         return out
 
-    def prefill_once(tokens_n):
+    def prefill_once(tokens_n, chunk=None):
         """One prompt of tokens_n tokens, whole or in chunks; the last token's logits are asked for."""
         slot = engine.alloc_slot()
-        chunk = args.prefill_chunk or tokens_n
+        chunk = chunk or args.prefill_chunk or tokens_n
         prompt = ids(tokens_n)
         for a in range(0, tokens_n, chunk):
             part = prompt[a:a + chunk]
             engine.step([StepEntry(slot, part, [len(part) - 1] if a + chunk >= tokens_n else [])])
         engine.free_slot(slot)
 
-    def prefill_run(tokens_n, reps):
-        prefill_once(tokens_n)
+    def prefill_run(tokens_n, reps, chunk=None, warm=True):
+        if warm:
+            prefill_once(tokens_n, chunk)
         torch.cuda.synchronize()
         t = time.perf_counter()
         for _ in range(reps):
-            prefill_once(tokens_n)
+            prefill_once(tokens_n, chunk)
         torch.cuda.synchronize()
         return (time.perf_counter() - t) / reps
+
+    def prefill_flops(T):
+        return 2.0 * T * (layers * per_layer) + 2.0 * V * H + layers * 4.0 * cfg.q_dim * T * (T + 1) / 2.0
 
     def unequal_run(contexts, steps, warmup):
         """(ms a step, GB/s) of one batch whose sequences hold `contexts` tokens after the timed
@@ -283,12 +300,12 @@ def main():
             for a in range(0, fill, 2048):
                 engine.step([StepEntry(s, ids(min(2048, fill - a)), [])])
         chooser = Sampler(SamplingParams(temperature=0.0), len(slots), V, engine.device)
-        ahead = chooser.choose_ahead(engine.step([StepEntry(s, ids(1), [0]) for s in slots]), range(len(slots)))
+        ahead = chooser.choose_ahead(engine.step([StepEntry(s, ids(1), [0]) for s in slots], keep_logits=False), range(len(slots)))
         for n in (warmup - 1, steps):
             torch.cuda.synchronize()
             t = time.perf_counter()
             for _ in range(n):
-                logits = engine.step([StepEntry(s, [0], [0]) for s in slots], tokens_on_device=ahead.device)
+                logits = engine.step([StepEntry(s, [0], [0]) for s in slots], tokens_on_device=ahead.device, keep_logits=False)
                 before, ahead = ahead, chooser.choose_ahead(logits, range(len(slots)))
                 chooser.read(before)
             torch.cuda.synchronize()
@@ -390,17 +407,36 @@ def main():
     if not args.no_points:
         T = args.prefill_tokens
         sec = prefill_run(T, 5)
-        flops = 2.0 * T * (layers * per_layer) + 2.0 * V * H \
-            + layers * 4.0 * cfg.q_dim * T * (T + 1) / 2.0
         peak = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
         out["prefill"] = {"value": round(T / sec, 1), "tokens": T, "ms": round(sec * 1e3, 3),
-                          "frac": round(flops / sec / peak, 4)}
+                          "frac": round(prefill_flops(T) / sec / peak, 4)}
         print(f"[bench] prefill {T}: {T / sec:.0f} tok/s", file=sys.stderr, flush=True)
         for batch in (1, 64):
             if batch != args.batch:
                 r = measure(batch)
                 add_points(points, batch, r)
                 print(f"[bench] decode b{batch}: {r[0][0]:.1f} tok/s, {r[0][1]:.3f} ms/step", file=sys.stderr, flush=True)
+        if long_points:
+            # further sizes and lengths, each in one pass over a cache filled by prefill in chunks
+            for T in LONG_PROMPTS:
+                sec = prefill_run(T, 2 if T <= 16384 else 1, chunk=LONG_CHUNK, warm=T == LONG_PROMPTS[0])
+                points[f"prefill_{T}"] = round(T / sec, 1)
+                points[f"prefill_{T}_frac"] = round(prefill_flops(T) / sec / peak, 4)
+                print(f"[bench] prefill {T} in chunks of {LONG_CHUNK}: {T / sec:.0f} tok/s", file=sys.stderr, flush=True)
+            few = min(args.steps, 12)
+
+            def add_long(batch, runs, label):
+                for c, v, ms_c in runs:
+                    key = f"decode_b{batch}" + (f"_ctx{c}" if label else "")
+                    gbs = step_gbs(batch, c - few / 2.0, ms_c)
+                    points[key], points[key + "_ms"] = round(v, 2), round(ms_c, 4)
+                    points[key + "_gbs"], points[key + "_frac"] = round(gbs, 1), round(gbs / HBM_GBS, 4)
+                    print(f"[bench] decode b{batch} at {c} tokens: {v:.1f} tok/s, {ms_c:.3f} ms/step", file=sys.stderr,
+                          flush=True)
+            add_long(args.batch, decode_run(args.batch, [(c, few, 3) for c in LONG_CONTEXTS], fill_chunk=LONG_CHUNK), True)
+            add_long(64, decode_run(64, [(LONG_CONTEXTS[0], few, 3)], fill_chunk=LONG_CHUNK), True)
+            for batch in LONG_BATCHES:
+                add_long(batch, decode_run(batch, [(context, few, 3)], fill_chunk=2048), False)
         if not args.no_workloads and not args.layers:
             del engine
             torch.cuda.empty_cache()

@@ -8,6 +8,12 @@ group's entries, so one table serves them all. A group with a window gives
 back the pages that no later query can see. A group of fixed-size state owns
 [entries, slots, *shape] and is cleared for a slot when the slot is taken.
 
+Beyond the slots and pages that sequences can hold there is one more of each:
+the padding slot (`Cache.pad_slot`), whose page table points at the padding page
+everywhere. Rows that fill a step up to a fixed size (a decode step that is
+replayed as a graph of the next larger batch size) write and read there and
+nowhere else; no sequence ever holds either.
+
 Per slot the host keeps the length (positions held = next position), as the
 reference keeps `seq_len` beside its storage
 (crates/backends/backend_common/src/kv_cache.rs:270-273).
@@ -38,12 +44,14 @@ class KVGroup:
         self.entries = list(entries)
         self.pages = FreeList(n_pages, "page")
         self.pages_per_slot = pages_for(max_positions)
-        self.pool = torch.zeros((len(self.entries), 2, n_pages, need.kv_heads, PAGE_TOKENS,
+        # (one page and one slot more than sequences can hold: the padding page and the padding slot)
+        self.pool = torch.zeros((len(self.entries), 2, n_pages + 1, need.kv_heads, PAGE_TOKENS,
                                  need.head_dim), dtype=dtype, device=device)
         self.table_host = np.full((n_slots, self.pages_per_slot), -1, dtype=np.int32)
         # entries of the device table that are not held point at page 0: a kernel never reads
         # them for a valid position, and an index that is always in range cannot fault
-        self.table = torch.zeros((n_slots, self.pages_per_slot), dtype=torch.int32, device=device)
+        self.table = torch.zeros((n_slots + 1, self.pages_per_slot), dtype=torch.int32, device=device)
+        self.table[n_slots] = n_pages
         # a slot holds the logical pages [first_page, held_end): it fills from the front as it grows,
         # a window gives pages back at the front, a roll-back at the end
         self.first_page = np.zeros(n_slots, dtype=np.int64)
@@ -51,7 +59,7 @@ class KVGroup:
 
     def view(self, entry):
         i = self.entries.index(entry)
-        n_pages = self.pool.shape[2]
+        n_pages = self.pool.shape[2]         # (with the padding page)
         k = self.pool[i, 0]
         v = self.pool[i, 1].view(n_pages, self.need.kv_heads, self.need.head_dim, PAGE_TOKENS)
         return LayerKV(k, v, self.table, PAGE_TOKENS, int(self.need.window or 0))
@@ -124,8 +132,8 @@ class StateGroup:
     def __init__(self, need, entries, n_slots, device):
         self.need = need
         self.entries = list(entries)
-        self.data = torch.zeros((len(self.entries), n_slots) + tuple(need.shape), dtype=need.dtype,
-                                device=device)
+        self.data = torch.zeros((len(self.entries), n_slots + 1) + tuple(need.shape), dtype=need.dtype,
+                                device=device)      # (the last: the padding slot's)
 
     def view(self, entry):
         return self.data[self.entries.index(entry)]
@@ -148,6 +156,7 @@ class Cache:
         self.n_pages = n_pages
         self.n_slots = int(max_slots) if max_slots else n_pages
         self.max_positions = int(max_positions)
+        self.pad_slot = self.n_slots        # never handed out: where a step's padding rows write and read
         self.slots = FreeList(self.n_slots, "slot")
         self.lengths = np.zeros(self.n_slots, dtype=np.int64)
         self.kv_groups = {}
@@ -171,6 +180,29 @@ class Cache:
                     self._state_of.setdefault(e, []).append(group)
             else:
                 raise CacheError(f"unknown cache need {need!r}")
+
+    @staticmethod
+    def bytes_needed(needs, max_tokens, dtype, max_slots=None):
+        """The GPU memory that a cache of these needs takes: the pools of keys and values (by
+        pages) and the fixed-size state (by slots), as the constructor allocates them."""
+        n_pages = pages_for(max(int(max_tokens), 1))
+        n_slots = (int(max_slots) if max_slots else n_pages) + 1        # with the padding slot
+        n_pages += 1                                                     # and the padding page
+        element = torch.empty((), dtype=dtype).element_size()
+        by_need = {}
+        for entry, need in needs.items():
+            for one in (need if isinstance(need, (tuple, list)) else (need,)):
+                by_need[one] = by_need.get(one, 0) + 1
+        total = 0
+        for need, entries in by_need.items():
+            if isinstance(need, KVNeed):
+                total += entries * 2 * n_pages * PAGE_TOKENS * need.kv_heads * need.head_dim * element
+            elif isinstance(need, StateNeed):
+                per_slot = 1
+                for d in need.shape:
+                    per_slot *= int(d)
+                total += entries * n_slots * per_slot * torch.empty((), dtype=need.dtype).element_size()
+        return total
 
     # ---- slots
     def alloc_slot(self):
@@ -221,6 +253,22 @@ class Cache:
         for slot, new_length in targets:
             for g in self.kv_groups.values():
                 g.ensure(slot, new_length)
+
+    def save_state(self, slots):
+        """A copy of the fixed-size state of `slots` (None for a cache that has none): what
+        `restore_state` puts back when the step that was to change it has failed."""
+        if not self.state_groups:
+            return None
+        index = torch.tensor(sorted(set(int(s) for s in slots)), dtype=torch.long)
+        saved = []
+        for g in self.state_groups.values():
+            at = index.to(g.data.device)
+            saved.append((g, at, g.data.index_select(1, at)))
+        return saved
+
+    def restore_state(self, saved):
+        for g, at, data in saved or ():
+            g.data.index_copy_(1, at, data)
 
     def unreserve(self, slot):
         """Give back what was reserved for a step that did not run: the pages behind the slot's

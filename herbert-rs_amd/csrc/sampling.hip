@@ -46,13 +46,17 @@ argmax_kernel(const float* __restrict__ logits, int ld, int V, int* __restrict__
         }
     } else {
         const float* row = logits + (size_t)r * ld;
+        bool nan_seen = false;
         for (int i = begin + threadIdx.x; i < end; i += blockDim.x) {
             const float v = row[i];
+            nan_seen |= v != v;
             if (v > bv) {
                 bv = v;
                 bi = i;
             }
         }
+        // nothing above -inf, but a NaN: a marker that wins over "nothing at all" among equals
+        if (nan_seen && bi == 0x7fffffff) bi = 0x7ffffffe;
     }
 #pragma unroll
     for (int off = HB_WAVE / 2; off > 0; off >>= 1) {
@@ -80,8 +84,10 @@ argmax_kernel(const float* __restrict__ logits, int ld, int V, int* __restrict__
             part_v[(size_t)r * chunks + blockIdx.y] = bv;
             part_i[(size_t)r * chunks + blockIdx.y] = bi;
         } else {
-            // a row without any value above -inf (or all NaN) gives index 0, as a scan from 0 would
-            out[r] = bi == 0x7fffffff ? 0 : bi;
+            // A row without any value above -inf gives index 0, as a scan from 0 would. If such a row
+            // holds a NaN (what a token id out of range leaves of a step: the embedding makes its row
+            // NaN) it gives -1, so that the host sees it instead of a token 0 that looks chosen.
+            out[r] = bi == 0x7fffffff ? 0 : bi == 0x7ffffffe ? -1 : bi;
         }
     }
 }

@@ -159,14 +159,26 @@ def pack(entries, start_lengths, device, staging=None):
         context_bucket=bucket(int(ctx.max())), unequal=unequal_level(ctx))
 
 
+def decode_batch_bucket(sequences):
+    """The batch size that a decode step of `sequences` sequences runs at: the next power of two.
+    The kernels' cost goes by classes of rows (up to 16, 32, 64, ...), not by the row; a batch whose
+    sequences end one after another then passes through 16, 8, 4, 2, 1 and not through every size
+    below its first, and each size is a shape that has to be run once by the host and captured."""
+    return 1 << max(0, int(sequences) - 1).bit_length()
+
+
 class StaticDecodeMeta:
     """The metadata of a step of B sequences with one token each, every logit wanted, in buffers
-    that stay where they are: a captured graph reads them, `update` refills them."""
+    that stay where they are: a captured graph reads them, `update` refills them. A step may
+    bring fewer sequences than B: the rows left over are padding, each a sequence of one token (id
+    0, position 0) in the cache's padding slot; what they compute is thrown away, and no other
+    row's result depends on them."""
 
     RANGE_LISTS = 4      # lists of ranges (BatchMeta.ranges_for) that the buffers have room for
 
-    def __init__(self, batch_size, device):
+    def __init__(self, batch_size, device, pad_slot=0):
         B = self.batch_size = batch_size
+        self.pad_slot = int(pad_slot)
         size = 7 * B + 1 + self.RANGE_LISTS * (B + 2)
         self.host = torch.zeros(size, dtype=torch.int32, pin_memory=torch.device(device).type == "cuda")
         self.copied = None       # event after the last copy out of `host`
@@ -195,7 +207,8 @@ class StaticDecodeMeta:
         if len(self.range_lists) == self.RANGE_LISTS:
             return None
         if self.dev.is_cuda and torch.cuda.is_current_stream_capturing():
-            raise RuntimeError("a list of ranges is first asked for while a graph is captured")
+            from ..errors import NeedsEagerStep
+            raise NeedsEagerStep("a list of ranges is first asked for while a graph is recorded")
         place = self._range_place(len(self.range_lists))
         self.range_lists.append((items, unit))
         self.host_array[place] = range_list(self.meta.host_context, items, unit)
@@ -203,16 +216,22 @@ class StaticDecodeMeta:
         return self.dev[place]
 
     def update(self, entries, start_lengths):
-        B = self.batch_size
+        B, n = self.batch_size, len(entries)
+        if n > B:
+            raise ValueError(f"{n} sequences do not fit a step of {B}")
         if self.copied is not None:
             self.copied.synchronize()        # the pinned buffer is free to be written again
         h = self.host_array
-        h[0:B] = [e.tokens[0] for e in entries]
-        h[B:2 * B] = start_lengths
-        h[3 * B:4 * B] = [e.slot for e in entries]
+        h[0:n] = [e.tokens[0] for e in entries]
+        h[B:B + n] = start_lengths
+        h[3 * B:3 * B + n] = [e.slot for e in entries]
+        if n < B:                            # padding rows
+            h[n:B] = 0
+            h[B + n:2 * B] = 0
+            h[3 * B + n:4 * B] = self.pad_slot
         context = h[5 * B + 1:6 * B + 1]
         np.add(h[B:2 * B], 1, out=context)
-        unequal = unequal_level(context)
+        unequal = unequal_level(context[:n])         # of the sequences themselves
         if unequal:                     # nobody reads the lists of a step whose sequences are alike
             for i, (items, unit) in enumerate(self.range_lists):
                 h[self._range_place(i)] = range_list(context, items, unit)

@@ -14,13 +14,13 @@ import torch
 
 from ..cache import Cache
 from ..config import load_config
-from ..errors import BackendError, ModelLoadError, RequestError
+from ..errors import BackendError, ModelLoadError, NeedsEagerStep, RequestError
 from ..parts import Runtime
 from ..weights import read_tensor, read_tensors
 from collections import OrderedDict
 
 from . import batch as batching
-from .batch import StaticDecodeMeta, StepEntry
+from .batch import StaticDecodeMeta, StepEntry, decode_batch_bucket
 from .model import Model
 
 _DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16,
@@ -34,7 +34,8 @@ class _DecodeState:
     def __init__(self, static, logits):
         self.static = static
         self.logits = logits
-        self.seen = {}          # (context bucket, unequal) -> eager steps run
+        self.seen = {}          # (context bucket, unequal) -> steps of that shape run so far
+        self.sized = False      # a step of this batch size has run outside a graph: its buffers exist
 
 
 # Captured graphs kept at any time, over all batch sizes and context buckets; the least recently
@@ -45,8 +46,7 @@ class _DecodeState:
 # graph: the cap leaves room for a few such batches' graphs, so that the next batch finds them.
 MAX_GRAPHS = 192
 # Decode steps write their logits into the first rows of one buffer [rows, vocab] float32 that the
-# engine keeps: what a decode step returns is therefore overwritten by the next decode step,
-# whatever its size. The buffer starts with this many rows (39 MB for a vocabulary of 151,936) or
+# engine keeps (`step` hands out a copy of them unless it is asked for the rows themselves). The buffer starts with this many rows (39 MB for a vocabulary of 151,936) or
 # as many as the cache has slots, if fewer; a larger batch makes a larger one (twice the rows, or
 # what the batch needs) and every graph, which holds the old one's address, is dropped.
 SHARED_LOGITS_ROWS = 64
@@ -72,10 +72,14 @@ class Engine:
         self.rt = Runtime(_DTYPES[dtype], self.device)
         self.model = Model(spec)
         self.model.load(tensors, self.rt)
-        self._check_cache_fits(max_tokens)
+        self._check_cache_fits(max_tokens, max_slots)
         self.cache = Cache(self.model.cache_needs(), max_tokens, spec.max_positions, self.rt.dtype,
                            self.device, max_slots)
         self.steps_run = 0
+        # Steps in which every sequence brings one token and wants its logits keep their metadata in
+        # fixed buffers and run at a power-of-two batch size (see _decode_step), as graphs if asked
+        # for: only for models whose parts do nothing but enqueue GPU work.
+        self.static_decode = self.model.graph_safe
         self.use_graphs = bool(use_graphs) and self.model.graph_safe
         self._decode = OrderedDict()    # batch size -> _DecodeState, least recently used first
         self._graphs = OrderedDict()    # (batch size, context bucket, unequal) -> graph, least recently used first
@@ -85,24 +89,17 @@ class Engine:
         self.ignored_tensors = []       # stored tensors that the model did not ask for
         self._tensor_source = None      # how get_tensor finds a tensor again: set by the constructors below
 
-    def _check_cache_fits(self, max_tokens):
+    def _check_cache_fits(self, max_tokens, max_slots=None):
         """Refuse a cache that the GPU's free memory cannot hold, in the library's own words,
-        before the allocator fails on it."""
-        from ..cache import KVNeed, PAGE_TOKENS
+        before the allocator fails on it: keys and values by pages, fixed-size state by slots."""
         if self.device.type != "cuda":
             return
-        pages = (max(int(max_tokens), 1) + PAGE_TOKENS - 1) // PAGE_TOKENS
-        element = 4 if self.rt.exact else 2
-        needed = 0
-        for need in self.model.cache_needs().values():
-            for one in (need if isinstance(need, (tuple, list)) else (need,)):
-                if isinstance(one, KVNeed):
-                    needed += 2 * pages * PAGE_TOKENS * one.kv_heads * one.head_dim * element
+        needed = Cache.bytes_needed(self.model.cache_needs(), max_tokens, self.rt.dtype, max_slots)
         free, _ = torch.cuda.mem_get_info(self.device)
         if needed > free:
             from ..errors import CacheError
-            raise CacheError(f"a cache of {max_tokens} tokens needs {needed / 2**30:.1f} GiB of keys and values, "
-                             f"{free / 2**30:.1f} GiB of GPU memory are free")
+            raise CacheError(f"a cache of {max_tokens} tokens needs {needed / 2**30:.1f} GiB of keys, values "
+                             f"and per-sequence state, {free / 2**30:.1f} GiB of GPU memory are free")
 
     # ---- construction
     @classmethod
@@ -168,12 +165,15 @@ class Engine:
 
     # ---- the step
     accepts_device_tokens = True
+    hands_out_copies = True         # `step(..., keep_logits=False)` gives the rows themselves
 
-    def step(self, entries, tokens_on_device=None):
+    def step(self, entries, tokens_on_device=None, keep_logits=True):
         """Run the entries' tokens; returns float32 logits [wanted, vocab] on the GPU
         (rows in the order of the entries and of their `want`), or None if nothing is wanted.
-        The logits of a step in which every sequence brings one token and wants its logits lie
-        in a buffer that the next such step writes again: copy what is to outlast it.
+        A step in which every sequence brings one token and wants its logits writes them into a
+        buffer of the engine's that the next such step writes again; what is returned is a copy
+        of the caller's own, unless `keep_logits` is false: then it is a view of that buffer, for
+        callers that are done with it before their next step (the generation loop).
         `tokens_on_device` (int32 [entries] on the GPU, every entry bringing one token): the
         tokens are taken from there, in the stream's order, and the entries' own are only
         placeholders; so a step can be put on the stream before the host has seen the tokens
@@ -182,7 +182,7 @@ class Engine:
             raise RequestError("a step needs at least one sequence")
         if tokens_on_device is not None:
             if (tokens_on_device.dtype != torch.int32 or tuple(tokens_on_device.shape) != (len(entries),)
-                    or not tokens_on_device.is_cuda or any(len(e.tokens) != 1 for e in entries)):
+                    or tokens_on_device.device != self.device or any(len(e.tokens) != 1 for e in entries)):
                 raise RequestError("tokens_on_device must be int32 [entries] on the engine's GPU, for entries "
                                    "of one token each")
         vocab = self.spec.vocab_size
@@ -216,9 +216,14 @@ class Engine:
             starts.append(start)
         # all pages of the step or none: a step that does not fit leaves the cache as it was
         self.cache.reserve_all([(e.slot, len(e.tokens)) for e in entries])
+        # fixed-size state is changed in place by the parts: what the step's slots hold is set aside
+        # first, so that a step that fails leaves them as they were (nothing for a cache without state)
+        state_before = self.cache.save_state([e.slot for e in entries])
         try:
-            if self.use_graphs and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
+            if self.static_decode and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
                 logits = self._decode_step(entries, starts, tokens_on_device)
+                if keep_logits:
+                    logits = logits.clone()
             else:
                 meta = batching.pack(entries, starts, self.device)
                 if tokens_on_device is not None:
@@ -227,6 +232,7 @@ class Engine:
         except Exception:
             for e in entries:       # nothing was committed: give back what was taken for the step
                 self.cache.unreserve(e.slot)
+            self.cache.restore_state(state_before)
             raise
         for e in entries:
             self.cache.commit(e.slot, len(e.tokens))
@@ -237,13 +243,17 @@ class Engine:
         """One token for each sequence, every logit wanted: the launch-bound case. The step's
         metadata lives in fixed buffers; from the second step of a shape on, the forward pass is a
         captured HIP graph that is replayed, so that the host launches one graph and not hundreds
-        of kernels. A graph is tied to the batch size, to the bucket of the longest context
+        of kernels. The step runs at the next power of two of its sequences, filled up with padding
+        rows in the cache's padding slot (the kernels' cost goes by classes of rows, and a batch
+        whose sequences end one after another then meets few new shapes instead of one a
+        sequence). A graph is tied to that batch size, to the bucket of the longest context
         (which sizes the attention grid) and to whether the contexts are of very unequal lengths
         (the attention then deals its grid out by a list). All graphs write their logits into the
         first rows of the engine's one buffer: what a step returns is overwritten by the next
         decode step. At most MAX_GRAPHS graphs and MAX_DECODE_BATCH_SIZES batch sizes are kept,
         the least recently used go first."""
-        B = len(entries)
+        n = len(entries)
+        B = decode_batch_bucket(n)          # the step runs at this size, the rows beyond n are padding
         state = self._decode.get(B)
         if state is None:
             if len(self._decode) >= MAX_DECODE_BATCH_SIZES:
@@ -256,30 +266,39 @@ class Engine:
                 torch.cuda.synchronize(self.device)     # nothing that writes the old buffer still runs
                 self._graphs.clear()
                 self._decode.clear()
-                rows = min(self.cache.n_slots, max(SHARED_LOGITS_ROWS, 2 * held, B))
+                rows = max(B, min(decode_batch_bucket(self.cache.n_slots), max(SHARED_LOGITS_ROWS, 2 * held)))
                 self._shared_logits = None
                 self._shared_logits = torch.empty((rows, self.spec.vocab_size), dtype=torch.float32,
                                                   device=self.device)
-            state = self._decode[B] = _DecodeState(StaticDecodeMeta(B, self.device), self._shared_logits[:B])
+            state = self._decode[B] = _DecodeState(StaticDecodeMeta(B, self.device, self.cache.pad_slot),
+                                                   self._shared_logits[:B])
         self._decode.move_to_end(B)
         meta = state.static.update(entries, starts)
         if tokens_on_device is not None:
-            meta.token_ids.copy_(tokens_on_device)      # behind the copy from the host, before the graph
+            meta.token_ids[:n].copy_(tokens_on_device)      # behind the copy from the host, before the graph
+        if not self.use_graphs:
+            return self.model.forward(self.rt, meta, self.cache, logits_out=state.logits)[:n]
         key = (B, meta.context_bucket, meta.unequal)
         graph = self._graphs.get(key)
         if graph is not None:
             self._graphs.move_to_end(key)
             graph.replay()
-            return state.logits
+            return state.logits[:n]
         seen = state.seen.get(key[1:], 0)
         state.seen[key[1:]] = seen + 1
-        if seen == 0:       # eager: also sizes every scratch buffer
-            return self.model.forward(self.rt, meta, self.cache, logits_out=state.logits)
+        if seen == 0 and not state.sized:
+            # the batch size's first step runs as it is: that also sizes every scratch buffer
+            state.sized = True
+            return self.model.forward(self.rt, meta, self.cache, logits_out=state.logits)[:n]
         if len(self._graphs) >= MAX_GRAPHS:
             torch.cuda.synchronize(self.device)      # no graph that is dropped here still runs
             while len(self._graphs) >= MAX_GRAPHS:
                 self._graphs.popitem(last=False)
-        # Captured on a stream of its own behind what the step's stream holds, without waiting for
+        # A shape whose batch size has run before is recorded at once, without a pass of its own
+        # outside a graph: the buffers are there. Where one turns out to be missing after all (a
+        # longer context's partial results, a list of ranges), the recording is given up and the
+        # step runs as it is; the shape's next step is then recorded.
+        # Recorded on a stream of its own behind what the step's stream holds, without waiting for
         # the GPU: the host records the kernels while the steps before still run. (torch.cuda.graph
         # as a context would first wait for the GPU and hand every cached block back to the driver.)
         graph = torch.cuda.CUDAGraph()
@@ -287,17 +306,30 @@ class Engine:
             self._capture_stream = torch.cuda.Stream(self.device)
         step_stream = torch.cuda.current_stream(self.device)
         self._capture_stream.wait_stream(step_stream)
-        with torch.cuda.stream(self._capture_stream):
-            graph.capture_begin()
-            try:
-                self.model.forward(self.rt, meta, self.cache, logits_out=state.logits)
-            finally:
-                graph.capture_end()
+        try:
+            with torch.cuda.stream(self._capture_stream):
+                graph.capture_begin()
+                try:
+                    self.model.forward(self.rt, meta, self.cache, logits_out=state.logits)
+                finally:
+                    graph.capture_end()
+        except NeedsEagerStep:
+            step_stream.wait_stream(self._capture_stream)
+            del graph
+            return self.model.forward(self.rt, meta, self.cache, logits_out=state.logits)[:n]
+        except Exception:
+            # Nothing of a failed recording has run. The two streams are joined again, and the shape
+            # starts over: its next step runs as it is (which shows the same failure outside a
+            # recording) instead of failing in a recording again at every step.
+            step_stream.wait_stream(self._capture_stream)
+            state.seen[key[1:]] = 0
+            state.sized = False
+            raise
         step_stream.wait_stream(self._capture_stream)
         self._graphs[key] = graph
         self.graphs_captured += 1
         graph.replay()
-        return state.logits
+        return state.logits[:n]
 
     def decode_graph_stats(self):
         """(graphs kept, batch sizes kept, bytes of the decode steps' logits buffers)."""

@@ -30,7 +30,7 @@ from dataclasses import dataclass, field
 from typing import List
 
 from ..cache import PAGE_TOKENS
-from ..errors import RequestError
+from ..errors import BackendError, RequestError
 from ..sampling import (EOS, INTERRUPTED, LENGTH, MAX_TOKENS, REPETITION_LOOP, STOP_TOKEN,
                         SamplingParams, detect_repetition_loop)
 from .batch import StepEntry
@@ -113,6 +113,9 @@ class Generator:
             make_chooser = Sampler
         self.make_chooser = make_chooser
         self.stats = GenerationStats()
+        # the loop is done with a decode step's logits before its next step: it takes the engine's
+        # own rows where the engine would otherwise hand out a copy
+        self._views = {"keep_logits": False} if getattr(engine, "hands_out_copies", False) else {}
 
     def generate(self, prompts, params=None, on_token=None, interrupt=None):
         """One GenerationResult per prompt (a list of token ids), in the prompts' order.
@@ -187,7 +190,7 @@ class Generator:
         def launch(order, device_tokens):
             entries = [StepEntry(slots[i], [generated[i][-1]] if device_tokens is None else [0], [0])
                        for i in order]
-            logits = eng.step(entries, tokens_on_device=device_tokens)
+            logits = eng.step(entries, tokens_on_device=device_tokens, **self._views)
             self.stats.decode_steps += 1
             return chooser.choose_ahead(logits, order), {i: eng.cache.length(slots[i]) for i in order}
 
@@ -272,6 +275,11 @@ class Generator:
                 for i, tok in zip(order, tokens):
                     if i not in slots:
                         continue
+                    if not 0 <= int(tok) < eng.spec.vocab_size:
+                        # (the chooser's answer for a row of logits without a finite value: what a
+                        # token id out of range, fed from the GPU where no host check sees it, leaves)
+                        raise BackendError(f"request {i}: no token could be chosen (got {int(tok)}): its logits "
+                                           "hold no finite value")
                     generated[i].append(int(tok))
                     self.stats.generated_tokens += 1
                     said = on_token(i, int(tok)) if on_token is not None else None
@@ -296,7 +304,7 @@ class Generator:
             else:
                 while live:
                     order = list(live)
-                    logits = eng.step([StepEntry(slots[i], [generated[i][-1]], [0]) for i in order])
+                    logits = eng.step([StepEntry(slots[i], [generated[i][-1]], [0]) for i in order], **self._views)
                     self.stats.decode_steps += 1
                     take(order, chooser.choose(logits, order))
             self.stats.decode_seconds += time.perf_counter() - t0

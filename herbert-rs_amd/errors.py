@@ -28,3 +28,9 @@ class CacheError(HerbertError):
 
 class RequestError(HerbertError):
     """A step or a generation request is malformed (empty sequence, bad token id, too long)."""
+
+
+class NeedsEagerStep(BackendError):
+    """While a step is recorded into a graph, something needs memory that it does not have yet
+    (a scratch buffer, room for a list): nothing can be allocated inside a recording, so the step
+    has to run outside one first. The engine catches this and does that; nobody else sees it."""

@@ -18,7 +18,8 @@ from ..errors import BackendError
 
 CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
 ARCH = "gfx950"
-MODULES = ("elementwise", "gemm_plain", "attention_plain", "sampling", "gemm_mfma", "attention_mfma")
+MODULES = ("elementwise", "gemm_plain", "attention_plain", "sampling", "gemm_mfma", "attention_mfma",
+           "random_weights")
 # packed float32 instructions are kept out of every kernel
 FLAGS = ["-O3", "-std=c++17", f"--offload-arch={ARCH}", "-shared", "-fPIC",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]

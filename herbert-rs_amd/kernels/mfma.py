@@ -26,42 +26,84 @@ lib.register_signatures("gemm_mfma", {
 })
 
 EPI_STORE, EPI_ADD, EPI_SWIGLU = 0, 1, 2
-_workspaces = {}
-_workspace_of = {}
-
-
 SLICE_WORKSPACE_FLOATS = 16 << 20     # most that the tiled product may use for its K slices (64 MB)
 
 
-def _slice_workspace(device, M, N, K, tile=0):
-    """(pointer, floats) of the scratch for products whose K may be cut into slices: those with few
-    tiles (whether it is cut, and how, is the kernel's estimate). It takes as many slices as fit in it. A buffer that
-    was handed out is kept for good: a captured graph may hold its address."""
-    if not isinstance(device, torch.device) or device.index is None:      # "the current device": not remembered
-        return _new_slice_workspace(device, M, N, K, tile)
-    key = (device, M, N, K, tile)
-    found = _workspace_of.get(key)           # (a buffer that was handed out stays valid: see above)
-    if found is not None:
-        return found
-    found = _workspace_of[key] = _new_slice_workspace(device, M, N, K, tile)
-    return found
+class Scratch:
+    """The device memory that these kernels use beyond their operands, for one owner: the workspace
+    of products whose K is cut into slices, and the partial results of the decode attention's
+    ranges. An engine's Runtime owns one, so that two engines of a process (each on a stream of its
+    own) never write the same scratch; callers without an owner (tests, measurements) share one a
+    device. A buffer that was handed out is kept for good, also when a larger one replaces it: a
+    captured graph may hold its address."""
+
+    def __init__(self):
+        self.workspaces = []         # float32 buffers, the newest and largest last
+        self.workspace_of = {}       # (device, M, N, K, tile) -> (pointer, floats)
+        self.partials = []           # (outputs, maxima and sums) of the decode attention's ranges
+
+    def newest_workspace(self):
+        return self.workspaces[-1] if self.workspaces else None
 
 
-def _new_slice_workspace(device, M, N, K, tile):
+def _not_while_recording(what):
+    """Nothing is allocated while a step is recorded into a graph: the step runs outside one first."""
+    if torch.cuda.is_current_stream_capturing():
+        from ..errors import NeedsEagerStep
+        raise NeedsEagerStep(f"{what} would have to be allocated while a graph is recorded")
+
+
+_shared_scratch = {}
+
+
+def _scratch_of(scratch, device):
+    if scratch is not None:
+        return scratch
     device = torch.device(device)
     if device.index is None:
         device = torch.device(device.type, torch.cuda.current_device())
+    found = _shared_scratch.get(device)
+    if found is None:
+        found = _shared_scratch[device] = Scratch()
+    return found
+
+
+def shared_scratch(device):
+    """The Scratch of callers that bring none, for `device`."""
+    return _scratch_of(None, device)
+
+
+def _slice_workspace_floats(M, N, K, tile=0):
+    """The floats of scratch that a product of these sizes is given for its K slices (0: it is never
+    cut): room for as many slices as the kernel's estimate may choose, up to SLICE_WORKSPACE_FLOATS.
+    Only products with few tiles are cut (whether, and how, is the kernel's estimate)."""
     tiles = ((M + 255) // 256) * ((N + 255) // 256)       # of the largest kind: under two rounds of them on 256 CUs
     slices = min(16, K // 256) if tiles < 512 or tile else 1
-    need = min(slices * M * N, SLICE_WORKSPACE_FLOATS)
     # (a product too large to be cut even in two still gets the room: where its rows are cut into
     # whole tiles and a rest, the rest's few rows are cut along K)
-    if slices < 2:
-        return None, 0
-    kept = _workspaces.setdefault(str(device), [])
-    if not kept or kept[-1].numel() < need:
-        kept.append(torch.empty(need, dtype=torch.float32, device=device))
-    return kept[-1].data_ptr(), kept[-1].numel()
+    return min(slices * M * N, SLICE_WORKSPACE_FLOATS) if slices >= 2 else 0
+
+
+def _slice_workspace(scratch, device, M, N, K, tile=0):
+    """(pointer, floats) of the scratch for a product whose K may be cut into slices."""
+    scratch = _scratch_of(scratch, device)
+    key = (device, M, N, K, tile)
+    found = scratch.workspace_of.get(key)           # (a buffer that was handed out stays valid)
+    if found is not None:
+        return found
+    need = _slice_workspace_floats(M, N, K, tile)
+    if need == 0:
+        found = (None, 0)
+    else:
+        kept = scratch.workspaces
+        if not kept or kept[-1].numel() < need:
+            _not_while_recording("the workspace of a product's K slices")
+            kept.append(torch.empty(need, dtype=torch.float32, device=device))
+        found = (kept[-1].data_ptr(), kept[-1].numel())
+    if len(scratch.workspace_of) > 4096:
+        scratch.workspace_of.clear()
+    scratch.workspace_of[key] = found
+    return found
 
 
 def gemm_supported(a, w, out=None, swiglu=False):
@@ -191,39 +233,43 @@ def _handoff_args(M, N, K, leave, row_scale, accumulate, norm):
     return args
 
 
-def gemm_plan(M, N, K, epi=EPI_STORE, normed_input=False, leaves_norm=False, finishes_norm=False, device="cuda",
+def gemm_plan(M, N, K, epi=EPI_STORE, normed_input=False, leaves_norm=False, finishes_norm=False, device=None,
               defer_slices=False):
     """Which kernel hb_gemm_mfma picks for a product, for tests and measurements: 0 = the few-row
-    kernel, otherwise the tile variant + 1000 x the K slices (if more than one), -1 = refused."""
-    _, ws_floats = _slice_workspace(torch.device(device), M, N, K)
+    kernel, otherwise the tile variant + 1000 x the K slices (if more than one), -1 = refused. The
+    choice is the host's and needs no GPU (`device` is not used): more scratch than a product is
+    given by _slice_workspace_floats never changes it, since that is room for every number of
+    slices the estimate considers."""
+    ws_floats = _slice_workspace_floats(M, N, K)
     return lib.load("gemm_mfma").hb_gemm_mfma_plan(M, N, K, epi, int(normed_input), int(leaves_norm),
                                                    int(finishes_norm), ws_floats, int(defer_slices))
 
 
-def gemm_split(M, N, K, epi=EPI_STORE, device="cuda"):
+def gemm_split(M, N, K, epi=EPI_STORE, device=None):
     """The rows that hb_gemm_mfma cuts off as a first product of their own (whole tiles; the rest
     follows as a second product), or 0 where it runs the product whole."""
-    _, ws_floats = _slice_workspace(torch.device(device), M, N, K)
+    ws_floats = _slice_workspace_floats(M, N, K)
     return lib.load("gemm_mfma").hb_gemm_mfma_split(M, N, K, epi, ws_floats)
 
 
-def gemm_plan_cost(M, N, K, epi=EPI_STORE, normed_input=False, leaves_norm=False, finishes_norm=False, device="cuda",
+def gemm_plan_cost(M, N, K, epi=EPI_STORE, normed_input=False, leaves_norm=False, finishes_norm=False, device=None,
                    defer_slices=False):
     """The estimated time in us of the plan gemm_plan gives; negative where no estimate chose it."""
-    _, ws_floats = _slice_workspace(torch.device(device), M, N, K)
+    ws_floats = _slice_workspace_floats(M, N, K)
     fn = lib.load("gemm_mfma").hb_gemm_mfma_plan_cost
     fn.restype = ctypes.c_double
     return fn(M, N, K, epi, int(normed_input), int(leaves_norm), int(finishes_norm), ws_floats, int(defer_slices))
 
 
 def gemm(a, w, out, accumulate=False, packed=False, norm=None, tile=0, leave=None, row_scale=None,
-         defer_slices=False):
+         defer_slices=False, scratch=None):
     """out f32 [M, N] (+)= a bf16 [M, K] @ w bf16 [N, K]^T (w as stored, or as pack_weight gives it).
     norm = (weight f32 [K], eps): a is the float32 residual stream and is RMS-normed on the way.
     leave, row_scale: see _handoff_args.
     defer_slices: if the kernel cuts K into slices it leaves their sums for the caller's next kernel
     to add up; returns (slices, pointer to the first, floats between two): with slices == 1 `out`
-    holds the product as usual, otherwise `out` is not written."""
+    holds the product as usual, otherwise `out` is not written.
+    scratch: the caller's Scratch (the K slices' workspace comes from it); None: the device's shared one."""
     M, K = a.shape
     norm_ptr, eps = _norm_args(a, norm, K)
     _check(w, "w", torch.bfloat16, (None, K))
@@ -232,7 +278,7 @@ def gemm(a, w, out, accumulate=False, packed=False, norm=None, tile=0, leave=Non
     if K % 32 or (norm is not None and accumulate):
         raise BackendError(f"gemm_mfma refuses M={M}, N={N}, K={K}")
     hand = _handoff_args(M, N, K, leave, row_scale, accumulate, norm)
-    ws_ptr, ws_floats = _slice_workspace(a.device, M, N, K, tile)
+    ws_ptr, ws_floats = _slice_workspace(scratch, a.device, M, N, K, tile)
     if defer_slices and (accumulate or leave is not None):
         raise BackendError("only a plain product leaves its slices to the next kernel")
     deferred = ctypes.c_int(1) if defer_slices else None
@@ -322,7 +368,7 @@ def interleave_gate_up(gate, up):
     return torch.stack([gate.view(I // 16, 16, K), up.view(I // 16, 16, K)], 1).reshape(2 * I, K).contiguous()
 
 
-def gemm_swiglu(a, w_interleaved, out, packed=False, norm=None, tile=0, row_scale=None):
+def gemm_swiglu(a, w_interleaved, out, packed=False, norm=None, tile=0, row_scale=None, scratch=None):
     """out bf16 [M, I] = silu(a @ gate^T) * (a @ up^T), the weights interleaved as above.
     row_scale: see _handoff_args (gate and up are scaled before the activation)."""
     M, K = a.shape
@@ -333,7 +379,7 @@ def gemm_swiglu(a, w_interleaved, out, packed=False, norm=None, tile=0, row_scal
     if K % 32 or N % 32:
         raise BackendError(f"gemm_mfma (SwiGLU) refuses M={M}, N={N}, K={K}")
     hand = _handoff_args(M, N, K, None, row_scale, False, norm)
-    ws_ptr, ws_floats = _slice_workspace(a.device, M, N, K, tile)
+    ws_ptr, ws_floats = _slice_workspace(scratch, a.device, M, N, K, tile)
     lib.call("gemm_mfma", "hb_gemm_mfma", a.data_ptr(), w_interleaved.data_ptr(), out.data_ptr(), M, N, K,
              N // 2, EPI_SWIGLU, 1 if packed else 0, norm_ptr, eps, int(tile), ws_ptr, ws_floats, *hand, None,
              _stream())
@@ -347,7 +393,6 @@ lib.register_signatures("attention_mfma", {
 
 ATTENTION_HEAD_DIMS = (32, 64, 128)
 QUERY_TILE = 32
-_partials = {}
 
 
 def attention_supported(q, kv, nq, nkv, hd):
@@ -367,6 +412,14 @@ def _prefill_tile_height(meta, nkv, group):
     Tiles of 64 must be worth their eight waves: those of at most 32 tokens (single tokens of
     running sequences beside a prompt, a prompt's short end) leave one half idle and walk their
     pages alone, so a step made mostly of them keeps tiles of 32."""
+    key = ("prefill_tile_height", nkv, group)
+    height = meta.derived.get(key)          # every layer's attention asks: worked out once a step
+    if height is None:
+        height = meta.derived[key] = _prefill_tile_height_of(meta, nkv, group)
+    return height
+
+
+def _prefill_tile_height_of(meta, nkv, group):
     tiles = full = 0
     for i in range(meta.num_seqs):
         n = int(meta.host_starts[i + 1]) - int(meta.host_starts[i])
@@ -455,13 +508,14 @@ def _decode_ranges(meta, nkv, window):
     return None if listed is None else (items, listed)
 
 
-def _partial_buffers(device, n_rows, splits, hd):
-    """(partial outputs, partial max / sum) of the decode kernel's ranges. Buffers that were handed
-    out are kept for good, also when larger ones replace them: a captured graph may hold their
-    addresses."""
-    kept = _partials.setdefault(str(device), [])
+def _partial_buffers(scratch, device, n_rows, splits, hd):
+    """(partial outputs, partial max / sum) of the decode kernel's ranges, from the caller's Scratch.
+    Buffers that were handed out are kept for good, also when larger ones replace them: a captured
+    graph may hold their addresses."""
+    kept = _scratch_of(scratch, device).partials
     need_o, need_ml = n_rows * splits * hd, n_rows * splits * 2
     if not kept or kept[-1][0].numel() < need_o or kept[-1][1].numel() < need_ml:
+        _not_while_recording("the decode attention's partial results")
         grow = 2 if kept else 1
         kept.append((torch.empty(max(need_o, grow * (kept[-1][0].numel() if kept else 0)), dtype=torch.float32,
                                  device=device),
@@ -479,7 +533,7 @@ def decode_fusable(meta, kv, nq, nkv, hd, rot_dims, dtype):
 
 
 def attention_decode_fused(qkv, q_norm_w, k_norm_w, cos, sin, meta, kv, out, nq, nkv, hd, eps, scale, window,
-                           qkv_slices=None):
+                           qkv_slices=None, scratch=None):
     """One token a sequence: per-head norm (if weights are given), rotation (if tables are given),
     the new key and value written to the pages, and attention over them, in one kernel (+ merge).
     qkv f32 [B, (nq + 2 nkv) hd]; cos / sin f32 [max_pos, hd / 2]; out bf16 [B, nq hd].
@@ -511,10 +565,10 @@ def attention_decode_fused(qkv, q_norm_w, k_norm_w, cos, sin, meta, kv, out, nq,
     listed = _decode_ranges(meta, nkv, window)
     if listed:
         (splits, ranges), per = listed, 1
-        po, pml = _partial_buffers(qkv.device, nq, splits, hd)
+        po, pml = _partial_buffers(scratch, qkv.device, nq, splits, hd)
     else:
         (splits, per), ranges = _decode_split(meta, nkv, window), None
-        po, pml = _partial_buffers(qkv.device, B * nq, splits, hd)
+        po, pml = _partial_buffers(scratch, qkv.device, B * nq, splits, hd)
     n_slices, src, stride = qkv_slices if qkv_slices is not None else (1, qkv.data_ptr(), 0)
     if n_slices > 1 and (n_slices not in DEFERRED_SLICES or hd != 128 or stride < qkv.numel()):
         raise BackendError(f"fused decode attention does not add up {n_slices} slices of the projection")
@@ -530,7 +584,7 @@ def attention_decode_fused(qkv, q_norm_w, k_norm_w, cos, sin, meta, kv, out, nq,
 DEFERRED_SLICES = (2, 4, 8)     # numbers of slices of the projection that the decode kernel adds up itself
 
 
-def attention(q, meta, kv, out, nq, nkv, hd, scale, window, tile_height=None):
+def attention(q, meta, kv, out, nq, nkv, hd, scale, window, tile_height=None, scratch=None):
     """Causal (and windowed) attention of the step's tokens over their slots' pages.
     One token a sequence: the split decode kernel; otherwise one of the two tiled prompt kernels
     (tile_height 32 or 64 asks for one by name; None: the host's choice, see _prefill_tile_height)."""
@@ -552,10 +606,10 @@ def attention(q, meta, kv, out, nq, nkv, hd, scale, window, tile_height=None):
         listed = _decode_ranges(meta, nkv, window)
         if listed:
             (splits, ranges), per = listed, 1
-            po, pml = _partial_buffers(q.device, nq, splits, hd)
+            po, pml = _partial_buffers(scratch, q.device, nq, splits, hd)
         else:
             (splits, per), ranges = _decode_split(meta, nkv, window), None
-            po, pml = _partial_buffers(q.device, T * nq, splits, hd)
+            po, pml = _partial_buffers(scratch, q.device, T * nq, splits, hd)
         lib.call("attention_mfma", "hb_attn_decode_mfma", q.data_ptr(), kv.k.data_ptr(), kv.v.data_ptr(),
                  out.data_ptr(), po.data_ptr(), pml.data_ptr(), meta.context_lens.data_ptr(),
                  meta.slots.data_ptr(), kv.page_table.data_ptr(), kv.page_table.shape[1], kv.page_size,

@@ -80,8 +80,8 @@ class Attention(Part):
         if not self.reads_cache_only:
             rows += [tensors[n["k"]], tensors[n["v"]]]
         # one fused projection [q rows | k rows | v rows]: the activations are read once
-        self.qkv = Linear(rt.weight(torch.cat([r.to(rt.device) for r in rows], 0)))
-        self.o = Linear(rt.weight(tensors[n["o"]]))
+        self.qkv = Linear(rt.weight(torch.cat([r.to(rt.device) for r in rows], 0)), scratch=rt.scratch)
+        self.o = Linear(rt.weight(tensors[n["o"]]), scratch=rt.scratch)
         if self.qk_norm:
             self.q_norm_w = rt.weight(tensors[n["q_norm"]], matrix=False)
             if not self.reads_cache_only:
@@ -140,7 +140,7 @@ class Attention(Part):
             # one token a sequence: norm, rotation, cache write and attention in one kernel
             mfma.attention_decode_fused(qkv, self.q_norm_w, self.k_norm_w, cos, sin, ctx.meta, kv, attn,
                                         self.nq, self.nkv, self.hd, self.eps, self.scale, self.window,
-                                        qkv_slices=slices)
+                                        qkv_slices=slices, scratch=rt.scratch)
             self.project_out(ctx, attn, x)
             return
         q = rt.buffer("q", (T, self.q_dim))
@@ -152,6 +152,7 @@ class Attention(Part):
     def attend(self, ctx, q, kv, out):
         if q.dtype == torch.bfloat16:
             if mfma.attention_supported(q, kv, self.nq, self.nkv, self.hd):
-                mfma.attention(q, ctx.meta, kv, out, self.nq, self.nkv, self.hd, self.scale, self.window)
+                mfma.attention(q, ctx.meta, kv, out, self.nq, self.nkv, self.hd, self.scale, self.window,
+                               scratch=ctx.rt.scratch)
                 return
         ops.attention_plain(q, ctx.meta, kv, out, self.nq, self.nkv, self.hd, self.scale, self.window)

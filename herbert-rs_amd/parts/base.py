@@ -24,6 +24,14 @@ from typing import Any
 import torch
 
 
+def _not_while_recording(device, what):
+    """Memory is never allocated while a step is recorded into a graph (it would belong to that
+    graph's pool): the step has to run outside a recording first."""
+    if device.type == "cuda" and torch.cuda.is_current_stream_capturing():
+        from ..errors import NeedsEagerStep
+        raise NeedsEagerStep(f"{what} would have to be allocated while a graph is recorded")
+
+
 class Part:
     kind = "?"
     # True if forward() only enqueues GPU work (no host synchronisation, no host-side copies):
@@ -51,6 +59,16 @@ class Runtime:
         self._buffers = {}
         self._views = {}         # (name, dtype, shape) -> the view of the buffer that was handed out last
         self._outgrown = []      # never freed: a captured graph may hold their addresses
+        self._scratch = None
+
+    @property
+    def scratch(self):
+        """The kernels' own scratch memory (K slices of products, partial results of the decode
+        attention) of this runtime's owner: see kernels.mfma.Scratch."""
+        if self._scratch is None:
+            from ..kernels.mfma import Scratch
+            self._scratch = Scratch()
+        return self._scratch
 
     @property
     def exact(self):
@@ -72,6 +90,7 @@ class Runtime:
         key = (name, dtype)
         buf = self._buffers.get(key)
         if buf is None or buf.numel() < n:
+            _not_while_recording(self.device, f"the scratch buffer {name!r}")
             if buf is not None:
                 self._outgrown.append(buf)
                 n_new = max(n, 2 * buf.numel())

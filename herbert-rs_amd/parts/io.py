@@ -30,7 +30,7 @@ class TokenEmbedding(Part):
     def load(self, tensors, rt, shared_with_head=False):
         """shared_with_head: the table is also the head's matrix; it is then kept in the order the
         head's kernels want, and rows are gathered from that order."""
-        self.linear = Linear(rt.weight(tensors[self.weight_name]), pack=shared_with_head)
+        self.linear = Linear(rt.weight(tensors[self.weight_name]), pack=shared_with_head, scratch=rt.scratch)
         self.table = self.linear.weight
 
     def forward(self, ctx, token_ids):
@@ -63,7 +63,7 @@ class OutputHead(Part):
         if self.tied:
             self.proj = embedding.linear
         else:
-            self.proj = Linear(rt.weight(tensors[self.weight_name]))
+            self.proj = Linear(rt.weight(tensors[self.weight_name]), scratch=rt.scratch)
 
     def forward(self, ctx, x, rows):
         y = self.norm.forward(ctx, x, rows, name="head_normed")

@@ -12,8 +12,10 @@ from ..kernels import mfma, ops
 
 
 class Linear:
-    def __init__(self, weight, pack=True):
-        """weight: [N, K] in the compute dtype on the GPU."""
+    def __init__(self, weight, pack=True, scratch=None):
+        """weight: [N, K] in the compute dtype on the GPU. scratch: the kernels' scratch memory of the
+        owner (Runtime.scratch); None: the device's shared one."""
+        self.scratch = scratch
         self.out_features, self.in_features = weight.shape
         self.packed = False
         if pack and weight.dtype == torch.bfloat16 and weight.is_cuda \
@@ -30,7 +32,7 @@ class Linear:
         if self.weight.dtype == torch.bfloat16 and a.dtype == torch.bfloat16:
             if self.packed or mfma.gemm_supported(a, self.weight, out):
                 return mfma.gemm(a, self.weight, out, accumulate, packed=self.packed, leave=leave,
-                                 row_scale=row_scale, defer_slices=defer_slices)
+                                 row_scale=row_scale, defer_slices=defer_slices, scratch=self.scratch)
         if leave is not None or row_scale is not None:
             raise ValueError("this product cannot hand a norm on (ask norm_handoff first)")
         ops.gemm_plain(a, self.weight, out, accumulate)
@@ -56,7 +58,8 @@ class Linear:
 
     def forward_swiglu(self, a, out, norm=None, row_scale=None):
         """out bf16 [M, N / 2] = silu(gate) * up for a weight whose rows are gate/up interleaved."""
-        mfma.gemm_swiglu(a, self.weight, out, packed=self.packed, norm=norm, row_scale=row_scale)
+        mfma.gemm_swiglu(a, self.weight, out, packed=self.packed, norm=norm, row_scale=row_scale,
+                         scratch=self.scratch)
 
     def fuses_norm(self, x):
         """True if RMSNorm(x) @ W^T runs as one kernel for this input (few rows, bfloat16 weights)."""
@@ -66,4 +69,4 @@ class Linear:
 
     def forward_normed(self, x, norm_weight, eps, out):
         """out[M, N] = RMSNorm(x; norm_weight, eps) @ W^T in one kernel (see fuses_norm)."""
-        mfma.gemm(x, self.weight, out, packed=self.packed, norm=(norm_weight, eps))
+        mfma.gemm(x, self.weight, out, packed=self.packed, norm=(norm_weight, eps), scratch=self.scratch)

@@ -40,10 +40,10 @@ class SwiGLU(Part):
                                and self.hidden_size % 32 == 0 and mfma.gemm_supported(
                                    gate[:1], gate, swiglu=True))
         if self.fused_epilogue:
-            self.gate_up = Linear(mfma.interleave_gate_up(gate, up))
+            self.gate_up = Linear(mfma.interleave_gate_up(gate, up), scratch=rt.scratch)
         else:
-            self.gate_up = Linear(torch.cat([gate, up], 0))
-        self.down = Linear(rt.weight(tensors[n["down"]]))
+            self.gate_up = Linear(torch.cat([gate, up], 0), scratch=rt.scratch)
+        self.down = Linear(rt.weight(tensors[n["down"]]), scratch=rt.scratch)
 
     def forward_from_residual(self, ctx, x, norm):
         """With few rows and the fused epilogue no norm kernel runs: the gate/up kernel takes what the

@@ -45,6 +45,7 @@ class Sampler:
         self._host_ring = []            # pinned buffers that tokens on their way to the host land in
         self._host_next = 0
         self._index = None
+        self._row_indices = {}          # (rows of a choice, the rows taken) -> their index on the GPU
         # a cap on think blocks: one counter a sequence, fed with every token chosen for it
         self.think = None
         if params.think_budget > 0:
@@ -142,12 +143,22 @@ class Sampler:
         pending.event.synchronize()
         return pending.host.tolist()
 
-    @staticmethod
-    def rows_of(pending, rows):
-        """The device tokens of some rows of a `choose_ahead`, in the given order."""
-        if list(rows) == list(range(pending.device.shape[0])):
+    def rows_of(self, pending, rows):
+        """The device tokens of some rows of a `choose_ahead`, in the given order. The index of a
+        choice of rows is kept: a batch that shrinks asks for the same rows step after step, and
+        making the index anew would wait for a copy from the host each time."""
+        rows = tuple(rows)
+        if rows == tuple(range(pending.device.shape[0])):
             return pending.device
-        return pending.device[torch.tensor(list(rows), dtype=torch.long, device=pending.device.device)]
+        key = (pending.device.shape[0], rows)
+        index = self._row_indices.get(key)
+        if index is None:
+            if len(self._row_indices) >= 256:
+                self._row_indices.clear()
+            host = torch.tensor(rows, dtype=torch.long).pin_memory() if self.device.type == "cuda" \
+                else torch.tensor(rows, dtype=torch.long)
+            index = self._row_indices[key] = host.to(self.device, non_blocking=True)
+        return pending.device[index]
 
     def _index_of(self, sequence_indices):
         """The rows' sequences as a tensor on the GPU; the one of the step before is kept, since a

@@ -43,7 +43,11 @@ def test_groups_have_storage_of_their_own():
     full = c.kv_groups[KVNeed(2, 8, None)]
     win = c.kv_groups[KVNeed(2, 8, 100)]
     assert full.entries == [0, 2] and win.entries == [1]
-    assert full.pool.shape == (2, 2, 12, 2, 64, 8) and win.pool.shape == (1, 2, 12, 2, 64, 8)
+    # twelve pages for sequences and the padding page, which only the padding slot's table names
+    assert full.pool.shape == (2, 2, 13, 2, 64, 8) and win.pool.shape == (1, 2, 13, 2, 64, 8)
+    assert c.pad_slot == c.n_slots == 12 and full.pages.count == 12
+    assert full.table.shape[0] == 13 and set(full.table[c.pad_slot].tolist()) == {12}
+    assert 12 not in set(full.table[:12].flatten().tolist())
     assert c.kv_view(0).k.data_ptr() != c.kv_view(2).k.data_ptr()
     assert c.kv_view(1).window == 100 and c.kv_view(0).window == 0
 
@@ -109,7 +113,7 @@ def test_state_is_cleared_when_a_slot_is_taken_again():
     c = make_cache(state=True)
     s = c.alloc_slot()
     views = c.state_views(1)
-    assert len(views) == 1 and views[0].shape == (c.n_slots, 4)
+    assert len(views) == 1 and views[0].shape == (c.n_slots + 1, 4)          # the last row: the padding slot
     views[0][s] = 5.0
     c.state_views(3)[0][s] = 2.0
     c.free_slot(s)
@@ -576,6 +580,38 @@ def test_turns_on_a_kept_slot_go_on_from_what_it_holds(ahead, rolls_back):
     with pytest.raises(RequestError, match="at least one token"):
         gen.extend(slot, [], SamplingParams(temperature=0.0, max_tokens=2), chooser)
     eng.free_slot(slot)
+    assert eng.cache.slots.held_count == 0
+
+
+def test_the_memory_a_cache_needs_counts_pages_and_state():
+    """What the engine compares with the GPU's free memory before it builds a cache: the pools of
+    keys and values by pages, and fixed-size state by slots, entries of equal need together."""
+    import torch
+    from herbert_rs_amd.cache import Cache, KVNeed, StateNeed
+    kv, state = KVNeed(2, 16, None), StateNeed((5, 8), torch.float32)
+    needs = {0: kv, 1: (kv, state), 3: state}
+    got = Cache.bytes_needed(needs, max_tokens=64 * 6 - 1, dtype=torch.bfloat16, max_slots=4)
+    assert got == 2 * 2 * (6 + 1) * 64 * 2 * 16 * 2 + 2 * (4 + 1) * 40 * 4       # one page and one slot more: the padding's
+    cache = Cache(needs, 64 * 6 - 1, 512, torch.bfloat16, "cpu", max_slots=4)
+    held = sum(g.pool.numel() * 2 for g in cache.kv_groups.values()) + \
+        sum(g.data.numel() * 4 for g in cache.state_groups.values())
+    assert held == got
+    # without a cap on the slots there are as many as pages
+    assert Cache.bytes_needed({0: state}, 64 * 3, torch.float32) == (3 + 1) * 40 * 4
+
+
+def test_a_token_that_is_none_ends_the_generation_with_an_error():
+    """A chooser's -1 (the GPU argmax's answer for a row without a finite logit) is an error of the
+    loop's, not a token; the slots still come back."""
+    from herbert_rs_amd.errors import BackendError
+
+    class NoneChooser(ArgmaxChooser):
+        def choose(self, logits, sequence_indices):
+            return [-1 for _ in sequence_indices]
+    eng = FakeEngine()
+    with pytest.raises(BackendError, match="no token could be chosen"):
+        Generator(eng, max_batch=2, make_chooser=NoneChooser).generate(
+            [[5], [6, 7]], SamplingParams(temperature=0.0, max_tokens=3, repeat_check=False))
     assert eng.cache.slots.held_count == 0
 
 

@@ -2,6 +2,7 @@
 import json
 import os
 
+import numpy as np
 import pytest
 import torch
 from safetensors.torch import load_file, save_file
@@ -277,6 +278,52 @@ def test_names_are_normalised_and_fused_tensors_cut(model_root, tmp_path):
     save_file(other, str(tmp_path / "model.safetensors"))
     with pytest.raises(ModelLoadError, match=r"qkv_proj.weight: expected \[320, 96\], got \[10, 96\]"):
         read_tensors(str(tmp_path), needs_of(TINY_B), name_map=NAMES)
+
+
+def counter_values(key, first, count, scale, offset):
+    """The random weights' formula in NumPy, written from its description alone: the bytes of
+    splitmix64(key, i) summed and centred, one float32 product, one float32 sum."""
+    mask = (1 << 64) - 1
+    sums = []
+    for i in range(first, first + count):
+        z = (key + (i + 1) * 0x9E3779B97F4A7C15) & mask
+        z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & mask
+        z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & mask
+        z ^= z >> 31
+        sums.append(sum((z >> (8 * b)) & 255 for b in range(8)) - 1020)
+    scaled = np.array(sums, dtype=np.float32) * np.float32(scale)
+    return (np.float32(offset) + scaled).astype(np.float32)
+
+
+def test_random_weights_are_a_function_of_seed_name_and_index():
+    """The host's values are the formula's, bit for bit, as float32 and rounded to bfloat16 (nearest,
+    ties to even); a tensor drawn in pieces is the tensor drawn whole; the deviates are near normal;
+    tensors do not depend on each other, norm weights with norm_std 0 are exactly 1."""
+    from herbert_rs_amd.weights import TensorNeed, random_tensors
+    from herbert_rs_amd.weights import random_init as ri
+    from .plain.sampler import f32_to_bf16_bits
+    key, n = 0x1234567890ABCDEF, 3000
+    assert counter_values(12345, 0, 4, 1.0, 0.0).tolist() == [-196.0, 342.0, -60.0, -390.0]     # by hand, in integers
+    for scale, offset in ((0.02 / ri.BYTE_SUM_SIGMA, 0.0), (0.1 / ri.BYTE_SUM_SIGMA, 1.0)):
+        want = counter_values(key, 0, n, scale, offset)
+        got = ri.counter_fill(torch.empty(n, dtype=torch.float32), key, scale, offset)
+        assert np.array_equal(got.numpy().view(np.uint32), want.view(np.uint32))
+        half = ri.counter_fill(torch.empty(n, dtype=torch.bfloat16), key, scale, offset)
+        assert half.view(torch.int16).numpy().astype(np.uint16).tolist() == [f32_to_bf16_bits(v) for v in want]
+        tail = ri.counter_fill(torch.empty(n - 1000, dtype=torch.float32), key, scale, offset, first=1000)
+        assert torch.equal(tail, got[1000:])
+    many = ri.counter_fill(torch.empty(1 << 20, dtype=torch.float32), 99, 1.0 / ri.BYTE_SUM_SIGMA).double()
+    assert abs(float(many.mean())) < 0.005 and abs(float(many.std()) - 1.0) < 0.005
+    assert abs(float((many ** 4).mean()) - 2.85) < 0.03 and float(many.abs().max()) <= 4.88
+    assert 0.66 < float((many.abs() < 1).double().mean()) < 0.70
+    needs = {"a.weight": TensorNeed((40, 24)), "n.weight": TensorNeed((24,), "scale")}
+    both = random_tensors(needs, 7, "float32", std=0.05, norm_std=0.0)
+    alone = random_tensors({"a.weight": needs["a.weight"]}, 7, "float32", std=0.05)
+    assert torch.equal(both["a.weight"], alone["a.weight"]) and bool((both["n.weight"] == 1.0).all())
+    other = random_tensors(needs, 8, "float32", std=0.05, norm_std=0.1)
+    assert not torch.equal(other["a.weight"], both["a.weight"]) and 0.05 < float(other["n.weight"].std()) < 0.2
+    want = counter_values(ri._tensor_seed(7, "a.weight"), 0, 960, 0.05 / ri.BYTE_SUM_SIGMA, 0.0)
+    assert np.array_equal(both["a.weight"].numpy().ravel(), want)
 
 
 def test_an_architecture_brings_its_own_names_default_and_initialisers(tmp_path):

@@ -452,6 +452,13 @@ def test_argmax_kernel_takes_the_first_of_equals(V):
     ops.argmax(logits.cuda(), out)
     assert out.tolist() == [plain_sampler.argmax(r.numpy()) for r in logits]
     assert out.tolist()[:4] == [77, V - 1, 0, 0]
+    # a row that holds NaN and nothing above -inf (what a token id out of range leaves of a step)
+    # gives -1, which the generation loop reports; NaN beside finite values is passed over
+    logits[3, V // 2] = float("nan")
+    logits[4] = float("nan")
+    logits[0, 5] = float("nan")
+    ops.argmax(logits.cuda(), out)
+    assert out.tolist() == [77, V - 1, 0, -1, -1]
 
 
 @pytest.mark.parametrize("V", [1500, 10000])
@@ -739,6 +746,114 @@ def test_sampling_through_generate_is_reproducible(model_root):
                 excused += 1
             seq.append(tok)
     assert excused <= 2
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_seed_gives_the_same_weights_on_the_gpu_and_in_a_folder(dtype, tmp_path):
+    """Engine.from_config draws its weights on the GPU, write_random_model on the host: the same
+    seed gives the same bits, so what the benchmark times can be written out and compared with the
+    plain implementation; and the two engines give the same logits."""
+    from herbert_rs_amd.config.registry import resolve_architecture
+    from .tiny import TINY_B
+    arch = resolve_architecture(TINY_B)
+    cfg = arch.config_class.from_dict(TINY_B)
+    drawn = hb.Engine.from_config(cfg, seed=11, dtype=dtype, std=0.05, norm_std=0.1, max_tokens=128)
+    folder = hb.write_random_model(str(tmp_path / "m"), TINY_B, seed=11, dtype=dtype, std=0.05, norm_std=0.1)
+    read = hb.load(folder, dtype=dtype, cache_tokens=128)
+    from safetensors import safe_open
+    with safe_open(os.path.join(folder, "model.safetensors"), framework="pt") as f:
+        names = list(f.keys())
+        assert len(names) == 3 * 11 + 3
+        for name in names:
+            stored = f.get_tensor(name)
+            again = drawn.get_tensor(name)
+            assert stored.dtype == again.dtype and torch.equal(stored, again), name
+    tokens = random_tokens(384, 40, 12)
+    a = drawn.step([StepEntry(drawn.alloc_slot(), tokens, list(range(40)))]).cpu()
+    b = read.step([StepEntry(read.alloc_slot(), tokens, list(range(40)))]).cpu()
+    assert torch.equal(a, b)
+    ref = plain_logits(folder, tokens)
+    assert close(a[39].numpy(), ref[39], dtype, "B")[0]
+
+
+def test_two_engines_on_two_streams_share_no_scratch(model_root):
+    """Each engine's kernels have scratch of their own (the partial results of the decode
+    attention's ranges, the K slices of products): two engines of one process, stepped in turn on
+    two streams without waiting for each other, give bit for bit what each gives alone."""
+    folder = make_folder(model_root, "D", "bfloat16")
+    seqs = [random_tokens(512, 700, 300 + i) for i in range(2)]
+
+    def decode(engine, tokens, stream, out):
+        with torch.cuda.stream(stream):
+            slot = engine.alloc_slot()
+            engine.step([StepEntry(slot, tokens[:640], [])])
+        for p in range(640, 700):
+            yield
+            with torch.cuda.stream(stream):
+                out.append(engine.step([StepEntry(slot, [tokens[p]], [0])]).clone())
+
+    alone = []
+    for t in seqs:
+        engine = hb.load(folder, dtype="bfloat16", cache_tokens=64 * 12)
+        got = []
+        for _ in decode(engine, t, torch.cuda.current_stream(), got):
+            pass
+        torch.cuda.synchronize()
+        alone.append(torch.stack(got).cpu())
+    engines = [hb.load(folder, dtype="bfloat16", cache_tokens=64 * 12) for _ in seqs]
+    assert engines[0].rt.scratch is not engines[1].rt.scratch
+    streams = [torch.cuda.Stream() for _ in seqs]
+    outs = [[], []]
+    runs = [decode(e, t, s, o) for e, t, s, o in zip(engines, seqs, streams, outs)]
+    live = list(runs)
+    while live:                                  # a step of one, a step of the other, nobody waits
+        for r in list(live):
+            try:
+                next(r)
+            except StopIteration:
+                live.remove(r)
+    torch.cuda.synchronize()
+    for e in engines:
+        assert e.rt.scratch.partials, "the decode attention of heads of 128 keeps partial results"
+    assert engines[0].rt.scratch.partials[-1][0].data_ptr() != engines[1].rt.scratch.partials[-1][0].data_ptr()
+    for i in range(2):
+        assert torch.equal(torch.stack(outs[i]).cpu(), alone[i]), i
+
+
+def test_a_capture_that_fails_leaves_the_shape_to_start_over(model_root):
+    """A forward pass that raises while a decode step is captured: the error reaches the caller,
+    the cache is as before, and the shape's next step runs eagerly again instead of going straight
+    into another capture; the step after that is captured, and replays give the eager logits."""
+    folder = make_folder(model_root, "B", "float32")
+    tokens = random_tokens(384, 40, 77)
+    engine = hb.Engine.from_folder(folder, dtype="float32", max_tokens=64 * 4)
+    plain_engine = hb.Engine.from_folder(folder, dtype="float32", max_tokens=64 * 4, use_graphs=False)
+    slot, slot0 = engine.alloc_slot(), plain_engine.alloc_slot()
+    engine.step([StepEntry(slot, tokens[:10], [])])
+    plain_engine.step([StepEntry(slot0, tokens[:10], [])])
+    real = engine.model.forward
+    state = {"failed": 0}
+
+    def failing(rt, meta, cache, logits_out=None):
+        if torch.cuda.is_current_stream_capturing() and not state["failed"]:
+            state["failed"] += 1
+            raise RuntimeError("this capture fails")
+        return real(rt, meta, cache, logits_out=logits_out)
+    engine.model.forward = failing
+    p = 10
+    got = engine.step([StepEntry(slot, [tokens[p]], [0])]).cpu()               # eager
+    want = plain_engine.step([StepEntry(slot0, [tokens[p]], [0])]).cpu()
+    assert torch.equal(got, want)
+    p += 1
+    with pytest.raises(RuntimeError, match="capture fails"):                    # the capture
+        engine.step([StepEntry(slot, [tokens[p]], [0])])
+    assert engine.cache.length(slot) == p and engine.graphs_captured == 0
+    engine.cache.check()
+    for p in range(11, 40):              # eager again, then captured, then replays
+        got = engine.step([StepEntry(slot, [tokens[p]], [0])]).cpu()
+        want = plain_engine.step([StepEntry(slot0, [tokens[p]], [0])]).cpu()
+        assert torch.equal(got, want), p
+    assert state["failed"] == 1 and engine.graphs_captured == 1
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

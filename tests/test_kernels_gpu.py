@@ -737,7 +737,7 @@ def test_gemm_mfma_leaves_its_slices_to_the_next_kernel(M, scaled):
     n, ptr, stride = mfma.gemm(a, wp, out, packed=True, row_scale=row_scale, defer_slices=True)
     assert n in mfma.DEFERRED_SLICES and stride == M * N and float(out.min()) == 7.0      # out is not written
     parts = torch.empty(n, M, N, device=dev())
-    ws = mfma._workspaces[str(dev())][-1]
+    ws = mfma.shared_scratch(dev()).newest_workspace()
     assert ws.data_ptr() == ptr
     parts.copy_(ws[:n * M * N].view(n, M, N))
     whole = torch.empty(M, N, device=dev())

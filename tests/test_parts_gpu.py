@@ -339,6 +339,45 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped():
         at += len(t)
 
 
+def test_a_step_that_fails_leaves_the_state_as_it_was():
+    """The toy layer runs twice in the schedule. A step whose forward pass fails after the first run
+    has changed its state (here: the second run's mixer raises) leaves every slot's state, length
+    and pages as they were: the same step, run again, gives what it gives on a cache that never
+    saw the failure."""
+    from herbert_rs_amd.weights import random_tensors
+    from herbert_rs_amd.engine.model import Model
+    spec = toy_spec()
+    w = random_tensors(Model(spec).tensor_needs(), 3, "float32", std=0.15, norm_std=0.1)
+    seqs = [[5, 9, 33, 2, 41, 17, 8, 11], [7, 3, 50, 1]]
+
+    def run(fail_once):
+        engine = Engine(None, spec, w, dtype="float32", max_tokens=256)
+        slots = [engine.alloc_slot() for _ in seqs]
+        engine.step([StepEntry(s, t[:3], []) for s, t in zip(slots, seqs)])
+        if fail_once:
+            mixer = engine.model.blocks[0].mixer
+            real, calls = mixer.forward, []
+
+            def failing(ctx, y, x):
+                calls.append(ctx.entry)
+                if ctx.entry == 2:
+                    raise RuntimeError("the second run fails")
+                return real(ctx, y, x)
+            mixer.forward = failing
+            before = [g.data.clone() for g in engine.cache.state_groups.values()]
+            with pytest.raises(RuntimeError, match="second run"):
+                engine.step([StepEntry(s, t[3:], [0]) for s, t in zip(slots, seqs)])
+            mixer.forward = real
+            assert calls == [0, 2]                      # the first run had changed its state already
+            for g, b in zip(engine.cache.state_groups.values(), before):
+                assert torch.equal(g.data, b)
+            assert [engine.cache.length(s) for s in slots] == [3, 3]
+            engine.cache.check()
+        return engine.step([StepEntry(s, t[3:], list(range(len(t) - 3))) for s, t in zip(slots, seqs)]).cpu()
+
+    assert torch.equal(run(True), run(False))
+
+
 # ---- a toy feed-forward with routing and a toy position encoding, defined here
 @register("feed_forward", "toy_routed")
 class ToyRoutedFeedForward(Part):

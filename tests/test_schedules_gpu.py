@@ -87,9 +87,10 @@ def test_decoding_a_batch_of_very_unequal_lengths(name, lengths, model_root):
             ok, err = close(got[row], ref[i][lengths[i] + j], "bfloat16", name, "unequal batch")
             assert ok, (i, j, err)
     items = 1024 // raw["num_key_value_heads"]
-    for B in (len(lengths), len(lengths) - 1):
+    from herbert_rs_amd.engine.batch import decode_batch_bucket
+    for B in {decode_batch_bucket(len(lengths)), decode_batch_bucket(len(lengths) - 1)}:      # (the steps' sizes)
         assert engine._decode[B].static.range_lists == [(items, 64)]      # the list was what ran
-    assert engine.graphs_captured >= 3
+    assert engine.graphs_captured >= 2          # (a context bucket's edge is passed on the way)
     for s in slots:
         engine.free_slot(s)
     engine.cache.check()
