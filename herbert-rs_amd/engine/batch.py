@@ -160,11 +160,20 @@ def pack(entries, start_lengths, device, staging=None):
 
 
 def decode_batch_bucket(sequences):
-    """The batch size that a decode step of `sequences` sequences runs at: the next power of two.
-    The kernels' cost goes by classes of rows (up to 16, 32, 64, ...), not by the row; a batch whose
-    sequences end one after another then passes through 16, 8, 4, 2, 1 and not through every size
-    below its first, and each size is a shape that has to be run once by the host and captured."""
-    return 1 << max(0, int(sequences) - 1).bit_length()
+    """The batch size that a decode step of `sequences` sequences runs at: 1, 2, 3, 4, 6, 8, then four
+    sizes for every doubling (10, 12, 14, 16, 20, 24, 28, 32, 40, ...), the rows beyond the sequences
+    being padding. Every size is a shape that the host has to walk through once and record; a batch
+    whose sequences end one after another then meets ten shapes on its way down from 16 instead of
+    sixteen. A padding row is not free where a kernel's time goes with its rows (the few-row product
+    reads its activations once a workgroup: about 2 % a row), so the sizes stay within an eighth to a
+    quarter of the sequences (measured on the 1.7B shape, 16 sequences that end 14 tokens apart:
+    rounding up to powers of two took 3 % more time for the 250 steps than exact sizes)."""
+    n = max(1, int(sequences))
+    if n <= 4:
+        return n
+    top = 1 << (n - 1).bit_length()          # the power of two at or above n
+    step = max(2, top // 8) if n > 8 else 2
+    return -(-n // step) * step
 
 
 class StaticDecodeMeta:

@@ -35,7 +35,6 @@ class _DecodeState:
         self.static = static
         self.logits = logits
         self.seen = {}          # (context bucket, unequal) -> steps of that shape run so far
-        self.sized = False      # a step of this batch size has run outside a graph: its buffers exist
 
 
 # Captured graphs kept at any time, over all batch sizes and context buckets; the least recently
@@ -85,6 +84,7 @@ class Engine:
         self._graphs = OrderedDict()    # (batch size, context bucket, unequal) -> graph, least recently used first
         self._shared_logits = None      # [rows, vocab], made by the first decode step, grown by a larger batch
         self._capture_stream = None     # the stream that graphs are captured on
+        self._sized_rows = 0            # the largest decode step that has run outside a graph: buffers for it exist
         self.graphs_captured = 0
         self.ignored_tensors = []       # stored tensors that the model did not ask for
         self._tensor_source = None      # how get_tensor finds a tensor again: set by the constructors below
@@ -286,16 +286,16 @@ class Engine:
             return state.logits[:n]
         seen = state.seen.get(key[1:], 0)
         state.seen[key[1:]] = seen + 1
-        if seen == 0 and not state.sized:
-            # the batch size's first step runs as it is: that also sizes every scratch buffer
-            state.sized = True
+        if B > self._sized_rows:
+            # no step this large has run yet: it runs as it is, which also sizes every scratch buffer
+            self._sized_rows = B
             return self.model.forward(self.rt, meta, self.cache, logits_out=state.logits)[:n]
         if len(self._graphs) >= MAX_GRAPHS:
             torch.cuda.synchronize(self.device)      # no graph that is dropped here still runs
             while len(self._graphs) >= MAX_GRAPHS:
                 self._graphs.popitem(last=False)
-        # A shape whose batch size has run before is recorded at once, without a pass of its own
-        # outside a graph: the buffers are there. Where one turns out to be missing after all (a
+        # A shape no larger than one that has run before is recorded at once, without a pass of its
+        # own outside a graph: the buffers are there. Where one turns out to be missing after all (a
         # longer context's partial results, a list of ranges), the recording is given up and the
         # step runs as it is; the shape's next step is then recorded.
         # Recorded on a stream of its own behind what the step's stream holds, without waiting for
@@ -323,7 +323,7 @@ class Engine:
             # recording) instead of failing in a recording again at every step.
             step_stream.wait_stream(self._capture_stream)
             state.seen[key[1:]] = 0
-            state.sized = False
+            self._sized_rows = 0
             raise
         step_stream.wait_stream(self._capture_stream)
         self._graphs[key] = graph
