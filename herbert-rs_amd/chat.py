@@ -112,23 +112,24 @@ class ChatSession:
         return result
 
 
-HELP = """--- Commands ---
-  /help, /h       Show this help
-  /quit, /q       Quit
-  /exit           Quit
-  /clear          Clear conversation
-  /stats          Show session statistics
-  /config         Show sampling config
-  /greedy         Set greedy decoding (temp=0)
-  /temp <val>     Set temperature (0 = greedy)
-  /topk <val>     Set top-k (0 = disabled)
-  /topp <val>     Set top-p (1 = disabled)
-  /think <N>      Set think budget (max tokens in <think>, 0 = unlimited)
-  /nothink        Disable thinking (a think block is closed at once)
-  /arch           Show the GPU this runs on
-  !<command>      Run shell command (e.g. !ls, !pwd)
+# The commands are the reference's (crates/cli/src/chat.rs:549-572: their names and what they do,
+# without those of tools, images and embeddings); the wording is this library's.
+HELP = """Commands of a conversation (a line that starts with / or !):
+  /help  /h        this list
+  /quit  /q  /exit leave
+  /clear           forget the conversation; the next message starts a new one
+  /stats           turns, tokens and speeds so far
+  /config          the sampling parameters in use
+  /greedy          always take the most likely token (temperature 0)
+  /temp <x>        temperature; 0 is greedy
+  /topk <n>        keep the n most likely tokens; 0 keeps all
+  /topp <p>        keep the most likely tokens up to a total probability p; 1 keeps all
+  /think <n>       at most n tokens inside a <think> block; 0 lifts the limit
+  /nothink         no thinking: a think block is closed as soon as it opens
+  /arch            the GPU this runs on
+  !<command>       run a shell command, e.g. !ls
 
-  Use \\ at end of line to continue input on next line."""
+A line that ends with \\ goes on in the next line."""
 
 
 def _rate(tokens, seconds):

@@ -776,6 +776,51 @@ def test_a_seed_gives_the_same_weights_on_the_gpu_and_in_a_folder(dtype, tmp_pat
     assert close(a[39].numpy(), ref[39], dtype, "B")[0]
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_padding_rows_of_a_decode_step_change_nothing(dtype, model_root):
+    """Decode steps run at a ladder of batch sizes (5 sequences as 6, 7 as 8, 9 as 10, 17 as 20), the
+    rows left over being padding in a slot and a page of their own. Every sequence's logits are
+    what it gets alone (in float32 bit for bit: those kernels sum every output the same way whatever
+    the batch), through eager steps, recordings and replays; the pages of the sequences hold what
+    they hold without the padding; the padding's slot and page are nobody's."""
+    from herbert_rs_amd.engine.batch import decode_batch_bucket
+    name = "D"
+    folder = make_folder(model_root, name, dtype)
+    vocab = CONFIGS[name][0]["vocab_size"]
+    assert [decode_batch_bucket(n) for n in (1, 2, 3, 4, 5, 7, 9, 16, 17, 33, 64, 65)] == \
+        [1, 2, 3, 4, 6, 8, 10, 16, 20, 40, 64, 80]
+    n_seqs, steps = 17, 6
+    seqs = [random_tokens(vocab, 20 + 9 * i + steps, 400 + i) for i in range(n_seqs)]
+    heads = [len(t) - steps for t in seqs]
+    alone_engine = hb.load(folder, dtype=dtype, cache_tokens=64 * 8)
+    alone = []
+    for t, h in zip(seqs, heads):
+        slot = alone_engine.alloc_slot()
+        alone_engine.step([StepEntry(slot, t[:h], [])])
+        alone.append(torch.stack([alone_engine.step([StepEntry(slot, [t[h + j]], [0])])[0] for j in range(steps)]).cpu())
+        alone_engine.free_slot(slot)
+    engine = hb.load(folder, dtype=dtype, cache_tokens=64 * 4 * n_seqs)
+    pad_slot = engine.cache.pad_slot
+    for n in (5, 7, 9, 17):
+        slots = [engine.alloc_slot() for _ in range(n)]
+        assert pad_slot not in slots
+        engine.step([StepEntry(s, t[:h], []) for s, t, h in zip(slots, seqs, heads)])
+        for j in range(steps):
+            got = engine.step([StepEntry(s, [t[h + j]], [0]) for s, t, h in zip(slots, seqs, heads)]).cpu()
+            assert got.shape == (n, vocab)
+            for i in range(n):
+                if dtype == "float32":
+                    assert torch.equal(got[i], alone[i][j]), (n, j, i)
+                else:
+                    assert close(got[i].numpy(), alone[i][j].numpy(), dtype, name, "padded step")[0], (n, j, i)
+        for s in slots:
+            engine.free_slot(s)
+        engine.cache.check()
+    assert sorted(engine._decode) == [6, 8, 10, 20] and engine.graphs_captured >= 4
+    for g in engine.cache.kv_groups.values():
+        assert g.pages.held_count == 0 and int(g.table[pad_slot].min()) == g.pool.shape[2] - 1
+
+
 def test_two_engines_on_two_streams_share_no_scratch(model_root):
     """Each engine's kernels have scratch of their own (the partial results of the decode
     attention's ranges, the K slices of products): two engines of one process, stepped in turn on
