@@ -2,7 +2,7 @@
 config.json gives varies at once (head sizes in steps of 16 up to 128, one to eight kv heads with
 one to eight query heads each, widths and vocabularies that are no power of two, one to three
 layers, windows on some layers, partial rotation, linear and yarn scaling, tied and separate
-heads), and so do the requests: up to six sequences of unequal lengths whose prompts come whole or
+heads), and so do the requests: up to seven sequences of unequal lengths whose prompts come whole or
 in pieces, then their next tokens one by one, the shorter ones ending earlier. Every position's
 logits are compared with the plain implementation in float32 and in bfloat16."""
 import random
@@ -47,7 +47,7 @@ def random_config(rng):
 
 
 def random_requests(rng):
-    n = rng.choice([1, 1, 2, 3, 4, 6])
+    n = rng.choice([1, 1, 2, 3, 4, 5, 6, 7])          # (5 and 7 run as decode steps of 6 and 8: one padding row)
     prompts = [rng.choice([1, 2, 5, 17, 63, 64, 65, 100, 129, 200, 300]) for _ in range(n)]
     more = [rng.choice([0, 1, 3, 8, 20]) for _ in range(n)]          # tokens fed one by one after the prompt
     piece = rng.choice([None, None, 16, 64, 100])                    # prompts in pieces of this many tokens
