@@ -40,6 +40,7 @@ class BatchMeta:
     derived: dict = None       # what kernels' host sides derive once a step (tile lists and the like)
     context_bucket: int = 0    # max_context rounded up (see bucket): sizes the decode kernels' grids
     unequal: int = 0           # how unequal the contexts' lengths are: 0 (alike), 1, 2 (see unequal_level)
+    num_real: int = 0          # sequences that are no padding rows (0: all of them)
     static: object = None      # the StaticDecodeMeta whose buffers these are, if any
 
     def ranges_for(self, items, unit):
@@ -161,18 +162,20 @@ def pack(entries, start_lengths, device, staging=None):
 
 def decode_batch_bucket(sequences):
     """The batch size that a decode step of `sequences` sequences runs at: 1, 2, 3, 4, 6, 8, then four
-    sizes for every doubling (10, 12, 14, 16, 20, 24, 28, 32, 40, ...), the rows beyond the sequences
-    being padding. Every size is a shape that the host has to walk through once and record; a batch
-    whose sequences end one after another then meets ten shapes on its way down from 16 instead of
-    sixteen. A padding row is not free where a kernel's time goes with its rows (the few-row product
-    reads its activations once a workgroup: about 2 % a row), so the sizes stay within an eighth to a
-    quarter of the sequences (measured on the 1.7B shape, 16 sequences that end 14 tokens apart:
-    rounding up to powers of two took 3 % more time for the 250 steps than exact sizes)."""
+    sizes for every doubling up to 64 (10, 12, 14, 16, 20, 24, 28, 32, 40, ...) and eight beyond (72,
+    80, 88, ...), the rows beyond the sequences being padding. Every size is a shape that the host
+    has to walk through once and record; a batch whose sequences end one after another then meets
+    ten shapes on its way down from 16 instead of sixteen. A padding row is not free where a
+    kernel's time goes with its rows (the few-row product reads its activations once a workgroup:
+    about 2 % a row; beyond 64 sequences every eighth more is another wave on some CUs of the
+    attention), so the sizes stay within an eighth to a quarter of the sequences (measured on the
+    1.7B shape, 16 sequences that end 14 tokens apart: rounding up to powers of two took 3 % more
+    time for the 250 steps than exact sizes)."""
     n = max(1, int(sequences))
     if n <= 4:
         return n
     top = 1 << (n - 1).bit_length()          # the power of two at or above n
-    step = max(2, top // 8) if n > 8 else 2
+    step = 2 if n <= 8 else top // 8 if n <= 64 else top // 16
     return -(-n // step) * step
 
 
@@ -255,4 +258,5 @@ class StaticDecodeMeta:
         m.max_position = m.max_context - 1
         m.context_bucket = bucket(m.max_context)
         m.unequal = unequal
+        m.num_real = n
         return m

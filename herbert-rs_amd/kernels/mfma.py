@@ -464,6 +464,8 @@ def _decode_split(meta, nkv, window):
         span = min(span, (window + 63) // 64 + 1)
     pairs = meta.num_seqs * nkv
     if 2 * pairs >= DECODE_WAVES:
+        # (how evenly the waves sit is a matter of the sequences themselves: padding rows' waves end at once)
+        pairs = (getattr(meta, "num_real", 0) or meta.num_seqs) * nkv
         # Two waves a CU already: a merge costs more than it gains (5 to 8 % of a step), as long as
         # the waves sit evenly. A wave that reads a whole context is a long job, and the time goes
         # with the CU that has the most of them (three where most have two: 65 sequences took a

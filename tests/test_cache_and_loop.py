@@ -583,6 +583,34 @@ def test_turns_on_a_kept_slot_go_on_from_what_it_holds(ahead, rolls_back):
     assert eng.cache.slots.held_count == 0
 
 
+def test_decode_steps_run_at_a_ladder_of_sizes_filled_up_with_padding():
+    """The fixed metadata of a decode step, without a GPU: a step of fewer sequences than its size
+    is filled up with rows of one token (id 0, position 0) in the padding slot; the lists of ranges
+    cover every row; how unequal the contexts are is judged on the sequences alone."""
+    from herbert_rs_amd.engine.batch import StaticDecodeMeta, StepEntry, decode_batch_bucket, range_list
+    ladder = [decode_batch_bucket(n) for n in range(1, 81)]
+    assert ladder[:16] == [1, 2, 3, 4, 6, 6, 8, 8, 10, 10, 12, 12, 14, 14, 16, 16]
+    assert sorted(set(ladder)) == [1, 2, 3, 4, 6, 8, 10, 12, 14, 16, 20, 24, 28, 32, 40, 48, 56, 64, 72, 80]
+    assert [decode_batch_bucket(n) for n in (81, 129, 130, 257)] == [88, 144, 144, 288]
+    assert all(b >= n and 4 * b <= 5 * n + 4 for n, b in enumerate(ladder, 1))      # within a quarter (and a row)
+    meta = StaticDecodeMeta(6, "cpu", pad_slot=99)
+    entries = [StepEntry(3, [11], [0]), StepEntry(7, [12], [0]), StepEntry(1, [13], [0]), StepEntry(2, [14], [0]),
+               StepEntry(5, [15], [0])]
+    m = meta.update(entries, [700, 9, 64, 0, 30])
+    assert m.num_seqs == m.num_tokens == 6 and m.token_ids.tolist() == [11, 12, 13, 14, 15, 0]
+    assert m.positions.tolist() == [700, 9, 64, 0, 30, 0] and m.slots.tolist() == [3, 7, 1, 2, 5, 99]
+    assert m.context_lens.tolist() == [701, 10, 65, 1, 31, 1] and m.want_rows.tolist() == list(range(6))
+    assert m.max_context == 701 and m.context_bucket == 768 and m.unequal == 2
+    ranges = m.ranges_for(16, 64)           # five sequences and the padding row, each at least one range
+    assert ranges.tolist() == range_list([701, 10, 65, 1, 31, 1], 16, 64).tolist() and ranges.tolist()[6] <= 16
+    # the next step brings fewer sequences: the rows that held sequences are padding now
+    m = meta.update(entries[:2], [701, 10])
+    assert m.slots.tolist() == [3, 7, 99, 99, 99, 99] and m.context_lens.tolist() == [702, 11, 1, 1, 1, 1]
+    assert m.token_ids.tolist()[2:] == [0, 0, 0, 0]
+    with pytest.raises(ValueError, match="do not fit"):
+        meta.update(entries + entries[:2], [1] * 7)
+
+
 def test_the_memory_a_cache_needs_counts_pages_and_state():
     """What the engine compares with the GPU's free memory before it builds a cache: the pools of
     keys and values by pages, and fixed-size state by slots, entries of equal need together."""

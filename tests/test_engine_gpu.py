@@ -788,7 +788,7 @@ def test_padding_rows_of_a_decode_step_change_nothing(dtype, model_root):
     folder = make_folder(model_root, name, dtype)
     vocab = CONFIGS[name][0]["vocab_size"]
     assert [decode_batch_bucket(n) for n in (1, 2, 3, 4, 5, 7, 9, 16, 17, 33, 64, 65)] == \
-        [1, 2, 3, 4, 6, 8, 10, 16, 20, 40, 64, 80]
+        [1, 2, 3, 4, 6, 8, 10, 16, 20, 40, 64, 72]
     n_seqs, steps = 17, 6
     seqs = [random_tokens(vocab, 20 + 9 * i + steps, 400 + i) for i in range(n_seqs)]
     heads = [len(t) - steps for t in seqs]
