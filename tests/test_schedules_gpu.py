@@ -169,6 +169,50 @@ def test_turns_on_a_kept_slot_leave_the_whole_conversation_in_the_cache(name, dt
     engine.cache.check()
 
 
+def test_seeded_turns_draw_the_same_with_and_without_a_step_ahead(model_root):
+    """A seeded conversation at temperature 0.8 whose sampler goes on from turn to turn: with decode
+    steps put on the stream one ahead of the host, a turn that ends on a token's value has drawn once
+    more than it has tokens; the draw is taken back, so that every turn's tokens and the generator's
+    state after it are those of the loop that waits for each token (one draw a token, as the
+    reference's sampler draws)."""
+    from herbert_rs_amd.engine.generate import Generator
+    from herbert_rs_amd.sampling import SamplingParams
+    from herbert_rs_amd.sampling.sampler import Sampler
+    folder = make_folder(model_root, "D", "float32")
+    vocab = CONFIGS["D"][0]["vocab_size"]
+    turns = [random_tokens(vocab, n, 430 + i) for i, n in enumerate((30, 4, 17))]
+    outcome = {}
+    for ahead in (False, True):
+        engine = hb.load(folder, dtype="float32", cache_tokens=64 * 6)
+        gen = Generator(engine, max_batch=1, run_ahead=ahead)
+        params = SamplingParams(temperature=0.8, top_k=20, top_p=1.0, max_tokens=12, ignore_eos=True,
+                                repeat_check=False, seed=5)
+        sampler = Sampler(params, 1, vocab, engine.device)
+        slot = engine.alloc_slot()
+        said, states, last = [], [], []
+        for turn, tokens in enumerate(turns):
+            count = []
+            # the caller ends the turn at its fifth token: a value nobody knew beforehand
+            r = gen.extend(slot, last + tokens, params, sampler,
+                           on_token=lambda i, t: count.append(t) or ("enough" if len(count) == 5 else None))
+            assert len(r.tokens) == 5
+            said.append(r.tokens)
+            states.append(int(sampler.states[0].item()))
+            last = [r.tokens[-1]]
+        outcome[ahead] = (said, states)
+        engine.free_slot(slot)
+        engine.cache.check()
+    assert outcome[True] == outcome[False]
+    # five draws a turn: the state after the turns is the seed's stream stepped 5, 10 and 15 times
+    from herbert_rs_amd.sampling import xorshift
+    state, want = xorshift.initial_state(5), []
+    for n in range(15):
+        state = xorshift.step(state)
+        if n % 5 == 4:
+            want.append(state - (1 << 64) if state >= (1 << 63) else state)
+    assert outcome[True][1] == want
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_a_windowed_cache_rolls_back_only_to_keys_it_still_has(dtype, model_root):
     """Configuration C: one layer sees 70 keys and has given up the pages before them. Rolling
