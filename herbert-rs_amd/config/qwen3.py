@@ -70,6 +70,16 @@ class Qwen3Config:
             if raw.get(key) is not None:
                 raise ConfigError(f"config.json: {key} is set; expert feed-forwards are not "
                                   "part of this architecture here")
+        # What the reference fixes in code for this family (no biases: crates/core/src/config.rs:508-512;
+        # SwiGLU: crates/backends/backend_common/src/loader_common.rs:853) a config.json may contradict: the
+        # reference never reads these keys and would run such a model wrongly; here it is refused.
+        for key in ("attention_bias", "mlp_bias"):
+            if raw.get(key) is True:
+                raise ConfigError(f"config.json: {key} is true; this architecture has no biases here "
+                                  "(stored bias tensors would be passed over)")
+        if raw.get("hidden_act") not in (None, "silu", "swish"):
+            raise ConfigError(f"config.json: hidden_act {raw.get('hidden_act')!r}; the feed-forward here is "
+                              "silu(gate) * up")
         r = Reader(raw)
         rope_theta = r.number("rope_theta")
         rope_params = raw.get("rope_parameters")

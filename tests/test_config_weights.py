@@ -280,6 +280,22 @@ def test_names_are_normalised_and_fused_tensors_cut(model_root, tmp_path):
         read_tensors(str(tmp_path), needs_of(TINY_B), name_map=NAMES)
 
 
+def test_keys_that_contradict_what_the_architecture_fixes_are_refused():
+    """The reference never reads attention_bias, mlp_bias or hidden_act (biases and the activation are
+    fixed for the family: crates/core/src/config.rs:508-512, loader_common.rs:853) and would run a
+    model that sets them otherwise wrongly; here such a config.json is an error, and the values that
+    the public Qwen3 checkpoints carry are accepted."""
+    ok = dict(TINY_A, attention_bias=False, hidden_act="silu", attention_dropout=0.0, use_cache=True,
+              sliding_window=None, use_sliding_window=False, max_window_layers=2, torch_dtype="bfloat16",
+              rope_scaling=None, bos_token_id=1, initializer_range=0.02)
+    cfg = resolve_architecture(ok).config_class.from_dict(ok)
+    assert cfg.hidden_size == TINY_A["hidden_size"] and cfg.layer_windows == (None, None)
+    for key, value, text in (("attention_bias", True, "no biases"), ("mlp_bias", True, "no biases"),
+                             ("hidden_act", "gelu", "silu")):
+        with pytest.raises(ConfigError, match=text):
+            resolve_architecture(ok).config_class.from_dict(dict(ok, **{key: value}))
+
+
 def counter_values(key, first, count, scale, offset):
     """The random weights' formula in NumPy, written from its description alone: the bytes of
     splitmix64(key, i) summed and centred, one float32 product, one float32 sum."""
