@@ -122,7 +122,7 @@ def run_workload(args, index, new=None):
         "steps": st.decode_steps, "warmup": 0, "ms_per_step": round(ms, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
-        "data": "synthetic: random weights N(0, 0.02), random token ids",
+        "data": "synthetic: random weights of standard deviation 0.02 (near normal: sums of eight random bytes), random token ids",
         "config": {"model": name, "layers": layers_full, "layers_run": cfg.num_hidden_layers,
                    "hidden_size": cfg.hidden_size,
                    "num_attention_heads": cfg.num_attention_heads,
@@ -390,8 +390,8 @@ def main():
         "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
-        "data": "synthetic: random weights N(0, 0.02), random token ids, cache filled by prefill of "
-                "random prompts",
+        "data": "synthetic: random weights of standard deviation 0.02 (near normal: sums of eight random bytes), "
+                "random token ids, cache filled by prefill of random prompts",
         "config": {
             "model": "Qwen3-8B shape", "layers": layers_full, "layers_run": layers,
             "hidden_size": H, "num_attention_heads": cfg.num_attention_heads,
