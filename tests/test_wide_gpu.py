@@ -12,6 +12,9 @@ import numpy as np
 import pytest
 import torch
 
+import herbert_rs_amd as hb
+from herbert_rs_amd.engine import StepEntry
+
 from . import replay_util as ru
 from .bounds import close
 from .plain_cache import forget, plain_rows
@@ -136,3 +139,46 @@ def test_prompt_of_2048_and_decoding_at_batch_1_8_64(dtype, wide_folder, tmp_pat
             assert ok, f"request {rid} position {pos} ({group} {kind}): error {err}"
     if dtype == "float32":
         forget(wide_folder)
+
+
+def test_decoding_at_every_batch_size_of_the_ladder_at_these_widths(wide_folder):
+    """Decode steps run at a ladder of batch sizes, and the host picks other kernels along it (the
+    few-row kernel up to 16 rows, tiles of 32 and of 64 rows with K slices and a second kernel that
+    norms, larger tiles beyond; an RMSNorm handed on half done or whole). Every size up to 80, with
+    one sequence fewer than the size where that leaves a padding row, at the 8B widths: the bfloat16
+    engine's logits against those of the float32 engine (which the other tests hold against the
+    plain implementation), within the bounds of these widths, for the prompts' last tokens and three
+    decode steps."""
+    from herbert_rs_amd.engine.batch import decode_batch_bucket
+    sizes = sorted({decode_batch_bucket(n) for n in range(1, 81)})
+    assert sizes[:10] == [1, 2, 3, 4, 6, 8, 10, 12, 14, 16] and sizes[-1] == 80
+    most = max(sizes)
+    engines = {d: hb.load(wide_folder, dtype=d, cache_tokens=64 * 4 * most) for d in ("bfloat16", "float32")}
+    worst = 0.0
+    for size in sizes:
+        n = size - 1 if size in (6, 10, 14, 20, 28, 40, 56, 72) else size      # every other size with a padding row
+        assert decode_batch_bucket(n) == size
+        lengths = [1 + (41 * i + 7 * size) % 150 for i in range(n)]
+        seqs = [random_tokens(VOCAB, m + 3, 2000 + 97 * size + i) for i, m in enumerate(lengths)]
+        outs = {}
+        for d, engine in engines.items():
+            slots = [engine.alloc_slot() for _ in range(n)]
+            rows = [engine.step([StepEntry(s, t[:m], [m - 1]) for s, t, m in zip(slots, seqs, lengths)])]
+            for j in range(3):
+                rows.append(engine.step([StepEntry(s, [t[m + j]], [0]) for s, t, m in zip(slots, seqs, lengths)]))
+            outs[d] = torch.stack(rows).double()                 # [4, n, vocab]
+            for s in slots:
+                engine.free_slot(s)
+            engine.cache.check()
+        ref, got = outs["float32"], outs["bfloat16"]
+        rms = ref.pow(2).mean(-1).sqrt().clamp_min(1e-30)
+        rel_max = ((got - ref).abs().amax(-1) / rms)
+        rel_l2 = ((got - ref).pow(2).mean(-1).sqrt() / rms)
+        from .bounds import BF16_REL_L2, BF16_REL_RMS
+        from .conftest import observe
+        observe("bfloat16 wide every size, against float32: max / rms", float(rel_max.max()))
+        observe("bfloat16 wide every size, against float32: rms / rms", float(rel_l2.max()))
+        assert float(rel_max.max()) <= BF16_REL_RMS["wide"] and float(rel_l2.max()) <= BF16_REL_L2["wide"], \
+            (size, n, float(rel_max.max()), float(rel_l2.max()))
+        worst = max(worst, float(rel_l2.max()))
+    assert worst > 0.0
