@@ -41,13 +41,15 @@ class _DecodeState:
 # replayed one is dropped for a new one. A graph holds no logits of its own and no scratch (the
 # parts' buffers are the runtime's), so a graph costs its kernel arguments only; the cap bounds
 # what a long run over many batch sizes and contexts accumulates. A batch whose sequences end one
-# after another passes through every size below its first, and each (size, context bucket) is a
-# graph: the cap leaves room for a few such batches' graphs, so that the next batch finds them.
+# after another passes through the sizes of the ladder below its first (batch.decode_batch_bucket),
+# and each (size, context bucket) is a graph: the cap leaves room for many such batches' graphs, so
+# that the next batch finds them.
 MAX_GRAPHS = 192
 # Decode steps write their logits into the first rows of one buffer [rows, vocab] float32 that the
-# engine keeps (`step` hands out a copy of them unless it is asked for the rows themselves). The buffer starts with this many rows (39 MB for a vocabulary of 151,936) or
-# as many as the cache has slots, if fewer; a larger batch makes a larger one (twice the rows, or
-# what the batch needs) and every graph, which holds the old one's address, is dropped.
+# engine keeps (`step` hands out a copy of them unless it is asked for the rows themselves). The
+# buffer starts with this many rows (39 MB for a vocabulary of 151,936) or as many as the cache's
+# slots need, if fewer; a larger batch makes a larger one (twice the rows, or what the batch needs)
+# and every graph, which holds the old one's address, is dropped.
 SHARED_LOGITS_ROWS = 64
 # Batch sizes whose fixed metadata buffers are kept; the least recently used goes, with its graphs.
 MAX_DECODE_BATCH_SIZES = 96
@@ -241,17 +243,17 @@ class Engine:
 
     def _decode_step(self, entries, starts, tokens_on_device=None):
         """One token for each sequence, every logit wanted: the launch-bound case. The step's
-        metadata lives in fixed buffers; from the second step of a shape on, the forward pass is a
-        captured HIP graph that is replayed, so that the host launches one graph and not hundreds
-        of kernels. The step runs at the next power of two of its sequences, filled up with padding
-        rows in the cache's padding slot (the kernels' cost goes by classes of rows, and a batch
-        whose sequences end one after another then meets few new shapes instead of one a
-        sequence). A graph is tied to that batch size, to the bucket of the longest context
-        (which sizes the attention grid) and to whether the contexts are of very unequal lengths
-        (the attention then deals its grid out by a list). All graphs write their logits into the
-        first rows of the engine's one buffer: what a step returns is overwritten by the next
-        decode step. At most MAX_GRAPHS graphs and MAX_DECODE_BATCH_SIZES batch sizes are kept,
-        the least recently used go first."""
+        metadata lives in fixed buffers, and the forward pass of a shape is recorded into a HIP graph
+        that is replayed from then on, so that the host launches one graph and not hundreds of
+        kernels. The step runs at the size of a ladder at or above its sequences
+        (batch.decode_batch_bucket), filled up with padding rows in the cache's padding slot: a batch
+        whose sequences end one after another then meets few new shapes instead of one a sequence.
+        A graph is tied to that batch size, to the bucket of the longest context (which sizes the
+        attention grid) and to whether the contexts are of very unequal lengths (the attention then
+        deals its grid out by a list). All graphs write their logits into the first rows of the
+        engine's one buffer; what is returned here is a view of those rows, which the next decode
+        step writes again (`step` copies it for callers that keep it). At most MAX_GRAPHS graphs and
+        MAX_DECODE_BATCH_SIZES batch sizes are kept, the least recently used go first."""
         n = len(entries)
         B = decode_batch_bucket(n)          # the step runs at this size, the rows beyond n are padding
         state = self._decode.get(B)

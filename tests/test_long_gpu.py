@@ -3,8 +3,8 @@
 The reference runs contexts out to 16,000 tokens (docs/benchmarks/qwen3-0.6b-results.md:41-49) and
 feeds long prompts in chunks that must give what the whole prompt gives
 (crates/backends/backend_common/src/generic_model.rs:445-522). Above 4,096 tokens the engine's
-decode steps change the width of their context buckets, the decode attention cuts a context into more
-than 32 ranges, a prompt's chunks attend over a long cache, and a batch with one long sequence
+decode steps change the width of their context buckets (512 tokens at 6,000, 1,024 at 9,000, 2,048
+at 17,000), the decode attention cuts a context into more than 32 ranges, a prompt's chunks attend over a long cache, and a batch with one long sequence
 beside short ones deals the attention's grid out by a list: every one of these is crossed here, in
 bfloat16 and in float32, with a model of heads of 128 and one of heads of 64.
 
@@ -70,6 +70,8 @@ def requests(vocab, tag):
     reqs = {"p9": (random_tokens(vocab, 9000 + DECODE_STEPS, 700), 9000, 2048)}
     if tag == "long128":
         reqs["p17"] = (random_tokens(vocab, 17000 + DECODE_STEPS, 701), 17000, 8192)
+    else:
+        reqs["p6"] = (random_tokens(vocab, 6000 + DECODE_STEPS, 702), 6000, 2048)
     # a batch of four that start together: one long, three short
     for i, n in enumerate([9300, 300, 1500, 70]):
         reqs[f"u{i}"] = (random_tokens(vocab, n + DECODE_STEPS - 3 * i, 710 + i), n, None)
@@ -105,7 +107,7 @@ def long_trace(reqs):
                     live.remove(rid)
             add(entries, end)
 
-    for rid in [r for r in ("p17", "p9") if r in reqs]:
+    for rid in [r for r in ("p17", "p9", "p6") if r in reqs]:
         toks, n, chunk = reqs[rid]
         places = prompt_places(n, chunk)
         for a in range(0, n, chunk):
