@@ -821,6 +821,28 @@ def test_padding_rows_of_a_decode_step_change_nothing(dtype, model_root):
         assert g.pages.held_count == 0 and int(g.table[pad_slot].min()) == g.pool.shape[2] - 1
 
 
+def test_a_decode_steps_logits_are_the_callers_own(model_root):
+    """What `step` returns for a decode step is a copy of the caller's own: the next decode step does
+    not change it. Asked for the rows themselves (`keep_logits=False`, as the generation loop asks),
+    the caller gets a view of the engine's buffer, which the next decode step writes again."""
+    folder = make_folder(model_root, "B", "float32")
+    tokens = random_tokens(384, 30, 61)
+    engine = hb.load(folder, dtype="float32", cache_tokens=64 * 2)
+    slot = engine.alloc_slot()
+    engine.step([StepEntry(slot, tokens[:20], [])])
+    own = engine.step([StepEntry(slot, [tokens[20]], [0])])
+    kept = own.clone()
+    view = engine.step([StepEntry(slot, [tokens[21]], [0])], keep_logits=False)
+    seen = view.clone()
+    assert torch.equal(own, kept) and not torch.equal(own, seen)
+    nxt = engine.step([StepEntry(slot, [tokens[22]], [0])])
+    assert torch.equal(own, kept) and torch.equal(view, nxt) and not torch.equal(view, seen)
+    assert own.data_ptr() != view.data_ptr() and nxt.data_ptr() != view.data_ptr()
+    ref = plain_logits(folder, tokens[:23])
+    for got, p in ((own, 20), (seen, 21), (nxt, 22)):
+        assert close(got[0].cpu().numpy(), ref[p], "float32", "B")[0], p
+
+
 def test_two_engines_on_two_streams_share_no_scratch(model_root):
     """Each engine's kernels have scratch of their own (the partial results of the decode
     attention's ranges, the K slices of products): two engines of one process, stepped in turn on
