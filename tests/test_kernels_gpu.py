@@ -2,6 +2,7 @@
 engine's: odd widths, heads and groups, sizes at and across tile edges."""
 import math
 
+import numpy as np
 import pytest
 import torch
 
@@ -878,3 +879,21 @@ def test_gemm_mfma_with_k_slices(M, N, K):
         c3 = base.clone()
         mfma.gemm(a, wp, c3, accumulate=True, packed=packed)
         assert torch.equal(c2, c3)                      # the same bits on every run
+
+
+# ---------------------------------------------------------------- random weights
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n,first", [(1, 0), (255, 7), (256, 0), (100003, 12345), (1 << 20, (1 << 33) + 5)])
+def test_random_fill_on_the_gpu_is_the_hosts(dtype, n, first):
+    """The kernel that draws weights on the GPU and the host's threads compute one function: the same
+    bits for any count, any first index (also beyond 2^32), as float32 and as bfloat16, with and without
+    an offset; and against the formula itself for the first values."""
+    from herbert_rs_amd.weights import random_init as ri
+    from .test_config_weights import counter_values
+    key = 0x0123456789ABCDEF ^ n
+    for scale, offset in ((0.02 / ri.BYTE_SUM_SIGMA, 0.0), (0.1 / ri.BYTE_SUM_SIGMA, 1.0)):
+        on_gpu = ri.counter_fill(torch.empty(n, dtype=dtype, device=dev()), key, scale, offset, first=first)
+        on_host = ri.counter_fill(torch.empty(n, dtype=dtype), key, scale, offset, first=first)
+        assert torch.equal(on_gpu.cpu(), on_host)
+        want = counter_values(key, first, min(n, 50), scale, offset)
+        assert np.array_equal(on_host[:50].float().numpy(), torch.tensor(want).to(dtype).float().numpy())
