@@ -9,6 +9,8 @@ prefill_with_token, decode_step and verify_draft_tokens
 cases are kept: empty input (:139-152), token id >= vocab (:165-171), position
 beyond max_position_embeddings (:531-537).
 """
+from collections import OrderedDict
+
 import numpy as np
 import torch
 
@@ -17,7 +19,6 @@ from ..config import load_config
 from ..errors import BackendError, ModelLoadError, NeedsEagerStep, RequestError
 from ..parts import Runtime
 from ..weights import read_tensor, read_tensors
-from collections import OrderedDict
 
 from . import batch as batching
 from .batch import StaticDecodeMeta, StepEntry, decode_batch_bucket
@@ -34,7 +35,6 @@ class _DecodeState:
     def __init__(self, static, logits):
         self.static = static
         self.logits = logits
-        self.seen = {}          # (context bucket, unequal) -> steps of that shape run so far
 
 
 # Captured graphs kept at any time, over all batch sizes and context buckets; the least recently
@@ -78,7 +78,7 @@ class Engine:
                            self.device, max_slots)
         self.steps_run = 0
         # Steps in which every sequence brings one token and wants its logits keep their metadata in
-        # fixed buffers and run at a power-of-two batch size (see _decode_step), as graphs if asked
+        # fixed buffers and run at a batch size of a ladder (see _decode_step), as graphs if asked
         # for: only for models whose parts do nothing but enqueue GPU work.
         self.static_decode = self.model.graph_safe
         self.use_graphs = bool(use_graphs) and self.model.graph_safe
@@ -286,8 +286,6 @@ class Engine:
             self._graphs.move_to_end(key)
             graph.replay()
             return state.logits[:n]
-        seen = state.seen.get(key[1:], 0)
-        state.seen[key[1:]] = seen + 1
         if B > self._sized_rows:
             # no step this large has run yet: it runs as it is, which also sizes every scratch buffer
             self._sized_rows = B
@@ -324,7 +322,6 @@ class Engine:
             # starts over: its next step runs as it is (which shows the same failure outside a
             # recording) instead of failing in a recording again at every step.
             step_stream.wait_stream(self._capture_stream)
-            state.seen[key[1:]] = 0
             self._sized_rows = 0
             raise
         step_stream.wait_stream(self._capture_stream)
