@@ -20,7 +20,10 @@ F32_ABS = 1e-4
 #  - the largest error: the maximum of V noisy values grows with V (about sqrt(2 ln V) times the
 #    rms: 0.017 to 0.033 for vocabularies of 256 to 512, 0.043 to 0.051 for 151936).
 # ("random": the drawn configurations of test_random_configs_gpu, worst seen 0.011 and 0.036, and
-#  0.015 and 0.057 over one-off sweeps of 380 draws;
+#  0.015 and 0.057 over one-off sweeps of 380 draws; a further sweep of 800 draws had one row of one
+#  draw beyond the bound, 0.0188 and 0.065 (one head of 128, a window of 5 on both layers, width 128:
+#  little to average over), the same to the last bit whether its sequence ran whole and alone or
+#  in the draw's schedule, so rounding and no fault of cache or batch; the bound stays;
 #  "long": contexts of 9,000 to 17,000 tokens with scores scaled up so that a few far keys hold a
 #  query's weight, which also carries the rounding of those scores into the output: worst seen
 #  0.0146 and 0.050; "deep": 1 to 36 layers at a quarter of the 8B width, vocabulary 4096: 0.0084 and
