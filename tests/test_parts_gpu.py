@@ -378,6 +378,72 @@ def test_a_step_that_fails_leaves_the_state_as_it_was():
     assert torch.equal(run(True), run(False))
 
 
+@register("mixer", "toy_decay_on_the_gpu")
+class ToyDecayOnTheGpu(ToyDecayMixer):
+    """The same recurrence, but a step in which every sequence brings one token does GPU work only:
+    the states of the step's slots are gathered, advanced and put back by index. So the part is
+    graph_safe, and the engine runs such steps at the sizes of its ladder, records them and replays
+    them. Rows of padding bring the cache's padding slot, whose state they advance and nobody
+    reads; the part needs no word about them. Prompts take the host's loop."""
+    graph_safe = True
+
+    def forward(self, ctx, y, x):
+        meta = ctx.meta
+        if meta.max_new > 1:
+            return super().forward(ctx, y, x)
+        state = ctx.cache.state_views(ctx.cache_entry)[0]           # [slots + the padding slot, hidden]
+        proj = (y.float()[:, None, :] * self.w[None]).sum(-1)
+        slots = meta.slots.long()
+        s = self.decay * state.index_select(0, slots) + proj
+        state.index_copy_(0, slots, s)
+        x += s
+
+
+def test_a_graph_safe_mixer_with_state_through_padded_and_replayed_decode_steps():
+    """Five sequences decode together (steps of six rows, one of them padding), then three of them go
+    on (steps of three): first as they are, then recorded, then replayed. The logits are those of
+    the mixer that loops on the host and is never recorded, and those of the sequences run whole;
+    the padding slot's state is made NaN beforehand, so a row that read it would show."""
+    import dataclasses
+    spec = toy_spec()
+    gpu_layer = dataclasses.replace(spec.layers[0], mixer=PartSpec("toy_decay_on_the_gpu", spec.layers[0].mixer.params))
+    gpu_spec = dataclasses.replace(spec, layers=[gpu_layer, spec.layers[1]])
+    from herbert_rs_amd.engine.model import Model
+    from herbert_rs_amd.weights import random_tensors
+    w = random_tensors(Model(spec).tensor_needs(), 3, "float32", std=0.15, norm_std=0.1)
+    g = torch.Generator().manual_seed(5)
+    lengths, more = [3, 9, 1, 6, 4], [20, 8, 20, 8, 20]
+    seqs = [torch.randint(0, 60, (n + m,), generator=g).tolist() for n, m in zip(lengths, more)]
+
+    def run(model_spec):
+        engine = Engine(None, model_spec, w, dtype="float32", max_tokens=64 * 8)
+        for group in engine.cache.state_groups.values():
+            group.data[:, engine.cache.pad_slot] = float("nan")
+        slots = [engine.alloc_slot() for _ in seqs]
+        rows = [[] for _ in seqs]
+        first = engine.step([StepEntry(s, t[:n], [n - 1]) for s, t, n in zip(slots, seqs, lengths)]).cpu()
+        for i in range(len(seqs)):
+            rows[i].append(first[i])
+        for step in range(max(more)):
+            live = [i for i in range(len(seqs)) if step < more[i]]
+            out = engine.step([StepEntry(slots[i], [seqs[i][lengths[i] + step]], [0]) for i in live]).cpu()
+            for r, i in enumerate(live):
+                rows[i].append(out[r])
+        return engine, [torch.stack(r) for r in rows]
+
+    on_gpu, got = run(gpu_spec)
+    on_host, want = run(spec)
+    assert on_gpu.use_graphs and on_gpu.graphs_captured >= 2 and sorted(on_gpu._decode) == [3, 6]
+    assert not on_host.use_graphs and on_host.graphs_captured == 0
+    for a, b in zip(got, want):
+        assert torch.isfinite(a).all() and torch.allclose(a, b, atol=1e-5)
+    for i, t in enumerate(seqs):            # and the sequences whole, alone
+        slot = on_host.alloc_slot()
+        whole = on_host.step([StepEntry(slot, t, list(range(lengths[i] - 1, len(t))))]).cpu()
+        on_host.free_slot(slot)
+        assert torch.allclose(got[i], whole, atol=1e-4)
+
+
 # ---- a toy feed-forward with routing and a toy position encoding, defined here
 @register("feed_forward", "toy_routed")
 class ToyRoutedFeedForward(Part):
