@@ -11,6 +11,7 @@ from herbert_rs_amd.cache import Cache, KVNeed, StateNeed
 from herbert_rs_amd.engine import Engine, StepEntry
 from herbert_rs_amd.engine import batch as batching
 from herbert_rs_amd.engine.model import SharedParts
+from herbert_rs_amd.parts.attention import Attention
 from herbert_rs_amd.parts import (LayerSpec, ModelSpec, Part, PartSpec, Runtime, ScheduleEntry, StepContext,
                                   build, register)
 from herbert_rs_amd.weights import TensorNeed
@@ -442,6 +443,60 @@ def test_a_graph_safe_mixer_with_state_through_padded_and_replayed_decode_steps(
         whole = on_host.step([StepEntry(slot, t, list(range(lengths[i] - 1, len(t))))]).cpu()
         on_host.free_slot(slot)
         assert torch.allclose(got[i], whole, atol=1e-4)
+
+
+@register("mixer", "toy_counting_attention")
+class ToyCountingAttention(Attention):
+    """The library's attention with a state of fixed size beside its keys and values: how many
+    tokens the sequence has brought so far. Its cache need is a pair, so the entry has pages in
+    a group of keys and values and a number a slot in a group of state. GPU work only."""
+
+    def cache_need(self):
+        return (super().cache_need(), StateNeed((1,), torch.float32))
+
+    def forward(self, ctx, y, x, **how):
+        counts = ctx.cache.state_views(ctx.cache_entry)[0]          # [slots + the padding slot, 1]
+        starts = ctx.meta.seq_starts
+        counts.index_add_(0, ctx.meta.slots.long(), (starts[1:] - starts[:-1]).float()[:, None])
+        super().forward(ctx, y, x, **how)
+
+
+def test_a_mixer_whose_cache_need_is_keys_and_values_and_a_state():
+    import dataclasses
+    from herbert_rs_amd.errors import CacheError
+    plain_spec = small_spec(2, [ScheduleEntry(0), ScheduleEntry(1)])
+    counting = dataclasses.replace(plain_spec.layers[0], mixer=PartSpec("toy_counting_attention",
+                                                                        plain_spec.layers[0].mixer.params))
+    spec = dataclasses.replace(plain_spec, layers=[counting, plain_spec.layers[1]])
+    w = weights_for(plain_spec, seed=11)
+    g = torch.Generator().manual_seed(2)
+    lengths, more = [7, 2, 70, 5, 1], [12, 12, 5, 12, 5]
+    seqs = [torch.randint(0, 60, (n + m,), generator=g).tolist() for n, m in zip(lengths, more)]
+
+    def run(model_spec):
+        engine = Engine(None, model_spec, w, dtype="float32", max_tokens=64 * 8, max_slots=len(seqs))
+        slots = [engine.alloc_slot() for _ in seqs]
+        out = [engine.step([StepEntry(s, t[:n], [n - 1]) for s, t, n in zip(slots, seqs, lengths)]).cpu()]
+        for step in range(max(more)):
+            live = [i for i in range(len(seqs)) if step < more[i]]
+            out.append(engine.step([StepEntry(slots[i], [seqs[i][lengths[i] + step]], [0]) for i in live]).cpu())
+        return engine, slots, torch.cat(out)
+
+    engine, slots, got = run(spec)
+    _, _, want = run(plain_spec)
+    assert torch.equal(got, want)                           # the attention itself is the library's
+    assert engine.use_graphs and engine.graphs_captured >= 2
+    needs = engine.model.cache_needs()
+    assert isinstance(needs[0], tuple) and isinstance(needs[1], KVNeed)
+    assert len(engine.cache.kv_groups) == 1 and len(engine.cache.state_groups) == 1     # both layers' pages in one group
+    counts = engine.cache.state_views(0)[0][:, 0].cpu()
+    assert [int(counts[s]) for s in slots] == [len(t) for t in seqs]
+    with pytest.raises(CacheError, match="state"):
+        engine.truncate(slots[0], 3)
+    engine.free_slot(slots[2])
+    again = engine.alloc_slot()
+    assert again == slots[2] and float(engine.cache.state_views(0)[0][again, 0]) == 0.0
+    engine.cache.check()
 
 
 # ---- a toy feed-forward with routing and a toy position encoding, defined here
