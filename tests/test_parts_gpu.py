@@ -227,6 +227,69 @@ def test_a_layer_named_twice_and_a_layer_that_reads_another_s_cache():
     assert "L1.k" not in Model(spec).tensor_needs()
 
 
+def test_layers_with_heads_of_different_sizes_and_numbers():
+    """Layer 0 has 4 query and 2 kv heads of 16, layer 1 has 6 and 3 of 32 with another rotation
+    and a feed-forward of another width: every part has its sizes as parameters, and the cache
+    keeps the two layers' keys and values in two groups with page tables of their own."""
+    hidden, vocab = 40, 60
+    sizes = [dict(nq=4, nkv=2, hd=16, rot=16, theta=1e4, inter=56), dict(nq=6, nkv=3, hd=32, rot=8, theta=1e6, inter=24)]
+    layers = []
+    for i, z in enumerate(sizes):
+        p = f"L{i}."
+        pos = PartSpec("rope", {"theta": z["theta"], "rotary_dims": z["rot"], "max_positions": 256})
+        mixer = PartSpec("attention", dict(hidden_size=hidden, num_heads=z["nq"], num_kv_heads=z["nkv"], head_dim=z["hd"],
+                                           eps=1e-6, position=pos,
+                                           names={k: p + k for k in ("q", "k", "v", "o", "q_norm", "k_norm")}))
+        ffn = PartSpec("swiglu", {"hidden_size": hidden, "intermediate_size": z["inter"],
+                                  "names": {"gate": p + "g", "up": p + "u", "down": p + "d"}})
+        norms = {"input": PartSpec("rmsnorm", {"size": hidden, "eps": 1e-6, "weight": p + "n1"}),
+                 "post_mixer": PartSpec("rmsnorm", {"size": hidden, "eps": 1e-6, "weight": p + "n2"})}
+        layers.append(LayerSpec(PartSpec("prenorm"), mixer, ffn, norms))
+    base = small_spec(1, [ScheduleEntry(0)])
+    spec = ModelSpec(hidden_size=hidden, vocab_size=vocab, max_positions=256, embedding=base.embedding, layers=layers,
+                     schedule=[ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(0)], final_norm=base.final_norm,
+                     head=base.head)
+    w = weights_for(spec, seed=21)
+    g = torch.Generator().manual_seed(21)
+    seqs = [torch.randint(0, vocab, (n,), generator=g).tolist() for n in (70, 9, 130)]
+
+    def plain(tokens):
+        positions = list(range(len(tokens)))
+        x = pops.embedding(tokens, w["emb"])
+        for i in (0, 1, 0):
+            z, p = sizes[i], f"L{i}."
+            y = pops.rms_norm(x, w[p + "n1"], 1e-6)
+            q = pops.head_rms_norm(pops.split_heads(pops.linear(y, w[p + "q"]), z["nq"], z["hd"]), w[p + "q_norm"], 1e-6)
+            k = pops.head_rms_norm(pops.split_heads(pops.linear(y, w[p + "k"]), z["nkv"], z["hd"]), w[p + "k_norm"], 1e-6)
+            q = pops.apply_rope(q, positions, z["theta"], rotary_ndims=z["rot"])
+            k = pops.apply_rope(k, positions, z["theta"], rotary_ndims=z["rot"])
+            v = pops.split_heads(pops.linear(y, w[p + "v"]), z["nkv"], z["hd"])
+            a = pops.causal_attention(q, k, v, positions).reshape(len(tokens), z["nq"] * z["hd"])
+            x = x + pops.linear(a, w[p + "o"])
+            x = x + pops.swiglu_mlp(pops.rms_norm(x, w[p + "n2"], 1e-6), w[p + "g"], w[p + "u"], w[p + "d"])
+        return pops.linear(pops.rms_norm(x, w["fn"], 1e-6), w["emb"])
+
+    engine = Engine(None, spec, w, dtype="float32", max_tokens=64 * 6)
+    assert sorted((n.kv_heads, n.head_dim) for n in engine.cache.kv_groups) == [(2, 16), (3, 32)]
+    assert [len(grp.entries) for need, grp in sorted(engine.cache.kv_groups.items(), key=lambda kv: kv[0].head_dim)] == [2, 1]
+    # the three together: prompts less their last five tokens in one step, then one token each
+    slots = [engine.alloc_slot() for _ in seqs]
+    first = engine.step([StepEntry(s, t[:-5], list(range(len(t) - 5))) for s, t in zip(slots, seqs)]).cpu()
+    rows, at = [], 0
+    for t in seqs:
+        rows.append([first[at:at + len(t) - 5]])
+        at += len(t) - 5
+    for j in range(5, 0, -1):
+        out = engine.step([StepEntry(s, [t[len(t) - j]], [0]) for s, t in zip(slots, seqs)]).cpu()
+        for i in range(len(seqs)):
+            rows[i].append(out[i:i + 1])
+    for i, t in enumerate(seqs):
+        assert torch.allclose(torch.cat(rows[i]), plain(t), atol=1e-4), i
+    for s in slots:
+        engine.free_slot(s)
+    engine.cache.check()
+
+
 def test_a_model_without_rotation():
     spec = small_spec(1, [ScheduleEntry(0)], rope=False)
     w = weights_for(spec, seed=4)
