@@ -227,12 +227,21 @@ def test_a_layer_named_twice_and_a_layer_that_reads_another_s_cache():
     assert "L1.k" not in Model(spec).tensor_needs()
 
 
-def test_layers_with_heads_of_different_sizes_and_numbers():
-    """Layer 0 has 4 query and 2 kv heads of 16, layer 1 has 6 and 3 of 32 with another rotation
+MIXED_LAYERS = {
+    "float32": (40, [dict(nq=4, nkv=2, hd=16, rot=16, theta=1e4, inter=56), dict(nq=6, nkv=3, hd=32, rot=8, theta=1e6, inter=24)]),
+    # (heads of 128 and of 64, rotated whole: the matrix-core kernels of both sizes in one model)
+    "bfloat16": (128, [dict(nq=4, nkv=2, hd=128, rot=128, theta=1e4, inter=256), dict(nq=6, nkv=3, hd=64, rot=64, theta=1e6, inter=96)]),
+}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_layers_with_heads_of_different_sizes_and_numbers(dtype):
+    """Layer 0 has 4 query and 2 kv heads, layer 1 has 6 and 3 of another size with another rotation
     and a feed-forward of another width: every part has its sizes as parameters, and the cache
     keeps the two layers' keys and values in two groups with page tables of their own."""
-    hidden, vocab = 40, 60
-    sizes = [dict(nq=4, nkv=2, hd=16, rot=16, theta=1e4, inter=56), dict(nq=6, nkv=3, hd=32, rot=8, theta=1e6, inter=24)]
+    from .bounds import close
+    vocab = 60
+    hidden, sizes = MIXED_LAYERS[dtype]
     layers = []
     for i, z in enumerate(sizes):
         p = f"L{i}."
@@ -245,13 +254,16 @@ def test_layers_with_heads_of_different_sizes_and_numbers():
         norms = {"input": PartSpec("rmsnorm", {"size": hidden, "eps": 1e-6, "weight": p + "n1"}),
                  "post_mixer": PartSpec("rmsnorm", {"size": hidden, "eps": 1e-6, "weight": p + "n2"})}
         layers.append(LayerSpec(PartSpec("prenorm"), mixer, ffn, norms))
-    base = small_spec(1, [ScheduleEntry(0)])
+    base = small_spec(1, [ScheduleEntry(0)], hidden=hidden)
     spec = ModelSpec(hidden_size=hidden, vocab_size=vocab, max_positions=256, embedding=base.embedding, layers=layers,
                      schedule=[ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(0)], final_norm=base.final_norm,
                      head=base.head)
-    w = weights_for(spec, seed=21)
+    from herbert_rs_amd.engine.model import Model
+    from herbert_rs_amd.weights import random_tensors
+    w = random_tensors(Model(spec).tensor_needs(), 21, "float32", std=0.15 if dtype == "float32" else 0.05, norm_std=0.1)
+    w = {k: v.to(torch.bfloat16).float() if v.dim() == 2 else v for k, v in w.items()}      # both dtypes run the same model
     g = torch.Generator().manual_seed(21)
-    seqs = [torch.randint(0, vocab, (n,), generator=g).tolist() for n in (70, 9, 130)]
+    seqs = [torch.randint(0, vocab, (n,), generator=g).tolist() for n in (70, 9, 130, 3, 64)]
 
     def plain(tokens):
         positions = list(range(len(tokens)))
@@ -269,22 +281,25 @@ def test_layers_with_heads_of_different_sizes_and_numbers():
             x = x + pops.swiglu_mlp(pops.rms_norm(x, w[p + "n2"], 1e-6), w[p + "g"], w[p + "u"], w[p + "d"])
         return pops.linear(pops.rms_norm(x, w["fn"], 1e-6), w["emb"])
 
-    engine = Engine(None, spec, w, dtype="float32", max_tokens=64 * 6)
-    assert sorted((n.kv_heads, n.head_dim) for n in engine.cache.kv_groups) == [(2, 16), (3, 32)]
-    assert [len(grp.entries) for need, grp in sorted(engine.cache.kv_groups.items(), key=lambda kv: kv[0].head_dim)] == [2, 1]
-    # the three together: prompts less their last five tokens in one step, then one token each
+    engine = Engine(None, spec, w, dtype=dtype, max_tokens=64 * 9)
+    assert sorted((n.kv_heads, n.head_dim) for n in engine.cache.kv_groups) == sorted((z["nkv"], z["hd"]) for z in sizes)
+    assert sorted(len(grp.entries) for grp in engine.cache.kv_groups.values()) == [1, 2]
+    # the five together (decode steps of six rows): prompts less their last two tokens in one step, then one token each
     slots = [engine.alloc_slot() for _ in seqs]
-    first = engine.step([StepEntry(s, t[:-5], list(range(len(t) - 5))) for s, t in zip(slots, seqs)]).cpu()
+    first = engine.step([StepEntry(s, t[:-2], list(range(len(t) - 2))) for s, t in zip(slots, seqs)]).cpu()
     rows, at = [], 0
     for t in seqs:
-        rows.append([first[at:at + len(t) - 5]])
-        at += len(t) - 5
-    for j in range(5, 0, -1):
+        rows.append([first[at:at + len(t) - 2]])
+        at += len(t) - 2
+    for j in range(2, 0, -1):
         out = engine.step([StepEntry(s, [t[len(t) - j]], [0]) for s, t in zip(slots, seqs)]).cpu()
         for i in range(len(seqs)):
             rows[i].append(out[i:i + 1])
     for i, t in enumerate(seqs):
-        assert torch.allclose(torch.cat(rows[i]), plain(t), atol=1e-4), i
+        got, want = torch.cat(rows[i]).numpy(), plain(t).numpy()
+        for p in range(len(t)):
+            ok, err = close(got[p], want[p], dtype, "random", "mixed layers")
+            assert ok, (i, p, err)
     for s in slots:
         engine.free_slot(s)
     engine.cache.check()
