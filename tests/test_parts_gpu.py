@@ -152,14 +152,14 @@ def test_embedding_and_head_parts():
 
 
 # ---- models put together in other ways
-def small_spec(layers, schedule, hidden=40, vocab=60, rope=True, share_from=None):
-    pos = PartSpec("rope", {"theta": 1e4, "rotary_dims": 16, "max_positions": 256}) if rope else PartSpec("none")
+def small_spec(layers, schedule, hidden=40, vocab=60, rope=True, share_from=None, nq=4, nkv=2, hd=16):
+    pos = PartSpec("rope", {"theta": 1e4, "rotary_dims": hd, "max_positions": 256}) if rope else PartSpec("none")
     specs = []
     for i in range(layers):
         p = f"L{i}."
         reads = share_from is not None and i in share_from
         names = {k: p + k for k in (("q", "o", "q_norm") if reads else ("q", "k", "v", "o", "q_norm", "k_norm"))}
-        mixer = PartSpec("attention", dict(hidden_size=hidden, num_heads=4, num_kv_heads=2, head_dim=16, eps=1e-6,
+        mixer = PartSpec("attention", dict(hidden_size=hidden, num_heads=nq, num_kv_heads=nkv, head_dim=hd, eps=1e-6,
                                            position=pos, names=names, reads_cache_only=reads))
         ffn = PartSpec("swiglu", {"hidden_size": hidden, "intermediate_size": 56,
                                   "names": {"gate": p + "g", "up": p + "u", "down": p + "d"}})
@@ -180,20 +180,20 @@ def weights_for(spec, seed=0):
     return random_tensors(Model(spec).tensor_needs(), seed, "float32", std=0.15, norm_std=0.1)
 
 
-def plain_layer(w, p, x, positions, k_v_from=None, rope=True):
+def plain_layer(w, p, x, positions, k_v_from=None, rope=True, nq=4, nkv=2, hd=16):
     """One pre-norm layer of the small model by the plain formulas; returns (x, (k, v))."""
     y = pops.rms_norm(x, w[p + "n1"], 1e-6)
-    q = pops.head_rms_norm(pops.split_heads(pops.linear(y, w[p + "q"]), 4, 16), w[p + "q_norm"], 1e-6)
+    q = pops.head_rms_norm(pops.split_heads(pops.linear(y, w[p + "q"]), nq, hd), w[p + "q_norm"], 1e-6)
     if rope:
         q = pops.apply_rope(q, positions, 1e4)
     if k_v_from is None:
-        k = pops.head_rms_norm(pops.split_heads(pops.linear(y, w[p + "k"]), 2, 16), w[p + "k_norm"], 1e-6)
+        k = pops.head_rms_norm(pops.split_heads(pops.linear(y, w[p + "k"]), nkv, hd), w[p + "k_norm"], 1e-6)
         if rope:
             k = pops.apply_rope(k, positions, 1e4)
-        v = pops.split_heads(pops.linear(y, w[p + "v"]), 2, 16)
+        v = pops.split_heads(pops.linear(y, w[p + "v"]), nkv, hd)
     else:
         k, v = k_v_from
-    a = pops.causal_attention(q, k, v, positions).reshape(len(positions), 64)
+    a = pops.causal_attention(q, k, v, positions).reshape(len(positions), nq * hd)
     x = x + pops.linear(a, w[p + "o"])
     y = pops.rms_norm(x, w[p + "n2"], 1e-6)
     return x + pops.swiglu_mlp(y, w[p + "g"], w[p + "u"], w[p + "d"]), (k, v)
@@ -303,6 +303,50 @@ def test_layers_with_heads_of_different_sizes_and_numbers(dtype):
     for s in slots:
         engine.free_slot(s)
     engine.cache.check()
+
+
+@pytest.mark.parametrize("hd", [128, 64])
+def test_a_layer_that_reads_another_s_cache_in_bfloat16(hd):
+    """The same schedule (layer 0, layer 1 on layer 0's keys and values, layer 0 again) in bfloat16
+    with heads that the matrix-core kernels take: the layer without keys of its own norms and
+    rotates its queries alone and attends over pages that another entry wrote, for prompts and for
+    single tokens (four sequences together, and a fifth row of padding when one has ended)."""
+    from .bounds import close
+    from herbert_rs_amd.engine.model import Model
+    from herbert_rs_amd.weights import random_tensors
+    nq, nkv, hidden = 6, 2, 128
+    spec = small_spec(2, [ScheduleEntry(0), ScheduleEntry(1, cache=0), ScheduleEntry(0)], hidden=hidden, share_from={1},
+                      nq=nq, nkv=nkv, hd=hd)
+    w = random_tensors(Model(spec).tensor_needs(), 31, "float32", std=0.05, norm_std=0.1)
+    w = {k: v.to(torch.bfloat16).float() if v.dim() == 2 else v for k, v in w.items()}
+    g = torch.Generator().manual_seed(31)
+    lengths, more = [70, 5, 129, 33, 64, 2], [6, 6, 6, 6, 6, 3]
+    seqs = [torch.randint(0, 60, (n + m,), generator=g).tolist() for n, m in zip(lengths, more)]
+    engine = Engine(None, spec, w, dtype="bfloat16", max_tokens=64 * 10)
+    assert sorted(engine.model.cache_needs()) == [0, 2]
+    slots = [engine.alloc_slot() for _ in seqs]
+    first = engine.step([StepEntry(s, t[:n], list(range(n))) for s, t, n in zip(slots, seqs, lengths)]).cpu()
+    rows, at = [], 0
+    for n in lengths:
+        rows.append([first[at:at + n]])
+        at += n
+    for step in range(max(more)):
+        live = [i for i in range(len(seqs)) if step < more[i]]          # six, then five: steps of six rows
+        out = engine.step([StepEntry(slots[i], [seqs[i][lengths[i] + step]], [0]) for i in live]).cpu()
+        for r, i in enumerate(live):
+            rows[i].append(out[r:r + 1])
+    assert engine.graphs_captured >= 1
+    for i, t in enumerate(seqs):
+        pos = list(range(len(t)))
+        x = pops.embedding(t, w["emb"])
+        x, kv0 = plain_layer(w, "L0.", x, pos, nq=nq, nkv=nkv, hd=hd)
+        x, _ = plain_layer(w, "L1.", x, pos, k_v_from=kv0, nq=nq, nkv=nkv, hd=hd)
+        x, _ = plain_layer(w, "L0.", x, pos, nq=nq, nkv=nkv, hd=hd)
+        want = pops.linear(pops.rms_norm(x, w["fn"], 1e-6), w["emb"]).numpy()
+        got = torch.cat(rows[i]).numpy()
+        for p in pos:
+            ok, err = close(got[p], want[p], "bfloat16", "random", "shared cache")
+            assert ok, (i, p, err)
 
 
 def test_a_model_without_rotation():
