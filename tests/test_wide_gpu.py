@@ -144,7 +144,7 @@ def test_prompt_of_2048_and_decoding_at_batch_1_8_64(dtype, wide_folder, tmp_pat
 def test_decoding_at_every_batch_size_of_the_ladder_at_these_widths(wide_folder):
     """Decode steps run at a ladder of batch sizes, and the host picks other kernels along it (the
     few-row kernel up to 16 rows, tiles of 32 and of 64 rows with K slices and a second kernel that
-    norms, larger tiles beyond; an RMSNorm handed on half done or whole). Every size up to 80, with
+    norms, larger tiles beyond; an RMSNorm handed on half done or whole). Every size up to 80 and three up to 256, with
     one sequence fewer than the size where that leaves a padding row, at the 8B widths: the bfloat16
     engine's logits against those of the float32 engine (which the other tests hold against the
     plain implementation), within the bounds of these widths, for the prompts' last tokens and three
@@ -152,11 +152,13 @@ def test_decoding_at_every_batch_size_of_the_ladder_at_these_widths(wide_folder)
     from herbert_rs_amd.engine.batch import decode_batch_bucket
     sizes = sorted({decode_batch_bucket(n) for n in range(1, 81)})
     assert sizes[:10] == [1, 2, 3, 4, 6, 8, 10, 12, 14, 16] and sizes[-1] == 80
+    few_of = {144: 136, 208: 200}           # beyond 64 the ladder's steps are wider: eight rows of padding
+    sizes += [144, 208, 256]
     most = max(sizes)
     engines = {d: hb.load(wide_folder, dtype=d, cache_tokens=64 * 4 * most) for d in ("bfloat16", "float32")}
     worst = 0.0
     for size in sizes:
-        n = size - 1 if size in (6, 10, 14, 20, 28, 40, 56, 72) else size      # every other size with a padding row
+        n = few_of.get(size, size - 1 if size in (6, 10, 14, 20, 28, 40, 56, 72) else size)      # every other size with a padding row
         assert decode_batch_bucket(n) == size
         lengths = [1 + (41 * i + 7 * size) % 150 for i in range(n)]
         seqs = [random_tokens(VOCAB, m + 3, 2000 + 97 * size + i) for i, m in enumerate(lengths)]
