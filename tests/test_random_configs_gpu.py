@@ -4,7 +4,8 @@ one to eight query heads each, widths and vocabularies that are no power of two,
 layers, windows on some layers, partial rotation, linear and yarn scaling, tied and separate
 heads), and so do the requests: up to seven sequences of unequal lengths whose prompts come whole or
 in pieces, then their next tokens one by one, the shorter ones ending earlier. Every position's
-logits are compared with the plain implementation in float32 and in bfloat16."""
+logits are compared with the plain implementation in float32 and in bfloat16. Six larger draws
+(heads of 64 and 128, widths to 1,024, up to twelve sequences, prompts to 1,500 tokens) follow."""
 import random
 
 import numpy as np
@@ -54,11 +55,51 @@ def random_requests(rng):
     return prompts, more, piece
 
 
+def larger_config(rng):
+    """Heads of 64 and of 128 (the matrix-core attention kernels), widths of 256 to 1,024, up to eight
+    kv heads with up to eight query heads each, vocabularies to 16,401."""
+    hd = rng.choice([64, 128, 128])
+    nkv = rng.choice([1, 2, 4, 8])
+    group = rng.choice([1, 2, 4, 5, 8])
+    layers = rng.choice([1, 2])
+    raw = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=layers,
+               hidden_size=rng.choice([256, 384, 512, 520, 768, 1024]), num_attention_heads=nkv * group,
+               num_key_value_heads=nkv, head_dim=hd, intermediate_size=rng.choice([256, 704, 1000, 1536, 2048]),
+               vocab_size=rng.choice([1000, 2048, 5000, 16384 + 17]), rope_theta=rng.choice([1e4, 1e6]),
+               rms_norm_eps=rng.choice([1e-6, 1e-5]), tie_word_embeddings=rng.random() < 0.5,
+               max_position_embeddings=2048, eos_token_id=1)
+    if rng.random() < 0.25:
+        raw["sliding_window"] = rng.choice([33, 128, 500])
+        raw["layer_types"] = [rng.choice(["sliding_attention", "full_attention"]) for _ in range(layers)]
+    if rng.random() < 0.15:
+        raw["partial_rotary_factor"] = 0.5
+    return raw
+
+
+def larger_requests(rng):
+    n = rng.choice([1, 2, 3, 5, 7, 9, 12])
+    prompts = [rng.choice([1, 5, 63, 64, 65, 200, 256, 257, 511, 700, 1024, 1500]) for _ in range(n)]
+    more = [rng.choice([0, 1, 3, 8, 20, 40]) for _ in range(n)]
+    piece = rng.choice([None, None, 64, 256, 300])
+    return prompts, more, piece
+
+
 @pytest.mark.parametrize("seed", range(24))
 def test_random_configuration_and_schedule(seed, tmp_path):
     rng = random.Random(seed)
-    raw = random_config(rng)
-    prompts, more, piece = random_requests(rng)
+    drawn(seed, tmp_path, random_config(rng), *random_requests(rng), bounds="random")
+
+
+@pytest.mark.parametrize("seed", range(1000, 1006))
+def test_larger_random_configuration_and_schedule(seed, tmp_path):
+    """The same with larger draws. A draw compares thousands of rows of up to 16,401 logits, and the
+    largest of so many rounding errors is further out: the bounds are those of the widest vocabulary
+    (a one-off sweep of 195 such draws: 3.2e-5 at worst in float32, 0.0184 and 0.072 in bfloat16)."""
+    rng = random.Random(seed)
+    drawn(seed, tmp_path, larger_config(rng), *larger_requests(rng), bounds="wide")
+
+
+def drawn(seed, tmp_path, raw, prompts, more, piece, bounds):
     print(f"seed {seed}: {raw} prompts {prompts} then {more} one by one, pieces of {piece}", flush=True)
     for dtype in ("float32", "bfloat16"):
         folder = make_folder_from(tmp_path, "m", raw, seed, dtype=dtype, std=0.05, norm_std=0.1)
@@ -99,5 +140,5 @@ def test_random_configuration_and_schedule(seed, tmp_path):
         engine.cache.check()
         for i, s in enumerate(seqs):
             for t in range(len(s)):
-                ok, err = close(got[i][t], refs[i][t], dtype, "random", "drawn")
+                ok, err = close(got[i][t], refs[i][t], dtype, bounds, "drawn")
                 assert ok, f"{dtype}: sequence {i}, position {t}: off by {err}"
