@@ -220,13 +220,13 @@ def main():
     def step_gbs(batch, mean_context, ms):
         return (weight_bytes + batch * mean_context * kv_bytes_per_token) / (ms * 1e-3) / 1e9
 
-    def decode_run(batch, plan, run_ahead=True, fill_chunk=2048):
+    def decode_run(batch, plan, run_ahead=True, fill_chunk=2048, params=None):
         """[(context, tokens/s, ms/step)] for each (context, steps, warmup) of `plan` (contexts
         ascending): `steps` timed decode steps at `batch` after `warmup` untimed ones, ending with
         every sequence holding `context` tokens; one pass over a cache that is filled by real
         prefill of random prompts up to where each run's steps begin."""
         slots = [engine.alloc_slot() for _ in range(batch)]
-        chooser = Sampler(SamplingParams(temperature=0.0), batch, V, engine.device)
+        chooser = Sampler(params or SamplingParams(temperature=0.0), batch, V, engine.device)
         tokens = [ids(1)[0] for _ in range(batch)]
         held, chunk, out = 0, fill_chunk, []
 
@@ -374,6 +374,11 @@ def main():
         _, v_sync, ms_sync = decode_run(args.batch, [(context, min(args.steps, 16), 3)], run_ahead=False)[0]
         points[f"decode_b{args.batch}_host_between_steps"] = round(v_sync, 2)
         points[f"decode_b{args.batch}_host_between_steps_ms"] = round(ms_sync, 4)
+        # and with the command line's default sampling (temperature 0.4, top-k 40, top-p 0.9) in place of argmax
+        _, v_drawn, ms_drawn = decode_run(args.batch, [(context, min(args.steps, 16), 3)],
+                                          params=SamplingParams(temperature=0.4, top_k=40, top_p=0.9, seed=1))[0]
+        points[f"decode_b{args.batch}_sampled"] = round(v_drawn, 2)
+        points[f"decode_b{args.batch}_sampled_ms"] = round(ms_drawn, 4)
         # a batch of unequal lengths: one sequence at the full context beside fifteen of a sixteenth
         mixed = [context] + [max(context // 16, 64)] * 15
         ms_mixed, gbs_mixed, _ = unequal_run(mixed, min(args.steps, 16), 3)
