@@ -159,6 +159,9 @@ def main():
                     help="feed the prompt of the prefill figure in steps of this many tokens (0: in one step)")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run the 2,048-token prefill alone (for profiles); prints no JSON line")
+    ap.add_argument("--temperature", type=float, default=0.0,
+                    help="choose the decode steps' tokens by sampling at this temperature (top-k 40, top-p 0.9) "
+                         "instead of argmax")
     ap.add_argument("--contexts", default=None,
                     help="decode one batch whose sequences hold these numbers of tokens (comma-separated, "
                          "e.g. 32768,1024,1024: unequal lengths); prints ms a step and GB/s, no JSON line")
@@ -217,6 +220,9 @@ def main():
     H, I, V = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
     weight_bytes, kv_bytes_per_token, per_layer = workload_bytes(cfg, layers, elem)
 
+    headline_params = SamplingParams(temperature=0.0) if args.temperature <= 0 else \
+        SamplingParams(temperature=args.temperature, top_k=40, top_p=0.9, seed=1)
+
     def step_gbs(batch, mean_context, ms):
         return (weight_bytes + batch * mean_context * kv_bytes_per_token) / (ms * 1e-3) / 1e9
 
@@ -226,7 +232,7 @@ def main():
         every sequence holding `context` tokens; one pass over a cache that is filled by real
         prefill of random prompts up to where each run's steps begin."""
         slots = [engine.alloc_slot() for _ in range(batch)]
-        chooser = Sampler(params or SamplingParams(temperature=0.0), batch, V, engine.device)
+        chooser = Sampler(params or headline_params, batch, V, engine.device)
         tokens = [ids(1)[0] for _ in range(batch)]
         held, chunk, out = 0, fill_chunk, []
 
@@ -390,7 +396,8 @@ def main():
         points.pop(key)          # the headline itself: `value`, `ms_per_step`, `roofline`
     out = {
         "metric": "decode tok/s at batch 8, Qwen3-8B shape, context 4096 (+ prefill tok/s at 2048 "
-                  "tokens, decode at batch 1 and 64)",
+                  "tokens, decode at batch 1 and 64)" + (f", tokens sampled at temperature {args.temperature}"
+                                                         if args.temperature > 0 else ""),
         "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None,
